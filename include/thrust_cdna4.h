@@ -1,0 +1,165 @@
+/*
+ * thrust_cdna4.h — C ABI of libthrust_cdna4.so, the gfx950 (MI355X) device system for Thrust.
+ *
+ * This is the boundary the header-only C++ dispatch layer (include/thrust/system/cdna4/)
+ * calls.  Every entry point is `extern "C"`, takes plain pointers and sizes, returns an
+ * `int` that is a hipError_t value (0 = success), never throws, and enqueues its work on
+ * `stream` (a hipStream_t passed as void*; NULL = the legacy default stream) without
+ * waiting for it.  All data pointers are DEVICE pointers owned by the caller.
+ *
+ * Algorithms follow the two-phase temporary-storage protocol that the reference uses for
+ * its own device primitives (thrust/system/cuda/detail/sort.h:330-365,
+ * scan.h:80-117, reduce_by_key.h:1012-1031): call once with `temp == NULL` and the entry
+ * point only writes the number of bytes it needs to `*temp_bytes`; call again with a
+ * device buffer of at least that many bytes (256-byte aligned) to run.
+ *
+ * Semantics are those of the reference's sequential system, which is what its tests
+ * compare the device result against:
+ *   sort          thrust/system/detail/sequential/stable_radix_sort.inl:43-596, sort.inl:54-105
+ *   scan          thrust/system/detail/sequential/scan.h:47-114
+ *   scan_by_key   thrust/system/detail/sequential/scan_by_key.h:46-142
+ *   reduce_by_key thrust/system/detail/sequential/reduce_by_key.h:43-95
+ */
+#ifndef THRUST_CDNA4_H
+#define THRUST_CDNA4_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define THRUST_CDNA4_ABI_VERSION 1
+
+/* Element types.  The numeric values are part of the ABI. */
+typedef enum thrust_cdna4_dtype {
+  THRUST_CDNA4_I8 = 0,
+  THRUST_CDNA4_U8 = 1,
+  THRUST_CDNA4_I16 = 2,
+  THRUST_CDNA4_U16 = 3,
+  THRUST_CDNA4_I32 = 4,
+  THRUST_CDNA4_U32 = 5,
+  THRUST_CDNA4_I64 = 6,
+  THRUST_CDNA4_U64 = 7,
+  THRUST_CDNA4_F32 = 8,
+  THRUST_CDNA4_F64 = 9
+} thrust_cdna4_dtype;
+
+/* Binary operators of thrust/functional.h that the kernels are specialised on. */
+typedef enum thrust_cdna4_op {
+  THRUST_CDNA4_PLUS = 0,       /* thrust::plus       */
+  THRUST_CDNA4_MULTIPLIES = 1, /* thrust::multiplies */
+  THRUST_CDNA4_MAXIMUM = 2,    /* thrust::maximum    */
+  THRUST_CDNA4_MINIMUM = 3     /* thrust::minimum    */
+} thrust_cdna4_op;
+
+/* Returns THRUST_CDNA4_ABI_VERSION of the loaded library. */
+int thrust_cdna4_abi_version(void);
+
+/* Human-readable text for a return code (wraps hipGetErrorString). */
+const char* thrust_cdna4_error_string(int code);
+
+/*
+ * Stable LSD radix sort of `n` keys in place.  Replaces
+ * cuda_cub::__radix_sort::radix_sort<SORT_ITEMS=false> and the
+ * cub::DeviceRadixSort::SortKeys / SortKeysDescending calls under it
+ * (thrust/system/cuda/detail/sort.h:213-259, :306-380).  The alternate key buffer lives in
+ * `temp`, as it does in the reference (:338-343); the result always ends in `keys`.
+ * Order: ascending by the reference's RadixEncoder bit order
+ * (sequential/stable_radix_sort.inl:43-139) — for floating-point keys that is the total
+ * order -NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN.  `descending != 0` gives the
+ * order of thrust::greater (sequential/sort.inl:54-75).  n must be < 2^30.
+ */
+int thrust_cdna4_sort_keys(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
+                           int64_t n, int descending, void* stream);
+
+/*
+ * Stable LSD radix sort of `n` (key, value) pairs in place; values are opaque items of
+ * `value_bytes` bytes (1, 2, 4 or 8).  Replaces radix_sort<SORT_ITEMS=true> and
+ * cub::DeviceRadixSort::SortPairs / SortPairsDescending
+ * (thrust/system/cuda/detail/sort.h:261-304, :306-380).  Equal keys keep their input
+ * order, also when `descending != 0` (sequential/sort.inl:78-105).
+ */
+int thrust_cdna4_sort_pairs(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
+                            int value_bytes, void* values, int64_t n, int descending,
+                            void* stream);
+
+/*
+ * Prefix scan of `n` elements of type `dtype` under `op`.  Replaces
+ * cuda_cub::detail::inclusive_scan_n_impl / exclusive_scan_n_impl and cub::DispatchScan
+ * (thrust/system/cuda/detail/scan.h:57-204).  `exclusive == 0`: out[i] = in[0] op ... op
+ * in[i].  `exclusive != 0`: out[0] = *init, out[i] = *init op in[0] op ... op in[i-1];
+ * `init` is a HOST pointer to one element of `dtype` (NULL = value-initialised, the
+ * reference's default, scan.h:347-348).  `in == out` is allowed
+ * (testing/scan.cu:86-105).  Integer results are bit-exact (two's-complement wraparound);
+ * floating-point results are a reassociation of the serial left fold.
+ */
+int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int op, int exclusive,
+                      const void* in, void* out, int64_t n, const void* init, void* stream);
+
+/*
+ * Segmented prefix scan: segments are maximal runs of consecutive equal keys
+ * (thrust::equal_to on adjacent keys).  Replaces inclusive_scan_by_key_n /
+ * exclusive_scan_by_key_n and cub::DispatchScanByKey
+ * (thrust/system/cuda/detail/scan_by_key.h:69-282).  The exclusive form restarts from
+ * `*init` at every segment head (sequential/scan_by_key.h:95-140).  `values == out` is
+ * allowed.
+ */
+int thrust_cdna4_scan_by_key(void* temp, size_t* temp_bytes, int key_dtype, int value_dtype,
+                             int op, int exclusive, const void* keys, const void* values,
+                             void* out, int64_t n, const void* init, void* stream);
+
+/*
+ * Run-length segmented reduction.  Replaces __reduce_by_key::reduce_by_key_dispatch,
+ * ReduceByKeyAgent and InitAgent (thrust/system/cuda/detail/reduce_by_key.h:204-1058).
+ * For each maximal run of equal consecutive keys writes the run's first key to keys_out
+ * and the left-to-right reduction of its values to values_out; writes the number of runs
+ * (int64) to the DEVICE location `num_runs_out`, which the caller reads back after
+ * synchronising (reduce_by_key.h:1049-1052).  Outputs must not overlap inputs.
+ */
+int thrust_cdna4_reduce_by_key(void* temp, size_t* temp_bytes, int key_dtype, int value_dtype,
+                               int op, const void* keys_in, const void* values_in,
+                               void* keys_out, void* values_out, int64_t* num_runs_out,
+                               int64_t n, void* stream);
+
+/*
+ * Histogram with `num_bins` equal-width bins over [lower, upper): sample x falls in bin
+ * floor((x - lower) * num_bins / (upper - lower)); samples outside the range are not
+ * counted.  counts[0..num_bins) are uint32 and are overwritten.  The reference has no such
+ * function: this is the device counterpart of the dense-histogram pattern of
+ * examples/histogram.cu:60-101 (sort + upper_bound + adjacent_difference), whose result
+ * for integer-valued samples with unit-width bins it reproduces.
+ */
+int thrust_cdna4_histogram_even(void* temp, size_t* temp_bytes, int sample_dtype,
+                                const void* samples, int64_t n, uint32_t* counts,
+                                int num_bins, double lower, double upper, void* stream);
+
+/*
+ * Temporary-storage allocator.  Replaces cuda_cub::malloc / cuda_cub::free
+ * (thrust/system/cuda/detail/malloc_and_free.h:53-116), which call cudaMalloc / cudaFree on
+ * every algorithm invocation.  Blocks are cached per device in power-of-two size classes
+ * and handed back without a driver call; a block freed on one stream is reused on another
+ * only after an event recorded at the free has completed.
+ */
+int thrust_cdna4_malloc(void** ptr, size_t bytes, void* stream);
+int thrust_cdna4_free(void* ptr, void* stream);
+/* Returns every cached block to the driver (hipFree). */
+int thrust_cdna4_pool_trim(void);
+/* Bytes currently held by the pool (cached + handed out) on the current device. */
+size_t thrust_cdna4_pool_bytes(void);
+
+/* Data movement used by device_vector and cross-system copy
+ * (thrust/system/cuda/detail/util.h:142-199, internal/copy_cross_system.h:89-223). */
+int thrust_cdna4_memcpy_htod(void* dst, const void* src, size_t bytes, void* stream);
+int thrust_cdna4_memcpy_dtoh(void* dst, const void* src, size_t bytes, void* stream);
+int thrust_cdna4_memcpy_dtod(void* dst, const void* src, size_t bytes, void* stream);
+/* Fills n elements of elem_bytes (1, 2, 4 or 8) with the pattern at HOST pointer `value`
+ * (uninitialized_fill / fill for arithmetic types, cuda/detail/fill.h:61-75). */
+int thrust_cdna4_fill(void* dst, const void* value, int elem_bytes, int64_t n, void* stream);
+int thrust_cdna4_stream_synchronize(void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* THRUST_CDNA4_H */

@@ -1,0 +1,72 @@
+"""ctypes binding of libthrust_cdna4.so (the C ABI declared in include/thrust_cdna4.h).
+
+There is no fallback: if the HIP library has not been built, loading raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libthrust_cdna4.so")
+
+I8, U8, I16, U16, I32, U32, I64, U64, F32, F64 = range(10)
+PLUS, MULTIPLIES, MAXIMUM, MINIMUM = range(4)
+
+# every symbol include/thrust_cdna4.h declares
+SYMBOLS = [
+    "thrust_cdna4_abi_version", "thrust_cdna4_error_string", "thrust_cdna4_sort_keys",
+    "thrust_cdna4_sort_pairs", "thrust_cdna4_scan", "thrust_cdna4_scan_by_key",
+    "thrust_cdna4_reduce_by_key", "thrust_cdna4_histogram_even", "thrust_cdna4_malloc",
+    "thrust_cdna4_free", "thrust_cdna4_pool_trim", "thrust_cdna4_pool_bytes",
+    "thrust_cdna4_memcpy_htod", "thrust_cdna4_memcpy_dtoh", "thrust_cdna4_memcpy_dtod",
+    "thrust_cdna4_fill", "thrust_cdna4_stream_synchronize",
+]
+
+
+class Cdna4Error(RuntimeError):
+    """A C-ABI entry point returned a non-zero hipError_t."""
+
+    def __init__(self, code, what, text):
+        super().__init__(f"{what}: hip error {code} ({text})")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `make -C thrust_amd/csrc` "
+            "(or __graft_entry__.build()); there is no CPU fallback")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, sz, i32, i64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int64
+    psz = ctypes.POINTER(ctypes.c_size_t)
+    dbl = ctypes.c_double
+    L.thrust_cdna4_abi_version.restype = i32
+    L.thrust_cdna4_error_string.restype = ctypes.c_char_p
+    L.thrust_cdna4_error_string.argtypes = [i32]
+    L.thrust_cdna4_sort_keys.argtypes = [vp, psz, i32, vp, i64, i32, vp]
+    L.thrust_cdna4_sort_pairs.argtypes = [vp, psz, i32, vp, i32, vp, i64, i32, vp]
+    L.thrust_cdna4_scan.argtypes = [vp, psz, i32, i32, i32, vp, vp, i64, vp, vp]
+    L.thrust_cdna4_scan_by_key.argtypes = [vp, psz, i32, i32, i32, i32, vp, vp, vp, i64, vp, vp]
+    L.thrust_cdna4_reduce_by_key.argtypes = [vp, psz, i32, i32, i32, vp, vp, vp, vp, vp, i64, vp]
+    L.thrust_cdna4_histogram_even.argtypes = [vp, psz, i32, vp, i64, vp, i32, dbl, dbl, vp]
+    L.thrust_cdna4_malloc.argtypes = [ctypes.POINTER(vp), sz, vp]
+    L.thrust_cdna4_free.argtypes = [vp, vp]
+    L.thrust_cdna4_pool_bytes.restype = sz
+    L.thrust_cdna4_memcpy_htod.argtypes = [vp, vp, sz, vp]
+    L.thrust_cdna4_memcpy_dtoh.argtypes = [vp, vp, sz, vp]
+    L.thrust_cdna4_memcpy_dtod.argtypes = [vp, vp, sz, vp]
+    L.thrust_cdna4_fill.argtypes = [vp, vp, i32, i64, vp]
+    L.thrust_cdna4_stream_synchronize.argtypes = [vp]
+    _lib = L
+    return L
+
+
+def check(code, what):
+    if code != 0:
+        text = lib().thrust_cdna4_error_string(code).decode()
+        raise Cdna4Error(code, what, text)

@@ -1,0 +1,217 @@
+// Runtime services behind the C ABI: error text, the cached temporary-storage allocator,
+// copies, fills and stream synchronisation.
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+namespace tcd {
+
+__global__ void zero_words_kernel(uint32_t* p, size_t nwords) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < nwords; i += stride) p[i] = 0u;
+}
+
+// bytes must be a multiple of 4 (all internal regions are 256-byte multiples)
+hipError_t zero_async(void* p, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return hipSuccess;
+  const size_t nwords = bytes / 4;
+  size_t blocks = (nwords + 1023) / 1024;
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                     static_cast<uint32_t*>(p), nwords);
+  return hipGetLastError();
+}
+
+template <class T>
+__global__ void fill_kernel(T* p, T v, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = v;
+}
+
+template <class T>
+static hipError_t fill_typed(void* dst, const void* value, int64_t n, hipStream_t s) {
+  T v;
+  memcpy(&v, value, sizeof(T));
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(fill_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<T*>(dst), v, n);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------
+// Temporary-storage pool.  Replaces the per-call cudaMalloc / cudaFree of
+// thrust/system/cuda/detail/malloc_and_free.h:53-116.  Blocks are binned by
+// power-of-two size (minimum 256 B).  A free records an event on the freeing stream; the
+// block is handed to a different stream only once that event has completed, and to the
+// same stream immediately (stream order already serialises the two uses).
+// ---------------------------------------------------------------------------------------
+struct Block {
+  void* ptr;
+  size_t bytes;
+  int device;
+  hipStream_t stream;  // stream of the last free
+  hipEvent_t event;    // recorded at the last free
+};
+
+struct Pool {
+  std::mutex mu;
+  std::unordered_map<void*, Block> live;              // handed out
+  std::unordered_map<uint64_t, std::vector<Block>> cached;  // key: device << 8 | bin
+  size_t bytes_held = 0;
+};
+
+static Pool& pool() {
+  static Pool* p = new Pool();  // never destroyed: the HIP runtime may unload first
+  return *p;
+}
+
+static int bin_of(size_t bytes) {
+  int b = 8;
+  while (((size_t)1 << b) < bytes) b++;
+  return b;
+}
+
+}  // namespace tcd
+
+using namespace tcd;
+
+extern "C" int thrust_cdna4_abi_version(void) { return THRUST_CDNA4_ABI_VERSION; }
+
+extern "C" const char* thrust_cdna4_error_string(int code) {
+  return hipGetErrorString(static_cast<hipError_t>(code));
+}
+
+extern "C" int thrust_cdna4_malloc(void** ptr, size_t bytes, void* stream) {
+  if (!ptr) return hipErrorInvalidValue;
+  *ptr = nullptr;
+  if (bytes == 0) return hipSuccess;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const int bin = bin_of(bytes);
+  const uint64_t key = ((uint64_t)dev << 8) | (uint64_t)bin;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  Pool& P = pool();
+  {
+    std::lock_guard<std::mutex> g(P.mu);
+    auto it = P.cached.find(key);
+    if (it != P.cached.end()) {
+      auto& v = it->second;
+      for (size_t i = v.size(); i-- > 0;) {
+        Block b = v[i];
+        const bool ready = (b.stream == s) || (hipEventQuery(b.event) == hipSuccess);
+        if (ready) {
+          v.erase(v.begin() + (long)i);
+          P.live[b.ptr] = b;
+          *ptr = b.ptr;
+          return hipSuccess;
+        }
+      }
+    }
+  }
+  Block b{};
+  b.bytes = (size_t)1 << bin;
+  b.device = dev;
+  e = hipMalloc(&b.ptr, b.bytes);
+  if (e != hipSuccess) {
+    // give cached memory back to the driver and retry once
+    thrust_cdna4_pool_trim();
+    e = hipMalloc(&b.ptr, b.bytes);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();  // clear the sticky error, as the reference does before throwing
+      return e;
+    }
+  }
+  e = hipEventCreateWithFlags(&b.event, hipEventDisableTiming);
+  if (e != hipSuccess) {
+    (void)hipFree(b.ptr);
+    return e;
+  }
+  std::lock_guard<std::mutex> g(P.mu);
+  P.live[b.ptr] = b;
+  P.bytes_held += b.bytes;
+  *ptr = b.ptr;
+  return hipSuccess;
+}
+
+extern "C" int thrust_cdna4_free(void* ptr, void* stream) {
+  if (!ptr) return hipSuccess;
+  Pool& P = pool();
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  Block b;
+  {
+    std::lock_guard<std::mutex> g(P.mu);
+    auto it = P.live.find(ptr);
+    if (it == P.live.end()) return hipErrorInvalidValue;
+    b = it->second;
+    P.live.erase(it);
+  }
+  b.stream = s;
+  hipError_t e = hipEventRecord(b.event, s);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> g(P.mu);
+  P.cached[((uint64_t)b.device << 8) | (uint64_t)bin_of(b.bytes)].push_back(b);
+  return hipSuccess;
+}
+
+extern "C" int thrust_cdna4_pool_trim(void) {
+  Pool& P = pool();
+  std::vector<Block> victims;
+  {
+    std::lock_guard<std::mutex> g(P.mu);
+    for (auto& kv : P.cached) {
+      for (auto& b : kv.second) victims.push_back(b);
+      kv.second.clear();
+    }
+    for (auto& b : victims) P.bytes_held -= b.bytes;
+  }
+  hipError_t rc = hipSuccess;
+  for (auto& b : victims) {
+    hipError_t e = hipEventSynchronize(b.event);
+    if (e != hipSuccess) rc = e;
+    (void)hipEventDestroy(b.event);
+    e = hipFree(b.ptr);
+    if (e != hipSuccess) rc = e;
+  }
+  return rc;
+}
+
+extern "C" size_t thrust_cdna4_pool_bytes(void) {
+  Pool& P = pool();
+  std::lock_guard<std::mutex> g(P.mu);
+  return P.bytes_held;
+}
+
+extern "C" int thrust_cdna4_memcpy_htod(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return hipSuccess;
+  return hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream));
+}
+extern "C" int thrust_cdna4_memcpy_dtoh(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return hipSuccess;
+  return hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream));
+}
+extern "C" int thrust_cdna4_memcpy_dtod(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return hipSuccess;
+  return hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int thrust_cdna4_fill(void* dst, const void* value, int elem_bytes, int64_t n, void* stream) {
+  if (n < 0 || (n > 0 && (!dst || !value))) return hipErrorInvalidValue;
+  if (n == 0) return hipSuccess;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (elem_bytes) {
+    case 1: return fill_typed<uint8_t>(dst, value, n, s);
+    case 2: return fill_typed<uint16_t>(dst, value, n, s);
+    case 4: return fill_typed<uint32_t>(dst, value, n, s);
+    case 8: return fill_typed<uint64_t>(dst, value, n, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+extern "C" int thrust_cdna4_stream_synchronize(void* stream) {
+  return hipStreamSynchronize(static_cast<hipStream_t>(stream));
+}

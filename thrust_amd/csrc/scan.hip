@@ -1,0 +1,191 @@
+// Single-pass prefix scan with decoupled look-back for gfx950.
+//
+// One launch reads every element once and writes it once.  A workgroup takes a tile by
+// atomic ticket, loads it with 128-bit accesses (thread t owns 16 bytes of every 16·BLOCK
+// byte chunk, so loads and stores of a wave are contiguous), scans it with DPP wave scans,
+// publishes the tile aggregate, obtains the prefix of all earlier tiles by look-back and
+// writes the result.  Semantics: thrust/system/detail/sequential/scan.h:47-114; replaces
+// thrust/system/cuda/detail/scan.h:57-204 (cub::DispatchScan).
+#include "common.h"
+
+namespace tcd {
+
+template <class T>
+struct alignas(16) Vec16 {
+  T v[16 / sizeof(T)];
+};
+
+template <class T, class Op, int BLOCK, int CHUNKS>
+__global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_t n, T init,
+                                                     int exclusive, uint64_t* desc,
+                                                     uint32_t* ticket, int vec_ok) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int NWAVES = BLOCK / kWave;
+  constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
+  // payload in the descriptor: at least one dword
+  using W = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
+
+  __shared__ T s_tot[CHUNKS][NWAVES];
+  __shared__ T s_prefix;
+  __shared__ uint32_t s_tile;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const T id = Op::template identity<T>();
+  auto op = [](T a, T b) { return Op::template apply<T>(a, b); };
+
+  if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+  __syncthreads();
+  const int64_t tile = s_tile;
+  const int64_t base = tile * TILE;
+  const bool fast = vec_ok && (base + TILE <= n);
+
+  T x[CHUNKS][VEC];
+  if (fast) {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+      Vec16<T> v = *reinterpret_cast<const Vec16<T>*>(in + base + ((int64_t)c * BLOCK + tid) * VEC);
+#pragma unroll
+      for (int j = 0; j < VEC; j++) x[c][j] = v.v[j];
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+#pragma unroll
+      for (int j = 0; j < VEC; j++) {
+        int64_t idx = base + ((int64_t)c * BLOCK + tid) * VEC + j;
+        x[c][j] = idx < n ? in[idx] : id;
+      }
+    }
+  }
+
+  // thread-local inclusive scan of each 16-byte group, then a wave scan of the group sums.
+  // Cross-lane traffic, LDS and descriptors carry W (a dword container for 1- and 2-byte T).
+  auto toW = [](T a) {
+    if constexpr (std::is_same<W, T>::value) return a;
+    else return (W)(typename unsigned_of<T>::type)a;
+  };
+  auto opW = [&](W a, W b) {
+    if constexpr (std::is_same<W, T>::value) return op(a, b);
+    else return (W)(typename unsigned_of<T>::type)op((T)a, (T)b);
+  };
+  const W idW = toW(id);
+  T excl[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; c++) {
+#pragma unroll
+    for (int j = 1; j < VEC; j++) x[c][j] = op(x[c][j - 1], x[c][j]);
+    W incl = wave_inclusive_scan(toW(x[c][VEC - 1]), idW, opW);
+    excl[c] = (T)wave_shift_up1(incl, idW);
+    if (lane == kWave - 1) s_tot[c][wave] = (T)incl;
+  }
+  __syncthreads();
+
+  // offsets of this thread's (chunk, wave) segments inside the tile, and the tile aggregate
+  T seg_base[CHUNKS];
+  T run = id;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; c++) {
+#pragma unroll
+    for (int w = 0; w < NWAVES; w++) {
+      if (w == wave) seg_base[c] = run;
+      run = op(run, s_tot[c][w]);
+    }
+  }
+  const T tile_agg = run;
+
+  if (wave == 0) {
+    T prefix;
+    if (tile == 0) {
+      prefix = exclusive ? init : id;
+      if (lane == 0) TileDesc<W>::store(desc, 0, kInclusive, toW(op(prefix, tile_agg)));
+    } else {
+      if (lane == 0) TileDesc<W>::store(desc, tile, kPartial, toW(tile_agg));
+      prefix = (T)wave_lookback<W>(desc, tile, idW, opW);
+      if (lane == 0) TileDesc<W>::store(desc, tile, kInclusive, toW(op(prefix, tile_agg)));
+    }
+    if (lane == 0) s_prefix = prefix;
+  }
+  __syncthreads();
+  const T prefix = s_prefix;
+
+#pragma unroll
+  for (int c = 0; c < CHUNKS; c++) {
+    const T off = op(op(prefix, seg_base[c]), excl[c]);
+    T r[VEC];
+    if (exclusive) {
+      r[0] = off;
+#pragma unroll
+      for (int j = 1; j < VEC; j++) r[j] = op(off, x[c][j - 1]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; j++) r[j] = op(off, x[c][j]);
+    }
+    if (fast) {
+      Vec16<T> v;
+#pragma unroll
+      for (int j = 0; j < VEC; j++) v.v[j] = r[j];
+      *reinterpret_cast<Vec16<T>*>(out + base + ((int64_t)c * BLOCK + tid) * VEC) = v;
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; j++) {
+        int64_t idx = base + ((int64_t)c * BLOCK + tid) * VEC + j;
+        if (idx < n) out[idx] = r[j];
+      }
+    }
+  }
+}
+
+template <class T>
+struct ScanConfig {
+  static constexpr int BLOCK = 256;
+  static constexpr int CHUNKS = 4;
+  static constexpr int64_t TILE = (int64_t)BLOCK * (16 / sizeof(T)) * CHUNKS;
+  using P = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
+};
+
+template <class T, class Op>
+static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, const void* in,
+                             void* out, int64_t n, const void* init, hipStream_t stream) {
+  using C = ScanConfig<T>;
+  const int64_t ntiles = ceil_div(n, C::TILE);
+  const size_t need = 256 + align_up((size_t)ntiles * TileDesc<typename C::P>::kBytesPerTile, 256);
+  if (temp == nullptr) {
+    *temp_bytes = need;
+    return hipSuccess;
+  }
+  if (*temp_bytes < need) return hipErrorInvalidValue;
+  if (n == 0) return hipSuccess;
+  hipError_t e = zero_async(temp, need, stream);
+  if (e != hipSuccess) return e;
+  T iv = T(0);
+  if (init) __builtin_memcpy(&iv, init, sizeof(T));
+  uint32_t* ticket = reinterpret_cast<uint32_t*>(temp);
+  uint64_t* desc = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256);
+  const int vec_ok = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  hipLaunchKernelGGL((scan_kernel<T, Op, C::BLOCK, C::CHUNKS>), dim3((unsigned)ntiles), dim3(C::BLOCK),
+                     0, stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
+                     desc, ticket, vec_ok);
+  return hipGetLastError();
+}
+
+}  // namespace tcd
+
+extern "C" int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int op, int exclusive,
+                                 const void* in, void* out, int64_t n, const void* init,
+                                 void* stream) {
+  using namespace tcd;
+  if (!temp_bytes || n < 0 || (n > 0 && temp && (!in || !out))) return hipErrorInvalidValue;
+  hipError_t rc = hipErrorInvalidValue;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  bool ok = dispatch_dtype(dtype, [&](auto t) {
+    using T = decltype(t);
+    dispatch_op(op, [&](auto o) {
+      using Op = decltype(o);
+      rc = scan_typed<T, Op>(temp, temp_bytes, exclusive, in, out, n, init, s);
+    });
+  });
+  (void)ok;
+  return (int)rc;
+}
