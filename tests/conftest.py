@@ -1,0 +1,82 @@
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def kat():
+    with open(os.path.join(ROOT, "tests", "golden", "kat.json")) as f:
+        return json.load(f)
+
+
+# Size ladder of the reference's variable-size tests (testing/unittest/testframework.cu:21-31),
+# cut at 2^20+1 so the oracle finishes in seconds.
+SIZES = [0, 1, 2, 3, 4, 5, 8, 10, 13, 16, 17, 19, 27, 30, 31, 32, 33, 35, 42, 53, 58, 63, 64, 65,
+         72, 97, 100, 127, 128, 129, 142, 183, 192, 201, 240, 255, 256, 257, 302, 511, 512, 513,
+         687, 900, 1023, 1024, 1025, 1565, 1786, 1973, 2047, 2048, 2049, 3050, 4095, 4096, 4097,
+         5030, 7791, 10000, 10027, 12345, 16384, 17354, 26255, 32768, 43718, 65533, 65536, 65539,
+         123456, 131072, 731588, 1048575, 1048576, 1048577]
+SMALL_SIZES = [s for s in SIZES if s <= 70000]
+
+INT_DTYPES = [np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64]
+FLOAT_DTYPES = [np.float32, np.float64]
+ALL_DTYPES = INT_DTYPES + FLOAT_DTYPES
+
+
+def splitmix64(seed, n, offset=0):
+    """Counter-based generator: element i depends only on (seed, i)."""
+    with np.errstate(over="ignore"):
+        z = (np.arange(offset, offset + n, dtype=np.uint64) + np.uint64(1)) * np.uint64(0x9E3779B97F4A7C15)
+        z = z + np.uint64(seed)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+def random_ints(seed, n, dtype):
+    """Uniform over the full range of an integer dtype."""
+    bits = splitmix64(seed, n)
+    return bits.astype(np.dtype(dtype).str.replace("i", "u")).view(dtype) if np.dtype(dtype).kind == "i" \
+        else bits.astype(dtype)
+
+
+def random_floats(seed, n, dtype, specials=True):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal(n).astype(dtype)
+    if specials and n >= 16:
+        tiny = np.finfo(dtype).tiny
+        sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, -np.nan, tiny / 4, -tiny / 4], dtype=dtype)
+        x[rng.choice(n, 8, replace=False)] = sp
+    return x
+
+
+def encoded(keys):
+    """Unsigned key whose natural order is the reference's radix order
+    (thrust/system/detail/sequential/stable_radix_sort.inl:43-139)."""
+    keys = np.ascontiguousarray(keys)
+    w = keys.dtype.itemsize * 8
+    u = keys.view(f"u{keys.dtype.itemsize}")
+    sign = np.array(1 << (w - 1), dtype=u.dtype)
+    if keys.dtype.kind == "u":
+        return u.copy()
+    if keys.dtype.kind == "i":
+        return u ^ sign
+    ones = np.array((1 << w) - 1, dtype=u.dtype)
+    return u ^ np.where(u >> np.array(w - 1, dtype=u.dtype), ones, sign).astype(u.dtype)
+
+
+def same_bits(a, b):
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b)
+    return a.dtype == b.dtype and a.shape == b.shape and a.tobytes() == b.tobytes()

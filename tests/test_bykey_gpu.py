@@ -1,0 +1,161 @@
+"""GPU parity of thrust_cdna4_scan_by_key and thrust_cdna4_reduce_by_key against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import thrust_amd
+from conftest import SMALL_SIZES, random_ints, same_bits
+from gpu_util import dev, host
+
+pytestmark = pytest.mark.gpu
+
+FP_RTOL = 1e-5
+
+
+def runs(seed, n, mean, kd=np.int32):
+    """Sorted runs of keys with geometric run lengths (BASELINE config 4)."""
+    rng = np.random.default_rng(seed)
+    if n == 0:
+        return np.zeros(0, dtype=kd)
+    if mean <= 1:
+        return np.arange(n).astype(kd)
+    lens = rng.geometric(1.0 / mean, max(8, int(2.5 * n / mean) + 8))
+    keys = np.repeat(np.arange(lens.size), lens)
+    while keys.size < n:
+        keys = np.concatenate([keys, keys + keys[-1] + 1])
+    return keys[:n].astype(kd)
+
+
+# ------------------------------------------------------------------ scan_by_key
+def test_scan_by_key_kat(kat):
+    for case in kat["scan_by_key"]:
+        for kd in [np.int32, np.uint8, np.int64, np.float32, np.int16]:
+            for vd in [np.int32, np.int64, np.float32, np.uint16]:
+                k = dev(np.array(case["keys"], dtype=kd))
+                v = dev(np.array(case["values"], dtype=vd))
+                if case["exclusive"]:
+                    out = thrust_amd.exclusive_scan_by_key(k, v, init=case["init"], op=case["op"])
+                else:
+                    out = thrust_amd.inclusive_scan_by_key(k, v, op=case["op"])
+                assert host(out).tolist() == case["expected"], (case["source"], kd, vd)
+
+
+@pytest.mark.parametrize("kd,vd", [(np.int32, np.int32), (np.uint8, np.int64), (np.int64, np.uint16),
+                                   (np.uint16, np.uint32), (np.float32, np.int32), (np.int32, np.int8)])
+def test_scan_by_key_ints_bit_exact(kd, vd):
+    for n in SMALL_SIZES[::2] + [300007]:
+        for mean in (1, 3, 300):
+            k = (runs(n + mean, n, mean, np.int64) % 120).astype(kd)
+            v = random_ints(n, n, vd)
+            dk, dv = dev(k), dev(v)
+            assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv)), oracle.scan_by_key(k, v)), (n, mean)
+            assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=10)),
+                             oracle.scan_by_key(k, v, exclusive=True, init=10)), (n, mean)
+
+
+def test_scan_by_key_ops_and_in_place():
+    n = 50021
+    k = runs(1, n, 5)
+    v = random_ints(2, n, np.int32)
+    for op in ["multiplies", "maximum", "minimum"]:
+        dk, dv = dev(k), dev(v)
+        thrust_amd.inclusive_scan_by_key(dk, dv, out=dv, op=op)
+        assert same_bits(host(dv), oracle.scan_by_key(k, v, op)), op
+        dv = dev(v)
+        thrust_amd.exclusive_scan_by_key(dk, dv, out=dv, init=3, op=op)
+        assert same_bits(host(dv), oracle.scan_by_key(k, v, op, exclusive=True, init=3)), op
+
+
+def test_scan_by_key_float_tolerance():
+    n = 1 << 20
+    k = runs(3, n, 512)
+    v = np.random.default_rng(4).standard_normal(n).astype(np.float32)
+    got = host(thrust_amd.inclusive_scan_by_key(dev(k), dev(v))).astype(np.float64)
+    # float64 segmented reference and the L1 norm of each segment prefix
+    heads = np.ones(n, dtype=bool)
+    heads[1:] = k[1:] != k[:-1]
+    seg = np.cumsum(heads) - 1
+    c = np.cumsum(v.astype(np.float64))
+    a = np.cumsum(np.abs(v.astype(np.float64)))
+    start = np.nonzero(heads)[0]
+    ref = c - (c[start] - v[start].astype(np.float64))[seg]
+    l1 = a - (a[start] - np.abs(v[start].astype(np.float64)))[seg]
+    assert (np.abs(got - ref) <= FP_RTOL * l1 + 1e-30).all()
+    serial = oracle.scan_by_key(k, v).astype(np.float64)
+    assert (np.abs(got - serial) <= FP_RTOL * l1 + 1e-30).all()
+
+
+# ------------------------------------------------------------------ reduce_by_key
+def test_reduce_by_key_kat(kat):
+    for case in kat["reduce_by_key"]:
+        for kd in [np.int32, np.uint8, np.uint64, np.float64, np.int16]:
+            for vd in [np.int32, np.int64, np.float32, np.uint8]:
+                gk, gv = thrust_amd.reduce_by_key(dev(np.array(case["keys"], dtype=kd)),
+                                                  dev(np.array(case["values"], dtype=vd)), op=case["op"])
+                assert host(gk).tolist() == case["expected_keys"], (case["source"], kd, vd)
+                assert host(gv).tolist() == case["expected_values"], (case["source"], kd, vd)
+
+
+@pytest.mark.parametrize("kd,vd", [(np.int32, np.int32), (np.uint8, np.int64), (np.int64, np.uint16),
+                                   (np.uint16, np.uint32), (np.int32, np.uint8), (np.uint64, np.int64)])
+def test_reduce_by_key_ints_bit_exact(kd, vd):
+    for n in SMALL_SIZES[::2] + [300007]:
+        for mean in (1, 8, 512):
+            k = (runs(n + mean, n, mean, np.int64) % 200).astype(kd)
+            v = random_ints(n, n, vd)
+            gk, gv = thrust_amd.reduce_by_key(dev(k), dev(v))
+            rk, rv = oracle.reduce_by_key(k, v)
+            assert same_bits(host(gk), rk) and same_bits(host(gv), rv), (n, mean)
+
+
+def test_reduce_by_key_config4_reduced():
+    # BASELINE config 4 at 2^21: int32 values in [-1000,1000] bit-exact; fp32 N(0,1) within
+    # 1e-5 of the run's L1 norm
+    n = 1 << 21
+    rng = np.random.default_rng(7)
+    for mean in (1, 8, 512):
+        k = runs(mean, n, mean)
+        vi = rng.integers(-1000, 1001, n).astype(np.int32)
+        gk, gv = thrust_amd.reduce_by_key(dev(k), dev(vi))
+        rk, rv = oracle.reduce_by_key(k, vi)
+        assert same_bits(host(gk), rk) and same_bits(host(gv), rv), mean
+        vf = rng.standard_normal(n).astype(np.float32)
+        gk, gv = thrust_amd.reduce_by_key(dev(k), dev(vf))
+        rk, rv = oracle.reduce_by_key(k, vf)
+        assert same_bits(host(gk), rk)
+        starts = np.nonzero(np.concatenate([[True], k[1:] != k[:-1]]))[0]
+        ref = np.add.reduceat(vf.astype(np.float64), starts)
+        l1 = np.add.reduceat(np.abs(vf.astype(np.float64)), starts)
+        assert (np.abs(host(gv).astype(np.float64) - ref) <= FP_RTOL * l1 + 1e-30).all(), mean
+        assert (np.abs(host(gv).astype(np.float64) - rv.astype(np.float64)) <= FP_RTOL * l1 + 1e-30).all()
+
+
+def test_reduce_by_key_ops_and_float_keys():
+    n = 40009
+    k = runs(11, n, 6)
+    v = random_ints(12, n, np.int32)
+    for op in ["maximum", "minimum", "multiplies"]:
+        gk, gv = thrust_amd.reduce_by_key(dev(k), dev(v), op=op)
+        rk, rv = oracle.reduce_by_key(k, v, op)
+        assert same_bits(host(gk), rk) and same_bits(host(gv), rv), op
+    keys = np.array([0.0, -0.0, 1.0, np.nan, np.nan, 2.0, 2.0], dtype=np.float32)
+    vals = np.arange(7, dtype=np.int32)
+    gk, gv = thrust_amd.reduce_by_key(dev(keys), dev(vals))
+    rk, rv = oracle.reduce_by_key(keys, vals)
+    assert same_bits(host(gk), rk) and host(gv).tolist() == [1, 2, 3, 4, 11]
+
+
+def test_reduce_by_key_empty_and_full_size_closed_form():
+    gk, gv = thrust_amd.reduce_by_key(torch.empty(0, dtype=torch.int32, device="cuda"),
+                                      torch.empty(0, dtype=torch.int32, device="cuda"))
+    assert gk.numel() == 0 and gv.numel() == 0
+    # 2^28 elements, keys = i // 512, values = 1: every run sums to 512
+    # (closed form, cf. testing/cuda/reduce_by_key.cu:339-400)
+    n = 1 << 28
+    keys = torch.arange(n, dtype=torch.int32, device="cuda") // 512
+    vals = torch.ones(n, dtype=torch.int32, device="cuda")
+    gk, gv = thrust_amd.reduce_by_key(keys, vals)
+    assert gk.numel() == n // 512
+    assert torch.equal(gk, torch.arange(n // 512, dtype=torch.int32, device="cuda"))
+    assert bool((gv == 512).all())

@@ -1,0 +1,108 @@
+"""GPU parity of thrust_cdna4_scan against the oracle: integers bit-exact, floating point
+within 1e-5 of the running L1 norm (a reassociated sum cannot match the serial fold bit for
+bit; the bound is relative to sum |x_j| because prefix sums cross zero)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import thrust_amd
+from conftest import INT_DTYPES, SIZES, random_ints, same_bits
+from gpu_util import dev, host
+
+pytestmark = pytest.mark.gpu
+
+FP_RTOL = 1e-5
+
+
+def test_scan_kat(kat):
+    for case in kat["scan"]:
+        for dt in [np.int8, np.int16, np.int32, np.int64, np.float32, np.float64]:
+            x = dev(np.array(case["input"], dtype=dt))
+            if case["exclusive"]:
+                out = thrust_amd.exclusive_scan(x, init=case["init"], op=case["op"])
+            else:
+                out = thrust_amd.inclusive_scan(x, op=case["op"])
+            assert host(out).tolist() == case["expected"], (case["source"], dt)
+            assert host(x).tolist() == case["input"]  # input untouched
+            if case["exclusive"]:
+                thrust_amd.exclusive_scan(x, out=x, init=case["init"], op=case["op"])  # in place
+            else:
+                thrust_amd.inclusive_scan(x, out=x, op=case["op"])
+            assert host(x).tolist() == case["expected"], (case["source"], dt, "in place")
+
+
+def test_scan_i32_size_ladder():
+    for n in SIZES:
+        x = (random_ints(n, n, np.uint32) % 16).astype(np.int32)
+        d = dev(x)
+        assert same_bits(host(thrust_amd.inclusive_scan(d)), oracle.scan(x)), n
+        assert same_bits(host(thrust_amd.exclusive_scan(d, init=3)), oracle.scan(x, exclusive=True, init=3)), n
+
+
+@pytest.mark.parametrize("dtype", INT_DTYPES)
+@pytest.mark.parametrize("op", ["plus", "multiplies", "maximum", "minimum"])
+def test_scan_int_types_and_ops(dtype, op):
+    for n in [1, 65, 4097, 100003]:
+        x = random_ints(5 + n, n, dtype)
+        d = dev(x)
+        assert same_bits(host(thrust_amd.inclusive_scan(d, op=op)), oracle.scan(x, op)), n
+        assert same_bits(host(thrust_amd.exclusive_scan(d, init=7, op=op)),
+                         oracle.scan(x, op, exclusive=True, init=7)), n
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_scan_float_plus_tolerance(dtype):
+    for n in [1, 100, 4097, 1 << 20]:
+        x = np.random.default_rng(n).uniform(-1, 1, n).astype(dtype)
+        d = dev(x)
+        ref = np.cumsum(x.astype(np.float64))
+        l1 = np.cumsum(np.abs(x.astype(np.float64)))
+        got = host(thrust_amd.inclusive_scan(d)).astype(np.float64)
+        assert (np.abs(got - ref) <= FP_RTOL * l1).all(), n
+        serial = oracle.scan(x).astype(np.float64)  # the reference's own left fold
+        assert (np.abs(got - serial) <= FP_RTOL * l1).all(), n
+        got = host(thrust_amd.exclusive_scan(d, init=0.5)).astype(np.float64)
+        ref_e = np.concatenate([[0.0], ref[:-1]]) + 0.5
+        assert (np.abs(got - ref_e) <= FP_RTOL * (l1 + 0.5)).all(), n
+
+
+def test_scan_float_max_min_exact():
+    x = np.random.default_rng(2).standard_normal(200001).astype(np.float32)
+    d = dev(x)
+    assert same_bits(host(thrust_amd.inclusive_scan(d, op="maximum")), np.maximum.accumulate(x))
+    assert same_bits(host(thrust_amd.inclusive_scan(d, op="minimum")), np.minimum.accumulate(x))
+
+
+def test_scan_unaligned_in_place():
+    x = (random_ints(9, 70001, np.uint32) % 16).astype(np.int32)
+    d = dev(x)
+    v = d[1:]
+    thrust_amd.inclusive_scan(v, out=v)
+    assert same_bits(host(v), oracle.scan(x[1:]))
+    assert host(d)[0] == x[0]
+
+
+def test_scan_full_size_closed_forms():
+    # 2^28 elements (BASELINE config 2): constants have closed-form scans
+    n = 1 << 28
+    ones = torch.ones(n, dtype=torch.int32, device="cuda")
+    out = thrust_amd.inclusive_scan(ones)
+    assert torch.equal(out, torch.arange(1, n + 1, dtype=torch.int32, device="cuda"))
+    thrust_amd.exclusive_scan(ones, out=ones, init=0)  # in place
+    assert torch.equal(ones, torch.arange(0, n, dtype=torch.int32, device="cuda"))
+    del ones, out
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randint(0, 16, (n,), dtype=torch.int32, device="cuda", generator=g)
+    incl = thrust_amd.inclusive_scan(x)
+    excl = thrust_amd.exclusive_scan(x, init=0)
+    assert torch.equal(incl - excl, x)  # inclusive[i] - exclusive[i] == x[i]
+    assert int(incl[-1].item()) == int(x.sum(dtype=torch.int64).item())
+    assert bool((incl[1:] >= incl[:-1]).all())
+
+
+def test_scan_repeat_determinism_ints():
+    x = dev((random_ints(4, 1 << 22, np.uint32) % 16).astype(np.int32))
+    first = host(thrust_amd.inclusive_scan(x)).tobytes()
+    for _ in range(5):
+        assert host(thrust_amd.inclusive_scan(x)).tobytes() == first

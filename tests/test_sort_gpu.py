@@ -1,0 +1,148 @@
+"""GPU parity of thrust_cdna4_sort_keys / sort_pairs against the oracle (bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import thrust_amd
+from conftest import (FLOAT_DTYPES, INT_DTYPES, SIZES, SMALL_SIZES, encoded, random_floats, random_ints,
+                      same_bits, splitmix64)
+from gpu_util import dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+def test_sort_keys_kat(kat):
+    for case in kat["sort_keys"]:
+        for dt in case["dtypes"]:
+            d = dev(np.array(case["keys"], dtype=dt))
+            thrust_amd.sort(d, case["descending"])
+            assert host(d).tolist() == case["expected"], (case["source"], dt)
+
+
+def test_sort_pairs_kat(kat):
+    for case in kat["sort_pairs"]:
+        for kd in case["key_dtypes"]:
+            for vd in case["value_dtypes"]:
+                k = dev(np.array(case["keys"], dtype=kd))
+                v = dev(np.array(case["values"], dtype=vd))
+                thrust_amd.sort_by_key(k, v, case["descending"])
+                assert host(k).tolist() == case["expected_keys"], (case["source"], kd, vd)
+                assert host(v).tolist() == case["expected_values"], (case["source"], kd, vd)
+
+
+@pytest.mark.parametrize("descending", [False, True])
+def test_sort_u32_size_ladder(descending):
+    for n in SIZES:
+        k = random_ints(100 + n, n, np.uint32)
+        d = dev(k)
+        thrust_amd.sort(d, descending)
+        assert same_bits(host(d), oracle.sort_keys(k, descending)), n
+
+
+@pytest.mark.parametrize("dtype", INT_DTYPES)
+def test_sort_int_keys_all_types(dtype):
+    for n in [0, 1, 63, 257, 4096, 4097, 12345, 131072 + 5]:
+        for descending in (False, True):
+            k = random_ints(3 + n, n, dtype)
+            d = dev(k)
+            thrust_amd.sort(d, descending)
+            assert same_bits(host(d), oracle.sort_keys(k, descending)), (n, descending)
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+def test_sort_float_keys_total_order(dtype):
+    # -NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN, as the reference's CPP system sorts
+    tiny = np.finfo(dtype).tiny
+    ordered = np.array([-np.nan, -np.inf, -1.5, -tiny / 4, -0.0, 0.0, tiny / 4, 1.5, np.inf, np.nan],
+                       dtype=dtype)
+    perm = np.random.default_rng(3).permutation(len(ordered))
+    d = dev(ordered[perm])
+    thrust_amd.sort(d)
+    assert same_bits(host(d), ordered)
+    for n in [100, 4099, 200003]:
+        for descending in (False, True):
+            k = random_floats(n, n, dtype)
+            d = dev(k)
+            thrust_amd.sort(d, descending)
+            assert same_bits(host(d), oracle.sort_keys(k, descending)), (n, descending)
+
+
+def test_sort_variable_bits():
+    # keys with only the low `bits` bits set (testing/sort_variable_bits.cu:17-43)
+    n = 20011
+    for bits in range(0, 33, 3):
+        mask = np.uint32((1 << bits) - 1) if bits < 32 else np.uint32(0xFFFFFFFF)
+        k = random_ints(bits, n, np.uint32) & mask
+        d = dev(k)
+        thrust_amd.sort(d)
+        assert same_bits(host(d), np.sort(k)), bits
+
+
+@pytest.mark.parametrize("kd,vd", [(np.uint64, np.uint32), (np.uint32, np.uint32), (np.int32, np.uint64),
+                                   (np.int8, np.uint16), (np.uint16, np.uint8), (np.float32, np.uint32),
+                                   (np.float64, np.uint64), (np.int64, np.uint8)])
+def test_sort_pairs_stability(kd, vd):
+    for n in SMALL_SIZES[::3] + [262144 + 7]:
+        for descending in (False, True):
+            if np.dtype(kd).kind == "f":
+                k = (np.random.default_rng(n).integers(-20, 20, n) / 4).astype(kd)
+            else:
+                k = (splitmix64(n, n) % np.uint64(41)).astype(kd)  # many duplicates
+            v = np.arange(n).astype(vd)
+            dk, dv = dev(k), dev(v)
+            thrust_amd.sort_by_key(dk, dv, descending)
+            rk, rv = oracle.sort_pairs(k, v, descending)
+            assert same_bits(host(dk), rk) and same_bits(host(dv), rv), (n, descending)
+
+
+def test_sort_pairs_u64_entropy_sweep():
+    # BASELINE config 3 at reduced n: keys = AND of k uniform words; values = original index
+    n = (1 << 20) + 17
+    for words in range(0, 5):
+        k = np.full(n, np.uint64(0xFFFFFFFFFFFFFFFF))
+        for w in range(words):
+            k &= splitmix64(1000 + w, n)
+        if words == 0:
+            k[:] = np.uint64(42)  # all-equal keys
+        v = np.arange(n, dtype=np.uint32)
+        dk, dv = dev(k), dev(v)
+        thrust_amd.sort_by_key(dk, dv)
+        rk, rv = oracle.sort_pairs(k, v)
+        assert same_bits(host(dk), rk) and same_bits(host(dv), rv), words
+
+
+def test_sort_unaligned_views_and_repeat_determinism():
+    k = random_ints(77, 100001, np.uint32)
+    base = dev(k)
+    view = base[3:]  # 12-byte offset: not 16-byte aligned
+    thrust_amd.sort(view)
+    assert same_bits(host(view), np.sort(k[3:]))
+    assert same_bits(host(base[:3]), k[:3])
+    # look-back bugs show up as run-to-run differences
+    k = random_ints(78, 1 << 21, np.uint64)
+    v = np.arange(k.size, dtype=np.uint32)
+    first = None
+    for _ in range(5):
+        dk, dv = dev(k), dev(v)
+        thrust_amd.sort_by_key(dk, dv)
+        got = (host(dk).tobytes(), host(dv).tobytes())
+        first = first or got
+        assert got == first
+
+
+def test_sort_full_size_properties():
+    # 2^28 u32 keys: sortedness + multiset preserved (checksums), no oracle at this size
+    n = 1 << 28
+    g = torch.Generator(device="cuda").manual_seed(1337)
+    k = torch.randint(-2**31, 2**31, (n,), dtype=torch.int32, device="cuda", generator=g)
+    s0 = k.sum(dtype=torch.int64).item()
+    x0 = 0
+    for chunk in k.view(16, -1):
+        x0 ^= int(np.bitwise_xor.reduce(chunk.cpu().numpy().view(np.uint32)))
+    u = k.view(torch.uint32) if hasattr(torch, "uint32") else k
+    thrust_amd.sort(u)
+    hk = k.cpu().numpy().view(np.uint32)
+    assert (hk[1:] >= hk[:-1]).all()
+    assert int(hk.view(np.int32).sum(dtype=np.int64)) == s0
+    assert int(np.bitwise_xor.reduce(hk)) == x0
