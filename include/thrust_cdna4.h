@@ -159,6 +159,18 @@ int thrust_cdna4_memcpy_dtod(void* dst, const void* src, size_t bytes, void* str
 int thrust_cdna4_fill(void* dst, const void* value, int elem_bytes, int64_t n, void* stream);
 int thrust_cdna4_stream_synchronize(void* stream);
 
+/*
+ * Launch profiling.  While enabled, every kernel the library launches is bracketed by HIP
+ * events recorded on the launch stream and logged under its kernel name; enable(…) also
+ * clears the log.  get() waits for record `index` and returns its name and duration in
+ * milliseconds.  This is the counterpart of the reference's compile-time launch log
+ * (THRUST_DEBUG_SYNC, thrust/system/cuda/detail/core/agent_launcher.h:523-559); it is what
+ * the benchmark uses to time one kernel inside a multi-kernel algorithm.
+ */
+int thrust_cdna4_profile_enable(int on);
+int thrust_cdna4_profile_count(void);
+int thrust_cdna4_profile_get(int index, const char** name, float* ms);
+
 #ifdef __cplusplus
 }
 #endif

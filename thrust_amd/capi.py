@@ -18,7 +18,8 @@ SYMBOLS = [
     "thrust_cdna4_reduce_by_key", "thrust_cdna4_histogram_even", "thrust_cdna4_malloc",
     "thrust_cdna4_free", "thrust_cdna4_pool_trim", "thrust_cdna4_pool_bytes",
     "thrust_cdna4_memcpy_htod", "thrust_cdna4_memcpy_dtoh", "thrust_cdna4_memcpy_dtod",
-    "thrust_cdna4_fill", "thrust_cdna4_stream_synchronize",
+    "thrust_cdna4_fill", "thrust_cdna4_stream_synchronize", "thrust_cdna4_profile_enable",
+    "thrust_cdna4_profile_count", "thrust_cdna4_profile_get",
 ]
 
 
@@ -62,8 +63,23 @@ def lib():
     L.thrust_cdna4_memcpy_dtod.argtypes = [vp, vp, sz, vp]
     L.thrust_cdna4_fill.argtypes = [vp, vp, i32, i64, vp]
     L.thrust_cdna4_stream_synchronize.argtypes = [vp]
+    L.thrust_cdna4_profile_enable.argtypes = [i32]
+    L.thrust_cdna4_profile_get.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p),
+                                           ctypes.POINTER(ctypes.c_float)]
     _lib = L
     return L
+
+
+def profile_records():
+    """[(kernel name, milliseconds)] logged since thrust_cdna4_profile_enable(1)."""
+    L = lib()
+    out = []
+    for i in range(L.thrust_cdna4_profile_count()):
+        name = ctypes.c_char_p()
+        ms = ctypes.c_float()
+        check(L.thrust_cdna4_profile_get(i, ctypes.byref(name), ctypes.byref(ms)), "profile_get")
+        out.append((name.value.decode(), ms.value))
+    return out
 
 
 def check(code, what):

@@ -292,7 +292,7 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
       const int vec_ok = ((reinterpret_cast<uintptr_t>(keys) | reinterpret_cast<uintptr_t>(values) |
                            reinterpret_cast<uintptr_t>(out)) & 15) == 0;
       const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
-      hipLaunchKernelGGL((scan_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), 0, s,
+      TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
                          static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
                          n, iv, exclusive, float_keys, vec_ok,
                          reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
@@ -326,7 +326,7 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
       if (rc != hipSuccess) return;
       const int vec_ok = ((reinterpret_cast<uintptr_t>(keys_in) | reinterpret_cast<uintptr_t>(values_in)) & 15) == 0;
       const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
-      hipLaunchKernelGGL((reduce_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), 0, s,
+      TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
                          static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
                          static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
                          vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),

@@ -163,9 +163,8 @@ __device__ inline T wave_inclusive_scan(T v, const T id, F f) {
   return v;
 }
 
-// Exclusive value of lane i from an inclusive scan: the inclusive value of lane i-1, or
-// `id` in lane 0 (wave_shr:1 is not available on gfx9, so go through ds_bpermute-free DPP:
-// row_shr:1 inside rows, and fix up the first lane of each row from the previous row).
+// Exclusive value of lane i from an inclusive scan: the inclusive value of lane i-1
+// (fetched with ds_bpermute), or `id` in lane 0.
 template <class T>
 __device__ inline T wave_shift_up1(const T& incl, const T id) {
   static_assert(sizeof(T) % 4 == 0, "whole dwords");
@@ -310,6 +309,20 @@ inline bool dispatch_op(int op, F&& f) {
   }
   return false;
 }
+
+// Optional launch profiling: when enabled, every kernel launch of the library is bracketed by
+// HIP events on the launch stream and logged under its name (the counterpart of the
+// reference's THRUST_DEBUG_SYNC launch log, thrust/system/cuda/detail/core/agent_launcher.h:523-559).
+bool profile_enabled();
+void profile_begin(const char* name, hipStream_t stream);
+void profile_end(hipStream_t stream);
+
+#define TCD_LAUNCH(name, kernel, grid, block, stream, ...)                   \
+  do {                                                                       \
+    if (::tcd::profile_enabled()) ::tcd::profile_begin(name, stream);        \
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, __VA_ARGS__);         \
+    if (::tcd::profile_enabled()) ::tcd::profile_end(stream);                \
+  } while (0)
 
 // A small zero-fill kernel: used instead of hipMemsetAsync so that every entry point can be
 // recorded into a HIP graph.

@@ -100,10 +100,10 @@ static hipError_t histogram_typed(const void* samples, int64_t n, uint32_t* coun
   if (num_bins <= kHistLdsWords) {
     int reps = kHistLdsWords / num_bins;
     if (reps > kHistWaves) reps = kHistWaves;
-    hipLaunchKernelGGL((histogram_kernel<T, true>), dim3((unsigned)blocks), dim3(kHistBlock), 0, s,
+    TCD_LAUNCH("histogram_kernel", (histogram_kernel<T, true>), dim3((unsigned)blocks), dim3(kHistBlock), s,
                        static_cast<const T*>(samples), n, counts, num_bins, lower, upper, scale, reps, vec_ok);
   } else {
-    hipLaunchKernelGGL((histogram_kernel<T, false>), dim3((unsigned)blocks), dim3(kHistBlock), 0, s,
+    TCD_LAUNCH("histogram_kernel", (histogram_kernel<T, false>), dim3((unsigned)blocks), dim3(kHistBlock), s,
                        static_cast<const T*>(samples), n, counts, num_bins, lower, upper, scale, 1, vec_ok);
   }
   return hipGetLastError();

@@ -20,9 +20,41 @@ hipError_t zero_async(void* p, size_t bytes, hipStream_t stream) {
   const size_t nwords = bytes / 4;
   size_t blocks = (nwords + 1023) / 1024;
   if (blocks > 2048) blocks = 2048;
-  hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
-                     static_cast<uint32_t*>(p), nwords);
+  TCD_LAUNCH("zero_words_kernel", zero_words_kernel, dim3((unsigned)blocks), dim3(256), stream,
+             static_cast<uint32_t*>(p), nwords);
   return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------
+// Launch profiling records
+// ---------------------------------------------------------------------------------------
+struct ProfileRecord {
+  const char* name;
+  hipEvent_t start, stop;
+};
+struct Profiler {
+  std::mutex mu;
+  bool on = false;
+  std::vector<ProfileRecord> recs;
+};
+static Profiler& profiler() {
+  static Profiler* p = new Profiler();
+  return *p;
+}
+bool profile_enabled() { return profiler().on; }
+void profile_begin(const char* name, hipStream_t stream) {
+  Profiler& P = profiler();
+  std::lock_guard<std::mutex> g(P.mu);
+  if (P.recs.size() >= 65536) return;
+  ProfileRecord r{name, nullptr, nullptr};
+  if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) return;
+  (void)hipEventRecord(r.start, stream);
+  P.recs.push_back(r);
+}
+void profile_end(hipStream_t stream) {
+  Profiler& P = profiler();
+  std::lock_guard<std::mutex> g(P.mu);
+  if (!P.recs.empty()) (void)hipEventRecord(P.recs.back().stop, stream);
 }
 
 template <class T>
@@ -38,7 +70,7 @@ static hipError_t fill_typed(void* dst, const void* value, int64_t n, hipStream_
   memcpy(&v, value, sizeof(T));
   int64_t blocks = (n + 255) / 256;
   if (blocks > 8192) blocks = 8192;
-  hipLaunchKernelGGL(fill_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<T*>(dst), v, n);
+  TCD_LAUNCH("fill_kernel", fill_kernel<T>, dim3((unsigned)blocks), dim3(256), s, static_cast<T*>(dst), v, n);
   return hipGetLastError();
 }
 
@@ -83,6 +115,38 @@ extern "C" int thrust_cdna4_abi_version(void) { return THRUST_CDNA4_ABI_VERSION;
 
 extern "C" const char* thrust_cdna4_error_string(int code) {
   return hipGetErrorString(static_cast<hipError_t>(code));
+}
+
+extern "C" int thrust_cdna4_profile_enable(int on) {
+  Profiler& P = profiler();
+  std::lock_guard<std::mutex> g(P.mu);
+  for (auto& r : P.recs) {
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  P.recs.clear();
+  P.on = on != 0;
+  return hipSuccess;
+}
+
+extern "C" int thrust_cdna4_profile_count(void) {
+  Profiler& P = profiler();
+  std::lock_guard<std::mutex> g(P.mu);
+  return (int)P.recs.size();
+}
+
+extern "C" int thrust_cdna4_profile_get(int index, const char** name, float* ms) {
+  Profiler& P = profiler();
+  ProfileRecord r;
+  {
+    std::lock_guard<std::mutex> g(P.mu);
+    if (index < 0 || index >= (int)P.recs.size() || !name || !ms) return hipErrorInvalidValue;
+    r = P.recs[(size_t)index];
+  }
+  hipError_t e = hipEventSynchronize(r.stop);
+  if (e != hipSuccess) return e;
+  *name = r.name;
+  return hipEventElapsedTime(ms, r.start, r.stop);
 }
 
 extern "C" int thrust_cdna4_malloc(void** ptr, size_t bytes, void* stream) {

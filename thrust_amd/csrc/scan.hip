@@ -164,9 +164,9 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   uint32_t* ticket = reinterpret_cast<uint32_t*>(temp);
   uint64_t* desc = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256);
   const int vec_ok = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-  hipLaunchKernelGGL((scan_kernel<T, Op, C::BLOCK, C::CHUNKS>), dim3((unsigned)ntiles), dim3(C::BLOCK),
-                     0, stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
-                     desc, ticket, vec_ok);
+  TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS>), dim3((unsigned)ntiles), dim3(C::BLOCK),
+             stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
+             desc, ticket, vec_ok);
   return hipGetLastError();
 }
 

@@ -338,15 +338,14 @@ static hipError_t sort_typed(void* temp, size_t* temp_bytes, void* keys, void* v
   const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & 15) == 0;
   int64_t hblocks = ceil_div(n, 256 * 64);
   if (hblocks > 2048) hblocks = 2048;
-  hipLaunchKernelGGL((radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(256), 0, stream,
-                     kbuf[0], n, xor_mask, ghist, vec_ok);
-  hipLaunchKernelGGL(radix_bins_kernel, dim3(P), dim3(256), 0, stream, ghist);
+  TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(256), stream,
+             kbuf[0], n, xor_mask, ghist, vec_ok);
+  TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(P), dim3(256), stream, ghist);
   int cur = 0;
   for (int p = 0; p < P; p++) {
-    hipLaunchKernelGGL((onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT>), dim3((unsigned)plan.ntiles),
-                       dim3(C::BLOCK), 0, stream, kbuf[cur], kbuf[cur ^ 1], vbuf[cur], vbuf[cur ^ 1], n,
-                       xor_mask, 8 * p, ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix,
-                       tickets + p);
+    TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT>), dim3((unsigned)plan.ntiles),
+               dim3(C::BLOCK), stream, kbuf[cur], kbuf[cur ^ 1], vbuf[cur], vbuf[cur ^ 1], n, xor_mask, 8 * p,
+               ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix, tickets + p);
     cur ^= 1;
   }
   e = hipGetLastError();
