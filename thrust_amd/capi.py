@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libthrust_cdna4.so")
+# THRUST_CDNA4_LIB points the harness at another build of the same C ABI (tuning builds).
+LIB_PATH = os.environ.get("THRUST_CDNA4_LIB") or os.path.join(_HERE, "lib", "libthrust_cdna4.so")
 
 I8, U8, I16, U16, I32, U32, I64, U64, F32, F64 = range(10)
 PLUS, MULTIPLIES, MAXIMUM, MINIMUM = range(4)

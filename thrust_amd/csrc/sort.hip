@@ -23,6 +23,7 @@ constexpr int kRadix = 1 << kRadixBits;
 
 // descriptor word: status in bits 31:30, count in bits 29:0
 constexpr uint32_t kCountMask = (1u << 30) - 1;
+constexpr int kLookW = 4;  // look-back descriptors loaded per round trip
 
 template <int BYTES>
 struct uint_of;
@@ -75,7 +76,16 @@ __global__ __launch_bounds__(256) void radix_hist_kernel(const U* __restrict__ k
   auto count = [&](U k) {
     const U e = encode_key<U, FLOAT>(k, xor_mask);
 #pragma unroll
-    for (int p = 0; p < P; p++) atomicAdd(&h[p][(uint32_t)(e >> (8 * p)) & 0xffu], 1u);
+    for (int p = 0; p < P; p++) {
+      const uint32_t d = (uint32_t)(e >> (8 * p)) & 0xffu;
+      // all active lanes on one digit (sorted / low-entropy keys): one atomic for the wave
+      const uint64_t active = __builtin_amdgcn_ballot_w64(true);
+      if (__builtin_amdgcn_ballot_w64(d != (uint32_t)__builtin_amdgcn_readfirstlane((int)d)) == 0) {
+        if (lane_id() == (int)__builtin_ctzll(active)) atomicAdd(&h[p][d], (uint32_t)__popcll(active));
+      } else {
+        atomicAdd(&h[p][d], 1u);
+      }
+    }
   };
 
   const int64_t gtid = (int64_t)blockIdx.x * blockDim.x + tid;
@@ -131,15 +141,40 @@ struct OnesweepSmem {
   static constexpr int TILE = BLOCK * IPT;
   static constexpr int ELEM = (int)sizeof(U) > VB ? (int)sizeof(U) : VB;
   alignas(16) unsigned char exch[(size_t)TILE * ELEM];  // key / value exchange buffer
-  uint32_t wave_cnt[BLOCK / kWave][kRadix];             // per-wave digit counters
-  uint32_t local_base[kRadix];                          // first local slot of each digit
+  uint32_t wave_cnt[BLOCK / kWave][kRadix];             // per-wave digit counts, then next free local slots
   uint32_t global_off[kRadix];                          // global slot of local slot 0, per digit
   uint32_t wave_tot[4];
   uint32_t tile;
 };
 
+// Lanes of this wavefront whose 8-bit digit equals this lane's digit, as two 32-bit halves.
+// Per bit: one v_bfe_i32 (0 / -1 per lane), one v_cmp (the ballot, an SGPR pair) and one
+// three-input bit operation per half:  m &= ~(ballot ^ bit)   (truth table 0x90).
+__device__ inline void match_digit(uint32_t d, uint32_t& m_lo, uint32_t& m_hi) {
+  m_lo = ~0u;
+  m_hi = ~0u;
+#pragma unroll
+  for (int b = 0; b < kRadixBits; b++) {
+    int32_t e = __builtin_amdgcn_sbfe((int)d, b, 1);
+    asm("" : "+v"(e));  // keep the compare on e itself instead of a second bit extraction
+    const uint64_t bal = __builtin_amdgcn_ballot_w64(e != 0);
+    m_lo = __builtin_amdgcn_bitop3_b32(m_lo, (uint32_t)bal, (uint32_t)e, 0x90);
+    m_hi = __builtin_amdgcn_bitop3_b32(m_hi, (uint32_t)(bal >> 32), (uint32_t)e, 0x90);
+  }
+}
+
+__device__ inline uint32_t lds_load(const uint32_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+}
+__device__ inline void lds_store(uint32_t* p, uint32_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+}
+
+#ifndef TCD_SORT_WPE
+#define TCD_SORT_WPE 4
+#endif
 template <class U, int VB, bool FLOAT, int BLOCK, int IPT>
-__global__ __launch_bounds__(BLOCK) void onesweep_kernel(const U* __restrict__ kin, U* __restrict__ kout,
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_WPE))) void onesweep_kernel(const U* __restrict__ kin, U* __restrict__ kout,
                                                          const void* __restrict__ vin_, void* __restrict__ vout_,
                                                          int64_t n, U xor_mask, int shift,
                                                          const uint32_t* __restrict__ gbase,
@@ -159,106 +194,130 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const U* __restrict__ k
   const int wave = tid / kWave;
 
   if (tid == 0) sm.tile = atomicAdd(ticket, 1u);
+  if (tid < kRadix) {
 #pragma unroll
-  for (int w = 0; w < NWAVES; w++)
-    if (tid < kRadix) sm.wave_cnt[w][tid] = 0;
+    for (int w = 0; w < NWAVES; w++) sm.wave_cnt[w][tid] = 0;
+  }
   __syncthreads();
   const int64_t tile = sm.tile;
   const int64_t base = tile * TILE;
   const int valid = (int)((n - base) < (int64_t)TILE ? (n - base) : (int64_t)TILE);
+  const bool full = valid == TILE;
+
+  auto digit_of = [&](U key) -> uint32_t {
+    return (uint32_t)(encode_key<U, FLOAT>(key, xor_mask) >> shift) & 0xffu;
+  };
 
   // ---- load: wave w owns a contiguous slab, item i of lane l is slab[i*64 + l], so the
   //      order (wave, item, lane) is the memory order and ranking in that order is stable.
-  const U pad = decode_key<U, FLOAT>(U(~U(0)), xor_mask);  // sorts after every real key
   const int slab = wave * (kWave * IPT) + lane;
   U k[IPT];
+  if (full) {
 #pragma unroll
-  for (int i = 0; i < IPT; i++) {
-    const int li = slab + i * kWave;
-    k[i] = li < valid ? kin[base + li] : pad;
+    for (int i = 0; i < IPT; i++) k[i] = kin[base + slab + i * kWave];
+  } else {
+    const U pad = decode_key<U, FLOAT>(U(~U(0)), xor_mask);  // sorts after every real key
+#pragma unroll
+    for (int i = 0; i < IPT; i++) {
+      const int li = slab + i * kWave;
+      k[i] = li < valid ? kin[base + li] : pad;
+    }
   }
 
-  // ---- rank: for each item, the lanes of this wave holding the same digit (8 ballots),
-  //      the count of such lanes below this one, and the wave's running counter.
-  volatile uint32_t* wc = sm.wave_cnt[wave];
-  const uint64_t lt_mask = (1ull << lane) - 1ull;
-  uint32_t pos[IPT];
+  // ---- early counts: per-wave digit histogram with LDS atomics, so that the tile's counts
+  //      are published before the (long) ranking phase and later tiles rarely wait for them
+  uint32_t* wc = sm.wave_cnt[wave];
 #pragma unroll
   for (int i = 0; i < IPT; i++) {
-    const uint32_t d = (uint32_t)(encode_key<U, FLOAT>(k[i], xor_mask) >> shift) & 0xffu;
-    uint64_t m = ~0ull;
-#pragma unroll
-    for (int b = 0; b < kRadixBits; b++) {
-      const bool bit = (d >> b) & 1u;
-      const uint64_t bal = __ballot(bit);
-      m &= bit ? bal : ~bal;
+    const uint32_t d = digit_of(k[i]);
+    // a wave whose 64 keys share one digit (sorted or low-entropy input) would serialise 64
+    // same-address atomics: let one lane add 64 instead
+    if (__builtin_amdgcn_ballot_w64(d != (uint32_t)__builtin_amdgcn_readfirstlane((int)d)) == 0) {
+      if (lane == 0) atomicAdd(wc + d, (uint32_t)kWave);
+    } else {
+      atomicAdd(wc + d, 1u);
     }
-    const uint32_t below = __popcll(m & lt_mask);
-    const uint32_t cnt = __popcll(m);
-    const uint32_t old = wc[d];
-    if (below == 0) wc[d] = old + cnt;
-    pos[i] = old + below;
   }
   __syncthreads();
 
-  // ---- per digit (thread d): exclusive offsets of the waves, tile count, publish, scan
-  uint32_t total = 0;
+  // ---- per digit (thread d): tile count, publish it, first local slot of each wave's keys
+  uint32_t total = 0, lbase = 0;
+  uint32_t wexcl[NWAVES];
   if (tid < kRadix) {
 #pragma unroll
     for (int w = 0; w < NWAVES; w++) {
-      const uint32_t c = sm.wave_cnt[w][tid];
-      sm.wave_cnt[w][tid] = total;
-      total += c;
+      wexcl[w] = total;
+      total += sm.wave_cnt[w][tid];
     }
     const uint32_t st = (tile == 0) ? kInclusive : kPartial;
     st_agent(&desc[tile * kRadix + tid], (st << 30) | total);
     const uint32_t incl = wave_inclusive_scan(total, 0u, [](uint32_t a, uint32_t b) { return a + b; });
     if (lane == 63) sm.wave_tot[wave] = incl;
-    sm.local_base[tid] = incl - total;  // completed below
+    lbase = incl - total;
   }
   __syncthreads();
   if (tid < kRadix) {
-    uint32_t wbase = 0;
-    for (int w = 0; w < wave; w++) wbase += sm.wave_tot[w];
-    const uint32_t lbase = sm.local_base[tid] + wbase;
-    // look-back over earlier tiles for this digit
+    for (int w = 0; w < wave; w++) lbase += sm.wave_tot[w];
+#pragma unroll
+    for (int w = 0; w < NWAVES; w++) sm.wave_cnt[w][tid] = lbase + wexcl[w];
+  }
+  __syncthreads();
+
+  // ---- rank and reorder: a wave's counter of a digit is its next free local slot; the lanes
+  //      holding the same digit (8 ballots) take consecutive slots in lane order
+  uint32_t pos[IPT];
+#pragma unroll
+  for (int i = 0; i < IPT; i++) {
+    const uint32_t d = digit_of(k[i]);
+    uint32_t m_lo, m_hi;
+    match_digit(d, m_lo, m_hi);
+    const uint32_t below = __builtin_amdgcn_mbcnt_hi(m_hi, __builtin_amdgcn_mbcnt_lo(m_lo, 0u));
+    const uint32_t cnt = __builtin_popcount(m_lo) + __builtin_popcount(m_hi);
+    const uint32_t old = lds_load(wc + d);         // every lane of the group reads the counter,
+    if (below == 0) lds_store(wc + d, old + cnt);  // then its first lane advances it
+    __builtin_amdgcn_wave_barrier();
+    pos[i] = old + below;
+    s_keys[pos[i]] = k[i];
+  }
+
+  // ---- look-back over earlier tiles (thread d for digit d), kLookW descriptors per round trip
+  if (tid < kRadix) {
     uint32_t prefix = 0;
     if (tile > 0) {
       int64_t t = tile - 1;
-      while (true) {
-        const uint32_t v = ld_agent(&desc[t * kRadix + tid]);
-        const uint32_t st = v >> 30;
-        if (st == kInvalid) {
-          __builtin_amdgcn_s_sleep(1);
-          continue;
+      bool done = false;
+      while (!done) {
+        uint32_t v[kLookW];
+#pragma unroll
+        for (int j = 0; j < kLookW; j++)
+          v[j] = (t - j >= 0) ? ld_agent(&desc[(t - j) * kRadix + tid]) : ((uint32_t)kInclusive << 30);
+        int used = 0;
+#pragma unroll
+        for (int j = 0; j < kLookW; j++) {
+          const uint32_t st = v[j] >> 30;
+          if (!done && used == j && st != kInvalid) {
+            prefix += v[j] & kCountMask;
+            used = j + 1;
+            done = st == kInclusive;
+          }
         }
-        prefix += v & kCountMask;
-        if (st == kInclusive) break;
-        --t;
+        t -= used;
+        if (used == 0) __builtin_amdgcn_s_sleep(2);
       }
       st_agent(&desc[tile * kRadix + tid], ((uint32_t)kInclusive << 30) | (prefix + total));
     }
     sm.global_off[tid] = gbase[tid] + prefix - lbase;
-    sm.local_base[tid] = lbase;
   }
   __syncthreads();
 
-  // ---- reorder keys through LDS, then write each digit's run contiguously
-#pragma unroll
-  for (int i = 0; i < IPT; i++) {
-    const uint32_t d = (uint32_t)(encode_key<U, FLOAT>(k[i], xor_mask) >> shift) & 0xffu;
-    pos[i] += sm.local_base[d] + sm.wave_cnt[wave][d];
-    s_keys[pos[i]] = k[i];
-  }
-  __syncthreads();
+  // ---- write each digit's run contiguously
   uint32_t gpos[IPT];
 #pragma unroll
   for (int j = 0; j < IPT; j++) {
     const int li = j * BLOCK + tid;
     const U key = s_keys[li];
-    const uint32_t d = (uint32_t)(encode_key<U, FLOAT>(key, xor_mask) >> shift) & 0xffu;
-    gpos[j] = sm.global_off[d] + (uint32_t)li;
-    if (li < valid) kout[gpos[j]] = key;
+    gpos[j] = sm.global_off[digit_of(key)] + (uint32_t)li;
+    if (full || li < valid) kout[gpos[j]] = key;
   }
 
   if constexpr (VB > 0) {
@@ -267,14 +326,14 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const U* __restrict__ k
     for (int i = 0; i < IPT; i++) {
       const int li = slab + i * kWave;
       V v = V(0);
-      if (li < valid) v = vin[base + li];
+      if (full || li < valid) v = vin[base + li];
       s_vals[pos[i]] = v;
     }
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < IPT; j++) {
       const int li = j * BLOCK + tid;
-      if (li < valid) vout[gpos[j]] = s_vals[li];
+      if (full || li < valid) vout[gpos[j]] = s_vals[li];
     }
   }
 }
@@ -284,8 +343,24 @@ __global__ __launch_bounds__(BLOCK) void onesweep_kernel(const U* __restrict__ k
 // ---------------------------------------------------------------------------------------
 template <class U, int VB>
 struct SortConfig {
-  static constexpr int BLOCK = 256;
-  static constexpr int IPT = (sizeof(U) + VB > 8) ? 12 : 16;
+  // Tile shape by bytes moved per item (key + value), measured on MI355X at n = 2^28:
+  // large tiles shorten the look-back chains and lengthen the per-digit output runs; the
+  // limit is LDS (two workgroups per CU must fit) and registers.
+#ifndef TCD_SORT_A_BLOCK
+#define TCD_SORT_A_BLOCK 512
+#define TCD_SORT_A_IPT 24
+#endif
+#ifndef TCD_SORT_B_BLOCK
+#define TCD_SORT_B_BLOCK 1024
+#define TCD_SORT_B_IPT 16
+#endif
+#ifndef TCD_SORT_C_BLOCK
+#define TCD_SORT_C_BLOCK 1024
+#define TCD_SORT_C_IPT 12
+#endif
+  static constexpr int BYTES = (int)sizeof(U) + VB;
+  static constexpr int BLOCK = BYTES <= 4 ? TCD_SORT_A_BLOCK : (BYTES <= 8 ? TCD_SORT_B_BLOCK : TCD_SORT_C_BLOCK);
+  static constexpr int IPT = BYTES <= 4 ? TCD_SORT_A_IPT : (BYTES <= 8 ? TCD_SORT_B_IPT : TCD_SORT_C_IPT);
   static constexpr int TILE = BLOCK * IPT;
 };
 
