@@ -65,10 +65,14 @@ struct alignas(N * sizeof(E)) VecN {
 // CHUNKS chunks; VEC is set by the wider of key and value so that no access exceeds 16 B.
 template <class T>
 struct SegGeom {
-  static constexpr int BLOCK = 256;
+#ifndef TCD_SEG_BLOCK
+#define TCD_SEG_BLOCK 256
+#define TCD_SEG_CHUNKS 4
+#endif
+  static constexpr int BLOCK = TCD_SEG_BLOCK;
   static constexpr int WIDE = (int)(sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T));
   static constexpr int VEC = 16 / WIDE;
-  static constexpr int CHUNKS = WIDE == 8 ? 4 : (WIDE == 4 ? 4 : 2);
+  static constexpr int CHUNKS = WIDE >= 4 ? TCD_SEG_CHUNKS : 2;
   static constexpr int NWAVES = BLOCK / kWave;
   static constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
 };

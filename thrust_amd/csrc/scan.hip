@@ -139,8 +139,15 @@ __global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_
 
 template <class T>
 struct ScanConfig {
-  static constexpr int BLOCK = 256;
-  static constexpr int CHUNKS = 4;
+#ifndef TCD_SCAN_BLOCK
+#define TCD_SCAN_BLOCK 512
+#define TCD_SCAN_CHUNKS 8
+#endif
+  // 128 bytes per thread for 4- and 8-byte elements (64 KiB tiles: fewer tickets and look-backs
+  // per byte; measured best on MI355X); fewer chunks for narrow types, which hold one element
+  // per register.
+  static constexpr int BLOCK = TCD_SCAN_BLOCK;
+  static constexpr int CHUNKS = sizeof(T) >= 4 ? TCD_SCAN_CHUNKS : (sizeof(T) == 2 ? 4 : 2);
   static constexpr int64_t TILE = (int64_t)BLOCK * (16 / sizeof(T)) * CHUNKS;
   using P = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
 };
