@@ -1,0 +1,12 @@
+// Helpers shared by the public algorithm headers: unwrap contiguous device iterators and
+// classify an iterator as device or host.
+#pragma once
+#include <iterator>
+#include <thrust/device_ptr.h>
+namespace thrust { namespace detail {
+template <class T> inline T* unwrap(thrust::device_ptr<T> p) { return p.get(); }
+template <class T> inline T* unwrap(T* p) { return p; }  // raw device pointer under an explicit device policy
+template <class It> struct value_of { typedef typename std::iterator_traits<It>::value_type type; };
+template <class It> using enable_if_device = typename std::enable_if<system::cdna4::detail::is_device_iterator<It>::value, int>::type;
+template <class It> using enable_if_host = typename std::enable_if<!system::cdna4::detail::is_device_iterator<It>::value, int>::type;
+}}  // namespace thrust::detail

@@ -1,0 +1,92 @@
+// thrust::device_ptr / device_reference / device_pointer_cast / raw_pointer_cast
+// (thrust/device_ptr.h, thrust/device_reference.h).  Reading or writing through a
+// device_reference is one synchronous element copy, as in the reference
+// (thrust/system/cuda/detail/get_value.h:47-58, assign_value.h).
+#pragma once
+#include <cstddef>
+#include <iterator>
+#include <thrust/system/cdna4/detail/core.h>
+
+namespace thrust {
+
+template <class T> class device_ptr;
+
+template <class T>
+class device_reference {
+ public:
+  typedef typename std::remove_const<T>::type value_type;
+  explicit device_reference(T* p) : p_(p) {}
+  operator value_type() const {
+    value_type v;
+    system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_dtoh(&v, p_, sizeof(T), nullptr), "get_value");
+    system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "get_value");
+    return v;
+  }
+  device_reference& operator=(const value_type& v) {
+    system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_htod(p_, &v, sizeof(T), nullptr), "assign_value");
+    system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "assign_value");
+    return *this;
+  }
+  device_reference& operator=(const device_reference& o) { return *this = static_cast<value_type>(o); }
+  device_ptr<T> operator&() const { return device_ptr<T>(p_); }
+
+ private:
+  T* p_;
+};
+
+template <class T>
+class device_ptr {
+ public:
+  typedef std::random_access_iterator_tag iterator_category;
+  typedef typename std::remove_const<T>::type value_type;
+  typedef std::ptrdiff_t difference_type;
+  typedef device_ptr pointer;
+  typedef device_reference<T> reference;
+  typedef system::cdna4::tag system_tag;
+
+  device_ptr() : p_(nullptr) {}
+  explicit device_ptr(T* p) : p_(p) {}
+  template <class U, class = typename std::enable_if<std::is_convertible<U*, T*>::value>::type>
+  device_ptr(const device_ptr<U>& o) : p_(o.get()) {}
+  T* get() const { return p_; }
+  reference operator*() const { return reference(p_); }
+  reference operator[](difference_type i) const { return reference(p_ + i); }
+  device_ptr& operator++() { ++p_; return *this; }
+  device_ptr operator++(int) { device_ptr t(*this); ++p_; return t; }
+  device_ptr& operator--() { --p_; return *this; }
+  device_ptr operator--(int) { device_ptr t(*this); --p_; return t; }
+  device_ptr& operator+=(difference_type d) { p_ += d; return *this; }
+  device_ptr& operator-=(difference_type d) { p_ -= d; return *this; }
+  friend device_ptr operator+(device_ptr a, difference_type d) { return device_ptr(a.p_ + d); }
+  friend device_ptr operator+(difference_type d, device_ptr a) { return device_ptr(a.p_ + d); }
+  friend device_ptr operator-(device_ptr a, difference_type d) { return device_ptr(a.p_ - d); }
+  friend difference_type operator-(device_ptr a, device_ptr b) { return a.p_ - b.p_; }
+  friend bool operator==(device_ptr a, device_ptr b) { return a.p_ == b.p_; }
+  friend bool operator!=(device_ptr a, device_ptr b) { return a.p_ != b.p_; }
+  friend bool operator<(device_ptr a, device_ptr b) { return a.p_ < b.p_; }
+  friend bool operator>(device_ptr a, device_ptr b) { return a.p_ > b.p_; }
+  friend bool operator<=(device_ptr a, device_ptr b) { return a.p_ <= b.p_; }
+  friend bool operator>=(device_ptr a, device_ptr b) { return a.p_ >= b.p_; }
+
+ private:
+  T* p_;
+};
+
+template <class T> inline device_ptr<T> device_pointer_cast(T* p) { return device_ptr<T>(p); }
+template <class T> inline device_ptr<T> device_pointer_cast(device_ptr<T> p) { return p; }
+template <class T> inline T* raw_pointer_cast(device_ptr<T> p) { return p.get(); }
+template <class T> inline T* raw_pointer_cast(T* p) { return p; }
+
+// Cached, stream-ordered device allocation (thrust/device_malloc.h, device_free.h).
+template <class T> inline device_ptr<T> device_malloc(std::size_t n) {
+  return device_ptr<T>(static_cast<T*>(system::cdna4::detail::malloc_bytes(n * sizeof(T), nullptr)));
+}
+template <class T> inline void device_free(device_ptr<T> p) { system::cdna4::detail::free_bytes(p.get(), nullptr); }
+
+namespace system { namespace cdna4 { namespace detail {
+// Contiguous device iterators are unwrapped to raw pointers before the C ABI is called
+// (thrust/type_traits/is_contiguous_iterator.h:246-, try_unwrap_contiguous_iterator).
+template <class It> struct is_device_iterator { static constexpr bool value = false; };
+template <class T> struct is_device_iterator<thrust::device_ptr<T>> { static constexpr bool value = true; };
+}}}  // namespace system::cdna4::detail
+}  // namespace thrust

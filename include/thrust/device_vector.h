@@ -1,0 +1,139 @@
+// thrust::device_vector for arithmetic element types (thrust/device_vector.h,
+// thrust/detail/vector_base.h).  Storage comes from the library's cached allocator; value
+// initialisation and fills run as typed fill kernels, transfers as async copies followed by
+// a stream synchronise (thrust/system/cuda/detail/util.h:142-199), so a TU that uses
+// device_vector needs no device compiler.
+#pragma once
+#include <algorithm>
+#include <cstddef>
+#include <initializer_list>
+#include <vector>
+
+#include <thrust/device_ptr.h>
+#include <thrust/host_vector.h>
+
+namespace thrust {
+
+template <class T>
+class device_vector {
+  static_assert(std::is_arithmetic<T>::value, "device_vector of the cdna4 system holds arithmetic types");
+  static_assert(sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8, "unsupported element size");
+  typedef system::cdna4::detail::temporary_storage storage_unused;
+
+ public:
+  typedef T value_type;
+  typedef std::size_t size_type;
+  typedef device_ptr<T> iterator;
+  typedef device_ptr<const T> const_iterator;
+  typedef device_ptr<T> pointer;
+  typedef device_reference<T> reference;
+  typedef device_reference<const T> const_reference;
+
+  device_vector() : p_(nullptr), n_(0), cap_(0) {}
+  explicit device_vector(size_type n) : device_vector() { resize(n); }
+  device_vector(size_type n, const T& v) : device_vector() { assign(n, v); }
+  device_vector(const device_vector& o) : device_vector() { assign_device(o.p_, o.n_); }
+  device_vector(device_vector&& o) noexcept : p_(o.p_), n_(o.n_), cap_(o.cap_) { o.p_ = nullptr; o.n_ = o.cap_ = 0; }
+  template <class A> device_vector(const std::vector<T, A>& h) : device_vector() { assign_host(h.data(), h.size()); }
+  device_vector(std::initializer_list<T> il) : device_vector() { assign_host(il.begin(), il.size()); }
+  template <class It, class = typename std::iterator_traits<It>::iterator_category>
+  device_vector(It first, It last) : device_vector() { assign(first, last); }
+  ~device_vector() { release(); }
+
+  device_vector& operator=(const device_vector& o) { if (this != &o) assign_device(o.p_, o.n_); return *this; }
+  device_vector& operator=(device_vector&& o) noexcept { swap(o); return *this; }
+  template <class A> device_vector& operator=(const std::vector<T, A>& h) { assign_host(h.data(), h.size()); return *this; }
+
+  iterator begin() { return iterator(p_); }
+  iterator end() { return iterator(p_ + n_); }
+  const_iterator begin() const { return const_iterator(p_); }
+  const_iterator end() const { return const_iterator(p_ + n_); }
+  const_iterator cbegin() const { return begin(); }
+  const_iterator cend() const { return end(); }
+  pointer data() { return pointer(p_); }
+  device_ptr<const T> data() const { return device_ptr<const T>(p_); }
+  size_type size() const { return n_; }
+  size_type capacity() const { return cap_; }
+  bool empty() const { return n_ == 0; }
+  reference operator[](size_type i) { return reference(p_ + i); }
+  const_reference operator[](size_type i) const { return const_reference(p_ + i); }
+  reference front() { return (*this)[0]; }
+  reference back() { return (*this)[n_ - 1]; }
+
+  void clear() { n_ = 0; }
+  void swap(device_vector& o) noexcept { std::swap(p_, o.p_); std::swap(n_, o.n_); std::swap(cap_, o.cap_); }
+  void reserve(size_type c) { if (c > cap_) regrow(c); }
+  void resize(size_type n) { resize(n, T()); }
+  void resize(size_type n, const T& v) {
+    if (n > cap_) regrow(n);
+    if (n > n_) fill_raw(p_ + n_, n - n_, v);
+    n_ = n;
+  }
+  void assign(size_type n, const T& v) { n_ = 0; if (n > cap_) regrow(n); fill_raw(p_, n, v); n_ = n; }
+  template <class It, class = typename std::iterator_traits<It>::iterator_category>
+  void assign(It first, It last) { assign_range(first, last, typename std::is_same<It, iterator>::type()); }
+  void push_back(const T& v) {
+    if (n_ == cap_) regrow(cap_ ? 2 * cap_ : 16);
+    fill_raw(p_ + n_, 1, v);
+    ++n_;
+  }
+
+  friend bool operator==(const device_vector& a, const device_vector& b) {
+    return host_vector<T>(a) == host_vector<T>(b);
+  }
+  friend bool operator!=(const device_vector& a, const device_vector& b) { return !(a == b); }
+
+ private:
+  static void check(int rc, const char* what) { system::cdna4::detail::throw_on_error(rc, what); }
+  static void sync() { check(thrust_cdna4_stream_synchronize(nullptr), "device_vector: synchronize"); }
+  void release() { if (p_) system::cdna4::detail::free_bytes(p_, nullptr); p_ = nullptr; n_ = cap_ = 0; }
+  void regrow(size_type c) {
+    T* q = static_cast<T*>(system::cdna4::detail::malloc_bytes(c * sizeof(T), nullptr));
+    if (n_) { check(thrust_cdna4_memcpy_dtod(q, p_, n_ * sizeof(T), nullptr), "device_vector: copy"); sync(); }
+    if (p_) system::cdna4::detail::free_bytes(p_, nullptr);
+    p_ = q;
+    cap_ = c;
+  }
+  static void fill_raw(T* dst, size_type n, const T& v) {
+    if (!n) return;
+    check(thrust_cdna4_fill(dst, &v, (int)sizeof(T), (int64_t)n, nullptr), "device_vector: fill");
+    sync();
+  }
+  void assign_host(const T* h, size_type n) {
+    n_ = 0;
+    if (n > cap_) regrow(n);
+    if (n) { check(thrust_cdna4_memcpy_htod(p_, h, n * sizeof(T), nullptr), "device_vector: copy from host"); sync(); }
+    n_ = n;
+  }
+  void assign_device(const T* d, size_type n) {
+    n_ = 0;
+    if (n > cap_) regrow(n);
+    if (n) { check(thrust_cdna4_memcpy_dtod(p_, d, n * sizeof(T), nullptr), "device_vector: copy"); sync(); }
+    n_ = n;
+  }
+  template <class It> void assign_range(It first, It last, std::true_type) { assign_device(first.get(), (size_type)(last - first)); }
+  template <class It> void assign_range(It first, It last, std::false_type) {
+    std::vector<T> tmp(first, last);
+    assign_host(tmp.data(), tmp.size());
+  }
+
+  T* p_;
+  size_type n_, cap_;
+};
+
+template <class T, class A>
+host_vector<T, A>::host_vector(const device_vector<T>& d) : base(d.size()) {
+  if (d.size()) {
+    system::cdna4::detail::throw_on_error(
+        thrust_cdna4_memcpy_dtoh(this->data(), d.begin().get(), d.size() * sizeof(T), nullptr), "copy to host");
+    system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "copy to host");
+  }
+}
+template <class T, class A>
+host_vector<T, A>& host_vector<T, A>::operator=(const device_vector<T>& d) {
+  host_vector tmp(d);
+  this->swap(tmp);
+  return *this;
+}
+
+}  // namespace thrust

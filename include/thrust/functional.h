@@ -1,0 +1,38 @@
+// Function objects the device kernels are specialised on (thrust/functional.h).
+#pragma once
+#include <functional>
+namespace thrust {
+template <class T = void> struct plus { constexpr T operator()(const T& a, const T& b) const { return a + b; } };
+template <class T = void> struct multiplies { constexpr T operator()(const T& a, const T& b) const { return a * b; } };
+template <class T = void> struct maximum { constexpr T operator()(const T& a, const T& b) const { return a < b ? b : a; } };
+template <class T = void> struct minimum { constexpr T operator()(const T& a, const T& b) const { return a < b ? a : b; } };
+template <class T = void> struct less { constexpr bool operator()(const T& a, const T& b) const { return a < b; } };
+template <class T = void> struct greater { constexpr bool operator()(const T& a, const T& b) const { return a > b; } };
+template <class T = void> struct equal_to { constexpr bool operator()(const T& a, const T& b) const { return a == b; } };
+template <class T = void> struct identity { constexpr const T& operator()(const T& a) const { return a; } };
+
+// transparent forms (thrust::plus<> etc.)
+template <> struct plus<void> { template <class A, class B> constexpr auto operator()(const A& a, const B& b) const -> decltype(a + b) { return a + b; } };
+template <> struct multiplies<void> { template <class A, class B> constexpr auto operator()(const A& a, const B& b) const -> decltype(a * b) { return a * b; } };
+template <> struct maximum<void> { template <class A> constexpr A operator()(const A& a, const A& b) const { return a < b ? b : a; } };
+template <> struct minimum<void> { template <class A> constexpr A operator()(const A& a, const A& b) const { return a < b ? a : b; } };
+template <> struct less<void> { template <class A, class B> constexpr bool operator()(const A& a, const B& b) const { return a < b; } };
+template <> struct greater<void> { template <class A, class B> constexpr bool operator()(const A& a, const B& b) const { return a > b; } };
+template <> struct equal_to<void> { template <class A, class B> constexpr bool operator()(const A& a, const B& b) const { return a == b; } };
+
+namespace system { namespace cdna4 { namespace detail {
+// C-ABI operator code of a functor type, or -1 when no kernel exists for it.
+template <class F> struct op_code { static constexpr int value = -1; };
+template <class T> struct op_code<thrust::plus<T>> { static constexpr int value = 0; };
+template <class T> struct op_code<thrust::multiplies<T>> { static constexpr int value = 1; };
+template <class T> struct op_code<thrust::maximum<T>> { static constexpr int value = 2; };
+template <class T> struct op_code<thrust::minimum<T>> { static constexpr int value = 3; };
+// 0 = ascending (less), 1 = descending (greater), -1 = not a radix-sortable comparator
+// (thrust/system/cuda/detail/sort.h:389-395, can_use_primitive_sort).
+template <class F> struct order_code { static constexpr int value = -1; };
+template <class T> struct order_code<thrust::less<T>> { static constexpr int value = 0; };
+template <class T> struct order_code<thrust::greater<T>> { static constexpr int value = 1; };
+template <class F> struct is_equal_to { static constexpr bool value = false; };
+template <class T> struct is_equal_to<thrust::equal_to<T>> { static constexpr bool value = true; };
+}}}  // namespace system::cdna4::detail
+}  // namespace thrust

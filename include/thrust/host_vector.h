@@ -1,0 +1,17 @@
+// thrust::host_vector (thrust/host_vector.h): a std::vector in host memory.
+#pragma once
+#include <vector>
+namespace thrust {
+template <class T> class device_vector;
+template <class T, class Alloc = std::allocator<T>>
+class host_vector : public std::vector<T, Alloc> {
+  typedef std::vector<T, Alloc> base;
+
+ public:
+  using base::base;
+  host_vector() = default;
+  host_vector(const base& v) : base(v) {}
+  host_vector(const device_vector<T>& d);
+  host_vector& operator=(const device_vector<T>& d);
+};
+}  // namespace thrust

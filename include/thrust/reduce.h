@@ -1,0 +1,84 @@
+// thrust::reduce_by_key (thrust/reduce.h:691-).  Device ranges go to the single-pass
+// segmented-reduction kernel; host ranges run the sequential loop
+// (thrust/system/detail/sequential/reduce_by_key.h:43-95).
+#pragma once
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/pair.h>
+#include <thrust/scan.h>
+#include <thrust/system/cdna4/detail/algorithms.h>
+
+namespace thrust {
+
+// ---- device
+template <class D, class KIt, class VIt, class KOut, class VOut, class Pred, class Op>
+pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
+                               KOut kout, VOut vout, Pred, Op) {
+  typedef typename detail::elem<KIt>::type K;
+  typedef typename detail::elem<VIt>::type V;
+  static_assert(std::is_same<K, typename detail::elem<KOut>::type>::value &&
+                std::is_same<V, typename detail::elem<VOut>::type>::value,
+                "cdna4 reduce_by_key: output element types must match the input's");
+  const std::int64_t runs = system::cdna4::detail::reduce_by_key(
+      exec.derived(), (const K*)detail::unwrap(kfirst), (const V*)detail::unwrap(vfirst), detail::unwrap(kout),
+      detail::unwrap(vout), (std::int64_t)(klast - kfirst), typename detail::rebind_op<Pred, K>::type(),
+      typename detail::rebind_op<Op, V>::type());
+  return thrust::make_pair(kout + runs, vout + runs);
+}
+template <class D, class KIt, class VIt, class KOut, class VOut, class Pred>
+pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred p) {
+  return reduce_by_key(exec, kf, kl, vf, ko, vo, p, plus<typename detail::elem<VIt>::type>());
+}
+template <class D, class KIt, class VIt, class KOut, class VOut>
+pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo) {
+  return reduce_by_key(exec, kf, kl, vf, ko, vo, equal_to<typename detail::elem<KIt>::type>());
+}
+
+// ---- host
+template <class KIt, class VIt, class KOut, class VOut, class Pred, class Op>
+pair<KOut, VOut> reduce_by_key(const system::cpp::detail::par_t&, KIt kfirst, KIt klast, VIt vfirst, KOut kout,
+                               VOut vout, Pred pred, Op op) {
+  typedef typename detail::elem<KIt>::type K;
+  typedef typename detail::elem<VIt>::type V;
+  if (kfirst != klast) {
+    K temp_key = *kfirst;
+    V temp_value = *vfirst;
+    for (++kfirst, ++vfirst; kfirst != klast; ++kfirst, ++vfirst) {
+      K key = *kfirst;
+      V value = *vfirst;
+      if (pred(temp_key, key)) {
+        temp_value = op(temp_value, value);
+      } else {
+        *kout = temp_key; *vout = temp_value;
+        ++kout; ++vout;
+        temp_key = key; temp_value = value;
+      }
+    }
+    *kout = temp_key; *vout = temp_value;
+    ++kout; ++vout;
+  }
+  return thrust::make_pair(kout, vout);
+}
+template <class KIt, class VIt, class KOut, class VOut, class Pred>
+pair<KOut, VOut> reduce_by_key(const system::cpp::detail::par_t& e, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred p) {
+  return reduce_by_key(e, kf, kl, vf, ko, vo, p, plus<typename detail::elem<VIt>::type>());
+}
+template <class KIt, class VIt, class KOut, class VOut>
+pair<KOut, VOut> reduce_by_key(const system::cpp::detail::par_t& e, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo) {
+  return reduce_by_key(e, kf, kl, vf, ko, vo, equal_to<typename detail::elem<KIt>::type>());
+}
+
+// ---- no policy
+#define THRUST_CDNA4_RBK(SYS, COND)                                                                                 \
+  template <class K, class V, class KO, class VO, COND<K> = 0>                                                       \
+  pair<KO, VO> reduce_by_key(K kf, K kl, V vf, KO ko, VO vo) { return reduce_by_key(SYS, kf, kl, vf, ko, vo); }       \
+  template <class K, class V, class KO, class VO, class P, COND<K> = 0>                                              \
+  pair<KO, VO> reduce_by_key(K kf, K kl, V vf, KO ko, VO vo, P p) { return reduce_by_key(SYS, kf, kl, vf, ko, vo, p); } \
+  template <class K, class V, class KO, class VO, class P, class O, COND<K> = 0>                                     \
+  pair<KO, VO> reduce_by_key(K kf, K kl, V vf, KO ko, VO vo, P p, O o) { return reduce_by_key(SYS, kf, kl, vf, ko, vo, p, o); }
+THRUST_CDNA4_RBK(device, detail::enable_if_device)
+THRUST_CDNA4_RBK(host, detail::enable_if_host)
+#undef THRUST_CDNA4_RBK
+
+}  // namespace thrust

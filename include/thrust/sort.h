@@ -1,0 +1,96 @@
+// thrust::sort / stable_sort / sort_by_key / stable_sort_by_key (thrust/sort.h:77-925).
+// Device ranges (device_vector iterators, device_ptr, or raw pointers under a device policy)
+// go to the radix-sort kernels; host ranges are sorted on the host.
+#pragma once
+#include <algorithm>
+#include <numeric>
+#include <vector>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/system/cdna4/detail/algorithms.h>
+
+namespace thrust {
+
+// ---- device, explicit policy ---------------------------------------------------------
+template <class D, class It, class Compare>
+void stable_sort(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) {
+  system::cdna4::detail::sort_keys(exec.derived(), detail::unwrap(first), (std::int64_t)(last - first), comp);
+}
+template <class D, class It>
+void stable_sort(const system::cdna4::execution_policy<D>& exec, It first, It last) {
+  stable_sort(exec, first, last, less<typename detail::value_of<It>::type>());
+}
+// sort forwards to stable_sort, as the generic layer does (thrust/system/detail/generic/sort.inl:56-62)
+template <class D, class It, class Compare>
+void sort(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) { stable_sort(exec, first, last, comp); }
+template <class D, class It>
+void sort(const system::cdna4::execution_policy<D>& exec, It first, It last) { stable_sort(exec, first, last); }
+
+template <class D, class KIt, class VIt, class Compare>
+void stable_sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
+  system::cdna4::detail::sort_pairs(exec.derived(), detail::unwrap(kfirst), detail::unwrap(vfirst),
+                                    (std::int64_t)(klast - kfirst), comp);
+}
+template <class D, class KIt, class VIt>
+void stable_sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst) {
+  stable_sort_by_key(exec, kfirst, klast, vfirst, less<typename detail::value_of<KIt>::type>());
+}
+template <class D, class KIt, class VIt, class Compare>
+void sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
+  stable_sort_by_key(exec, kfirst, klast, vfirst, comp);
+}
+template <class D, class KIt, class VIt>
+void sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst) {
+  stable_sort_by_key(exec, kfirst, klast, vfirst);
+}
+
+// ---- host, explicit policy -----------------------------------------------------------
+template <class It, class Compare>
+void stable_sort(const system::cpp::detail::par_t&, It first, It last, Compare comp) { std::stable_sort(first, last, comp); }
+template <class It>
+void stable_sort(const system::cpp::detail::par_t&, It first, It last) { std::stable_sort(first, last); }
+template <class It, class Compare>
+void sort(const system::cpp::detail::par_t&, It first, It last, Compare comp) { std::stable_sort(first, last, comp); }
+template <class It>
+void sort(const system::cpp::detail::par_t&, It first, It last) { std::stable_sort(first, last); }
+template <class KIt, class VIt, class Compare>
+void stable_sort_by_key(const system::cpp::detail::par_t&, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
+  typedef typename detail::value_of<KIt>::type K;
+  typedef typename detail::value_of<VIt>::type V;
+  const std::size_t n = (std::size_t)(klast - kfirst);
+  std::vector<std::size_t> idx(n);
+  std::iota(idx.begin(), idx.end(), std::size_t(0));
+  std::vector<K> k(kfirst, klast);
+  std::vector<V> v(vfirst, vfirst + n);
+  std::stable_sort(idx.begin(), idx.end(), [&](std::size_t a, std::size_t b) { return comp(k[a], k[b]); });
+  for (std::size_t i = 0; i < n; i++) { kfirst[i] = k[idx[i]]; vfirst[i] = v[idx[i]]; }
+}
+template <class KIt, class VIt>
+void stable_sort_by_key(const system::cpp::detail::par_t& e, KIt kfirst, KIt klast, VIt vfirst) {
+  stable_sort_by_key(e, kfirst, klast, vfirst, less<typename detail::value_of<KIt>::type>());
+}
+template <class KIt, class VIt, class Compare>
+void sort_by_key(const system::cpp::detail::par_t& e, KIt kfirst, KIt klast, VIt vfirst, Compare comp) { stable_sort_by_key(e, kfirst, klast, vfirst, comp); }
+template <class KIt, class VIt>
+void sort_by_key(const system::cpp::detail::par_t& e, KIt kfirst, KIt klast, VIt vfirst) { stable_sort_by_key(e, kfirst, klast, vfirst); }
+
+// ---- no policy: the iterator's system decides (thrust/detail/sort.inl:202-339) --------
+#define THRUST_CDNA4_SORT_DISPATCH(NAME)                                                                         \
+  template <class It, detail::enable_if_device<It> = 0> void NAME(It f, It l) { NAME(device, f, l); }              \
+  template <class It, class C, detail::enable_if_device<It> = 0> void NAME(It f, It l, C c) { NAME(device, f, l, c); } \
+  template <class It, detail::enable_if_host<It> = 0> void NAME(It f, It l) { NAME(host, f, l); }                  \
+  template <class It, class C, detail::enable_if_host<It> = 0> void NAME(It f, It l, C c) { NAME(host, f, l, c); }
+THRUST_CDNA4_SORT_DISPATCH(sort)
+THRUST_CDNA4_SORT_DISPATCH(stable_sort)
+#undef THRUST_CDNA4_SORT_DISPATCH
+#define THRUST_CDNA4_SORT_BY_KEY_DISPATCH(NAME)                                                                  \
+  template <class K, class V, detail::enable_if_device<K> = 0> void NAME(K f, K l, V v) { NAME(device, f, l, v); }  \
+  template <class K, class V, class C, detail::enable_if_device<K> = 0> void NAME(K f, K l, V v, C c) { NAME(device, f, l, v, c); } \
+  template <class K, class V, detail::enable_if_host<K> = 0> void NAME(K f, K l, V v) { NAME(host, f, l, v); }      \
+  template <class K, class V, class C, detail::enable_if_host<K> = 0> void NAME(K f, K l, V v, C c) { NAME(host, f, l, v, c); }
+THRUST_CDNA4_SORT_BY_KEY_DISPATCH(sort_by_key)
+THRUST_CDNA4_SORT_BY_KEY_DISPATCH(stable_sort_by_key)
+#undef THRUST_CDNA4_SORT_BY_KEY_DISPATCH
+
+}  // namespace thrust

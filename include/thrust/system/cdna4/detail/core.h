@@ -1,0 +1,212 @@
+// Core of the cdna4 device system: execution policies, error mapping, element-type traits
+// and temporary storage.  Everything here is host code that calls the C ABI of
+// libthrust_cdna4.so; a translation unit that includes it builds with a plain C++14 host
+// compiler, no device compiler needed.
+//
+// Mirrors, for this system:
+//   thrust/system/cuda/detail/execution_policy.h:48-71   (tag, execution_policy<Derived>)
+//   thrust/system/cuda/detail/par.h:44-238               (par, par.on(stream), par_nosync)
+//   thrust/system/cuda/detail/util.h:46-140, :207-292    (stream(), synchronize_optional(), throw_on_error())
+//   thrust/system/cuda/detail/malloc_and_free.h:53-116   (malloc / free)
+//   thrust/detail/temporary_array.h:50-111               (algorithm-scoped temporary storage)
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <new>
+#include <string>
+#include <system_error>
+#include <type_traits>
+
+#include "thrust_cdna4.h"
+
+#define THRUST_CDNA4_SYSTEM 1
+// The version of the API surface this layer mirrors (Thrust 2.2.0).
+#define THRUST_VERSION 200200
+#define THRUST_DEVICE_SYSTEM_CDNA4 5
+#define THRUST_DEVICE_SYSTEM THRUST_DEVICE_SYSTEM_CDNA4
+
+namespace thrust {
+
+// ------------------------------------------------------------------------------------
+// Errors: thrust::system_error with a hip error category; thrust::system::detail::bad_alloc
+// for allocation failures (thrust/system/cuda/detail/malloc_and_free.h:79-83).
+// ------------------------------------------------------------------------------------
+using system_error = std::system_error;
+using error_code = std::error_code;
+using error_category = std::error_category;
+
+namespace system {
+namespace detail {
+class bad_alloc : public std::bad_alloc {
+ public:
+  explicit bad_alloc(const std::string& w) : what_("std::bad_alloc: " + w) {}
+  const char* what() const noexcept override { return what_.c_str(); }
+
+ private:
+  std::string what_;
+};
+}  // namespace detail
+
+namespace cdna4 {
+namespace detail {
+class hip_error_category : public std::error_category {
+ public:
+  const char* name() const noexcept override { return "cdna4"; }
+  std::string message(int ev) const override { return thrust_cdna4_error_string(ev); }
+};
+}  // namespace detail
+}  // namespace cdna4
+}  // namespace system
+
+inline const error_category& cdna4_category() {
+  static system::cdna4::detail::hip_error_category cat;
+  return cat;
+}
+
+namespace system {
+namespace cdna4 {
+
+// ------------------------------------------------------------------------------------
+// Execution policies
+// ------------------------------------------------------------------------------------
+struct tag {};
+
+template <class Derived>
+struct execution_policy {
+  typedef tag tag_type;
+  operator tag() const { return tag(); }
+  const Derived& derived() const { return static_cast<const Derived&>(*this); }
+};
+
+namespace detail {
+
+struct execute_on_stream : execution_policy<execute_on_stream> {
+  void* stream_;
+  bool sync_;
+  execute_on_stream(void* s, bool sync) : stream_(s), sync_(sync) {}
+};
+
+// thrust::device / thrust::cdna4::par: work goes to the legacy default stream and the call
+// returns after it has completed (thrust/system/cuda/detail/util.h:46-55, :113-140).
+struct par_t : execution_policy<par_t> {
+  execute_on_stream on(void* stream) const { return execute_on_stream(stream, true); }
+};
+// par_nosync: the call may return before the work has completed, except where a result has
+// to be read back (thrust/system/cuda/detail/par.h:102-107, :181-186).
+struct par_nosync_t : execution_policy<par_nosync_t> {
+  execute_on_stream on(void* stream) const { return execute_on_stream(stream, false); }
+};
+
+inline void* stream_of(const par_t&) { return nullptr; }
+inline void* stream_of(const par_nosync_t&) { return nullptr; }
+inline void* stream_of(const execute_on_stream& p) { return p.stream_; }
+inline bool must_sync(const par_t&) { return true; }
+inline bool must_sync(const par_nosync_t&) { return false; }
+inline bool must_sync(const execute_on_stream& p) { return p.sync_; }
+
+// Clears nothing on success; on failure throws thrust::system_error with the hip code
+// (thrust/system/cuda/detail/util.h:207-292).
+inline void throw_on_error(int status, const char* msg) {
+  if (status != 0) throw thrust::system_error(status, thrust::cdna4_category(), msg);
+}
+
+template <class Policy>
+inline void synchronize(const Policy& p, const char* msg) {
+  throw_on_error(thrust_cdna4_stream_synchronize(stream_of(p)), msg);
+}
+template <class Policy>
+inline void synchronize_optional(const Policy& p, const char* msg) {
+  if (must_sync(p)) synchronize(p, msg);
+}
+
+// ------------------------------------------------------------------------------------
+// Element types the kernels are built for.  Anything else is rejected at compile time:
+// there is no fallback that would run a device algorithm on the host.
+// ------------------------------------------------------------------------------------
+template <class T, class = void>
+struct dtype_of {
+  static constexpr bool supported = false;
+  static constexpr int value = -1;
+};
+template <class T>
+struct dtype_of<T, typename std::enable_if<std::is_integral<T>::value && !std::is_same<T, bool>::value>::type> {
+  static constexpr bool supported = sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8;
+  static constexpr int value =
+      sizeof(T) == 1 ? (std::is_signed<T>::value ? THRUST_CDNA4_I8 : THRUST_CDNA4_U8)
+    : sizeof(T) == 2 ? (std::is_signed<T>::value ? THRUST_CDNA4_I16 : THRUST_CDNA4_U16)
+    : sizeof(T) == 4 ? (std::is_signed<T>::value ? THRUST_CDNA4_I32 : THRUST_CDNA4_U32)
+                     : (std::is_signed<T>::value ? THRUST_CDNA4_I64 : THRUST_CDNA4_U64);
+};
+template <>
+struct dtype_of<float, void> {
+  static constexpr bool supported = true;
+  static constexpr int value = THRUST_CDNA4_F32;
+};
+template <>
+struct dtype_of<double, void> {
+  static constexpr bool supported = true;
+  static constexpr int value = THRUST_CDNA4_F64;
+};
+
+// ------------------------------------------------------------------------------------
+// Memory: cached, stream-ordered allocation through the library's pool.
+// ------------------------------------------------------------------------------------
+inline void* malloc_bytes(std::size_t bytes, void* stream) {
+  void* p = nullptr;
+  const int rc = thrust_cdna4_malloc(&p, bytes, stream);
+  if (rc != 0) throw thrust::system::detail::bad_alloc(thrust_cdna4_error_string(rc));
+  return p;
+}
+inline void free_bytes(void* p, void* stream) noexcept { (void)thrust_cdna4_free(p, stream); }
+
+// Byte buffer that lives for one algorithm call (thrust::detail::temporary_array<uint8_t>).
+class temporary_storage {
+ public:
+  temporary_storage(std::size_t bytes, void* stream) : stream_(stream), bytes_(bytes), ptr_(nullptr) {
+    if (bytes_) ptr_ = malloc_bytes(bytes_, stream_);
+  }
+  ~temporary_storage() {
+    if (ptr_) free_bytes(ptr_, stream_);
+  }
+  temporary_storage(const temporary_storage&) = delete;
+  temporary_storage& operator=(const temporary_storage&) = delete;
+  void* data() const { return ptr_; }
+  std::size_t size() const { return bytes_; }
+
+ private:
+  void* stream_;
+  std::size_t bytes_;
+  void* ptr_;
+};
+
+}  // namespace detail
+
+static const detail::par_t par;
+static const detail::par_nosync_t par_nosync;
+
+}  // namespace cdna4
+}  // namespace system
+
+namespace cdna4 {
+using thrust::system::cdna4::execution_policy;
+using thrust::system::cdna4::par;
+using thrust::system::cdna4::par_nosync;
+using thrust::system::cdna4::tag;
+}  // namespace cdna4
+
+// Host system: the sequential implementations in this layer run for host_vector and raw
+// host ranges under thrust::host (the counterpart of THRUST_HOST_SYSTEM_CPP).
+namespace system {
+namespace cpp {
+struct tag {};
+namespace detail {
+struct par_t {};
+}  // namespace detail
+}  // namespace cpp
+}  // namespace system
+
+static const system::cdna4::detail::par_t device;
+static const system::cpp::detail::par_t host;
+
+}  // namespace thrust

@@ -1,0 +1,77 @@
+"""CPU-only: user code written against the Thrust API surface builds with a plain host
+compiler against include/thrust (no device compiler in the user's build), and the headers
+refuse what the device system has no kernel for instead of falling back to the host."""
+import os
+import subprocess
+import textwrap
+
+from conftest import ROOT
+
+INC = os.path.join(ROOT, "include")
+
+
+def compile_snippet(tmp_path, body, extra=()):
+    src = tmp_path / "t.cpp"
+    src.write_text(textwrap.dedent(body))
+    return subprocess.run(["g++", "-std=c++14", "-fsyntax-only", "-I", INC, *extra, str(src)],
+                          capture_output=True, text=True)
+
+
+def test_cpp_tests_compile_with_gxx():
+    r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    for name in ["test_sort", "test_scan", "test_by_key", "test_system"]:
+        assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
+
+
+def test_existing_thrust_code_compiles_unchanged(tmp_path):
+    r = compile_snippet(tmp_path, """
+        #include <thrust/device_vector.h>
+        #include <thrust/host_vector.h>
+        #include <thrust/execution_policy.h>
+        #include <thrust/sort.h>
+        #include <thrust/scan.h>
+        #include <thrust/reduce.h>
+        #include <thrust/functional.h>
+        int main() {
+          thrust::host_vector<int> h(1000);
+          thrust::device_vector<int> d = h, o(1000), k(1000), v(1000);
+          thrust::sort(d.begin(), d.end());
+          thrust::sort(thrust::device, d.begin(), d.end(), thrust::greater<int>());
+          thrust::sort_by_key(d.begin(), d.end(), o.begin());
+          thrust::inclusive_scan(thrust::device, d.begin(), d.end(), o.begin());
+          thrust::exclusive_scan(d.begin(), d.end(), o.begin(), 0, thrust::plus<int>());
+          thrust::inclusive_scan_by_key(d.begin(), d.end(), o.begin(), v.begin());
+          auto e = thrust::reduce_by_key(d.begin(), d.end(), o.begin(), k.begin(), v.begin());
+          return (int)(e.first - k.begin());
+        }""")
+    assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_headers_shadow_any_other_thrust(tmp_path):
+    # /opt/rocm/include also holds a <thrust/...>; with -I include first ours must win
+    r = compile_snippet(tmp_path, """
+        #include <thrust/version.h>
+        #include <thrust/sort.h>
+        static_assert(THRUST_CDNA4_VERSION >= 100, "resolved to a foreign thrust");
+        int main() { return 0; }""", extra=("-isystem", "/opt/rocm/include"))
+    assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_unsupported_comparator_is_a_compile_error_not_a_host_fallback(tmp_path):
+    r = compile_snippet(tmp_path, """
+        #include <thrust/device_vector.h>
+        #include <thrust/sort.h>
+        struct by_mod3 { bool operator()(int a, int b) const { return a % 3 < b % 3; } };
+        int main() { thrust::device_vector<int> d(10); thrust::sort(d.begin(), d.end(), by_mod3()); }""")
+    assert r.returncode != 0
+    assert "radix kernel" in r.stderr
+
+
+def test_exclusive_scan_init_type_must_be_the_element_type(tmp_path):
+    r = compile_snippet(tmp_path, """
+        #include <thrust/device_vector.h>
+        #include <thrust/scan.h>
+        int main() { thrust::device_vector<float> d(10), o(10); thrust::exclusive_scan(d.begin(), d.end(), o.begin(), 0); }""")
+    assert r.returncode != 0
+    assert "accumulator type" in r.stderr
