@@ -19,6 +19,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+# measured HBM traffic of one onesweep launch over 2^28 uint32 keys
+# (profiles/onesweep_u32_sort_2p28_and_extras.md)
+ONESWEEP_U32_TRAFFIC_BYTES = 2.463e9
 
 
 def parse():
@@ -308,7 +311,10 @@ def main():
                    "whole_sort_roofline_frac": round(sort_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": "onesweep_kernel<uint32, keys only>",
                      "achieved": round(onesweep_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(onesweep_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(onesweep_gbs / HBM_PEAK_GBS, 4),
+                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000),
+                     # scale factors from a plain 1 GiB copy; summary under profiles/ (n = 2^28 only)
+                     "traffic": ONESWEEP_U32_TRAFFIC_BYTES if args.log2n == 28 else None,
                      "avg_launch_ms": round(onesweep_ms, 4), "launches_timed": onesweep_launches,
                      "algorithmic_bytes_per_launch": onesweep_bytes},
         "cpu_baseline": cpu,
