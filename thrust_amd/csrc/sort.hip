@@ -23,7 +23,10 @@ constexpr int kRadix = 1 << kRadixBits;
 
 // descriptor word: status in bits 31:30, count in bits 29:0
 constexpr uint32_t kCountMask = (1u << 30) - 1;
-constexpr int kLookW = 4;  // look-back descriptors loaded per round trip
+#ifndef TCD_SORT_LOOKW
+#define TCD_SORT_LOOKW 4
+#endif
+constexpr int kLookW = TCD_SORT_LOOKW;  // look-back descriptors loaded per round trip
 
 template <int BYTES>
 struct uint_of;
@@ -151,15 +154,21 @@ struct OnesweepSmem {
 // Per bit: one v_bfe_i32 (0 / -1 per lane), one v_cmp (the ballot, an SGPR pair) and one
 // three-input bit operation per half:  m &= ~(ballot ^ bit)   (truth table 0x90).
 __device__ inline void match_digit(uint32_t d, uint32_t& m_lo, uint32_t& m_hi) {
+  int32_t e[kRadixBits];
+  uint64_t bal[kRadixBits];
+#pragma unroll
+  for (int b = 0; b < kRadixBits; b++) {
+    e[b] = __builtin_amdgcn_sbfe((int)d, b, 1);
+    asm("" : "+v"(e[b]));  // keep the compare on e itself instead of a second bit extraction
+  }
+#pragma unroll
+  for (int b = 0; b < kRadixBits; b++) bal[b] = __builtin_amdgcn_ballot_w64(e[b] != 0);
   m_lo = ~0u;
   m_hi = ~0u;
 #pragma unroll
   for (int b = 0; b < kRadixBits; b++) {
-    int32_t e = __builtin_amdgcn_sbfe((int)d, b, 1);
-    asm("" : "+v"(e));  // keep the compare on e itself instead of a second bit extraction
-    const uint64_t bal = __builtin_amdgcn_ballot_w64(e != 0);
-    m_lo = __builtin_amdgcn_bitop3_b32(m_lo, (uint32_t)bal, (uint32_t)e, 0x90);
-    m_hi = __builtin_amdgcn_bitop3_b32(m_hi, (uint32_t)(bal >> 32), (uint32_t)e, 0x90);
+    m_lo = __builtin_amdgcn_bitop3_b32(m_lo, (uint32_t)bal[b], (uint32_t)e[b], 0x90);
+    m_hi = __builtin_amdgcn_bitop3_b32(m_hi, (uint32_t)(bal[b] >> 32), (uint32_t)e[b], 0x90);
   }
 }
 
@@ -204,9 +213,9 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_
   const int valid = (int)((n - base) < (int64_t)TILE ? (n - base) : (int64_t)TILE);
   const bool full = valid == TILE;
 
-  auto digit_of = [&](U key) -> uint32_t {
-    return (uint32_t)(encode_key<U, FLOAT>(key, xor_mask) >> shift) & 0xffu;
-  };
+  // registers and the LDS exchange buffer hold ENCODED keys (one copy per key); the original
+  // bit pattern is restored when a key is written back to global memory
+  auto digit_of = [&](U enc) -> uint32_t { return (uint32_t)(enc >> shift) & 0xffu; };
 
   // ---- load: wave w owns a contiguous slab, item i of lane l is slab[i*64 + l], so the
   //      order (wave, item, lane) is the memory order and ranking in that order is stable.
@@ -214,28 +223,38 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_
   U k[IPT];
   if (full) {
 #pragma unroll
-    for (int i = 0; i < IPT; i++) k[i] = kin[base + slab + i * kWave];
+    for (int i = 0; i < IPT; i++) k[i] = encode_key<U, FLOAT>(kin[base + slab + i * kWave], xor_mask);
   } else {
-    const U pad = decode_key<U, FLOAT>(U(~U(0)), xor_mask);  // sorts after every real key
 #pragma unroll
     for (int i = 0; i < IPT; i++) {
       const int li = slab + i * kWave;
-      k[i] = li < valid ? kin[base + li] : pad;
+      k[i] = li < valid ? encode_key<U, FLOAT>(kin[base + li], xor_mask) : U(~U(0));  // padding sorts last
     }
   }
 
   // ---- early counts: per-wave digit histogram with LDS atomics, so that the tile's counts
   //      are published before the (long) ranking phase and later tiles rarely wait for them
   uint32_t* wc = sm.wave_cnt[wave];
+  {
+    // A wave whose 64 keys share one digit (sorted or low-entropy input) would serialise 64
+    // same-address atomics; such a wave lets one lane add 64 instead.  The first item decides
+    // which loop the wave runs, so random keys pay for no test at all.
+    const uint32_t f = digit_of(k[0]);
+    const bool careful = __builtin_amdgcn_ballot_w64(f != (uint32_t)__builtin_amdgcn_readfirstlane((int)f)) == 0;
+    if (!careful) {
 #pragma unroll
-  for (int i = 0; i < IPT; i++) {
-    const uint32_t d = digit_of(k[i]);
-    // a wave whose 64 keys share one digit (sorted or low-entropy input) would serialise 64
-    // same-address atomics: let one lane add 64 instead
-    if (__builtin_amdgcn_ballot_w64(d != (uint32_t)__builtin_amdgcn_readfirstlane((int)d)) == 0) {
-      if (lane == 0) atomicAdd(wc + d, (uint32_t)kWave);
+      for (int i = 0; i < IPT; i++) atomicAdd(wc + digit_of(k[i]), 1u);
     } else {
-      atomicAdd(wc + d, 1u);
+#pragma unroll
+      for (int i = 0; i < IPT; i++) {
+        const uint32_t d = digit_of(k[i]);
+        const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+        if (__builtin_amdgcn_ballot_w64(d != d0) == 0) {
+          if (lane == 0) atomicAdd(wc + d0, (uint32_t)kWave);
+        } else {
+          atomicAdd(wc + d, 1u);
+        }
+      }
     }
   }
   __syncthreads();
@@ -269,15 +288,17 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_
 #pragma unroll
   for (int i = 0; i < IPT; i++) {
     const uint32_t d = digit_of(k[i]);
+    const uint32_t old = lds_load(wc + d);  // every lane of the group reads the counter (issued early:
+                                            // the match below hides the LDS latency)
     uint32_t m_lo, m_hi;
     match_digit(d, m_lo, m_hi);
     const uint32_t below = __builtin_amdgcn_mbcnt_hi(m_hi, __builtin_amdgcn_mbcnt_lo(m_lo, 0u));
     const uint32_t cnt = __builtin_popcount(m_lo) + __builtin_popcount(m_hi);
-    const uint32_t old = lds_load(wc + d);         // every lane of the group reads the counter,
-    if (below == 0) lds_store(wc + d, old + cnt);  // then its first lane advances it
+    if (below == 0) lds_store(wc + d, old + cnt);  // the group's first lane advances the counter
     __builtin_amdgcn_wave_barrier();
     pos[i] = old + below;
     s_keys[pos[i]] = k[i];
+    __builtin_amdgcn_sched_barrier(0);  // keep iterations apart: low register pressure, enough ILP inside one
   }
 
   // ---- look-back over earlier tiles (thread d for digit d), kLookW descriptors per round trip
@@ -310,31 +331,44 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_
   }
   __syncthreads();
 
-  // ---- write each digit's run contiguously
+  // ---- write each digit's run contiguously.  Full tiles (all but the last) take a path with
+  //      no per-item bounds test, so the LDS reads of several items are in flight together.
   uint32_t gpos[IPT];
-#pragma unroll
-  for (int j = 0; j < IPT; j++) {
-    const int li = j * BLOCK + tid;
-    const U key = s_keys[li];
-    gpos[j] = sm.global_off[digit_of(key)] + (uint32_t)li;
-    if (full || li < valid) kout[gpos[j]] = key;
-  }
-
-  if constexpr (VB > 0) {
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < IPT; i++) {
-      const int li = slab + i * kWave;
-      V v = V(0);
-      if (full || li < valid) v = vin[base + li];
-      s_vals[pos[i]] = v;
-    }
-    __syncthreads();
+  auto write_keys = [&](auto full_tag) {
+    constexpr bool kFull = decltype(full_tag)::value;
 #pragma unroll
     for (int j = 0; j < IPT; j++) {
       const int li = j * BLOCK + tid;
-      if (full || li < valid) vout[gpos[j]] = s_vals[li];
+      const U key = s_keys[li];
+      gpos[j] = sm.global_off[digit_of(key)] + (uint32_t)li;
+      if (kFull || li < valid) kout[gpos[j]] = decode_key<U, FLOAT>(key, xor_mask);
     }
+  };
+  if (full) write_keys(std::true_type{}); else write_keys(std::false_type{});
+
+  if constexpr (VB > 0) {
+    __syncthreads();
+    auto stage_values = [&](auto full_tag) {
+      constexpr bool kFull = decltype(full_tag)::value;
+#pragma unroll
+      for (int i = 0; i < IPT; i++) {
+        const int li = slab + i * kWave;
+        V v = V(0);
+        if (kFull || li < valid) v = vin[base + li];
+        s_vals[pos[i]] = v;
+      }
+    };
+    if (full) stage_values(std::true_type{}); else stage_values(std::false_type{});
+    __syncthreads();
+    auto write_values = [&](auto full_tag) {
+      constexpr bool kFull = decltype(full_tag)::value;
+#pragma unroll
+      for (int j = 0; j < IPT; j++) {
+        const int li = j * BLOCK + tid;
+        if (kFull || li < valid) vout[gpos[j]] = s_vals[li];
+      }
+    };
+    if (full) write_values(std::true_type{}); else write_values(std::false_type{});
   }
 }
 
@@ -348,7 +382,7 @@ struct SortConfig {
   // limit is LDS (two workgroups per CU must fit) and registers.
 #ifndef TCD_SORT_A_BLOCK
 #define TCD_SORT_A_BLOCK 512
-#define TCD_SORT_A_IPT 24
+#define TCD_SORT_A_IPT 21
 #endif
 #ifndef TCD_SORT_B_BLOCK
 #define TCD_SORT_B_BLOCK 1024
