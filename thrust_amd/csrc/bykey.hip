@@ -56,13 +56,49 @@ __device__ inline bool keys_differ(KU a, KU b, int float_keys) {
   return a != b;
 }
 
-template <int N, class E>
-struct alignas(N * sizeof(E)) VecN {
-  E v[N];
-};
+template <int BYTES> struct bits_of;
+template <> struct bits_of<1> { using type = uint8_t; };
+template <> struct bits_of<2> { using type = uint16_t; };
+template <> struct bits_of<4> { using type = uint32_t; };
+template <> struct bits_of<8> { using type = uint64_t; };
 
-// Geometry shared by both kernels: a thread owns VEC consecutive elements of each of
-// CHUNKS chunks; VEC is set by the wider of key and value so that no access exceeds 16 B.
+// N consecutive elements from a pointer aligned to min(16, N*sizeof(E)) bytes, as 128-bit
+// (or one narrower) accesses.
+template <int N, class E>
+__device__ inline void load_group(const E* p, E (&dst)[N]) {
+  constexpr int BYTES = N * (int)sizeof(E);
+  if constexpr (BYTES >= 16) {
+#pragma unroll
+    for (int q = 0; q < BYTES / 16; q++) {
+      const uint4 t = reinterpret_cast<const uint4*>(p)[q];
+      __builtin_memcpy(reinterpret_cast<char*>(dst) + 16 * q, &t, 16);
+    }
+  } else {
+    const typename bits_of<BYTES>::type t = *reinterpret_cast<const typename bits_of<BYTES>::type*>(p);
+    __builtin_memcpy(dst, &t, BYTES);
+  }
+}
+template <int N, class E>
+__device__ inline void store_group(E* p, const E (&src)[N]) {
+  constexpr int BYTES = N * (int)sizeof(E);
+  if constexpr (BYTES >= 16) {
+#pragma unroll
+    for (int q = 0; q < BYTES / 16; q++) {
+      uint4 t;
+      __builtin_memcpy(&t, reinterpret_cast<const char*>(src) + 16 * q, 16);
+      reinterpret_cast<uint4*>(p)[q] = t;
+    }
+  } else {
+    typename bits_of<BYTES>::type t;
+    __builtin_memcpy(&t, src, BYTES);
+    *reinterpret_cast<typename bits_of<BYTES>::type*>(p) = t;
+  }
+}
+
+// Geometry shared by both kernels: a thread owns VEC consecutive elements of each of CHUNKS
+// chunks; the wider of key and value fills 32 bytes per thread and chunk (two 128-bit accesses),
+// capped at 16 elements.  Long per-thread groups keep the cross-lane scans (one per chunk) cheap
+// per element.
 template <class T>
 struct SegGeom {
 #ifndef TCD_SEG_BLOCK
@@ -71,16 +107,17 @@ struct SegGeom {
 #endif
   static constexpr int BLOCK = TCD_SEG_BLOCK;
   static constexpr int WIDE = (int)(sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T));
-  static constexpr int VEC = 16 / WIDE;
-  static constexpr int CHUNKS = WIDE >= 4 ? TCD_SEG_CHUNKS : 2;
+  static constexpr int VEC = 32 / WIDE > 16 ? 16 : 32 / WIDE;
+  static constexpr int CHUNKS = TCD_SEG_CHUNKS;
   static constexpr int NWAVES = BLOCK / kWave;
   static constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
 };
 
-// Loads a tile, computes head flags, scans it and resolves the tile prefix by look-back.
-// On return: key/val/head hold the thread's elements, incl[c][j] the segmented inclusive
-// pair of element (c, j) counted from the start of the thread's group, and off[c] the pair
-// of everything before the group (all earlier tiles included).
+// Loads a tile, finds the segment heads, reduces it and resolves the prefix of all earlier
+// tiles by look-back.  On return key/val hold the thread's elements, bit j of heads[c] says
+// whether element (c, j) starts a segment, and off[c] is the pair (heads seen, value of the
+// open segment) of everything before the thread's group of chunk c.  The kernels then walk
+// their elements once more from off[c]; nothing per element is kept in between.
 template <class T, class Op>
 struct SegTile {
   using G = SegGeom<T>;
@@ -95,15 +132,17 @@ struct SegTile {
 
   KU key[CHUNKS][VEC];
   T val[CHUNKS][VEC];
-  bool head[CHUNKS][VEC];
-  Pair incl[CHUNKS][VEC];
+  uint32_t heads[CHUNKS];
   Pair off[CHUNKS];
   int64_t base;
   int64_t tile;
+  bool full;  // every element of the tile exists, the tile is not the last one, pointers are aligned
 
   __device__ int64_t index(int c, int j) const {
     return base + ((int64_t)c * BLOCK + threadIdx.x) * VEC + j;
   }
+
+  __device__ static Pair comb(const Pair& a, const Pair& b) { return seg_combine<T, Op>(a, b); }
 
   __device__ void run(Smem& sm, const KU* keys, const T* vals, int64_t n, int float_keys, int vec_ok,
                       uint64_t* desc, uint32_t* ticket) {
@@ -112,25 +151,27 @@ struct SegTile {
     const int wave = tid / kWave;
     const T id = Op::template identity<T>();
     const Pair idp{0u, id};
-    auto comb = [](const Pair& a, const Pair& b) { return seg_combine<T, Op>(a, b); };
 
     if (tid == 0) sm.tile = atomicAdd(ticket, 1u);
     __syncthreads();
     tile = sm.tile;
     base = tile * G::TILE;
-    const bool fast = vec_ok && (base + G::TILE <= n);
+    full = vec_ok && (base + G::TILE < n);
 
+    KU prev[CHUNKS];
+    if (full) {
 #pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-      const int64_t i0 = index(c, 0);
-      KU prev = 0;
-      if (i0 > 0 && i0 < n) prev = keys[i0 - 1];
-      if (fast) {
-        const auto kv = *reinterpret_cast<const VecN<VEC, KU>*>(keys + i0);
-        const auto vv = *reinterpret_cast<const VecN<VEC, T>*>(vals + i0);
+      for (int c = 0; c < CHUNKS; c++) {
+        const int64_t i0 = index(c, 0);
+        prev[c] = i0 > 0 ? keys[i0 - 1] : KU(0);
+        load_group<VEC>(keys + i0, key[c]);
+        load_group<VEC>(vals + i0, val[c]);
+      }
+    } else {
 #pragma unroll
-        for (int j = 0; j < VEC; j++) { key[c][j] = kv.v[j]; val[c][j] = vv.v[j]; }
-      } else {
+      for (int c = 0; c < CHUNKS; c++) {
+        const int64_t i0 = index(c, 0);
+        prev[c] = (i0 > 0 && i0 < n) ? keys[i0 - 1] : KU(0);
 #pragma unroll
         for (int j = 0; j < VEC; j++) {
           const int64_t idx = i0 + j;
@@ -138,21 +179,24 @@ struct SegTile {
           val[c][j] = idx < n ? vals[idx] : id;
         }
       }
-#pragma unroll
-      for (int j = 0; j < VEC; j++) {
-        const int64_t idx = i0 + j;
-        const KU p = j == 0 ? prev : key[c][j - 1];
-        head[c][j] = idx < n && (idx == 0 || keys_differ(p, key[c][j], float_keys));
-      }
     }
 
     Pair excl_w[CHUNKS];
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
-      incl[c][0] = Pair{head[c][0] ? 1u : 0u, val[c][0]};
+      const int64_t i0 = index(c, 0);
+      uint32_t h = 0;
+      Pair agg = idp;
 #pragma unroll
-      for (int j = 1; j < VEC; j++) incl[c][j] = comb(incl[c][j - 1], Pair{head[c][j] ? 1u : 0u, val[c][j]});
-      const Pair w = wave_inclusive_scan(incl[c][VEC - 1], idp, comb);
+      for (int j = 0; j < VEC; j++) {
+        const KU p = j == 0 ? prev[c] : key[c][j - 1];
+        const bool is_head = (full || i0 + j < n) && (i0 + j == 0 || keys_differ(p, key[c][j], float_keys));
+        h |= (is_head ? 1u : 0u) << j;
+        agg.v = is_head ? val[c][j] : Op::template apply<T>(agg.v, val[c][j]);
+      }
+      heads[c] = h;
+      agg.c = __builtin_popcount(h);
+      const Pair w = wave_inclusive_scan(agg, idp, comb);
       excl_w[c] = wave_shift_up1(w, idp);
       if (lane == kWave - 1) sm.tot[c][wave] = w;
     }
@@ -200,26 +244,21 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) void scan_by_key_kernel(
   ST t;
   t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket);
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS;
-  const bool fast = vec_ok && (t.base + SegGeom<T>::TILE <= n);
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
     T r[VEC];
+    T open = t.off[c].v;  // value of the open segment just before the element
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
-      if (!exclusive) {
-        r[j] = seg_combine<T, Op>(t.off[c], t.incl[c][j]).v;
-      } else {
-        // value of the open segment just before this element
-        const T before = j == 0 ? t.off[c].v : seg_combine<T, Op>(t.off[c], t.incl[c][j - 1]).v;
-        r[j] = t.head[c][j] ? init : Op::template apply<T>(init, before);
-      }
+      const bool is_head = (t.heads[c] >> j) & 1u;
+      const T x = t.val[c][j];
+      if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
+      open = is_head ? x : Op::template apply<T>(open, x);
+      if (!exclusive) r[j] = open;
     }
     const int64_t i0 = t.index(c, 0);
-    if (fast) {
-      VecN<VEC, T> v;
-#pragma unroll
-      for (int j = 0; j < VEC; j++) v.v[j] = r[j];
-      *reinterpret_cast<VecN<VEC, T>*>(out + i0) = v;
+    if (t.full) {
+      store_group<VEC>(out + i0, r);
     } else {
 #pragma unroll
       for (int j = 0; j < VEC; j++)
@@ -242,20 +281,24 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) void reduce_by_key_kernel(
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS;
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
+    // (runs started so far, value of the open run) before the current element
+    SegPair<T> run = t.off[c];
+    const int64_t i0 = t.index(c, 0);
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
-      const int64_t idx = t.index(c, j);
-      if (idx >= n) continue;
-      // pair of everything before this element: (runs started so far, value of the open run)
-      const SegPair<T> before = j == 0 ? t.off[c] : seg_combine<T, Op>(t.off[c], t.incl[c][j - 1]);
-      if (t.head[c][j]) {
-        keys_out[before.c] = t.key[c][j];
-        if (idx > 0) vals_out[before.c - 1] = before.v;
+      const bool exists = t.full || i0 + j < n;
+      if ((t.heads[c] >> j) & 1u) {
+        // a head closes the run before it and opens run number run.c
+        keys_out[run.c] = t.key[c][j];
+        if (run.c) vals_out[run.c - 1] = run.v;
+        run.c += 1;
+        run.v = t.val[c][j];
+      } else if (exists) {
+        run.v = Op::template apply<T>(run.v, t.val[c][j]);
       }
-      if (idx == n - 1) {
-        const SegPair<T> last = seg_combine<T, Op>(t.off[c], t.incl[c][j]);
-        vals_out[last.c - 1] = last.v;
-        *num_runs = (int64_t)last.c;
+      if (!t.full && i0 + j == n - 1) {  // the last element closes the last run
+        vals_out[run.c - 1] = run.v;
+        *num_runs = (int64_t)run.c;
       }
     }
   }
