@@ -22,11 +22,11 @@ __global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NWAVES = BLOCK / kWave;
   constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
-  // payload in the descriptor: at least one dword
+  static_assert(CHUNKS * NWAVES <= kWave, "one wavefront scans the (chunk, wave) totals");
+  // cross-lane traffic, LDS and descriptors carry W (a dword container for 1- and 2-byte T)
   using W = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
 
-  __shared__ T s_tot[CHUNKS][NWAVES];
-  __shared__ T s_prefix;
+  __shared__ W s_tot[CHUNKS * NWAVES];  // inclusive total of (chunk, wave), then its exclusive offset
   __shared__ uint32_t s_tile;
 
   const int tid = threadIdx.x;
@@ -34,34 +34,6 @@ __global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_
   const int wave = tid / kWave;
   const T id = Op::template identity<T>();
   auto op = [](T a, T b) { return Op::template apply<T>(a, b); };
-
-  if (tid == 0) s_tile = atomicAdd(ticket, 1u);
-  __syncthreads();
-  const int64_t tile = s_tile;
-  const int64_t base = tile * TILE;
-  const bool fast = vec_ok && (base + TILE <= n);
-
-  T x[CHUNKS][VEC];
-  if (fast) {
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-      Vec16<T> v = *reinterpret_cast<const Vec16<T>*>(in + base + ((int64_t)c * BLOCK + tid) * VEC);
-#pragma unroll
-      for (int j = 0; j < VEC; j++) x[c][j] = v.v[j];
-    }
-  } else {
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-#pragma unroll
-      for (int j = 0; j < VEC; j++) {
-        int64_t idx = base + ((int64_t)c * BLOCK + tid) * VEC + j;
-        x[c][j] = idx < n ? in[idx] : id;
-      }
-    }
-  }
-
-  // thread-local inclusive scan of each 16-byte group, then a wave scan of the group sums.
-  // Cross-lane traffic, LDS and descriptors carry W (a dword container for 1- and 2-byte T).
   auto toW = [](T a) {
     if constexpr (std::is_same<W, T>::value) return a;
     else return (W)(typename unsigned_of<T>::type)a;
@@ -71,67 +43,93 @@ __global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_
     else return (W)(typename unsigned_of<T>::type)op((T)a, (T)b);
   };
   const W idW = toW(id);
+
+  if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+  __syncthreads();
+  const int64_t tile = s_tile;
+  const int64_t base = tile * TILE;
+  const bool fast = vec_ok && (base + TILE <= n);  // whole tile present, 16-byte aligned pointers
+  const T* tin = in + base + (int64_t)tid * VEC;
+  T* tout = out + base + (int64_t)tid * VEC;
+
+  T x[CHUNKS][VEC];
+  if (fast) {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+      const Vec16<T> v = *reinterpret_cast<const Vec16<T>*>(tin + c * BLOCK * VEC);
+#pragma unroll
+      for (int j = 0; j < VEC; j++) x[c][j] = v.v[j];
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+#pragma unroll
+      for (int j = 0; j < VEC; j++) {
+        const int64_t idx = base + ((int64_t)c * BLOCK + tid) * VEC + j;
+        x[c][j] = idx < n ? in[idx] : id;
+      }
+    }
+  }
+
+  // thread-local inclusive scan of each 16-byte group, then a wave scan of the group sums
   T excl[CHUNKS];
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
 #pragma unroll
     for (int j = 1; j < VEC; j++) x[c][j] = op(x[c][j - 1], x[c][j]);
-    W incl = wave_inclusive_scan(toW(x[c][VEC - 1]), idW, opW);
+    const W incl = wave_inclusive_scan(toW(x[c][VEC - 1]), idW, opW);
     excl[c] = (T)wave_shift_up1(incl, idW);
-    if (lane == kWave - 1) s_tot[c][wave] = (T)incl;
+    if (lane == kWave - 1) s_tot[c * NWAVES + wave] = incl;
   }
   __syncthreads();
 
-  // offsets of this thread's (chunk, wave) segments inside the tile, and the tile aggregate
-  T seg_base[CHUNKS];
-  T run = id;
-#pragma unroll
-  for (int c = 0; c < CHUNKS; c++) {
-#pragma unroll
-    for (int w = 0; w < NWAVES; w++) {
-      if (w == wave) seg_base[c] = run;
-      run = op(run, s_tot[c][w]);
-    }
-  }
-  const T tile_agg = run;
-
+  // wave 0: exclusive scan of the (chunk, wave) totals in tile order, then the look-back
   if (wave == 0) {
-    T prefix;
+    const W mine = lane < CHUNKS * NWAVES ? s_tot[lane] : idW;
+    const W incl = wave_inclusive_scan(mine, idW, opW);
+    const W tile_agg = readlane(incl, kWave - 1);
+    const W before = wave_shift_up1(incl, idW);
+    W prefix;
     if (tile == 0) {
-      prefix = exclusive ? init : id;
-      if (lane == 0) TileDesc<W>::store(desc, 0, kInclusive, toW(op(prefix, tile_agg)));
+      prefix = exclusive ? toW(init) : idW;
+      if (lane == 0) TileDesc<W>::store(desc, 0, kInclusive, opW(prefix, tile_agg));
     } else {
-      if (lane == 0) TileDesc<W>::store(desc, tile, kPartial, toW(tile_agg));
-      prefix = (T)wave_lookback<W>(desc, tile, idW, opW);
-      if (lane == 0) TileDesc<W>::store(desc, tile, kInclusive, toW(op(prefix, tile_agg)));
+      if (lane == 0) TileDesc<W>::store(desc, tile, kPartial, tile_agg);
+      prefix = wave_lookback<W>(desc, tile, idW, opW);
+      if (lane == 0) TileDesc<W>::store(desc, tile, kInclusive, opW(prefix, tile_agg));
     }
-    if (lane == 0) s_prefix = prefix;
+    if (lane < CHUNKS * NWAVES) s_tot[lane] = opW(prefix, before);  // offset of (chunk, wave) in the whole input
   }
   __syncthreads();
-  const T prefix = s_prefix;
 
+  // results: element (c, j) = offset of its (chunk, wave) (+) lanes before it (+) its group prefix
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
-    const T off = op(op(prefix, seg_base[c]), excl[c]);
-    T r[VEC];
+    const T off = op((T)s_tot[c * NWAVES + wave], excl[c]);
     if (exclusive) {
-      r[0] = off;
 #pragma unroll
-      for (int j = 1; j < VEC; j++) r[j] = op(off, x[c][j - 1]);
+      for (int j = VEC - 1; j > 0; j--) x[c][j] = op(off, x[c][j - 1]);
+      x[c][0] = off;
     } else {
 #pragma unroll
-      for (int j = 0; j < VEC; j++) r[j] = op(off, x[c][j]);
+      for (int j = 0; j < VEC; j++) x[c][j] = op(off, x[c][j]);
     }
-    if (fast) {
+  }
+  if (fast) {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
       Vec16<T> v;
 #pragma unroll
-      for (int j = 0; j < VEC; j++) v.v[j] = r[j];
-      *reinterpret_cast<Vec16<T>*>(out + base + ((int64_t)c * BLOCK + tid) * VEC) = v;
-    } else {
+      for (int j = 0; j < VEC; j++) v.v[j] = x[c][j];
+      *reinterpret_cast<Vec16<T>*>(tout + c * BLOCK * VEC) = v;
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
 #pragma unroll
       for (int j = 0; j < VEC; j++) {
-        int64_t idx = base + ((int64_t)c * BLOCK + tid) * VEC + j;
-        if (idx < n) out[idx] = r[j];
+        const int64_t idx = base + ((int64_t)c * BLOCK + tid) * VEC + j;
+        if (idx < n) out[idx] = x[c][j];
       }
     }
   }
