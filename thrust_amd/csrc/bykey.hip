@@ -275,22 +275,31 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) void reduce_by_key_kernel(
     const KU* keys, const T* vals, KU* keys_out, T* vals_out, int64_t* num_runs, int64_t n,
     int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket) {
   using ST = SegTile<T, Op>;
+  constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS, NWAVES = ST::NWAVES;
   __shared__ typename ST::Smem sm;
+  // Per-wave staging of one chunk's output: the heads of a wave's 64*VEC consecutive elements go
+  // to consecutive output slots, so they are compacted in LDS and written with coalesced stores
+  // (no workgroup barrier: the buffer is private to the wave).
+  __shared__ KU s_keys[NWAVES][kWave * VEC];
+  __shared__ T s_vals[NWAVES][kWave * VEC];
   ST t;
   t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket);
-  constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS;
+  const int lane = threadIdx.x & (kWave - 1);
+  KU* sk = s_keys[threadIdx.x / kWave];
+  T* sv = s_vals[threadIdx.x / kWave];
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
     // (runs started so far, value of the open run) before the current element
     SegPair<T> run = t.off[c];
+    const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)run.c);  // runs before this wave's chunk
     const int64_t i0 = t.index(c, 0);
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
       const bool exists = t.full || i0 + j < n;
       if ((t.heads[c] >> j) & 1u) {
         // a head closes the run before it and opens run number run.c
-        keys_out[run.c] = t.key[c][j];
-        if (run.c) vals_out[run.c - 1] = run.v;
+        sk[run.c - first] = t.key[c][j];
+        sv[run.c - first] = run.v;
         run.c += 1;
         run.v = t.val[c][j];
       } else if (exists) {
@@ -301,6 +310,13 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) void reduce_by_key_kernel(
         *num_runs = (int64_t)run.c;
       }
     }
+    const uint32_t count = (uint32_t)__builtin_amdgcn_readlane((int)run.c, kWave - 1) - first;
+    __builtin_amdgcn_wave_barrier();
+    for (uint32_t i = lane; i < count; i += kWave) {
+      keys_out[first + i] = sk[i];
+      if (first + i) vals_out[first + i - 1] = sv[i];  // value of the run that ended at this head
+    }
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
