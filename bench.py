@@ -21,7 +21,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # measured HBM traffic of one onesweep launch over 2^28 uint32 keys
 # (profiles/onesweep_u32_sort_2p28_and_extras.md)
-ONESWEEP_U32_TRAFFIC_BYTES = 2.463e9
+ONESWEEP_U32_TRAFFIC_BYTES = 2.482e9
 
 
 def parse():
@@ -276,10 +276,10 @@ def main():
     if not args.no_cpu:
         import oracle
         threads = oracle.omp_max_threads()
-        m = 1 << 26
+        m = n  # the whole GPU workload: a few seconds per repetition on 16 cores
         ks = np.random.default_rng(1337).integers(0, 2**32, m, dtype=np.uint64).astype(np.uint32)
         best = None
-        for _ in range(2):
+        for _ in range(3):
             k = ks.copy()
             t0 = time.perf_counter()
             oracle.omp_sort(k, None, threads)
@@ -288,8 +288,8 @@ def main():
         assert (k[1:] >= k[:-1]).all()
         cpu = {
             "value": round(m / best / 1e9, 4), "unit": "Gkeys/s", "cores": threads, "kind": "port",
-            "sample": f"2^26 uniform uint32 keys (1/4 of the GPU workload), best of 2; oracle restatement "
-                      f"of the reference OpenMP sort (per-thread radix sort + pairwise merges)",
+            "sample": f"2^{args.log2n} uniform uint32 keys (the whole GPU workload), best of 3; oracle "
+                      f"restatement of the reference OpenMP sort (per-thread radix sort + pairwise merges)",
         }
 
     out = {
