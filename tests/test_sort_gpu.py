@@ -146,3 +146,30 @@ def test_sort_full_size_properties():
     assert (hk[1:] >= hk[:-1]).all()
     assert int(hk.view(np.int32).sum(dtype=np.int64)) == s0
     assert int(np.bitwise_xor.reduce(hk)) == x0
+
+
+def test_lds_atomic_order_selftest():
+    """The stable ranking of the sort kernels assumes that returning LDS atomics of one wavefront
+    instruction are served in lane order; the library's self-test checks that on this device."""
+    import ctypes
+
+    from thrust_amd import capi
+    L = capi.lib()
+    bad = ctypes.c_longlong(-1)
+    rc = L.thrust_cdna4_selftest_lds_atomic_order(ctypes.byref(bad), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    assert bad.value == 0
+
+
+def test_sort_skewed_digits_stability():
+    """Keys whose digits are heavily skewed (most lanes of a wavefront share a digit) take the
+    careful ranking loop; pairs must stay stable."""
+    rng = np.random.default_rng(99)
+    n = 300_001
+    for hot_frac in (0.3, 0.9, 1.0):
+        keys = np.where(rng.random(n) < hot_frac, np.uint32(0x07070707), rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32))
+        vals = np.arange(n, dtype=np.uint32)
+        ek, ev = oracle.sort_pairs(keys.copy(), vals.copy(), False)
+        k, v = dev(keys), dev(vals)
+        thrust_amd.sort_by_key(k, v, False)
+        assert same_bits(host(k), ek) and same_bits(host(v), ev), hot_frac

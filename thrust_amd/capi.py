@@ -21,6 +21,7 @@ SYMBOLS = [
     "thrust_cdna4_memcpy_htod", "thrust_cdna4_memcpy_dtoh", "thrust_cdna4_memcpy_dtod",
     "thrust_cdna4_fill", "thrust_cdna4_stream_synchronize", "thrust_cdna4_profile_enable",
     "thrust_cdna4_profile_count", "thrust_cdna4_profile_get",
+    "thrust_cdna4_selftest_lds_atomic_order",
 ]
 
 
@@ -65,6 +66,7 @@ def lib():
     L.thrust_cdna4_fill.argtypes = [vp, vp, i32, i64, vp]
     L.thrust_cdna4_stream_synchronize.argtypes = [vp]
     L.thrust_cdna4_profile_enable.argtypes = [i32]
+    L.thrust_cdna4_selftest_lds_atomic_order.argtypes = [ctypes.POINTER(ctypes.c_longlong), vp]
     L.thrust_cdna4_profile_get.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p),
                                            ctypes.POINTER(ctypes.c_float)]
     _lib = L

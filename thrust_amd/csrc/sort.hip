@@ -4,11 +4,15 @@
 //                          digit places, merged into global memory with atomics.
 //   2. radix_bins_kernel   exclusive scan of each digit place's 256 bins.
 //   3. onesweep_kernel     one launch per 8-bit digit.  A workgroup takes a tile by ticket,
-//                          ranks its keys stably (wave64 ballot "match" ranking on per-wave
-//                          LDS counters), publishes its 256 digit counts, finds the counts
+//                          ranks its keys stably (returning LDS atomics on per-wave digit
+//                          counters), publishes its 256 digit counts, finds the counts
 //                          of all earlier tiles by decoupled look-back (one thread per
 //                          digit), reorders the tile through LDS so that every digit's keys
 //                          are contiguous, and writes each run with coalesced stores.
+//
+// Stability of the ranking rests on one property of the LDS unit: the lanes of one wavefront
+// instruction that add to the same LDS address receive their old values in lane order.
+// thrust_cdna4_selftest_lds_atomic_order() (below) checks it on the device at hand.
 //
 // Keys stay in their original representation in memory; the digit is taken from the
 // order-preserving encoding of thrust/system/detail/sequential/stable_radix_sort.inl:43-139
@@ -150,28 +154,6 @@ struct OnesweepSmem {
   uint32_t tile;
 };
 
-// Lanes of this wavefront whose 8-bit digit equals this lane's digit, as two 32-bit halves.
-// Per bit: one v_bfe_i32 (0 / -1 per lane), one v_cmp (the ballot, an SGPR pair) and one
-// three-input bit operation per half:  m &= ~(ballot ^ bit)   (truth table 0x90).
-__device__ inline void match_digit(uint32_t d, uint32_t& m_lo, uint32_t& m_hi) {
-  int32_t e[kRadixBits];
-  uint64_t bal[kRadixBits];
-#pragma unroll
-  for (int b = 0; b < kRadixBits; b++) {
-    e[b] = __builtin_amdgcn_sbfe((int)d, b, 1);
-    asm("" : "+v"(e[b]));  // keep the compare on e itself instead of a second bit extraction
-  }
-#pragma unroll
-  for (int b = 0; b < kRadixBits; b++) bal[b] = __builtin_amdgcn_ballot_w64(e[b] != 0);
-  m_lo = ~0u;
-  m_hi = ~0u;
-#pragma unroll
-  for (int b = 0; b < kRadixBits; b++) {
-    m_lo = __builtin_amdgcn_bitop3_b32(m_lo, (uint32_t)bal[b], (uint32_t)e[b], 0x90);
-    m_hi = __builtin_amdgcn_bitop3_b32(m_hi, (uint32_t)(bal[b] >> 32), (uint32_t)e[b], 0x90);
-  }
-}
-
 __device__ inline uint32_t lds_load(const uint32_t* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
 }
@@ -179,11 +161,8 @@ __device__ inline void lds_store(uint32_t* p, uint32_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
 }
 
-#ifndef TCD_SORT_WPE
-#define TCD_SORT_WPE 4
-#endif
-template <class U, int VB, bool FLOAT, int BLOCK, int IPT>
-__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_WPE))) void onesweep_kernel(const U* __restrict__ kin, U* __restrict__ kout,
+template <class U, int VB, bool FLOAT, int BLOCK, int IPT, int WPE>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) void onesweep_kernel(const U* __restrict__ kin, U* __restrict__ kout,
                                                          const void* __restrict__ vin_, void* __restrict__ vout_,
                                                          int64_t n, U xor_mask, int shift,
                                                          const uint32_t* __restrict__ gbase,
@@ -232,28 +211,39 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_
     }
   }
 
-  // ---- early counts: per-wave digit histogram with LDS atomics, so that the tile's counts
-  //      are published before the (long) ranking phase and later tiles rarely wait for them
+  // ---- rank within (wave, digit): the value returned by the wave's LDS atomic add.  The LDS
+  //      unit serves the lanes of one instruction that hit the same address in lane order, so
+  //      the returned values number a digit's keys in (item, lane) order, which is the memory
+  //      order of the wave's slab: the ranking is stable.  Afterwards the counters hold the
+  //      per-wave digit counts, published before the reorder so that later tiles rarely wait.
   uint32_t* wc = sm.wave_cnt[wave];
+  uint32_t pos[IPT];
   {
     // A wave whose 64 keys share one digit (sorted or low-entropy input) would serialise 64
-    // same-address atomics; such a wave lets one lane add 64 instead.  The first item decides
-    // which loop the wave runs, so random keys pay for no test at all.
+    // same-address atomics.  The first item decides which loop the wave runs (random keys pay
+    // for no test at all); the careful loop ranks the lanes that share the first lane's digit
+    // with one ballot and lets only the others issue atomics.
     const uint32_t f = digit_of(k[0]);
-    const bool careful = __builtin_amdgcn_ballot_w64(f != (uint32_t)__builtin_amdgcn_readfirstlane((int)f)) == 0;
+    const bool careful = __builtin_popcountll(__builtin_amdgcn_ballot_w64(
+                             f == (uint32_t)__builtin_amdgcn_readfirstlane((int)f))) >= kWave / 4;
     if (!careful) {
 #pragma unroll
-      for (int i = 0; i < IPT; i++) atomicAdd(wc + digit_of(k[i]), 1u);
+      for (int i = 0; i < IPT; i++) pos[i] = atomicAdd(wc + digit_of(k[i]), 1u);
     } else {
 #pragma unroll
       for (int i = 0; i < IPT; i++) {
         const uint32_t d = digit_of(k[i]);
         const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
-        if (__builtin_amdgcn_ballot_w64(d != d0) == 0) {
-          if (lane == 0) atomicAdd(wc + d0, (uint32_t)kWave);
+        const uint64_t same = __builtin_amdgcn_ballot_w64(d == d0);
+        if (d == d0) {
+          const uint32_t old = lds_load(wc + d0);
+          const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(same >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)same, 0u));
+          if (below == 0) lds_store(wc + d0, old + (uint32_t)__builtin_popcountll(same));
+          pos[i] = old + below;
         } else {
-          atomicAdd(wc + d, 1u);
+          pos[i] = atomicAdd(wc + d, 1u);
         }
+        __builtin_amdgcn_wave_barrier();
       }
     }
   }
@@ -282,23 +272,11 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_
   }
   __syncthreads();
 
-  // ---- rank and reorder: a wave's counter of a digit is its next free local slot; the lanes
-  //      holding the same digit (8 ballots) take consecutive slots in lane order
-  uint32_t pos[IPT];
+  // ---- reorder: local slot = first slot of the wave's keys of that digit + rank
 #pragma unroll
   for (int i = 0; i < IPT; i++) {
-    const uint32_t d = digit_of(k[i]);
-    const uint32_t old = lds_load(wc + d);  // every lane of the group reads the counter (issued early:
-                                            // the match below hides the LDS latency)
-    uint32_t m_lo, m_hi;
-    match_digit(d, m_lo, m_hi);
-    const uint32_t below = __builtin_amdgcn_mbcnt_hi(m_hi, __builtin_amdgcn_mbcnt_lo(m_lo, 0u));
-    const uint32_t cnt = __builtin_popcount(m_lo) + __builtin_popcount(m_hi);
-    if (below == 0) lds_store(wc + d, old + cnt);  // the group's first lane advances the counter
-    __builtin_amdgcn_wave_barrier();
-    pos[i] = old + below;
+    pos[i] += wc[digit_of(k[i])];
     s_keys[pos[i]] = k[i];
-    __builtin_amdgcn_sched_barrier(0);  // keep iterations apart: low register pressure, enough ILP inside one
   }
 
   // ---- look-back over earlier tiles (thread d for digit d), kLookW descriptors per round trip
@@ -373,29 +351,82 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(TCD_SORT_
 }
 
 // ---------------------------------------------------------------------------------------
+// Self-test of the LDS property the ranking relies on
+// ---------------------------------------------------------------------------------------
+// Every wave adds 1 to pseudo-random counters of its own (uniform digits, one hot digit, and a
+// bank-structured pattern) and compares each returned value with the counter's value before
+// the instruction plus the number of lower lanes that hit the same counter.
+__global__ __launch_bounds__(512) void lds_atomic_order_kernel(unsigned long long* mismatches, int iters) {
+  __shared__ uint32_t cnt[8][kRadix];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  for (int i = threadIdx.x; i < 8 * kRadix; i += 512) (&cnt[0][0])[i] = 0;
+  __syncthreads();
+  unsigned long long bad = 0;
+  for (int it = 0; it < iters; it++) {
+    uint32_t h = (blockIdx.x * 512u + threadIdx.x) * 7919u + (uint32_t)it * 104729u + 12345u;
+    h ^= h >> 16; h *= 0x7feb352du; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+    const int mode = it % 3;
+    const uint32_t d = mode == 0 ? (h & 0xffu) : mode == 1 ? ((h % 5u == 0) ? ((h >> 8) & 0xffu) : 3u)
+                                                           : (((uint32_t)lane * 4u + (h & 3u)) & 0xffu);
+    uint64_t same = ~0ull;
+#pragma unroll
+    for (int b = 0; b < kRadixBits; b++) {
+      const bool bit = (d >> b) & 1u;
+      const uint64_t m = __builtin_amdgcn_ballot_w64(bit);
+      same &= bit ? m : ~m;
+    }
+    const uint32_t lower = (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
+    const uint32_t before = lds_load(&cnt[wave][d]);
+    __builtin_amdgcn_wave_barrier();
+    const uint32_t got = atomicAdd(&cnt[wave][d], 1u);
+    __builtin_amdgcn_wave_barrier();
+    bad += got != before + lower;
+  }
+  if (bad) atomicAdd(mismatches, bad);
+}
+
+// ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
 template <class U, int VB>
 struct SortConfig {
-  // Tile shape by bytes moved per item (key + value), measured on MI355X at n = 2^28:
-  // large tiles shorten the look-back chains and lengthen the per-digit output runs; the
-  // limit is LDS (two workgroups per CU must fit) and registers.
+  // Tile shape by bytes moved per item (key + value), measured on MI355X at n = 2^28.  The
+  // time of a pass grows by about 9 ns per tile (ticket, barriers, descriptor traffic and
+  // look-back latency do not shrink with the tile), so tiles are as large as LDS and registers
+  // allow: 4-byte items run two 1024-thread workgroups per CU at 64 VGPRs.
 #ifndef TCD_SORT_A_BLOCK
-#define TCD_SORT_A_BLOCK 512
-#define TCD_SORT_A_IPT 21
+#define TCD_SORT_A_BLOCK 1024
+#endif
+#ifndef TCD_SORT_A_IPT
+#define TCD_SORT_A_IPT 14
 #endif
 #ifndef TCD_SORT_B_BLOCK
 #define TCD_SORT_B_BLOCK 1024
+#endif
+#ifndef TCD_SORT_B_IPT
 #define TCD_SORT_B_IPT 16
 #endif
 #ifndef TCD_SORT_C_BLOCK
 #define TCD_SORT_C_BLOCK 1024
+#endif
+#ifndef TCD_SORT_C_IPT
 #define TCD_SORT_C_IPT 12
+#endif
+#ifndef TCD_SORT_A_WPE
+#define TCD_SORT_A_WPE 8
+#endif
+#ifndef TCD_SORT_B_WPE
+#define TCD_SORT_B_WPE 4
+#endif
+#ifndef TCD_SORT_C_WPE
+#define TCD_SORT_C_WPE 4
 #endif
   static constexpr int BYTES = (int)sizeof(U) + VB;
   static constexpr int BLOCK = BYTES <= 4 ? TCD_SORT_A_BLOCK : (BYTES <= 8 ? TCD_SORT_B_BLOCK : TCD_SORT_C_BLOCK);
   static constexpr int IPT = BYTES <= 4 ? TCD_SORT_A_IPT : (BYTES <= 8 ? TCD_SORT_B_IPT : TCD_SORT_C_IPT);
   static constexpr int TILE = BLOCK * IPT;
+  // wavefronts per SIMD the register allocation aims for
+  static constexpr int WPE = BYTES <= 4 ? TCD_SORT_A_WPE : (BYTES <= 8 ? TCD_SORT_B_WPE : TCD_SORT_C_WPE);
 };
 
 struct SortPlan {
@@ -452,7 +483,7 @@ static hipError_t sort_typed(void* temp, size_t* temp_bytes, void* keys, void* v
   TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(P), dim3(256), stream, ghist);
   int cur = 0;
   for (int p = 0; p < P; p++) {
-    TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT>), dim3((unsigned)plan.ntiles),
+    TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT, C::WPE>), dim3((unsigned)plan.ntiles),
                dim3(C::BLOCK), stream, kbuf[cur], kbuf[cur ^ 1], vbuf[cur], vbuf[cur ^ 1], n, xor_mask, 8 * p,
                ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix, tickets + p);
     cur ^= 1;
@@ -518,4 +549,24 @@ extern "C" int thrust_cdna4_sort_pairs(void* temp, size_t* temp_bytes, int key_d
     case 8: return (int)tcd::sort_dispatch<8>(temp, temp_bytes, key_dtype, keys, values, n, descending, s);
   }
   return hipErrorInvalidValue;
+}
+
+extern "C" int thrust_cdna4_selftest_lds_atomic_order(long long* mismatches, void* stream) {
+  using namespace tcd;
+  if (!mismatches) return hipErrorInvalidValue;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  unsigned long long* d = nullptr;
+  hipError_t e = hipMalloc(&d, sizeof(*d));
+  if (e != hipSuccess) return (int)e;
+  e = zero_async(d, sizeof(*d), s);
+  if (e == hipSuccess) {
+    TCD_LAUNCH("lds_atomic_order_kernel", lds_atomic_order_kernel, dim3(1024), dim3(512), s, d, 600);
+    e = hipGetLastError();
+  }
+  unsigned long long h = 0;
+  if (e == hipSuccess) e = hipMemcpyAsync(&h, d, sizeof(h), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  hipFree(d);
+  *mismatches = (long long)h;
+  return (int)e;
 }
