@@ -102,7 +102,7 @@ __device__ inline void store_group(E* p, const E (&src)[N]) {
 template <class T>
 struct SegGeom {
 #ifndef TCD_SEG_BLOCK
-#define TCD_SEG_BLOCK 256
+#define TCD_SEG_BLOCK 512
 #define TCD_SEG_CHUNKS 4
 #endif
   static constexpr int BLOCK = TCD_SEG_BLOCK;
@@ -123,10 +123,10 @@ struct SegTile {
   using G = SegGeom<T>;
   using Pair = SegPair<T>;
   static constexpr int VEC = G::VEC, CHUNKS = G::CHUNKS, NWAVES = G::NWAVES, BLOCK = G::BLOCK;
+  static_assert(CHUNKS * NWAVES <= kWave, "one wavefront scans the (chunk, wave) totals");
 
   struct Smem {
-    Pair tot[CHUNKS][NWAVES];
-    Pair prefix;
+    Pair tot[CHUNKS * NWAVES];  // inclusive total of (chunk, wave), then its prefix over the whole input
     uint32_t tile;
   };
 
@@ -158,12 +158,10 @@ struct SegTile {
     base = tile * G::TILE;
     full = vec_ok && (base + G::TILE < n);
 
-    KU prev[CHUNKS];
     if (full) {
 #pragma unroll
       for (int c = 0; c < CHUNKS; c++) {
         const int64_t i0 = index(c, 0);
-        prev[c] = i0 > 0 ? keys[i0 - 1] : KU(0);
         load_group<VEC>(keys + i0, key[c]);
         load_group<VEC>(vals + i0, val[c]);
       }
@@ -171,7 +169,6 @@ struct SegTile {
 #pragma unroll
       for (int c = 0; c < CHUNKS; c++) {
         const int64_t i0 = index(c, 0);
-        prev[c] = (i0 > 0 && i0 < n) ? keys[i0 - 1] : KU(0);
 #pragma unroll
         for (int j = 0; j < VEC; j++) {
           const int64_t idx = i0 + j;
@@ -179,6 +176,17 @@ struct SegTile {
           val[c][j] = idx < n ? vals[idx] : id;
         }
       }
+    }
+    // the key before a thread's group is the last key of the lane below (its group precedes this
+    // one in memory); only lane 0 of each wave fetches it from memory
+    using KW = typename std::conditional<(sizeof(KU) < 4), uint32_t, KU>::type;
+    KU prev[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+      const int64_t i0 = index(c, 0);
+      KU first = KU(0);
+      if (lane == 0 && i0 > 0 && i0 < n) first = keys[i0 - 1];
+      prev[c] = (KU)wave_shift_up1((KW)key[c][VEC - 1], (KW)first);
     }
 
     Pair excl_w[CHUNKS];
@@ -198,23 +206,17 @@ struct SegTile {
       agg.c = __builtin_popcount(h);
       const Pair w = wave_inclusive_scan(agg, idp, comb);
       excl_w[c] = wave_shift_up1(w, idp);
-      if (lane == kWave - 1) sm.tot[c][wave] = w;
+      if (lane == kWave - 1) sm.tot[c * NWAVES + wave] = w;
     }
     __syncthreads();
 
-    Pair seg_base[CHUNKS];
-    Pair run = idp;
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-#pragma unroll
-      for (int w = 0; w < NWAVES; w++) {
-        if (w == wave) seg_base[c] = run;
-        run = comb(run, sm.tot[c][w]);
-      }
-    }
-    const Pair tile_agg = run;
-
+    // wave 0: scan of the (chunk, wave) totals in tile order, look-back, then each (chunk, wave)'s
+    // prefix over the whole input goes back into the table
     if (wave == 0) {
+      const Pair mine = lane < CHUNKS * NWAVES ? sm.tot[lane] : idp;
+      const Pair incl = wave_inclusive_scan(mine, idp, comb);
+      const Pair tile_agg = readlane(incl, kWave - 1);
+      const Pair before = wave_shift_up1(incl, idp);
       Pair prefix = idp;
       if (tile == 0) {
         if (lane == 0) TileDesc<Pair>::store(desc, 0, kInclusive, tile_agg);
@@ -223,12 +225,11 @@ struct SegTile {
         prefix = wave_lookback<Pair>(desc, tile, idp, comb);
         if (lane == 0) TileDesc<Pair>::store(desc, tile, kInclusive, comb(prefix, tile_agg));
       }
-      if (lane == 0) sm.prefix = prefix;
+      if (lane < CHUNKS * NWAVES) sm.tot[lane] = comb(prefix, before);
     }
     __syncthreads();
-    const Pair prefix = sm.prefix;
 #pragma unroll
-    for (int c = 0; c < CHUNKS; c++) off[c] = comb(comb(prefix, seg_base[c]), excl_w[c]);
+    for (int c = 0; c < CHUNKS; c++) off[c] = comb(sm.tot[c * NWAVES + wave], excl_w[c]);
   }
 };
 
