@@ -56,6 +56,12 @@ __device__ inline bool keys_differ(KU a, KU b, int float_keys) {
   return a != b;
 }
 
+#ifndef TCD_RBK_ATTR
+#define TCD_RBK_ATTR
+#endif
+#ifndef TCD_SBK_ATTR
+#define TCD_SBK_ATTR
+#endif
 template <int BYTES> struct bits_of;
 template <> struct bits_of<1> { using type = uint8_t; };
 template <> struct bits_of<2> { using type = uint16_t; };
@@ -237,7 +243,7 @@ struct SegTile {
 // scan_by_key
 // ---------------------------------------------------------------------------------------
 template <class T, class Op>
-__global__ __launch_bounds__(SegGeom<T>::BLOCK) void scan_by_key_kernel(
+__global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_key_kernel(
     const KU* keys, const T* vals, T* out, int64_t n, T init, int exclusive, int float_keys, int vec_ok,
     uint64_t* desc, uint32_t* ticket) {
   using ST = SegTile<T, Op>;
@@ -272,7 +278,7 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) void scan_by_key_kernel(
 // reduce_by_key
 // ---------------------------------------------------------------------------------------
 template <class T, class Op>
-__global__ __launch_bounds__(SegGeom<T>::BLOCK) void reduce_by_key_kernel(
+__global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_RBK_ATTR void reduce_by_key_kernel(
     const KU* keys, const T* vals, KU* keys_out, T* vals_out, int64_t* num_runs, int64_t n,
     int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket) {
   using ST = SegTile<T, Op>;

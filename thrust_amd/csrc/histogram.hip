@@ -1,25 +1,24 @@
-// Even-bin histogram for gfx950: LDS-privatised, per-wave replicated sub-histograms merged
-// into global memory with atomics.  The reference has no histogram function; this is the
-// device counterpart of the pattern in examples/histogram.cu:60-101.
+// Even-bin histogram for gfx950: LDS-privatised counters, replicated per LANE, merged into
+// global memory with atomics.  The reference has no histogram function; this is the device
+// counterpart of the pattern in examples/histogram.cu:60-101.
 //
 // Bin mapping (identical on host and device, all in IEEE double without contraction):
 //   v = (double)x;  dropped unless lower <= v < upper;
 //   bin = (int)((v - lower) * scale), scale = num_bins / (upper - lower), clamped to num_bins-1.
 //
-// Contention: samples that share a bin within one wave instruction serialise in the LDS atomic
-// unit.  When a quarter or more of a wave's lanes hit the bin of its first lane ("hot" bin:
-// skewed data, e.g. Zipf ranks), those lanes are counted with one ballot and a single atomic,
-// and only the remaining lanes issue their own.
+// LDS layout: counter of (bin, copy) at word bin*copies + copy, copy = lane % copies, copies a
+// power of two <= 32.  With 32 copies (up to 512 bins) lane l always hits bank l % 32: no bank
+// conflicts and no two lanes of a half-wave on one address, whatever the data (uniform, a few
+// hot bins, constant).  Fewer copies (more bins) get one padding word per 32 so that bins hit
+// with a power-of-two stride do not fall into a few banks; there, samples that share a bin
+// within one instruction still serialise, and when a quarter or more of a wave's lanes hit the
+// bin of its first lane those lanes are counted with one ballot and a single atomic.
 #include "common.h"
 
 namespace tcd {
 
 constexpr int kHistBlock = 512;
-constexpr int kHistWaves = kHistBlock / kWave;
-
-// LDS slot of bin b: one padding word per 32 bins, so that bins hit with a power-of-two stride
-// (e.g. 8-bit samples spread over 4096 bins: every 16th bin) do not all fall into two banks.
-__host__ __device__ inline int lds_slot(int b) { return b + (b >> 5); }
+constexpr int kHistLdsWords = 16384;  // counters per workgroup (64 KiB); 16896 words with padding
 
 template <class T>
 __device__ inline int bin_of_sample(T x, double lower, double upper, double scale, int num_bins) {
@@ -29,69 +28,70 @@ __device__ inline int bin_of_sample(T x, double lower, double upper, double scal
   return b >= num_bins ? num_bins - 1 : b;
 }
 
-// LDS_WORDS > 0: counters live in LDS (replicated `reps` times, replica = wave % reps);
-//           = 0: counters are the global array itself (more bins than fit in LDS).
-// MODE 0: general mapping; 1: 1-byte samples through a 256-entry table built per workgroup;
-//      2: 1-byte unsigned samples whose bin is the sample value (lower 0, upper 256, 256 bins).
-template <class T, int LDS_WORDS, int MODE>
+// LDS > 0: counters live in LDS (LDS words, plus padding); LDS = 0: counters are the global
+// array itself (more bins than fit in LDS).
+// MODE 0: general mapping.  MODE 2 (1-byte samples): the workgroup counts the 256 raw byte
+// values (always 32 copies, conflict-free) and maps each value's count to its bin only when it
+// merges into global memory, so the per-sample work does not depend on the bin mapping at all.
+template <class T, int LDS, int MODE>
 __global__ __launch_bounds__(kHistBlock) void histogram_kernel(const T* __restrict__ samples, int64_t n,
                                                                uint32_t* counts, int num_bins, double lower,
-                                                               double upper, double scale, int reps,
+                                                               double upper, double scale, int copies_log2,
                                                                int vec_ok) {
   constexpr int VEC = 16 / sizeof(T);
-  __shared__ uint32_t s_hist[LDS_WORDS > 0 ? LDS_WORDS + LDS_WORDS / 32 : 1];
-  __shared__ int s_lut[MODE == 1 ? 256 : 1];
+  constexpr int kHistUnroll = sizeof(T) <= 2 ? 4 : 2;  // independent 128-bit loads in flight per thread
+  __shared__ uint32_t s_hist[LDS > 0 ? LDS + LDS / 32 : 1];
+  __shared__ uint32_t s_out[MODE == 2 ? 256 : 1];
   const int tid = threadIdx.x;
-  const int wave = tid / kWave;
+  const int lds_bins = MODE == 2 ? 256 : num_bins;  // counters kept per copy
+  const int copies = 1 << copies_log2;
+  const bool padded = copies < 32;
+  const uint32_t my_copy = (uint32_t)tid & (uint32_t)(copies - 1);
 
-  if constexpr (LDS_WORDS > 0) {
-    for (int i = tid; i < reps * lds_slot(num_bins); i += kHistBlock) s_hist[i] = 0;
-  }
-  if constexpr (MODE == 1) {
-    if (tid < 256) {
-      T x;
-      const uint8_t raw = (uint8_t)tid;
-      __builtin_memcpy(&x, &raw, 1);
-      s_lut[tid] = bin_of_sample<T>(x, lower, upper, scale, num_bins);
-    }
+  if constexpr (LDS > 0) {
+    const int words = (lds_bins << copies_log2) + (padded ? (lds_bins << copies_log2) >> 5 : 0);
+    for (int i = tid; i < words; i += kHistBlock) s_hist[i] = 0;
   }
   __syncthreads();
 
-  uint32_t* my = LDS_WORDS > 0 ? s_hist + (wave % reps) * lds_slot(num_bins) : counts;
-  auto slot = [](int b) { return LDS_WORDS > 0 ? lds_slot(b) : b; };
+  auto slot = [&](int b, uint32_t copy) -> uint32_t {
+    const uint32_t a = ((uint32_t)b << copies_log2) + copy;
+    return padded ? a + (a >> 5) : a;
+  };
   auto bin_of = [&](T x) -> int {
     if constexpr (MODE == 2) {
       uint8_t raw;
       __builtin_memcpy(&raw, &x, 1);
       return (int)raw;
-    } else if constexpr (MODE == 1) {
-      uint8_t raw;
-      __builtin_memcpy(&raw, &x, 1);
-      return s_lut[raw];
     } else {
       return bin_of_sample<T>(x, lower, upper, scale, num_bins);
     }
   };
+  auto add = [&](int b, uint32_t v) {
+    if constexpr (LDS > 0) atomicAdd(&s_hist[slot(b, my_copy)], v);
+    else atomicAdd(&counts[b], v);
+  };
   auto count_plain = [&](int b) {
-    if (MODE == 2 || b >= 0) atomicAdd(&my[slot(b)], 1u);
+    if (MODE == 2 || b >= 0) add(b, 1u);  // a raw byte value is always a valid counter
   };
   // counts the lanes sharing the first active lane's bin with one atomic, the rest one by one
   auto count_peeled = [&](int b) {
     const int hot = __builtin_amdgcn_readfirstlane(b);
     const uint64_t same = __builtin_amdgcn_ballot_w64(b == hot);
     if (b == hot) {
-      if (hot >= 0 && lane_id() == (int)__builtin_ctzll(same)) atomicAdd(&my[slot(hot)], (uint32_t)__popcll(same));
+      if (hot >= 0 && lane_id() == (int)__builtin_ctzll(same)) add(hot, (uint32_t)__popcll(same));
     } else if (b >= 0) {
-      atomicAdd(&my[slot(b)], 1u);
+      add(b, 1u);
     }
   };
   auto count_group = [&](const T (&v)[VEC]) {
     int b[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; j++) b[j] = bin_of(v[j]);
-    // skew test on the first sample of the group: decides the path for all of them
+    // skew test on the first sample of the group: decides the path for all of them (not
+    // needed with 16 or more copies, where lanes rarely share an address)
     const int hot = __builtin_amdgcn_readfirstlane(b[0]);
-    if (__popcll(__builtin_amdgcn_ballot_w64(b[0] == hot)) >= kWave / 4) {
+    if (copies_log2 < 4 && __popcll(__builtin_amdgcn_ballot_w64(b[0] == hot)) >= kWave / 4) {
 #pragma unroll
       for (int j = 0; j < VEC; j++) count_peeled(b[j]);
     } else {
@@ -106,7 +106,15 @@ __global__ __launch_bounds__(kHistBlock) void histogram_kernel(const T* __restri
     struct alignas(16) V16 { T v[VEC]; };
     const int64_t nvec = n / VEC;
     const V16* sv = reinterpret_cast<const V16*>(samples);
-    for (int64_t i = gtid; i < nvec; i += gstride) {
+    int64_t i = gtid;
+    for (; i + (kHistUnroll - 1) * gstride < nvec; i += kHistUnroll * gstride) {
+      V16 v[kHistUnroll];
+#pragma unroll
+      for (int u = 0; u < kHistUnroll; u++) v[u] = sv[i + u * gstride];
+#pragma unroll
+      for (int u = 0; u < kHistUnroll; u++) count_group(v[u].v);
+    }
+    for (; i < nvec; i += gstride) {
       const V16 v = sv[i];
       count_group(v.v);
     }
@@ -115,28 +123,54 @@ __global__ __launch_bounds__(kHistBlock) void histogram_kernel(const T* __restri
     for (int64_t i = gtid; i < n; i += gstride) count_plain(bin_of(samples[i]));
   }
 
-  if constexpr (LDS_WORDS > 0) {
+  if constexpr (LDS > 0) {
     __syncthreads();
-    for (int b = tid; b < num_bins; b += kHistBlock) {
-      uint32_t c = 0;
-      for (int r = 0; r < reps; r++) c += s_hist[r * lds_slot(num_bins) + lds_slot(b)];
-      if (c) atomicAdd(&counts[b], c);
+    if constexpr (MODE == 2) {
+      // counts of byte values -> bins.  Few bins: combine in LDS first, so that a workgroup
+      // sends one atomic per bin (global atomics on one cache line serialise).
+      const bool combine = num_bins <= 256;
+      if (combine && tid < 256) s_out[tid] = 0;
+      if (combine) __syncthreads();
+      if (tid < 256) {
+        uint32_t c = 0;
+        for (int r = 0; r < 32; r++) c += s_hist[(tid << 5) + ((r + tid) & 31)];  // rotated: no bank conflicts
+        T x;
+        const uint8_t raw = (uint8_t)tid;
+        __builtin_memcpy(&x, &raw, 1);
+        const int bin = bin_of_sample<T>(x, lower, upper, scale, num_bins);
+        if (c && bin >= 0) {
+          if (combine) atomicAdd(&s_out[bin], c);
+          else atomicAdd(&counts[bin], c);
+        }
+      }
+      if (combine) {
+        __syncthreads();
+        if (tid < num_bins && s_out[tid]) atomicAdd(&counts[tid], s_out[tid]);
+      }
+    } else {
+      for (int b = tid; b < num_bins; b += kHistBlock) {
+        uint32_t c = 0;
+        // rotated by the bin so that the threads of a wave read different banks
+        for (int r = 0; r < copies; r++) c += s_hist[slot(b, (uint32_t)(r + b) & (uint32_t)(copies - 1))];
+        if (c) atomicAdd(&counts[b], c);
+      }
     }
   }
 }
 
-template <class T, int LDS_WORDS, int MODE>
+template <class T, int LDS, int MODE>
 static void launch_hist(const T* samples, int64_t n, uint32_t* counts, int num_bins, double lower, double upper,
                         double scale, int vec_ok, int blocks_per_cu, hipStream_t s) {
-  int reps = LDS_WORDS > 0 ? (LDS_WORDS + LDS_WORDS / 32) / lds_slot(num_bins) : 1;
-  if (reps < 1) reps = 1;
-  if (reps > kHistWaves) reps = kHistWaves;
+  const int lds_bins = MODE == 2 ? 256 : num_bins;
+  int copies_log2 = 0;
+  if (LDS > 0)
+    while (copies_log2 < 5 && ((int64_t)lds_bins << (copies_log2 + 1)) <= LDS) copies_log2++;
   int64_t blocks = ceil_div(n, (int64_t)kHistBlock * (16 / (int)sizeof(T)) * 4);
   const int64_t cap = 256 * (int64_t)blocks_per_cu;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
-  TCD_LAUNCH("histogram_kernel", (histogram_kernel<T, LDS_WORDS, MODE>), dim3((unsigned)blocks), dim3(kHistBlock), s,
-             samples, n, counts, num_bins, lower, upper, scale, reps, vec_ok);
+  TCD_LAUNCH("histogram_kernel", (histogram_kernel<T, LDS, MODE>), dim3((unsigned)blocks), dim3(kHistBlock), s,
+             samples, n, counts, num_bins, lower, upper, scale, copies_log2, vec_ok);
 }
 
 template <class T>
@@ -147,16 +181,17 @@ static hipError_t histogram_typed(const void* samples_, int64_t n, uint32_t* cou
   const T* samples = static_cast<const T*>(samples_);
   const double scale = (double)num_bins / (upper - lower);
   const int vec_ok = (reinterpret_cast<uintptr_t>(samples) & 15) == 0;
-  constexpr bool kByte = sizeof(T) == 1;
-  const bool identity8 = std::is_same<T, uint8_t>::value && num_bins == 256 && lower == 0.0 && upper == 256.0;
-  // two LDS footprints: 8 KiB (four workgroups per CU) for up to 2048 counters, 64 KiB otherwise
-  if (num_bins <= 2048) {  // (the LDS arrays carry the padding words on top of these sizes)
-    if (identity8) launch_hist<T, 2048, kByte ? 2 : 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 4, s);
-    else launch_hist<T, 2048, kByte ? 1 : 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 4, s);
-  } else if (num_bins <= 16384) {
-    launch_hist<T, 16384, kByte ? 1 : 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 2, s);
+  // two LDS footprints: 32 KiB while 32 copies of every counter fit (always the case for 1-byte
+  // samples), 64 KiB up to 16384 bins; beyond that the counts go straight to global memory.
+  // Workgroups per CU as measured: four for 1-byte samples, two otherwise.
+  if constexpr (sizeof(T) == 1) {
+    launch_hist<T, 8192, 2>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 4, s);
+  } else if (num_bins <= 256) {
+    launch_hist<T, 8192, 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 2, s);
+  } else if (num_bins <= kHistLdsWords) {
+    launch_hist<T, kHistLdsWords, 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 2, s);
   } else {
-    launch_hist<T, 0, kByte ? 1 : 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 4, s);
+    launch_hist<T, 0, 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 4, s);
   }
   return hipGetLastError();
 }
