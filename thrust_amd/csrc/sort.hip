@@ -1,7 +1,8 @@
 // Onesweep least-significant-digit radix sort for gfx950.
 //
 //   1. radix_hist_kernel   one read of the keys; LDS-privatised 256-bin histograms of ALL
-//                          digit places, merged into global memory with atomics.
+//                          digit places (replicated per lane), merged into global memory
+//                          with atomics.
 //   2. radix_bins_kernel   exclusive scan of each digit place's 256 bins.
 //   3. onesweep_kernel     one launch per 8-bit digit.  A workgroup takes a tile by ticket,
 //                          ranks its keys stably (returning LDS atomics on per-wave digit
@@ -69,52 +70,74 @@ __device__ __host__ inline U decode_key(U e, U xor_mask) {
 // ---------------------------------------------------------------------------------------
 // 1. Histogram of every digit place
 // ---------------------------------------------------------------------------------------
+// Counters are replicated per lane: the counter of (place, digit, copy) lives at word
+// (place*256 + digit)*COPIES + copy with copy = lane % COPIES, so the lanes of a wave spread
+// over the LDS banks whatever the keys are (random, sorted, constant) instead of meeting on
+// the few banks their digits select.  64 KiB per workgroup: 16 copies for 4-byte keys, 8 for
+// 8-byte keys, 32 for narrower ones.
+#ifndef TCD_SORT_HIST_BLOCKS
+#define TCD_SORT_HIST_BLOCKS 512
+#endif
+constexpr int kHistThreads = 512;
+template <class U>
+struct RadixHistGeom {
+  static constexpr int P = sizeof(U);
+  static constexpr int COPIES = 16384 / (P * kRadix) > 32 ? 32 : 16384 / (P * kRadix);
+};
+
 template <class U, bool FLOAT>
-__global__ __launch_bounds__(256) void radix_hist_kernel(const U* __restrict__ keys, int64_t n,
-                                                         U xor_mask, uint32_t* ghist, int vec_ok) {
-  constexpr int P = sizeof(U);
+__global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const U* __restrict__ keys, int64_t n,
+                                                                  U xor_mask, uint32_t* ghist, int vec_ok) {
+  constexpr int P = RadixHistGeom<U>::P;
+  constexpr int COPIES = RadixHistGeom<U>::COPIES;
   constexpr int VEC = 16 / sizeof(U);
-  __shared__ uint32_t h[P][kRadix];
+  constexpr int UNROLL = 2;
+  __shared__ uint32_t h[P * kRadix * COPIES];
   const int tid = threadIdx.x;
-#pragma unroll
-  for (int p = 0; p < P; p++) h[p][tid] = 0;
+  for (int i = tid; i < P * kRadix * COPIES; i += kHistThreads) h[i] = 0;
   __syncthreads();
 
+  uint32_t* mine = h + (tid & (COPIES - 1));
   auto count = [&](U k) {
     const U e = encode_key<U, FLOAT>(k, xor_mask);
 #pragma unroll
     for (int p = 0; p < P; p++) {
       const uint32_t d = (uint32_t)(e >> (8 * p)) & 0xffu;
-      // all active lanes on one digit (sorted / low-entropy keys): one atomic for the wave
-      const uint64_t active = __builtin_amdgcn_ballot_w64(true);
-      if (__builtin_amdgcn_ballot_w64(d != (uint32_t)__builtin_amdgcn_readfirstlane((int)d)) == 0) {
-        if (lane_id() == (int)__builtin_ctzll(active)) atomicAdd(&h[p][d], (uint32_t)__popcll(active));
-      } else {
-        atomicAdd(&h[p][d], 1u);
-      }
+      atomicAdd(mine + (p * kRadix + d) * COPIES, 1u);
     }
   };
 
-  const int64_t gtid = (int64_t)blockIdx.x * blockDim.x + tid;
-  const int64_t gstride = (int64_t)gridDim.x * blockDim.x;
+  const int64_t gtid = (int64_t)blockIdx.x * kHistThreads + tid;
+  const int64_t gstride = (int64_t)gridDim.x * kHistThreads;
   if (vec_ok) {
     struct alignas(16) V16 { U v[VEC]; };
     const int64_t nvec = n / VEC;
     const V16* kv = reinterpret_cast<const V16*>(keys);
-    for (int64_t i = gtid; i < nvec; i += gstride) {
-      V16 v = kv[i];
+    int64_t i = gtid;
+    for (; i + (UNROLL - 1) * gstride < nvec; i += UNROLL * gstride) {
+      V16 v[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; u++) v[u] = kv[i + u * gstride];
+#pragma unroll
+      for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+        for (int j = 0; j < VEC; j++) count(v[u].v[j]);
+    }
+    for (; i < nvec; i += gstride) {
+      const V16 v = kv[i];
 #pragma unroll
       for (int j = 0; j < VEC; j++) count(v.v[j]);
     }
-    for (int64_t i = nvec * VEC + gtid; i < n; i += gstride) count(keys[i]);
+    for (int64_t r = nvec * VEC + gtid; r < n; r += gstride) count(keys[r]);
   } else {
-    for (int64_t i = gtid; i < n; i += gstride) count(keys[i]);
+    for (int64_t r = gtid; r < n; r += gstride) count(keys[r]);
   }
   __syncthreads();
+  for (int b = tid; b < P * kRadix; b += kHistThreads) {
+    uint32_t c = 0;
 #pragma unroll
-  for (int p = 0; p < P; p++) {
-    const uint32_t c = h[p][tid];
-    if (c) atomicAdd(&ghist[p * kRadix + tid], c);
+    for (int r = 0; r < COPIES; r++) c += h[b * COPIES + ((r + b) & (COPIES - 1))];  // rotated: spread over banks
+    if (c) atomicAdd(&ghist[b], c);
   }
 }
 
@@ -476,9 +499,9 @@ static hipError_t sort_typed(void* temp, size_t* temp_bytes, void* keys, void* v
   if (e != hipSuccess) return e;
 
   const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & 15) == 0;
-  int64_t hblocks = ceil_div(n, 256 * 64);
-  if (hblocks > 2048) hblocks = 2048;
-  TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(256), stream,
+  int64_t hblocks = ceil_div(n, kHistThreads * 64);
+  if (hblocks > TCD_SORT_HIST_BLOCKS) hblocks = TCD_SORT_HIST_BLOCKS;  // two workgroups per CU
+  TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(kHistThreads), stream,
              kbuf[0], n, xor_mask, ghist, vec_ok);
   TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(P), dim3(256), stream, ghist);
   int cur = 0;
