@@ -56,11 +56,13 @@ __device__ inline bool keys_differ(KU a, KU b, int float_keys) {
   return a != b;
 }
 
+// Both kernels are compiled for 4 wavefronts per SIMD (at most 128 VGPRs): two 512-thread
+// workgroups per CU.  Left alone, the register allocator may trade that occupancy away.
 #ifndef TCD_RBK_ATTR
-#define TCD_RBK_ATTR
+#define TCD_RBK_ATTR __attribute__((amdgpu_waves_per_eu(4)))
 #endif
 #ifndef TCD_SBK_ATTR
-#define TCD_SBK_ATTR
+#define TCD_SBK_ATTR __attribute__((amdgpu_waves_per_eu(4)))
 #endif
 template <int BYTES> struct bits_of;
 template <> struct bits_of<1> { using type = uint8_t; };
@@ -101,32 +103,45 @@ __device__ inline void store_group(E* p, const E (&src)[N]) {
   }
 }
 
-// Geometry shared by both kernels: a thread owns VEC consecutive elements of each of CHUNKS
-// chunks; the wider of key and value fills 32 bytes per thread and chunk (two 128-bit accesses),
-// capped at 16 elements.  Long per-thread groups keep the cross-lane scans (one per chunk) cheap
-// per element.
-template <class T>
+// Tile geometry: a thread owns VEC consecutive elements of each of CHUNKS chunks; the wider of
+// key and value fills GROUP_BYTES per thread and chunk, capped at 16 elements.  Measured on
+// MI355X, 16-byte groups (one 128-bit access; every wave access is one contiguous 1 KiB
+// segment) with 8 chunks beat 32- and 64-byte groups for both kernels.
+template <class T, int GROUP_BYTES, int CHUNKS_>
 struct SegGeom {
 #ifndef TCD_SEG_BLOCK
 #define TCD_SEG_BLOCK 512
-#define TCD_SEG_CHUNKS 4
 #endif
   static constexpr int BLOCK = TCD_SEG_BLOCK;
   static constexpr int WIDE = (int)(sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T));
-  static constexpr int VEC = 32 / WIDE > 16 ? 16 : 32 / WIDE;
-  static constexpr int CHUNKS = TCD_SEG_CHUNKS;
+  static constexpr int VEC = GROUP_BYTES / WIDE > 16 ? 16 : GROUP_BYTES / WIDE;
+  // at most 32 elements per thread: narrow types hold one element per register
+  static constexpr int CHUNKS = VEC * CHUNKS_ > 32 ? 32 / VEC : CHUNKS_;
   static constexpr int NWAVES = BLOCK / kWave;
   static constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
 };
+#ifndef TCD_SBK_GROUP
+#define TCD_SBK_GROUP 16
+#endif
+#ifndef TCD_SBK_CHUNKS
+#define TCD_SBK_CHUNKS 8
+#endif
+#ifndef TCD_RBK_GROUP
+#define TCD_RBK_GROUP 16
+#endif
+#ifndef TCD_RBK_CHUNKS
+#define TCD_RBK_CHUNKS 8
+#endif
+template <class T> using ScanByKeyGeom = SegGeom<T, TCD_SBK_GROUP, TCD_SBK_CHUNKS>;
+template <class T> using ReduceByKeyGeom = SegGeom<T, TCD_RBK_GROUP, TCD_RBK_CHUNKS>;
 
 // Loads a tile, finds the segment heads, reduces it and resolves the prefix of all earlier
 // tiles by look-back.  On return key/val hold the thread's elements, bit j of heads[c] says
 // whether element (c, j) starts a segment, and off[c] is the pair (heads seen, value of the
 // open segment) of everything before the thread's group of chunk c.  The kernels then walk
 // their elements once more from off[c]; nothing per element is kept in between.
-template <class T, class Op>
+template <class T, class Op, class G>
 struct SegTile {
-  using G = SegGeom<T>;
   using Pair = SegPair<T>;
   static constexpr int VEC = G::VEC, CHUNKS = G::CHUNKS, NWAVES = G::NWAVES, BLOCK = G::BLOCK;
   static_assert(CHUNKS * NWAVES <= kWave, "one wavefront scans the (chunk, wave) totals");
@@ -243,10 +258,10 @@ struct SegTile {
 // scan_by_key
 // ---------------------------------------------------------------------------------------
 template <class T, class Op>
-__global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_key_kernel(
+__global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_key_kernel(
     const KU* keys, const T* vals, T* out, int64_t n, T init, int exclusive, int float_keys, int vec_ok,
     uint64_t* desc, uint32_t* ticket) {
-  using ST = SegTile<T, Op>;
+  using ST = SegTile<T, Op, ScanByKeyGeom<T>>;
   __shared__ typename ST::Smem sm;
   ST t;
   t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket);
@@ -278,10 +293,10 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_key_ke
 // reduce_by_key
 // ---------------------------------------------------------------------------------------
 template <class T, class Op>
-__global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_RBK_ATTR void reduce_by_key_kernel(
+__global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce_by_key_kernel(
     const KU* keys, const T* vals, KU* keys_out, T* vals_out, int64_t* num_runs, int64_t n,
     int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket) {
-  using ST = SegTile<T, Op>;
+  using ST = SegTile<T, Op, ReduceByKeyGeom<T>>;
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS, NWAVES = ST::NWAVES;
   __shared__ typename ST::Smem sm;
   // Per-wave staging of one chunk's output: the heads of a wave's 64*VEC consecutive elements go
@@ -327,9 +342,9 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_RBK_ATTR void reduce_by_key_
   }
 }
 
-template <class T>
+template <class T, class G>
 static size_t bykey_temp_bytes(int64_t n) {
-  const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
+  const int64_t ntiles = ceil_div(n, G::TILE);
   return 256 + align_up((size_t)ntiles * TileDesc<SegPair<T>>::kBytesPerTile, 256);
 }
 
@@ -351,7 +366,7 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
     using T = decltype(tv);
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
-      const size_t need = bykey_temp_bytes<T>(n);
+      const size_t need = bykey_temp_bytes<T, ScanByKeyGeom<T>>(n);
       if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
       if (*temp_bytes < need) return;
       if (n == 0) { rc = hipSuccess; return; }
@@ -361,8 +376,8 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
       if (init) __builtin_memcpy(&iv, init, sizeof(T));
       const int vec_ok = ((reinterpret_cast<uintptr_t>(keys) | reinterpret_cast<uintptr_t>(values) |
                            reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-      const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
-      TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
+      const int64_t ntiles = ceil_div(n, ScanByKeyGeom<T>::TILE);
+      TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(ScanByKeyGeom<T>::BLOCK), s,
                          static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
                          n, iv, exclusive, float_keys, vec_ok,
                          reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
@@ -385,7 +400,7 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
     using T = decltype(tv);
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
-      const size_t need = bykey_temp_bytes<T>(n);
+      const size_t need = bykey_temp_bytes<T, ReduceByKeyGeom<T>>(n);
       if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
       if (*temp_bytes < need) return;
       if (n == 0) {  // no runs: only the count is written
@@ -395,8 +410,8 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
       rc = zero_async(temp, need, s);
       if (rc != hipSuccess) return;
       const int vec_ok = ((reinterpret_cast<uintptr_t>(keys_in) | reinterpret_cast<uintptr_t>(values_in)) & 15) == 0;
-      const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
-      TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
+      const int64_t ntiles = ceil_div(n, ReduceByKeyGeom<T>::TILE);
+      TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(ReduceByKeyGeom<T>::BLOCK), s,
                          static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
                          static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
                          vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
