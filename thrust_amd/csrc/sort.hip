@@ -274,13 +274,9 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
 
   // ---- per digit (thread d): tile count, publish it, first local slot of each wave's keys
   uint32_t total = 0, lbase = 0;
-  uint32_t wexcl[NWAVES];
   if (tid < kRadix) {
 #pragma unroll
-    for (int w = 0; w < NWAVES; w++) {
-      wexcl[w] = total;
-      total += sm.wave_cnt[w][tid];
-    }
+    for (int w = 0; w < NWAVES; w++) total += sm.wave_cnt[w][tid];
     const uint32_t st = (tile == 0) ? kInclusive : kPartial;
     st_agent(&desc[tile * kRadix + tid], (st << 30) | total);
     const uint32_t incl = wave_inclusive_scan(total, 0u, [](uint32_t a, uint32_t b) { return a + b; });
@@ -290,8 +286,13 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
   __syncthreads();
   if (tid < kRadix) {
     for (int w = 0; w < wave; w++) lbase += sm.wave_tot[w];
+    uint32_t run = lbase;  // counts -> first local slot of each wave's keys of this digit
 #pragma unroll
-    for (int w = 0; w < NWAVES; w++) sm.wave_cnt[w][tid] = lbase + wexcl[w];
+    for (int w = 0; w < NWAVES; w++) {
+      const uint32_t c = sm.wave_cnt[w][tid];
+      sm.wave_cnt[w][tid] = run;
+      run += c;
+    }
   }
   __syncthreads();
 
@@ -416,12 +417,13 @@ struct SortConfig {
   // Tile shape by bytes moved per item (key + value), measured on MI355X at n = 2^28.  The
   // time of a pass grows by about 9 ns per tile (ticket, barriers, descriptor traffic and
   // look-back latency do not shrink with the tile), so tiles are as large as LDS and registers
-  // allow: 4-byte items run two 1024-thread workgroups per CU at 64 VGPRs.
+  // allow: 4-byte items run two 1024-thread workgroups per CU (15 keys per thread, 64 VGPRs,
+  // 77 KiB of LDS each).
 #ifndef TCD_SORT_A_BLOCK
 #define TCD_SORT_A_BLOCK 1024
 #endif
 #ifndef TCD_SORT_A_IPT
-#define TCD_SORT_A_IPT 14
+#define TCD_SORT_A_IPT 15
 #endif
 #ifndef TCD_SORT_B_BLOCK
 #define TCD_SORT_B_BLOCK 1024
