@@ -173,3 +173,33 @@ def test_sort_skewed_digits_stability():
         k, v = dev(keys), dev(vals)
         thrust_amd.sort_by_key(k, v, False)
         assert same_bits(host(k), ek) and same_bits(host(v), ev), hot_frac
+
+
+@pytest.mark.parametrize("dtype", INT_DTYPES + FLOAT_DTYPES)
+def test_sort_keys_large_tiles_all_types(dtype):
+    """Inputs of 2^21 keys and more run the large-tile kernels (smaller ones the 512 x 16 tiles);
+    every key type goes through them here, with a ragged last tile."""
+    n = (1 << 21) + 1234
+    for descending in (False, True):
+        k = random_floats(n, n, dtype) if np.dtype(dtype).kind == "f" else random_ints(11 + n, n, dtype)
+        d = dev(k)
+        thrust_amd.sort(d, descending)
+        assert same_bits(host(d), oracle.sort_keys(k, descending)), descending
+
+
+@pytest.mark.parametrize("kd,vd", [(np.uint64, np.uint32), (np.uint32, np.uint32), (np.int32, np.uint64),
+                                   (np.int8, np.uint16), (np.uint16, np.uint8), (np.float32, np.uint32),
+                                   (np.float64, np.uint64), (np.int64, np.uint8), (np.uint32, np.uint8)])
+def test_sort_pairs_large_tiles_stability(kd, vd):
+    """2^22 pairs and more run the large-tile kernels; duplicate-heavy keys check stability."""
+    n = (1 << 22) + 77
+    for descending, spread in ((False, 41), (True, 70001)):
+        if np.dtype(kd).kind == "f":
+            k = (np.random.default_rng(n).integers(-spread, spread, n) / 4).astype(kd)
+        else:
+            k = (splitmix64(n, n) % np.uint64(spread)).astype(kd)
+        v = (np.arange(n) % (1 << (8 * np.dtype(vd).itemsize))).astype(vd) if np.dtype(vd).itemsize < 4 else np.arange(n).astype(vd)
+        dk, dv = dev(k), dev(v)
+        thrust_amd.sort_by_key(dk, dv, descending)
+        rk, rv = oracle.sort_pairs(k, v, descending)
+        assert same_bits(host(dk), rk) and same_bits(host(dv), rv), descending

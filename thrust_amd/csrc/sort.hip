@@ -171,7 +171,7 @@ struct OnesweepSmem {
   static constexpr int TILE = BLOCK * IPT;
   static constexpr int ELEM = (int)sizeof(U) > VB ? (int)sizeof(U) : VB;
   alignas(16) unsigned char exch[(size_t)TILE * ELEM];  // key / value exchange buffer
-  uint32_t wave_cnt[BLOCK / kWave][kRadix];             // per-wave digit counts, then next free local slots
+  uint16_t wave_cnt[BLOCK / kWave][kRadix];             // per-wave digit counts (two per LDS word), then first local slots
   uint32_t global_off[kRadix];                          // global slot of local slot 0, per digit
   uint32_t wave_tot[4];
   uint32_t tile;
@@ -205,9 +205,9 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
   const int wave = tid / kWave;
 
   if (tid == 0) sm.tile = atomicAdd(ticket, 1u);
-  if (tid < kRadix) {
+  if (tid < kRadix / 2) {
 #pragma unroll
-    for (int w = 0; w < NWAVES; w++) sm.wave_cnt[w][tid] = 0;
+    for (int w = 0; w < NWAVES; w++) reinterpret_cast<uint32_t*>(sm.wave_cnt[w])[tid] = 0;
   }
   __syncthreads();
   const int64_t tile = sm.tile;
@@ -239,8 +239,18 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
   //      the returned values number a digit's keys in (item, lane) order, which is the memory
   //      order of the wave's slab: the ranking is stable.  Afterwards the counters hold the
   //      per-wave digit counts, published before the reorder so that later tiles rarely wait.
-  uint32_t* wc = sm.wave_cnt[wave];
-  uint32_t pos[IPT];
+  // Counters are 16 bits wide (a wave holds at most 64*IPT keys), two digits per LDS word: the
+  // atomic adds 1 to the half of the key's digit and the rank is that half of the old value.
+  // Ranks are kept two per register until the reorder.
+  static_assert(kWave * IPT < 65536 && TILE < 65536, "16-bit counters and local slots");
+  uint32_t* wc = reinterpret_cast<uint32_t*>(sm.wave_cnt[wave]);
+  const uint16_t* wc16 = sm.wave_cnt[wave];
+  uint32_t rk[(IPT + 1) / 2];
+  auto keep_rank = [&](int i, uint32_t old, uint32_t sh) {
+    const uint32_t r = (old >> sh) & 0xffffu;
+    if (i & 1) rk[i / 2] |= r << 16;
+    else rk[i / 2] = r;
+  };
   {
     // A wave whose 64 keys share one digit (sorted or low-entropy input) would serialise 64
     // same-address atomics.  The first item decides which loop the wave runs (random keys pay
@@ -251,20 +261,25 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
                              f == (uint32_t)__builtin_amdgcn_readfirstlane((int)f))) >= kWave / 4;
     if (!careful) {
 #pragma unroll
-      for (int i = 0; i < IPT; i++) pos[i] = atomicAdd(wc + digit_of(k[i]), 1u);
+      for (int i = 0; i < IPT; i++) {
+        const uint32_t d = digit_of(k[i]);
+        const uint32_t sh = (d & 1u) << 4;
+        keep_rank(i, atomicAdd(wc + (d >> 1), 1u << sh), sh);
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < IPT; i++) {
         const uint32_t d = digit_of(k[i]);
+        const uint32_t sh = (d & 1u) << 4;
         const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
         const uint64_t same = __builtin_amdgcn_ballot_w64(d == d0);
         if (d == d0) {
-          const uint32_t old = lds_load(wc + d0);
+          const uint32_t old = lds_load(wc + (d0 >> 1));
           const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(same >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)same, 0u));
-          if (below == 0) lds_store(wc + d0, old + (uint32_t)__builtin_popcountll(same));
-          pos[i] = old + below;
+          if (below == 0) lds_store(wc + (d0 >> 1), old + ((uint32_t)__builtin_popcountll(same) << sh));
+          keep_rank(i, old + (below << sh), sh);
         } else {
-          pos[i] = atomicAdd(wc + d, 1u);
+          keep_rank(i, atomicAdd(wc + (d >> 1), 1u << sh), sh);
         }
         __builtin_amdgcn_wave_barrier();
       }
@@ -290,16 +305,18 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
 #pragma unroll
     for (int w = 0; w < NWAVES; w++) {
       const uint32_t c = sm.wave_cnt[w][tid];
-      sm.wave_cnt[w][tid] = run;
+      sm.wave_cnt[w][tid] = (uint16_t)run;
       run += c;
     }
   }
   __syncthreads();
 
   // ---- reorder: local slot = first slot of the wave's keys of that digit + rank
+  uint32_t pos[IPT];
 #pragma unroll
   for (int i = 0; i < IPT; i++) {
-    pos[i] += wc[digit_of(k[i])];
+    const uint32_t r = (i & 1) ? rk[i / 2] >> 16 : rk[i / 2] & 0xffffu;
+    pos[i] = r + wc16[digit_of(k[i])];
     s_keys[pos[i]] = k[i];
   }
 
@@ -412,47 +429,56 @@ __global__ __launch_bounds__(512) void lds_atomic_order_kernel(unsigned long lon
 // ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
-template <class U, int VB>
+template <class U, int VB, bool SMALL>
 struct SortConfig {
-  // Tile shape by bytes moved per item (key + value), measured on MI355X at n = 2^28.  The
-  // time of a pass grows by about 9 ns per tile (ticket, barriers, descriptor traffic and
-  // look-back latency do not shrink with the tile), so tiles are as large as LDS and registers
-  // allow: 4-byte items run two 1024-thread workgroups per CU (15 keys per thread, 64 VGPRs,
-  // 77 KiB of LDS each).
-#ifndef TCD_SORT_A_BLOCK
-#define TCD_SORT_A_BLOCK 1024
+  // Tile shape by the widest element that goes through the LDS exchange buffer and by whether
+  // values follow the keys, measured on MI355X at n = 2^28.  The time of a pass grows by about
+  // 9 ns per tile (ticket, barriers, descriptor traffic and look-back latency do not shrink
+  // with the tile) and longer per-digit runs write fuller cache lines, so tiles are as large as
+  // LDS and registers allow: one 1024-thread workgroup per CU with up to 128 VGPRs and
+  // 120-155 KiB of LDS (32768 keys of up to 4 bytes, with or without values; 18432 wider ones).
+#ifndef TCD_SORT_SMALL_IPT
+#define TCD_SORT_SMALL_IPT 16
 #endif
 #ifndef TCD_SORT_A_IPT
-#define TCD_SORT_A_IPT 15
-#endif
-#ifndef TCD_SORT_B_BLOCK
-#define TCD_SORT_B_BLOCK 1024
-#endif
-#ifndef TCD_SORT_B_IPT
-#define TCD_SORT_B_IPT 16
-#endif
-#ifndef TCD_SORT_C_BLOCK
-#define TCD_SORT_C_BLOCK 1024
-#endif
-#ifndef TCD_SORT_C_IPT
-#define TCD_SORT_C_IPT 12
+#define TCD_SORT_A_IPT 32
 #endif
 #ifndef TCD_SORT_A_WPE
-#define TCD_SORT_A_WPE 8
+#define TCD_SORT_A_WPE 4
+#endif
+#ifndef TCD_SORT_P_IPT
+#define TCD_SORT_P_IPT 32
+#endif
+#ifndef TCD_SORT_P_WPE
+#define TCD_SORT_P_WPE 4
+#endif
+#ifndef TCD_SORT_B_IPT
+#define TCD_SORT_B_IPT 18
 #endif
 #ifndef TCD_SORT_B_WPE
 #define TCD_SORT_B_WPE 4
 #endif
+#ifndef TCD_SORT_C_IPT
+#define TCD_SORT_C_IPT 18
+#endif
 #ifndef TCD_SORT_C_WPE
 #define TCD_SORT_C_WPE 4
 #endif
-  static constexpr int BYTES = (int)sizeof(U) + VB;
-  static constexpr int BLOCK = BYTES <= 4 ? TCD_SORT_A_BLOCK : (BYTES <= 8 ? TCD_SORT_B_BLOCK : TCD_SORT_C_BLOCK);
-  static constexpr int IPT = BYTES <= 4 ? TCD_SORT_A_IPT : (BYTES <= 8 ? TCD_SORT_B_IPT : TCD_SORT_C_IPT);
+  static constexpr int ELEM = (int)sizeof(U) > VB ? (int)sizeof(U) : VB;
+  static constexpr int CLASS = ELEM <= 4 ? (VB == 0 ? 0 : 1) : (VB == 0 ? 2 : 3);  // A, P, B, C
+  // Inputs too small to give every CU a few of those tiles use 512 x 16 tiles instead.
+  static constexpr int BLOCK = SMALL ? 512 : 1024;
+  static constexpr int IPT = SMALL ? TCD_SORT_SMALL_IPT
+                                   : CLASS == 0 ? TCD_SORT_A_IPT : CLASS == 1 ? TCD_SORT_P_IPT : CLASS == 2 ? TCD_SORT_B_IPT : TCD_SORT_C_IPT;
   static constexpr int TILE = BLOCK * IPT;
   // wavefronts per SIMD the register allocation aims for
-  static constexpr int WPE = BYTES <= 4 ? TCD_SORT_A_WPE : (BYTES <= 8 ? TCD_SORT_B_WPE : TCD_SORT_C_WPE);
+  static constexpr int WPE = SMALL ? 4 : CLASS == 0 ? TCD_SORT_A_WPE : CLASS == 1 ? TCD_SORT_P_WPE : CLASS == 2 ? TCD_SORT_B_WPE : TCD_SORT_C_WPE;
 };
+// Below this many items the small tiles are faster (measured crossover: 2^21 keys, 2^22 pairs).
+#ifndef TCD_SORT_SMALL_LOG2N
+#define TCD_SORT_SMALL_LOG2N 21
+#endif
+constexpr int64_t small_sort_limit(int value_bytes) { return int64_t(1) << (TCD_SORT_SMALL_LOG2N + (value_bytes ? 1 : 0)); }
 
 struct SortPlan {
   size_t keys_alt, vals_alt, hist, tickets, desc, total;
@@ -460,9 +486,8 @@ struct SortPlan {
   int64_t ntiles;
 };
 
-template <class U, int VB>
+template <class U, int VB, class C>
 static SortPlan make_plan(int64_t n) {
-  using C = SortConfig<U, VB>;
   constexpr int P = sizeof(U);
   SortPlan p{};
   p.ntiles = ceil_div(n, C::TILE);
@@ -478,12 +503,11 @@ static SortPlan make_plan(int64_t n) {
   return p;
 }
 
-template <class U, int VB, bool FLOAT>
-static hipError_t sort_typed(void* temp, size_t* temp_bytes, void* keys, void* values, int64_t n,
-                             U xor_mask, hipStream_t stream) {
-  using C = SortConfig<U, VB>;
+template <class U, int VB, bool FLOAT, class C>
+static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* values, int64_t n,
+                            U xor_mask, hipStream_t stream) {
   constexpr int P = sizeof(U);
-  const SortPlan plan = make_plan<U, VB>(n);
+  const SortPlan plan = make_plan<U, VB, C>(n);
   if (temp == nullptr) {
     *temp_bytes = plan.total;
     return hipSuccess;
@@ -521,6 +545,14 @@ static hipError_t sort_typed(void* temp, size_t* temp_bytes, void* keys, void* v
     if (VB) e = hipMemcpyAsync(vbuf[0], vbuf[1], (size_t)n * VB, hipMemcpyDeviceToDevice, stream);
   }
   return e;
+}
+
+template <class U, int VB, bool FLOAT>
+static hipError_t sort_typed(void* temp, size_t* temp_bytes, void* keys, void* values, int64_t n,
+                             U xor_mask, hipStream_t stream) {
+  // the choice depends on n only, so the size query and the run agree
+  if (n < small_sort_limit(VB)) return sort_with<U, VB, FLOAT, SortConfig<U, VB, true>>(temp, temp_bytes, keys, values, n, xor_mask, stream);
+  return sort_with<U, VB, FLOAT, SortConfig<U, VB, false>>(temp, temp_bytes, keys, values, n, xor_mask, stream);
 }
 
 template <int VB>
