@@ -180,6 +180,31 @@ __device__ inline T wave_shift_up1(const T& incl, const T id) {
   return lane == 0 ? id : out;
 }
 
+// 16-byte streaming accesses.  Data that a kernel touches exactly once is loaded and stored
+// with the non-temporal hint, which keeps it from displacing other lines in the L2.
+#ifndef TCD_NT
+#define TCD_NT 3  // bit 0: stores, bit 1: loads
+#endif
+typedef unsigned int tcd_v4u __attribute__((ext_vector_type(4)));
+template <class V, class E>
+__device__ inline V load16(const E* p) {
+  static_assert(sizeof(V) == 16, "16-byte vector");
+  tcd_v4u r;
+  if (TCD_NT & 2) r = __builtin_nontemporal_load(reinterpret_cast<const tcd_v4u*>(p));
+  else r = *reinterpret_cast<const tcd_v4u*>(p);
+  V v;
+  __builtin_memcpy(&v, &r, 16);
+  return v;
+}
+template <class V, class E>
+__device__ inline void store16(E* p, const V& v) {
+  static_assert(sizeof(V) == 16, "16-byte vector");
+  tcd_v4u r;
+  __builtin_memcpy(&r, &v, 16);
+  if (TCD_NT & 1) __builtin_nontemporal_store(r, reinterpret_cast<tcd_v4u*>(p));
+  else *reinterpret_cast<tcd_v4u*>(p) = r;
+}
+
 // ---------------------------------------------------------------------------------------
 // Tile descriptors for decoupled look-back.
 //

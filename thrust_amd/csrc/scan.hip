@@ -16,13 +16,12 @@ struct alignas(16) Vec16 {
 };
 
 template <class T, class Op, int BLOCK, int CHUNKS>
-__global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_t n, T init,
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void scan_kernel(const T* in, T* out, int64_t n, T init,
                                                      int exclusive, uint64_t* desc,
                                                      uint32_t* ticket, int vec_ok) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NWAVES = BLOCK / kWave;
   constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
-  static_assert(CHUNKS * NWAVES <= kWave, "one wavefront scans the (chunk, wave) totals");
   // cross-lane traffic, LDS and descriptors carry W (a dword container for 1- and 2-byte T)
   using W = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
 
@@ -56,7 +55,7 @@ __global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_
   if (fast) {
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
-      const Vec16<T> v = *reinterpret_cast<const Vec16<T>*>(tin + c * BLOCK * VEC);
+      const Vec16<T> v = load16<Vec16<T>>(tin + c * BLOCK * VEC);
 #pragma unroll
       for (int j = 0; j < VEC; j++) x[c][j] = v.v[j];
     }
@@ -83,12 +82,21 @@ __global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_
   }
   __syncthreads();
 
-  // wave 0: exclusive scan of the (chunk, wave) totals in tile order, then the look-back
+  // wave 0: exclusive scan of the (chunk, wave) totals in tile order (PER consecutive totals per
+  // lane), then the look-back
   if (wave == 0) {
-    const W mine = lane < CHUNKS * NWAVES ? s_tot[lane] : idW;
-    const W incl = wave_inclusive_scan(mine, idW, opW);
+    constexpr int NTOT = CHUNKS * NWAVES;
+    constexpr int PER = (NTOT + kWave - 1) / kWave;
+    W mine[PER];
+#pragma unroll
+    for (int q = 0; q < PER; q++) {
+      const int idx = lane * PER + q;
+      mine[q] = idx < NTOT ? s_tot[idx] : idW;
+      if (q > 0) mine[q] = opW(mine[q - 1], mine[q]);
+    }
+    const W incl = wave_inclusive_scan(mine[PER - 1], idW, opW);
     const W tile_agg = readlane(incl, kWave - 1);
-    const W before = wave_shift_up1(incl, idW);
+    const W before = wave_shift_up1(incl, idW);  // totals of the lanes below
     W prefix;
     if (tile == 0) {
       prefix = exclusive ? toW(init) : idW;
@@ -98,7 +106,13 @@ __global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_
       prefix = wave_lookback<W>(desc, tile, idW, opW);
       if (lane == 0) TileDesc<W>::store(desc, tile, kInclusive, opW(prefix, tile_agg));
     }
-    if (lane < CHUNKS * NWAVES) s_tot[lane] = opW(prefix, before);  // offset of (chunk, wave) in the whole input
+    const W base_w = opW(prefix, before);
+    // offset of (chunk, wave) in the whole input = everything before it
+#pragma unroll
+    for (int q = 0; q < PER; q++) {
+      const int idx = lane * PER + q;
+      if (idx < NTOT) s_tot[idx] = q == 0 ? base_w : opW(base_w, mine[q - 1]);
+    }
   }
   __syncthreads();
 
@@ -121,7 +135,7 @@ __global__ __launch_bounds__(BLOCK) void scan_kernel(const T* in, T* out, int64_
       Vec16<T> v;
 #pragma unroll
       for (int j = 0; j < VEC; j++) v.v[j] = x[c][j];
-      *reinterpret_cast<Vec16<T>*>(tout + c * BLOCK * VEC) = v;
+      store16(tout + c * BLOCK * VEC, v);
     }
   } else {
 #pragma unroll
@@ -139,13 +153,15 @@ template <class T>
 struct ScanConfig {
 #ifndef TCD_SCAN_BLOCK
 #define TCD_SCAN_BLOCK 512
-#define TCD_SCAN_CHUNKS 8
 #endif
-  // 128 bytes per thread for 4- and 8-byte elements (64 KiB tiles: fewer tickets and look-backs
-  // per byte; measured best on MI355X); fewer chunks for narrow types, which hold one element
-  // per register.
+#ifndef TCD_SCAN_CHUNKS
+#define TCD_SCAN_CHUNKS 16
+#endif
+  // 256 bytes per thread for 4- and 8-byte elements (128 KiB tiles: fewer tickets and look-backs
+  // per byte; measured best on MI355X: 64 KiB tiles are 10 % slower, 192 KiB tiles 3 %); fewer
+  // chunks for narrow types, which hold one element per register.
   static constexpr int BLOCK = TCD_SCAN_BLOCK;
-  static constexpr int CHUNKS = sizeof(T) >= 4 ? TCD_SCAN_CHUNKS : (sizeof(T) == 2 ? 4 : 2);
+  static constexpr int CHUNKS = sizeof(T) >= 4 ? TCD_SCAN_CHUNKS : (sizeof(T) == 2 ? 8 : 4);
   static constexpr int64_t TILE = (int64_t)BLOCK * (16 / sizeof(T)) * CHUNKS;
   using P = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
 };
