@@ -78,7 +78,7 @@ __device__ inline void load_group(const E* p, E (&dst)[N]) {
   if constexpr (BYTES >= 16) {
 #pragma unroll
     for (int q = 0; q < BYTES / 16; q++) {
-      const uint4 t = reinterpret_cast<const uint4*>(p)[q];
+      const tcd_v4u t = load16<tcd_v4u>(reinterpret_cast<const char*>(p) + 16 * q);
       __builtin_memcpy(reinterpret_cast<char*>(dst) + 16 * q, &t, 16);
     }
   } else {
@@ -92,9 +92,9 @@ __device__ inline void store_group(E* p, const E (&src)[N]) {
   if constexpr (BYTES >= 16) {
 #pragma unroll
     for (int q = 0; q < BYTES / 16; q++) {
-      uint4 t;
+      tcd_v4u t;
       __builtin_memcpy(&t, reinterpret_cast<const char*>(src) + 16 * q, 16);
-      reinterpret_cast<uint4*>(p)[q] = t;
+      store16(reinterpret_cast<char*>(p) + 16 * q, t);
     }
   } else {
     typename bits_of<BYTES>::type t;

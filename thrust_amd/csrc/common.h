@@ -181,7 +181,9 @@ __device__ inline T wave_shift_up1(const T& incl, const T id) {
 }
 
 // 16-byte streaming accesses.  Data that a kernel touches exactly once is loaded and stored
-// with the non-temporal hint, which keeps it from displacing other lines in the L2.
+// with the non-temporal hint, which keeps it from displacing other lines in the L2 (scan and
+// by-key kernels gain 3-4 %).  The sort's scattered 4- and 8-byte stores must NOT use it: they
+// rely on the L2 to merge the pieces of a line written by different waves (measured 25 % slower).
 #ifndef TCD_NT
 #define TCD_NT 3  // bit 0: stores, bit 1: loads
 #endif

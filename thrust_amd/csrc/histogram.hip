@@ -110,12 +110,12 @@ __global__ __launch_bounds__(kHistBlock) void histogram_kernel(const T* __restri
     for (; i + (kHistUnroll - 1) * gstride < nvec; i += kHistUnroll * gstride) {
       V16 v[kHistUnroll];
 #pragma unroll
-      for (int u = 0; u < kHistUnroll; u++) v[u] = sv[i + u * gstride];
+      for (int u = 0; u < kHistUnroll; u++) v[u] = load16<V16>(&sv[i + u * gstride]);
 #pragma unroll
       for (int u = 0; u < kHistUnroll; u++) count_group(v[u].v);
     }
     for (; i < nvec; i += gstride) {
-      const V16 v = sv[i];
+      const V16 v = load16<V16>(&sv[i]);
       count_group(v.v);
     }
     for (int64_t i = nvec * VEC + gtid; i < n; i += gstride) count_plain(bin_of(samples[i]));

@@ -117,14 +117,14 @@ __global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const U* __res
     for (; i + (UNROLL - 1) * gstride < nvec; i += UNROLL * gstride) {
       V16 v[UNROLL];
 #pragma unroll
-      for (int u = 0; u < UNROLL; u++) v[u] = kv[i + u * gstride];
+      for (int u = 0; u < UNROLL; u++) v[u] = load16<V16>(&kv[i + u * gstride]);
 #pragma unroll
       for (int u = 0; u < UNROLL; u++)
 #pragma unroll
         for (int j = 0; j < VEC; j++) count(v[u].v[j]);
     }
     for (; i < nvec; i += gstride) {
-      const V16 v = kv[i];
+      const V16 v = load16<V16>(&kv[i]);
 #pragma unroll
       for (int j = 0; j < VEC; j++) count(v.v[j]);
     }
