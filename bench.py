@@ -252,6 +252,11 @@ def main():
         b = torch.empty_like(a)
         ms = timed(lambda: b.copy_(a), lambda: None, 10, 2)
         extras["device_copy_ceiling_GBs"] = round(8.0 * n / float(np.median(ms)) / 1e6, 1)
+        # the library's own device-to-device copy (one 16-byte access per thread)
+        nbytes = ctypes.c_size_t(4 * n)
+        ms = timed(lambda: capi.check(L.thrust_cdna4_memcpy_dtod(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()),
+                                                                  nbytes, sp), "memcpy_dtod"), lambda: None, 10, 2)
+        extras["library_copy_GBs"] = round(8.0 * n / float(np.median(ms)) / 1e6, 1)
 
     all_extras = {
         "sort_by_key": extra_sort_pairs,

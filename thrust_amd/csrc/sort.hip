@@ -540,9 +540,9 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (cur == 1) {  // odd number of passes: bring the result home
-    e = hipMemcpyAsync(kbuf[0], kbuf[1], (size_t)n * sizeof(U), hipMemcpyDeviceToDevice, stream);
+    e = copy_async(kbuf[0], kbuf[1], (size_t)n * sizeof(U), stream);
     if (e != hipSuccess) return e;
-    if (VB) e = hipMemcpyAsync(vbuf[0], vbuf[1], (size_t)n * VB, hipMemcpyDeviceToDevice, stream);
+    if (VB) e = copy_async(vbuf[0], vbuf[1], (size_t)n * VB, stream);
   }
   return e;
 }
