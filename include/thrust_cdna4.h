@@ -69,7 +69,7 @@ const char* thrust_cdna4_error_string(int code);
  * Order: ascending by the reference's RadixEncoder bit order
  * (sequential/stable_radix_sort.inl:43-139) — for floating-point keys that is the total
  * order -NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN.  `descending != 0` gives the
- * order of thrust::greater (sequential/sort.inl:54-75).  n must be < 2^30.
+ * order of thrust::greater (sequential/sort.inl:54-75).  n must be < 2^32 - 1.
  */
 int thrust_cdna4_sort_keys(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
                            int64_t n, int descending, void* stream);

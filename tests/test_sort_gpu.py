@@ -203,3 +203,26 @@ def test_sort_pairs_large_tiles_stability(kd, vd):
         thrust_amd.sort_by_key(dk, dv, descending)
         rk, rv = oracle.sort_pairs(k, v, descending)
         assert same_bits(host(dk), rk) and same_bits(host(dv), rv), descending
+
+
+def test_sort_beyond_2p30_items():
+    """n >= 2^30 switches the tile descriptors to 64-bit words (digit counts no longer fit 30
+    bits).  No oracle at this size: sortedness, multiset checksums, and for pairs stability and
+    key/value association, all checked on the device."""
+    n = (1 << 30) + 12345
+    g = torch.Generator(device="cuda").manual_seed(2030)
+    k = torch.randint(-2**31, 2**31, (n,), dtype=torch.int32, device="cuda", generator=g)
+    s0 = int(k.sum(dtype=torch.int64).item())
+    thrust_amd.sort(k)
+    assert bool((k[1:] >= k[:-1]).all())
+    assert int(k.sum(dtype=torch.int64).item()) == s0
+    del k
+    torch.cuda.empty_cache()
+    # pairs: few distinct keys, so every digit count of the top passes exceeds 2^30 / 256 by far
+    src = torch.randint(0, 1000, (n,), dtype=torch.int32, device="cuda", generator=g)
+    k = src.clone()
+    v = torch.arange(n, dtype=torch.int32, device="cuda")
+    thrust_amd.sort_by_key(k, v)
+    assert bool((k[1:] >= k[:-1]).all())
+    assert bool(((k[1:] > k[:-1]) | (v[1:] > v[:-1])).all())  # equal keys keep their input order
+    assert bool((src[v.long()] == k).all())

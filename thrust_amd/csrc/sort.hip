@@ -26,8 +26,16 @@ namespace tcd {
 constexpr int kRadixBits = 8;
 constexpr int kRadix = 1 << kRadixBits;
 
-// descriptor word: status in bits 31:30, count in bits 29:0
-constexpr uint32_t kCountMask = (1u << 30) - 1;
+// Descriptor word D (uint32_t for n < 2^30, uint64_t up to the limit of 32-bit positions):
+// status in the two top bits, count below.
+template <class D>
+struct DescWord {
+  static constexpr int kShift = 8 * (int)sizeof(D) - 2;
+  static constexpr D kCountMask = (D(1) << kShift) - 1;
+  __device__ static D make(uint32_t status, uint32_t count) { return (D(status) << kShift) | D(count); }
+  __device__ static uint32_t status(D w) { return (uint32_t)(w >> kShift); }
+  __device__ static uint32_t count(D w) { return (uint32_t)(w & kCountMask); }
+};
 #ifndef TCD_SORT_LOOKW
 #define TCD_SORT_LOOKW 4
 #endif
@@ -184,12 +192,12 @@ __device__ inline void lds_store(uint32_t* p, uint32_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
 }
 
-template <class U, int VB, bool FLOAT, int BLOCK, int IPT, int WPE>
+template <class U, int VB, bool FLOAT, int BLOCK, int IPT, int WPE, class D>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) void onesweep_kernel(const U* __restrict__ kin, U* __restrict__ kout,
                                                          const void* __restrict__ vin_, void* __restrict__ vout_,
                                                          int64_t n, U xor_mask, int shift,
                                                          const uint32_t* __restrict__ gbase,
-                                                         uint32_t* desc, uint32_t* ticket) {
+                                                         D* desc, uint32_t* ticket) {
   static_assert(BLOCK % 256 == 0, "one thread per digit needs at least 256 threads");
   using V = typename value_of<VB>::type;
   constexpr int NWAVES = BLOCK / kWave;
@@ -293,7 +301,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
 #pragma unroll
     for (int w = 0; w < NWAVES; w++) total += sm.wave_cnt[w][tid];
     const uint32_t st = (tile == 0) ? kInclusive : kPartial;
-    st_agent(&desc[tile * kRadix + tid], (st << 30) | total);
+    st_agent(&desc[tile * kRadix + tid], DescWord<D>::make(st, total));
     const uint32_t incl = wave_inclusive_scan(total, 0u, [](uint32_t a, uint32_t b) { return a + b; });
     if (lane == 63) sm.wave_tot[wave] = incl;
     lbase = incl - total;
@@ -327,16 +335,16 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
       int64_t t = tile - 1;
       bool done = false;
       while (!done) {
-        uint32_t v[kLookW];
+        D v[kLookW];
 #pragma unroll
         for (int j = 0; j < kLookW; j++)
-          v[j] = (t - j >= 0) ? ld_agent(&desc[(t - j) * kRadix + tid]) : ((uint32_t)kInclusive << 30);
+          v[j] = (t - j >= 0) ? ld_agent(&desc[(t - j) * kRadix + tid]) : DescWord<D>::make(kInclusive, 0u);
         int used = 0;
 #pragma unroll
         for (int j = 0; j < kLookW; j++) {
-          const uint32_t st = v[j] >> 30;
+          const uint32_t st = DescWord<D>::status(v[j]);
           if (!done && used == j && st != kInvalid) {
-            prefix += v[j] & kCountMask;
+            prefix += DescWord<D>::count(v[j]);
             used = j + 1;
             done = st == kInclusive;
           }
@@ -344,7 +352,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
         t -= used;
         if (used == 0) __builtin_amdgcn_s_sleep(2);
       }
-      st_agent(&desc[tile * kRadix + tid], ((uint32_t)kInclusive << 30) | (prefix + total));
+      st_agent(&desc[tile * kRadix + tid], DescWord<D>::make(kInclusive, prefix + total));
     }
     sm.global_off[tid] = gbase[tid] + prefix - lbase;
   }
@@ -478,6 +486,8 @@ struct SortConfig {
 #ifndef TCD_SORT_SMALL_LOG2N
 #define TCD_SORT_SMALL_LOG2N 21
 #endif
+// positions, digit counts and their prefix sums are 32-bit
+constexpr int64_t kSortMaxN = (int64_t(1) << 32) - 1;
 constexpr int64_t small_sort_limit(int value_bytes) { return int64_t(1) << (TCD_SORT_SMALL_LOG2N + (value_bytes ? 1 : 0)); }
 
 struct SortPlan {
@@ -486,7 +496,7 @@ struct SortPlan {
   int64_t ntiles;
 };
 
-template <class U, int VB, class C>
+template <class U, int VB, class C, class D>
 static SortPlan make_plan(int64_t n) {
   constexpr int P = sizeof(U);
   SortPlan p{};
@@ -497,17 +507,17 @@ static SortPlan make_plan(int64_t n) {
   p.zero_begin = off;
   p.hist = off; off += align_up((size_t)P * kRadix * 4, 256);
   p.tickets = off; off += 256;
-  p.desc = off; off += align_up((size_t)P * p.ntiles * kRadix * 4, 256);
+  p.desc = off; off += align_up((size_t)P * p.ntiles * kRadix * sizeof(D), 256);
   p.zero_bytes = off - p.zero_begin;
   p.total = off;
   return p;
 }
 
-template <class U, int VB, bool FLOAT, class C>
+template <class U, int VB, bool FLOAT, class C, class D>
 static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* values, int64_t n,
                             U xor_mask, hipStream_t stream) {
   constexpr int P = sizeof(U);
-  const SortPlan plan = make_plan<U, VB, C>(n);
+  const SortPlan plan = make_plan<U, VB, C, D>(n);
   if (temp == nullptr) {
     *temp_bytes = plan.total;
     return hipSuccess;
@@ -519,7 +529,7 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   char* vbuf[2] = {static_cast<char*>(values), t + plan.vals_alt};
   uint32_t* ghist = reinterpret_cast<uint32_t*>(t + plan.hist);
   uint32_t* tickets = reinterpret_cast<uint32_t*>(t + plan.tickets);
-  uint32_t* desc = reinterpret_cast<uint32_t*>(t + plan.desc);
+  D* desc = reinterpret_cast<D*>(t + plan.desc);
 
   hipError_t e = zero_async(t + plan.zero_begin, plan.zero_bytes, stream);
   if (e != hipSuccess) return e;
@@ -532,7 +542,7 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(P), dim3(256), stream, ghist);
   int cur = 0;
   for (int p = 0; p < P; p++) {
-    TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT, C::WPE>), dim3((unsigned)plan.ntiles),
+    TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT, C::WPE, D>), dim3((unsigned)plan.ntiles),
                dim3(C::BLOCK), stream, kbuf[cur], kbuf[cur ^ 1], vbuf[cur], vbuf[cur ^ 1], n, xor_mask, 8 * p,
                ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix, tickets + p);
     cur ^= 1;
@@ -551,8 +561,11 @@ template <class U, int VB, bool FLOAT>
 static hipError_t sort_typed(void* temp, size_t* temp_bytes, void* keys, void* values, int64_t n,
                              U xor_mask, hipStream_t stream) {
   // the choice depends on n only, so the size query and the run agree
-  if (n < small_sort_limit(VB)) return sort_with<U, VB, FLOAT, SortConfig<U, VB, true>>(temp, temp_bytes, keys, values, n, xor_mask, stream);
-  return sort_with<U, VB, FLOAT, SortConfig<U, VB, false>>(temp, temp_bytes, keys, values, n, xor_mask, stream);
+  if (n < small_sort_limit(VB))
+    return sort_with<U, VB, FLOAT, SortConfig<U, VB, true>, uint32_t>(temp, temp_bytes, keys, values, n, xor_mask, stream);
+  if (n < (int64_t(1) << 30))  // counts fit the 30 bits of a 32-bit descriptor word
+    return sort_with<U, VB, FLOAT, SortConfig<U, VB, false>, uint32_t>(temp, temp_bytes, keys, values, n, xor_mask, stream);
+  return sort_with<U, VB, FLOAT, SortConfig<U, VB, false>, uint64_t>(temp, temp_bytes, keys, values, n, xor_mask, stream);
 }
 
 template <int VB>
@@ -587,7 +600,7 @@ static hipError_t sort_dispatch(void* temp, size_t* temp_bytes, int key_dtype, v
 
 extern "C" int thrust_cdna4_sort_keys(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
                                       int64_t n, int descending, void* stream) {
-  if (!temp_bytes || n < 0 || n >= ((int64_t)1 << 30) || (n > 0 && temp && !keys))
+  if (!temp_bytes || n < 0 || n >= tcd::kSortMaxN || (n > 0 && temp && !keys))
     return hipErrorInvalidValue;
   return (int)tcd::sort_dispatch<0>(temp, temp_bytes, key_dtype, keys, nullptr, n, descending,
                                     static_cast<hipStream_t>(stream));
@@ -596,7 +609,7 @@ extern "C" int thrust_cdna4_sort_keys(void* temp, size_t* temp_bytes, int key_dt
 extern "C" int thrust_cdna4_sort_pairs(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
                                        int value_bytes, void* values, int64_t n, int descending,
                                        void* stream) {
-  if (!temp_bytes || n < 0 || n >= ((int64_t)1 << 30) || (n > 0 && temp && (!keys || !values)))
+  if (!temp_bytes || n < 0 || n >= tcd::kSortMaxN || (n > 0 && temp && (!keys || !values)))
     return hipErrorInvalidValue;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (value_bytes) {
