@@ -258,7 +258,19 @@ def main():
                                                                   nbytes, sp), "memcpy_dtod"), lambda: None, 10, 2)
         extras["library_copy_GBs"] = round(8.0 * n / float(np.median(ms)) / 1e6, 1)
 
+    def extra_merge_sort():
+        # comparison sort with a user comparator: kernel templates, so a C++ binary built by hipcc
+        # (tests/cpp/bench_merge_sort.cpp) measures it; 2^26 keys
+        import subprocess
+        exe = os.path.join(ROOT, "tests", "cpp", "build", "bench_merge_sort")
+        if not os.path.exists(exe):
+            return
+        r = subprocess.run([exe, "26"], capture_output=True, text=True, timeout=300)
+        if r.returncode == 0:
+            extras.update(json.loads(r.stdout.strip().splitlines()[-1]))
+
     all_extras = {
+        "merge_sort": extra_merge_sort,
         "sort_by_key": extra_sort_pairs,
         "scan_i32": lambda: extra_scan("i32"),
         "scan_f32": lambda: extra_scan("f32"),

@@ -1,4 +1,4 @@
-// thrust::device_vector for arithmetic element types (thrust/device_vector.h,
+// thrust::device_vector for trivially copyable element types (thrust/device_vector.h,
 // thrust/detail/vector_base.h).  Storage comes from the library's cached allocator; value
 // initialisation and fills run as typed fill kernels, transfers as async copies followed by
 // a stream synchronise (thrust/system/cuda/detail/util.h:142-199), so a TU that uses
@@ -16,8 +16,7 @@ namespace thrust {
 
 template <class T>
 class device_vector {
-  static_assert(std::is_arithmetic<T>::value, "device_vector of the cdna4 system holds arithmetic types");
-  static_assert(sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8, "unsupported element size");
+  static_assert(std::is_trivially_copyable<T>::value, "device_vector of the cdna4 system holds trivially copyable types");
   typedef system::cdna4::detail::temporary_storage storage_unused;
 
  public:
@@ -96,7 +95,12 @@ class device_vector {
   }
   static void fill_raw(T* dst, size_type n, const T& v) {
     if (!n) return;
-    check(thrust_cdna4_fill(dst, &v, (int)sizeof(T), (int64_t)n, nullptr), "device_vector: fill");
+    if (sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8) {
+      check(thrust_cdna4_fill(dst, &v, (int)sizeof(T), (int64_t)n, nullptr), "device_vector: fill");
+    } else {  // other element sizes (user structs): staged through the host
+      const std::vector<T> tmp(n, v);
+      check(thrust_cdna4_memcpy_htod(dst, tmp.data(), n * sizeof(T), nullptr), "device_vector: fill");
+    }
     sync();
   }
   void assign_host(const T* h, size_type n) {

@@ -1,24 +1,31 @@
 // Function objects the device kernels are specialised on (thrust/functional.h).
 #pragma once
 #include <functional>
+// Callable from kernels when the translation unit is compiled by hipcc (comparison sort with
+// these functors); plain host functions under a host compiler.
+#if defined(__HIPCC__)
+#define THRUST_CDNA4_HD __host__ __device__
+#else
+#define THRUST_CDNA4_HD
+#endif
 namespace thrust {
-template <class T = void> struct plus { constexpr T operator()(const T& a, const T& b) const { return a + b; } };
-template <class T = void> struct multiplies { constexpr T operator()(const T& a, const T& b) const { return a * b; } };
-template <class T = void> struct maximum { constexpr T operator()(const T& a, const T& b) const { return a < b ? b : a; } };
-template <class T = void> struct minimum { constexpr T operator()(const T& a, const T& b) const { return a < b ? a : b; } };
-template <class T = void> struct less { constexpr bool operator()(const T& a, const T& b) const { return a < b; } };
-template <class T = void> struct greater { constexpr bool operator()(const T& a, const T& b) const { return a > b; } };
-template <class T = void> struct equal_to { constexpr bool operator()(const T& a, const T& b) const { return a == b; } };
-template <class T = void> struct identity { constexpr const T& operator()(const T& a) const { return a; } };
+template <class T = void> struct plus { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a + b; } };
+template <class T = void> struct multiplies { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a * b; } };
+template <class T = void> struct maximum { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a < b ? b : a; } };
+template <class T = void> struct minimum { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a < b ? a : b; } };
+template <class T = void> struct less { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a < b; } };
+template <class T = void> struct greater { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a > b; } };
+template <class T = void> struct equal_to { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a == b; } };
+template <class T = void> struct identity { THRUST_CDNA4_HD constexpr const T& operator()(const T& a) const { return a; } };
 
 // transparent forms (thrust::plus<> etc.)
-template <> struct plus<void> { template <class A, class B> constexpr auto operator()(const A& a, const B& b) const -> decltype(a + b) { return a + b; } };
-template <> struct multiplies<void> { template <class A, class B> constexpr auto operator()(const A& a, const B& b) const -> decltype(a * b) { return a * b; } };
-template <> struct maximum<void> { template <class A> constexpr A operator()(const A& a, const A& b) const { return a < b ? b : a; } };
-template <> struct minimum<void> { template <class A> constexpr A operator()(const A& a, const A& b) const { return a < b ? a : b; } };
-template <> struct less<void> { template <class A, class B> constexpr bool operator()(const A& a, const B& b) const { return a < b; } };
-template <> struct greater<void> { template <class A, class B> constexpr bool operator()(const A& a, const B& b) const { return a > b; } };
-template <> struct equal_to<void> { template <class A, class B> constexpr bool operator()(const A& a, const B& b) const { return a == b; } };
+template <> struct plus<void> { template <class A, class B> THRUST_CDNA4_HD constexpr auto operator()(const A& a, const B& b) const -> decltype(a + b) { return a + b; } };
+template <> struct multiplies<void> { template <class A, class B> THRUST_CDNA4_HD constexpr auto operator()(const A& a, const B& b) const -> decltype(a * b) { return a * b; } };
+template <> struct maximum<void> { template <class A> THRUST_CDNA4_HD constexpr A operator()(const A& a, const A& b) const { return a < b ? b : a; } };
+template <> struct minimum<void> { template <class A> THRUST_CDNA4_HD constexpr A operator()(const A& a, const A& b) const { return a < b ? a : b; } };
+template <> struct less<void> { template <class A, class B> THRUST_CDNA4_HD constexpr bool operator()(const A& a, const B& b) const { return a < b; } };
+template <> struct greater<void> { template <class A, class B> THRUST_CDNA4_HD constexpr bool operator()(const A& a, const B& b) const { return a > b; } };
+template <> struct equal_to<void> { template <class A, class B> THRUST_CDNA4_HD constexpr bool operator()(const A& a, const B& b) const { return a == b; } };
 
 namespace system { namespace cdna4 { namespace detail {
 // C-ABI operator code of a functor type, or -1 when no kernel exists for it.

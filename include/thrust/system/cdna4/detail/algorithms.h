@@ -10,15 +10,20 @@
 #include <cstdint>
 #include <thrust/functional.h>
 #include <thrust/system/cdna4/detail/core.h>
+#if defined(__HIPCC__)
+#include <thrust/system/cdna4/detail/merge_sort.h>
+#endif
 
 namespace thrust { namespace system { namespace cdna4 { namespace detail {
 
+// Arithmetic keys under thrust::less / thrust::greater take the radix kernels behind the C ABI
+// (thrust/system/cuda/detail/sort.h:389-395, can_use_primitive_sort); everything else is a
+// comparison sort with kernel templates, which exist only when this header is compiled by hipcc.
+template <class K, class Compare>
+struct use_radix_sort : std::integral_constant<bool, dtype_of<K>::supported && (order_code<Compare>::value >= 0)> {};
+
 template <class Policy, class K, class Compare>
-void sort_keys(const Policy& exec, K* keys, std::int64_t n, Compare) {
-  static_assert(dtype_of<K>::supported, "cdna4 sort: keys must be an arithmetic type");
-  static_assert(order_code<Compare>::value >= 0,
-                "cdna4 sort: only thrust::less / thrust::greater have a radix kernel (comparison sort is not built)");
-  if (n <= 0) return;  // thrust/system/cuda/detail/sort.h:140-143
+void sort_keys_impl(const Policy& exec, K* keys, std::int64_t n, Compare, std::true_type) {
   void* s = stream_of(exec);
   std::size_t bytes = 0;
   throw_on_error(thrust_cdna4_sort_keys(nullptr, &bytes, dtype_of<K>::value, keys, n, order_code<Compare>::value, s),
@@ -26,18 +31,28 @@ void sort_keys(const Policy& exec, K* keys, std::int64_t n, Compare) {
   temporary_storage tmp(bytes, s);
   throw_on_error(thrust_cdna4_sort_keys(tmp.data(), &bytes, dtype_of<K>::value, keys, n, order_code<Compare>::value, s),
                  "sort: launch");
+}
+template <class Policy, class K, class Compare>
+void sort_keys_impl(const Policy& exec, K* keys, std::int64_t n, Compare comp, std::false_type) {
+#if defined(__HIPCC__)
+  merge::stable_sort(stream_of(exec), keys, static_cast<merge::no_value*>(nullptr), n, comp);
+#else
+  static_assert(sizeof(K) == 0,
+                "cdna4 sort: a custom comparator or non-arithmetic key needs the comparison-sort kernel templates; "
+                "compile this translation unit with hipcc --offload-arch=gfx950");
+  (void)exec; (void)keys; (void)n; (void)comp;
+#endif
+}
+
+template <class Policy, class K, class Compare>
+void sort_keys(const Policy& exec, K* keys, std::int64_t n, Compare comp) {
+  if (n <= 0) return;  // thrust/system/cuda/detail/sort.h:140-143
+  sort_keys_impl(exec, keys, n, comp, use_radix_sort<K, Compare>());
   synchronize_optional(exec, "sort: failed to synchronize");
 }
 
 template <class Policy, class K, class V, class Compare>
-void sort_pairs(const Policy& exec, K* keys, V* values, std::int64_t n, Compare) {
-  static_assert(dtype_of<K>::supported, "cdna4 sort_by_key: keys must be an arithmetic type");
-  static_assert(sizeof(V) == 1 || sizeof(V) == 2 || sizeof(V) == 4 || sizeof(V) == 8,
-                "cdna4 sort_by_key: values must be 1, 2, 4 or 8 bytes wide");
-  static_assert(std::is_trivially_copyable<V>::value, "cdna4 sort_by_key: values must be trivially copyable");
-  static_assert(order_code<Compare>::value >= 0,
-                "cdna4 sort_by_key: only thrust::less / thrust::greater have a radix kernel");
-  if (n <= 0) return;
+void sort_pairs_impl(const Policy& exec, K* keys, V* values, std::int64_t n, Compare, std::true_type) {
   void* s = stream_of(exec);
   std::size_t bytes = 0;
   throw_on_error(thrust_cdna4_sort_pairs(nullptr, &bytes, dtype_of<K>::value, keys, (int)sizeof(V), values, n,
@@ -45,6 +60,26 @@ void sort_pairs(const Policy& exec, K* keys, V* values, std::int64_t n, Compare)
   temporary_storage tmp(bytes, s);
   throw_on_error(thrust_cdna4_sort_pairs(tmp.data(), &bytes, dtype_of<K>::value, keys, (int)sizeof(V), values, n,
                                          order_code<Compare>::value, s), "sort_by_key: launch");
+}
+template <class Policy, class K, class V, class Compare>
+void sort_pairs_impl(const Policy& exec, K* keys, V* values, std::int64_t n, Compare comp, std::false_type) {
+#if defined(__HIPCC__)
+  merge::stable_sort(stream_of(exec), keys, values, n, comp);
+#else
+  static_assert(sizeof(K) == 0,
+                "cdna4 sort_by_key: a custom comparator, non-arithmetic key or value wider than 8 bytes needs the "
+                "comparison-sort kernel templates; compile this translation unit with hipcc --offload-arch=gfx950");
+  (void)exec; (void)keys; (void)values; (void)n; (void)comp;
+#endif
+}
+
+template <class Policy, class K, class V, class Compare>
+void sort_pairs(const Policy& exec, K* keys, V* values, std::int64_t n, Compare comp) {
+  static_assert(std::is_trivially_copyable<V>::value, "cdna4 sort_by_key: values must be trivially copyable");
+  if (n <= 0) return;
+  constexpr bool radix_value = sizeof(V) == 1 || sizeof(V) == 2 || sizeof(V) == 4 || sizeof(V) == 8;
+  sort_pairs_impl(exec, keys, values, n, comp,
+                  std::integral_constant<bool, use_radix_sort<K, Compare>::value && radix_value>());
   synchronize_optional(exec, "sort_by_key: failed to synchronize");
 }
 

@@ -1,0 +1,306 @@
+// Stable comparison (merge) sort for gfx950, for keys or comparators the radix kernels cannot
+// take: user-defined comparison functors, non-arithmetic trivially copyable keys.  This is
+// the second branch of the reference's sort dispatch (thrust/system/cuda/detail/sort.h:59-205,
+// :410-429, cub::DispatchMergeSort); semantics: thrust/system/detail/sequential/
+// stable_merge_sort.inl (a stable sort: equal keys keep their input order).
+//
+// Unlike the radix path, the comparator is user code, so these are kernel TEMPLATES: the
+// translation unit that instantiates them must be compiled by hipcc (--offload-arch=gfx950)
+// and the comparator's operator() must be __host__ __device__.  Temporary storage comes from
+// the library's stream-ordered pool.
+//
+//   1. block_sort_kernel   a 256-thread workgroup sorts a tile of 2048 items: every thread
+//                          sorts its 8 consecutive items in registers (odd-even transposition,
+//                          stable), then log2(256) rounds of merge-path merging through LDS.
+//   2. merge_partition_kernel + merge_kernel, once per doubling of the run width: one thread
+//                          per output tile finds where the tile starts in the two runs it
+//                          merges (binary search on the merge path, ties to the left run);
+//                          a workgroup then loads the two pieces into LDS, every thread merges
+//                          its 8 outputs, and the tile is written back with contiguous stores.
+//      Values follow their keys through LDS by source index.
+#pragma once
+#if !defined(__HIPCC__)
+#error "thrust/system/cdna4/detail/merge_sort.h holds device kernel templates: compile with hipcc"
+#endif
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <type_traits>
+#include <thrust/system/cdna4/detail/core.h>
+
+namespace thrust { namespace system { namespace cdna4 { namespace detail { namespace merge {
+
+constexpr int kBlock = 256;
+constexpr int kIpt = 8;
+constexpr int kTile = kBlock * kIpt;
+
+struct no_value {};
+
+// Pins a value that was just read from LDS into registers HERE.  A workgroup barrier does not
+// wait for LDS reads that are still in flight, and the compiler only waits for a read where its
+// result is first used; in a loop that reads LDS into registers, passes a barrier and writes
+// those registers back to LDS, a read could otherwise still be pending when another wave
+// overwrites its source after the barrier.
+template <class T>
+__device__ inline void settle(const T& x) {
+  constexpr int NW = (int)((sizeof(T) + 3) / 4);
+  std::uint32_t w[NW] = {};
+  __builtin_memcpy(w, &x, sizeof(T));
+#pragma unroll
+  for (int i = 0; i < NW; i++) asm volatile("" ::"v"(w[i]));
+}
+
+// Number of items the first `diag` outputs of merge(a[0,na), b[0,nb)) take from a, with ties
+// going to a (stability: a is the earlier run).
+template <class K, class Compare>
+__device__ inline int merge_path(const K* a, int na, const K* b, int nb, int diag, Compare comp) {
+  int lo = diag > nb ? diag - nb : 0;
+  int hi = diag < na ? diag : na;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (!comp(b[diag - 1 - mid], a[mid])) lo = mid + 1;  // a[mid] <= b[...]: a[mid] is among the first diag
+    else hi = mid;
+  }
+  return lo;
+}
+
+// ---------------------------------------------------------------------------------------
+// 1. Tile sort
+// ---------------------------------------------------------------------------------------
+template <class K, class V, class Compare>
+__global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, std::int64_t n, Compare comp) {
+  constexpr bool kHasValues = !std::is_same<V, no_value>::value;
+  __shared__ K s_keys[kTile];
+  __shared__ std::uint16_t s_idx[kTile];
+  __shared__ typename std::conditional<kHasValues, V, char>::type s_vals[kHasValues ? kTile : 1];
+
+  const int tid = threadIdx.x;
+  const std::int64_t base = (std::int64_t)blockIdx.x * kTile;
+  const int valid = (int)((n - base) < (std::int64_t)kTile ? (n - base) : (std::int64_t)kTile);
+
+  // Items past the end of the input (last tile only) order after every real item; they are
+  // recognised by their original position, which every item carries along.
+  auto before = [&](const K& a, int ia, const K& b, int ib) -> bool {
+    if (ib >= valid) return ia < valid;
+    if (ia >= valid) return false;
+    return comp(a, b);
+  };
+
+  K k[kIpt];
+  int idx[kIpt];
+#pragma unroll
+  for (int j = 0; j < kIpt; j++) {
+    idx[j] = tid * kIpt + j;
+    if (idx[j] < valid) {
+      k[j] = keys[base + idx[j]];
+      if constexpr (kHasValues) s_vals[idx[j]] = values[base + idx[j]];
+    } else {
+      k[j] = keys[base];  // any initialised value: never compared as a key
+    }
+  }
+
+  // thread-local stable sort: odd-even transposition, swapping only strictly out-of-order pairs
+#pragma unroll
+  for (int round = 0; round < kIpt; round++) {
+#pragma unroll
+    for (int j = round & 1; j + 1 < kIpt; j += 2) {
+      if (before(k[j + 1], idx[j + 1], k[j], idx[j])) {
+        const K tk = k[j]; k[j] = k[j + 1]; k[j + 1] = tk;
+        const int ti = idx[j]; idx[j] = idx[j + 1]; idx[j + 1] = ti;
+      }
+    }
+  }
+
+  // merge runs of `width` items pairwise, doubling the width
+  for (int width = kIpt; width < kTile; width *= 2) {
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kIpt; j++) {
+      s_keys[tid * kIpt + j] = k[j];
+      s_idx[tid * kIpt + j] = (std::uint16_t)idx[j];
+    }
+    __syncthreads();
+    const int start = (tid * kIpt) & ~(2 * width - 1);
+    const int diag = tid * kIpt - start;
+    const K* a = s_keys + start;
+    const K* b = a + width;
+    const std::uint16_t* ia = s_idx + start;
+    const std::uint16_t* ib = ia + width;
+    // merge path with the position-aware order
+    int lo = diag > width ? diag - width : 0;
+    int hi = diag < width ? diag : width;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (!before(b[diag - 1 - mid], ib[diag - 1 - mid], a[mid], ia[mid])) lo = mid + 1;
+      else hi = mid;
+    }
+    int pa = lo, pb = diag - lo;
+#pragma unroll
+    for (int j = 0; j < kIpt; j++) {
+      bool take_a;
+      if (pa >= width) take_a = false;
+      else if (pb >= width) take_a = true;
+      else take_a = !before(b[pb], ib[pb], a[pa], ia[pa]);
+      if (take_a) { k[j] = a[pa]; idx[j] = ia[pa]; pa++; }
+      else { k[j] = b[pb]; idx[j] = ib[pb]; pb++; }
+    }
+#pragma unroll
+    for (int j = 0; j < kIpt; j++) {  // all LDS reads of this round have landed before the next barrier
+      settle(k[j]);
+      settle(idx[j]);
+    }
+  }
+
+  // the first `valid` outputs are the real items, in order
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kIpt; j++) {
+    const int o = tid * kIpt + j;
+    if (o < valid) {
+      keys[base + o] = k[j];
+      if constexpr (kHasValues) values[base + o] = s_vals[idx[j]];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// 2. One merge pass: runs of `width` items -> runs of 2*width
+// ---------------------------------------------------------------------------------------
+struct pair_geometry {
+  std::int64_t a0, na, b0, nb, diag;
+};
+__device__ inline pair_geometry geometry_of(std::int64_t tile, std::int64_t width, std::int64_t n) {
+  pair_geometry g;
+  const std::int64_t out0 = tile * kTile;
+  const std::int64_t pstart = out0 / (2 * width) * (2 * width);
+  g.a0 = pstart;
+  const std::int64_t a1 = pstart + width < n ? pstart + width : n;
+  const std::int64_t b1 = pstart + 2 * width < n ? pstart + 2 * width : n;
+  g.na = a1 - g.a0;
+  g.b0 = a1;
+  g.nb = b1 - a1;
+  g.diag = out0 - pstart;
+  return g;
+}
+
+// splits[t] = how many items of the left run precede output tile t (binary search in global memory)
+template <class K, class Compare>
+__global__ __launch_bounds__(256) void merge_partition_kernel(const K* keys, std::int64_t n, std::int64_t width,
+                                                              std::int64_t ntiles, std::int64_t* splits,
+                                                              Compare comp) {
+  const std::int64_t t = (std::int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= ntiles) return;
+  const pair_geometry g = geometry_of(t, width, n);
+  const K* a = keys + g.a0;
+  const K* b = keys + g.b0;
+  std::int64_t lo = g.diag > g.nb ? g.diag - g.nb : 0;
+  std::int64_t hi = g.diag < g.na ? g.diag : g.na;
+  while (lo < hi) {
+    const std::int64_t mid = (lo + hi) >> 1;
+    if (!comp(b[g.diag - 1 - mid], a[mid])) lo = mid + 1;
+    else hi = mid;
+  }
+  splits[t] = lo;
+}
+
+template <class K, class V, class Compare>
+__global__ __launch_bounds__(kBlock) void merge_kernel(const K* kin, const V* vin, K* kout, V* vout, std::int64_t n,
+                                                       std::int64_t width, std::int64_t ntiles,
+                                                       const std::int64_t* splits, Compare comp) {
+  constexpr bool kHasValues = !std::is_same<V, no_value>::value;
+  __shared__ K s_keys[kTile];
+  __shared__ typename std::conditional<kHasValues, V, char>::type s_vals[kHasValues ? kTile : 1];
+
+  const int tid = threadIdx.x;
+  const std::int64_t tile = blockIdx.x;
+  const pair_geometry g = geometry_of(tile, width, n);
+  const std::int64_t total = g.na + g.nb;                                 // outputs of the pair
+  const int count = (int)(total - g.diag < kTile ? total - g.diag : kTile);  // outputs of this tile
+  // left-run items before this tile and before the next one (the pair's last tile takes the rest)
+  const std::int64_t sa0 = splits[tile];
+  const bool last_of_pair = g.diag + kTile >= total;
+  const std::int64_t sa1 = last_of_pair ? g.na : splits[tile + 1];
+  const int na = (int)(sa1 - sa0);
+  const int nb = count - na;
+
+  for (int i = tid; i < count; i += kBlock) {
+    const std::int64_t src = i < na ? (g.a0 + sa0 + i) : (g.b0 + (g.diag - sa0) + (i - na));
+    s_keys[i] = kin[src];
+    if constexpr (kHasValues) s_vals[i] = vin[src];
+  }
+  __syncthreads();
+
+  const K* a = s_keys;
+  const K* b = s_keys + na;
+  int d = tid * kIpt;
+  if (d > count) d = count;
+  int pa = merge_path(a, na, b, nb, d, comp);
+  int pb = d - pa;
+  K k[kIpt];
+  std::uint16_t src[kIpt];
+#pragma unroll
+  for (int j = 0; j < kIpt; j++) {
+    bool take_a;
+    if (pa >= na) take_a = false;
+    else if (pb >= nb) take_a = true;
+    else take_a = !comp(b[pb], a[pa]);
+    if (d + j < count) {
+      if (take_a) { k[j] = a[pa]; src[j] = (std::uint16_t)pa; pa++; }
+      else { k[j] = b[pb]; src[j] = (std::uint16_t)(na + pb); pb++; }
+    }
+  }
+  const std::int64_t out0 = tile * kTile;
+#pragma unroll
+  for (int j = 0; j < kIpt; j++) {
+    if (d + j < count) {
+      kout[out0 + d + j] = k[j];
+      if constexpr (kHasValues) vout[out0 + d + j] = s_vals[src[j]];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------
+inline std::size_t align256(std::size_t x) { return (x + 255) & ~std::size_t(255); }
+
+template <class K, class V, class Compare>
+void stable_sort(void* stream_, K* keys, V* values, std::int64_t n, Compare comp) {
+  static_assert(std::is_trivially_copyable<K>::value, "cdna4 merge sort: keys must be trivially copyable");
+  static_assert(std::is_trivially_copyable<V>::value, "cdna4 merge sort: values must be trivially copyable");
+  static_assert(sizeof(K) + sizeof(V) <= 28, "cdna4 merge sort: a tile of keys and values must fit the 64 KiB of static LDS");
+  constexpr bool kHasValues = !std::is_same<V, no_value>::value;
+  if (n <= 1) return;
+  hipStream_t s = static_cast<hipStream_t>(stream_);
+  const std::int64_t ntiles = (n + kTile - 1) / kTile;
+
+  hipLaunchKernelGGL((block_sort_kernel<K, V, Compare>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, keys, values, n, comp);
+  throw_on_error((int)hipGetLastError(), "merge sort: tile sort launch");
+  if (ntiles == 1) return;
+
+  const std::size_t kbytes = align256((std::size_t)n * sizeof(K));
+  const std::size_t vbytes = kHasValues ? align256((std::size_t)n * sizeof(V)) : 0;
+  const std::size_t sbytes = align256((std::size_t)(ntiles + 1) * sizeof(std::int64_t));
+  temporary_storage tmp(kbytes + vbytes + sbytes, stream_);
+  char* t = static_cast<char*>(tmp.data());
+  K* kbuf[2] = {keys, reinterpret_cast<K*>(t)};
+  V* vbuf[2] = {values, reinterpret_cast<V*>(t + kbytes)};
+  std::int64_t* splits = reinterpret_cast<std::int64_t*>(t + kbytes + vbytes);
+
+  int cur = 0;
+  for (std::int64_t width = kTile; width < n; width *= 2) {
+    hipLaunchKernelGGL((merge_partition_kernel<K, Compare>), dim3((unsigned)((ntiles + 255) / 256)), dim3(256), 0, s,
+                       kbuf[cur], n, width, ntiles, splits, comp);
+    hipLaunchKernelGGL((merge_kernel<K, V, Compare>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, kbuf[cur], vbuf[cur],
+                       kbuf[cur ^ 1], vbuf[cur ^ 1], n, width, ntiles, splits, comp);
+    throw_on_error((int)hipGetLastError(), "merge sort: merge pass launch");
+    cur ^= 1;
+  }
+  if (cur == 1) {  // odd number of passes: bring the result home
+    throw_on_error(thrust_cdna4_memcpy_dtod(kbuf[0], kbuf[1], (std::size_t)n * sizeof(K), stream_), "merge sort: copy back");
+    if (kHasValues)
+      throw_on_error(thrust_cdna4_memcpy_dtod(vbuf[0], vbuf[1], (std::size_t)n * sizeof(V), stream_), "merge sort: copy back");
+  }
+  // the temporary buffer is returned to the pool in stream order when `tmp` goes out of scope
+}
+
+}}}}}  // namespace thrust::system::cdna4::detail::merge

@@ -54,6 +54,12 @@ void assert_equal(const A& a, const B& b, const char* expr, const char* file, in
     fail(file, line, os.str());
   }
 }
+// characters print as numbers; everything else as it is
+template <class T, typename std::enable_if<std::is_arithmetic<T>::value, int>::type = 0>
+auto printable(const T& x) -> decltype(+x) { return +x; }
+template <class T, typename std::enable_if<!std::is_arithmetic<T>::value, int>::type = 0>
+const T& printable(const T& x) { return x; }
+
 template <class T, class U>
 void assert_equal_vec(const std::vector<T>& a, const std::vector<U>& b, const char* expr, const char* file, int line) {
   if (a.size() != b.size()) {
@@ -64,7 +70,7 @@ void assert_equal_vec(const std::vector<T>& a, const std::vector<U>& b, const ch
   for (std::size_t i = 0; i < a.size(); i++) {
     if (!(a[i] == (T)b[i])) {
       std::ostringstream os;
-      os << expr << " failed at [" << i << "] of " << a.size() << ": " << +a[i] << " vs " << +b[i];
+      os << expr << " failed at [" << i << "] of " << a.size() << ": " << printable(a[i]) << " vs " << printable(b[i]);
       fail(file, line, os.str());
     }
   }

@@ -17,10 +17,10 @@ def compile_snippet(tmp_path, body, extra=()):
                           capture_output=True, text=True)
 
 
-def test_cpp_tests_compile_with_gxx():
+def test_cpp_tests_compile():
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    for name in ["test_sort", "test_scan", "test_by_key", "test_system"]:
+    for name in ["test_sort", "test_scan", "test_by_key", "test_system", "test_merge_sort", "bench_merge_sort"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
 
 
@@ -65,7 +65,21 @@ def test_unsupported_comparator_is_a_compile_error_not_a_host_fallback(tmp_path)
         struct by_mod3 { bool operator()(int a, int b) const { return a % 3 < b % 3; } };
         int main() { thrust::device_vector<int> d(10); thrust::sort(d.begin(), d.end(), by_mod3()); }""")
     assert r.returncode != 0
-    assert "radix kernel" in r.stderr
+    assert "compile this translation unit with hipcc" in r.stderr
+
+
+def test_custom_comparator_compiles_with_hipcc(tmp_path):
+    # the same code builds when the device compiler can instantiate the comparison-sort kernels
+    src = tmp_path / "t.cpp"
+    src.write_text(textwrap.dedent("""
+        #include <thrust/device_vector.h>
+        #include <thrust/sort.h>
+        struct by_mod3 { __host__ __device__ bool operator()(int a, int b) const { return a % 3 < b % 3; } };
+        int main() { thrust::device_vector<int> d(10), v(10); thrust::sort(d.begin(), d.end(), by_mod3());
+                     thrust::stable_sort_by_key(d.begin(), d.end(), v.begin(), by_mod3()); }"""))
+    r = subprocess.run(["/opt/rocm/bin/hipcc", "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-fsyntax-only",
+                        "-I", INC, str(src)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
 
 
 def test_exclusive_scan_init_type_must_be_the_element_type(tmp_path):

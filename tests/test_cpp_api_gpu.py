@@ -1,4 +1,4 @@
-"""Runs the C++ API tests (tests/cpp/*.cpp) on the GPU.  They are plain g++ translation
+"""Runs the C++ API tests (tests/cpp/*.cpp) on the GPU.  All but one are plain g++ translation
 units that use thrust::device_vector, thrust::sort, thrust::inclusive_scan,
 thrust::reduce_by_key ... from include/thrust and link only against libthrust_cdna4.so; each
 mirrors one of the reference's own test files and compares host and device results."""
@@ -10,7 +10,8 @@ import pytest
 from conftest import ROOT
 
 BIN_DIR = os.path.join(ROOT, "tests", "cpp", "build")
-BINARIES = ["test_sort", "test_scan", "test_by_key", "test_system"]
+# test_merge_sort instantiates kernel templates with user comparators and is compiled by hipcc
+BINARIES = ["test_sort", "test_scan", "test_by_key", "test_system", "test_merge_sort"]
 
 
 @pytest.mark.gpu
