@@ -9,14 +9,16 @@
 // and the comparator's operator() must be __host__ __device__.  Temporary storage comes from
 // the library's stream-ordered pool.
 //
-//   1. block_sort_kernel   a 256-thread workgroup sorts a tile of 2048 items: every thread
-//                          sorts its 8 consecutive items in registers (odd-even transposition,
-//                          stable), then log2(256) rounds of merge-path merging through LDS.
+//   1. block_sort_kernel   a workgroup of kBlock threads sorts a tile of kBlock*kIpt items (512 x 4
+//                          measured best: the per-thread serial merge is the critical path, so
+//                          few items per thread and many threads): every thread
+//                          sorts its kIpt consecutive items in registers (odd-even transposition,
+//                          stable), then log2(kBlock) rounds of merge-path merging through LDS.
 //   2. merge_partition_kernel + merge_kernel, once per doubling of the run width: one thread
 //                          per output tile finds where the tile starts in the two runs it
 //                          merges (binary search on the merge path, ties to the left run);
 //                          a workgroup then loads the two pieces into LDS, every thread merges
-//                          its 8 outputs, and the tile is written back with contiguous stores.
+//                          its kIpt outputs, and the tile is written back with contiguous stores.
 //      Values follow their keys through LDS by source index.
 #pragma once
 #if !defined(__HIPCC__)
@@ -29,9 +31,16 @@
 
 namespace thrust { namespace system { namespace cdna4 { namespace detail { namespace merge {
 
-constexpr int kBlock = 256;
-constexpr int kIpt = 8;
+#ifndef THRUST_CDNA4_MERGE_BLOCK
+#define THRUST_CDNA4_MERGE_BLOCK 512
+#endif
+constexpr int kBlock = THRUST_CDNA4_MERGE_BLOCK;  // threads per workgroup
+#ifndef THRUST_CDNA4_MERGE_IPT
+#define THRUST_CDNA4_MERGE_IPT 4
+#endif
+constexpr int kIpt = THRUST_CDNA4_MERGE_IPT;  // items per thread
 constexpr int kTile = kBlock * kIpt;
+static_assert((kIpt & (kIpt - 1)) == 0 && kTile <= 65536, "run widths double from kIpt; 16-bit positions in a tile");
 
 struct no_value {};
 
@@ -133,15 +142,20 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
       if (!before(b[diag - 1 - mid], ib[diag - 1 - mid], a[mid], ia[mid])) lo = mid + 1;
       else hi = mid;
     }
+    // serial merge with the two candidate items held in registers: one LDS read per output
     int pa = lo, pb = diag - lo;
+    K ka = a[pa < width ? pa : width - 1], kb = b[pb < width ? pb : width - 1];
+    int xa = ia[pa < width ? pa : width - 1], xb = ib[pb < width ? pb : width - 1];
 #pragma unroll
     for (int j = 0; j < kIpt; j++) {
-      bool take_a;
-      if (pa >= width) take_a = false;
-      else if (pb >= width) take_a = true;
-      else take_a = !before(b[pb], ib[pb], a[pa], ia[pa]);
-      if (take_a) { k[j] = a[pa]; idx[j] = ia[pa]; pa++; }
-      else { k[j] = b[pb]; idx[j] = ib[pb]; pb++; }
+      const bool take_a = pb >= width || (pa < width && !before(kb, xb, ka, xa));
+      if (take_a) {
+        k[j] = ka; idx[j] = xa; pa++;
+        if (pa < width) { ka = a[pa]; xa = ia[pa]; }
+      } else {
+        k[j] = kb; idx[j] = xb; pb++;
+        if (pb < width) { kb = b[pb]; xb = ib[pb]; }
+      }
     }
 #pragma unroll
     for (int j = 0; j < kIpt; j++) {  // all LDS reads of this round have landed before the next barrier
@@ -237,15 +251,20 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(const K* kin, const V* vi
   int pb = d - pa;
   K k[kIpt];
   std::uint16_t src[kIpt];
+  // serial merge with the two candidate keys held in registers: one LDS read per output
+  // (the tile is never empty, so index 0 is always readable)
+  K ka = a[pa < na ? pa : 0], kb = s_keys[pb < nb ? na + pb : 0];
 #pragma unroll
   for (int j = 0; j < kIpt; j++) {
-    bool take_a;
-    if (pa >= na) take_a = false;
-    else if (pb >= nb) take_a = true;
-    else take_a = !comp(b[pb], a[pa]);
     if (d + j < count) {
-      if (take_a) { k[j] = a[pa]; src[j] = (std::uint16_t)pa; pa++; }
-      else { k[j] = b[pb]; src[j] = (std::uint16_t)(na + pb); pb++; }
+      const bool take_a = pb >= nb || (pa < na && !comp(kb, ka));
+      if (take_a) {
+        k[j] = ka; src[j] = (std::uint16_t)pa; pa++;
+        if (pa < na) ka = a[pa];
+      } else {
+        k[j] = kb; src[j] = (std::uint16_t)(na + pb); pb++;
+        if (pb < nb) kb = b[pb];
+      }
     }
   }
   const std::int64_t out0 = tile * kTile;
@@ -267,7 +286,7 @@ template <class K, class V, class Compare>
 void stable_sort(void* stream_, K* keys, V* values, std::int64_t n, Compare comp) {
   static_assert(std::is_trivially_copyable<K>::value, "cdna4 merge sort: keys must be trivially copyable");
   static_assert(std::is_trivially_copyable<V>::value, "cdna4 merge sort: values must be trivially copyable");
-  static_assert(sizeof(K) + sizeof(V) <= 28, "cdna4 merge sort: a tile of keys and values must fit the 64 KiB of static LDS");
+  static_assert((sizeof(K) + sizeof(V) + 2) * kTile <= 65536, "cdna4 merge sort: a tile of keys and values must fit the 64 KiB of static LDS");
   constexpr bool kHasValues = !std::is_same<V, no_value>::value;
   if (n <= 1) return;
   hipStream_t s = static_cast<hipStream_t>(stream_);

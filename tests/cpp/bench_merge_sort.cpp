@@ -71,9 +71,9 @@ int main(int argc, char** argv) {
   };
   const float ms_pairs = median_ms(run_pairs, restore, 5);
 
-  // passes over the data: one tile sort + ceil(log2(n / 2048)) merges, each reading and writing every item
+  // passes over the data: one tile sort + ceil(log2(n / tile)) merges, each reading and writing every item
   int passes = 1;
-  for (std::size_t w = 2048; w < n; w *= 2) passes++;
+  for (std::size_t w = thrust::system::cdna4::detail::merge::kTile; w < n; w *= 2) passes++;
   std::printf(
       "{\"merge_sort_u32_custom_less\": {\"value\": %.3f, \"unit\": \"Gkeys/s\", \"ms\": %.3f, \"n\": %zu, \"passes\": %d, "
       "\"traffic_GBs\": %.1f, \"sorted\": %s}, \"merge_sort_by_key_u32_u32_custom_less\": {\"value\": %.3f, \"unit\": "
