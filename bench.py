@@ -269,7 +269,18 @@ def main():
         if r.returncode == 0:
             extras.update(json.loads(r.stdout.strip().splitlines()[-1]))
 
+    def extra_generic():
+        # transform / reduce with user functors (kernel templates): tests/cpp/bench_generic.cpp, 2^28 floats
+        import subprocess
+        exe = os.path.join(ROOT, "tests", "cpp", "build", "bench_generic")
+        if not os.path.exists(exe):
+            return
+        r = subprocess.run([exe, str(args.log2n)], capture_output=True, text=True, timeout=300)
+        if r.returncode == 0:
+            extras.update(json.loads(r.stdout.strip().splitlines()[-1]))
+
     all_extras = {
+        "generic": extra_generic,
         "merge_sort": extra_merge_sort,
         "sort_by_key": extra_sort_pairs,
         "scan_i32": lambda: extra_scan("i32"),

@@ -1,0 +1,29 @@
+// thrust::count / count_if (thrust/count.h): a transform_reduce of 0/1 flags.
+#pragma once
+#include <cstddef>
+#include <thrust/transform_reduce.h>
+
+namespace thrust {
+namespace detail {
+template <class F> struct flag_of {
+  F pred;
+  template <class T> THRUST_CDNA4_HD std::ptrdiff_t operator()(const T& x) const { return pred(x) ? 1 : 0; }
+};
+template <class V> struct equals_value {
+  V v;
+  template <class T> THRUST_CDNA4_HD bool operator()(const T& x) const { return x == v; }
+};
+}  // namespace detail
+template <class Policy, class It, class Pred>
+std::ptrdiff_t count_if(const Policy& exec, It first, It last, Pred pred) {
+  return transform_reduce(exec, first, last, detail::flag_of<Pred>{pred}, std::ptrdiff_t(0), plus<std::ptrdiff_t>());
+}
+template <class Policy, class It, class V, class = typename std::iterator_traits<It>::iterator_category>
+std::ptrdiff_t count(const Policy& exec, It first, It last, const V& value) {
+  return count_if(exec, first, last, detail::equals_value<V>{value});
+}
+template <class It, class Pred, detail::enable_if_device<It> = 0> std::ptrdiff_t count_if(It f, It l, Pred p) { return count_if(device, f, l, p); }
+template <class It, class Pred, detail::enable_if_host<It> = 0> std::ptrdiff_t count_if(It f, It l, Pred p) { return count_if(host, f, l, p); }
+template <class It, class V, detail::enable_if_device<It> = 0> std::ptrdiff_t count(It f, It l, const V& v) { return count(device, f, l, v); }
+template <class It, class V, detail::enable_if_host<It> = 0> std::ptrdiff_t count(It f, It l, const V& v) { return count(host, f, l, v); }
+}  // namespace thrust

@@ -1,0 +1,28 @@
+// thrust::for_each / for_each_n (thrust/for_each.h; thrust/system/cuda/detail/for_each.h).
+#pragma once
+#include <algorithm>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
+namespace thrust {
+template <class D, class It, class F>
+It for_each(const system::cdna4::execution_policy<D>& exec, It first, It last, F f) {
+  system::cdna4::detail::for_each_n(exec.derived(), detail::unwrap(first), (std::int64_t)(last - first), f);
+  return last;
+}
+template <class D, class It, class Size, class F>
+It for_each_n(const system::cdna4::execution_policy<D>& exec, It first, Size n, F f) {
+  system::cdna4::detail::for_each_n(exec.derived(), detail::unwrap(first), (std::int64_t)n, f);
+  return first + n;
+}
+template <class It, class F>
+It for_each(const system::cpp::detail::par_t&, It first, It last, F f) { std::for_each(first, last, f); return last; }
+template <class It, class Size, class F>
+It for_each_n(const system::cpp::detail::par_t&, It first, Size n, F f) { std::for_each(first, first + n, f); return first + n; }
+
+template <class It, class F, detail::enable_if_device<It> = 0> It for_each(It f, It l, F fn) { return for_each(device, f, l, fn); }
+template <class It, class F, detail::enable_if_host<It> = 0> It for_each(It f, It l, F fn) { return for_each(host, f, l, fn); }
+template <class It, class Size, class F, detail::enable_if_device<It> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(device, f, n, fn); }
+template <class It, class Size, class F, detail::enable_if_host<It> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(host, f, n, fn); }
+}  // namespace thrust

@@ -16,6 +16,19 @@ template <class T = void> struct minimum { THRUST_CDNA4_HD constexpr T operator(
 template <class T = void> struct less { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a < b; } };
 template <class T = void> struct greater { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a > b; } };
 template <class T = void> struct equal_to { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a == b; } };
+template <class T = void> struct minus { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a - b; } };
+template <class T = void> struct divides { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a / b; } };
+template <class T = void> struct modulus { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a % b; } };
+template <class T = void> struct negate { THRUST_CDNA4_HD constexpr T operator()(const T& a) const { return -a; } };
+template <class T = void> struct not_equal_to { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a != b; } };
+template <class T = void> struct less_equal { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a <= b; } };
+template <class T = void> struct greater_equal { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a >= b; } };
+template <class T = void> struct logical_and { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a && b; } };
+template <class T = void> struct logical_or { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a || b; } };
+template <class T = void> struct logical_not { THRUST_CDNA4_HD constexpr bool operator()(const T& a) const { return !a; } };
+template <class T = void> struct bit_and { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a & b; } };
+template <class T = void> struct bit_or { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a | b; } };
+template <class T = void> struct bit_xor { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a ^ b; } };
 template <class T = void> struct identity { THRUST_CDNA4_HD constexpr const T& operator()(const T& a) const { return a; } };
 
 // transparent forms (thrust::plus<> etc.)

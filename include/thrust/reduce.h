@@ -1,8 +1,11 @@
-// thrust::reduce_by_key (thrust/reduce.h:691-).  Device ranges go to the single-pass
-// segmented-reduction kernel; host ranges run the sequential loop
-// (thrust/system/detail/sequential/reduce_by_key.h:43-95).
+// thrust::reduce (thrust/reduce.h:78-) and thrust::reduce_by_key (thrust/reduce.h:691-).
+// reduce_by_key: device ranges go to the single-pass segmented-reduction kernel; host ranges run
+// the sequential loop (thrust/system/detail/sequential/reduce_by_key.h:43-95).  reduce: device
+// ranges go to the generic reduction kernel templates (a translation unit compiled by hipcc).
 #pragma once
+#include <numeric>
 #include <thrust/detail/iterator_util.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
 #include <thrust/pair.h>
@@ -80,5 +83,38 @@ pair<KOut, VOut> reduce_by_key(const system::cpp::detail::par_t& e, KIt kf, KIt 
 THRUST_CDNA4_RBK(device, detail::enable_if_device)
 THRUST_CDNA4_RBK(host, detail::enable_if_host)
 #undef THRUST_CDNA4_RBK
+
+
+// ---------------------------------------------------------------------------------------
+// reduce
+// ---------------------------------------------------------------------------------------
+template <class D, class It, class T, class Op>
+T reduce(const system::cdna4::execution_policy<D>& exec, It first, It last, T init, Op op) {
+  typedef typename detail::value_of<It>::type V;
+  return system::cdna4::detail::transform_reduce_n(exec.derived(), (const V*)detail::unwrap(first),
+                                                   (std::int64_t)(last - first), identity<V>(), init, op);
+}
+template <class D, class It, class T>
+T reduce(const system::cdna4::execution_policy<D>& exec, It first, It last, T init) { return reduce(exec, first, last, init, plus<T>()); }
+template <class D, class It>
+typename detail::value_of<It>::type reduce(const system::cdna4::execution_policy<D>& exec, It first, It last) {
+  typedef typename detail::value_of<It>::type V;
+  return reduce(exec, first, last, V(0), plus<V>());
+}
+template <class It, class T, class Op>
+T reduce(const system::cpp::detail::par_t&, It first, It last, T init, Op op) { return std::accumulate(first, last, init, op); }
+template <class It, class T>
+T reduce(const system::cpp::detail::par_t&, It first, It last, T init) { return std::accumulate(first, last, init); }
+template <class It>
+typename detail::value_of<It>::type reduce(const system::cpp::detail::par_t&, It first, It last) {
+  typedef typename detail::value_of<It>::type V;
+  return std::accumulate(first, last, V(0));
+}
+template <class It, detail::enable_if_device<It> = 0> typename detail::value_of<It>::type reduce(It f, It l) { return reduce(device, f, l); }
+template <class It, detail::enable_if_host<It> = 0> typename detail::value_of<It>::type reduce(It f, It l) { return reduce(host, f, l); }
+template <class It, class T, detail::enable_if_device<It> = 0> T reduce(It f, It l, T init) { return reduce(device, f, l, init); }
+template <class It, class T, detail::enable_if_host<It> = 0> T reduce(It f, It l, T init) { return reduce(host, f, l, init); }
+template <class It, class T, class Op, detail::enable_if_device<It> = 0> T reduce(It f, It l, T init, Op op) { return reduce(device, f, l, init, op); }
+template <class It, class T, class Op, detail::enable_if_host<It> = 0> T reduce(It f, It l, T init, Op op) { return reduce(host, f, l, init, op); }
 
 }  // namespace thrust

@@ -1,0 +1,33 @@
+// thrust::sequence (thrust/sequence.h): first[i] = init + i * step.
+#pragma once
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
+namespace thrust {
+template <class D, class It, class T>
+void sequence(const system::cdna4::execution_policy<D>& exec, It first, It last, T init, T step) {
+  typedef typename detail::value_of<It>::type V;
+  system::cdna4::detail::sequence_n(exec.derived(), detail::unwrap(first), (std::int64_t)(last - first), (V)init, (V)step);
+}
+template <class It, class T>
+void sequence(const system::cpp::detail::par_t&, It first, It last, T init, T step) {
+  typedef typename detail::value_of<It>::type V;
+  std::size_t i = 0;
+  for (; first != last; ++first, ++i) *first = (V)((V)init + (V)i * (V)step);
+}
+template <class Policy, class It, class T>
+void sequence(const Policy& exec, It first, It last, T init) { sequence(exec, first, last, init, T(1)); }
+template <class Policy, class It, class = typename std::iterator_traits<It>::iterator_category>
+void sequence(const Policy& exec, It first, It last) {
+  typedef typename detail::value_of<It>::type V;
+  sequence(exec, first, last, V(0), V(1));
+}
+
+template <class It, detail::enable_if_device<It> = 0> void sequence(It f, It l) { sequence(device, f, l); }
+template <class It, detail::enable_if_host<It> = 0> void sequence(It f, It l) { sequence(host, f, l); }
+template <class It, class T, detail::enable_if_device<It> = 0> void sequence(It f, It l, T init) { sequence(device, f, l, init); }
+template <class It, class T, detail::enable_if_host<It> = 0> void sequence(It f, It l, T init) { sequence(host, f, l, init); }
+template <class It, class T, detail::enable_if_device<It> = 0> void sequence(It f, It l, T init, T step) { sequence(device, f, l, init, step); }
+template <class It, class T, detail::enable_if_host<It> = 0> void sequence(It f, It l, T init, T step) { sequence(host, f, l, init, step); }
+}  // namespace thrust

@@ -1,0 +1,40 @@
+// thrust::transform, unary and binary (thrust/transform.h; thrust/system/cuda/detail/transform.h).
+#pragma once
+#include <algorithm>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
+namespace thrust {
+template <class D, class In, class Out, class F>
+Out transform(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, F f) {
+  const std::int64_t n = (std::int64_t)(last - first);
+  system::cdna4::detail::transform_n(exec.derived(), (const typename detail::value_of<In>::type*)detail::unwrap(first),
+                                     detail::unwrap(out), n, f);
+  return out + n;
+}
+template <class D, class In1, class In2, class Out, class F>
+Out transform(const system::cdna4::execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out out, F f) {
+  const std::int64_t n = (std::int64_t)(last1 - first1);
+  system::cdna4::detail::transform_n(exec.derived(), (const typename detail::value_of<In1>::type*)detail::unwrap(first1),
+                                     (const typename detail::value_of<In2>::type*)detail::unwrap(first2), detail::unwrap(out), n, f);
+  return out + n;
+}
+template <class In, class Out, class F>
+Out transform(const system::cpp::detail::par_t&, In first, In last, Out out, F f) { return std::transform(first, last, out, f); }
+template <class In1, class In2, class Out, class F>
+Out transform(const system::cpp::detail::par_t&, In1 first1, In1 last1, In2 first2, Out out, F f) {
+  return std::transform(first1, last1, first2, out, f);
+}
+
+template <class In, class Out, class F, detail::enable_if_device<In> = 0>
+Out transform(In f, In l, Out o, F fn) { return transform(device, f, l, o, fn); }
+template <class In, class Out, class F, detail::enable_if_host<In> = 0>
+Out transform(In f, In l, Out o, F fn) { return transform(host, f, l, o, fn); }
+template <class In1, class In2, class Out, class F, detail::enable_if_device<In1> = 0,
+          class = typename std::iterator_traits<In2>::iterator_category>
+Out transform(In1 f, In1 l, In2 f2, Out o, F fn) { return transform(device, f, l, f2, o, fn); }
+template <class In1, class In2, class Out, class F, detail::enable_if_host<In1> = 0,
+          class = typename std::iterator_traits<In2>::iterator_category>
+Out transform(In1 f, In1 l, In2 f2, Out o, F fn) { return transform(host, f, l, f2, o, fn); }
+}  // namespace thrust

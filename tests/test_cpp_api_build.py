@@ -20,7 +20,8 @@ def compile_snippet(tmp_path, body, extra=()):
 def test_cpp_tests_compile():
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    for name in ["test_sort", "test_scan", "test_by_key", "test_system", "test_merge_sort", "bench_merge_sort"]:
+    for name in ["test_sort", "test_scan", "test_by_key", "test_system", "test_merge_sort", "bench_merge_sort", "test_generic",
+                 "bench_generic"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
 
 
@@ -89,3 +90,33 @@ def test_exclusive_scan_init_type_must_be_the_element_type(tmp_path):
         int main() { thrust::device_vector<float> d(10), o(10); thrust::exclusive_scan(d.begin(), d.end(), o.begin(), 0); }""")
     assert r.returncode != 0
     assert "accumulator type" in r.stderr
+
+
+def test_user_functor_on_device_range_needs_hipcc(tmp_path):
+    body = """
+        #include <thrust/device_vector.h>
+        #include <thrust/transform.h>
+        #include <thrust/reduce.h>
+        struct twice { THRUST_CDNA4_HD int operator()(int x) const { return 2 * x; } };
+        int main() { thrust::device_vector<int> d(10), o(10); thrust::transform(d.begin(), d.end(), o.begin(), twice());
+                     return thrust::reduce(o.begin(), o.end(), 0); }"""
+    r = compile_snippet(tmp_path, body)
+    assert r.returncode != 0
+    assert "compile this translation unit with hipcc" in r.stderr
+    src = tmp_path / "t.cpp"
+    r = subprocess.run(["/opt/rocm/bin/hipcc", "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-fsyntax-only",
+                        "-I", INC, str(src)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_host_ranges_with_functors_build_with_gxx(tmp_path):
+    r = compile_snippet(tmp_path, """
+        #include <thrust/host_vector.h>
+        #include <thrust/transform.h>
+        #include <thrust/reduce.h>
+        #include <thrust/sequence.h>
+        #include <thrust/count.h>
+        int main() { thrust::host_vector<int> h(10), o(10); thrust::sequence(h.begin(), h.end());
+                     thrust::transform(h.begin(), h.end(), o.begin(), thrust::negate<int>());
+                     return thrust::reduce(o.begin(), o.end()) + (int)thrust::count(o.begin(), o.end(), -3); }""")
+    assert r.returncode == 0, r.stderr[-3000:]
