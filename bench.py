@@ -279,8 +279,19 @@ def main():
         if r.returncode == 0:
             extras.update(json.loads(r.stdout.strip().splitlines()[-1]))
 
+    def extra_select():
+        # copy_if / unique / unique_by_key with user predicates (kernel templates): tests/cpp/bench_select.cpp
+        import subprocess
+        exe = os.path.join(ROOT, "tests", "cpp", "build", "bench_select")
+        if not os.path.exists(exe):
+            return
+        r = subprocess.run([exe, str(args.log2n)], capture_output=True, text=True, timeout=300)
+        if r.returncode == 0:
+            extras.update(json.loads(r.stdout.strip().splitlines()[-1]))
+
     all_extras = {
         "generic": extra_generic,
+        "select": extra_select,
         "merge_sort": extra_merge_sort,
         "sort_by_key": extra_sort_pairs,
         "scan_i32": lambda: extra_scan("i32"),

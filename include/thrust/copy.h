@@ -48,3 +48,39 @@ OutIt copy(InIt first, InIt last, OutIt out) {
   return std::copy(first, last, out);
 }
 }  // namespace thrust
+
+// thrust::copy_if, with and without a stencil (thrust/copy.h; thrust/system/cuda/detail/copy_if.h):
+// stable compaction with a user predicate — kernel templates on device ranges.
+#include <thrust/execution_policy.h>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+namespace thrust {
+template <class D, class In, class Out, class Pred>
+Out copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Pred pred) {
+  typedef typename detail::value_of<In>::type V;
+  const V* in = (const V*)detail::unwrap(first);
+  return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), in, detail::unwrap(out), (std::int64_t)(last - first), pred);
+}
+template <class D, class In, class St, class Out, class Pred>
+Out copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, St stencil, Out out, Pred pred) {
+  typedef typename detail::value_of<In>::type V;
+  typedef typename detail::value_of<St>::type S;
+  return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), (const V*)detail::unwrap(first), (const S*)detail::unwrap(stencil),
+                                                            detail::unwrap(out), (std::int64_t)(last - first), pred);
+}
+template <class In, class Out, class Pred>
+Out copy_if(const system::cpp::detail::par_t&, In first, In last, Out out, Pred pred) { return std::copy_if(first, last, out, pred); }
+template <class In, class St, class Out, class Pred>
+Out copy_if(const system::cpp::detail::par_t&, In first, In last, St stencil, Out out, Pred pred) {
+  for (; first != last; ++first, ++stencil) if (pred(*stencil)) { *out = *first; ++out; }
+  return out;
+}
+template <class In, class Out, class Pred, detail::enable_if_device<In> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(device, f, l, o, p); }
+template <class In, class Out, class Pred, detail::enable_if_host<In> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(host, f, l, o, p); }
+template <class In, class St, class Out, class Pred, detail::enable_if_device<In> = 0,
+          class = typename std::iterator_traits<St>::iterator_category>
+Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(device, f, l, s, o, p); }
+template <class In, class St, class Out, class Pred, detail::enable_if_host<In> = 0,
+          class = typename std::iterator_traits<St>::iterator_category>
+Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(host, f, l, s, o, p); }
+}  // namespace thrust

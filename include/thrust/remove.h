@@ -1,0 +1,42 @@
+// thrust::remove / remove_if / remove_copy / remove_copy_if (thrust/remove.h;
+// thrust/system/cuda/detail/remove.h): stable; the in-place forms compact from a temporary copy.
+#pragma once
+#include <algorithm>
+#include <thrust/count.h>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
+namespace thrust {
+template <class D, class In, class Out, class Pred>
+Out remove_copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Pred pred) {
+  typedef typename detail::value_of<In>::type V;
+  const V* in = (const V*)detail::unwrap(first);
+  return out + system::cdna4::detail::copy_flagged_n<true>(exec.derived(), in, detail::unwrap(out), (std::int64_t)(last - first), pred);
+}
+template <class D, class In, class Pred>
+In remove_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Pred pred) {
+  typedef typename detail::value_of<In>::type V;
+  const std::int64_t n = (std::int64_t)(last - first);
+  system::cdna4::detail::scratch_copy<V> tmp((const V*)detail::unwrap(first), n, system::cdna4::detail::stream_of(exec.derived()));
+  return first + system::cdna4::detail::copy_flagged_n<true>(exec.derived(), tmp.data(), detail::unwrap(first), n, pred);
+}
+template <class In, class Out, class Pred>
+Out remove_copy_if(const system::cpp::detail::par_t&, In first, In last, Out out, Pred pred) { return std::remove_copy_if(first, last, out, pred); }
+template <class In, class Pred>
+In remove_if(const system::cpp::detail::par_t&, In first, In last, Pred pred) { return std::remove_if(first, last, pred); }
+
+template <class Policy, class In, class Out, class V, class = typename std::iterator_traits<In>::iterator_category>
+Out remove_copy(const Policy& exec, In first, In last, Out out, const V& value) {
+  return remove_copy_if(exec, first, last, out, detail::equals_value<V>{value});
+}
+template <class Policy, class In, class V, class = typename std::iterator_traits<In>::iterator_category>
+In remove(const Policy& exec, In first, In last, const V& value) { return remove_if(exec, first, last, detail::equals_value<V>{value}); }
+
+template <class In, class Out, class Pred, detail::enable_if_device<In> = 0> Out remove_copy_if(In f, In l, Out o, Pred p) { return remove_copy_if(device, f, l, o, p); }
+template <class In, class Out, class Pred, detail::enable_if_host<In> = 0> Out remove_copy_if(In f, In l, Out o, Pred p) { return remove_copy_if(host, f, l, o, p); }
+template <class In, class Pred, detail::enable_if_device<In> = 0> In remove_if(In f, In l, Pred p) { return remove_if(device, f, l, p); }
+template <class In, class Pred, detail::enable_if_host<In> = 0> In remove_if(In f, In l, Pred p) { return remove_if(host, f, l, p); }
+template <class In, class V, detail::enable_if_device<In> = 0> In remove(In f, In l, const V& v) { return remove(device, f, l, v); }
+template <class In, class V, detail::enable_if_host<In> = 0> In remove(In f, In l, const V& v) { return remove(host, f, l, v); }
+}  // namespace thrust

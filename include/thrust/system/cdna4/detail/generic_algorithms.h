@@ -96,4 +96,107 @@ T transform_reduce_n(const Policy& exec, const In* in, std::int64_t n, F f, T in
 #endif
 }
 
+// ---- stable compaction (copy_if / remove_if / unique / unique_by_key) ------------------
+#if defined(__HIPCC__)
+// keep in[i] when pred(in[i]) != NEGATE
+template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
+  typedef In item;
+  const In* in; Out* out; Pred pred;
+  __device__ item load(std::int64_t i, bool& keep) const {
+    const In x = in[i];
+    keep = (bool)pred(x) != NEGATE;
+    return x;
+  }
+  __device__ void store(const item& x, std::int64_t pos) const { out[pos] = x; }
+};
+// keep in[i] when pred(stencil[i]) != NEGATE
+template <class In, class S, class Out, class Pred, bool NEGATE> struct keep_if_stencil_op {
+  typedef In item;
+  const In* in; const S* stencil; Out* out; Pred pred;
+  __device__ item load(std::int64_t i, bool& keep) const {
+    keep = (bool)pred(stencil[i]) != NEGATE;
+    return in[i];
+  }
+  __device__ void store(const item& x, std::int64_t pos) const { out[pos] = x; }
+};
+// keep the first element of every run; element 0 compares with itself and is kept by index
+template <class K, class KOut, class Eq> struct run_head_op {
+  typedef K item;
+  const K* keys; KOut* out; Eq eq;
+  __device__ item load(std::int64_t i, bool& keep) const {
+    const K cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
+    keep = (i == 0) | !(bool)eq(prev, cur);
+    return cur;
+  }
+  __device__ void store(const item& x, std::int64_t pos) const { out[pos] = x; }
+};
+template <class K, class V, class KOut, class VOut, class Eq> struct run_head_by_key_op {
+  struct item { K key; V value; };
+  const K* keys; const V* values; KOut* kout; VOut* vout; Eq eq;
+  __device__ item load(std::int64_t i, bool& keep) const {
+    const K cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
+    keep = (i == 0) | !(bool)eq(prev, cur);
+    return item{cur, values[i]};
+  }
+  __device__ void store(const item& x, std::int64_t pos) const { kout[pos] = x.key; vout[pos] = x.value; }
+};
+#endif
+
+// out[0, count) = the in[i] with pred(in[i]) != NEGATE, in order; returns count
+template <bool NEGATE, class Policy, class In, class Out, class Pred>
+std::int64_t copy_flagged_n(const Policy& exec, const In* in, Out* out, std::int64_t n, Pred pred) {
+  THRUST_CDNA4_NEEDS_HIPCC(Pred);
+#if defined(__HIPCC__)
+  return generic::select(stream_of(exec), n, keep_if_op<In, Out, Pred, NEGATE>{in, out, pred});
+#else
+  (void)exec; (void)in; (void)out; (void)n; (void)pred;
+  return 0;
+#endif
+}
+// the same with the predicate applied to stencil[i]
+template <bool NEGATE, class Policy, class In, class S, class Out, class Pred>
+std::int64_t copy_flagged_n(const Policy& exec, const In* in, const S* stencil, Out* out, std::int64_t n, Pred pred) {
+  THRUST_CDNA4_NEEDS_HIPCC(Pred);
+#if defined(__HIPCC__)
+  return generic::select(stream_of(exec), n, keep_if_stencil_op<In, S, Out, Pred, NEGATE>{in, stencil, out, pred});
+#else
+  (void)exec; (void)in; (void)stencil; (void)out; (void)n; (void)pred;
+  return 0;
+#endif
+}
+// out[0, count) = the first element of every run of equal elements; returns count
+template <class Policy, class K, class KOut, class Eq>
+std::int64_t unique_copy_n(const Policy& exec, const K* in, KOut* out, std::int64_t n, Eq eq) {
+  THRUST_CDNA4_NEEDS_HIPCC(Eq);
+#if defined(__HIPCC__)
+  return generic::select(stream_of(exec), n, run_head_op<K, KOut, Eq>{in, out, eq});
+#else
+  (void)exec; (void)in; (void)out; (void)n; (void)eq;
+  return 0;
+#endif
+}
+template <class Policy, class K, class V, class KOut, class VOut, class Eq>
+std::int64_t unique_by_key_copy_n(const Policy& exec, const K* keys, const V* vals, KOut* kout, VOut* vout, std::int64_t n, Eq eq) {
+  THRUST_CDNA4_NEEDS_HIPCC(Eq);
+#if defined(__HIPCC__)
+  return generic::select(stream_of(exec), n, run_head_by_key_op<K, V, KOut, VOut, Eq>{keys, vals, kout, vout, eq});
+#else
+  (void)exec; (void)keys; (void)vals; (void)kout; (void)vout; (void)n; (void)eq;
+  return 0;
+#endif
+}
+
+// A device copy of [p, p + n) from the pool, for the in-place variants (the compaction reads its
+// whole input while other tiles already write the front of the output).
+template <class T>
+class scratch_copy {
+ public:
+  scratch_copy(const T* p, std::int64_t n, void* stream) : tmp_((std::size_t)n * sizeof(T), stream) {
+    if (n > 0) throw_on_error(thrust_cdna4_memcpy_dtod(tmp_.data(), p, (std::size_t)n * sizeof(T), stream), "temporary copy");
+  }
+  const T* data() const { return static_cast<const T*>(tmp_.data()); }
+ private:
+  temporary_storage tmp_;
+};
+
 }}}}  // namespace thrust::system::cdna4::detail

@@ -3,12 +3,13 @@
 // They carry user functors, so the translation unit that instantiates them is compiled by
 // hipcc (--offload-arch=gfx950) and the functors' operator() must be __host__ __device__.
 // for_each, transform, sequence, transform_reduce, reduce and count_if in the public headers are
-// thin wrappers over these two.
+// thin wrappers over these two; copy_if, remove_if and unique over the select engine below.
 #pragma once
 #if !defined(__HIPCC__)
 #error "thrust/system/cdna4/detail/parallel_for.h holds device kernel templates: compile with hipcc"
 #endif
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <cstdint>
 #include <type_traits>
 #include <thrust/system/cdna4/detail/core.h>
@@ -115,6 +116,170 @@ T transform_reduce(void* stream_, std::int64_t n, Unary unary, T init, Op op) {
   throw_on_error(thrust_cdna4_memcpy_dtoh(&result, out, sizeof(T), stream_), "reduce: read back");
   throw_on_error(thrust_cdna4_stream_synchronize(stream_), "reduce: failed to synchronize");
   return result;
+}
+
+// ---------------------------------------------------------------------------------------
+// select: stable compaction of the indices i in [0, n) that an operation keeps, in one pass
+// (the shape of the reference's select engine, thrust/system/cuda/detail/copy_if.h:221-520, on
+// 64-wide wavefronts).  The operation supplies
+//     typedef ... item;                               what travels from the load to the store
+//     item load(int64 i, bool& keep) const;           reads element i and decides
+//     void store(const item&, int64 position) const;  writes a kept element
+// A tile loads its elements (all loads of a thread in flight together: load() must not branch on
+// what it reads), ranks the kept ones inside the tile (wave ballots + a table of (row, wave)
+// counts in LDS, scanned by wave 0), learns how many elements the tiles before it kept from a
+// chain of tile descriptors (decoupled look-back, 64 descriptors per round, one per lane of
+// wave 0) and stores from registers.  copy_if, remove_if, unique and unique_by_key are such
+// operations.  Traffic: the inputs once, the kept outputs once.
+//
+// A descriptor is one 64-bit word, status in bits 63:62 (0 empty, 1 the tile's own count,
+// 2 the count of all tiles up to and including it) and the count below, written and read with
+// relaxed agent-scope atomics: the value travels inside the word, so no fence is needed.
+// Tiles take their index from a ticket counter, so every tile a waiting tile looks back at has
+// started already and the wait ends.  One same-address atomic costs about 12 ns of the whole
+// device's time, which is why a tile is 128 KiB of items.
+// ---------------------------------------------------------------------------------------
+constexpr int kSelBlock = 1024;
+constexpr int kSelWaves = kSelBlock / 64;
+constexpr unsigned long long kSelValueMask = (1ull << 62) - 1ull;
+// rows of kSelBlock items per tile: 128 bytes of items per thread, 4 to 32 rows
+constexpr int select_rows(std::size_t item_bytes) {
+  return item_bytes <= 4 ? 32 : item_bytes <= 8 ? 16 : item_bytes <= 16 ? 8 : 4;
+}
+// Register budget: 32 rows of 4-byte items need about 72 registers (one workgroup per CU);
+// 8- to 32-byte items fit 64 registers, and the second workgroup per CU is worth 12 %.
+constexpr int select_waves_per_simd(std::size_t item_bytes) { return item_bytes > 4 && item_bytes <= 32 ? 8 : 4; }
+
+// words[0, tiles) are the descriptors, words[tiles] the ticket counter, words[tiles + 1] the result
+template <class Word>
+__global__ __launch_bounds__(256) void select_init_kernel(Word* words, std::int64_t count) {
+  const std::int64_t i = (std::int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < count) words[i] = Word(0);
+}
+
+template <class Op>
+__global__ __launch_bounds__(kSelBlock)
+__attribute__((amdgpu_waves_per_eu(select_waves_per_simd(sizeof(typename Op::item)), select_waves_per_simd(sizeof(typename Op::item)))))
+void select_kernel(std::int64_t n, Op op, unsigned long long* words, std::int64_t tiles) {
+  typedef typename Op::item Item;
+  constexpr int ROWS = select_rows(sizeof(Item));
+  constexpr int TILE = kSelBlock * ROWS;
+  constexpr int CELLS = ROWS * kSelWaves;  // (row, wave) counts
+  constexpr int PER_LANE = CELLS / 64;     // cells each lane of wave 0 scans
+  __shared__ unsigned s_cnt[CELLS];        // kept in (row, wave), then its exclusive prefix in the tile
+  __shared__ unsigned long long s_tile, s_prefix;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x / 64;
+  if (threadIdx.x == 0)
+    s_tile = __hip_atomic_fetch_add(&words[tiles], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const std::int64_t tile = (std::int64_t)s_tile;
+  const std::int64_t base = tile * TILE + threadIdx.x;
+  Item items[ROWS];
+  unsigned mine = 0;  // bit j: row j's element is kept
+  if ((tile + 1) * TILE <= n) {
+#pragma unroll
+    for (int j = 0; j < ROWS; j++) {
+      bool keep;
+      items[j] = op.load(base + (std::int64_t)j * kSelBlock, keep);
+      mine |= (keep ? 1u : 0u) << j;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < ROWS; j++) {
+      const std::int64_t i = base + (std::int64_t)j * kSelBlock;
+      if (i < n) {
+        bool keep;
+        items[j] = op.load(i, keep);
+        mine |= (keep ? 1u : 0u) << j;
+      }
+    }
+  }
+  unsigned below[ROWS / 4];  // kept lanes below this one in row j, a byte each
+#pragma unroll
+  for (int j = 0; j < ROWS; j++) {
+    const unsigned long long m = __builtin_amdgcn_ballot_w64((mine >> j) & 1u);
+    const unsigned b = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
+    below[j / 4] = (j % 4 == 0) ? b : (below[j / 4] | (b << (8 * (j % 4))));
+    if (lane == 0) s_cnt[j * kSelWaves + wave] = (unsigned)__builtin_popcountll(m);
+  }
+  __syncthreads();
+  if (wave == 0) {
+    unsigned c[PER_LANE], sum = 0;
+#pragma unroll
+    for (int q = 0; q < PER_LANE; q++) {
+      c[q] = s_cnt[lane * PER_LANE + q];
+      sum += c[q];
+    }
+    unsigned inc = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const unsigned up = __shfl_up(inc, d, 64);
+      if (lane >= d) inc += up;
+    }
+    unsigned run = inc - sum;
+#pragma unroll
+    for (int q = 0; q < PER_LANE; q++) {
+      s_cnt[lane * PER_LANE + q] = run;
+      run += c[q];
+    }
+    const unsigned long long total = (unsigned long long)__shfl(inc, 63, 64);
+    unsigned long long prefix = 0;  // kept by all tiles before this one
+    if (tile > 0) {
+      if (lane == 0) __hip_atomic_store(&words[tile], (1ull << 62) | total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      std::int64_t nearest = tile - 1;
+      for (;;) {
+        const std::int64_t t = nearest - lane;  // lane 0 looks at the nearest tile before this one
+        const unsigned long long w =
+            t >= 0 ? __hip_atomic_load(&words[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : (2ull << 62);
+        const unsigned status = (unsigned)(w >> 62);
+        const unsigned long long full = __builtin_amdgcn_ballot_w64(status == 2u);
+        const unsigned long long empty = __builtin_amdgcn_ballot_w64(status == 0u);
+        // lanes up to and including the nearest complete descriptor contribute
+        const unsigned long long use = full ? ((full & (0ull - full)) << 1) - 1ull : ~0ull;
+        if (empty & use) {
+          __builtin_amdgcn_s_sleep(1);
+          continue;
+        }
+        unsigned long long v = ((use >> lane) & 1ull) ? (w & kSelValueMask) : 0ull;
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d, 64);
+        prefix += v;
+        if (full) break;
+        nearest -= 64;
+      }
+    }
+    if (lane == 0) {
+      __hip_atomic_store(&words[tile], (2ull << 62) | (prefix + total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_prefix = prefix;
+      if (tile == tiles - 1) words[tiles + 1] = prefix + total;
+    }
+  }
+  __syncthreads();
+  const std::int64_t tile_off = (std::int64_t)s_prefix;
+#pragma unroll
+  for (int j = 0; j < ROWS; j++) {
+    if ((mine >> j) & 1u)
+      op.store(items[j], tile_off + s_cnt[j * kSelWaves + wave] + ((below[j / 4] >> (8 * (j % 4))) & 0xffu));
+  }
+}
+
+// Returns the number of kept elements; blocks until it is known (the callers return an end
+// iterator that depends on it, as the reference's do).
+template <class Op>
+std::int64_t select(void* stream_, std::int64_t n, Op op) {
+  if (n <= 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream_);
+  constexpr std::int64_t kTile = (std::int64_t)kSelBlock * select_rows(sizeof(typename Op::item));
+  const std::int64_t tiles = (n + kTile - 1) / kTile;
+  temporary_storage tmp((std::size_t)(tiles + 2) * sizeof(unsigned long long), stream_);
+  unsigned long long* words = static_cast<unsigned long long*>(tmp.data());
+  hipLaunchKernelGGL((select_init_kernel<unsigned long long>), dim3((unsigned)((tiles + 2 + 255) / 256)), dim3(256), 0, s, words, tiles + 2);
+  hipLaunchKernelGGL((select_kernel<Op>), dim3((unsigned)tiles), dim3(kSelBlock), 0, s, n, op, words, tiles);
+  throw_on_error((int)hipGetLastError(), "select: launch");
+  unsigned long long kept = 0;
+  throw_on_error(thrust_cdna4_memcpy_dtoh(&kept, words + tiles + 1, sizeof(kept), stream_), "select: read back");
+  throw_on_error(thrust_cdna4_stream_synchronize(stream_), "select: failed to synchronize");
+  return (std::int64_t)kept;
 }
 
 }}}}}  // namespace thrust::system::cdna4::detail::generic

@@ -1,0 +1,106 @@
+// thrust::unique / unique_copy / unique_by_key / unique_by_key_copy (thrust/unique.h;
+// thrust/system/cuda/detail/unique.h, unique_by_key.h): the first element of every run of
+// consecutive equal elements, in order; the in-place forms compact from a temporary copy.
+#pragma once
+#include <algorithm>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/pair.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
+namespace thrust {
+// ---- device
+template <class D, class In, class Out, class Eq>
+Out unique_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Eq eq) {
+  typedef typename detail::value_of<In>::type V;
+  return out + system::cdna4::detail::unique_copy_n(exec.derived(), (const V*)detail::unwrap(first), detail::unwrap(out),
+                                                    (std::int64_t)(last - first), eq);
+}
+template <class D, class In, class Eq>
+In unique(const system::cdna4::execution_policy<D>& exec, In first, In last, Eq eq) {
+  typedef typename detail::value_of<In>::type V;
+  const std::int64_t n = (std::int64_t)(last - first);
+  system::cdna4::detail::scratch_copy<V> tmp((const V*)detail::unwrap(first), n, system::cdna4::detail::stream_of(exec.derived()));
+  return first + system::cdna4::detail::unique_copy_n(exec.derived(), tmp.data(), detail::unwrap(first), n, eq);
+}
+template <class D, class KIn, class VIn, class KOut, class VOut, class Eq>
+pair<KOut, VOut> unique_by_key_copy(const system::cdna4::execution_policy<D>& exec, KIn kfirst, KIn klast, VIn vfirst,
+                                    KOut kout, VOut vout, Eq eq) {
+  typedef typename detail::value_of<KIn>::type K;
+  typedef typename detail::value_of<VIn>::type V;
+  const std::int64_t c = system::cdna4::detail::unique_by_key_copy_n(
+      exec.derived(), (const K*)detail::unwrap(kfirst), (const V*)detail::unwrap(vfirst), detail::unwrap(kout),
+      detail::unwrap(vout), (std::int64_t)(klast - kfirst), eq);
+  return thrust::make_pair(kout + c, vout + c);
+}
+template <class D, class KIn, class VIn, class Eq>
+pair<KIn, VIn> unique_by_key(const system::cdna4::execution_policy<D>& exec, KIn kfirst, KIn klast, VIn vfirst, Eq eq) {
+  typedef typename detail::value_of<KIn>::type K;
+  typedef typename detail::value_of<VIn>::type V;
+  const std::int64_t n = (std::int64_t)(klast - kfirst);
+  void* s = system::cdna4::detail::stream_of(exec.derived());
+  system::cdna4::detail::scratch_copy<K> tk((const K*)detail::unwrap(kfirst), n, s);
+  system::cdna4::detail::scratch_copy<V> tv((const V*)detail::unwrap(vfirst), n, s);
+  const std::int64_t c = system::cdna4::detail::unique_by_key_copy_n(exec.derived(), tk.data(), tv.data(), detail::unwrap(kfirst),
+                                                                     detail::unwrap(vfirst), n, eq);
+  return thrust::make_pair(kfirst + c, vfirst + c);
+}
+// ---- host
+template <class In, class Out, class Eq>
+Out unique_copy(const system::cpp::detail::par_t&, In first, In last, Out out, Eq eq) { return std::unique_copy(first, last, out, eq); }
+template <class In, class Eq>
+In unique(const system::cpp::detail::par_t&, In first, In last, Eq eq) { return std::unique(first, last, eq); }
+template <class KIn, class VIn, class KOut, class VOut, class Eq>
+pair<KOut, VOut> unique_by_key_copy(const system::cpp::detail::par_t&, KIn kfirst, KIn klast, VIn vfirst, KOut kout, VOut vout, Eq eq) {
+  if (kfirst == klast) return thrust::make_pair(kout, vout);
+  auto prev = *kfirst;
+  *kout = prev; *vout = *vfirst; ++kout; ++vout;
+  for (++kfirst, ++vfirst; kfirst != klast; ++kfirst, ++vfirst) {
+    if (!eq(prev, *kfirst)) { *kout = *kfirst; *vout = *vfirst; ++kout; ++vout; }
+    prev = *kfirst;
+  }
+  return thrust::make_pair(kout, vout);
+}
+template <class KIn, class VIn, class Eq>
+pair<KIn, VIn> unique_by_key(const system::cpp::detail::par_t& e, KIn kfirst, KIn klast, VIn vfirst, Eq eq) {
+  return unique_by_key_copy(e, kfirst, klast, vfirst, kfirst, vfirst, eq);  // outputs trail the inputs
+}
+// ---- default equality, any policy
+template <class Policy, class In, class Out, class = typename std::iterator_traits<In>::iterator_category,
+          class = typename std::iterator_traits<Out>::iterator_category>
+Out unique_copy(const Policy& exec, In first, In last, Out out) { return unique_copy(exec, first, last, out, equal_to<typename detail::value_of<In>::type>()); }
+template <class Policy, class In, class = typename std::iterator_traits<In>::iterator_category>
+In unique(const Policy& exec, In first, In last) { return unique(exec, first, last, equal_to<typename detail::value_of<In>::type>()); }
+template <class Policy, class KIn, class VIn, class = typename std::iterator_traits<VIn>::iterator_category>
+pair<KIn, VIn> unique_by_key(const Policy& exec, KIn kfirst, KIn klast, VIn vfirst) {
+  return unique_by_key(exec, kfirst, klast, vfirst, equal_to<typename detail::value_of<KIn>::type>());
+}
+template <class Policy, class KIn, class VIn, class KOut, class VOut, class = typename std::iterator_traits<VOut>::iterator_category>
+pair<KOut, VOut> unique_by_key_copy(const Policy& exec, KIn kfirst, KIn klast, VIn vfirst, KOut kout, VOut vout) {
+  return unique_by_key_copy(exec, kfirst, klast, vfirst, kout, vout, equal_to<typename detail::value_of<KIn>::type>());
+}
+// ---- no policy
+template <class In, detail::enable_if_device<In> = 0> In unique(In f, In l) { return unique(device, f, l); }
+template <class In, detail::enable_if_host<In> = 0> In unique(In f, In l) { return unique(host, f, l); }
+template <class In, class Eq, detail::enable_if_device<In> = 0> In unique(In f, In l, Eq eq) { return unique(device, f, l, eq); }
+template <class In, class Eq, detail::enable_if_host<In> = 0> In unique(In f, In l, Eq eq) { return unique(host, f, l, eq); }
+template <class In, class Out, detail::enable_if_device<In> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(device, f, l, o); }
+template <class In, class Out, detail::enable_if_host<In> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(host, f, l, o); }
+template <class K, class V, detail::enable_if_device<K> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(device, f, l, v); }
+template <class K, class V, detail::enable_if_host<K> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(host, f, l, v); }
+template <class In, class Out, class Eq, detail::enable_if_device<In> = 0, class = typename std::iterator_traits<Out>::iterator_category>
+Out unique_copy(In f, In l, Out o, Eq eq) { return unique_copy(device, f, l, o, eq); }
+template <class In, class Out, class Eq, detail::enable_if_host<In> = 0, class = typename std::iterator_traits<Out>::iterator_category>
+Out unique_copy(In f, In l, Out o, Eq eq) { return unique_copy(host, f, l, o, eq); }
+template <class K, class V, class Eq, detail::enable_if_device<K> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(device, f, l, v, eq); }
+template <class K, class V, class Eq, detail::enable_if_host<K> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(host, f, l, v, eq); }
+template <class K, class V, class KO, class VO, class Eq, detail::enable_if_device<K> = 0>
+pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo, Eq eq) { return unique_by_key_copy(device, f, l, v, ko, vo, eq); }
+template <class K, class V, class KO, class VO, class Eq, detail::enable_if_host<K> = 0>
+pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo, Eq eq) { return unique_by_key_copy(host, f, l, v, ko, vo, eq); }
+template <class K, class V, class KO, class VO, detail::enable_if_device<K> = 0>
+pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(device, f, l, v, ko, vo); }
+template <class K, class V, class KO, class VO, detail::enable_if_host<K> = 0>
+pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(host, f, l, v, ko, vo); }
+}  // namespace thrust

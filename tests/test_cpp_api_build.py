@@ -20,7 +20,7 @@ def compile_snippet(tmp_path, body, extra=()):
 def test_cpp_tests_compile():
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    for name in ["test_sort", "test_scan", "test_by_key", "test_system", "test_merge_sort", "bench_merge_sort", "test_generic",
+    for name in ["test_sort", "test_scan", "test_by_key", "test_system", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select",
                  "bench_generic"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
 
@@ -119,4 +119,42 @@ def test_host_ranges_with_functors_build_with_gxx(tmp_path):
         int main() { thrust::host_vector<int> h(10), o(10); thrust::sequence(h.begin(), h.end());
                      thrust::transform(h.begin(), h.end(), o.begin(), thrust::negate<int>());
                      return thrust::reduce(o.begin(), o.end()) + (int)thrust::count(o.begin(), o.end(), -3); }""")
+    assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_select_family_on_device_range_needs_hipcc(tmp_path):
+    body = """
+        #include <thrust/device_vector.h>
+        #include <thrust/copy.h>
+        #include <thrust/remove.h>
+        #include <thrust/unique.h>
+        struct odd { THRUST_CDNA4_HD bool operator()(int x) const { return x & 1; } };
+        int main() { thrust::device_vector<int> d(10), o(10), v(10);
+                     auto e = thrust::copy_if(d.begin(), d.end(), o.begin(), odd());
+                     auto r = thrust::remove_if(d.begin(), d.end(), odd());
+                     auto u = thrust::unique(d.begin(), d.end());
+                     auto p = thrust::unique_by_key(d.begin(), d.end(), v.begin());
+                     return (int)((e - o.begin()) + (r - d.begin()) + (u - d.begin()) + (p.first - d.begin())); }"""
+    r = compile_snippet(tmp_path, body)
+    assert r.returncode != 0
+    assert "compile this translation unit with hipcc" in r.stderr
+    src = tmp_path / "t.cpp"
+    r = subprocess.run(["/opt/rocm/bin/hipcc", "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-fsyntax-only",
+                        "-I", INC, str(src)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_select_family_on_host_ranges_builds_with_gxx(tmp_path):
+    r = compile_snippet(tmp_path, """
+        #include <thrust/host_vector.h>
+        #include <thrust/copy.h>
+        #include <thrust/remove.h>
+        #include <thrust/unique.h>
+        struct odd { bool operator()(int x) const { return x & 1; } };
+        int main() { thrust::host_vector<int> h(10), o(10), v(10);
+                     auto e = thrust::copy_if(h.begin(), h.end(), o.begin(), odd());
+                     auto r = thrust::remove(h.begin(), h.end(), 3);
+                     auto u = thrust::unique(h.begin(), h.end());
+                     auto p = thrust::unique_by_key(h.begin(), h.end(), v.begin());
+                     return (int)((e - o.begin()) + (r - h.begin()) + (u - h.begin()) + (p.first - h.begin())); }""")
     assert r.returncode == 0, r.stderr[-3000:]
