@@ -2,6 +2,7 @@
 // classify an iterator as device or host.
 #pragma once
 #include <iterator>
+#include <type_traits>
 #include <thrust/device_ptr.h>
 namespace thrust { namespace detail {
 template <class T> inline T* unwrap(thrust::device_ptr<T> p) { return p.get(); }
@@ -9,4 +10,9 @@ template <class T> inline T* unwrap(T* p) { return p; }  // raw device pointer u
 template <class It> struct value_of { typedef typename std::iterator_traits<It>::value_type type; };
 template <class It> using enable_if_device = typename std::enable_if<system::cdna4::detail::is_device_iterator<It>::value, int>::type;
 template <class It> using enable_if_host = typename std::enable_if<!system::cdna4::detail::is_device_iterator<It>::value, int>::type;
+// an execution policy of either system (tells policy-first overloads from iterator-first ones)
+template <class P> struct is_policy {
+  static constexpr bool value = std::is_base_of<system::cdna4::execution_policy<P>, P>::value || std::is_same<P, system::cpp::detail::par_t>::value;
+};
+template <class P> using enable_if_policy = typename std::enable_if<is_policy<P>::value, int>::type;
 }}  // namespace thrust::detail

@@ -1,0 +1,122 @@
+// thrust::partition / stable_partition / partition_copy / stable_partition_copy, with and
+// without a stencil (thrust/partition.h; thrust/system/cuda/detail/partition.h:138-606).
+// All four are stable here: one pass of the select kernel writes the elements the predicate
+// accepts and the ones it rejects, each in input order.  The in-place forms read a temporary
+// copy and collect the rejected elements in a second temporary before appending them.
+#pragma once
+#include <algorithm>
+#include <vector>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/pair.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
+namespace thrust {
+// ---- device
+template <class D, class In, class St, class OutT, class OutF, class Pred>
+pair<OutT, OutF> stable_partition_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, St stencil,
+                                       OutT out_true, OutF out_false, Pred pred) {
+  typedef typename detail::value_of<In>::type V;
+  typedef typename detail::value_of<St>::type S;
+  const std::int64_t n = (std::int64_t)(last - first);
+  const std::int64_t c = system::cdna4::detail::partition_copy_n(exec.derived(), (const V*)detail::unwrap(first), (const S*)detail::unwrap(stencil),
+                                                                 detail::unwrap(out_true), detail::unwrap(out_false), n, pred);
+  return thrust::make_pair(out_true + c, out_false + (n - c));
+}
+template <class D, class In, class OutT, class OutF, class Pred, class = typename std::iterator_traits<OutF>::iterator_category>
+pair<OutT, OutF> stable_partition_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, OutT out_true, OutF out_false, Pred pred) {
+  return stable_partition_copy(exec, first, last, first, out_true, out_false, pred);
+}
+template <class D, class It, class St, class Pred, class = typename std::iterator_traits<St>::iterator_category>
+It stable_partition(const system::cdna4::execution_policy<D>& exec, It first, It last, St stencil, Pred pred) {
+  namespace sd = system::cdna4::detail;
+  typedef typename detail::value_of<It>::type V;
+  typedef typename detail::value_of<St>::type S;
+  const std::int64_t n = (std::int64_t)(last - first);
+  if (n <= 0) return first;
+  void* s = sd::stream_of(exec.derived());
+  V* data = (V*)detail::unwrap(first);
+  sd::scratch_copy<V> in(data, n, s);
+  sd::temporary_storage rejected((std::size_t)n * sizeof(V), s);
+  const S* st = (const void*)detail::unwrap(stencil) == (const void*)data ? (const S*)in.data() : (const S*)detail::unwrap(stencil);
+  const std::int64_t c = sd::partition_copy_n(exec.derived(), in.data(), st, data, static_cast<V*>(rejected.data()), n, pred);
+  if (c < n) {
+    sd::throw_on_error(thrust_cdna4_memcpy_dtod(data + c, rejected.data(), (std::size_t)(n - c) * sizeof(V), s), "partition: append");
+    sd::throw_on_error(thrust_cdna4_stream_synchronize(s), "partition: failed to synchronize");
+  }
+  return first + c;
+}
+template <class D, class It, class Pred>
+It stable_partition(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) {
+  return stable_partition(exec, first, last, first, pred);
+}
+// ---- host
+template <class In, class St, class OutT, class OutF, class Pred>
+pair<OutT, OutF> stable_partition_copy(const system::cpp::detail::par_t&, In first, In last, St stencil, OutT out_true, OutF out_false, Pred pred) {
+  for (; first != last; ++first, ++stencil) {
+    if (pred(*stencil)) { *out_true = *first; ++out_true; }
+    else { *out_false = *first; ++out_false; }
+  }
+  return thrust::make_pair(out_true, out_false);
+}
+template <class In, class OutT, class OutF, class Pred, class = typename std::iterator_traits<OutF>::iterator_category>
+pair<OutT, OutF> stable_partition_copy(const system::cpp::detail::par_t& e, In first, In last, OutT out_true, OutF out_false, Pred pred) {
+  return stable_partition_copy(e, first, last, first, out_true, out_false, pred);
+}
+template <class It, class St, class Pred, class = typename std::iterator_traits<St>::iterator_category>
+It stable_partition(const system::cpp::detail::par_t& e, It first, It last, St stencil, Pred pred) {
+  typedef typename std::iterator_traits<It>::value_type V;
+  std::vector<V> yes(last - first), no(last - first);
+  auto ends = stable_partition_copy(e, first, last, stencil, yes.begin(), no.begin(), pred);
+  It mid = std::copy(yes.begin(), ends.first, first);
+  std::copy(no.begin(), ends.second, mid);
+  return mid;
+}
+template <class It, class Pred>
+It stable_partition(const system::cpp::detail::par_t&, It first, It last, Pred pred) { return std::stable_partition(first, last, pred); }
+
+// ---- partition and partition_copy are the stable forms, any policy
+template <class Policy, class It, class Pred, detail::enable_if_policy<Policy> = 0>
+It partition(const Policy& exec, It first, It last, Pred pred) { return stable_partition(exec, first, last, pred); }
+template <class Policy, class It, class St, class Pred, detail::enable_if_policy<Policy> = 0,
+          class = typename std::iterator_traits<St>::iterator_category>
+It partition(const Policy& exec, It first, It last, St stencil, Pred pred) { return stable_partition(exec, first, last, stencil, pred); }
+template <class Policy, class In, class OutT, class OutF, class Pred, detail::enable_if_policy<Policy> = 0,
+          class = typename std::iterator_traits<OutF>::iterator_category>
+pair<OutT, OutF> partition_copy(const Policy& exec, In first, In last, OutT out_true, OutF out_false, Pred pred) {
+  return stable_partition_copy(exec, first, last, out_true, out_false, pred);
+}
+template <class Policy, class In, class St, class OutT, class OutF, class Pred, detail::enable_if_policy<Policy> = 0>
+pair<OutT, OutF> partition_copy(const Policy& exec, In first, In last, St stencil, OutT out_true, OutF out_false, Pred pred) {
+  return stable_partition_copy(exec, first, last, stencil, out_true, out_false, pred);
+}
+// ---- no policy
+#define THRUST_CDNA4_PARTITION_NO_POLICY(NAME)                                                                          \
+  template <class It, class Pred, detail::enable_if_device<It> = 0>                                                     \
+  It NAME(It f, It l, Pred p) { return NAME(device, f, l, p); }                                                         \
+  template <class It, class Pred, detail::enable_if_host<It> = 0>                                                       \
+  It NAME(It f, It l, Pred p) { return NAME(host, f, l, p); }                                                           \
+  template <class It, class St, class Pred, detail::enable_if_device<It> = 0,                                           \
+            class = typename std::iterator_traits<St>::iterator_category>                                               \
+  It NAME(It f, It l, St s, Pred p) { return NAME(device, f, l, s, p); }                                                \
+  template <class It, class St, class Pred, detail::enable_if_host<It> = 0,                                             \
+            class = typename std::iterator_traits<St>::iterator_category>                                               \
+  It NAME(It f, It l, St s, Pred p) { return NAME(host, f, l, s, p); }
+THRUST_CDNA4_PARTITION_NO_POLICY(partition)
+THRUST_CDNA4_PARTITION_NO_POLICY(stable_partition)
+#undef THRUST_CDNA4_PARTITION_NO_POLICY
+#define THRUST_CDNA4_PARTITION_COPY_NO_POLICY(NAME)                                                                     \
+  template <class In, class OutT, class OutF, class Pred, detail::enable_if_device<In> = 0>                             \
+  pair<OutT, OutF> NAME(In f, In l, OutT t, OutF o, Pred p) { return NAME(device, f, l, t, o, p); }                     \
+  template <class In, class OutT, class OutF, class Pred, detail::enable_if_host<In> = 0>                               \
+  pair<OutT, OutF> NAME(In f, In l, OutT t, OutF o, Pred p) { return NAME(host, f, l, t, o, p); }                       \
+  template <class In, class St, class OutT, class OutF, class Pred, detail::enable_if_device<In> = 0,                   \
+            class = typename std::iterator_traits<OutF>::iterator_category>                                             \
+  pair<OutT, OutF> NAME(In f, In l, St s, OutT t, OutF o, Pred p) { return NAME(device, f, l, s, t, o, p); }            \
+  template <class In, class St, class OutT, class OutF, class Pred, detail::enable_if_host<In> = 0,                     \
+            class = typename std::iterator_traits<OutF>::iterator_category>                                             \
+  pair<OutT, OutF> NAME(In f, In l, St s, OutT t, OutF o, Pred p) { return NAME(host, f, l, s, t, o, p); }
+THRUST_CDNA4_PARTITION_COPY_NO_POLICY(partition_copy)
+THRUST_CDNA4_PARTITION_COPY_NO_POLICY(stable_partition_copy)
+#undef THRUST_CDNA4_PARTITION_COPY_NO_POLICY
+}  // namespace thrust

@@ -101,6 +101,7 @@ T transform_reduce_n(const Policy& exec, const In* in, std::int64_t n, F f, T in
 // keep in[i] when pred(in[i]) != NEGATE
 template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
   typedef In item;
+  static constexpr bool rejects = false;
   const In* in; Out* out; Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     const In x = in[i];
@@ -112,6 +113,7 @@ template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
 // keep in[i] when pred(stencil[i]) != NEGATE
 template <class In, class S, class Out, class Pred, bool NEGATE> struct keep_if_stencil_op {
   typedef In item;
+  static constexpr bool rejects = false;
   const In* in; const S* stencil; Out* out; Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     keep = (bool)pred(stencil[i]) != NEGATE;
@@ -119,9 +121,22 @@ template <class In, class S, class Out, class Pred, bool NEGATE> struct keep_if_
   }
   __device__ void store(const item& x, std::int64_t pos) const { out[pos] = x; }
 };
+// in[i] goes to out_true when pred(stencil[i]), else to out_false, both in order
+template <class In, class S, class OutT, class OutF, class Pred> struct partition_op {
+  typedef In item;
+  static constexpr bool rejects = true;
+  const In* in; const S* stencil; OutT* out_true; OutF* out_false; Pred pred;
+  __device__ item load(std::int64_t i, bool& keep) const {
+    keep = (bool)pred(stencil[i]);
+    return in[i];
+  }
+  __device__ void store(const item& x, std::int64_t pos) const { out_true[pos] = x; }
+  __device__ void store_rejected(const item& x, std::int64_t pos) const { out_false[pos] = x; }
+};
 // keep the first element of every run; element 0 compares with itself and is kept by index
 template <class K, class KOut, class Eq> struct run_head_op {
   typedef K item;
+  static constexpr bool rejects = false;
   const K* keys; KOut* out; Eq eq;
   __device__ item load(std::int64_t i, bool& keep) const {
     const K cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
@@ -132,6 +147,7 @@ template <class K, class KOut, class Eq> struct run_head_op {
 };
 template <class K, class V, class KOut, class VOut, class Eq> struct run_head_by_key_op {
   struct item { K key; V value; };
+  static constexpr bool rejects = false;
   const K* keys; const V* values; KOut* kout; VOut* vout; Eq eq;
   __device__ item load(std::int64_t i, bool& keep) const {
     const K cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
@@ -161,6 +177,17 @@ std::int64_t copy_flagged_n(const Policy& exec, const In* in, const S* stencil, 
   return generic::select(stream_of(exec), n, keep_if_stencil_op<In, S, Out, Pred, NEGATE>{in, stencil, out, pred});
 #else
   (void)exec; (void)in; (void)stencil; (void)out; (void)n; (void)pred;
+  return 0;
+#endif
+}
+// stable two-way split by pred(stencil[i]); returns the number that went to out_true
+template <class Policy, class In, class S, class OutT, class OutF, class Pred>
+std::int64_t partition_copy_n(const Policy& exec, const In* in, const S* stencil, OutT* out_true, OutF* out_false, std::int64_t n, Pred pred) {
+  THRUST_CDNA4_NEEDS_HIPCC(Pred);
+#if defined(__HIPCC__)
+  return generic::select(stream_of(exec), n, partition_op<In, S, OutT, OutF, Pred>{in, stencil, out_true, out_false, pred});
+#else
+  (void)exec; (void)in; (void)stencil; (void)out_true; (void)out_false; (void)n; (void)pred;
   return 0;
 #endif
 }

@@ -125,6 +125,8 @@ T transform_reduce(void* stream_, std::int64_t n, Unary unary, T init, Op op) {
 //     typedef ... item;                               what travels from the load to the store
 //     item load(int64 i, bool& keep) const;           reads element i and decides
 //     void store(const item&, int64 position) const;  writes a kept element
+//     static const bool rejects;                      true: the others go to store_rejected(item,
+//                                                     position among the rejected) — partition
 // A tile loads its elements (all loads of a thread in flight together: load() must not branch on
 // what it reads), ranks the kept ones inside the tile (wave ballots + a table of (row, wave)
 // counts in LDS, scanned by wave 0), learns how many elements the tiles before it kept from a
@@ -258,8 +260,13 @@ void select_kernel(std::int64_t n, Op op, unsigned long long* words, std::int64_
   const std::int64_t tile_off = (std::int64_t)s_prefix;
 #pragma unroll
   for (int j = 0; j < ROWS; j++) {
+    // kept elements before this one in the whole input
+    const std::int64_t before = tile_off + s_cnt[j * kSelWaves + wave] + ((below[j / 4] >> (8 * (j % 4))) & 0xffu);
+    const std::int64_t i = base + (std::int64_t)j * kSelBlock;
     if ((mine >> j) & 1u)
-      op.store(items[j], tile_off + s_cnt[j * kSelWaves + wave] + ((below[j / 4] >> (8 * (j % 4))) & 0xffu));
+      op.store(items[j], before);
+    else if (Op::rejects && i < n)
+      op.store_rejected(items[j], i - before);  // rejected elements before this one
   }
 }
 
