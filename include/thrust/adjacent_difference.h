@@ -1,0 +1,49 @@
+// thrust::adjacent_difference (thrust/adjacent_difference.h;
+// thrust/system/cuda/detail/adjacent_difference.h): out[0] = in[0], out[i] = op(in[i], in[i-1]).
+// The output may be the input range itself: the input is then read from a temporary copy.
+#pragma once
+#include <numeric>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
+namespace thrust {
+namespace detail {
+template <class A, class B> inline bool same_address(A, B) { return false; }
+template <class T, class U> inline bool same_address(T* a, U* b) { return (const void*)a == (const void*)b; }
+}  // namespace detail
+template <class D, class In, class Out, class Op>
+Out adjacent_difference(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Op op) {
+  namespace sd = system::cdna4::detail;
+  typedef typename detail::value_of<In>::type V;
+  const std::int64_t n = (std::int64_t)(last - first);
+  if (n <= 0) return out;
+  auto in = detail::unwrap(first);
+  auto o = detail::unwrap(out);
+  if (detail::same_address(in, o)) {
+    sd::scratch_copy<V> tmp((const V*)(const void*)sd::address_of(in), n, sd::stream_of(exec.derived()));
+    sd::adjacent_difference_n(exec.derived(), tmp.data(), o, n, op);
+    // the temporary goes back to the pool in stream order, after the kernel that reads it
+  } else {
+    sd::adjacent_difference_n(exec.derived(), in, o, n, op);
+  }
+  return out + n;
+}
+template <class In, class Out, class Op>
+Out adjacent_difference(const system::cpp::detail::par_t&, In first, In last, Out out, Op op) {
+  return std::adjacent_difference(first, last, out, op);
+}
+template <class Policy, class In, class Out, detail::enable_if_policy<Policy> = 0>
+Out adjacent_difference(const Policy& exec, In first, In last, Out out) {
+  return adjacent_difference(exec, first, last, out, minus<typename detail::value_of<In>::type>());
+}
+template <class In, class Out, detail::enable_if_device<In> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(device, f, l, o); }
+template <class In, class Out, detail::enable_if_host<In> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(host, f, l, o); }
+template <class In, class Out, class Op, detail::enable_if_device<In> = 0,
+          class = typename std::iterator_traits<Out>::iterator_category>
+Out adjacent_difference(In f, In l, Out o, Op op) { return adjacent_difference(device, f, l, o, op); }
+template <class In, class Out, class Op, detail::enable_if_host<In> = 0,
+          class = typename std::iterator_traits<Out>::iterator_category>
+Out adjacent_difference(In f, In l, Out o, Op op) { return adjacent_difference(host, f, l, o, op); }
+}  // namespace thrust

@@ -1,0 +1,97 @@
+// thrust::lower_bound / upper_bound / binary_search (thrust/binary_search.h;
+// thrust/system/detail/generic/binary_search.inl): the vectorised forms run one search per
+// thread over the sorted range; the scalar forms are a one-element vectorised search.
+#pragma once
+#include <algorithm>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/device_vector.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
+namespace thrust {
+namespace detail {
+template <int MODE, class D, class Hay, class Needles, class Out, class Comp>
+Out vector_search(const system::cdna4::execution_policy<D>& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out, Comp comp) {
+  const std::int64_t n = (std::int64_t)(vlast - vfirst);
+  system::cdna4::detail::binary_search_n<MODE>(exec.derived(), unwrap(first), (std::int64_t)(last - first), unwrap(vfirst), unwrap(out), n, comp);
+  return out + n;
+}
+template <int MODE, class Hay, class Needles, class Out, class Comp>
+Out vector_search(const system::cpp::detail::par_t&, Hay first, Hay last, Needles vfirst, Needles vlast, Out out, Comp comp) {
+  for (; vfirst != vlast; ++vfirst, ++out) {
+    if (MODE == 0) *out = std::lower_bound(first, last, *vfirst, comp) - first;
+    else if (MODE == 1) *out = std::upper_bound(first, last, *vfirst, comp) - first;
+    else *out = std::binary_search(first, last, *vfirst, comp);
+  }
+  return out;
+}
+// one value: search from a one-element device vector, read the answer back
+template <int MODE, class D, class Hay, class T, class Comp>
+std::ptrdiff_t scalar_search(const system::cdna4::execution_policy<D>& exec, Hay first, Hay last, const T& value, Comp comp) {
+  thrust::device_vector<T> needle(1, value);
+  thrust::device_vector<std::ptrdiff_t> answer(1);
+  vector_search<MODE>(exec, first, last, needle.begin(), needle.end(), answer.begin(), comp);
+  system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(system::cdna4::detail::stream_of(exec.derived())), "binary search");
+  return answer[0];
+}
+template <int MODE, class Hay, class T, class Comp>
+std::ptrdiff_t scalar_search(const system::cpp::detail::par_t&, Hay first, Hay last, const T& value, Comp comp) {
+  if (MODE == 0) return std::lower_bound(first, last, value, comp) - first;
+  if (MODE == 1) return std::upper_bound(first, last, value, comp) - first;
+  return std::binary_search(first, last, value, comp);
+}
+}  // namespace detail
+
+#define THRUST_CDNA4_SEARCH(NAME, MODE)                                                                                  \
+  template <class Policy, class Hay, class Needles, class Out, class Comp, detail::enable_if_policy<Policy> = 0>         \
+  Out NAME(const Policy& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out, Comp comp) {                 \
+    return detail::vector_search<MODE>(exec, first, last, vfirst, vlast, out, comp);                                     \
+  }                                                                                                                      \
+  template <class Policy, class Hay, class Needles, class Out, detail::enable_if_policy<Policy> = 0>                     \
+  Out NAME(const Policy& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out) {                            \
+    return detail::vector_search<MODE>(exec, first, last, vfirst, vlast, out, less<typename detail::value_of<Hay>::type>()); \
+  }                                                                                                                      \
+  template <class Hay, class Needles, class Out, detail::enable_if_device<Hay> = 0,                                      \
+            class = typename std::iterator_traits<Out>::iterator_category>                                               \
+  Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o) { return NAME(device, f, l, vf, vl, o); }                        \
+  template <class Hay, class Needles, class Out, detail::enable_if_host<Hay> = 0,                                        \
+            class = typename std::iterator_traits<Out>::iterator_category>                                               \
+  Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o) { return NAME(host, f, l, vf, vl, o); }                          \
+  template <class Hay, class Needles, class Out, class Comp, detail::enable_if_device<Hay> = 0,                          \
+            class = typename std::iterator_traits<Out>::iterator_category>                                               \
+  Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o, Comp c) { return NAME(device, f, l, vf, vl, o, c); }             \
+  template <class Hay, class Needles, class Out, class Comp, detail::enable_if_host<Hay> = 0,                            \
+            class = typename std::iterator_traits<Out>::iterator_category>                                               \
+  Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o, Comp c) { return NAME(host, f, l, vf, vl, o, c); }
+THRUST_CDNA4_SEARCH(lower_bound, 0)
+THRUST_CDNA4_SEARCH(upper_bound, 1)
+THRUST_CDNA4_SEARCH(binary_search, 2)
+#undef THRUST_CDNA4_SEARCH
+
+// scalar forms: an iterator for the bounds, a bool for binary_search
+#define THRUST_CDNA4_SCALAR_BOUND(NAME, MODE)                                                                            \
+  template <class Policy, class Hay, class T, class Comp, detail::enable_if_policy<Policy> = 0>                          \
+  Hay NAME(const Policy& exec, Hay first, Hay last, const T& value, Comp comp) {                                         \
+    return first + detail::scalar_search<MODE>(exec, first, last, value, comp);                                          \
+  }                                                                                                                      \
+  template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>                                      \
+  Hay NAME(const Policy& exec, Hay first, Hay last, const T& value) {                                                    \
+    return first + detail::scalar_search<MODE>(exec, first, last, value, less<T>());                                     \
+  }                                                                                                                      \
+  template <class Hay, class T, detail::enable_if_device<Hay> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(device, f, l, v); } \
+  template <class Hay, class T, detail::enable_if_host<Hay> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(host, f, l, v); }
+THRUST_CDNA4_SCALAR_BOUND(lower_bound, 0)
+THRUST_CDNA4_SCALAR_BOUND(upper_bound, 1)
+#undef THRUST_CDNA4_SCALAR_BOUND
+template <class Policy, class Hay, class T, class Comp, detail::enable_if_policy<Policy> = 0>
+bool binary_search(const Policy& exec, Hay first, Hay last, const T& value, Comp comp) {
+  return detail::scalar_search<2>(exec, first, last, value, comp) != 0;
+}
+template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>
+bool binary_search(const Policy& exec, Hay first, Hay last, const T& value) {
+  return detail::scalar_search<2>(exec, first, last, value, less<T>()) != 0;
+}
+template <class Hay, class T, detail::enable_if_device<Hay> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(device, f, l, v); }
+template <class Hay, class T, detail::enable_if_host<Hay> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(host, f, l, v); }
+}  // namespace thrust

@@ -58,14 +58,13 @@ namespace thrust {
 template <class D, class In, class Out, class Pred>
 Out copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Pred pred) {
   typedef typename detail::value_of<In>::type V;
-  const V* in = (const V*)detail::unwrap(first);
-  return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), in, detail::unwrap(out), (std::int64_t)(last - first), pred);
+  return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), detail::unwrap(first), detail::unwrap(out), (std::int64_t)(last - first), pred);
 }
 template <class D, class In, class St, class Out, class Pred>
 Out copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, St stencil, Out out, Pred pred) {
   typedef typename detail::value_of<In>::type V;
   typedef typename detail::value_of<St>::type S;
-  return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), (const V*)detail::unwrap(first), (const S*)detail::unwrap(stencil),
+  return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), detail::unwrap(first), detail::unwrap(stencil),
                                                             detail::unwrap(out), (std::int64_t)(last - first), pred);
 }
 template <class In, class Out, class Pred>
@@ -83,4 +82,34 @@ Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(device, f, l, s, o
 template <class In, class St, class Out, class Pred, detail::enable_if_host<In> = 0,
           class = typename std::iterator_traits<St>::iterator_category>
 Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(host, f, l, s, o, p); }
+
+// thrust::copy from a fancy device iterator (counting, transform, zip, permutation ...): an
+// identity transform on the device; a host destination receives it through a device temporary.
+namespace detail {
+template <class It> struct is_fancy_device_iterator { static constexpr bool value = system::cdna4::detail::is_device_iterator<It>::value; };
+template <class T> struct is_fancy_device_iterator<device_ptr<T>> { static constexpr bool value = false; };
+}  // namespace detail
+template <class D, class In, class Out>
+Out copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out) {
+  const std::int64_t n = (std::int64_t)(last - first);
+  system::cdna4::detail::transform_n(exec.derived(), detail::unwrap(first), detail::unwrap(out), n, identity<typename detail::value_of<In>::type>());
+  return out + n;
+}
+template <class In, class Out>
+Out copy(const system::cpp::detail::par_t&, In first, In last, Out out) { return std::copy(first, last, out); }
+template <class In, class Out,
+          typename std::enable_if<detail::is_fancy_device_iterator<In>::value && system::cdna4::detail::is_device_iterator<Out>::value, int>::type = 0>
+Out copy(In first, In last, Out out) { return copy(device, first, last, out); }
+template <class In, class Out,
+          typename std::enable_if<detail::is_fancy_device_iterator<In>::value && !system::cdna4::detail::is_device_iterator<Out>::value, long>::type = 0>
+Out copy(In first, In last, Out out) {
+  typedef typename detail::value_of<In>::type V;
+  const std::size_t n = (std::size_t)(last - first);
+  V* tmp = static_cast<V*>(system::cdna4::detail::malloc_bytes(n * sizeof(V), nullptr));
+  copy(device, first, last, device_ptr<V>(tmp));
+  std::vector<V> host(n);
+  system::cdna4::detail::copy_bytes(host.data(), tmp, n * sizeof(V), 1);
+  system::cdna4::detail::free_bytes(tmp, nullptr);
+  return std::copy(host.begin(), host.end(), out);
+}
 }  // namespace thrust

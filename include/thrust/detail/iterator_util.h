@@ -5,8 +5,18 @@
 #include <type_traits>
 #include <thrust/device_ptr.h>
 namespace thrust { namespace detail {
-template <class T> inline T* unwrap(thrust::device_ptr<T> p) { return p.get(); }
-template <class T> inline T* unwrap(T* p) { return p; }  // raw device pointer under an explicit device policy
+// What a kernel receives for an iterator: device_ptr<T> becomes T*, a fancy iterator the same
+// iterator over unwrapped bases, anything else (a raw device pointer under an explicit device
+// policy, a counting iterator, a user's own device iterator) itself.
+template <class It> struct unwrap_iterator {
+  typedef It type;
+  static type apply(It it) { return it; }
+};
+template <class T> struct unwrap_iterator<thrust::device_ptr<T>> {
+  typedef T* type;
+  static type apply(thrust::device_ptr<T> p) { return p.get(); }
+};
+template <class It> inline typename unwrap_iterator<It>::type unwrap(It it) { return unwrap_iterator<It>::apply(it); }
 template <class It> struct value_of { typedef typename std::iterator_traits<It>::value_type type; };
 template <class It> using enable_if_device = typename std::enable_if<system::cdna4::detail::is_device_iterator<It>::value, int>::type;
 template <class It> using enable_if_host = typename std::enable_if<!system::cdna4::detail::is_device_iterator<It>::value, int>::type;

@@ -8,12 +8,12 @@
 namespace thrust {
 template <class D, class It, class F>
 It for_each(const system::cdna4::execution_policy<D>& exec, It first, It last, F f) {
-  system::cdna4::detail::for_each_n(exec.derived(), detail::unwrap(first), (std::int64_t)(last - first), f);
+  system::cdna4::detail::apply_n(exec.derived(), detail::unwrap(first), (std::int64_t)(last - first), f);
   return last;
 }
 template <class D, class It, class Size, class F>
 It for_each_n(const system::cdna4::execution_policy<D>& exec, It first, Size n, F f) {
-  system::cdna4::detail::for_each_n(exec.derived(), detail::unwrap(first), (std::int64_t)n, f);
+  system::cdna4::detail::apply_n(exec.derived(), detail::unwrap(first), (std::int64_t)n, f);
   return first + n;
 }
 template <class It, class F>

@@ -1,0 +1,24 @@
+// thrust::counting_iterator (thrust/iterator/counting_iterator.h): element n is first + n.
+#pragma once
+#include <thrust/detail/iterator_util.h>
+#include <thrust/iterator/detail/fancy_base.h>
+
+namespace thrust {
+template <class T>
+class counting_iterator : public detail::fancy_base<counting_iterator<T>, T> {
+ public:
+  typedef T value_type;
+  typedef T reference;
+  counting_iterator() : v_() {}
+  THRUST_CDNA4_HD explicit counting_iterator(T v) : v_(v) {}
+  THRUST_CDNA4_HD T at(std::ptrdiff_t n) const { return (T)(v_ + (T)n); }
+  THRUST_CDNA4_HD void advance(std::ptrdiff_t n) { v_ = (T)(v_ + (T)n); }
+  THRUST_CDNA4_HD std::ptrdiff_t distance_to(const counting_iterator& o) const { return (std::ptrdiff_t)(o.v_ - v_); }
+ private:
+  T v_;
+};
+template <class T> THRUST_CDNA4_HD counting_iterator<T> make_counting_iterator(T v) { return counting_iterator<T>(v); }
+namespace system { namespace cdna4 { namespace detail {
+template <class T> struct is_device_iterator<thrust::counting_iterator<T>> { static constexpr bool value = true; };
+}}}
+}  // namespace thrust

@@ -1,0 +1,28 @@
+// thrust::discard_iterator (thrust/iterator/discard_iterator.h): an output that ignores what is
+// assigned to it.
+#pragma once
+#include <thrust/detail/iterator_util.h>
+#include <thrust/iterator/detail/fancy_base.h>
+
+namespace thrust {
+namespace detail {
+struct discard_proxy {
+  template <class T> THRUST_CDNA4_HD const discard_proxy& operator=(const T&) const { return *this; }
+};
+}  // namespace detail
+class discard_iterator : public detail::fancy_base<discard_iterator, detail::discard_proxy> {
+ public:
+  typedef detail::discard_proxy value_type;
+  typedef detail::discard_proxy reference;
+  THRUST_CDNA4_HD explicit discard_iterator(std::ptrdiff_t pos = 0) : pos_(pos) {}
+  THRUST_CDNA4_HD detail::discard_proxy at(std::ptrdiff_t) const { return detail::discard_proxy(); }
+  THRUST_CDNA4_HD void advance(std::ptrdiff_t n) { pos_ += n; }
+  THRUST_CDNA4_HD std::ptrdiff_t distance_to(const discard_iterator& o) const { return o.pos_ - pos_; }
+ private:
+  std::ptrdiff_t pos_;
+};
+THRUST_CDNA4_HD inline discard_iterator make_discard_iterator(std::ptrdiff_t pos = 0) { return discard_iterator(pos); }
+namespace system { namespace cdna4 { namespace detail {
+template <> struct is_device_iterator<thrust::discard_iterator> { static constexpr bool value = true; };
+}}}
+}  // namespace thrust

@@ -1,0 +1,40 @@
+// thrust::transform_iterator (thrust/iterator/transform_iterator.h): element n is f(base[n]).
+#pragma once
+#include <type_traits>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/iterator/detail/fancy_base.h>
+
+namespace thrust {
+namespace detail {
+template <class F, class It> struct transformed_value {
+  typedef typename std::decay<decltype(std::declval<const F&>()(std::declval<typename std::iterator_traits<It>::value_type>()))>::type type;
+};
+}  // namespace detail
+template <class F, class It>
+class transform_iterator : public detail::fancy_base<transform_iterator<F, It>, typename detail::transformed_value<F, It>::type> {
+ public:
+  typedef typename detail::transformed_value<F, It>::type value_type;
+  typedef value_type reference;
+  transform_iterator() : it_(), f_() {}
+  THRUST_CDNA4_HD transform_iterator(It it, F f) : it_(it), f_(f) {}
+  THRUST_CDNA4_HD value_type at(std::ptrdiff_t n) const { return f_(it_[n]); }
+  THRUST_CDNA4_HD void advance(std::ptrdiff_t n) { it_ += n; }
+  THRUST_CDNA4_HD std::ptrdiff_t distance_to(const transform_iterator& o) const { return o.it_ - it_; }
+  THRUST_CDNA4_HD It base() const { return it_; }
+  THRUST_CDNA4_HD F functor() const { return f_; }
+ private:
+  It it_;
+  F f_;
+};
+template <class F, class It>
+THRUST_CDNA4_HD transform_iterator<F, It> make_transform_iterator(It it, F f) { return transform_iterator<F, It>(it, f); }
+namespace system { namespace cdna4 { namespace detail {
+template <class F, class It> struct is_device_iterator<thrust::transform_iterator<F, It>> : is_device_iterator<It> {};
+}}}
+namespace detail {
+template <class F, class It> struct unwrap_iterator<thrust::transform_iterator<F, It>> {
+  typedef thrust::transform_iterator<F, typename unwrap_iterator<It>::type> type;
+  static type apply(const thrust::transform_iterator<F, It>& it) { return type(unwrap(it.base()), it.functor()); }
+};
+}  // namespace detail
+}  // namespace thrust

@@ -19,7 +19,7 @@ pair<OutT, OutF> stable_partition_copy(const system::cdna4::execution_policy<D>&
   typedef typename detail::value_of<In>::type V;
   typedef typename detail::value_of<St>::type S;
   const std::int64_t n = (std::int64_t)(last - first);
-  const std::int64_t c = system::cdna4::detail::partition_copy_n(exec.derived(), (const V*)detail::unwrap(first), (const S*)detail::unwrap(stencil),
+  const std::int64_t c = system::cdna4::detail::partition_copy_n(exec.derived(), detail::unwrap(first), detail::unwrap(stencil),
                                                                  detail::unwrap(out_true), detail::unwrap(out_false), n, pred);
   return thrust::make_pair(out_true + c, out_false + (n - c));
 }

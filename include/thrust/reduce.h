@@ -18,15 +18,18 @@ namespace thrust {
 template <class D, class KIt, class VIt, class KOut, class VOut, class Pred, class Op>
 pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
                                KOut kout, VOut vout, Pred, Op) {
+  namespace sd = system::cdna4::detail;
   typedef typename detail::elem<KIt>::type K;
   typedef typename detail::elem<VIt>::type V;
-  static_assert(std::is_same<K, typename detail::elem<KOut>::type>::value &&
-                std::is_same<V, typename detail::elem<VOut>::type>::value,
-                "cdna4 reduce_by_key: output element types must match the input's");
-  const std::int64_t runs = system::cdna4::detail::reduce_by_key(
-      exec.derived(), (const K*)detail::unwrap(kfirst), (const V*)detail::unwrap(vfirst), detail::unwrap(kout),
-      detail::unwrap(vout), (std::int64_t)(klast - kfirst), typename detail::rebind_op<Pred, K>::type(),
-      typename detail::rebind_op<Op, V>::type());
+  const std::int64_t n = (std::int64_t)(klast - kfirst);
+  sd::contiguous_input<K, typename detail::unwrap_iterator<KIt>::type> keys(exec.derived(), detail::unwrap(kfirst), n);
+  sd::contiguous_input<V, typename detail::unwrap_iterator<VIt>::type> vals(exec.derived(), detail::unwrap(vfirst), n);
+  sd::contiguous_output<K, typename detail::unwrap_iterator<KOut>::type> ko(exec.derived(), detail::unwrap(kout), n);
+  sd::contiguous_output<V, typename detail::unwrap_iterator<VOut>::type> vo(exec.derived(), detail::unwrap(vout), n);
+  const std::int64_t runs = sd::reduce_by_key(exec.derived(), keys.data(), vals.data(), ko.data(), vo.data(), n,
+                                              typename detail::rebind_op<Pred, K>::type(), typename detail::rebind_op<Op, V>::type());
+  ko.flush(exec.derived(), runs);
+  vo.flush(exec.derived(), runs);
   return thrust::make_pair(kout + runs, vout + runs);
 }
 template <class D, class KIt, class VIt, class KOut, class VOut, class Pred>
@@ -91,7 +94,7 @@ THRUST_CDNA4_RBK(host, detail::enable_if_host)
 template <class D, class It, class T, class Op>
 T reduce(const system::cdna4::execution_policy<D>& exec, It first, It last, T init, Op op) {
   typedef typename detail::value_of<It>::type V;
-  return system::cdna4::detail::transform_reduce_n(exec.derived(), (const V*)detail::unwrap(first),
+  return system::cdna4::detail::transform_reduce_n(exec.derived(), detail::unwrap(first),
                                                    (std::int64_t)(last - first), identity<V>(), init, op);
 }
 template <class D, class It, class T>

@@ -11,7 +11,7 @@ namespace thrust {
 template <class D, class In, class Out, class Pred>
 Out remove_copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Pred pred) {
   typedef typename detail::value_of<In>::type V;
-  const V* in = (const V*)detail::unwrap(first);
+  const V* in = detail::unwrap(first);
   return out + system::cdna4::detail::copy_flagged_n<true>(exec.derived(), in, detail::unwrap(out), (std::int64_t)(last - first), pred);
 }
 template <class D, class In, class Pred>

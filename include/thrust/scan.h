@@ -7,6 +7,7 @@
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
 #include <thrust/system/cdna4/detail/algorithms.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
 
@@ -23,13 +24,14 @@ template <template <class> class F, class T> struct rebind_op<F<void>, T> { type
 // ===================================================================== scan, device
 template <class D, class InIt, class OutIt, class Op>
 OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, Op) {
+  namespace sd = system::cdna4::detail;
   typedef typename detail::elem<InIt>::type T;
-  static_assert(std::is_same<T, typename detail::elem<OutIt>::type>::value,
-                "cdna4 inclusive_scan: input and output element types must match");
-  system::cdna4::detail::scan(exec.derived(), (const T*)detail::unwrap(first), detail::unwrap(result),
-                              (std::int64_t)(last - first), false, (const T*)nullptr,
-                              typename detail::rebind_op<Op, T>::type());
-  return result + (last - first);
+  const std::int64_t n = (std::int64_t)(last - first);
+  sd::contiguous_input<T, typename detail::unwrap_iterator<InIt>::type> in(exec.derived(), detail::unwrap(first), n);
+  sd::contiguous_output<T, typename detail::unwrap_iterator<OutIt>::type> out(exec.derived(), detail::unwrap(result), n);
+  sd::scan(exec.derived(), in.data(), out.data(), n, false, (const T*)nullptr, typename detail::rebind_op<Op, T>::type());
+  out.flush(exec.derived(), n);
+  return result + n;
 }
 template <class D, class InIt, class OutIt>
 OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result) {
@@ -39,14 +41,16 @@ OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first,
 // the kernels accumulate in the element type, so the two must be the same type.
 template <class D, class InIt, class OutIt, class T, class Op>
 OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, T init, Op) {
+  namespace sd = system::cdna4::detail;
   typedef typename detail::elem<InIt>::type V;
-  static_assert(std::is_same<V, typename detail::elem<OutIt>::type>::value,
-                "cdna4 exclusive_scan: input and output element types must match");
   static_assert(std::is_same<V, T>::value,
                 "cdna4 exclusive_scan: init must have the element type (it is the accumulator type)");
-  system::cdna4::detail::scan(exec.derived(), (const V*)detail::unwrap(first), detail::unwrap(result),
-                              (std::int64_t)(last - first), true, &init, typename detail::rebind_op<Op, V>::type());
-  return result + (last - first);
+  const std::int64_t n = (std::int64_t)(last - first);
+  sd::contiguous_input<V, typename detail::unwrap_iterator<InIt>::type> in(exec.derived(), detail::unwrap(first), n);
+  sd::contiguous_output<V, typename detail::unwrap_iterator<OutIt>::type> out(exec.derived(), detail::unwrap(result), n);
+  sd::scan(exec.derived(), in.data(), out.data(), n, true, &init, typename detail::rebind_op<Op, V>::type());
+  out.flush(exec.derived(), n);
+  return result + n;
 }
 template <class D, class InIt, class OutIt, class T>
 OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, T init) {
@@ -125,14 +129,17 @@ OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init, Op op) { return exclusive_
 template <class D, class KIt, class VIt, class OutIt, class Pred, class Op>
 OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
                             OutIt result, Pred, Op) {
+  namespace sd = system::cdna4::detail;
   typedef typename detail::elem<KIt>::type K;
   typedef typename detail::elem<VIt>::type V;
-  static_assert(std::is_same<V, typename detail::elem<OutIt>::type>::value,
-                "cdna4 inclusive_scan_by_key: value and output element types must match");
-  system::cdna4::detail::scan_by_key(exec.derived(), (const K*)detail::unwrap(kfirst), (const V*)detail::unwrap(vfirst),
-                                     detail::unwrap(result), (std::int64_t)(klast - kfirst), false, (const V*)nullptr,
-                                     typename detail::rebind_op<Pred, K>::type(), typename detail::rebind_op<Op, V>::type());
-  return result + (klast - kfirst);
+  const std::int64_t n = (std::int64_t)(klast - kfirst);
+  sd::contiguous_input<K, typename detail::unwrap_iterator<KIt>::type> keys(exec.derived(), detail::unwrap(kfirst), n);
+  sd::contiguous_input<V, typename detail::unwrap_iterator<VIt>::type> vals(exec.derived(), detail::unwrap(vfirst), n);
+  sd::contiguous_output<V, typename detail::unwrap_iterator<OutIt>::type> out(exec.derived(), detail::unwrap(result), n);
+  sd::scan_by_key(exec.derived(), keys.data(), vals.data(), out.data(), n, false, (const V*)nullptr,
+                  typename detail::rebind_op<Pred, K>::type(), typename detail::rebind_op<Op, V>::type());
+  out.flush(exec.derived(), n);
+  return result + n;
 }
 template <class D, class KIt, class VIt, class OutIt, class Pred>
 OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, Pred p) {
@@ -145,14 +152,18 @@ OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt 
 template <class D, class KIt, class VIt, class OutIt, class T, class Pred, class Op>
 OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
                             OutIt result, T init, Pred, Op) {
+  namespace sd = system::cdna4::detail;
   typedef typename detail::elem<KIt>::type K;
   typedef typename detail::elem<VIt>::type V;
-  static_assert(std::is_same<V, typename detail::elem<OutIt>::type>::value && std::is_same<V, T>::value,
-                "cdna4 exclusive_scan_by_key: values, output and init must have one element type");
-  system::cdna4::detail::scan_by_key(exec.derived(), (const K*)detail::unwrap(kfirst), (const V*)detail::unwrap(vfirst),
-                                     detail::unwrap(result), (std::int64_t)(klast - kfirst), true, &init,
-                                     typename detail::rebind_op<Pred, K>::type(), typename detail::rebind_op<Op, V>::type());
-  return result + (klast - kfirst);
+  static_assert(std::is_same<V, T>::value, "cdna4 exclusive_scan_by_key: init must have the values' element type");
+  const std::int64_t n = (std::int64_t)(klast - kfirst);
+  sd::contiguous_input<K, typename detail::unwrap_iterator<KIt>::type> keys(exec.derived(), detail::unwrap(kfirst), n);
+  sd::contiguous_input<V, typename detail::unwrap_iterator<VIt>::type> vals(exec.derived(), detail::unwrap(vfirst), n);
+  sd::contiguous_output<V, typename detail::unwrap_iterator<OutIt>::type> out(exec.derived(), detail::unwrap(result), n);
+  sd::scan_by_key(exec.derived(), keys.data(), vals.data(), out.data(), n, true, &init,
+                  typename detail::rebind_op<Pred, K>::type(), typename detail::rebind_op<Op, V>::type());
+  out.flush(exec.derived(), n);
+  return result + n;
 }
 template <class D, class KIt, class VIt, class OutIt, class T, class Pred>
 OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, T init, Pred p) {

@@ -4,6 +4,7 @@
 // says so (never a host fallback).
 #pragma once
 #include <cstdint>
+#include <iterator>
 #include <thrust/functional.h>
 #include <thrust/system/cdna4/detail/core.h>
 #if defined(__HIPCC__)
@@ -22,41 +23,44 @@ template <class T> struct needs_hipcc { static constexpr bool value = sizeof(T) 
                 "translation unit with hipcc --offload-arch=gfx950")
 #endif
 
+// In the bodies below an "iterator" is whatever detail::unwrap gives a kernel: a raw pointer or a
+// fancy iterator over raw pointers, indexable on the device.
 #if defined(__HIPCC__)
-template <class In, class F> struct for_each_body {
-  In* p; F f;
+template <class It> struct value_of_it { typedef typename std::iterator_traits<It>::value_type type; };
+template <class It, class F> struct for_each_body {
+  It p; F f;
   __device__ void operator()(std::int64_t i) { f(p[i]); }
 };
 template <class In, class Out, class F> struct transform1_body {
-  const In* in; Out* out; F f;
+  In in; Out out; F f;
   __device__ void operator()(std::int64_t i) { out[i] = f(in[i]); }
 };
 template <class In1, class In2, class Out, class F> struct transform2_body {
-  const In1* a; const In2* b; Out* out; F f;
+  In1 a; In2 b; Out out; F f;
   __device__ void operator()(std::int64_t i) { out[i] = f(a[i], b[i]); }
 };
-template <class T> struct sequence_body {
-  T* out; T init, step;
+template <class Out, class T> struct sequence_body {
+  Out out; T init, step;
   __device__ void operator()(std::int64_t i) { out[i] = (T)(init + (T)i * step); }
 };
 template <class In, class F, class T> struct load_transform {
-  const In* in; F f;
+  In in; F f;
   __device__ T operator()(std::int64_t i) const { return (T)f(in[i]); }
 };
 #endif
 
-template <class Policy, class In, class F>
-void for_each_n(const Policy& exec, In* p, std::int64_t n, F f) {
+template <class Policy, class It, class F>
+void apply_n(const Policy& exec, It p, std::int64_t n, F f) {
   THRUST_CDNA4_NEEDS_HIPCC(F);
 #if defined(__HIPCC__)
-  generic::parallel_for(stream_of(exec), n, for_each_body<In, F>{p, f});
+  generic::parallel_for(stream_of(exec), n, for_each_body<It, F>{p, f});
   synchronize_optional(exec, "for_each: failed to synchronize");
 #else
   (void)exec; (void)p; (void)n; (void)f;
 #endif
 }
 template <class Policy, class In, class Out, class F>
-void transform_n(const Policy& exec, const In* in, Out* out, std::int64_t n, F f) {
+void transform_n(const Policy& exec, In in, Out out, std::int64_t n, F f) {
   THRUST_CDNA4_NEEDS_HIPCC(F);
 #if defined(__HIPCC__)
   generic::parallel_for(stream_of(exec), n, transform1_body<In, Out, F>{in, out, f});
@@ -66,7 +70,7 @@ void transform_n(const Policy& exec, const In* in, Out* out, std::int64_t n, F f
 #endif
 }
 template <class Policy, class In1, class In2, class Out, class F>
-void transform_n(const Policy& exec, const In1* a, const In2* b, Out* out, std::int64_t n, F f) {
+void transform_n(const Policy& exec, In1 a, In2 b, Out out, std::int64_t n, F f) {
   THRUST_CDNA4_NEEDS_HIPCC(F);
 #if defined(__HIPCC__)
   generic::parallel_for(stream_of(exec), n, transform2_body<In1, In2, Out, F>{a, b, out, f});
@@ -75,18 +79,18 @@ void transform_n(const Policy& exec, const In1* a, const In2* b, Out* out, std::
   (void)exec; (void)a; (void)b; (void)out; (void)n; (void)f;
 #endif
 }
-template <class Policy, class T>
-void sequence_n(const Policy& exec, T* out, std::int64_t n, T init, T step) {
+template <class Policy, class Out, class T>
+void sequence_n(const Policy& exec, Out out, std::int64_t n, T init, T step) {
   THRUST_CDNA4_NEEDS_HIPCC(T);
 #if defined(__HIPCC__)
-  generic::parallel_for(stream_of(exec), n, sequence_body<T>{out, init, step});
+  generic::parallel_for(stream_of(exec), n, sequence_body<Out, T>{out, init, step});
   synchronize_optional(exec, "sequence: failed to synchronize");
 #else
   (void)exec; (void)out; (void)n; (void)init; (void)step;
 #endif
 }
 template <class Policy, class In, class F, class T, class Op>
-T transform_reduce_n(const Policy& exec, const In* in, std::int64_t n, F f, T init, Op op) {
+T transform_reduce_n(const Policy& exec, In in, std::int64_t n, F f, T init, Op op) {
   THRUST_CDNA4_NEEDS_HIPCC(F);
 #if defined(__HIPCC__)
   return generic::transform_reduce(stream_of(exec), n, load_transform<In, F, T>{in, f}, init, op);
@@ -96,15 +100,15 @@ T transform_reduce_n(const Policy& exec, const In* in, std::int64_t n, F f, T in
 #endif
 }
 
-// ---- stable compaction (copy_if / remove_if / unique / unique_by_key) ------------------
+// ---- stable compaction (copy_if / remove_if / unique / unique_by_key / partition) -------
 #if defined(__HIPCC__)
 // keep in[i] when pred(in[i]) != NEGATE
 template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
-  typedef In item;
+  typedef typename value_of_it<In>::type item;
   static constexpr bool rejects = false;
-  const In* in; Out* out; Pred pred;
+  In in; Out out; Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
-    const In x = in[i];
+    const item x = in[i];
     keep = (bool)pred(x) != NEGATE;
     return x;
   }
@@ -112,9 +116,9 @@ template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
 };
 // keep in[i] when pred(stencil[i]) != NEGATE
 template <class In, class S, class Out, class Pred, bool NEGATE> struct keep_if_stencil_op {
-  typedef In item;
+  typedef typename value_of_it<In>::type item;
   static constexpr bool rejects = false;
-  const In* in; const S* stencil; Out* out; Pred pred;
+  In in; S stencil; Out out; Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     keep = (bool)pred(stencil[i]) != NEGATE;
     return in[i];
@@ -123,9 +127,9 @@ template <class In, class S, class Out, class Pred, bool NEGATE> struct keep_if_
 };
 // in[i] goes to out_true when pred(stencil[i]), else to out_false, both in order
 template <class In, class S, class OutT, class OutF, class Pred> struct partition_op {
-  typedef In item;
+  typedef typename value_of_it<In>::type item;
   static constexpr bool rejects = true;
-  const In* in; const S* stencil; OutT* out_true; OutF* out_false; Pred pred;
+  In in; S stencil; OutT out_true; OutF out_false; Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     keep = (bool)pred(stencil[i]);
     return in[i];
@@ -134,21 +138,23 @@ template <class In, class S, class OutT, class OutF, class Pred> struct partitio
   __device__ void store_rejected(const item& x, std::int64_t pos) const { out_false[pos] = x; }
 };
 // keep the first element of every run; element 0 compares with itself and is kept by index
-template <class K, class KOut, class Eq> struct run_head_op {
-  typedef K item;
+template <class KIn, class KOut, class Eq> struct run_head_op {
+  typedef typename value_of_it<KIn>::type item;
   static constexpr bool rejects = false;
-  const K* keys; KOut* out; Eq eq;
+  KIn keys; KOut out; Eq eq;
   __device__ item load(std::int64_t i, bool& keep) const {
-    const K cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
+    const item cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
     keep = (i == 0) | !(bool)eq(prev, cur);
     return cur;
   }
   __device__ void store(const item& x, std::int64_t pos) const { out[pos] = x; }
 };
-template <class K, class V, class KOut, class VOut, class Eq> struct run_head_by_key_op {
+template <class KIn, class VIn, class KOut, class VOut, class Eq> struct run_head_by_key_op {
+  typedef typename value_of_it<KIn>::type K;
+  typedef typename value_of_it<VIn>::type V;
   struct item { K key; V value; };
   static constexpr bool rejects = false;
-  const K* keys; const V* values; KOut* kout; VOut* vout; Eq eq;
+  KIn keys; VIn values; KOut kout; VOut vout; Eq eq;
   __device__ item load(std::int64_t i, bool& keep) const {
     const K cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
     keep = (i == 0) | !(bool)eq(prev, cur);
@@ -160,7 +166,7 @@ template <class K, class V, class KOut, class VOut, class Eq> struct run_head_by
 
 // out[0, count) = the in[i] with pred(in[i]) != NEGATE, in order; returns count
 template <bool NEGATE, class Policy, class In, class Out, class Pred>
-std::int64_t copy_flagged_n(const Policy& exec, const In* in, Out* out, std::int64_t n, Pred pred) {
+std::int64_t copy_flagged_n(const Policy& exec, In in, Out out, std::int64_t n, Pred pred) {
   THRUST_CDNA4_NEEDS_HIPCC(Pred);
 #if defined(__HIPCC__)
   return generic::select(stream_of(exec), n, keep_if_op<In, Out, Pred, NEGATE>{in, out, pred});
@@ -171,7 +177,7 @@ std::int64_t copy_flagged_n(const Policy& exec, const In* in, Out* out, std::int
 }
 // the same with the predicate applied to stencil[i]
 template <bool NEGATE, class Policy, class In, class S, class Out, class Pred>
-std::int64_t copy_flagged_n(const Policy& exec, const In* in, const S* stencil, Out* out, std::int64_t n, Pred pred) {
+std::int64_t copy_flagged_n(const Policy& exec, In in, S stencil, Out out, std::int64_t n, Pred pred) {
   THRUST_CDNA4_NEEDS_HIPCC(Pred);
 #if defined(__HIPCC__)
   return generic::select(stream_of(exec), n, keep_if_stencil_op<In, S, Out, Pred, NEGATE>{in, stencil, out, pred});
@@ -182,7 +188,7 @@ std::int64_t copy_flagged_n(const Policy& exec, const In* in, const S* stencil, 
 }
 // stable two-way split by pred(stencil[i]); returns the number that went to out_true
 template <class Policy, class In, class S, class OutT, class OutF, class Pred>
-std::int64_t partition_copy_n(const Policy& exec, const In* in, const S* stencil, OutT* out_true, OutF* out_false, std::int64_t n, Pred pred) {
+std::int64_t partition_copy_n(const Policy& exec, In in, S stencil, OutT out_true, OutF out_false, std::int64_t n, Pred pred) {
   THRUST_CDNA4_NEEDS_HIPCC(Pred);
 #if defined(__HIPCC__)
   return generic::select(stream_of(exec), n, partition_op<In, S, OutT, OutF, Pred>{in, stencil, out_true, out_false, pred});
@@ -192,26 +198,141 @@ std::int64_t partition_copy_n(const Policy& exec, const In* in, const S* stencil
 #endif
 }
 // out[0, count) = the first element of every run of equal elements; returns count
-template <class Policy, class K, class KOut, class Eq>
-std::int64_t unique_copy_n(const Policy& exec, const K* in, KOut* out, std::int64_t n, Eq eq) {
+template <class Policy, class KIn, class KOut, class Eq>
+std::int64_t unique_copy_n(const Policy& exec, KIn in, KOut out, std::int64_t n, Eq eq) {
   THRUST_CDNA4_NEEDS_HIPCC(Eq);
 #if defined(__HIPCC__)
-  return generic::select(stream_of(exec), n, run_head_op<K, KOut, Eq>{in, out, eq});
+  return generic::select(stream_of(exec), n, run_head_op<KIn, KOut, Eq>{in, out, eq});
 #else
   (void)exec; (void)in; (void)out; (void)n; (void)eq;
   return 0;
 #endif
 }
-template <class Policy, class K, class V, class KOut, class VOut, class Eq>
-std::int64_t unique_by_key_copy_n(const Policy& exec, const K* keys, const V* vals, KOut* kout, VOut* vout, std::int64_t n, Eq eq) {
+template <class Policy, class KIn, class VIn, class KOut, class VOut, class Eq>
+std::int64_t unique_by_key_copy_n(const Policy& exec, KIn keys, VIn vals, KOut kout, VOut vout, std::int64_t n, Eq eq) {
   THRUST_CDNA4_NEEDS_HIPCC(Eq);
 #if defined(__HIPCC__)
-  return generic::select(stream_of(exec), n, run_head_by_key_op<K, V, KOut, VOut, Eq>{keys, vals, kout, vout, eq});
+  return generic::select(stream_of(exec), n, run_head_by_key_op<KIn, VIn, KOut, VOut, Eq>{keys, vals, kout, vout, eq});
 #else
   (void)exec; (void)keys; (void)vals; (void)kout; (void)vout; (void)n; (void)eq;
   return 0;
 #endif
 }
+
+// ---- adjacent_difference, vectorised binary searches ------------------------------------
+#if defined(__HIPCC__)
+template <class In, class Out, class Op> struct adjacent_difference_body {
+  In in; Out out; Op op;
+  __device__ void operator()(std::int64_t i) {
+    typedef typename value_of_it<In>::type T;
+    const T cur = in[i];
+    if (i == 0) out[i] = cur;
+    else out[i] = op(cur, (T)in[i - 1]);
+  }
+};
+// MODE 0: first position whose element is not less than the value (lower bound); 1: first
+// position whose element is greater (upper bound); 2: whether an equivalent element exists
+template <int MODE, class Hay, class Needles, class Out, class Comp> struct binary_search_body {
+  Hay hay; std::int64_t count; Needles needles; Out out; Comp comp;
+  __device__ void operator()(std::int64_t i) {
+    const auto v = needles[i];
+    std::int64_t lo = 0, len = count;
+    while (len > 0) {
+      const std::int64_t half = len >> 1;
+      const bool right = MODE == 1 ? !(bool)comp(v, hay[lo + half]) : (bool)comp(hay[lo + half], v);
+      lo = right ? lo + half + 1 : lo;
+      len = right ? len - half - 1 : half;
+    }
+    if (MODE == 2) out[i] = lo < count && !(bool)comp(v, hay[lo]);
+    else out[i] = lo;
+  }
+};
+#endif
+template <class Policy, class In, class Out, class Op>
+void adjacent_difference_n(const Policy& exec, In in, Out out, std::int64_t n, Op op) {
+  THRUST_CDNA4_NEEDS_HIPCC(Op);
+#if defined(__HIPCC__)
+  generic::parallel_for(stream_of(exec), n, adjacent_difference_body<In, Out, Op>{in, out, op});
+  synchronize_optional(exec, "adjacent_difference: failed to synchronize");
+#else
+  (void)exec; (void)in; (void)out; (void)n; (void)op;
+#endif
+}
+template <int MODE, class Policy, class Hay, class Needles, class Out, class Comp>
+void binary_search_n(const Policy& exec, Hay hay, std::int64_t count, Needles needles, Out out, std::int64_t n, Comp comp) {
+  THRUST_CDNA4_NEEDS_HIPCC(Comp);
+#if defined(__HIPCC__)
+  generic::parallel_for(stream_of(exec), n, binary_search_body<MODE, Hay, Needles, Out, Comp>{hay, count, needles, out, comp});
+  synchronize_optional(exec, "binary search: failed to synchronize");
+#else
+  (void)exec; (void)hay; (void)count; (void)needles; (void)out; (void)n; (void)comp;
+#endif
+}
+
+// ---- fancy iterators around the C-ABI algorithms (sort, scan, by-key) --------------------
+// Those kernels read and write contiguous arrays.  A raw pointer passes through; any other
+// iterator is read into (input) or written from (output) a pool temporary by one generic kernel.
+template <class T, class It, bool RAW = std::is_pointer<It>::value> class contiguous_input;
+template <class T, class It> class contiguous_input<T, It, true> {
+ public:
+  template <class Policy> contiguous_input(const Policy&, It it, std::int64_t) : p_(it) {
+    static_assert(std::is_same<T, typename std::remove_const<typename std::remove_pointer<It>::type>::type>::value,
+                  "cdna4: the element type of this range must match the algorithm's");
+  }
+  const T* data() const { return p_; }
+ private:
+  const T* p_;
+};
+template <class T, class It> class contiguous_input<T, It, false> {
+ public:
+  template <class Policy> contiguous_input(const Policy& exec, It it, std::int64_t n)
+      : tmp_((std::size_t)(n > 0 ? n : 0) * sizeof(T), stream_of(exec)) {
+    THRUST_CDNA4_NEEDS_HIPCC(It);
+#if defined(__HIPCC__)
+    generic::parallel_for(stream_of(exec), n, transform1_body<It, T*, thrust::identity<T>>{it, static_cast<T*>(tmp_.data()), thrust::identity<T>()});
+#else
+    (void)it;
+#endif
+  }
+  const T* data() const { return static_cast<const T*>(tmp_.data()); }
+ private:
+  temporary_storage tmp_;
+};
+template <class T, class It, bool RAW = std::is_pointer<It>::value> class contiguous_output;
+template <class T, class It> class contiguous_output<T, It, true> {
+ public:
+  template <class Policy> contiguous_output(const Policy&, It it, std::int64_t) : p_(it) {
+    static_assert(std::is_same<T, typename std::remove_pointer<It>::type>::value,
+                  "cdna4: the element type of the output range must match the algorithm's");
+  }
+  T* data() const { return p_; }
+  template <class Policy> void flush(const Policy&, std::int64_t) {}
+ private:
+  T* p_;
+};
+template <class T, class It> class contiguous_output<T, It, false> {
+ public:
+  template <class Policy> contiguous_output(const Policy& exec, It it, std::int64_t n)
+      : it_(it), tmp_((std::size_t)(n > 0 ? n : 0) * sizeof(T), stream_of(exec)) {}
+  T* data() const { return static_cast<T*>(tmp_.data()); }
+  // the first count elements go to the iterator
+  template <class Policy> void flush(const Policy& exec, std::int64_t count) {
+    THRUST_CDNA4_NEEDS_HIPCC(It);
+#if defined(__HIPCC__)
+    generic::parallel_for(stream_of(exec), count, transform1_body<const T*, It, thrust::identity<T>>{data(), it_, thrust::identity<T>()});
+    synchronize_optional(exec, "output: failed to synchronize");
+#else
+    (void)exec; (void)count;
+#endif
+  }
+ private:
+  It it_;
+  temporary_storage tmp_;
+};
+
+// the address behind a raw pointer (only raw pointers can alias an output range)
+template <class T> inline const void* address_of(T* p) { return p; }
+template <class It> inline const void* address_of(It) { return nullptr; }
 
 // A device copy of [p, p + n) from the pool, for the in-place variants (the compaction reads its
 // whole input while other tiles already write the front of the output).

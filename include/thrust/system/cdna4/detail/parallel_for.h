@@ -159,6 +159,13 @@ __global__ __launch_bounds__(256) void select_init_kernel(Word* words, std::int6
   if (i < count) words[i] = Word(0);
 }
 
+template <bool REJECTS> struct select_rejected {
+  template <class Op, class Item> __device__ static void store(const Op& op, const Item& x, std::int64_t pos) { op.store_rejected(x, pos); }
+};
+template <> struct select_rejected<false> {
+  template <class Op, class Item> __device__ static void store(const Op&, const Item&, std::int64_t) {}
+};
+
 template <class Op>
 __global__ __launch_bounds__(kSelBlock)
 __attribute__((amdgpu_waves_per_eu(select_waves_per_simd(sizeof(typename Op::item)), select_waves_per_simd(sizeof(typename Op::item)))))
@@ -266,7 +273,7 @@ void select_kernel(std::int64_t n, Op op, unsigned long long* words, std::int64_
     if ((mine >> j) & 1u)
       op.store(items[j], before);
     else if (Op::rejects && i < n)
-      op.store_rejected(items[j], i - before);  // rejected elements before this one
+      select_rejected<Op::rejects>::store(op, items[j], i - before);  // rejected elements before this one
   }
 }
 

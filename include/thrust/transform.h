@@ -9,15 +9,15 @@ namespace thrust {
 template <class D, class In, class Out, class F>
 Out transform(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, F f) {
   const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::transform_n(exec.derived(), (const typename detail::value_of<In>::type*)detail::unwrap(first),
+  system::cdna4::detail::transform_n(exec.derived(), detail::unwrap(first),
                                      detail::unwrap(out), n, f);
   return out + n;
 }
 template <class D, class In1, class In2, class Out, class F>
 Out transform(const system::cdna4::execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out out, F f) {
   const std::int64_t n = (std::int64_t)(last1 - first1);
-  system::cdna4::detail::transform_n(exec.derived(), (const typename detail::value_of<In1>::type*)detail::unwrap(first1),
-                                     (const typename detail::value_of<In2>::type*)detail::unwrap(first2), detail::unwrap(out), n, f);
+  system::cdna4::detail::transform_n(exec.derived(), detail::unwrap(first1),
+                                     detail::unwrap(first2), detail::unwrap(out), n, f);
   return out + n;
 }
 template <class In, class Out, class F>

@@ -7,7 +7,7 @@
 namespace thrust {
 template <class D, class It, class F, class T, class Op>
 T transform_reduce(const system::cdna4::execution_policy<D>& exec, It first, It last, F f, T init, Op op) {
-  return system::cdna4::detail::transform_reduce_n(exec.derived(), (const typename detail::value_of<It>::type*)detail::unwrap(first),
+  return system::cdna4::detail::transform_reduce_n(exec.derived(), detail::unwrap(first),
                                                    (std::int64_t)(last - first), f, init, op);
 }
 template <class It, class F, class T, class Op>

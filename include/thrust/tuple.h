@@ -1,0 +1,124 @@
+// thrust::tuple / get / make_tuple / tie / tuple_element / tuple_size (thrust/tuple.h): a small
+// tuple whose members are callable on the device (std::tuple's assignment is not, before C++20),
+// with element-wise conversion and assignment so that a tuple of references — what a
+// zip_iterator dereferences to — reads from and writes to a tuple of values.
+#pragma once
+#include <cstddef>
+#include <type_traits>
+#include <utility>
+#include <thrust/functional.h>
+
+namespace thrust {
+template <class... Ts> struct tuple;
+
+namespace detail {
+template <std::size_t I, class T> struct tuple_leaf {
+  T value;
+};
+// a reference member assigns through (and keeps tuples of values trivially copyable)
+template <std::size_t I, class T> struct tuple_leaf<I, T&> {
+  T& value;
+  THRUST_CDNA4_HD tuple_leaf& operator=(const tuple_leaf& o) {
+    value = o.value;
+    return *this;
+  }
+};
+template <std::size_t I, class... Ts> struct nth_type;
+template <class T, class... Ts> struct nth_type<0, T, Ts...> { typedef T type; };
+template <std::size_t I, class T, class... Ts> struct nth_type<I, T, Ts...> { typedef typename nth_type<I - 1, Ts...>::type type; };
+
+template <class... Us> struct is_single_tuple : std::false_type {};
+template <class... Ts> struct is_single_tuple<tuple<Ts...>> : std::true_type {};
+
+template <class Seq, class... Ts> struct tuple_impl;
+template <std::size_t... Is, class... Ts>
+struct tuple_impl<std::index_sequence<Is...>, Ts...> : tuple_leaf<Is, Ts>... {
+  tuple_impl() = default;
+  THRUST_CDNA4_HD constexpr tuple_impl(const Ts&... vs) : tuple_leaf<Is, Ts>{vs}... {}
+  template <class... Us>
+  THRUST_CDNA4_HD constexpr tuple_impl(const tuple_impl<std::index_sequence<Is...>, Us...>& o)
+      : tuple_leaf<Is, Ts>{static_cast<const tuple_leaf<Is, Us>&>(o).value}... {}
+  template <class... Us>
+  THRUST_CDNA4_HD void assign(const tuple_impl<std::index_sequence<Is...>, Us...>& o) {
+    int unused[] = {0, ((void)(static_cast<tuple_leaf<Is, Ts>&>(*this).value = static_cast<const tuple_leaf<Is, Us>&>(o).value), 0)...};
+    (void)unused;
+  }
+  template <class... Us>
+  THRUST_CDNA4_HD constexpr bool equals(const tuple_impl<std::index_sequence<Is...>, Us...>& o) const {
+    bool same = true;
+    int unused[] = {0, ((void)(same = same && (static_cast<const tuple_leaf<Is, Ts>&>(*this).value == static_cast<const tuple_leaf<Is, Us>&>(o).value)), 0)...};
+    (void)unused;
+    return same;
+  }
+};
+}  // namespace detail
+
+template <class... Ts>
+struct tuple : detail::tuple_impl<std::index_sequence_for<Ts...>, Ts...> {
+  typedef detail::tuple_impl<std::index_sequence_for<Ts...>, Ts...> base;
+  tuple() = default;
+  tuple(const tuple&) = default;
+  template <class... Us, class = typename std::enable_if<sizeof...(Us) == sizeof...(Ts) && (sizeof...(Ts) > 0) &&
+                                                         !detail::is_single_tuple<typename std::decay<Us>::type...>::value>::type>
+  THRUST_CDNA4_HD constexpr tuple(Us&&... vs) : base(static_cast<Us&&>(vs)...) {}
+  template <class... Us, class = typename std::enable_if<sizeof...(Us) == sizeof...(Ts)>::type>
+  THRUST_CDNA4_HD constexpr tuple(const tuple<Us...>& o) : base(static_cast<const typename tuple<Us...>::base&>(o)) {}
+  tuple& operator=(const tuple&) = default;
+  template <class... Us>
+  THRUST_CDNA4_HD tuple& operator=(const tuple<Us...>& o) {
+    base::assign(static_cast<const typename tuple<Us...>::base&>(o));
+    return *this;
+  }
+  // a tuple of references assigns through them, also when it is a temporary
+  template <class... Us>
+  THRUST_CDNA4_HD const tuple& operator=(const tuple<Us...>& o) const {
+    const_cast<tuple*>(this)->base::assign(static_cast<const typename tuple<Us...>::base&>(o));
+    return *this;
+  }
+};
+template <> struct tuple<> {};
+
+template <std::size_t I, class T> struct tuple_element;
+template <std::size_t I, class... Ts> struct tuple_element<I, tuple<Ts...>> { typedef typename detail::nth_type<I, Ts...>::type type; };
+template <std::size_t I, class T> struct tuple_element<I, const T> { typedef typename std::add_const<typename tuple_element<I, T>::type>::type type; };
+template <class T> struct tuple_size;
+template <class... Ts> struct tuple_size<tuple<Ts...>> : std::integral_constant<std::size_t, sizeof...(Ts)> {};
+template <class T> struct tuple_size<const T> : tuple_size<T> {};
+
+template <std::size_t I, class... Ts>
+THRUST_CDNA4_HD constexpr typename detail::nth_type<I, Ts...>::type& get(tuple<Ts...>& t) {
+  return static_cast<detail::tuple_leaf<I, typename detail::nth_type<I, Ts...>::type>&>(t).value;
+}
+template <std::size_t I, class... Ts>
+THRUST_CDNA4_HD constexpr const typename detail::nth_type<I, Ts...>::type& get(const tuple<Ts...>& t) {
+  return static_cast<const detail::tuple_leaf<I, typename detail::nth_type<I, Ts...>::type>&>(t).value;
+}
+template <class... Ts>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<Ts>::type...> make_tuple(const Ts&... vs) {
+  return tuple<typename std::decay<Ts>::type...>(vs...);
+}
+template <class... Ts>
+THRUST_CDNA4_HD constexpr tuple<Ts&...> tie(Ts&... vs) { return tuple<Ts&...>(vs...); }
+
+template <class... Ts, class... Us>
+THRUST_CDNA4_HD constexpr bool operator==(const tuple<Ts...>& a, const tuple<Us...>& b) {
+  return a.equals(static_cast<const typename tuple<Us...>::base&>(b));
+}
+template <class... Ts, class... Us>
+THRUST_CDNA4_HD constexpr bool operator!=(const tuple<Ts...>& a, const tuple<Us...>& b) { return !(a == b); }
+
+namespace detail {
+template <std::size_t I, std::size_t N> struct tuple_less {
+  template <class A, class B> THRUST_CDNA4_HD static constexpr bool run(const A& a, const B& b) {
+    return get<I>(a) < get<I>(b) ? true : get<I>(b) < get<I>(a) ? false : tuple_less<I + 1, N>::run(a, b);
+  }
+};
+template <std::size_t N> struct tuple_less<N, N> {
+  template <class A, class B> THRUST_CDNA4_HD static constexpr bool run(const A&, const B&) { return false; }
+};
+}  // namespace detail
+template <class... Ts, class... Us>
+THRUST_CDNA4_HD constexpr bool operator<(const tuple<Ts...>& a, const tuple<Us...>& b) {
+  return detail::tuple_less<0, sizeof...(Ts)>::run(a, b);
+}
+}  // namespace thrust

@@ -14,7 +14,7 @@ namespace thrust {
 template <class D, class In, class Out, class Eq>
 Out unique_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Eq eq) {
   typedef typename detail::value_of<In>::type V;
-  return out + system::cdna4::detail::unique_copy_n(exec.derived(), (const V*)detail::unwrap(first), detail::unwrap(out),
+  return out + system::cdna4::detail::unique_copy_n(exec.derived(), detail::unwrap(first), detail::unwrap(out),
                                                     (std::int64_t)(last - first), eq);
 }
 template <class D, class In, class Eq>
@@ -30,7 +30,7 @@ pair<KOut, VOut> unique_by_key_copy(const system::cdna4::execution_policy<D>& ex
   typedef typename detail::value_of<KIn>::type K;
   typedef typename detail::value_of<VIn>::type V;
   const std::int64_t c = system::cdna4::detail::unique_by_key_copy_n(
-      exec.derived(), (const K*)detail::unwrap(kfirst), (const V*)detail::unwrap(vfirst), detail::unwrap(kout),
+      exec.derived(), detail::unwrap(kfirst), detail::unwrap(vfirst), detail::unwrap(kout),
       detail::unwrap(vout), (std::int64_t)(klast - kfirst), eq);
   return thrust::make_pair(kout + c, vout + c);
 }
