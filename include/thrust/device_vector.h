@@ -9,18 +9,19 @@
 #include <initializer_list>
 #include <vector>
 
+#include <thrust/device_allocator.h>
 #include <thrust/device_ptr.h>
 #include <thrust/host_vector.h>
 
 namespace thrust {
 
-template <class T>
+template <class T, class Alloc>
 class device_vector {
   static_assert(std::is_trivially_copyable<T>::value, "device_vector of the cdna4 system holds trivially copyable types");
-  typedef system::cdna4::detail::temporary_storage storage_unused;
 
  public:
   typedef T value_type;
+  typedef Alloc allocator_type;
   typedef std::size_t size_type;
   typedef device_ptr<T> iterator;
   typedef device_ptr<const T> const_iterator;
@@ -28,11 +29,14 @@ class device_vector {
   typedef device_reference<T> reference;
   typedef device_reference<const T> const_reference;
 
-  device_vector() : p_(nullptr), n_(0), cap_(0) {}
+  device_vector() : p_(nullptr), n_(0), cap_(0), alloc_() {}
+  explicit device_vector(const Alloc& alloc) : p_(nullptr), n_(0), cap_(0), alloc_(alloc) {}
+  device_vector(size_type n, const T& v, const Alloc& alloc) : device_vector(alloc) { assign(n, v); }
+  allocator_type get_allocator() const { return alloc_; }
   explicit device_vector(size_type n) : device_vector() { resize(n); }
   device_vector(size_type n, const T& v) : device_vector() { assign(n, v); }
-  device_vector(const device_vector& o) : device_vector() { assign_device(o.p_, o.n_); }
-  device_vector(device_vector&& o) noexcept : p_(o.p_), n_(o.n_), cap_(o.cap_) { o.p_ = nullptr; o.n_ = o.cap_ = 0; }
+  device_vector(const device_vector& o) : device_vector(o.alloc_) { assign_device(o.p_, o.n_); }
+  device_vector(device_vector&& o) noexcept : p_(o.p_), n_(o.n_), cap_(o.cap_), alloc_(o.alloc_) { o.p_ = nullptr; o.n_ = o.cap_ = 0; }
   template <class A> device_vector(const std::vector<T, A>& h) : device_vector() { assign_host(h.data(), h.size()); }
   device_vector(std::initializer_list<T> il) : device_vector() { assign_host(il.begin(), il.size()); }
   template <class It, class = typename std::iterator_traits<It>::iterator_category>
@@ -60,7 +64,7 @@ class device_vector {
   reference back() { return (*this)[n_ - 1]; }
 
   void clear() { n_ = 0; }
-  void swap(device_vector& o) noexcept { std::swap(p_, o.p_); std::swap(n_, o.n_); std::swap(cap_, o.cap_); }
+  void swap(device_vector& o) noexcept { std::swap(p_, o.p_); std::swap(n_, o.n_); std::swap(cap_, o.cap_); std::swap(alloc_, o.alloc_); }
   void reserve(size_type c) { if (c > cap_) regrow(c); }
   void resize(size_type n) { resize(n, T()); }
   void resize(size_type n, const T& v) {
@@ -85,11 +89,11 @@ class device_vector {
  private:
   static void check(int rc, const char* what) { system::cdna4::detail::throw_on_error(rc, what); }
   static void sync() { check(thrust_cdna4_stream_synchronize(nullptr), "device_vector: synchronize"); }
-  void release() { if (p_) system::cdna4::detail::free_bytes(p_, nullptr); p_ = nullptr; n_ = cap_ = 0; }
+  void release() { if (p_) alloc_.deallocate(typename Alloc::pointer(p_), cap_); p_ = nullptr; n_ = cap_ = 0; }
   void regrow(size_type c) {
-    T* q = static_cast<T*>(system::cdna4::detail::malloc_bytes(c * sizeof(T), nullptr));
+    T* q = alloc_.allocate(c).get();
     if (n_) { check(thrust_cdna4_memcpy_dtod(q, p_, n_ * sizeof(T), nullptr), "device_vector: copy"); sync(); }
-    if (p_) system::cdna4::detail::free_bytes(p_, nullptr);
+    if (p_) alloc_.deallocate(typename Alloc::pointer(p_), cap_);
     p_ = q;
     cap_ = c;
   }
@@ -123,10 +127,12 @@ class device_vector {
 
   T* p_;
   size_type n_, cap_;
+  Alloc alloc_;
 };
 
 template <class T, class A>
-host_vector<T, A>::host_vector(const device_vector<T>& d) : base(d.size()) {
+template <class DA>
+host_vector<T, A>::host_vector(const device_vector<T, DA>& d) : base(d.size()) {
   if (d.size()) {
     system::cdna4::detail::throw_on_error(
         thrust_cdna4_memcpy_dtoh(this->data(), d.begin().get(), d.size() * sizeof(T), nullptr), "copy to host");
@@ -134,7 +140,8 @@ host_vector<T, A>::host_vector(const device_vector<T>& d) : base(d.size()) {
   }
 }
 template <class T, class A>
-host_vector<T, A>& host_vector<T, A>::operator=(const device_vector<T>& d) {
+template <class DA>
+host_vector<T, A>& host_vector<T, A>::operator=(const device_vector<T, DA>& d) {
   host_vector tmp(d);
   this->swap(tmp);
   return *this;

@@ -1,0 +1,174 @@
+// thrust::device_event / device_future / when_all (thrust/event.h, thrust/future.h;
+// thrust/system/cuda/detail/future.inl:691-960, :1349-): the handle an asynchronous algorithm
+// returns.  An event owns the stream its work was submitted to; ready() polls it, wait() blocks
+// on it, and the destructor waits, so work never outlives the handle (as in the reference).  A
+// future also owns the device storage of its result; get() waits and reads it back once.
+#pragma once
+#include <memory>
+#include <stdexcept>
+#include <type_traits>
+#include <utility>
+#include <vector>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/core.h>
+
+namespace thrust {
+namespace system { namespace cdna4 { namespace detail {
+// The state shared by an event and the events that depend on it: a stream of its own, plus
+// whatever must stay alive until the stream's work is done.
+class async_signal {
+ public:
+  async_signal() : stream_(nullptr), submitted_(nullptr) { throw_on_error(thrust_cdna4_stream_create(&stream_), "async: stream"); }
+  ~async_signal() {
+    (void)thrust_cdna4_stream_synchronize(stream_);
+    keep_.clear();
+    if (submitted_) (void)thrust_cdna4_event_destroy(submitted_);
+    (void)thrust_cdna4_stream_destroy(stream_);
+  }
+  async_signal(const async_signal&) = delete;
+  async_signal& operator=(const async_signal&) = delete;
+  void* stream() const { return stream_; }
+  // Called once everything has been submitted: ready() then polls an event recorded behind the
+  // work (a stream that holds only a wait on another stream's event does not answer a stream
+  // query reliably).
+  void mark_submitted() {
+    if (!submitted_) throw_on_error(thrust_cdna4_event_create(&submitted_), "async: event");
+    throw_on_error(thrust_cdna4_event_record(submitted_, stream_), "async: record");
+  }
+  bool ready() const {
+    int done = 0;
+    if (submitted_) throw_on_error(thrust_cdna4_event_query(submitted_, &done), "async: query");
+    else throw_on_error(thrust_cdna4_stream_query(stream_, &done), "async: query");
+    return done != 0;
+  }
+  void wait() const { throw_on_error(thrust_cdna4_stream_synchronize(stream_), "async: wait"); }
+  // this stream's later work starts after everything submitted so far to `other`
+  void depend_on(const async_signal& other) {
+    void* e = nullptr;
+    throw_on_error(thrust_cdna4_event_create(&e), "async: event");
+    int rc = thrust_cdna4_event_record(e, other.stream_);
+    if (rc == 0) rc = thrust_cdna4_stream_wait_event(stream_, e);
+    (void)thrust_cdna4_event_destroy(e);  // the wait already holds what it needs
+    throw_on_error(rc, "async: dependency");
+  }
+  void keep_alive(std::shared_ptr<void> p) { keep_.push_back(std::move(p)); }
+ private:
+  void* stream_;
+  void* submitted_;
+  std::vector<std::shared_ptr<void>> keep_;
+};
+}}}  // namespace system::cdna4::detail
+
+struct new_stream_t {};
+static const new_stream_t new_stream = {};
+
+class device_event {
+ public:
+  device_event() = default;  // no state
+  explicit device_event(new_stream_t) : signal_(std::make_shared<system::cdna4::detail::async_signal>()) {}
+  // takes over a signal whose work has all been submitted
+  explicit device_event(std::shared_ptr<system::cdna4::detail::async_signal> s) : signal_(std::move(s)) {
+    if (signal_) signal_->mark_submitted();
+  }
+  device_event(device_event&&) = default;
+  device_event& operator=(device_event&& o) {
+    if (this != &o) {
+      if (valid_stream()) wait();
+      signal_ = std::move(o.signal_);
+    }
+    return *this;
+  }
+  device_event(const device_event&) = delete;
+  device_event& operator=(const device_event&) = delete;
+  ~device_event() {
+    if (valid_stream()) (void)thrust_cdna4_stream_synchronize(signal_->stream());
+  }
+  bool valid_stream() const { return bool(signal_); }
+  bool ready() const { return valid_stream() && signal_->ready(); }
+  void wait() const { state().wait(); }
+  void* stream() const { return state().stream(); }  // the native stream handle
+  const std::shared_ptr<system::cdna4::detail::async_signal>& signal() const { return signal_; }
+ protected:
+  system::cdna4::detail::async_signal& state() const {
+    if (!signal_) throw std::logic_error("thrust::device_event: no state");
+    return *signal_;
+  }
+  std::shared_ptr<system::cdna4::detail::async_signal> signal_;
+};
+
+template <class T>
+class device_future : public device_event {
+  static_assert(std::is_trivially_copyable<T>::value, "device_future: the value type must be trivially copyable");
+ public:
+  typedef T value_type;
+  device_future() : data_(nullptr), have_(false) {}
+  // the signal keeps the storage alive; data points into it
+  device_future(std::shared_ptr<system::cdna4::detail::async_signal> s, T* data) : device_event(std::move(s)), data_(data), have_(false) {}
+  device_future(device_future&&) = default;
+  device_future& operator=(device_future&&) = default;
+  bool valid_content() const { return data_ != nullptr || have_; }
+  // waits for the work, reads the value back (once) and returns it
+  T get() {
+    if (!have_) {
+      if (!data_) throw std::logic_error("thrust::device_future: no state");
+      wait();
+      system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_dtoh(&value_, data_, sizeof(T), stream()), "future: read back");
+      wait();
+      have_ = true;
+    }
+    return value_;
+  }
+  T extract() {
+    T v = get();
+    data_ = nullptr;
+    have_ = false;
+    signal_.reset();
+    return v;
+  }
+  T* raw_data() const { return data_; }  // the device address of the result
+ private:
+  T* data_;
+  T value_;
+  bool have_;
+};
+
+namespace system { namespace cdna4 { namespace detail {
+// thrust::device.after(events...): the next asynchronous algorithm starts after these
+struct execute_after : execution_policy<execute_after> {
+  std::vector<std::shared_ptr<async_signal>> deps;
+};
+inline void collect(execute_after&) {}
+template <class E, class... Es>
+void collect(execute_after& p, E&& e, Es&&... es) {
+  if (e.valid_stream()) p.deps.push_back(e.signal());
+  collect(p, std::forward<Es>(es)...);
+}
+// a fresh signal whose stream waits for the dependencies and keeps them alive
+inline std::shared_ptr<async_signal> make_signal(const execute_after& p) {
+  auto s = std::make_shared<async_signal>();
+  for (const auto& d : p.deps) {
+    s->depend_on(*d);
+    s->keep_alive(d);
+  }
+  return s;
+}
+inline std::shared_ptr<async_signal> make_signal(const par_t&) { return std::make_shared<async_signal>(); }
+inline std::shared_ptr<async_signal> make_signal(const par_nosync_t&) { return std::make_shared<async_signal>(); }
+}}}  // namespace system::cdna4::detail
+
+namespace system { namespace cdna4 { namespace detail {
+template <class... Events>
+execute_after par_t::after(Events&&... events) const {
+  execute_after p;
+  collect(p, std::forward<Events>(events)...);
+  return p;
+}
+}}}  // namespace system::cdna4::detail
+// an event that is ready when all of the given ones are
+template <class... Events>
+device_event when_all(Events&&... events) {
+  system::cdna4::detail::execute_after p;
+  system::cdna4::detail::collect(p, std::forward<Events>(events)...);
+  return device_event(system::cdna4::detail::make_signal(p));
+}
+}  // namespace thrust

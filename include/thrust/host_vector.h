@@ -2,7 +2,8 @@
 #pragma once
 #include <vector>
 namespace thrust {
-template <class T> class device_vector;
+template <class T> class device_allocator;
+template <class T, class Alloc = device_allocator<T>> class device_vector;
 template <class T, class Alloc = std::allocator<T>>
 class host_vector : public std::vector<T, Alloc> {
   typedef std::vector<T, Alloc> base;
@@ -11,7 +12,7 @@ class host_vector : public std::vector<T, Alloc> {
   using base::base;
   host_vector() = default;
   host_vector(const base& v) : base(v) {}
-  host_vector(const device_vector<T>& d);
-  host_vector& operator=(const device_vector<T>& d);
+  template <class DA> host_vector(const device_vector<T, DA>& d);
+  template <class DA> host_vector& operator=(const device_vector<T, DA>& d);
 };
 }  // namespace thrust

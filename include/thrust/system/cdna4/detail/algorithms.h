@@ -28,7 +28,7 @@ void sort_keys_impl(const Policy& exec, K* keys, std::int64_t n, Compare, std::t
   std::size_t bytes = 0;
   throw_on_error(thrust_cdna4_sort_keys(nullptr, &bytes, dtype_of<K>::value, keys, n, order_code<Compare>::value, s),
                  "sort: temporary storage query");
-  temporary_storage tmp(bytes, s);
+  temporary_storage tmp(bytes, exec);
   throw_on_error(thrust_cdna4_sort_keys(tmp.data(), &bytes, dtype_of<K>::value, keys, n, order_code<Compare>::value, s),
                  "sort: launch");
 }
@@ -57,7 +57,7 @@ void sort_pairs_impl(const Policy& exec, K* keys, V* values, std::int64_t n, Com
   std::size_t bytes = 0;
   throw_on_error(thrust_cdna4_sort_pairs(nullptr, &bytes, dtype_of<K>::value, keys, (int)sizeof(V), values, n,
                                          order_code<Compare>::value, s), "sort_by_key: temporary storage query");
-  temporary_storage tmp(bytes, s);
+  temporary_storage tmp(bytes, exec);
   throw_on_error(thrust_cdna4_sort_pairs(tmp.data(), &bytes, dtype_of<K>::value, keys, (int)sizeof(V), values, n,
                                          order_code<Compare>::value, s), "sort_by_key: launch");
 }
@@ -92,7 +92,7 @@ void scan(const Policy& exec, const T* in, T* out, std::int64_t n, bool exclusiv
   std::size_t bytes = 0;
   throw_on_error(thrust_cdna4_scan(nullptr, &bytes, dtype_of<T>::value, op_code<Op>::value, exclusive, in, out, n, init, s),
                  "scan: temporary storage query");
-  temporary_storage tmp(bytes, s);
+  temporary_storage tmp(bytes, exec);
   throw_on_error(thrust_cdna4_scan(tmp.data(), &bytes, dtype_of<T>::value, op_code<Op>::value, exclusive, in, out, n, init, s),
                  "scan: launch");
   synchronize_optional(exec, "scan: failed to synchronize");
@@ -109,7 +109,7 @@ void scan_by_key(const Policy& exec, const K* keys, const T* in, T* out, std::in
   std::size_t bytes = 0;
   throw_on_error(thrust_cdna4_scan_by_key(nullptr, &bytes, dtype_of<K>::value, dtype_of<T>::value, op_code<Op>::value,
                                           exclusive, keys, in, out, n, init, s), "scan_by_key: temporary storage query");
-  temporary_storage tmp(bytes, s);
+  temporary_storage tmp(bytes, exec);
   throw_on_error(thrust_cdna4_scan_by_key(tmp.data(), &bytes, dtype_of<K>::value, dtype_of<T>::value, op_code<Op>::value,
                                           exclusive, keys, in, out, n, init, s), "scan_by_key: launch");
   synchronize_optional(exec, "scan_by_key: failed to synchronize");
@@ -129,7 +129,7 @@ std::int64_t reduce_by_key(const Policy& exec, const K* keys, const T* vals, K* 
   throw_on_error(thrust_cdna4_reduce_by_key(nullptr, &bytes, dtype_of<K>::value, dtype_of<T>::value, op_code<Op>::value,
                                             keys, vals, keys_out, vals_out, nullptr, n, s),
                  "reduce_by_key: temporary storage query");
-  temporary_storage tmp(bytes + 256, s);  // + the run counter
+  temporary_storage tmp(bytes + 256, exec);  // + the run counter
   std::int64_t* d_runs = reinterpret_cast<std::int64_t*>(static_cast<char*>(tmp.data()) + bytes);
   throw_on_error(thrust_cdna4_reduce_by_key(tmp.data(), &bytes, dtype_of<K>::value, dtype_of<T>::value, op_code<Op>::value,
                                             keys, vals, keys_out, vals_out, d_runs, n, s), "reduce_by_key: launch");

@@ -12,6 +12,7 @@
 #pragma once
 
 #include <cstddef>
+#include <utility>
 #include <cstdint>
 #include <new>
 #include <string>
@@ -89,14 +90,34 @@ struct execute_on_stream : execution_policy<execute_on_stream> {
 
 // thrust::device / thrust::cdna4::par: work goes to the legacy default stream and the call
 // returns after it has completed (thrust/system/cuda/detail/util.h:46-55, :113-140).
+struct execute_after;  // thrust/event.h
+template <class Alloc> struct execute_with_allocator;
 struct par_t : execution_policy<par_t> {
   execute_on_stream on(void* stream) const { return execute_on_stream(stream, true); }
+  // thrust::device.after(events...): policy of an asynchronous algorithm that starts after them
+  // (defined in thrust/event.h)
+  template <class... Events> execute_after after(Events&&... events) const;
+  template <class Alloc> execute_with_allocator<Alloc> operator()(Alloc& alloc) const;
 };
 // par_nosync: the call may return before the work has completed, except where a result has
 // to be read back (thrust/system/cuda/detail/par.h:102-107, :181-186).
 struct par_nosync_t : execution_policy<par_nosync_t> {
   execute_on_stream on(void* stream) const { return execute_on_stream(stream, false); }
 };
+
+// thrust::cdna4::par(alloc): temporary storage of the algorithm comes from the user's allocator
+// (allocate(n) / deallocate(p, n) in units of its value_type) instead of the library's pool
+// (thrust/system/cuda/detail/par.h:43-76, examples/cuda/custom_temporary_allocation.cu).
+template <class Alloc>
+struct execute_with_allocator : execution_policy<execute_with_allocator<Alloc>> {
+  Alloc& alloc_;
+  void* stream_;
+  bool sync_;
+  execute_with_allocator(Alloc& a, void* s, bool sync) : alloc_(a), stream_(s), sync_(sync) {}
+  execute_with_allocator on(void* stream) const { return execute_with_allocator(alloc_, stream, sync_); }
+};
+template <class Alloc> inline void* stream_of(const execute_with_allocator<Alloc>& p) { return p.stream_; }
+template <class Alloc> inline bool must_sync(const execute_with_allocator<Alloc>& p) { return p.sync_; }
 
 inline void* stream_of(const par_t&) { return nullptr; }
 inline void* stream_of(const par_nosync_t&) { return nullptr; }
@@ -160,14 +181,41 @@ inline void* malloc_bytes(std::size_t bytes, void* stream) {
 }
 inline void free_bytes(void* p, void* stream) noexcept { (void)thrust_cdna4_free(p, stream); }
 
+template <class Alloc>
+execute_with_allocator<Alloc> par_t::operator()(Alloc& alloc) const { return execute_with_allocator<Alloc>(alloc, nullptr, true); }
+
+// raw address of what an allocator returned (a raw pointer or a pointer-like object with get())
+template <class T> inline void* address_of_allocation(T* p) { return const_cast<typename std::remove_const<T>::type*>(p); }
+template <class P> inline auto address_of_allocation(const P& p) -> decltype((void*)p.get()) { return (void*)p.get(); }
+
 // Byte buffer that lives for one algorithm call (thrust::detail::temporary_array<uint8_t>).
+// It comes from the library's stream-ordered pool, or from the policy's allocator.
 class temporary_storage {
  public:
-  temporary_storage(std::size_t bytes, void* stream) : stream_(stream), bytes_(bytes), ptr_(nullptr) {
+  temporary_storage(std::size_t bytes, void* stream) : stream_(stream), bytes_(bytes), ptr_(nullptr), user_(nullptr), release_(nullptr) {
     if (bytes_) ptr_ = malloc_bytes(bytes_, stream_);
   }
+  template <class Policy>
+  temporary_storage(std::size_t bytes, const Policy& exec) : temporary_storage(bytes, stream_of(exec)) {}
+  template <class Alloc>
+  temporary_storage(std::size_t bytes, const execute_with_allocator<Alloc>& exec)
+      : stream_(exec.stream_), bytes_(bytes), ptr_(nullptr), user_(&exec.alloc_), release_(nullptr) {
+    typedef typename Alloc::value_type V;
+    if (bytes_) {
+      const std::size_t count = (bytes_ + sizeof(V) - 1) / sizeof(V);
+      ptr_ = address_of_allocation(exec.alloc_.allocate(count));
+      release_ = [](void* alloc, void* p, std::size_t n, void* stream) {
+        // the allocator may hand the block out again at once: wait for the work that uses it
+        (void)thrust_cdna4_stream_synchronize(stream);
+        typedef decltype(std::declval<Alloc&>().allocate(1)) pointer;
+        static_cast<Alloc*>(alloc)->deallocate(pointer(static_cast<V*>(p)), (n + sizeof(V) - 1) / sizeof(V));
+      };
+    }
+  }
   ~temporary_storage() {
-    if (ptr_) free_bytes(ptr_, stream_);
+    if (!ptr_) return;
+    if (release_) release_(user_, ptr_, bytes_, stream_);
+    else free_bytes(ptr_, stream_);
   }
   temporary_storage(const temporary_storage&) = delete;
   temporary_storage& operator=(const temporary_storage&) = delete;
@@ -178,6 +226,8 @@ class temporary_storage {
   void* stream_;
   std::size_t bytes_;
   void* ptr_;
+  void* user_;
+  void (*release_)(void* alloc, void* p, std::size_t bytes, void* stream);
 };
 
 }  // namespace detail

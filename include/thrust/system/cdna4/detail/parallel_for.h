@@ -86,6 +86,10 @@ __global__ __launch_bounds__(kBlock) void reduce_partials_kernel(std::int64_t n,
 // out[0] = op(init, partial[0] (+) ... (+) partial[count-1])
 template <class T, class Op>
 __global__ __launch_bounds__(kBlock) void reduce_final_kernel(const T* partial, int count, T init, Op op, T* out) {
+  if (count <= 0) {  // an empty range reduces to init
+    if (threadIdx.x == 0) out[0] = init;
+    return;
+  }
   T acc{};
   int i = threadIdx.x;
   if (i < count) {
@@ -94,6 +98,23 @@ __global__ __launch_bounds__(kBlock) void reduce_final_kernel(const T* partial, 
   }
   acc = block_reduce(acc, count < kBlock ? count : kBlock, op);
   if (threadIdx.x == 0) out[0] = op(init, acc);
+}
+
+// Stores op(init, unary(0) (+) ... (+) unary(n-1)) at device address out, in stream order and
+// without waiting (the asynchronous reductions; n == 0 stores init).
+template <class T, class Unary, class Op>
+void transform_reduce_into(void* stream_, std::int64_t n, Unary unary, T init, Op op, T* out) {
+  static_assert(std::is_trivially_copyable<T>::value, "cdna4 reduce: the result type must be trivially copyable");
+  hipStream_t s = static_cast<hipStream_t>(stream_);
+  std::int64_t blocks = (n + kBlock - 1) / kBlock;
+  const std::int64_t enough = 2048;
+  if (blocks > enough) blocks = enough;
+  temporary_storage tmp((std::size_t)(blocks > 0 ? blocks : 1) * sizeof(T), stream_);
+  T* partial = static_cast<T*>(tmp.data());
+  if (blocks > 0)
+    hipLaunchKernelGGL((reduce_partials_kernel<T, Unary, Op>), dim3((unsigned)blocks), dim3(kBlock), 0, s, n, unary, op, partial);
+  hipLaunchKernelGGL((reduce_final_kernel<T, Op>), dim3(1), dim3(kBlock), 0, s, partial, (int)blocks, init, op, out);
+  throw_on_error((int)hipGetLastError(), "reduce: launch");
 }
 
 // Returns op(init, unary(0) (+) ... (+) unary(n-1)); blocks until the value is on the host

@@ -21,7 +21,7 @@ void histogram_even(const thrust::system::cdna4::execution_policy<D>& exec, It f
   d::throw_on_error(thrust_cdna4_histogram_even(nullptr, &bytes, d::dtype_of<T>::value, thrust::detail::unwrap(first),
                                                 (std::int64_t)(last - first), nullptr, num_bins, lower, upper, s),
                     "histogram_even: temporary storage query");
-  d::temporary_storage tmp(bytes, s);
+  d::temporary_storage tmp(bytes, exec.derived());
   d::throw_on_error(thrust_cdna4_histogram_even(tmp.data(), &bytes, d::dtype_of<T>::value, thrust::detail::unwrap(first),
                                                 (std::int64_t)(last - first),
                                                 reinterpret_cast<std::uint32_t*>(thrust::detail::unwrap(counts)), num_bins,

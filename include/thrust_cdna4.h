@@ -160,6 +160,32 @@ int thrust_cdna4_fill(void* dst, const void* value, int elem_bytes, int64_t n, v
 int thrust_cdna4_stream_synchronize(void* stream);
 
 /*
+ * Streams and events behind thrust::async::* / device_event / device_future
+ * (thrust/system/cuda/detail/future.inl:60-300: unique_stream, unique_event, ready(), wait(),
+ * depend_on(), record()).  A created stream does not synchronise with the default stream and
+ * has the default priority.  stream_query / event_query store 1 in *done when all work submitted
+ * to the stream / before the event's record has completed, else 0; work still running is not an
+ * error.  (A stream that holds nothing but a wait on an event can keep answering 0 after it
+ * has been synchronised; an event recorded behind the wait answers correctly, which is what
+ * device_event::ready() polls.)
+ */
+int thrust_cdna4_stream_create(void** stream);
+int thrust_cdna4_stream_destroy(void* stream);
+int thrust_cdna4_stream_query(void* stream, int* done);
+int thrust_cdna4_event_create(void** event);
+int thrust_cdna4_event_destroy(void* event);
+int thrust_cdna4_event_record(void* event, void* stream);
+int thrust_cdna4_event_query(void* event, int* done);
+int thrust_cdna4_stream_wait_event(void* stream, void* event);
+/*
+ * Device memory straight from the driver (hipMalloc / hipFree), bypassing the pool: the
+ * upstream resource of thrust::mr pools built by users
+ * (thrust/system/cuda/memory_resource.h:46-100, cuda_memory_resource<cudaMalloc, cudaFree>).
+ */
+int thrust_cdna4_malloc_direct(void** ptr, size_t bytes);
+int thrust_cdna4_free_direct(void* ptr);
+
+/*
  * Launch profiling.  While enabled, every kernel the library launches is bracketed by HIP
  * events recorded on the launch stream and logged under its kernel name; enable(…) also
  * clears the log.  get() waits for record `index` and returns its name and duration in

@@ -22,6 +22,9 @@ SYMBOLS = [
     "thrust_cdna4_fill", "thrust_cdna4_stream_synchronize", "thrust_cdna4_profile_enable",
     "thrust_cdna4_profile_count", "thrust_cdna4_profile_get",
     "thrust_cdna4_selftest_lds_atomic_order",
+    "thrust_cdna4_stream_create", "thrust_cdna4_stream_destroy", "thrust_cdna4_stream_query",
+    "thrust_cdna4_event_create", "thrust_cdna4_event_destroy", "thrust_cdna4_event_record", "thrust_cdna4_event_query",
+    "thrust_cdna4_stream_wait_event", "thrust_cdna4_malloc_direct", "thrust_cdna4_free_direct",
 ]
 
 
@@ -65,6 +68,16 @@ def lib():
     L.thrust_cdna4_memcpy_dtod.argtypes = [vp, vp, sz, vp]
     L.thrust_cdna4_fill.argtypes = [vp, vp, i32, i64, vp]
     L.thrust_cdna4_stream_synchronize.argtypes = [vp]
+    L.thrust_cdna4_stream_create.argtypes = [ctypes.POINTER(vp)]
+    L.thrust_cdna4_stream_destroy.argtypes = [vp]
+    L.thrust_cdna4_stream_query.argtypes = [vp, ctypes.POINTER(ctypes.c_int)]
+    L.thrust_cdna4_event_create.argtypes = [ctypes.POINTER(vp)]
+    L.thrust_cdna4_event_destroy.argtypes = [vp]
+    L.thrust_cdna4_event_record.argtypes = [vp, vp]
+    L.thrust_cdna4_event_query.argtypes = [vp, ctypes.POINTER(ctypes.c_int)]
+    L.thrust_cdna4_stream_wait_event.argtypes = [vp, vp]
+    L.thrust_cdna4_malloc_direct.argtypes = [ctypes.POINTER(vp), sz]
+    L.thrust_cdna4_free_direct.argtypes = [vp]
     L.thrust_cdna4_profile_enable.argtypes = [i32]
     L.thrust_cdna4_selftest_lds_atomic_order.argtypes = [ctypes.POINTER(ctypes.c_longlong), vp]
     L.thrust_cdna4_profile_get.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p),

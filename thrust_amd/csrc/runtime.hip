@@ -304,3 +304,68 @@ extern "C" int thrust_cdna4_fill(void* dst, const void* value, int elem_bytes, i
 extern "C" int thrust_cdna4_stream_synchronize(void* stream) {
   return hipStreamSynchronize(static_cast<hipStream_t>(stream));
 }
+
+// Streams and events for the asynchronous algorithms.  Streams are non-blocking (they do not
+// synchronise with the legacy default stream) and keep the default priority; events carry no
+// timing.
+extern "C" int thrust_cdna4_stream_create(void** stream) {
+  if (!stream) return hipErrorInvalidValue;
+  hipStream_t s = nullptr;
+  const hipError_t rc = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);
+  *stream = s;
+  return rc;
+}
+extern "C" int thrust_cdna4_stream_destroy(void* stream) {
+  if (!stream) return hipErrorInvalidValue;  // the default stream is not the library's to destroy
+  return hipStreamDestroy(static_cast<hipStream_t>(stream));
+}
+extern "C" int thrust_cdna4_stream_query(void* stream, int* done) {
+  if (!done) return hipErrorInvalidValue;
+  const hipError_t rc = hipStreamQuery(static_cast<hipStream_t>(stream));
+  *done = rc == hipSuccess;
+  if (rc == hipErrorNotReady) {
+    (void)hipGetLastError();  // not an error: work is still running
+    return hipSuccess;
+  }
+  return rc;
+}
+extern "C" int thrust_cdna4_event_create(void** event) {
+  if (!event) return hipErrorInvalidValue;
+  hipEvent_t e = nullptr;
+  const hipError_t rc = hipEventCreateWithFlags(&e, hipEventDisableTiming);
+  *event = e;
+  return rc;
+}
+extern "C" int thrust_cdna4_event_destroy(void* event) {
+  if (!event) return hipErrorInvalidValue;
+  return hipEventDestroy(static_cast<hipEvent_t>(event));
+}
+extern "C" int thrust_cdna4_event_record(void* event, void* stream) {
+  if (!event) return hipErrorInvalidValue;
+  return hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream));
+}
+extern "C" int thrust_cdna4_event_query(void* event, int* done) {
+  if (!event || !done) return hipErrorInvalidValue;
+  const hipError_t rc = hipEventQuery(static_cast<hipEvent_t>(event));
+  *done = rc == hipSuccess;
+  if (rc == hipErrorNotReady) {
+    (void)hipGetLastError();
+    return hipSuccess;
+  }
+  return rc;
+}
+extern "C" int thrust_cdna4_stream_wait_event(void* stream, void* event) {
+  if (!event) return hipErrorInvalidValue;
+  return hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0);
+}
+// Plain device memory from the driver, without the pool: the upstream of user-built pools.
+extern "C" int thrust_cdna4_malloc_direct(void** ptr, size_t bytes) {
+  if (!ptr) return hipErrorInvalidValue;
+  *ptr = nullptr;
+  if (bytes == 0) return hipSuccess;
+  return hipMalloc(ptr, bytes);
+}
+extern "C" int thrust_cdna4_free_direct(void* ptr) {
+  if (!ptr) return hipSuccess;
+  return hipFree(ptr);
+}
