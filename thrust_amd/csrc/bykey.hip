@@ -103,15 +103,38 @@ __device__ inline void store_group(E* p, const E (&src)[N]) {
   }
 }
 
-// Tile geometry: a thread owns VEC consecutive elements of each of CHUNKS chunks; the wider of
-// key and value fills GROUP_BYTES per thread and chunk, capped at 16 elements.  Measured on
-// MI355X, 16-byte groups (one 128-bit access; every wave access is one contiguous 1 KiB
-// segment) with 8 chunks beat 32- and 64-byte groups for both kernels.
-template <class T, int GROUP_BYTES, int CHUNKS_>
-struct SegGeom {
+// Tile geometry.  Two layouts exist; the blocked one is the default.  (The striped one, kept for
+// comparison with -DTCD_SEG_BLOCKED=0: a thread owns VEC consecutive elements of each of CHUNKS
+// chunks, the wider of key and value fills GROUP_BYTES per thread and chunk; 16-byte groups with
+// 8 chunks beat 32- and 64-byte groups.  On MI355X at 2^28 int32 pairs it is 2 % faster when every
+// element is a run of its own and 3-5 % slower at mean run lengths 8 and 512.)
+#ifndef TCD_SEG_BLOCKED
+#define TCD_SEG_BLOCKED 1
+#endif
 #ifndef TCD_SEG_BLOCK
 #define TCD_SEG_BLOCK 512
 #endif
+#if TCD_SEG_BLOCKED
+// Blocked tiles: a thread owns VEC consecutive elements (128 bytes of the wider of key and
+// value, at most 32 elements), a wavefront 64 * VEC consecutive ones.  Global memory is read
+// and written in wave-wide contiguous 1 KiB accesses and transposed to the blocked order through
+// a wave-private LDS buffer, so one sequential walk per thread and ONE wavefront scan per tile
+// replace a scan per 16-byte group: a third of the vector instructions of the striped layout.
+template <class T, int GROUP_BYTES, int CHUNKS_>
+struct SegGeom {
+  static constexpr bool BLOCKED = true;
+  static constexpr int BLOCK = TCD_SEG_BLOCK;
+  static constexpr int WIDE = (int)(sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T));
+  static constexpr int VEC = WIDE == 8 ? 16 : 32;
+  static constexpr int CHUNKS = 1;
+  static constexpr int NWAVES = BLOCK / kWave;
+  static constexpr int64_t TILE = (int64_t)BLOCK * VEC;
+  static constexpr int XPOSE_SLOTS = 512;  // 16-byte slots of a wavefront's transpose buffer (8 KiB)
+};
+#else
+template <class T, int GROUP_BYTES, int CHUNKS_>
+struct SegGeom {
+  static constexpr bool BLOCKED = false;
   static constexpr int BLOCK = TCD_SEG_BLOCK;
   static constexpr int WIDE = (int)(sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T));
   static constexpr int VEC = GROUP_BYTES / WIDE > 16 ? 16 : GROUP_BYTES / WIDE;
@@ -119,7 +142,57 @@ struct SegGeom {
   static constexpr int CHUNKS = VEC * CHUNKS_ > 32 ? 32 / VEC : CHUNKS_;
   static constexpr int NWAVES = BLOCK / kWave;
   static constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
+  static constexpr int XPOSE_SLOTS = 1;
 };
+#endif
+
+// Orders a wavefront's LDS accesses around an exchange through its private buffer (the LDS
+// executes one wavefront's instructions in order; this keeps the compiler from reordering them).
+__device__ inline void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+// 16-byte slot s of a wavefront's buffer lives at slot xpose_slot(s): both the striped order
+// (slot q * 64 + lane) and the blocked order (slot lane * NQ + i) then spread over all banks.
+__device__ inline int xpose_slot(int s) { return s ^ ((s >> 3) & 7); }
+
+// The wavefront's 64 * VEC consecutive elements at src (16-byte aligned): lane l receives
+// elements [l * VEC, (l + 1) * VEC).  Every global access is one contiguous 1 KiB per wavefront.
+template <int VEC, class E>
+__device__ inline void wave_load_blocked(const E* src, E (&dst)[VEC], tcd_v4u* buf, int lane) {
+  constexpr int NQ = VEC * (int)sizeof(E) / 16;
+  static_assert(NQ >= 1 && NQ * 16 == VEC * (int)sizeof(E), "a thread's elements are whole 16-byte slots");
+  tcd_v4u t[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; q++) t[q] = load16<tcd_v4u>(reinterpret_cast<const char*>(src) + (q * kWave + lane) * 16);
+#pragma unroll
+  for (int q = 0; q < NQ; q++) buf[xpose_slot(q * kWave + lane)] = t[q];
+  wave_lds_sync();
+#pragma unroll
+  for (int i = 0; i < NQ; i++) {
+    const tcd_v4u r = buf[xpose_slot(lane * NQ + i)];
+    __builtin_memcpy(reinterpret_cast<char*>(dst) + 16 * i, &r, 16);
+  }
+  wave_lds_sync();
+}
+// The inverse: lane l's VEC consecutive elements go to dst[l * VEC ...], written as contiguous
+// 1 KiB accesses.
+template <int VEC, class E>
+__device__ inline void wave_store_blocked(E* dst, const E (&src)[VEC], tcd_v4u* buf, int lane) {
+  constexpr int NQ = VEC * (int)sizeof(E) / 16;
+  static_assert(NQ >= 1 && NQ * 16 == VEC * (int)sizeof(E), "a thread's elements are whole 16-byte slots");
+#pragma unroll
+  for (int i = 0; i < NQ; i++) {
+    tcd_v4u r;
+    __builtin_memcpy(&r, reinterpret_cast<const char*>(src) + 16 * i, 16);
+    buf[xpose_slot(lane * NQ + i)] = r;
+  }
+  wave_lds_sync();
+#pragma unroll
+  for (int q = 0; q < NQ; q++) store16(reinterpret_cast<char*>(dst) + (q * kWave + lane) * 16, buf[xpose_slot(q * kWave + lane)]);
+  wave_lds_sync();
+}
 #ifndef TCD_SBK_GROUP
 #define TCD_SBK_GROUP 16
 #endif
@@ -165,8 +238,9 @@ struct SegTile {
 
   __device__ static Pair comb(const Pair& a, const Pair& b) { return seg_combine<T, Op>(a, b); }
 
+  // xbuf: the wavefront's transpose buffer (blocked geometry only)
   __device__ void run(Smem& sm, const KU* keys, const T* vals, int64_t n, int float_keys, int vec_ok,
-                      uint64_t* desc, uint32_t* ticket) {
+                      uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -180,11 +254,17 @@ struct SegTile {
     full = vec_ok && (base + G::TILE < n);
 
     if (full) {
+      if constexpr (G::BLOCKED) {
+        const int64_t w0 = base + (int64_t)wave * (kWave * VEC);
+        wave_load_blocked<VEC>(keys + w0, key[0], xbuf, lane);
+        wave_load_blocked<VEC>(vals + w0, val[0], xbuf, lane);
+      } else {
 #pragma unroll
-      for (int c = 0; c < CHUNKS; c++) {
-        const int64_t i0 = index(c, 0);
-        load_group<VEC>(keys + i0, key[c]);
-        load_group<VEC>(vals + i0, val[c]);
+        for (int c = 0; c < CHUNKS; c++) {
+          const int64_t i0 = index(c, 0);
+          load_group<VEC>(keys + i0, key[c]);
+          load_group<VEC>(vals + i0, val[c]);
+        }
       }
     } else {
 #pragma unroll
@@ -261,10 +341,13 @@ template <class T, class Op>
 __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_key_kernel(
     const KU* keys, const T* vals, T* out, int64_t n, T init, int exclusive, int float_keys, int vec_ok,
     uint64_t* desc, uint32_t* ticket) {
-  using ST = SegTile<T, Op, ScanByKeyGeom<T>>;
+  using G = ScanByKeyGeom<T>;
+  using ST = SegTile<T, Op, G>;
   __shared__ typename ST::Smem sm;
+  __shared__ tcd_v4u s_x[G::BLOCKED ? G::NWAVES : 1][G::XPOSE_SLOTS];
+  tcd_v4u* xbuf = s_x[G::BLOCKED ? threadIdx.x / kWave : 0];
   ST t;
-  t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket);
+  t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf);
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS;
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
@@ -280,7 +363,10 @@ __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_
     }
     const int64_t i0 = t.index(c, 0);
     if (t.full) {
-      store_group<VEC>(out + i0, r);
+      if constexpr (G::BLOCKED)
+        wave_store_blocked<VEC>(out + t.base + (int64_t)(threadIdx.x / kWave) * (kWave * VEC), r, xbuf, threadIdx.x & (kWave - 1));
+      else
+        store_group<VEC>(out + i0, r);
     } else {
 #pragma unroll
       for (int j = 0; j < VEC; j++)
@@ -296,19 +382,76 @@ template <class T, class Op>
 __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce_by_key_kernel(
     const KU* keys, const T* vals, KU* keys_out, T* vals_out, int64_t* num_runs, int64_t n,
     int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket) {
-  using ST = SegTile<T, Op, ReduceByKeyGeom<T>>;
+  using G = ReduceByKeyGeom<T>;
+  using ST = SegTile<T, Op, G>;
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS, NWAVES = ST::NWAVES;
   __shared__ typename ST::Smem sm;
+  const int lane = threadIdx.x & (kWave - 1);
+  if constexpr (G::BLOCKED) {
+    // The heads of a wavefront's 64 * VEC consecutive elements go to consecutive output slots.
+    // They are compacted in the wavefront's buffer — keys first, then, through the same 8 KiB,
+    // the values of the runs they close — and written with contiguous stores.
+    static_assert(kWave * VEC * sizeof(KU) <= G::XPOSE_SLOTS * 16 && kWave * VEC * sizeof(T) <= G::XPOSE_SLOTS * 16,
+                  "a wavefront's heads fit its buffer");
+    __shared__ tcd_v4u s_x[NWAVES][G::XPOSE_SLOTS];
+    tcd_v4u* xbuf = s_x[threadIdx.x / kWave];
+    ST t;
+    t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf);
+    SegPair<T> run = t.off[0];  // (runs started so far, value of the open run) before the current element
+    const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)run.c);  // runs before this wavefront
+    const uint32_t heads = t.heads[0];
+    const uint32_t mine = run.c - first;  // slot of this thread's first head
+    const uint32_t count = (uint32_t)__builtin_amdgcn_readlane((int)(mine + __builtin_popcount(heads)), kWave - 1);
+    const int64_t i0 = t.index(0, 0);
+    // Slot i lives at sw(i): when most elements are heads a thread's slots start VEC apart, which
+    // is one LDS bank for all lanes; the swizzle spreads them (and the copy-out reads) over all.
+    constexpr uint32_t kLogVec = VEC == 32 ? 5 : 4;
+    static_assert((1u << kLogVec) == (uint32_t)VEC, "VEC is 16 or 32");
+    const auto sw = [](uint32_t i) { return i ^ ((i >> kLogVec) & (uint32_t)(VEC - 1)); };
+    KU* sk = reinterpret_cast<KU*>(xbuf);
+    {
+      uint32_t slot = mine;
+#pragma unroll
+      for (int j = 0; j < VEC; j++)
+        if ((heads >> j) & 1u) sk[sw(slot++)] = t.key[0][j];
+    }
+    wave_lds_sync();
+    for (uint32_t i = lane; i < count; i += kWave) keys_out[first + i] = sk[sw(i)];
+    wave_lds_sync();
+    T* sv = reinterpret_cast<T*>(xbuf);
+    {
+      uint32_t slot = mine;
+#pragma unroll
+      for (int j = 0; j < VEC; j++) {
+        const bool exists = t.full || i0 + j < n;
+        if ((heads >> j) & 1u) {
+          // a head closes the run before it and opens run number run.c
+          sv[sw(slot++)] = run.v;
+          run.c += 1;
+          run.v = t.val[0][j];
+        } else if (exists) {
+          run.v = Op::template apply<T>(run.v, t.val[0][j]);
+        }
+        if (!t.full && i0 + j == n - 1) {  // the last element closes the last run
+          vals_out[run.c - 1] = run.v;
+          *num_runs = (int64_t)run.c;
+        }
+      }
+    }
+    wave_lds_sync();
+    for (uint32_t i = lane; i < count; i += kWave)
+      if (first + i) vals_out[first + i - 1] = sv[sw(i)];  // value of the run that ended at this head
+    return;
+  }
   // Per-wave staging of one chunk's output: the heads of a wave's 64*VEC consecutive elements go
   // to consecutive output slots, so they are compacted in LDS and written with coalesced stores
   // (no workgroup barrier: the buffer is private to the wave).
-  __shared__ KU s_keys[NWAVES][kWave * VEC];
-  __shared__ T s_vals[NWAVES][kWave * VEC];
+  __shared__ KU s_keys[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
+  __shared__ T s_vals[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
   ST t;
-  t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket);
-  const int lane = threadIdx.x & (kWave - 1);
-  KU* sk = s_keys[threadIdx.x / kWave];
-  T* sv = s_vals[threadIdx.x / kWave];
+  t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, nullptr);
+  KU* sk = s_keys[G::BLOCKED ? 0 : threadIdx.x / kWave];
+  T* sv = s_vals[G::BLOCKED ? 0 : threadIdx.x / kWave];
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
     // (runs started so far, value of the open run) before the current element
