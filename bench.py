@@ -218,6 +218,25 @@ def main():
         add_extra(f"reduce_by_key_i32_mean{mean}", n, ms, 8.0 * n + 8.0 * r, "Gelem/s")
         extras[f"reduce_by_key_i32_mean{mean}"]["runs"] = r
 
+    def extra_sbk(mean):
+        # inclusive_scan_by_key with plus: int32 keys (geometric run lengths), int32 values
+        heads = torch.rand(n, device=dev, generator=gen(20 + mean)) < (1.0 / mean)
+        keys = torch.cumsum(heads.to(torch.int32), 0, dtype=torch.int32)
+        del heads
+        vals = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device=dev, generator=gen(9))
+        out = torch.empty_like(vals)
+        call = lambda t, nb: L.thrust_cdna4_scan_by_key(
+            t, ctypes.byref(nb), capi.I32, capi.I32, capi.PLUS, 0, ctypes.c_void_p(keys.data_ptr()),
+            ctypes.c_void_p(vals.data_ptr()), ctypes.c_void_p(out.data_ptr()), n, None, sp)
+        tmp, nb = two_phase(call)
+        tp = ctypes.c_void_p(tmp.data_ptr())
+        ms = timed(lambda: capi.check(call(tp, nb), "scan_by_key"), lambda: None, 10, 2)
+        # the last element of every run is the run's sum: together they add up to the total
+        last = torch.ones(n, dtype=torch.bool, device=dev)
+        last[:-1] = keys[1:] != keys[:-1]
+        assert int(out[last].sum(dtype=torch.int64).item()) == int(vals.sum(dtype=torch.int64).item())
+        add_extra(f"inclusive_scan_by_key_i32_mean{mean}", n, ms, 12.0 * n, "Gelem/s")
+
     def extra_hist():
         m = 1 << min(30, args.log2n + 2)
         s = torch.randint(0, 256, (m,), dtype=torch.uint8, device=dev, generator=gen(11))
@@ -300,6 +319,7 @@ def main():
         "rbk1": lambda: extra_rbk(1),
         "rbk8": lambda: extra_rbk(8),
         "rbk512": lambda: extra_rbk(512),
+        "sbk8": lambda: extra_sbk(8),
         "hist": extra_hist,
         "copy": extra_copy_ceiling,
     }
