@@ -162,7 +162,10 @@ T transform_reduce(void* stream_, std::int64_t n, Unary unary, T init, Op op) {
 // started already and the wait ends.  One same-address atomic costs about 12 ns of the whole
 // device's time, which is why a tile is 128 KiB of items.
 // ---------------------------------------------------------------------------------------
-constexpr int kSelBlock = 1024;
+#ifndef THRUST_CDNA4_SELECT_BLOCK
+#define THRUST_CDNA4_SELECT_BLOCK 1024
+#endif
+constexpr int kSelBlock = THRUST_CDNA4_SELECT_BLOCK;
 constexpr int kSelWaves = kSelBlock / 64;
 constexpr unsigned long long kSelValueMask = (1ull << 62) - 1ull;
 // rows of kSelBlock items per tile: 128 bytes of items per thread, 4 to 32 rows
@@ -171,7 +174,10 @@ constexpr int select_rows(std::size_t item_bytes) {
 }
 // Register budget: 32 rows of 4-byte items need about 72 registers (one workgroup per CU);
 // 8- to 32-byte items fit 64 registers, and the second workgroup per CU is worth 12 %.
-constexpr int select_waves_per_simd(std::size_t item_bytes) { return item_bytes > 4 && item_bytes <= 32 ? 8 : 4; }
+#ifndef THRUST_CDNA4_SELECT_WPE4
+#define THRUST_CDNA4_SELECT_WPE4 4
+#endif
+constexpr int select_waves_per_simd(std::size_t item_bytes) { return item_bytes > 4 && item_bytes <= 32 ? 8 : THRUST_CDNA4_SELECT_WPE4; }
 
 // words[0, tiles) are the descriptors, words[tiles] the ticket counter, words[tiles + 1] the result
 template <class Word>

@@ -186,6 +186,19 @@ int thrust_cdna4_malloc_direct(void** ptr, size_t bytes);
 int thrust_cdna4_free_direct(void* ptr);
 
 /*
+ * Scan, scan_by_key and reduce_by_key chain their tiles by look-back.  When the output does not
+ * overlap the input, a tile is the workgroup of the same index and a workgroup never waits
+ * unboundedly for another: a tile descriptor that is still missing after `polls` polls is
+ * recomputed from the input by the workgroup that needs it.  (With overlapping ranges tiles are
+ * handed out by an atomic ticket instead, which makes every wait finite by construction; the
+ * reference relies on cub's look-back, thrust/system/cuda/detail/scan.h:57-204.)  Sets the
+ * number of polls for later launches and returns the previous value; a negative value restores
+ * the default (256); 0 never waits, which the tests use to drive the recomputation path.
+ * Results do not depend on it except for the rounding order of floating-point sums.
+ */
+int thrust_cdna4_set_lookback_patience(int polls);
+
+/*
  * Launch profiling.  While enabled, every kernel the library launches is bracketed by HIP
  * events recorded on the launch stream and logged under its kernel name; enable(…) also
  * clears the log.  get() waits for record `index` and returns its name and duration in

@@ -106,3 +106,52 @@ def test_scan_repeat_determinism_ints():
     first = host(thrust_amd.inclusive_scan(x)).tobytes()
     for _ in range(5):
         assert host(thrust_amd.inclusive_scan(x)).tobytes() == first
+
+
+@pytest.fixture
+def no_patience():
+    """Look-back never waits: every tile descriptor that is not there yet is recomputed from the
+    input by the workgroup that needs it (the forward-progress path of the ticketless kernels)."""
+    from thrust_amd import capi
+    L = capi.lib()
+    previous = L.thrust_cdna4_set_lookback_patience(0)
+    yield
+    L.thrust_cdna4_set_lookback_patience(previous)
+
+
+def test_scan_recompute_path_matches_oracle(no_patience):
+    for n in [1, 4097, 32768, 32769, 200_003, (1 << 22) + 5]:
+        x = random_ints(50 + n, n, np.int32)
+        d = dev(x)
+        assert same_bits(host(thrust_amd.inclusive_scan(d)), oracle.scan(x, "plus")), n
+        assert same_bits(host(thrust_amd.exclusive_scan(d, init=7)), oracle.scan(x, "plus", exclusive=True, init=7)), n
+    x = random_ints(9, 1 << 21, np.uint64)
+    assert same_bits(host(thrust_amd.inclusive_scan(dev(x), op="maximum")), oracle.scan(x, "maximum"))
+    f = np.random.default_rng(3).uniform(-1, 1, 300_001).astype(np.float32)
+    got = host(thrust_amd.inclusive_scan(dev(f))).astype(np.float64)
+    ref = np.cumsum(f.astype(np.float64))
+    assert (np.abs(got - ref) <= FP_RTOL * np.cumsum(np.abs(f.astype(np.float64)))).all()
+
+
+def test_scan_full_size_recompute_path(no_patience):
+    n = 1 << 28
+    x = torch.ones(n, dtype=torch.int32, device="cuda")
+    out = thrust_amd.inclusive_scan(x)
+    assert int(out[-1].item()) == n and int(out[12345678].item()) == 12345679
+    assert bool((out[1:] - out[:-1] == 1).all())
+
+
+def test_scan_in_place_takes_the_ticket_path_and_out_of_place_does_not():
+    # both paths give the same bits; partially overlapping ranges count as in place
+    x = random_ints(123, (1 << 20) + 3, np.int32)
+    ref = oracle.scan(x, "plus")
+    d = dev(x)
+    assert same_bits(host(thrust_amd.inclusive_scan(d)), ref)
+    thrust_amd.inclusive_scan(d, out=d)
+    assert same_bits(host(d), ref)
+    buf = torch.empty(x.size + 64, dtype=torch.int32, device="cuda")
+    src = buf[64:]
+    src.copy_(dev(x))
+    dst = buf[:x.size]  # starts 256 bytes before the input
+    thrust_amd.inclusive_scan(src, out=dst)
+    assert same_bits(host(dst), ref)

@@ -21,7 +21,7 @@ SYMBOLS = [
     "thrust_cdna4_memcpy_htod", "thrust_cdna4_memcpy_dtoh", "thrust_cdna4_memcpy_dtod",
     "thrust_cdna4_fill", "thrust_cdna4_stream_synchronize", "thrust_cdna4_profile_enable",
     "thrust_cdna4_profile_count", "thrust_cdna4_profile_get",
-    "thrust_cdna4_selftest_lds_atomic_order",
+    "thrust_cdna4_selftest_lds_atomic_order", "thrust_cdna4_set_lookback_patience",
     "thrust_cdna4_stream_create", "thrust_cdna4_stream_destroy", "thrust_cdna4_stream_query",
     "thrust_cdna4_event_create", "thrust_cdna4_event_destroy", "thrust_cdna4_event_record", "thrust_cdna4_event_query",
     "thrust_cdna4_stream_wait_event", "thrust_cdna4_malloc_direct", "thrust_cdna4_free_direct",
@@ -78,6 +78,7 @@ def lib():
     L.thrust_cdna4_stream_wait_event.argtypes = [vp, vp]
     L.thrust_cdna4_malloc_direct.argtypes = [ctypes.POINTER(vp), sz]
     L.thrust_cdna4_free_direct.argtypes = [vp]
+    L.thrust_cdna4_set_lookback_patience.argtypes = [i32]
     L.thrust_cdna4_profile_enable.argtypes = [i32]
     L.thrust_cdna4_selftest_lds_atomic_order.argtypes = [ctypes.POINTER(ctypes.c_longlong), vp]
     L.thrust_cdna4_profile_get.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p),

@@ -295,6 +295,69 @@ __device__ inline P wave_lookback(const uint64_t* desc, int64_t tile, const P id
   return prefix;
 }
 
+// Look-back for kernels whose tile index is the workgroup index (no ticket).  Nothing then
+// guarantees that a tile this waits on has started, so the wait is bounded: a descriptor that is
+// still missing after `patience` polls is not waited for any longer — the wavefront computes
+// that tile's aggregate itself with aggregate_of(tile_index) (called by all 64 lanes, returns
+// the same value in all) and carries on.  Every loop ends whatever the other workgroups do.
+// With patience 0 nothing is ever waited for, which is how the tests drive this path.
+// aggregate_of reads the tile's INPUT: the caller must not use this when the kernel's output
+// may overwrite its input (the owner of a tile that has not published has not written any
+// output yet, but it may while the input is being read here); after computing, the descriptor
+// is read once more and, if the owner has published meanwhile, its word is taken instead.
+template <class P, class F, class A>
+__device__ inline P wave_lookback_or_compute(const uint64_t* desc, int64_t tile, const P id, F f, int patience,
+                                             A aggregate_of) {
+  const int lane = lane_id();
+  P prefix = id;
+  int64_t nearest = tile - 1;  // lane l inspects tile nearest - l
+  while (true) {
+    const int64_t pos = nearest - lane;
+    P val = id;
+    uint32_t st = kInclusive;  // tiles before tile 0: an empty, fully known prefix
+    if (pos >= 0) {
+      st = TileDesc<P>::load(desc, pos, val);
+      for (int polls = 0; st == kInvalid && polls < patience; polls++) {
+        __builtin_amdgcn_s_sleep(1);
+        st = TileDesc<P>::load(desc, pos, val);
+      }
+    }
+    uint64_t incl = __ballot(st == kInclusive);
+    int first = incl ? __builtin_ctzll(incl) : 64;
+    uint64_t missing = __ballot(st == kInvalid && lane <= first);  // only tiles that count
+    while (missing) {  // wave-uniform
+      const int l = __builtin_ctzll(missing);
+      missing &= missing - 1;
+      const P agg = aggregate_of(nearest - l);
+      P now = id;
+      const uint32_t st_now = TileDesc<P>::load(desc, nearest - l, now);
+      if (lane == l) {
+        if (st_now != kInvalid) { val = now; st = st_now; }
+        else { val = agg; st = kPartial; }
+      }
+    }
+    incl = __ballot(st == kInclusive);
+    first = incl ? __builtin_ctzll(incl) : 64;
+    P contrib = (lane <= first) ? val : id;
+    // ordered reduction: lane 63 (farthest tile) is leftmost
+    P red = wave_inclusive_scan(contrib, id, [&](const P& a, const P& b) { return f(b, a); });
+    red = readlane(red, 63);
+    prefix = f(red, prefix);
+    if (incl) break;
+    nearest -= 64;
+  }
+  return prefix;
+}
+// Polls of a missing tile descriptor before a ticketless kernel computes it itself (default
+// kDefaultLookbackPatience); set by thrust_cdna4_set_lookback_patience.
+constexpr int kDefaultLookbackPatience = 256;
+int lookback_patience();
+// true when [a, a + na) and [b, b + nb) share a byte
+inline bool ranges_overlap(const void* a, size_t na, const void* b, size_t nb) {
+  const uintptr_t x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
+  return x < y + nb && y < x + na;
+}
+
 // ---------------------------------------------------------------------------------------
 // Host-side dtype helpers
 // ---------------------------------------------------------------------------------------

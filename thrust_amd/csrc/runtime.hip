@@ -5,6 +5,7 @@
 #include <vector>
 
 #include "common.h"
+#include <atomic>
 
 namespace tcd {
 
@@ -299,6 +300,14 @@ extern "C" int thrust_cdna4_fill(void* dst, const void* value, int elem_bytes, i
     case 8: return fill_typed<uint64_t>(dst, value, n, s);
   }
   return hipErrorInvalidValue;
+}
+
+namespace tcd {
+static std::atomic<int> g_lookback_patience{kDefaultLookbackPatience};
+int lookback_patience() { return g_lookback_patience.load(std::memory_order_relaxed); }
+}  // namespace tcd
+extern "C" int thrust_cdna4_set_lookback_patience(int polls) {
+  return tcd::g_lookback_patience.exchange(polls < 0 ? tcd::kDefaultLookbackPatience : polls, std::memory_order_relaxed);
 }
 
 extern "C" int thrust_cdna4_stream_synchronize(void* stream) {

@@ -15,10 +15,14 @@ struct alignas(16) Vec16 {
   T v[16 / sizeof(T)];
 };
 
-template <class T, class Op, int BLOCK, int CHUNKS>
+// TICKET: tiles are handed out by an atomic counter, so every tile a tile waits on has started
+// (used when the output overlaps the input).  Otherwise a tile is the workgroup of the same
+// index — no atomic and no barrier before the loads, 6 % faster at 2^28 and 25 % at 2^24 — and a
+// descriptor that stays missing is recomputed from the input after `patience` polls.
+template <class T, class Op, int BLOCK, int CHUNKS, bool TICKET>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void scan_kernel(const T* in, T* out, int64_t n, T init,
                                                      int exclusive, uint64_t* desc,
-                                                     uint32_t* ticket, int vec_ok) {
+                                                     uint32_t* ticket, int vec_ok, int patience) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NWAVES = BLOCK / kWave;
   constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
@@ -43,9 +47,12 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
   };
   const W idW = toW(id);
 
-  if (tid == 0) s_tile = atomicAdd(ticket, 1u);
-  __syncthreads();
-  const int64_t tile = s_tile;
+  int64_t tile = blockIdx.x;
+  if constexpr (TICKET) {
+    if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+    __syncthreads();
+    tile = s_tile;
+  }
   const int64_t base = tile * TILE;
   const bool fast = vec_ok && (base + TILE <= n);  // whole tile present, 16-byte aligned pointers
   const T* tin = in + base + (int64_t)tid * VEC;
@@ -103,7 +110,19 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
       if (lane == 0) TileDesc<W>::store(desc, 0, kInclusive, opW(prefix, tile_agg));
     } else {
       if (lane == 0) TileDesc<W>::store(desc, tile, kPartial, tile_agg);
-      prefix = wave_lookback<W>(desc, tile, idW, opW);
+      if constexpr (TICKET) {
+        prefix = wave_lookback<W>(desc, tile, idW, opW);
+      } else {
+        // the aggregate of an earlier tile (always a whole one), straight from the input
+        const auto aggregate_of = [&](int64_t t) -> W {
+          const T* p = in + t * TILE + lane;
+          T acc = p[0];
+#pragma unroll 8
+          for (int k = 1; k < (int)(TILE / kWave); k++) acc = op(acc, p[(int64_t)k * kWave]);
+          return readlane(wave_inclusive_scan(toW(acc), idW, opW), kWave - 1);
+        };
+        prefix = wave_lookback_or_compute<W>(desc, tile, idW, opW, patience, aggregate_of);
+      }
       if (lane == 0) TileDesc<W>::store(desc, tile, kInclusive, opW(prefix, tile_agg));
     }
     const W base_w = opW(prefix, before);
@@ -185,9 +204,15 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   uint32_t* ticket = reinterpret_cast<uint32_t*>(temp);
   uint64_t* desc = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256);
   const int vec_ok = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-  TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS>), dim3((unsigned)ntiles), dim3(C::BLOCK),
-             stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
-             desc, ticket, vec_ok);
+  if (ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T))) {
+    TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS, true>), dim3((unsigned)ntiles), dim3(C::BLOCK),
+               stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
+               desc, ticket, vec_ok, 0);
+  } else {
+    TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS, false>), dim3((unsigned)ntiles), dim3(C::BLOCK),
+               stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
+               desc, ticket, vec_ok, lookback_patience());
+  }
   return hipGetLastError();
 }
 
