@@ -159,3 +159,44 @@ def test_reduce_by_key_empty_and_full_size_closed_form():
     assert gk.numel() == n // 512
     assert torch.equal(gk, torch.arange(n // 512, dtype=torch.int32, device="cuda"))
     assert bool((gv == 512).all())
+
+
+# ------------------------------------------------------------------ forward-progress path
+@pytest.fixture
+def no_patience():
+    """Look-back never waits: every tile descriptor that is not there yet is recomputed from the
+    input by the workgroup that needs it (the forward-progress path of the ticketless kernels)."""
+    from thrust_amd import capi
+    L = capi.lib()
+    previous = L.thrust_cdna4_set_lookback_patience(0)
+    yield
+    L.thrust_cdna4_set_lookback_patience(previous)
+
+
+@pytest.mark.parametrize("kd,vd", [(np.int32, np.int32), (np.uint8, np.int64), (np.float32, np.int32),
+                                   (np.uint64, np.uint16)])
+def test_by_key_recompute_path_matches_oracle(no_patience, kd, vd):
+    for n in [1, 16384, 16385, 100_003, (1 << 21) + 77]:
+        for mean in (1, 8, 5000):
+            k = (runs(n + mean, n, mean, np.int64) % 200).astype(kd)
+            v = random_ints(n + 1, n, vd)
+            dk, dv = dev(k), dev(v)
+            assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv)), oracle.scan_by_key(k, v)), (n, mean)
+            assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=3)),
+                             oracle.scan_by_key(k, v, exclusive=True, init=3)), (n, mean)
+            gk, gv = thrust_amd.reduce_by_key(dk, dv)
+            rk, rv = oracle.reduce_by_key(k, v)
+            assert same_bits(host(gk), rk) and same_bits(host(gv), rv), (n, mean)
+
+
+def test_by_key_aliased_outputs_take_the_ticket_path():
+    n = (1 << 20) + 9
+    k = (runs(5, n, 8, np.int64) % 200).astype(np.int32)
+    v = random_ints(6, n, np.int32)
+    dk, dv = dev(k), dev(v)
+    thrust_amd.inclusive_scan_by_key(dk, dv, out=dv)  # in place on the values
+    assert same_bits(host(dv), oracle.scan_by_key(k, v))
+    dk, dv = dev(k), dev(v)
+    gk, gv = thrust_amd.reduce_by_key(dk, dv, keys_out=dk, values_out=dv)  # compaction in place
+    rk, rv = oracle.reduce_by_key(k, v)
+    assert same_bits(host(gk), rk) and same_bits(host(gv), rv)

@@ -238,18 +238,25 @@ struct SegTile {
 
   __device__ static Pair comb(const Pair& a, const Pair& b) { return seg_combine<T, Op>(a, b); }
 
-  // xbuf: the wavefront's transpose buffer (blocked geometry only)
+  // xbuf: the wavefront's transpose buffer (blocked geometry only).  TICKET: tiles are handed out
+  // by an atomic counter (every tile waited for has started; used when an output overlaps an
+  // input); otherwise a tile is the workgroup of the same index and a descriptor that stays
+  // missing after `patience` polls is recomputed from the input.
+  template <bool TICKET>
   __device__ void run(Smem& sm, const KU* keys, const T* vals, int64_t n, int float_keys, int vec_ok,
-                      uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf) {
+                      uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf, int patience) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const T id = Op::template identity<T>();
     const Pair idp{0u, id};
 
-    if (tid == 0) sm.tile = atomicAdd(ticket, 1u);
-    __syncthreads();
-    tile = sm.tile;
+    tile = blockIdx.x;
+    if constexpr (TICKET) {
+      if (tid == 0) sm.tile = atomicAdd(ticket, 1u);
+      __syncthreads();
+      tile = sm.tile;
+    }
     base = tile * G::TILE;
     full = vec_ok && (base + G::TILE < n);
 
@@ -323,7 +330,28 @@ struct SegTile {
         if (lane == 0) TileDesc<Pair>::store(desc, 0, kInclusive, tile_agg);
       } else {
         if (lane == 0) TileDesc<Pair>::store(desc, tile, kPartial, tile_agg);
-        prefix = wave_lookback<Pair>(desc, tile, idp, comb);
+        if constexpr (TICKET) {
+          prefix = wave_lookback<Pair>(desc, tile, idp, comb);
+        } else {
+          // the aggregate of an earlier tile (always a whole one), straight from the input: each
+          // lane folds a contiguous piece, the pieces combine in lane order
+          const auto aggregate_of = [&](int64_t t) -> Pair {
+            constexpr int PIECE = (int)(G::TILE / kWave);
+            const int64_t start = t * G::TILE + (int64_t)lane * PIECE;
+            KU before = start > 0 ? keys[start - 1] : KU(0);
+            Pair a = idp;
+            for (int k = 0; k < PIECE; k++) {
+              const KU kk = keys[start + k];
+              const T vv = vals[start + k];
+              const bool is_head = start + k == 0 || keys_differ(before, kk, float_keys);
+              a.c += is_head ? 1u : 0u;
+              a.v = is_head ? vv : Op::template apply<T>(a.v, vv);
+              before = kk;
+            }
+            return readlane(wave_inclusive_scan(a, idp, comb), kWave - 1);
+          };
+          prefix = wave_lookback_or_compute<Pair>(desc, tile, idp, comb, patience, aggregate_of);
+        }
         if (lane == 0) TileDesc<Pair>::store(desc, tile, kInclusive, comb(prefix, tile_agg));
       }
       if (lane < CHUNKS * NWAVES) sm.tot[lane] = comb(prefix, before);
@@ -337,17 +365,17 @@ struct SegTile {
 // ---------------------------------------------------------------------------------------
 // scan_by_key
 // ---------------------------------------------------------------------------------------
-template <class T, class Op>
+template <class T, class Op, bool TICKET>
 __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_key_kernel(
     const KU* keys, const T* vals, T* out, int64_t n, T init, int exclusive, int float_keys, int vec_ok,
-    uint64_t* desc, uint32_t* ticket) {
+    uint64_t* desc, uint32_t* ticket, int patience) {
   using G = ScanByKeyGeom<T>;
   using ST = SegTile<T, Op, G>;
   __shared__ typename ST::Smem sm;
   __shared__ tcd_v4u s_x[G::BLOCKED ? G::NWAVES : 1][G::XPOSE_SLOTS];
   tcd_v4u* xbuf = s_x[G::BLOCKED ? threadIdx.x / kWave : 0];
   ST t;
-  t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf);
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience);
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS;
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
@@ -378,10 +406,10 @@ __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_
 // ---------------------------------------------------------------------------------------
 // reduce_by_key
 // ---------------------------------------------------------------------------------------
-template <class T, class Op>
+template <class T, class Op, bool TICKET>
 __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce_by_key_kernel(
     const KU* keys, const T* vals, KU* keys_out, T* vals_out, int64_t* num_runs, int64_t n,
-    int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket) {
+    int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket, int patience) {
   using G = ReduceByKeyGeom<T>;
   using ST = SegTile<T, Op, G>;
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS, NWAVES = ST::NWAVES;
@@ -396,7 +424,7 @@ __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce
     __shared__ tcd_v4u s_x[NWAVES][G::XPOSE_SLOTS];
     tcd_v4u* xbuf = s_x[threadIdx.x / kWave];
     ST t;
-    t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf);
+    t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience);
     SegPair<T> run = t.off[0];  // (runs started so far, value of the open run) before the current element
     const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)run.c);  // runs before this wavefront
     const uint32_t heads = t.heads[0];
@@ -449,7 +477,7 @@ __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce
   __shared__ KU s_keys[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
   __shared__ T s_vals[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
   ST t;
-  t.run(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, nullptr);
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, nullptr, patience);
   KU* sk = s_keys[G::BLOCKED ? 0 : threadIdx.x / kWave];
   T* sv = s_vals[G::BLOCKED ? 0 : threadIdx.x / kWave];
 #pragma unroll
@@ -520,11 +548,22 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
       const int vec_ok = ((reinterpret_cast<uintptr_t>(keys) | reinterpret_cast<uintptr_t>(values) |
                            reinterpret_cast<uintptr_t>(out)) & 15) == 0;
       const int64_t ntiles = ceil_div(n, ScanByKeyGeom<T>::TILE);
-      TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(ScanByKeyGeom<T>::BLOCK), s,
-                         static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
-                         n, iv, exclusive, float_keys, vec_ok,
-                         reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
-                         reinterpret_cast<uint32_t*>(temp));
+      // an output that overlaps an input: tiles by ticket
+      const bool aliased = ranges_overlap(out, (size_t)n * sizeof(T), values, (size_t)n * sizeof(T)) ||
+                           ranges_overlap(out, (size_t)n * sizeof(T), keys, (size_t)n * sizeof(KU));
+      if (aliased) {
+        TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(ScanByKeyGeom<T>::BLOCK), s,
+                           static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
+                           n, iv, exclusive, float_keys, vec_ok,
+                           reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
+                           reinterpret_cast<uint32_t*>(temp), 0);
+      } else {
+        TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, false>), dim3((unsigned)ntiles), dim3(ScanByKeyGeom<T>::BLOCK), s,
+                           static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
+                           n, iv, exclusive, float_keys, vec_ok,
+                           reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
+                           reinterpret_cast<uint32_t*>(temp), lookback_patience());
+      }
       rc = hipGetLastError();
     });
   });
@@ -554,11 +593,23 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
       if (rc != hipSuccess) return;
       const int vec_ok = ((reinterpret_cast<uintptr_t>(keys_in) | reinterpret_cast<uintptr_t>(values_in)) & 15) == 0;
       const int64_t ntiles = ceil_div(n, ReduceByKeyGeom<T>::TILE);
-      TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op>), dim3((unsigned)ntiles), dim3(ReduceByKeyGeom<T>::BLOCK), s,
-                         static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
-                         static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
-                         vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
-                         reinterpret_cast<uint32_t*>(temp));
+      // an output that overlaps an input: tiles by ticket
+      const size_t kb = (size_t)n * sizeof(KU), vb = (size_t)n * sizeof(T);
+      const bool aliased = ranges_overlap(keys_out, kb, keys_in, kb) || ranges_overlap(keys_out, kb, values_in, vb) ||
+                           ranges_overlap(values_out, vb, keys_in, kb) || ranges_overlap(values_out, vb, values_in, vb);
+      if (aliased) {
+        TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(ReduceByKeyGeom<T>::BLOCK), s,
+                           static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
+                           static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
+                           vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
+                           reinterpret_cast<uint32_t*>(temp), 0);
+      } else {
+        TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, false>), dim3((unsigned)ntiles), dim3(ReduceByKeyGeom<T>::BLOCK), s,
+                           static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
+                           static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
+                           vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
+                           reinterpret_cast<uint32_t*>(temp), lookback_patience());
+      }
       rc = hipGetLastError();
     });
   });
