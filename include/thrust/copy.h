@@ -95,6 +95,20 @@ Out copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out 
   system::cdna4::detail::transform_n(exec.derived(), detail::unwrap(first), detail::unwrap(out), n, identity<typename detail::value_of<In>::type>());
   return out + n;
 }
+// contiguous device ranges of one type: a stream-ordered memcpy, no kernel template
+template <class D, class T>
+device_ptr<typename std::remove_const<T>::type> copy(const system::cdna4::execution_policy<D>& exec, device_ptr<T> first, device_ptr<T> last,
+                                                     device_ptr<typename std::remove_const<T>::type> out) {
+  namespace sd = system::cdna4::detail;
+  const std::size_t n = (std::size_t)(last - first);
+  if (n) sd::throw_on_error(thrust_cdna4_memcpy_dtod(out.get(), first.get(), n * sizeof(T), sd::stream_of(exec.derived())), "copy");
+  sd::synchronize_optional(exec.derived(), "copy: failed to synchronize");
+  return out + n;
+}
+template <class Policy, class In, class Size, class Out, detail::enable_if_policy<Policy> = 0>
+Out copy_n(const Policy& exec, In first, Size n, Out out) { return copy(exec, first, first + n, out); }
+template <class In, class Size, class Out, typename std::enable_if<!detail::is_policy<In>::value, int>::type = 0>
+Out copy_n(In first, Size n, Out out) { return copy(first, first + n, out); }
 template <class In, class Out>
 Out copy(const system::cpp::detail::par_t&, In first, In last, Out out) { return std::copy(first, last, out); }
 template <class In, class Out,

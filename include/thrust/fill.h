@@ -1,16 +1,53 @@
-// thrust::fill (thrust/fill.h; thrust/system/cuda/detail/fill.h:61-75).
+// thrust::fill / fill_n (thrust/fill.h; thrust/system/cuda/detail/fill.h:61-75).  Contiguous
+// device ranges of 1-, 2-, 4- and 8-byte elements go to the library's typed fill kernel (no
+// device compiler needed in the caller); other element sizes and fancy outputs instantiate a
+// kernel template.
 #pragma once
 #include <algorithm>
-#include <thrust/device_ptr.h>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+
 namespace thrust {
-template <class T, class V>
-void fill(device_ptr<T> first, device_ptr<T> last, const V& value) {
+namespace detail {
+template <class T> struct fill_value {
+  T v;
+  template <class U> THRUST_CDNA4_HD T operator()(const U&) const { return v; }
+};
+template <class Policy, class T, class V>
+typename std::enable_if<sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8>::type
+fill_device(const Policy& exec, device_ptr<T> first, std::int64_t n, const V& value) {
+  namespace sd = system::cdna4::detail;
   const T v = static_cast<T>(value);
-  if (last - first <= 0) return;
-  system::cdna4::detail::throw_on_error(
-      thrust_cdna4_fill(first.get(), &v, (int)sizeof(T), (int64_t)(last - first), nullptr), "fill");
-  system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "fill");
+  if (n <= 0) return;
+  sd::throw_on_error(thrust_cdna4_fill(first.get(), &v, (int)sizeof(T), n, sd::stream_of(exec)), "fill");
+  sd::synchronize_optional(exec, "fill: failed to synchronize");
 }
-template <class It, class V, class = typename std::enable_if<!system::cdna4::detail::is_device_iterator<It>::value>::type>
-void fill(It first, It last, const V& value) { std::fill(first, last, value); }
+template <class Policy, class T, class V>
+typename std::enable_if<!(sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8)>::type
+fill_device(const Policy& exec, device_ptr<T> first, std::int64_t n, const V& value) {
+  system::cdna4::detail::transform_n(exec, first.get(), first.get(), n, fill_value<T>{static_cast<T>(value)});
+}
+template <class Policy, class Out, class V>
+void fill_device(const Policy& exec, Out first, std::int64_t n, const V& value) {  // fancy output
+  typedef typename value_of<Out>::type T;
+  system::cdna4::detail::transform_n(exec, unwrap(first), unwrap(first), n, fill_value<T>{static_cast<T>(value)});
+}
+}  // namespace detail
+
+template <class D, class It, class V>
+void fill(const system::cdna4::execution_policy<D>& exec, It first, It last, const V& value) {
+  detail::fill_device(exec.derived(), first, (std::int64_t)(last - first), value);
+}
+template <class It, class V>
+void fill(const system::cpp::detail::par_t&, It first, It last, const V& value) { std::fill(first, last, value); }
+template <class Policy, class It, class Size, class V, detail::enable_if_policy<Policy> = 0>
+It fill_n(const Policy& exec, It first, Size n, const V& value) {
+  fill(exec, first, first + n, value);
+  return first + n;
+}
+template <class It, class V, detail::enable_if_device<It> = 0> void fill(It f, It l, const V& v) { fill(device, f, l, v); }
+template <class It, class V, detail::enable_if_host<It> = 0> void fill(It f, It l, const V& v) { fill(host, f, l, v); }
+template <class It, class Size, class V, detail::enable_if_device<It> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(device, f, n, v); }
+template <class It, class Size, class V, detail::enable_if_host<It> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(host, f, n, v); }
 }  // namespace thrust

@@ -42,6 +42,34 @@ void TestSortOnStream() {
 }
 DECLARE_UNITTEST(TestSortOnStream);
 
+// fill / fill_n / copy / copy_n with execution policies (testing/fill.cu:20-110, copy.cu:100-180,
+// copy_n.cu): contiguous ranges of arithmetic types need no device compiler in the caller
+void TestFillAndCopyWithPolicies() {
+  hipStream_t s;
+  ASSERT_EQUAL((int)hipStreamCreate(&s), 0);
+  thrust::device_vector<int> v(5, 0);
+  thrust::fill(thrust::device, v.begin() + 1, v.begin() + 4, 7);
+  ASSERT_EQUAL(v, thrust::host_vector<int>({0, 7, 7, 7, 0}));
+  auto e = thrust::fill_n(v.begin(), 3, 2);
+  ASSERT_EQUAL(e - v.begin(), (std::ptrdiff_t)3);
+  ASSERT_EQUAL(v, thrust::host_vector<int>({2, 2, 2, 7, 0}));
+  thrust::device_vector<double> big(100003), copy(100003);
+  thrust::fill(thrust::cdna4::par.on(s), big.begin(), big.end(), 1.5);
+  auto ce = thrust::copy(thrust::cdna4::par.on(s), big.begin(), big.end(), copy.begin());
+  ASSERT_TRUE(ce == copy.end());
+  ASSERT_EQUAL(copy, thrust::host_vector<double>(100003, 1.5));
+  thrust::device_vector<double> head(10);
+  thrust::copy_n(thrust::device, big.begin(), 10, head.begin());
+  ASSERT_EQUAL(head, thrust::host_vector<double>(10, 1.5));
+  thrust::host_vector<short> h(9);
+  thrust::fill(thrust::host, h.begin(), h.end(), (short)-3);
+  thrust::device_vector<short> d(9);
+  thrust::copy_n(h.begin(), 9, d.begin());
+  ASSERT_EQUAL(d, h);
+  ASSERT_EQUAL((int)hipStreamDestroy(s), 0);
+}
+DECLARE_UNITTEST(TestFillAndCopyWithPolicies);
+
 void TestEmptyRanges() {
   thrust::device_vector<int> d, o;
   thrust::sort(d.begin(), d.end());
