@@ -9,13 +9,72 @@
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
 #include <thrust/system/cdna4/detail/algorithms.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
 
 // ---- device, explicit policy ---------------------------------------------------------
+namespace detail {
+// a contiguous device range (device_ptr or raw pointer), as opposed to a fancy iterator
+template <class It> struct is_contiguous_device : std::is_pointer<typename unwrap_iterator<It>::type> {};
+
+template <class Policy, class It, class Compare>
+void sort_range(const Policy& exec, It first, It last, Compare comp, std::true_type) {
+  system::cdna4::detail::sort_keys(exec, unwrap(first), (std::int64_t)(last - first), comp);
+}
+// A fancy range (zip, permutation, ...) is sorted in a contiguous temporary of its value type and
+// written back.
+template <class Policy, class It, class Compare>
+void sort_range(const Policy& exec, It first, It last, Compare comp, std::false_type) {
+  namespace sd = system::cdna4::detail;
+  typedef typename value_of<It>::type T;
+  const std::int64_t n = (std::int64_t)(last - first);
+  if (n <= 0) return;
+  const sd::execute_on_stream inner(sd::stream_of(exec), false);  // same stream, no waits in between
+  sd::temporary_storage tmp((std::size_t)n * sizeof(T), exec);
+  T* p = static_cast<T*>(tmp.data());
+  sd::transform_n(inner, unwrap(first), p, n, identity<T>());
+  sd::sort_keys(inner, p, n, comp);
+  sd::transform_n(exec, p, unwrap(first), n, identity<T>());
+}
+
+template <class K, class U> K* pick_keys(U* contiguous, void*) { return const_cast<K*>(static_cast<const K*>(contiguous)); }
+template <class K, class It> K* pick_keys(It, void* temporary) { return static_cast<K*>(temporary); }
+template <class Policy, class KIt, class VIt, class Compare>
+void sort_pairs_range(const Policy& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp, std::true_type) {
+  system::cdna4::detail::sort_pairs(exec, unwrap(kfirst), unwrap(vfirst), (std::int64_t)(klast - kfirst), comp);
+}
+// Fancy keys or values (typically a zip_iterator of several value arrays): the keys are sorted
+// together with their positions, then the values are permuted through a temporary.
+template <class Policy, class KIt, class VIt, class Compare>
+void sort_pairs_range(const Policy& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp, std::false_type) {
+  namespace sd = system::cdna4::detail;
+  typedef typename value_of<KIt>::type K;
+  typedef typename value_of<VIt>::type V;
+  const std::int64_t n = (std::int64_t)(klast - kfirst);
+  if (n <= 0) return;
+  if (n >= (std::int64_t(1) << 32) - 1) sd::throw_on_error(1, "sort_by_key: more than 2^32 - 2 elements");
+  const sd::execute_on_stream inner(sd::stream_of(exec), false);
+  sd::temporary_storage index_bytes((std::size_t)n * sizeof(std::uint32_t), exec);
+  std::uint32_t* index = static_cast<std::uint32_t*>(index_bytes.data());
+  sd::sequence_n(inner, index, n, std::uint32_t(0), std::uint32_t(1));
+  {
+    sd::temporary_storage key_bytes(is_contiguous_device<KIt>::value ? 0 : (std::size_t)n * sizeof(K), exec);
+    K* keys = pick_keys<K>(unwrap(kfirst), key_bytes.data());
+    if (!is_contiguous_device<KIt>::value) sd::transform_n(inner, unwrap(kfirst), keys, n, identity<K>());
+    sd::sort_pairs(inner, keys, index, n, comp);
+    if (!is_contiguous_device<KIt>::value) sd::transform_n(inner, keys, unwrap(kfirst), n, identity<K>());
+  }
+  sd::temporary_storage value_bytes((std::size_t)n * sizeof(V), exec);
+  V* moved = static_cast<V*>(value_bytes.data());
+  sd::gather_n(inner, unwrap(vfirst), index, moved, n);
+  sd::transform_n(exec, moved, unwrap(vfirst), n, identity<V>());
+}
+}  // namespace detail
+
 template <class D, class It, class Compare>
 void stable_sort(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) {
-  system::cdna4::detail::sort_keys(exec.derived(), detail::unwrap(first), (std::int64_t)(last - first), comp);
+  detail::sort_range(exec.derived(), first, last, comp, typename detail::is_contiguous_device<It>::type());
 }
 template <class D, class It>
 void stable_sort(const system::cdna4::execution_policy<D>& exec, It first, It last) {
@@ -29,8 +88,8 @@ void sort(const system::cdna4::execution_policy<D>& exec, It first, It last) { s
 
 template <class D, class KIt, class VIt, class Compare>
 void stable_sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
-  system::cdna4::detail::sort_pairs(exec.derived(), detail::unwrap(kfirst), detail::unwrap(vfirst),
-                                    (std::int64_t)(klast - kfirst), comp);
+  detail::sort_pairs_range(exec.derived(), kfirst, klast, vfirst, comp,
+                           std::integral_constant<bool, detail::is_contiguous_device<KIt>::value && detail::is_contiguous_device<VIt>::value>());
 }
 template <class D, class KIt, class VIt>
 void stable_sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst) {

@@ -269,6 +269,24 @@ void binary_search_n(const Policy& exec, Hay hay, std::int64_t count, Needles ne
 #endif
 }
 
+// out[i] = in[index[i]]
+#if defined(__HIPCC__)
+template <class In, class Index, class Out> struct gather_body {
+  In in; Index index; Out out;
+  __device__ void operator()(std::int64_t i) { out[i] = in[index[i]]; }
+};
+#endif
+template <class Policy, class In, class Index, class Out>
+void gather_n(const Policy& exec, In in, Index index, Out out, std::int64_t n) {
+  THRUST_CDNA4_NEEDS_HIPCC(In);
+#if defined(__HIPCC__)
+  generic::parallel_for(stream_of(exec), n, gather_body<In, Index, Out>{in, index, out});
+  synchronize_optional(exec, "gather: failed to synchronize");
+#else
+  (void)exec; (void)in; (void)index; (void)out; (void)n;
+#endif
+}
+
 // ---- fancy iterators around the C-ABI algorithms (sort, scan, by-key) --------------------
 // Those kernels read and write contiguous arrays.  A raw pointer passes through; any other
 // iterator is read into (input) or written from (output) a pool temporary by one generic kernel.

@@ -348,4 +348,51 @@ void TestScanWithFancyIterators() {
 }
 DECLARE_UNITTEST(TestScanWithFancyIterators);
 
+// testing/zip_iterator_sort_by_key.cu, zip_iterator_sort.cu: zipped values follow their keys; a
+// range of tuples sorts lexicographically
+struct first_then_second {
+  __host__ __device__ bool operator()(const thrust::tuple<int, int>& a, const thrust::tuple<int, int>& b) const {
+    return thrust::get<0>(a) < thrust::get<0>(b) || (thrust::get<0>(a) == thrust::get<0>(b) && thrust::get<1>(a) < thrust::get<1>(b));
+  }
+};
+void TestSortWithZipIterators() {
+  for (std::size_t n : {std::size_t(0), std::size_t(1), std::size_t(1000), std::size_t(300007)}) {
+    thrust::host_vector<int> hk = unittest::random_integers<int>(n);
+    for (std::size_t i = 0; i < n; i++) hk[i] %= 97;  // many equal keys: stability shows
+    thrust::host_vector<int> ha(n);
+    thrust::host_vector<float> hb(n);
+    for (std::size_t i = 0; i < n; i++) { ha[i] = (int)i; hb[i] = 0.5f * (float)i; }
+    thrust::device_vector<int> k = hk, a = ha;
+    thrust::device_vector<float> b = hb;
+    thrust::stable_sort_by_key(k.begin(), k.end(), thrust::make_zip_iterator(thrust::make_tuple(a.begin(), b.begin())));
+    std::vector<std::size_t> order(n);
+    std::iota(order.begin(), order.end(), std::size_t(0));
+    std::stable_sort(order.begin(), order.end(), [&](std::size_t x, std::size_t y) { return hk[x] < hk[y]; });
+    thrust::host_vector<int> ek(n), ea(n);
+    thrust::host_vector<float> eb(n);
+    for (std::size_t i = 0; i < n; i++) { ek[i] = hk[order[i]]; ea[i] = ha[order[i]]; eb[i] = hb[order[i]]; }
+    ASSERT_EQUAL(k, ek);
+    ASSERT_EQUAL(a, ea);
+    ASSERT_EQUAL(b, eb);
+    // a range of (key, tiebreak) tuples, sorted lexicographically: with operator< and with a functor
+    thrust::host_vector<int> h1 = unittest::random_integers<int>(n, 4);
+    for (std::size_t i = 0; i < n; i++) h1[i] %= 1000;
+    thrust::device_vector<int> p = hk, q = h1, p2 = hk, q2 = h1;
+    auto zfirst = thrust::make_zip_iterator(thrust::make_tuple(p.begin(), q.begin()));
+    thrust::sort(zfirst, zfirst + n);
+    auto zfirst2 = thrust::make_zip_iterator(thrust::make_tuple(p2.begin(), q2.begin()));
+    thrust::sort(thrust::device, zfirst2, zfirst2 + n, first_then_second());
+    std::vector<std::pair<int, int>> pairs(n);
+    for (std::size_t i = 0; i < n; i++) pairs[i] = std::make_pair((int)hk[i], (int)h1[i]);
+    std::sort(pairs.begin(), pairs.end());
+    thrust::host_vector<int> ep(n), eq(n);
+    for (std::size_t i = 0; i < n; i++) { ep[i] = pairs[i].first; eq[i] = pairs[i].second; }
+    ASSERT_EQUAL(p, ep);
+    ASSERT_EQUAL(q, eq);
+    ASSERT_EQUAL(p2, ep);
+    ASSERT_EQUAL(q2, eq);
+  }
+}
+DECLARE_UNITTEST(TestSortWithZipIterators);
+
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
