@@ -14,7 +14,7 @@ FP_RTOL = 1e-5
 
 
 def runs(seed, n, mean, kd=np.int32):
-    """Sorted runs of keys with geometric run lengths (BASELINE config 4)."""
+    """Sorted runs of keys with geometric run lengths (benchmark configuration 4)."""
     rng = np.random.default_rng(seed)
     if n == 0:
         return np.zeros(0, dtype=kd)
@@ -110,7 +110,7 @@ def test_reduce_by_key_ints_bit_exact(kd, vd):
 
 
 def test_reduce_by_key_config4_reduced():
-    # BASELINE config 4 at 2^21: int32 values in [-1000,1000] bit-exact; fp32 N(0,1) within
+    # benchmark configuration 4 at 2^21: int32 values in [-1000,1000] bit-exact; fp32 N(0,1) within
     # 1e-5 of the run's L1 norm
     n = 1 << 21
     rng = np.random.default_rng(7)

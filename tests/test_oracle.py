@@ -90,7 +90,7 @@ def test_sort_brute_force_tiny():
 
 
 def test_config1_plumbing_sort_2_25_u32_seed_1337():
-    # BASELINE config 1: 2^25 uniform u32 keys, seed 1337, ascending == std::sort order.
+    # benchmark configuration 1: 2^25 uniform u32 keys, seed 1337, ascending == std::sort order.
     k = splitmix64(1337, 1 << 25).astype(np.uint32)
     got = oracle.sort_keys(k)
     assert same_bits(got, np.sort(k))

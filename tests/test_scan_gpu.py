@@ -84,7 +84,7 @@ def test_scan_unaligned_in_place():
 
 
 def test_scan_full_size_closed_forms():
-    # 2^28 elements (BASELINE config 2): constants have closed-form scans
+    # 2^28 elements (benchmark configuration 2): constants have closed-form scans
     n = 1 << 28
     ones = torch.ones(n, dtype=torch.int32, device="cuda")
     out = thrust_amd.inclusive_scan(ones)

@@ -97,7 +97,7 @@ def test_sort_pairs_stability(kd, vd):
 
 
 def test_sort_pairs_u64_entropy_sweep():
-    # BASELINE config 3 at reduced n: keys = AND of k uniform words; values = original index
+    # benchmark configuration 3 at reduced n: keys = AND of k uniform words; values = original index
     n = (1 << 20) + 17
     for words in range(0, 5):
         k = np.full(n, np.uint64(0xFFFFFFFFFFFFFFFF))
