@@ -75,6 +75,48 @@ class device_vector {
   void assign(size_type n, const T& v) { n_ = 0; if (n > cap_) regrow(n); fill_raw(p_, n, v); n_ = n; }
   template <class It, class = typename std::iterator_traits<It>::iterator_category>
   void assign(It first, It last) { assign_range(first, last, typename std::is_same<It, iterator>::type()); }
+  void pop_back() { --n_; }
+  void shrink_to_fit() {
+    if (n_ == cap_) return;
+    device_vector tight(alloc_);
+    tight.assign_device(p_, n_);
+    swap(tight);
+  }
+  // erase [first, last): the tail moves down (the usual partner of remove_if / unique)
+  iterator erase(iterator first, iterator last) {
+    const size_type at = (size_type)(first - begin()), count = (size_type)(last - first), tail = n_ - at - count;
+    if (count == 0) return first;
+    if (tail) {
+      // the ranges may overlap: go through a temporary
+      device_vector moved(alloc_);
+      moved.assign_device(p_ + at + count, tail);
+      check(thrust_cdna4_memcpy_dtod(p_ + at, moved.p_, tail * sizeof(T), nullptr), "device_vector: erase");
+      sync();
+    }
+    n_ -= count;
+    return begin() + at;
+  }
+  iterator erase(iterator pos) { return erase(pos, pos + 1); }
+  // insert [first, last) (a device or a host range) before pos
+  template <class It, class = typename std::iterator_traits<It>::iterator_category>
+  iterator insert(iterator pos, It first, It last) {
+    const size_type at = (size_type)(pos - begin());
+    device_vector added(alloc_);
+    added.assign(first, last);
+    device_vector tail(alloc_);
+    tail.assign_device(p_ + at, n_ - at);
+    const size_type total = n_ + added.n_;
+    if (total > cap_) regrow(std::max(total, 2 * cap_));
+    if (added.n_) check(thrust_cdna4_memcpy_dtod(p_ + at, added.p_, added.n_ * sizeof(T), nullptr), "device_vector: insert");
+    if (tail.n_) check(thrust_cdna4_memcpy_dtod(p_ + at + added.n_, tail.p_, tail.n_ * sizeof(T), nullptr), "device_vector: insert");
+    sync();
+    n_ = total;
+    return begin() + at;
+  }
+  iterator insert(iterator pos, const T& v) {
+    const T one[1] = {v};
+    return insert(pos, one, one + 1);
+  }
   void push_back(const T& v) {
     if (n_ == cap_) regrow(cap_ ? 2 * cap_ : 16);
     fill_raw(p_ + n_, 1, v);

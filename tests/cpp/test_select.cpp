@@ -162,6 +162,10 @@ void TestRemoveSimple() {
   ASSERT_EQUAL(data, vec<T>({1, 1, 3}));
 
   data = vec<T>({1, 2, 1, 3, 2});
+  data.erase(thrust::remove(data.begin(), data.end(), (T)2), data.end());  // the erase-remove idiom
+  ASSERT_EQUAL(data, vec<T>({1, 1, 3}));
+
+  data = vec<T>({1, 2, 1, 3, 2});
   end = thrust::remove_if(data.begin(), data.end(), is_even<T>());
   ASSERT_EQUAL(end - data.begin(), (std::ptrdiff_t)3);
   data.resize(3);

@@ -70,6 +70,32 @@ void TestFillAndCopyWithPolicies() {
 }
 DECLARE_UNITTEST(TestFillAndCopyWithPolicies);
 
+// thrust/device_vector.h: erase / insert / pop_back / shrink_to_fit (testing/vector_manipulation.cu,
+// vector_insert.cu); erase(new_end, end()) is how remove_if / unique results are trimmed
+void TestDeviceVectorEraseInsert() {
+  thrust::device_vector<int> v(thrust::host_vector<int>({0, 1, 2, 3, 4, 5, 6, 7}));
+  auto it = v.erase(v.begin() + 2, v.begin() + 5);
+  ASSERT_EQUAL(it - v.begin(), (std::ptrdiff_t)2);
+  ASSERT_EQUAL(v, thrust::host_vector<int>({0, 1, 5, 6, 7}));
+  v.erase(v.begin());
+  ASSERT_EQUAL(v, thrust::host_vector<int>({1, 5, 6, 7}));
+  v.erase(v.begin() + 2, v.end());
+  ASSERT_EQUAL(v, thrust::host_vector<int>({1, 5}));
+  const int more[3] = {8, 9, 10};
+  v.insert(v.begin() + 1, more, more + 3);
+  ASSERT_EQUAL(v, thrust::host_vector<int>({1, 8, 9, 10, 5}));
+  thrust::device_vector<int> d2(2, 4);
+  v.insert(v.end(), d2.begin(), d2.end());
+  v.insert(v.begin(), -1);
+  ASSERT_EQUAL(v, thrust::host_vector<int>({-1, 1, 8, 9, 10, 5, 4, 4}));
+  v.pop_back();
+  v.shrink_to_fit();
+  ASSERT_EQUAL(v.size(), (std::size_t)7);
+  ASSERT_EQUAL(v.capacity(), (std::size_t)7);
+  ASSERT_EQUAL((int)v.back(), 4);
+}
+DECLARE_UNITTEST(TestDeviceVectorEraseInsert);
+
 void TestEmptyRanges() {
   thrust::device_vector<int> d, o;
   thrust::sort(d.begin(), d.end());
