@@ -37,7 +37,7 @@ struct DescWord {
   __device__ static uint32_t count(D w) { return (uint32_t)(w & kCountMask); }
 };
 #ifndef TCD_SORT_LOOKW
-#define TCD_SORT_LOOKW 4
+#define TCD_SORT_LOOKW 8
 #endif
 constexpr int kLookW = TCD_SORT_LOOKW;  // look-back descriptors loaded per round trip
 
