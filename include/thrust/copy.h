@@ -119,11 +119,11 @@ template <class In, class Out,
 Out copy(In first, In last, Out out) {
   typedef typename detail::value_of<In>::type V;
   const std::size_t n = (std::size_t)(last - first);
-  V* tmp = static_cast<V*>(system::cdna4::detail::malloc_bytes(n * sizeof(V), nullptr));
+  system::cdna4::detail::temporary_storage staging(n * sizeof(V), nullptr);
+  V* tmp = static_cast<V*>(staging.data());
   copy(device, first, last, device_ptr<V>(tmp));
   std::vector<V> host(n);
   system::cdna4::detail::copy_bytes(host.data(), tmp, n * sizeof(V), 1);
-  system::cdna4::detail::free_bytes(tmp, nullptr);
   return std::copy(host.begin(), host.end(), out);
 }
 }  // namespace thrust
