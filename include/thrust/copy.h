@@ -119,7 +119,7 @@ template <class In, class Out,
 Out copy(In first, In last, Out out) {
   typedef typename detail::value_of<In>::type V;
   const std::size_t n = (std::size_t)(last - first);
-  system::cdna4::detail::temporary_storage staging(n * sizeof(V), nullptr);
+  system::cdna4::detail::temporary_storage staging(n * sizeof(V), static_cast<void*>(nullptr));
   V* tmp = static_cast<V*>(staging.data());
   copy(device, first, last, device_ptr<V>(tmp));
   std::vector<V> host(n);

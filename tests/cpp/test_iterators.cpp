@@ -170,6 +170,9 @@ void TestCountingAndConstantIterators() {
   thrust::device_vector<int> out(4);
   thrust::copy(first, first + 4, out.begin());
   ASSERT_EQUAL(out, vec<int>({1, 2, 3, 4}));
+  thrust::host_vector<int> hout(4);
+  thrust::copy(first + 10, first + 14, hout.begin());  // a device-side range copied to the host
+  ASSERT_EQUAL(hout, vec<int>({11, 12, 13, 14}));
   const long long n = 1000003;
   thrust::counting_iterator<long long> c(0);
   ASSERT_EQUAL(thrust::reduce(c, c + n), n * (n - 1) / 2);
