@@ -105,10 +105,7 @@ device_ptr<typename std::remove_const<T>::type> copy(const system::cdna4::execut
   sd::synchronize_optional(exec.derived(), "copy: failed to synchronize");
   return out + n;
 }
-template <class Policy, class In, class Size, class Out, detail::enable_if_policy<Policy> = 0>
-Out copy_n(const Policy& exec, In first, Size n, Out out) { return copy(exec, first, first + n, out); }
-template <class In, class Size, class Out, typename std::enable_if<!detail::is_policy<In>::value, int>::type = 0>
-Out copy_n(In first, Size n, Out out) { return copy(first, first + n, out); }
+
 template <class In, class Out>
 Out copy(const system::cpp::detail::par_t&, In first, In last, Out out) { return std::copy(first, last, out); }
 template <class In, class Out,
@@ -126,4 +123,8 @@ Out copy(In first, In last, Out out) {
   system::cdna4::detail::copy_bytes(host.data(), tmp, n * sizeof(V), 1);
   return std::copy(host.begin(), host.end(), out);
 }
+template <class Policy, class In, class Size, class Out, detail::enable_if_policy<Policy> = 0>
+Out copy_n(const Policy& exec, In first, Size n, Out out) { return thrust::copy(exec, first, first + n, out); }
+template <class In, class Size, class Out, typename std::enable_if<!detail::is_policy<In>::value, int>::type = 0>
+Out copy_n(In first, Size n, Out out) { return thrust::copy(first, first + n, out); }
 }  // namespace thrust
