@@ -18,7 +18,7 @@ namespace thrust { namespace system { namespace cdna4 { namespace detail {
 #else
 template <class T> struct needs_hipcc { static constexpr bool value = sizeof(T) == 0; };
 #define THRUST_CDNA4_NEEDS_HIPCC(T)                                                                        \
-  static_assert(needs_hipcc<T>::value,                                                                     \
+  static_assert(::thrust::system::cdna4::detail::needs_hipcc<T>::value,                                     \
                 "cdna4: algorithms with user functors on device ranges are kernel templates; compile this " \
                 "translation unit with hipcc --offload-arch=gfx950")
 #endif

@@ -158,3 +158,16 @@ def test_select_family_on_host_ranges_builds_with_gxx(tmp_path):
                      auto p = thrust::unique_by_key(h.begin(), h.end(), v.begin());
                      return (int)((e - o.begin()) + (r - h.begin()) + (u - h.begin()) + (p.first - h.begin())); }""")
     assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_every_public_header_compiles_on_its_own(tmp_path):
+    """Each header under include/thrust (not detail/) is self-contained under g++."""
+    import glob
+    headers = sorted(h for h in glob.glob(os.path.join(INC, "thrust", "**", "*.h"), recursive=True) if "/detail/" not in h)
+    assert len(headers) > 40
+    body = "".join('#include <%s>\n' % os.path.relpath(h, INC) for h in headers) + "int main() { return 0; }\n"
+    r = compile_snippet(tmp_path, body)
+    assert r.returncode == 0, r.stderr[-3000:]
+    for h in headers:  # and each one alone
+        r = compile_snippet(tmp_path, '#include <%s>\nint main() { return 0; }\n' % os.path.relpath(h, INC))
+        assert r.returncode == 0, (h, r.stderr[-2000:])
