@@ -200,3 +200,36 @@ def test_by_key_aliased_outputs_take_the_ticket_path():
     gk, gv = thrust_amd.reduce_by_key(dk, dv, keys_out=dk, values_out=dv)  # compaction in place
     rk, rv = oracle.reduce_by_key(k, v)
     assert same_bits(host(gk), rk) and same_bits(host(gv), rv)
+
+
+def piecewise_keys(seed, n, kd):
+    """Stretches of very different run lengths side by side: none (one long run), 1 in 1000, 1 in 10,
+    just below and just above every second element, every element.  A wavefront of a tile handles
+    its heads one way when they are few and another when they are many; both, and wavefronts with
+    no head at all, meet inside one input."""
+    rng = np.random.default_rng(seed)
+    densities = [0.0, 0.001, 0.1, 0.47, 0.49, 0.6, 1.0, 0.0, 0.3]
+    piece = -(-n // len(densities))
+    head = np.concatenate([rng.random(piece) < d if d < 1.0 else np.ones(piece, bool) for d in densities])[:n]
+    ids = np.cumsum(head)
+    if np.dtype(kd).kind == "f":
+        return ids.astype(kd)
+    return (ids % 97).astype(kd)  # neighbours still differ at every head
+
+
+@pytest.mark.parametrize("kd,vd", [(np.int32, np.int32), (np.int64, np.int32), (np.int32, np.int64),
+                                   (np.uint8, np.uint16), (np.float32, np.float64), (np.uint16, np.int8)])
+def test_by_key_mixed_run_lengths_match_oracle(kd, vd):
+    for n in (9 * 40000 + 123, 9 * 2048 * 3):
+        k = piecewise_keys(n, n, kd)
+        is_fp = np.dtype(vd).kind == "f"
+        v = (np.random.default_rng(n).integers(-50, 50, n)).astype(vd) if is_fp else random_ints(n + 1, n, vd)
+        dk, dv = dev(k), dev(v)
+        for op in ("plus", "maximum", "minimum"):
+            ko, vo = thrust_amd.reduce_by_key(dk, dv, op=op)
+            rk, rv = oracle.reduce_by_key(k, v, op=op)
+            assert same_bits(host(ko), rk), (n, op)
+            assert same_bits(host(vo), rv), (n, op)  # small integers: exact in floating point too
+            assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op=op)), oracle.scan_by_key(k, v, op=op)), (n, op)
+        assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=3)),
+                         oracle.scan_by_key(k, v, exclusive=True, init=3)), n

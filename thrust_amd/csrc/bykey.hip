@@ -227,6 +227,7 @@ struct SegTile {
   KU key[CHUNKS][VEC];
   T val[CHUNKS][VEC];
   uint32_t heads[CHUNKS];
+  Pair excl_w[CHUNKS];  // everything before the thread's group within its wavefront's part of chunk c
   Pair off[CHUNKS];
   int64_t base;
   int64_t tile;
@@ -242,9 +243,9 @@ struct SegTile {
   // by an atomic counter (every tile waited for has started; used when an output overlaps an
   // input); otherwise a tile is the workgroup of the same index and a descriptor that stays
   // missing after `patience` polls is recomputed from the input.
-  template <bool TICKET>
+  template <bool TICKET, class Meanwhile>
   __device__ void run(Smem& sm, const KU* keys, const T* vals, int64_t n, int float_keys, int vec_ok,
-                      uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf, int patience) {
+                      uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf, int patience, Meanwhile meanwhile) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -297,7 +298,6 @@ struct SegTile {
       prev[c] = (KU)wave_shift_up1((KW)key[c][VEC - 1], (KW)first);
     }
 
-    Pair excl_w[CHUNKS];
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
       const int64_t i0 = index(c, 0);
@@ -320,16 +320,19 @@ struct SegTile {
 
     // wave 0: scan of the (chunk, wave) totals in tile order, look-back, then each (chunk, wave)'s
     // prefix over the whole input goes back into the table
+    Pair tile_agg = idp, before = idp;
     if (wave == 0) {
       const Pair mine = lane < CHUNKS * NWAVES ? sm.tot[lane] : idp;
       const Pair incl = wave_inclusive_scan(mine, idp, comb);
-      const Pair tile_agg = readlane(incl, kWave - 1);
-      const Pair before = wave_shift_up1(incl, idp);
+      tile_agg = readlane(incl, kWave - 1);
+      before = wave_shift_up1(incl, idp);
+      if (lane == 0) TileDesc<Pair>::store(desc, tile, tile == 0 ? kInclusive : kPartial, tile_agg);
+    }
+    // work that needs nothing from earlier tiles runs while their aggregates arrive
+    meanwhile();
+    if (wave == 0) {
       Pair prefix = idp;
-      if (tile == 0) {
-        if (lane == 0) TileDesc<Pair>::store(desc, 0, kInclusive, tile_agg);
-      } else {
-        if (lane == 0) TileDesc<Pair>::store(desc, tile, kPartial, tile_agg);
+      if (tile != 0) {
         if constexpr (TICKET) {
           prefix = wave_lookback<Pair>(desc, tile, idp, comb);
         } else {
@@ -375,8 +378,64 @@ __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_
   __shared__ tcd_v4u s_x[G::BLOCKED ? G::NWAVES : 1][G::XPOSE_SLOTS];
   tcd_v4u* xbuf = s_x[G::BLOCKED ? threadIdx.x / kWave : 0];
   ST t;
-  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience);
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS;
+  // Whole tiles of the blocked layout: each wavefront scans its elements from the wavefront's
+  // own start and parks the result in its buffer (in the order of the later contiguous stores)
+  // BEFORE the look-back.  Afterwards only the elements of the run that came into the wavefront
+  // open (those before its first head, `first_head` of them) still take the value of that run
+  // so far; the four operators are commutative, so it is applied on top of the parked result.
+  constexpr int NQ = G::BLOCKED ? VEC * (int)sizeof(T) / 16 : 1;
+  constexpr int EPP = 16 / (int)sizeof(T);  // elements per 16-byte slot
+  bool parked = false;
+  uint32_t first_head = 0;
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, [&] {
+    if constexpr (G::BLOCKED) {
+      if (!t.full) return;
+      parked = true;
+      const int lane = threadIdx.x & (kWave - 1);
+      T r[VEC];
+      T open = t.excl_w[0].v;
+#pragma unroll
+      for (int j = 0; j < VEC; j++) {
+        const bool is_head = (t.heads[0] >> j) & 1u;
+        const T x = t.val[0][j];
+        if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
+        open = is_head ? x : Op::template apply<T>(open, x);
+        if (!exclusive) r[j] = open;
+      }
+      const uint64_t has = __ballot(t.heads[0] != 0u);
+      first_head = kWave * VEC;
+      if (has) {
+        const int owner = __builtin_ctzll(has);
+        first_head = (uint32_t)(owner * VEC + __builtin_ctz((uint32_t)__builtin_amdgcn_readlane((int)t.heads[0], owner)));
+      }
+#pragma unroll
+      for (int i = 0; i < NQ; i++) {
+        tcd_v4u piece;
+        __builtin_memcpy(&piece, reinterpret_cast<const char*>(r) + 16 * i, 16);
+        xbuf[xpose_slot(lane * NQ + i)] = piece;
+      }
+    }
+  });
+  if (parked) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const T carried = sm.tot[wave].v;  // the open run's value over everything before the wavefront
+    char* dst = reinterpret_cast<char*>(out + t.base + (int64_t)wave * (kWave * VEC));
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+      tcd_v4u piece = xbuf[xpose_slot(q * kWave + lane)];
+      if ((uint32_t)(q * kWave * EPP) < first_head) {  // wave-uniform
+        T x[EPP];
+        __builtin_memcpy(x, &piece, 16);
+#pragma unroll
+        for (int e = 0; e < EPP; e++)
+          if ((uint32_t)((q * kWave + lane) * EPP + e) < first_head) x[e] = Op::template apply<T>(carried, x[e]);
+        __builtin_memcpy(&piece, x, 16);
+      }
+      store16(dst + (q * kWave + lane) * 16, piece);
+    }
+    return;
+  }
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
     T r[VEC];
@@ -424,20 +483,69 @@ __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce
     __shared__ tcd_v4u s_x[NWAVES][G::XPOSE_SLOTS];
     tcd_v4u* xbuf = s_x[threadIdx.x / kWave];
     ST t;
-    t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience);
+    // Slot i lives at sw(i): when most elements are heads a thread's slots start VEC apart, which
+    // is one LDS bank for all lanes; the swizzle (within aligned groups of VEC slots) spreads them
+    // and the copy-out reads over all banks.
+    constexpr uint32_t kLogVec = VEC == 32 ? 5 : 4;
+    static_assert((1u << kLogVec) == (uint32_t)VEC, "VEC is 16 or 32");
+    const auto sw = [](uint32_t i) { return i ^ ((i >> kLogVec) & (uint32_t)(VEC - 1)); };
+    // A wavefront with few enough heads compacts them BEFORE the look-back, while the aggregates
+    // of earlier tiles are still on their way: keys into the lower half of its buffer, the values
+    // of the runs they close into the upper half.  Only the output position and the start of the
+    // run open at the wavefront's first element depend on earlier tiles; both are applied during
+    // the copy-out.  (Not in the last tile, which also closes the last run.)
+    constexpr uint32_t kHalfBytes = G::XPOSE_SLOTS * 16 / 2;
+    constexpr uint32_t kEarlyMax = kHalfBytes / (sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T)) - VEC;
+    KU* const early_k = reinterpret_cast<KU*>(xbuf);
+    T* const early_v = reinterpret_cast<T*>(reinterpret_cast<char*>(xbuf) + kHalfBytes);
+    bool early = false;
+    uint32_t count = 0;
+    t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, [&] {
+      count = (uint32_t)__builtin_amdgcn_readlane((int)(t.excl_w[0].c + __builtin_popcount(t.heads[0])), kWave - 1);
+      early = t.full && count <= kEarlyMax;
+      if (!early) {
+        if (t.full) {  // the keys alone always fit
+          uint32_t slot = t.excl_w[0].c;
+#pragma unroll
+          for (int j = 0; j < VEC; j++)
+            if ((t.heads[0] >> j) & 1u) early_k[sw(slot++)] = t.key[0][j];
+        }
+        return;
+      }
+      uint32_t slot = t.excl_w[0].c;
+      T open = t.excl_w[0].v;  // the open run's value over the wavefront's earlier elements
+#pragma unroll
+      for (int j = 0; j < VEC; j++) {
+        if ((t.heads[0] >> j) & 1u) {
+          early_k[sw(slot)] = t.key[0][j];
+          early_v[sw(slot)] = open;
+          slot++;
+          open = t.val[0][j];
+        } else {
+          open = Op::template apply<T>(open, t.val[0][j]);
+        }
+      }
+    });
+    if (early) {
+      const SegPair<T> before_wave = sm.tot[threadIdx.x / kWave];
+      const uint32_t first = before_wave.c;
+      for (uint32_t i = lane; i < count; i += kWave) {
+        keys_out[first + i] = early_k[sw(i)];
+        T v = early_v[sw(i)];
+        if (i == 0) v = Op::template apply<T>(before_wave.v, v);  // the run came into the wavefront open
+        if (first + i) vals_out[first + i - 1] = v;
+      }
+      return;
+    }
     SegPair<T> run = t.off[0];  // (runs started so far, value of the open run) before the current element
     const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)run.c);  // runs before this wavefront
     const uint32_t heads = t.heads[0];
     const uint32_t mine = run.c - first;  // slot of this thread's first head
-    const uint32_t count = (uint32_t)__builtin_amdgcn_readlane((int)(mine + __builtin_popcount(heads)), kWave - 1);
     const int64_t i0 = t.index(0, 0);
-    // Slot i lives at sw(i): when most elements are heads a thread's slots start VEC apart, which
-    // is one LDS bank for all lanes; the swizzle spreads them (and the copy-out reads) over all.
-    constexpr uint32_t kLogVec = VEC == 32 ? 5 : 4;
-    static_assert((1u << kLogVec) == (uint32_t)VEC, "VEC is 16 or 32");
-    const auto sw = [](uint32_t i) { return i ^ ((i >> kLogVec) & (uint32_t)(VEC - 1)); };
+    // Too many heads for both halves (or the last tile): the values go through the buffer after
+    // the keys.  A whole tile's keys were compacted before the look-back.
     KU* sk = reinterpret_cast<KU*>(xbuf);
-    {
+    if (!t.full) {
       uint32_t slot = mine;
 #pragma unroll
       for (int j = 0; j < VEC; j++)
@@ -477,7 +585,7 @@ __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce
   __shared__ KU s_keys[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
   __shared__ T s_vals[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
   ST t;
-  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, nullptr, patience);
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, nullptr, patience, [] {});
   KU* sk = s_keys[G::BLOCKED ? 0 : threadIdx.x / kWave];
   T* sv = s_vals[G::BLOCKED ? 0 : threadIdx.x / kWave];
 #pragma unroll
