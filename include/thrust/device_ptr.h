@@ -18,8 +18,7 @@ class device_reference {
   explicit device_reference(T* p) : p_(p) {}
   operator value_type() const {
     value_type v;
-    system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_dtoh(&v, p_, sizeof(T), nullptr), "get_value");
-    system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "get_value");
+    system::cdna4::detail::throw_on_error(thrust_cdna4_read_back(&v, p_, sizeof(T), nullptr), "get_value");
     return v;
   }
   device_reference& operator=(const value_type& v) {

@@ -112,8 +112,7 @@ class device_future : public device_event {
     if (!have_) {
       if (!data_) throw std::logic_error("thrust::device_future: no state");
       wait();
-      system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_dtoh(&value_, data_, sizeof(T), stream()), "future: read back");
-      wait();
+      system::cdna4::detail::throw_on_error(thrust_cdna4_read_back(&value_, data_, sizeof(T), stream()), "future: read back");
       have_ = true;
     }
     return value_;

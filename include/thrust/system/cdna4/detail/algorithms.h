@@ -134,8 +134,7 @@ std::int64_t reduce_by_key(const Policy& exec, const K* keys, const T* vals, K* 
   throw_on_error(thrust_cdna4_reduce_by_key(tmp.data(), &bytes, dtype_of<K>::value, dtype_of<T>::value, op_code<Op>::value,
                                             keys, vals, keys_out, vals_out, d_runs, n, s), "reduce_by_key: launch");
   std::int64_t runs = 0;
-  throw_on_error(thrust_cdna4_memcpy_dtoh(&runs, d_runs, sizeof(runs), s), "reduce_by_key: read run count");
-  synchronize(exec, "reduce_by_key: failed to synchronize");
+  throw_on_error(thrust_cdna4_read_back(&runs, d_runs, sizeof(runs), s), "reduce_by_key: read run count");
   return runs;
 }
 

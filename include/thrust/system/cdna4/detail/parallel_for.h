@@ -134,8 +134,7 @@ T transform_reduce(void* stream_, std::int64_t n, Unary unary, T init, Op op) {
   hipLaunchKernelGGL((reduce_final_kernel<T, Op>), dim3(1), dim3(kBlock), 0, s, partial, (int)blocks, init, op, out);
   throw_on_error((int)hipGetLastError(), "reduce: launch");
   T result;
-  throw_on_error(thrust_cdna4_memcpy_dtoh(&result, out, sizeof(T), stream_), "reduce: read back");
-  throw_on_error(thrust_cdna4_stream_synchronize(stream_), "reduce: failed to synchronize");
+  throw_on_error(thrust_cdna4_read_back(&result, out, sizeof(T), stream_), "reduce: read back");
   return result;
 }
 
@@ -321,8 +320,7 @@ std::int64_t select(void* stream_, std::int64_t n, Op op) {
   hipLaunchKernelGGL((select_kernel<Op>), dim3((unsigned)tiles), dim3(kSelBlock), 0, s, n, op, words, tiles);
   throw_on_error((int)hipGetLastError(), "select: launch");
   unsigned long long kept = 0;
-  throw_on_error(thrust_cdna4_memcpy_dtoh(&kept, words + tiles + 1, sizeof(kept), stream_), "select: read back");
-  throw_on_error(thrust_cdna4_stream_synchronize(stream_), "select: failed to synchronize");
+  throw_on_error(thrust_cdna4_read_back(&kept, words + tiles + 1, sizeof(kept), stream_), "select: read back");
   return (std::int64_t)kept;
 }
 

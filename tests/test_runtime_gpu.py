@@ -86,3 +86,38 @@ def test_streams_and_events_order_work_across_streams():
     capi.check(L.thrust_cdna4_stream_destroy(s2), "stream_destroy")
     assert L.thrust_cdna4_stream_destroy(None) != 0  # the default stream is not ours to destroy
     assert L.thrust_cdna4_event_record(None, None) != 0
+
+
+def test_read_back_waits_for_the_stream_and_handles_every_size():
+    """Small results go through the thread's pinned buffer, larger ones straight to the
+    destination; either way the bytes are there when the call returns, also when the producing
+    work was only just enqueued on another stream, and from a second host thread."""
+    import threading
+
+    L = capi.lib()
+    side = torch.cuda.Stream()
+    for nbytes in (1, 8, 4096, 4097, 1 << 20):
+        with torch.cuda.stream(side):
+            src = torch.arange(nbytes, device="cuda", dtype=torch.int64).to(torch.uint8)  # enqueued, not waited for
+            dst = np.zeros(nbytes, dtype=np.uint8)
+            capi.check(L.thrust_cdna4_read_back(vp(dst.ctypes.data), vp(src.data_ptr()), nbytes, vp(side.cuda_stream)),
+                       "read_back")
+        assert np.array_equal(dst, np.arange(nbytes, dtype=np.int64).astype(np.uint8)), nbytes
+    capi.check(L.thrust_cdna4_read_back(None, None, 0, None), "read_back of nothing")
+    assert L.thrust_cdna4_read_back(None, None, 8, None) != 0
+
+    src = torch.full((16,), 7, device="cuda", dtype=torch.int32)
+    torch.cuda.synchronize()
+    got = {}
+
+    def worker(i):
+        out = np.zeros(16, dtype=np.int32)
+        rc = L.thrust_cdna4_read_back(vp(out.ctypes.data), vp(src.data_ptr()), 64, None)
+        got[i] = (rc, out.copy())
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert all(rc == 0 and (out == 7).all() for rc, out in got.values()) and len(got) == 4

@@ -18,7 +18,7 @@ SYMBOLS = [
     "thrust_cdna4_sort_pairs", "thrust_cdna4_scan", "thrust_cdna4_scan_by_key",
     "thrust_cdna4_reduce_by_key", "thrust_cdna4_histogram_even", "thrust_cdna4_malloc",
     "thrust_cdna4_free", "thrust_cdna4_pool_trim", "thrust_cdna4_pool_bytes",
-    "thrust_cdna4_memcpy_htod", "thrust_cdna4_memcpy_dtoh", "thrust_cdna4_memcpy_dtod",
+    "thrust_cdna4_memcpy_htod", "thrust_cdna4_memcpy_dtoh", "thrust_cdna4_memcpy_dtod", "thrust_cdna4_read_back",
     "thrust_cdna4_fill", "thrust_cdna4_stream_synchronize", "thrust_cdna4_profile_enable",
     "thrust_cdna4_profile_count", "thrust_cdna4_profile_get",
     "thrust_cdna4_selftest_lds_atomic_order", "thrust_cdna4_set_lookback_patience",
@@ -65,6 +65,7 @@ def lib():
     L.thrust_cdna4_pool_bytes.restype = sz
     L.thrust_cdna4_memcpy_htod.argtypes = [vp, vp, sz, vp]
     L.thrust_cdna4_memcpy_dtoh.argtypes = [vp, vp, sz, vp]
+    L.thrust_cdna4_read_back.argtypes = [vp, vp, sz, vp]
     L.thrust_cdna4_memcpy_dtod.argtypes = [vp, vp, sz, vp]
     L.thrust_cdna4_fill.argtypes = [vp, vp, i32, i64, vp]
     L.thrust_cdna4_stream_synchronize.argtypes = [vp]

@@ -4,6 +4,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include <cstring>
 #include "common.h"
 #include <atomic>
 
@@ -258,6 +259,34 @@ extern "C" int thrust_cdna4_memcpy_htod(void* dst, const void* src, size_t bytes
 extern "C" int thrust_cdna4_memcpy_dtoh(void* dst, const void* src, size_t bytes, void* stream) {
   if (bytes == 0) return hipSuccess;
   return hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream));
+}
+namespace tcd {
+// One pinned bounce buffer per host thread, allocated at its first read-back and kept until the
+// process ends.
+struct PinnedSlot {
+  static constexpr size_t kBytes = 4096;
+  void* p = nullptr;
+  void* get() {
+    if (!p && hipHostMalloc(&p, kBytes, hipHostMallocPortable) != hipSuccess) {
+      (void)hipGetLastError();
+      p = nullptr;
+    }
+    return p;
+  }
+};
+static thread_local PinnedSlot t_slot;
+}  // namespace tcd
+extern "C" int thrust_cdna4_read_back(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return hipSuccess;
+  if (!dst || !src) return hipErrorInvalidValue;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  void* slot = bytes <= tcd::PinnedSlot::kBytes ? tcd::t_slot.get() : nullptr;
+  hipError_t e = hipMemcpyAsync(slot ? slot : dst, src, bytes, hipMemcpyDeviceToHost, s);
+  if (e != hipSuccess) return (int)e;
+  e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return (int)e;
+  if (slot) std::memcpy(dst, slot, bytes);
+  return hipSuccess;
 }
 // Device-to-device copy: one 16-byte load and store per thread, many small workgroups.  On
 // MI355X this plain shape streams faster than longer per-thread loops and than the runtime's
