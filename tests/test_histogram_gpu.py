@@ -55,7 +55,7 @@ def test_histogram_all_types_general_ranges(dtype):
         s = rng.integers(max(info.min, -300), min(info.max, 300), n, endpoint=True).astype(dtype)
     for bins, lo, hi in [(7, -100.0, 100.0), (256, -128.0, 128.0), (257, -100.0, 157.0), (512, -256.0, 256.0),
                          (513, -256.0, 257.0), (1000, 0.0, 250.0), (8192, -300.0, 300.0), (2048, -64.0, 64.0), (2049, -64.0, 64.0),
-                         (16384, -300.0, 300.0), (70000, -300.5, 300.5)]:
+                         (4097, -300.0, 300.0), (8193, -300.0, 300.0), (16384, -300.0, 300.0), (70000, -300.5, 300.5)]:
         got = counts(thrust_amd.histogram_even(dev(s), bins, lo, hi))
         assert same_bits(got, oracle.histogram_even(s, bins, lo, hi)), (bins, lo, hi)
 

@@ -7,7 +7,7 @@
 //   bin = (int)((v - lower) * scale), scale = num_bins / (upper - lower), clamped to num_bins-1.
 //
 // LDS layout: counter of (bin, copy) at word bin*copies + copy, copy = lane % copies, copies a
-// power of two <= 32.  With 32 copies (up to 512 bins) lane l always hits bank l % 32: no bank
+// power of two <= 32.  With 32 copies (up to 256 bins) lane l always hits bank l % 32: no bank
 // conflicts and no two lanes of a half-wave on one address, whatever the data (uniform, a few
 // hot bins, constant).  Fewer copies (more bins) get one padding word per 32 so that bins hit
 // with a power-of-two stride do not fall into a few banks; there, samples that share a bin
@@ -39,11 +39,17 @@ __global__ __launch_bounds__(kHistBlock) void histogram_kernel(const T* __restri
                                                                double upper, double scale, int copies_log2,
                                                                int vec_ok) {
   constexpr int VEC = 16 / sizeof(T);
-  constexpr int kHistUnroll = sizeof(T) <= 2 ? 4 : 2;  // independent 128-bit loads in flight per thread
+  // independent 128-bit loads in flight per thread.  1-byte samples: eight, with ONE workgroup
+  // per CU — the per-sample LDS instruction (16 per load) is the scarce resource there, and few
+  // wavefronts with deep queues of loads measured 25 % faster than many with shallow ones.
+  constexpr int kHistUnroll = sizeof(T) == 1 ? 8 : sizeof(T) == 2 ? 4 : 2;
   __shared__ uint32_t s_hist[LDS > 0 ? LDS + LDS / 32 : 1];
   __shared__ uint32_t s_out[MODE == 2 ? 256 : 1];
   const int tid = threadIdx.x;
   const int lds_bins = MODE == 2 ? 256 : num_bins;  // counters kept per copy
+  // byte counting (MODE 2) always has 32 unpadded copies: known at compile time, which keeps the
+  // per-sample address arithmetic at one shift-or
+  if constexpr (MODE == 2) copies_log2 = 5;
   const int copies = 1 << copies_log2;
   const bool padded = copies < 32;
   const uint32_t my_copy = (uint32_t)tid & (uint32_t)(copies - 1);
@@ -181,13 +187,16 @@ static hipError_t histogram_typed(const void* samples_, int64_t n, uint32_t* cou
   const T* samples = static_cast<const T*>(samples_);
   const double scale = (double)num_bins / (upper - lower);
   const int vec_ok = (reinterpret_cast<uintptr_t>(samples) & 15) == 0;
-  // two LDS footprints: 32 KiB while 32 copies of every counter fit (always the case for 1-byte
-  // samples), 64 KiB up to 16384 bins; beyond that the counts go straight to global memory.
-  // Workgroups per CU as measured: four for 1-byte samples, two otherwise.
+  // Two LDS footprints: 8192 counters (32 KiB, plus padding) up to 8192 bins — as many copies of
+  // every counter as fit, 32 up to 256 bins, 2 at 4096 — and 16384 counters up to 16384 bins;
+  // beyond that the counts go straight to global memory.  Workgroups per CU as measured on
+  // MI355X at 2^30 samples: one for 1-byte samples (see kHistUnroll), three with the small
+  // footprint (2^30 floats into 256 / 4096 bins: 0.66 ms against 0.74 ms with two workgroups of
+  // the large one, Zipf or uniform; four are slower again), two with the large one.
   if constexpr (sizeof(T) == 1) {
-    launch_hist<T, 8192, 2>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 4, s);
-  } else if (num_bins <= 256) {
-    launch_hist<T, 8192, 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 2, s);
+    launch_hist<T, 8192, 2>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 1, s);
+  } else if (num_bins <= 8192) {
+    launch_hist<T, 8192, 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 3, s);
   } else if (num_bins <= kHistLdsWords) {
     launch_hist<T, kHistLdsWords, 0>(samples, n, counts, num_bins, lower, upper, scale, vec_ok, 2, s);
   } else {
