@@ -9,9 +9,9 @@
 // and the comparator's operator() must be __host__ __device__.  Temporary storage comes from
 // the library's stream-ordered pool.
 //
-//   1. block_sort_kernel   a workgroup of kBlock threads sorts a tile of kBlock*kIpt items (512 x 4
-//                          measured best: the per-thread serial merge is the critical path, so
-//                          few items per thread and many threads): every thread
+//   1. block_sort_kernel   a workgroup of kBlock threads sorts a tile of kBlock*kIpt items (512
+//                          threads; 8 items per thread for narrow keys alone, else 4: the
+//                          per-thread search and serial merge are the critical path): every thread
 //                          sorts its kIpt consecutive items in registers (odd-even transposition,
 //                          stable), then log2(kBlock) rounds of merge-path merging through LDS.
 //   2. merge_partition_kernel + merge_kernel, once per doubling of the run width: one thread
@@ -35,12 +35,20 @@ namespace thrust { namespace system { namespace cdna4 { namespace detail { names
 #define THRUST_CDNA4_MERGE_BLOCK 512
 #endif
 constexpr int kBlock = THRUST_CDNA4_MERGE_BLOCK;  // threads per workgroup
+// Items per thread: a template parameter of the kernels, chosen by the host from the item size.
+// Eight for keys of up to 4 bytes sorted alone (the merge-path search is paid once per thread, so
+// more items amortise it: 3.4 ms against 4.0 ms for 2^26 uint32 keys), four otherwise (pairs gain
+// nothing from eight, and a tile of wide items would not fit LDS).
+#ifndef THRUST_CDNA4_MERGE_IPT_NARROW
+#define THRUST_CDNA4_MERGE_IPT_NARROW 8
+#endif
 #ifndef THRUST_CDNA4_MERGE_IPT
 #define THRUST_CDNA4_MERGE_IPT 4
 #endif
-constexpr int kIpt = THRUST_CDNA4_MERGE_IPT;  // items per thread
-constexpr int kTile = kBlock * kIpt;
-static_assert((kIpt & (kIpt - 1)) == 0 && kTile <= 65536, "run widths double from kIpt; 16-bit positions in a tile");
+template <class K, class V>
+constexpr int items_per_thread() {
+  return (std::is_empty<V>::value && sizeof(K) <= 4) ? THRUST_CDNA4_MERGE_IPT_NARROW : THRUST_CDNA4_MERGE_IPT;
+}
 
 struct no_value {};
 
@@ -62,10 +70,10 @@ __device__ inline void settle(const T& x) {
 // 16-byte words and the array is 16-byte aligned, it moves with 128-bit accesses (a wavefront then
 // touches every byte of the lines it writes with one instruction instead of a quarter of them
 // with each of four).
-template <class T>
-struct alignas(16) item_block { T v[kIpt]; };
-template <class T>
-constexpr bool blockable() { return sizeof(item_block<T>) == sizeof(T) * kIpt; }
+template <class T, int IPT>
+struct alignas(16) item_block { T v[IPT]; };
+template <class T, int IPT>
+constexpr bool blockable() { return sizeof(item_block<T, IPT>) == sizeof(T) * IPT; }
 template <class T>
 __device__ inline bool block_aligned(const T* p) { return (reinterpret_cast<std::uintptr_t>(p) & 15) == 0; }
 
@@ -86,8 +94,10 @@ __device__ inline int merge_path(const K* a, int na, const K* b, int nb, int dia
 // ---------------------------------------------------------------------------------------
 // 1. Tile sort
 // ---------------------------------------------------------------------------------------
-template <class K, class V, class Compare>
+template <int IPT, class K, class V, class Compare>
 __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, std::int64_t n, Compare comp) {
+  constexpr int kIpt = IPT, kTile = kBlock * IPT;
+  static_assert((kIpt & (kIpt - 1)) == 0 && kTile <= 65536, "run widths double from kIpt; 16-bit positions in a tile");
   constexpr bool kHasValues = !std::is_same<V, no_value>::value;
   __shared__ K s_keys[kTile];
   __shared__ std::uint16_t s_idx[kTile];
@@ -108,8 +118,8 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
   K k[kIpt];
   int idx[kIpt];
   const bool whole = valid == kTile;
-  if (whole && blockable<K>() && block_aligned(keys)) {
-    const item_block<K> blk = *reinterpret_cast<const item_block<K>*>(keys + base + tid * kIpt);
+  if (whole && blockable<K, IPT>() && block_aligned(keys)) {
+    const item_block<K, IPT> blk = *reinterpret_cast<const item_block<K, IPT>*>(keys + base + tid * kIpt);
 #pragma unroll
     for (int j = 0; j < kIpt; j++) {
       idx[j] = tid * kIpt + j;
@@ -190,17 +200,17 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
 
   // the first `valid` outputs are the real items, in order
   __syncthreads();
-  if (whole && blockable<K>() && block_aligned(keys)) {
-    item_block<K> blk;
+  if (whole && blockable<K, IPT>() && block_aligned(keys)) {
+    item_block<K, IPT> blk;
 #pragma unroll
     for (int j = 0; j < kIpt; j++) blk.v[j] = k[j];
-    *reinterpret_cast<item_block<K>*>(keys + base + tid * kIpt) = blk;
+    *reinterpret_cast<item_block<K, IPT>*>(keys + base + tid * kIpt) = blk;
     if constexpr (kHasValues) {
-      if (blockable<V>() && block_aligned(values)) {
-        item_block<V> vb;
+      if (blockable<V, IPT>() && block_aligned(values)) {
+        item_block<V, IPT> vb;
 #pragma unroll
         for (int j = 0; j < kIpt; j++) vb.v[j] = s_vals[idx[j]];
-        *reinterpret_cast<item_block<V>*>(values + base + tid * kIpt) = vb;
+        *reinterpret_cast<item_block<V, IPT>*>(values + base + tid * kIpt) = vb;
       } else {
 #pragma unroll
         for (int j = 0; j < kIpt; j++) values[base + tid * kIpt + j] = s_vals[idx[j]];
@@ -224,7 +234,7 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
 struct pair_geometry {
   std::int64_t a0, na, b0, nb, diag;
 };
-__device__ inline pair_geometry geometry_of(std::int64_t tile, std::int64_t width, std::int64_t n) {
+__device__ inline pair_geometry geometry_of(std::int64_t tile, std::int64_t width, std::int64_t n, int kTile) {
   pair_geometry g;
   const std::int64_t out0 = tile * kTile;
   const std::int64_t pstart = out0 / (2 * width) * (2 * width);
@@ -239,13 +249,14 @@ __device__ inline pair_geometry geometry_of(std::int64_t tile, std::int64_t widt
 }
 
 // splits[t] = how many items of the left run precede output tile t (binary search in global memory)
-template <class K, class Compare>
+template <int IPT, class K, class Compare>
 __global__ __launch_bounds__(256) void merge_partition_kernel(const K* keys, std::int64_t n, std::int64_t width,
                                                               std::int64_t ntiles, std::int64_t* splits,
                                                               Compare comp) {
+  constexpr int kTile = kBlock * IPT;
   const std::int64_t t = (std::int64_t)blockIdx.x * 256 + threadIdx.x;
   if (t >= ntiles) return;
-  const pair_geometry g = geometry_of(t, width, n);
+  const pair_geometry g = geometry_of(t, width, n, kTile);
   const K* a = keys + g.a0;
   const K* b = keys + g.b0;
   std::int64_t lo = g.diag > g.nb ? g.diag - g.nb : 0;
@@ -258,17 +269,18 @@ __global__ __launch_bounds__(256) void merge_partition_kernel(const K* keys, std
   splits[t] = lo;
 }
 
-template <class K, class V, class Compare>
+template <int IPT, class K, class V, class Compare>
 __global__ __launch_bounds__(kBlock) void merge_kernel(const K* kin, const V* vin, K* kout, V* vout, std::int64_t n,
                                                        std::int64_t width, std::int64_t ntiles,
                                                        const std::int64_t* splits, Compare comp) {
+  constexpr int kIpt = IPT, kTile = kBlock * IPT;
   constexpr bool kHasValues = !std::is_same<V, no_value>::value;
   __shared__ K s_keys[kTile];
   __shared__ typename std::conditional<kHasValues, V, char>::type s_vals[kHasValues ? kTile : 1];
 
   const int tid = threadIdx.x;
   const std::int64_t tile = blockIdx.x;
-  const pair_geometry g = geometry_of(tile, width, n);
+  const pair_geometry g = geometry_of(tile, width, n, kTile);
   const std::int64_t total = g.na + g.nb;                                 // outputs of the pair
   const int count = (int)(total - g.diag < kTile ? total - g.diag : kTile);  // outputs of this tile
   // left-run items before this tile and before the next one (the pair's last tile takes the rest)
@@ -311,21 +323,21 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(const K* kin, const V* vi
   }
   const std::int64_t out0 = tile * kTile;
   if (count == kTile) {  // a whole tile: every thread has kIpt outputs
-    if (blockable<K>() && block_aligned(kout)) {
-      item_block<K> blk;
+    if (blockable<K, IPT>() && block_aligned(kout)) {
+      item_block<K, IPT> blk;
 #pragma unroll
       for (int j = 0; j < kIpt; j++) blk.v[j] = k[j];
-      *reinterpret_cast<item_block<K>*>(kout + out0 + d) = blk;
+      *reinterpret_cast<item_block<K, IPT>*>(kout + out0 + d) = blk;
     } else {
 #pragma unroll
       for (int j = 0; j < kIpt; j++) kout[out0 + d + j] = k[j];
     }
     if constexpr (kHasValues) {
-      if (blockable<V>() && block_aligned(vout)) {
-        item_block<V> blk;
+      if (blockable<V, IPT>() && block_aligned(vout)) {
+        item_block<V, IPT> blk;
 #pragma unroll
         for (int j = 0; j < kIpt; j++) blk.v[j] = s_vals[src[j]];
-        *reinterpret_cast<item_block<V>*>(vout + out0 + d) = blk;
+        *reinterpret_cast<item_block<V, IPT>*>(vout + out0 + d) = blk;
       } else {
 #pragma unroll
         for (int j = 0; j < kIpt; j++) vout[out0 + d + j] = s_vals[src[j]];
@@ -351,13 +363,15 @@ template <class K, class V, class Compare>
 void stable_sort(void* stream_, K* keys, V* values, std::int64_t n, Compare comp) {
   static_assert(std::is_trivially_copyable<K>::value, "cdna4 merge sort: keys must be trivially copyable");
   static_assert(std::is_trivially_copyable<V>::value, "cdna4 merge sort: values must be trivially copyable");
+  constexpr int IPT = items_per_thread<K, V>();
+  constexpr int kTile = kBlock * IPT;
   static_assert((sizeof(K) + sizeof(V) + 2) * kTile <= 65536, "cdna4 merge sort: a tile of keys and values must fit the 64 KiB of static LDS");
   constexpr bool kHasValues = !std::is_same<V, no_value>::value;
   if (n <= 1) return;
   hipStream_t s = static_cast<hipStream_t>(stream_);
   const std::int64_t ntiles = (n + kTile - 1) / kTile;
 
-  hipLaunchKernelGGL((block_sort_kernel<K, V, Compare>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, keys, values, n, comp);
+  hipLaunchKernelGGL((block_sort_kernel<IPT, K, V, Compare>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, keys, values, n, comp);
   throw_on_error((int)hipGetLastError(), "merge sort: tile sort launch");
   if (ntiles == 1) return;
 
@@ -372,9 +386,9 @@ void stable_sort(void* stream_, K* keys, V* values, std::int64_t n, Compare comp
 
   int cur = 0;
   for (std::int64_t width = kTile; width < n; width *= 2) {
-    hipLaunchKernelGGL((merge_partition_kernel<K, Compare>), dim3((unsigned)((ntiles + 255) / 256)), dim3(256), 0, s,
+    hipLaunchKernelGGL((merge_partition_kernel<IPT, K, Compare>), dim3((unsigned)((ntiles + 255) / 256)), dim3(256), 0, s,
                        kbuf[cur], n, width, ntiles, splits, comp);
-    hipLaunchKernelGGL((merge_kernel<K, V, Compare>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, kbuf[cur], vbuf[cur],
+    hipLaunchKernelGGL((merge_kernel<IPT, K, V, Compare>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, kbuf[cur], vbuf[cur],
                        kbuf[cur ^ 1], vbuf[cur ^ 1], n, width, ntiles, splits, comp);
     throw_on_error((int)hipGetLastError(), "merge sort: merge pass launch");
     cur ^= 1;

@@ -72,13 +72,19 @@ int main(int argc, char** argv) {
   const float ms_pairs = median_ms(run_pairs, restore, 5);
 
   // passes over the data: one tile sort + ceil(log2(n / tile)) merges, each reading and writing every item
-  int passes = 1;
-  for (std::size_t w = thrust::system::cdna4::detail::merge::kTile; w < n; w *= 2) passes++;
+  namespace ms = thrust::system::cdna4::detail::merge;
+  auto passes_of = [&](int items_per_thread) {
+    int p = 1;
+    for (std::size_t w = (std::size_t)ms::kBlock * items_per_thread; w < n; w *= 2) p++;
+    return p;
+  };
+  const int passes = passes_of(ms::items_per_thread<unsigned, ms::no_value>());
+  const int passes_pairs = passes_of(ms::items_per_thread<unsigned, unsigned>());
   std::printf(
       "{\"merge_sort_u32_custom_less\": {\"value\": %.3f, \"unit\": \"Gkeys/s\", \"ms\": %.3f, \"n\": %zu, \"passes\": %d, "
       "\"traffic_GBs\": %.1f, \"sorted\": %s}, \"merge_sort_by_key_u32_u32_custom_less\": {\"value\": %.3f, \"unit\": "
       "\"Gkeys/s\", \"ms\": %.3f, \"traffic_GBs\": %.1f}}\n",
       n / ms_keys / 1e6, ms_keys, n, passes, passes * 8.0 * n / ms_keys / 1e6, ok ? "true" : "false", n / ms_pairs / 1e6,
-      ms_pairs, passes * 16.0 * n / ms_pairs / 1e6);
+      ms_pairs, passes_pairs * 16.0 * n / ms_pairs / 1e6);
   return ok ? 0 : 1;
 }
