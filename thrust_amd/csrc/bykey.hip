@@ -231,7 +231,7 @@ struct SegTile {
   Pair off[CHUNKS];
   int64_t base;
   int64_t tile;
-  bool full;  // every element of the tile exists, the tile is not the last one, pointers are aligned
+  bool full;  // every element of the tile exists, the tile is not the last one, pointers are aligned to their elements
 
   __device__ int64_t index(int c, int j) const {
     return base + ((int64_t)c * BLOCK + threadIdx.x) * VEC + j;
@@ -653,8 +653,9 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
       if (rc != hipSuccess) return;
       T iv = T(0);
       if (init) __builtin_memcpy(&iv, init, sizeof(T));
-      const int vec_ok = ((reinterpret_cast<uintptr_t>(keys) | reinterpret_cast<uintptr_t>(values) |
-                           reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+      // 128-bit accesses need no more than the elements' own alignment (see load16)
+      const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & (sizeof(KU) - 1)) == 0 &&
+                         ((reinterpret_cast<uintptr_t>(values) | reinterpret_cast<uintptr_t>(out)) & (sizeof(T) - 1)) == 0;
       const int64_t ntiles = ceil_div(n, ScanByKeyGeom<T>::TILE);
       // an output that overlaps an input: tiles by ticket
       const bool aliased = ranges_overlap(out, (size_t)n * sizeof(T), values, (size_t)n * sizeof(T)) ||
@@ -699,7 +700,9 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
       }
       rc = zero_async(temp, need, s);
       if (rc != hipSuccess) return;
-      const int vec_ok = ((reinterpret_cast<uintptr_t>(keys_in) | reinterpret_cast<uintptr_t>(values_in)) & 15) == 0;
+      // 128-bit accesses need no more than the elements' own alignment (see load16)
+      const int vec_ok = (reinterpret_cast<uintptr_t>(keys_in) & (sizeof(KU) - 1)) == 0 &&
+                         (reinterpret_cast<uintptr_t>(values_in) & (sizeof(T) - 1)) == 0;
       const int64_t ntiles = ceil_div(n, ReduceByKeyGeom<T>::TILE);
       // an output that overlaps an input: tiles by ticket
       const size_t kb = (size_t)n * sizeof(KU), vb = (size_t)n * sizeof(T);

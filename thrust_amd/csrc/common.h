@@ -188,12 +188,18 @@ __device__ inline T wave_shift_up1(const T& incl, const T id) {
 #define TCD_NT 3  // bit 0: stores, bit 1: loads
 #endif
 typedef unsigned int tcd_v4u __attribute__((ext_vector_type(4)));
+// The same 16 bytes at ANY address in global memory: gfx950 under the HSA ABI runs with unaligned
+// global access enabled, and the compiler emits the one 128-bit instruction for this type as it
+// does for the aligned one.  load16 / store16 use it, so a range that starts a few elements into
+// an allocation (v.begin() + 1) takes the same vector paths as an aligned one; only LDS accesses
+// go through the aligned tcd_v4u.
+typedef tcd_v4u tcd_v4u_anywhere __attribute__((aligned(1)));
 template <class V, class E>
 __device__ inline V load16(const E* p) {
   static_assert(sizeof(V) == 16, "16-byte vector");
   tcd_v4u r;
-  if (TCD_NT & 2) r = __builtin_nontemporal_load(reinterpret_cast<const tcd_v4u*>(p));
-  else r = *reinterpret_cast<const tcd_v4u*>(p);
+  if (TCD_NT & 2) r = __builtin_nontemporal_load(reinterpret_cast<const tcd_v4u_anywhere*>(p));
+  else r = *reinterpret_cast<const tcd_v4u_anywhere*>(p);
   V v;
   __builtin_memcpy(&v, &r, 16);
   return v;
@@ -203,8 +209,8 @@ __device__ inline void store16(E* p, const V& v) {
   static_assert(sizeof(V) == 16, "16-byte vector");
   tcd_v4u r;
   __builtin_memcpy(&r, &v, 16);
-  if (TCD_NT & 1) __builtin_nontemporal_store(r, reinterpret_cast<tcd_v4u*>(p));
-  else *reinterpret_cast<tcd_v4u*>(p) = r;
+  if (TCD_NT & 1) __builtin_nontemporal_store(r, reinterpret_cast<tcd_v4u_anywhere*>(p));
+  else *reinterpret_cast<tcd_v4u_anywhere*>(p) = r;
 }
 
 // ---------------------------------------------------------------------------------------

@@ -186,7 +186,7 @@ static hipError_t histogram_typed(const void* samples_, int64_t n, uint32_t* cou
   if (e != hipSuccess || n == 0) return e;
   const T* samples = static_cast<const T*>(samples_);
   const double scale = (double)num_bins / (upper - lower);
-  const int vec_ok = (reinterpret_cast<uintptr_t>(samples) & 15) == 0;
+  const int vec_ok = (reinterpret_cast<uintptr_t>(samples) & (sizeof(T) - 1)) == 0;  // see load16
   // Two LDS footprints: 8192 counters (32 KiB, plus padding) up to 8192 bins — as many copies of
   // every counter as fit, 32 up to 256 bins, 2 at 4096 — and 16384 counters up to 16384 bins;
   // beyond that the counts go straight to global memory.  Workgroups per CU as measured on

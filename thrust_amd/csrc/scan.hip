@@ -54,7 +54,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     tile = s_tile;
   }
   const int64_t base = tile * TILE;
-  const bool fast = vec_ok && (base + TILE <= n);  // whole tile present, 16-byte aligned pointers
+  const bool fast = vec_ok && (base + TILE <= n);  // whole tile present, pointers aligned to their elements
   const T* tin = in + base + (int64_t)tid * VEC;
   T* tout = out + base + (int64_t)tid * VEC;
 
@@ -203,7 +203,8 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   if (init) __builtin_memcpy(&iv, init, sizeof(T));
   uint32_t* ticket = reinterpret_cast<uint32_t*>(temp);
   uint64_t* desc = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256);
-  const int vec_ok = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  // 128-bit accesses need no more than the elements' own alignment (see load16)
+  const int vec_ok = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & (sizeof(T) - 1)) == 0;
   if (ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T))) {
     TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS, true>), dim3((unsigned)ntiles), dim3(C::BLOCK),
                stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,

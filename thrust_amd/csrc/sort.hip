@@ -534,7 +534,7 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   hipError_t e = zero_async(t + plan.zero_begin, plan.zero_bytes, stream);
   if (e != hipSuccess) return e;
 
-  const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & 15) == 0;
+  const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & (sizeof(U) - 1)) == 0;  // see load16
   int64_t hblocks = ceil_div(n, kHistThreads * 64);
   if (hblocks > TCD_SORT_HIST_BLOCKS) hblocks = TCD_SORT_HIST_BLOCKS;  // two workgroups per CU
   TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(kHistThreads), stream,
