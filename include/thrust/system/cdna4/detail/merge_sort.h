@@ -66,16 +66,14 @@ __device__ inline void settle(const T& x) {
   for (int i = 0; i < NW; i++) asm volatile("" ::"v"(w[i]));
 }
 
-// A thread's kIpt consecutive items as one aligned block: when the block is a whole number of
-// 16-byte words and the array is 16-byte aligned, it moves with 128-bit accesses (a wavefront then
-// touches every byte of the lines it writes with one instruction instead of a quarter of them
-// with each of four).
+// A thread's kIpt consecutive items as one block: when the block is a whole number of 16-byte
+// words it moves with 128-bit accesses (a wavefront then touches every byte of the lines it
+// writes with one instruction instead of a quarter of them with each of four).  The copies are
+// memcpys at the items' own alignment, for which the compiler emits those accesses on gfx950.
 template <class T, int IPT>
 struct alignas(16) item_block { T v[IPT]; };
 template <class T, int IPT>
 constexpr bool blockable() { return sizeof(item_block<T, IPT>) == sizeof(T) * IPT; }
-template <class T>
-__device__ inline bool block_aligned(const T* p) { return (reinterpret_cast<std::uintptr_t>(p) & 15) == 0; }
 
 // Number of items the first `diag` outputs of merge(a[0,na), b[0,nb)) take from a, with ties
 // going to a (stability: a is the earlier run).
@@ -118,8 +116,9 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
   K k[kIpt];
   int idx[kIpt];
   const bool whole = valid == kTile;
-  if (whole && blockable<K, IPT>() && block_aligned(keys)) {
-    const item_block<K, IPT> blk = *reinterpret_cast<const item_block<K, IPT>*>(keys + base + tid * kIpt);
+  if (whole && blockable<K, IPT>()) {
+    item_block<K, IPT> blk;
+    __builtin_memcpy(&blk, keys + base + tid * kIpt, sizeof(blk));
 #pragma unroll
     for (int j = 0; j < kIpt; j++) {
       idx[j] = tid * kIpt + j;
@@ -200,17 +199,17 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
 
   // the first `valid` outputs are the real items, in order
   __syncthreads();
-  if (whole && blockable<K, IPT>() && block_aligned(keys)) {
+  if (whole && blockable<K, IPT>()) {
     item_block<K, IPT> blk;
 #pragma unroll
     for (int j = 0; j < kIpt; j++) blk.v[j] = k[j];
-    *reinterpret_cast<item_block<K, IPT>*>(keys + base + tid * kIpt) = blk;
+    __builtin_memcpy(keys + base + tid * kIpt, &blk, sizeof(blk));
     if constexpr (kHasValues) {
-      if (blockable<V, IPT>() && block_aligned(values)) {
+      if (blockable<V, IPT>()) {
         item_block<V, IPT> vb;
 #pragma unroll
         for (int j = 0; j < kIpt; j++) vb.v[j] = s_vals[idx[j]];
-        *reinterpret_cast<item_block<V, IPT>*>(values + base + tid * kIpt) = vb;
+        __builtin_memcpy(values + base + tid * kIpt, &vb, sizeof(vb));
       } else {
 #pragma unroll
         for (int j = 0; j < kIpt; j++) values[base + tid * kIpt + j] = s_vals[idx[j]];
@@ -323,21 +322,21 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(const K* kin, const V* vi
   }
   const std::int64_t out0 = tile * kTile;
   if (count == kTile) {  // a whole tile: every thread has kIpt outputs
-    if (blockable<K, IPT>() && block_aligned(kout)) {
+    if (blockable<K, IPT>()) {
       item_block<K, IPT> blk;
 #pragma unroll
       for (int j = 0; j < kIpt; j++) blk.v[j] = k[j];
-      *reinterpret_cast<item_block<K, IPT>*>(kout + out0 + d) = blk;
+      __builtin_memcpy(kout + out0 + d, &blk, sizeof(blk));
     } else {
 #pragma unroll
       for (int j = 0; j < kIpt; j++) kout[out0 + d + j] = k[j];
     }
     if constexpr (kHasValues) {
-      if (blockable<V, IPT>() && block_aligned(vout)) {
+      if (blockable<V, IPT>()) {
         item_block<V, IPT> blk;
 #pragma unroll
         for (int j = 0; j < kIpt; j++) blk.v[j] = s_vals[src[j]];
-        *reinterpret_cast<item_block<V, IPT>*>(vout + out0 + d) = blk;
+        __builtin_memcpy(vout + out0 + d, &blk, sizeof(blk));
       } else {
 #pragma unroll
         for (int j = 0; j < kIpt; j++) vout[out0 + d + j] = s_vals[src[j]];
