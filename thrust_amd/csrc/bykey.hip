@@ -193,6 +193,63 @@ __device__ inline void wave_store_blocked(E* dst, const E (&src)[VEC], tcd_v4u* 
   for (int q = 0; q < NQ; q++) store16(reinterpret_cast<char*>(dst) + (q * kWave + lane) * 16, buf[xpose_slot(q * kWave + lane)]);
   wave_lds_sync();
 }
+// The same for a wavefront whose elements end before its 64 * VEC-th: only `avail` elements exist
+// at src (possibly none, possibly all).  16-byte pieces that exist entirely move as above, the one
+// piece the end falls into is read or written element by element, the rest is zero / untouched.
+template <int VEC, class E>
+__device__ inline void wave_load_blocked_partial(const E* src, E (&dst)[VEC], tcd_v4u* buf, int lane, int64_t avail) {
+  constexpr int NQ = VEC * (int)sizeof(E) / 16;
+  constexpr int EPP = 16 / (int)sizeof(E);
+  tcd_v4u t[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; q++) {
+    const int64_t e0 = (int64_t)(q * kWave + lane) * EPP;
+    t[q] = tcd_v4u{0u, 0u, 0u, 0u};
+    if (e0 + EPP <= avail) {
+      t[q] = load16<tcd_v4u>(reinterpret_cast<const char*>(src) + (q * kWave + lane) * 16);
+    } else if (e0 < avail) {
+      E part[EPP] = {};
+      for (int e = 0; e < EPP; e++)
+        if (e0 + e < avail) part[e] = src[e0 + e];
+      __builtin_memcpy(&t[q], part, 16);
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < NQ; q++) buf[xpose_slot(q * kWave + lane)] = t[q];
+  wave_lds_sync();
+#pragma unroll
+  for (int i = 0; i < NQ; i++) {
+    const tcd_v4u r = buf[xpose_slot(lane * NQ + i)];
+    __builtin_memcpy(reinterpret_cast<char*>(dst) + 16 * i, &r, 16);
+  }
+  wave_lds_sync();
+}
+template <int VEC, class E>
+__device__ inline void wave_store_blocked_partial(E* dst, const E (&src)[VEC], tcd_v4u* buf, int lane, int64_t avail) {
+  constexpr int NQ = VEC * (int)sizeof(E) / 16;
+  constexpr int EPP = 16 / (int)sizeof(E);
+#pragma unroll
+  for (int i = 0; i < NQ; i++) {
+    tcd_v4u r;
+    __builtin_memcpy(&r, reinterpret_cast<const char*>(src) + 16 * i, 16);
+    buf[xpose_slot(lane * NQ + i)] = r;
+  }
+  wave_lds_sync();
+#pragma unroll
+  for (int q = 0; q < NQ; q++) {
+    const int64_t e0 = (int64_t)(q * kWave + lane) * EPP;
+    const tcd_v4u piece = buf[xpose_slot(q * kWave + lane)];
+    if (e0 + EPP <= avail) {
+      store16(reinterpret_cast<char*>(dst) + (q * kWave + lane) * 16, piece);
+    } else if (e0 < avail) {
+      E part[EPP];
+      __builtin_memcpy(part, &piece, 16);
+      for (int e = 0; e < EPP; e++)
+        if (e0 + e < avail) dst[e0 + e] = part[e];
+    }
+  }
+  wave_lds_sync();
+}
 #ifndef TCD_SBK_GROUP
 #define TCD_SBK_GROUP 16
 #endif
@@ -273,6 +330,18 @@ struct SegTile {
           load_group<VEC>(keys + i0, key[c]);
           load_group<VEC>(vals + i0, val[c]);
         }
+      }
+    } else if (G::BLOCKED && vec_ok) {
+      // the last tile: the same contiguous accesses up to the end of the input; elements that
+      // do not exist read as key 0 and the operator's identity
+      if constexpr (G::BLOCKED) {
+        const int64_t w0 = base + (int64_t)wave * (kWave * VEC);
+        wave_load_blocked_partial<VEC>(keys + w0, key[0], xbuf, lane, n - w0);
+        wave_load_blocked_partial<VEC>(vals + w0, val[0], xbuf, lane, n - w0);
+        const int64_t i0 = index(0, 0);
+#pragma unroll
+        for (int j = 0; j < VEC; j++)
+          if (i0 + j >= n) val[0][j] = id;
       }
     } else {
 #pragma unroll
@@ -454,6 +523,11 @@ __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_
         wave_store_blocked<VEC>(out + t.base + (int64_t)(threadIdx.x / kWave) * (kWave * VEC), r, xbuf, threadIdx.x & (kWave - 1));
       else
         store_group<VEC>(out + i0, r);
+    } else if (G::BLOCKED && vec_ok) {
+      if constexpr (G::BLOCKED) {
+        const int64_t w0 = t.base + (int64_t)(threadIdx.x / kWave) * (kWave * VEC);
+        wave_store_blocked_partial<VEC>(out + w0, r, xbuf, threadIdx.x & (kWave - 1), n - w0);
+      }
     } else {
 #pragma unroll
       for (int j = 0; j < VEC; j++)
