@@ -11,7 +11,9 @@
  * its own device primitives (thrust/system/cuda/detail/sort.h:330-365,
  * scan.h:80-117, reduce_by_key.h:1012-1031): call once with `temp == NULL` and the entry
  * point only writes the number of bytes it needs to `*temp_bytes`; call again with a
- * device buffer of at least that many bytes (256-byte aligned) to run.
+ * device buffer of at least that many bytes (256-byte aligned) to run.  Data pointers need the
+ * alignment of their element type and no more: a range that starts a few elements into an
+ * allocation runs at the same speed as one that starts at it.
  *
  * Semantics are those of the reference's sequential system, which is what its tests
  * compare the device result against:
