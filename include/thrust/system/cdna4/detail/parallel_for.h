@@ -224,12 +224,12 @@ void select_kernel(std::int64_t n, Op op, unsigned long long* words, std::int64_
   } else {
 #pragma unroll
     for (int j = 0; j < ROWS; j++) {
+      // the last tile: every thread loads (the last element where it has none of its own), so
+      // that the loads stay independent of each other; what it loaded there is never kept
       const std::int64_t i = base + (std::int64_t)j * kSelBlock;
-      if (i < n) {
-        bool keep;
-        items[j] = op.load(i, keep);
-        mine |= (keep ? 1u : 0u) << j;
-      }
+      bool keep;
+      items[j] = op.load(i < n ? i : n - 1, keep);
+      mine |= (keep && i < n ? 1u : 0u) << j;
     }
   }
 #pragma unroll

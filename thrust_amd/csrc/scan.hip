@@ -72,7 +72,8 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 #pragma unroll
       for (int j = 0; j < VEC; j++) {
         const int64_t idx = base + ((int64_t)c * BLOCK + tid) * VEC + j;
-        x[c][j] = idx < n ? in[idx] : id;
+        const T got = in[idx < n ? idx : n - 1];  // unconditional: a load under a branch waits for the one before
+        x[c][j] = idx < n ? got : id;
       }
     }
   }

@@ -237,8 +237,11 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
   } else {
 #pragma unroll
     for (int i = 0; i < IPT; i++) {
+      // every lane loads (the last valid key where it has none of its own): a load under a
+      // per-item branch would wait for the one before it
       const int li = slab + i * kWave;
-      k[i] = li < valid ? encode_key<U, FLOAT>(kin[base + li], xor_mask) : U(~U(0));  // padding sorts last
+      const U got = encode_key<U, FLOAT>(kin[base + (li < valid ? li : valid - 1)], xor_mask);
+      k[i] = li < valid ? got : U(~U(0));  // padding sorts last
     }
   }
 
@@ -380,8 +383,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
 #pragma unroll
       for (int i = 0; i < IPT; i++) {
         const int li = slab + i * kWave;
-        V v = V(0);
-        if (kFull || li < valid) v = vin[base + li];
+        const V v = vin[base + (kFull || li < valid ? li : valid - 1)];  // unconditional, as for the keys
         s_vals[pos[i]] = v;
       }
     };
