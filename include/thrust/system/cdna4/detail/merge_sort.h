@@ -36,9 +36,9 @@ namespace thrust { namespace system { namespace cdna4 { namespace detail { names
 #endif
 constexpr int kBlock = THRUST_CDNA4_MERGE_BLOCK;  // threads per workgroup
 // Items per thread: a template parameter of the kernels, chosen by the host from the item size.
-// Eight for keys of up to 4 bytes sorted alone (the merge-path search is paid once per thread, so
-// more items amortise it: 3.4 ms against 4.0 ms for 2^26 uint32 keys), four otherwise (pairs gain
-// nothing from eight, and a tile of wide items would not fit LDS).
+// Eight while key and value together take up to 8 bytes (the merge-path search is paid once per
+// thread, so more items amortise it, and there is one pass fewer: 2^26 uint32 keys 3.4 ms against
+// 4.0 ms, with uint32 values 3.8 against 4.2), four for wider items, whose tiles would crowd LDS.
 #ifndef THRUST_CDNA4_MERGE_IPT_NARROW
 #define THRUST_CDNA4_MERGE_IPT_NARROW 8
 #endif
@@ -47,7 +47,7 @@ constexpr int kBlock = THRUST_CDNA4_MERGE_BLOCK;  // threads per workgroup
 #endif
 template <class K, class V>
 constexpr int items_per_thread() {
-  return (std::is_empty<V>::value && sizeof(K) <= 4) ? THRUST_CDNA4_MERGE_IPT_NARROW : THRUST_CDNA4_MERGE_IPT;
+  return sizeof(K) + (std::is_empty<V>::value ? 0 : sizeof(V)) <= 8 ? THRUST_CDNA4_MERGE_IPT_NARROW : THRUST_CDNA4_MERGE_IPT;
 }
 
 struct no_value {};
@@ -289,10 +289,28 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(const K* kin, const V* vi
   const int na = (int)(sa1 - sa0);
   const int nb = count - na;
 
-  for (int i = tid; i < count; i += kBlock) {
-    const std::int64_t src = i < na ? (g.a0 + sa0 + i) : (g.b0 + (g.diag - sa0) + (i - na));
-    s_keys[i] = kin[src];
-    if constexpr (kHasValues) s_vals[i] = vin[src];
+  // kIpt independent loads per thread, all in flight together: the index is clamped rather than
+  // tested, because a load under a branch (or in a loop of unknown length) waits for the one
+  // before it
+  {
+    K lk[kIpt];
+    typename std::conditional<kHasValues, V, char>::type lv[kIpt];
+#pragma unroll
+    for (int u = 0; u < kIpt; u++) {
+      const int i = tid + u * kBlock;
+      const int ic = i < count ? i : count - 1;  // count >= 1: a tile is never empty
+      const std::int64_t src = ic < na ? (g.a0 + sa0 + ic) : (g.b0 + (g.diag - sa0) + (ic - na));
+      lk[u] = kin[src];
+      if constexpr (kHasValues) lv[u] = vin[src];
+    }
+#pragma unroll
+    for (int u = 0; u < kIpt; u++) {
+      const int i = tid + u * kBlock;
+      if (i < count) {
+        s_keys[i] = lk[u];
+        if constexpr (kHasValues) s_vals[i] = lv[u];
+      }
+    }
   }
   __syncthreads();
 
