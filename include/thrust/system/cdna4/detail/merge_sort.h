@@ -152,50 +152,73 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
     }
   }
 
-  // merge runs of `width` items pairwise, doubling the width
-  for (int width = kIpt; width < kTile; width *= 2) {
-    __syncthreads();
+  // Merge runs of `width` items pairwise, doubling the width.  In a whole tile the comparator
+  // alone orders the items (no padding to recognise), and the positions travel only when there
+  // are values to fetch by them.  The serial merge is branch-free: one LDS read per output, of the
+  // next item of whichever run the output came from, at a clamped index.
+  auto rounds = [&](auto whole_tag) {
+    constexpr bool kWhole = decltype(whole_tag)::value;
+    constexpr bool kIdx = kHasValues || !kWhole;
+    for (int width = kIpt; width < kTile; width *= 2) {
+      __syncthreads();
 #pragma unroll
-    for (int j = 0; j < kIpt; j++) {
-      s_keys[tid * kIpt + j] = k[j];
-      s_idx[tid * kIpt + j] = (std::uint16_t)idx[j];
-    }
-    __syncthreads();
-    const int start = (tid * kIpt) & ~(2 * width - 1);
-    const int diag = tid * kIpt - start;
-    const K* a = s_keys + start;
-    const K* b = a + width;
-    const std::uint16_t* ia = s_idx + start;
-    const std::uint16_t* ib = ia + width;
-    // merge path with the position-aware order
-    int lo = diag > width ? diag - width : 0;
-    int hi = diag < width ? diag : width;
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (!before(b[diag - 1 - mid], ib[diag - 1 - mid], a[mid], ia[mid])) lo = mid + 1;
-      else hi = mid;
-    }
-    // serial merge with the two candidate items held in registers: one LDS read per output
-    int pa = lo, pb = diag - lo;
-    K ka = a[pa < width ? pa : width - 1], kb = b[pb < width ? pb : width - 1];
-    int xa = ia[pa < width ? pa : width - 1], xb = ib[pb < width ? pb : width - 1];
-#pragma unroll
-    for (int j = 0; j < kIpt; j++) {
-      const bool take_a = pb >= width || (pa < width && !before(kb, xb, ka, xa));
-      if (take_a) {
-        k[j] = ka; idx[j] = xa; pa++;
-        if (pa < width) { ka = a[pa]; xa = ia[pa]; }
-      } else {
-        k[j] = kb; idx[j] = xb; pb++;
-        if (pb < width) { kb = b[pb]; xb = ib[pb]; }
+      for (int j = 0; j < kIpt; j++) {
+        s_keys[tid * kIpt + j] = k[j];
+        if constexpr (kIdx) s_idx[tid * kIpt + j] = (std::uint16_t)idx[j];
       }
-    }
+      __syncthreads();
+      const int start = (tid * kIpt) & ~(2 * width - 1);
+      const int diag = tid * kIpt - start;
+      const K* a = s_keys + start;  // the right run follows the left one: b[i] == a[width + i]
+      const std::uint16_t* ia = s_idx + start;
+      int lo = diag > width ? diag - width : 0;
+      int hi = diag < width ? diag : width;
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        const int m = width + diag - 1 - mid;
+        bool right_first;
+        if constexpr (kWhole) right_first = comp(a[m], a[mid]);
+        else right_first = before(a[m], ia[m], a[mid], ia[mid]);
+        if (!right_first) lo = mid + 1;
+        else hi = mid;
+      }
+      int pa = lo, pb = diag - lo;
+      const int fa = pa < width ? pa : width - 1, fb = width + (pb < width ? pb : width - 1);
+      K ka = a[fa], kb = a[fb];
+      int xa = 0, xb = 0;
+      if constexpr (kIdx) { xa = ia[fa]; xb = ia[fb]; }
 #pragma unroll
-    for (int j = 0; j < kIpt; j++) {  // all LDS reads of this round have landed before the next barrier
-      settle(k[j]);
-      settle(idx[j]);
+      for (int j = 0; j < kIpt; j++) {
+        bool right_first;
+        if constexpr (kWhole) right_first = comp(kb, ka);
+        else right_first = before(kb, xb, ka, xa);
+        const bool take_a = pb >= width || (pa < width && !right_first);
+        k[j] = take_a ? ka : kb;
+        if constexpr (kIdx) idx[j] = take_a ? xa : xb;
+        pa += take_a ? 1 : 0;
+        pb += take_a ? 0 : 1;
+        const int next = take_a ? (pa < width ? pa : width - 1) : width + (pb < width ? pb : width - 1);
+        const K kn = a[next];
+        ka = take_a ? kn : ka;
+        kb = take_a ? kb : kn;
+        if constexpr (kIdx) {
+          const int xn = ia[next];
+          xa = take_a ? xn : xa;
+          xb = take_a ? xb : xn;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kIpt; j++) {  // all LDS reads of this round have landed before the next barrier
+        settle(k[j]);
+        if constexpr (kIdx) settle(idx[j]);
+      }
+      settle(ka);
+      settle(kb);
+      if constexpr (kIdx) { settle(xa); settle(xb); }
     }
-  }
+  };
+  if (whole) rounds(std::true_type{});
+  else rounds(std::false_type{});
 
   // the first `valid` outputs are the real items, in order
   __syncthreads();
@@ -326,17 +349,16 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(const K* kin, const V* vi
   // (the tile is never empty, so index 0 is always readable)
   K ka = a[pa < na ? pa : 0], kb = s_keys[pb < nb ? na + pb : 0];
 #pragma unroll
-  for (int j = 0; j < kIpt; j++) {
-    if (d + j < count) {
-      const bool take_a = pb >= nb || (pa < na && !comp(kb, ka));
-      if (take_a) {
-        k[j] = ka; src[j] = (std::uint16_t)pa; pa++;
-        if (pa < na) ka = a[pa];
-      } else {
-        k[j] = kb; src[j] = (std::uint16_t)(na + pb); pb++;
-        if (pb < nb) kb = b[pb];
-      }
-    }
+  for (int j = 0; j < kIpt; j++) {  // branch-free; outputs past `count` are computed and not stored
+    const bool take_a = pb >= nb || (pa < na && !comp(kb, ka));
+    k[j] = take_a ? ka : kb;
+    src[j] = (std::uint16_t)(take_a ? pa : na + pb);
+    pa += take_a ? 1 : 0;
+    pb += take_a ? 0 : 1;
+    const int next = take_a ? (pa < na ? pa : 0) : (pb < nb ? na + pb : 0);
+    const K kn = s_keys[next];
+    ka = take_a ? kn : ka;
+    kb = take_a ? kb : kn;
   }
   const std::int64_t out0 = tile * kTile;
   if (count == kTile) {  // a whole tile: every thread has kIpt outputs
