@@ -199,4 +199,37 @@ void TestStableSortRepeatable() {
 }
 DECLARE_UNITTEST(TestStableSortRepeatable);
 
+// Ranges that start a few elements into an allocation and end a few before its end: the tile
+// sort and the merge passes move a thread's items as 16-byte blocks at the items' own alignment
+// (2 bytes here for the pairs), whole tiles and the partial last one alike.
+template <class K>
+void TestStableSortOffsetRanges() {
+  for (std::size_t n : {std::size_t(5000), std::size_t(4096 * 9 + 2), std::size_t(300007)}) {
+    for (std::size_t skip : {std::size_t(1), std::size_t(3)}) {
+      thrust::host_vector<K> h = unittest::random_integers<K>(n + skip + 2, 7 * n + skip);
+      thrust::host_vector<K> hv(n + skip + 2);
+      for (std::size_t i = 0; i < hv.size(); i++) hv[i] = (K)i;
+      // keys alone
+      thrust::device_vector<K> d = h;
+      std::vector<K> ref(h.begin(), h.end());
+      std::stable_sort(ref.begin() + skip, ref.begin() + skip + n, less_div_10<K>());
+      thrust::stable_sort(d.begin() + skip, d.begin() + skip + n, less_div_10<K>());
+      ASSERT_EQUAL(d, thrust::host_vector<K>(ref.begin(), ref.end()));  // the elements around the range are untouched
+      // pairs: the values record where each key came from
+      thrust::device_vector<K> dk = h, dv = hv;
+      std::vector<std::size_t> order(n);
+      std::iota(order.begin(), order.end(), skip);
+      std::stable_sort(order.begin(), order.end(), [&](std::size_t a, std::size_t b) { return less_div_10<K>()(h[a], h[b]); });
+      thrust::stable_sort_by_key(dk.begin() + skip, dk.begin() + skip + n, dv.begin() + skip, less_div_10<K>());
+      thrust::host_vector<K> ek = h, ev = hv;
+      for (std::size_t i = 0; i < n; i++) { ek[skip + i] = h[order[i]]; ev[skip + i] = hv[order[i]]; }
+      ASSERT_EQUAL(dk, ek);
+      ASSERT_EQUAL(dv, ev);
+    }
+  }
+}
+DECLARE_TYPED_UNITTEST(TestStableSortOffsetRanges, uint16_t);
+DECLARE_TYPED_UNITTEST(TestStableSortOffsetRanges, unsigned);
+DECLARE_TYPED_UNITTEST(TestStableSortOffsetRanges, int64_t);
+
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
