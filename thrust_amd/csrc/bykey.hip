@@ -723,17 +723,22 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
       if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
       if (*temp_bytes < need) return;
       if (n == 0) { rc = hipSuccess; return; }
-      rc = zero_async(temp, need, s);
-      if (rc != hipSuccess) return;
+      const int64_t ntiles = ceil_div(n, ScanByKeyGeom<T>::TILE);
+      // one tile consults no descriptor and reads all its input before it writes: no clearing
+      // launch, no tickets
+      const bool single = ntiles == 1;
+      if (!single) {
+        rc = zero_async(temp, need, s);
+        if (rc != hipSuccess) return;
+      }
       T iv = T(0);
       if (init) __builtin_memcpy(&iv, init, sizeof(T));
       // 128-bit accesses need no more than the elements' own alignment (see load16)
       const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & (sizeof(KU) - 1)) == 0 &&
                          ((reinterpret_cast<uintptr_t>(values) | reinterpret_cast<uintptr_t>(out)) & (sizeof(T) - 1)) == 0;
-      const int64_t ntiles = ceil_div(n, ScanByKeyGeom<T>::TILE);
       // an output that overlaps an input: tiles by ticket
-      const bool aliased = ranges_overlap(out, (size_t)n * sizeof(T), values, (size_t)n * sizeof(T)) ||
-                           ranges_overlap(out, (size_t)n * sizeof(T), keys, (size_t)n * sizeof(KU));
+      const bool aliased = !single && (ranges_overlap(out, (size_t)n * sizeof(T), values, (size_t)n * sizeof(T)) ||
+                           ranges_overlap(out, (size_t)n * sizeof(T), keys, (size_t)n * sizeof(KU)));
       if (aliased) {
         TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(ScanByKeyGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
@@ -772,16 +777,20 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
         rc = zero_async(num_runs_out, sizeof(int64_t), s);
         return;
       }
-      rc = zero_async(temp, need, s);
-      if (rc != hipSuccess) return;
+      const int64_t ntiles = ceil_div(n, ReduceByKeyGeom<T>::TILE);
+      const bool single = ntiles == 1;  // as in scan_by_key
+      if (!single) {
+        rc = zero_async(temp, need, s);
+        if (rc != hipSuccess) return;
+      }
       // 128-bit accesses need no more than the elements' own alignment (see load16)
       const int vec_ok = (reinterpret_cast<uintptr_t>(keys_in) & (sizeof(KU) - 1)) == 0 &&
                          (reinterpret_cast<uintptr_t>(values_in) & (sizeof(T) - 1)) == 0;
-      const int64_t ntiles = ceil_div(n, ReduceByKeyGeom<T>::TILE);
       // an output that overlaps an input: tiles by ticket
       const size_t kb = (size_t)n * sizeof(KU), vb = (size_t)n * sizeof(T);
-      const bool aliased = ranges_overlap(keys_out, kb, keys_in, kb) || ranges_overlap(keys_out, kb, values_in, vb) ||
-                           ranges_overlap(values_out, vb, keys_in, kb) || ranges_overlap(values_out, vb, values_in, vb);
+      const bool aliased = !single &&
+                           (ranges_overlap(keys_out, kb, keys_in, kb) || ranges_overlap(keys_out, kb, values_in, vb) ||
+                            ranges_overlap(values_out, vb, keys_in, kb) || ranges_overlap(values_out, vb, values_in, vb));
       if (aliased) {
         TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(ReduceByKeyGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),

@@ -198,15 +198,20 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   }
   if (*temp_bytes < need) return hipErrorInvalidValue;
   if (n == 0) return hipSuccess;
-  hipError_t e = zero_async(temp, need, stream);
-  if (e != hipSuccess) return e;
+  // One tile consults no descriptor and reads its whole input before it writes any output: it
+  // needs neither the cleared descriptors (a launch less: a third of a small call) nor tickets.
+  const bool single = ntiles == 1;
+  if (!single) {
+    const hipError_t e = zero_async(temp, need, stream);
+    if (e != hipSuccess) return e;
+  }
   T iv = T(0);
   if (init) __builtin_memcpy(&iv, init, sizeof(T));
   uint32_t* ticket = reinterpret_cast<uint32_t*>(temp);
   uint64_t* desc = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256);
   // 128-bit accesses need no more than the elements' own alignment (see load16)
   const int vec_ok = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & (sizeof(T) - 1)) == 0;
-  if (ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T))) {
+  if (!single && ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T))) {
     TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS, true>), dim3((unsigned)ntiles), dim3(C::BLOCK),
                stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
                desc, ticket, vec_ok, 0);
