@@ -402,6 +402,99 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
 }
 
 // ---------------------------------------------------------------------------------------
+// Inputs of up to kTileSortMax items: ONE workgroup sorts them, every pass of the LSD radix sort
+// inside LDS (the shape of the reference's single-tile path, cub::DeviceRadixSortSingleTileKernel
+// behind thrust/system/cuda/detail/sort.h:213-380).  No histogram pass, no descriptors, no
+// alternate buffer: one launch instead of two plus one per digit, which is what a small sort
+// costs.  Ranking is the onesweep kernel's: wave w owns a contiguous slab, item i of lane l is
+// slab[i*64 + l], and the value returned by the wave's LDS atomic add on its counter of the key's
+// digit numbers that digit's keys in (item, lane) order, the memory order: the sort is stable.
+// ---------------------------------------------------------------------------------------
+constexpr int kTileSortThreads = 512;
+constexpr int kTileSortIpt = 8;
+constexpr int kTileSortMax = kTileSortThreads * kTileSortIpt;
+
+template <class U, int VB, bool FLOAT>
+__global__ __launch_bounds__(kTileSortThreads) void tile_sort_kernel(U* keys, void* values_, int n, U xor_mask) {
+  using V = typename value_of<VB>::type;
+  constexpr int IPT = kTileSortIpt, BLOCK = kTileSortThreads, NW = BLOCK / kWave, P = (int)sizeof(U);
+  __shared__ U s_keys[BLOCK * IPT];
+  __shared__ V s_vals[VB ? BLOCK * IPT : 1];
+  __shared__ uint32_t s_cnt[NW][kRadix];  // per-wave digit counts, then the first slot of each (wave, digit)
+  __shared__ uint32_t s_wtot[kRadix / kWave];
+  V* values = static_cast<V*>(values_);
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int slab = wave * (kWave * IPT) + lane;
+
+  U k[IPT];
+  V v[IPT];
+#pragma unroll
+  for (int i = 0; i < IPT; i++) {  // every lane loads (a clamped index); padding sorts last and stays last
+    const int li = slab + i * kWave;
+    const int at = li < n ? li : n - 1;
+    const U got = encode_key<U, FLOAT>(keys[at], xor_mask);
+    k[i] = li < n ? got : U(~U(0));
+    if (VB) v[i] = values[at];
+  }
+
+  for (int p = 0; p < P; p++) {
+    const int shift = 8 * p;
+    for (int j = tid; j < NW * kRadix; j += BLOCK) (&s_cnt[0][0])[j] = 0;
+    __syncthreads();
+    uint32_t rank[IPT];
+#pragma unroll
+    for (int i = 0; i < IPT; i++) rank[i] = atomicAdd(&s_cnt[wave][(uint32_t)(k[i] >> shift) & 0xffu], 1u);
+    __syncthreads();
+    // thread d: the digit's count per wave, the exclusive prefix over the digits, then the first
+    // slot of every (wave, digit)
+    uint32_t c[NW], lbase = 0;
+    if (tid < kRadix) {
+      uint32_t total = 0;
+#pragma unroll
+      for (int w = 0; w < NW; w++) {
+        c[w] = s_cnt[w][tid];
+        total += c[w];
+      }
+      const uint32_t incl = wave_inclusive_scan(total, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+      if (lane == kWave - 1) s_wtot[wave] = incl;
+      lbase = incl - total;
+    }
+    __syncthreads();
+    if (tid < kRadix) {
+      for (int w = 0; w < wave; w++) lbase += s_wtot[w];
+      uint32_t run = lbase;
+#pragma unroll
+      for (int w = 0; w < NW; w++) {
+        s_cnt[w][tid] = run;
+        run += c[w];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < IPT; i++) {
+      const uint32_t pos = s_cnt[wave][(uint32_t)(k[i] >> shift) & 0xffu] + rank[i];
+      s_keys[pos] = k[i];
+      if (VB) s_vals[pos] = v[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < IPT; i++) {
+      k[i] = s_keys[slab + i * kWave];
+      if (VB) v[i] = s_vals[slab + i * kWave];
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < IPT; i++) {
+    const int li = slab + i * kWave;
+    if (li < n) {
+      keys[li] = decode_key<U, FLOAT>(k[i], xor_mask);
+      if (VB) values[li] = v[i];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Self-test of the LDS property the ranking relies on
 // ---------------------------------------------------------------------------------------
 // Every wave adds 1 to pseudo-random counters of its own (uniform digits, one hot digit, and a
@@ -526,6 +619,11 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   }
   if (*temp_bytes < plan.total) return hipErrorInvalidValue;
   if (n == 0) return hipSuccess;
+  if (n <= kTileSortMax) {  // one workgroup, one launch, nothing of `temp` is used
+    TCD_LAUNCH("tile_sort_kernel", (tile_sort_kernel<U, VB, FLOAT>), dim3(1), dim3(kTileSortThreads), stream,
+               static_cast<U*>(keys), values, (int)n, xor_mask);
+    return hipGetLastError();
+  }
   char* t = static_cast<char*>(temp);
   U* kbuf[2] = {static_cast<U*>(keys), reinterpret_cast<U*>(t + plan.keys_alt)};
   char* vbuf[2] = {static_cast<char*>(values), t + plan.vals_alt};
