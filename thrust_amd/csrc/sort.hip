@@ -83,8 +83,11 @@ __device__ __host__ inline U decode_key(U e, U xor_mask) {
 // over the LDS banks whatever the keys are (random, sorted, constant) instead of meeting on
 // the few banks their digits select.  64 KiB per workgroup: 16 copies for 4-byte keys, 8 for
 // 8-byte keys, 32 for narrower ones.
+#ifndef TCD_SORT_HIST_UNROLL
+#define TCD_SORT_HIST_UNROLL 8  // 128-bit loads in flight per thread
+#endif
 #ifndef TCD_SORT_HIST_BLOCKS
-#define TCD_SORT_HIST_BLOCKS 512
+#define TCD_SORT_HIST_BLOCKS 256
 #endif
 constexpr int kHistThreads = 512;
 template <class U>
@@ -99,7 +102,7 @@ __global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const U* __res
   constexpr int P = RadixHistGeom<U>::P;
   constexpr int COPIES = RadixHistGeom<U>::COPIES;
   constexpr int VEC = 16 / sizeof(U);
-  constexpr int UNROLL = 2;
+  constexpr int UNROLL = TCD_SORT_HIST_UNROLL;
   __shared__ uint32_t h[P * kRadix * COPIES];
   const int tid = threadIdx.x;
   for (int i = tid; i < P * kRadix * COPIES; i += kHistThreads) h[i] = 0;
@@ -636,7 +639,7 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
 
   const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & (sizeof(U) - 1)) == 0;  // see load16
   int64_t hblocks = ceil_div(n, kHistThreads * 64);
-  if (hblocks > TCD_SORT_HIST_BLOCKS) hblocks = TCD_SORT_HIST_BLOCKS;  // two workgroups per CU
+  if (hblocks > TCD_SORT_HIST_BLOCKS) hblocks = TCD_SORT_HIST_BLOCKS;  // one workgroup per CU, eight loads in flight per thread: 1 % of a 2^28 sort over two with two
   TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(kHistThreads), stream,
              kbuf[0], n, xor_mask, ghist, vec_ok);
   TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(P), dim3(256), stream, ghist);
