@@ -106,6 +106,7 @@ T transform_reduce_n(const Policy& exec, In in, std::int64_t n, F f, T init, Op 
 template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
   typedef typename value_of_it<In>::type item;
   static constexpr bool rejects = false;
+  static constexpr int rows = sizeof(item) <= 4 ? 64 : generic::select_rows(sizeof(item));  // tiles of 64 rows: see select_rows_of
   In in; Out out; Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     const item x = in[i];
