@@ -106,7 +106,7 @@ T transform_reduce_n(const Policy& exec, In in, std::int64_t n, F f, T init, Op 
 template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
   typedef typename value_of_it<In>::type item;
   static constexpr bool rejects = false;
-  static constexpr int rows = sizeof(item) <= 4 ? 64 : generic::select_rows(sizeof(item));  // tiles of 64 rows: see select_rows_of
+  static constexpr int rows = sizeof(item) <= 4 ? 64 : sizeof(item) == 8 ? 32 : generic::select_rows(sizeof(item));  // 256 KiB tiles: see select_rows_of
   In in; Out out; Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     const item x = in[i];
@@ -155,6 +155,7 @@ template <class KIn, class VIn, class KOut, class VOut, class Eq> struct run_hea
   typedef typename value_of_it<VIn>::type V;
   struct item { K key; V value; };
   static constexpr bool rejects = false;
+  static constexpr int rows = sizeof(item) == 8 ? 32 : generic::select_rows(sizeof(item));  // 256-byte tiles per thread: see select_rows_of
   KIn keys; VIn values; KOut kout; VOut vout; Eq eq;
   __device__ item load(std::int64_t i, bool& keep) const {
     const K cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
