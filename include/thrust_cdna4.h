@@ -205,6 +205,15 @@ int thrust_cdna4_free_direct(void* ptr);
  * Results do not depend on it except for the rounding order of floating-point sums.
  */
 int thrust_cdna4_set_lookback_patience(int polls);
+/*
+ * Test knob for that recomputation path; no counterpart in the reference.  Tile 0 of the
+ * ticketless scan, scan_by_key and reduce_by_key kernels sleeps `sleeps` times (a few
+ * microseconds each, clamped to 100000) before it publishes its descriptor, so that with
+ * patience 0 every later tile deterministically finds it missing, also at the second look.
+ * Every kernel still runs to completion.  Returns the previous value; 0 (the default) switches
+ * it off.
+ */
+int thrust_cdna4_set_test_publish_delay(int sleeps);
 
 /*
  * Launch profiling.  While enabled, every kernel the library launches is bracketed by HIP

@@ -189,6 +189,35 @@ def test_by_key_recompute_path_matches_oracle(no_patience, kd, vd):
             assert same_bits(host(gk), rk) and same_bits(host(gv), rv), (n, mean)
 
 
+@pytest.fixture
+def tile0_publishes_late():
+    """Tile 0 sleeps ~10 ms (a bounded number of sleeps) before it publishes, so with patience 0
+    every later tile finds its descriptor missing twice and uses its own recomputed aggregate."""
+    from thrust_amd import capi
+    L = capi.lib()
+    previous = L.thrust_cdna4_set_test_publish_delay(3000)
+    yield
+    L.thrust_cdna4_set_test_publish_delay(previous)
+
+
+@pytest.mark.parametrize("op", ["plus", "multiplies", "maximum", "minimum"])
+def test_by_key_with_a_recomputed_tile0(no_patience, tile0_publishes_late, op):
+    # init restarts at every segment head (sequential/scan_by_key.h:95-140); it is applied where
+    # results are formed, never stored in a tile descriptor, so a recomputed tile 0 loses nothing
+    for kd, vd, n in [(np.int32, np.int32, 100_003), (np.uint64, np.int64, 50_001), (np.uint8, np.uint16, 70_000)]:
+        for mean in (1, 8, 40_000):
+            k = (runs(n + mean, n, mean, np.int64) % 200).astype(kd)
+            v = random_ints(n + 3, n, vd)
+            dk, dv = dev(k), dev(v)
+            assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=7, op=op)),
+                             oracle.scan_by_key(k, v, op=op, exclusive=True, init=7)), (kd, vd, n, mean)
+            assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op=op)),
+                             oracle.scan_by_key(k, v, op=op)), (kd, vd, n, mean)
+            gk, gv = thrust_amd.reduce_by_key(dk, dv, op=op)
+            rk, rv = oracle.reduce_by_key(k, v, op=op)
+            assert same_bits(host(gk), rk) and same_bits(host(gv), rv), (kd, vd, n, mean)
+
+
 def test_by_key_aliased_outputs_take_the_ticket_path():
     n = (1 << 20) + 9
     k = (runs(5, n, 8, np.int64) % 200).astype(np.int32)

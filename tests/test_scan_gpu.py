@@ -119,6 +119,35 @@ def no_patience():
     L.thrust_cdna4_set_lookback_patience(previous)
 
 
+@pytest.fixture
+def tile0_publishes_late():
+    """Tile 0 sleeps ~10 ms (a bounded number of sleeps) before it publishes its descriptor, so
+    with patience 0 every later tile finds it missing at the first AND at the second look and
+    has to use the aggregate it recomputed from the input.  Every kernel still exits normally."""
+    from thrust_amd import capi
+    L = capi.lib()
+    previous = L.thrust_cdna4_set_test_publish_delay(3000)
+    yield
+    L.thrust_cdna4_set_test_publish_delay(previous)
+
+
+@pytest.mark.parametrize("op", ["plus", "multiplies", "maximum", "minimum"])
+def test_exclusive_scan_init_survives_a_recomputed_tile0(no_patience, tile0_publishes_late, op):
+    # semantics: thrust/system/detail/sequential/scan.h:95-111 (out[0] = init, then init op x0 ...)
+    for dtype, n in [(np.int32, 200_003), (np.int64, 70_001), (np.uint8, 300_000), (np.int16, 300_001)]:
+        x = random_ints(77 + n, n, dtype)
+        d = dev(x)
+        for init in (7, 0):
+            got = host(thrust_amd.exclusive_scan(d, init=init, op=op))
+            assert same_bits(got, oracle.scan(x, op, exclusive=True, init=init)), (dtype, n, init)
+        assert same_bits(host(thrust_amd.inclusive_scan(d, op=op)), oracle.scan(x, op)), (dtype, n)
+    f = np.random.default_rng(8).uniform(-1, 1, 150_001).astype(np.float32)
+    got = host(thrust_amd.exclusive_scan(dev(f), init=0.5, op="plus")).astype(np.float64)
+    ref = np.concatenate([[0.0], np.cumsum(f.astype(np.float64))[:-1]]) + 0.5
+    l1 = np.concatenate([[0.0], np.cumsum(np.abs(f.astype(np.float64)))[:-1]]) + 0.5
+    assert (np.abs(got - ref) <= FP_RTOL * l1).all()
+
+
 def test_scan_recompute_path_matches_oracle(no_patience):
     for n in [1, 4097, 32768, 32769, 200_003, (1 << 22) + 5]:
         x = random_ints(50 + n, n, np.int32)

@@ -302,7 +302,8 @@ struct SegTile {
   // missing after `patience` polls is recomputed from the input.
   template <bool TICKET, class Meanwhile>
   __device__ void run(Smem& sm, const KU* keys, const T* vals, int64_t n, int float_keys, int vec_ok,
-                      uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf, int patience, Meanwhile meanwhile) {
+                      uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf, int patience, int publish_delay,
+                      Meanwhile meanwhile) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -395,6 +396,8 @@ struct SegTile {
       const Pair incl = wave_inclusive_scan(mine, idp, comb);
       tile_agg = readlane(incl, kWave - 1);
       before = wave_shift_up1(incl, idp);
+      if (tile == 0)
+        for (int i = 0; i < publish_delay; i++) __builtin_amdgcn_s_sleep(127);  // test knob, 0 in normal use
       if (lane == 0) TileDesc<Pair>::store(desc, tile, tile == 0 ? kInclusive : kPartial, tile_agg);
     }
     // work that needs nothing from earlier tiles runs while their aggregates arrive
@@ -440,7 +443,7 @@ struct SegTile {
 template <class T, class Op, bool TICKET>
 __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_key_kernel(
     const KU* keys, const T* vals, T* out, int64_t n, T init, int exclusive, int float_keys, int vec_ok,
-    uint64_t* desc, uint32_t* ticket, int patience) {
+    uint64_t* desc, uint32_t* ticket, int patience, int publish_delay) {
   using G = ScanByKeyGeom<T>;
   using ST = SegTile<T, Op, G>;
   __shared__ typename ST::Smem sm;
@@ -457,7 +460,7 @@ __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_
   constexpr int EPP = 16 / (int)sizeof(T);  // elements per 16-byte slot
   bool parked = false;
   uint32_t first_head = 0;
-  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, [&] {
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, [&] {
     if constexpr (G::BLOCKED) {
       if (!t.full) return;
       parked = true;
@@ -542,7 +545,7 @@ __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_
 template <class T, class Op, bool TICKET>
 __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce_by_key_kernel(
     const KU* keys, const T* vals, KU* keys_out, T* vals_out, int64_t* num_runs, int64_t n,
-    int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket, int patience) {
+    int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket, int patience, int publish_delay) {
   using G = ReduceByKeyGeom<T>;
   using ST = SegTile<T, Op, G>;
   constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS, NWAVES = ST::NWAVES;
@@ -574,7 +577,7 @@ __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce
     T* const early_v = reinterpret_cast<T*>(reinterpret_cast<char*>(xbuf) + kHalfBytes);
     bool early = false;
     uint32_t count = 0;
-    t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, [&] {
+    t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, [&] {
       count = (uint32_t)__builtin_amdgcn_readlane((int)(t.excl_w[0].c + __builtin_popcount(t.heads[0])), kWave - 1);
       early = t.full && count <= kEarlyMax;
       if (!early) {
@@ -659,7 +662,7 @@ __global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce
   __shared__ KU s_keys[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
   __shared__ T s_vals[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
   ST t;
-  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, nullptr, patience, [] {});
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, nullptr, patience, publish_delay, [] {});
   KU* sk = s_keys[G::BLOCKED ? 0 : threadIdx.x / kWave];
   T* sv = s_vals[G::BLOCKED ? 0 : threadIdx.x / kWave];
 #pragma unroll
@@ -744,13 +747,13 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
                            static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
                            n, iv, exclusive, float_keys, vec_ok,
                            reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
-                           reinterpret_cast<uint32_t*>(temp), 0);
+                           reinterpret_cast<uint32_t*>(temp), 0, 0);
       } else {
         TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, false>), dim3((unsigned)ntiles), dim3(ScanByKeyGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
                            n, iv, exclusive, float_keys, vec_ok,
                            reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
-                           reinterpret_cast<uint32_t*>(temp), lookback_patience());
+                           reinterpret_cast<uint32_t*>(temp), lookback_patience(), lookback_test_publish_delay());
       }
       rc = hipGetLastError();
     });
@@ -796,13 +799,13 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
                            static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
                            static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
                            vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
-                           reinterpret_cast<uint32_t*>(temp), 0);
+                           reinterpret_cast<uint32_t*>(temp), 0, 0);
       } else {
         TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, false>), dim3((unsigned)ntiles), dim3(ReduceByKeyGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
                            static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
                            vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
-                           reinterpret_cast<uint32_t*>(temp), lookback_patience());
+                           reinterpret_cast<uint32_t*>(temp), lookback_patience(), lookback_test_publish_delay());
       }
       rc = hipGetLastError();
     });

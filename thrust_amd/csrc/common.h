@@ -358,6 +358,9 @@ __device__ inline P wave_lookback_or_compute(const uint64_t* desc, int64_t tile,
 // kDefaultLookbackPatience); set by thrust_cdna4_set_lookback_patience.
 constexpr int kDefaultLookbackPatience = 256;
 int lookback_patience();
+// Test knob (thrust_cdna4_set_test_publish_delay): tile 0 of a ticketless kernel sleeps this many
+// times (a few microseconds each) before it publishes its descriptor.  0 in normal use.
+int lookback_test_publish_delay();
 // true when [a, a + na) and [b, b + nb) share a byte
 inline bool ranges_overlap(const void* a, size_t na, const void* b, size_t nb) {
   const uintptr_t x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);

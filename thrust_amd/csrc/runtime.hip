@@ -339,6 +339,16 @@ extern "C" int thrust_cdna4_set_lookback_patience(int polls) {
   return tcd::g_lookback_patience.exchange(polls < 0 ? tcd::kDefaultLookbackPatience : polls, std::memory_order_relaxed);
 }
 
+namespace tcd {
+static std::atomic<int> g_publish_delay{0};
+int lookback_test_publish_delay() { return g_publish_delay.load(std::memory_order_relaxed); }
+}  // namespace tcd
+extern "C" int thrust_cdna4_set_test_publish_delay(int sleeps) {
+  if (sleeps < 0) sleeps = 0;
+  if (sleeps > 100000) sleeps = 100000;  // bounded: a third of a second at most
+  return tcd::g_publish_delay.exchange(sleeps, std::memory_order_relaxed);
+}
+
 extern "C" int thrust_cdna4_stream_synchronize(void* stream) {
   return hipStreamSynchronize(static_cast<hipStream_t>(stream));
 }

@@ -22,7 +22,7 @@ struct alignas(16) Vec16 {
 template <class T, class Op, int BLOCK, int CHUNKS, bool TICKET>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void scan_kernel(const T* in, T* out, int64_t n, T init,
                                                      int exclusive, uint64_t* desc,
-                                                     uint32_t* ticket, int vec_ok, int patience) {
+                                                     uint32_t* ticket, int vec_ok, int patience, int publish_delay) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NWAVES = BLOCK / kWave;
   constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
@@ -105,10 +105,13 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     const W incl = wave_inclusive_scan(mine[PER - 1], idW, opW);
     const W tile_agg = readlane(incl, kWave - 1);
     const W before = wave_shift_up1(incl, idW);  // totals of the lanes below
-    W prefix;
+    // Descriptors carry sums of INPUT elements only.  `init` of an exclusive scan is applied by
+    // every tile to its own prefix below, so a tile aggregate recomputed from the input by a
+    // later tile (wave_lookback_or_compute) is the same value its owner would have published.
+    W prefix = idW;
     if (tile == 0) {
-      prefix = exclusive ? toW(init) : idW;
-      if (lane == 0) TileDesc<W>::store(desc, 0, kInclusive, opW(prefix, tile_agg));
+      for (int i = 0; i < publish_delay; i++) __builtin_amdgcn_s_sleep(127);  // test knob, 0 in normal use
+      if (lane == 0) TileDesc<W>::store(desc, 0, kInclusive, tile_agg);
     } else {
       if (lane == 0) TileDesc<W>::store(desc, tile, kPartial, tile_agg);
       if constexpr (TICKET) {
@@ -126,6 +129,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
       }
       if (lane == 0) TileDesc<W>::store(desc, tile, kInclusive, opW(prefix, tile_agg));
     }
+    if (exclusive) prefix = opW(toW(init), prefix);
     const W base_w = opW(prefix, before);
     // offset of (chunk, wave) in the whole input = everything before it
 #pragma unroll
@@ -214,11 +218,11 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   if (!single && ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T))) {
     TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS, true>), dim3((unsigned)ntiles), dim3(C::BLOCK),
                stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
-               desc, ticket, vec_ok, 0);
+               desc, ticket, vec_ok, 0, 0);
   } else {
     TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS, false>), dim3((unsigned)ntiles), dim3(C::BLOCK),
                stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
-               desc, ticket, vec_ok, lookback_patience());
+               desc, ticket, vec_ok, lookback_patience(), lookback_test_publish_delay());
   }
   return hipGetLastError();
 }
