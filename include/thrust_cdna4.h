@@ -101,6 +101,24 @@ int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int op, int exc
                       const void* in, void* out, int64_t n, const void* init, void* stream);
 
 /*
+ * thrust_cdna4_scan for callers that cannot allocate: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference, whose scan
+ * always takes caller-provided temporary storage (thrust/system/cuda/detail/scan.h:80-117).  Same
+ * arguments, results and kernels as thrust_cdna4_scan without `temp` / `temp_bytes`: the tile
+ * descriptors live in a fixed 256 KiB array inside the library's device image (one copy per GPU,
+ * held until the process ends), whose device address is looked up on the first call on each
+ * device; no call allocates or frees memory.  Limit: at most 16384 tiles, i.e.
+ * n <= 2^29 elements of 1, 2 or 4 bytes (32768 per tile) and n <= 2^28 elements of 8 bytes
+ * (16384 per tile); a larger n returns hipErrorOutOfMemory (2) before anything else is looked
+ * at, and launches nothing.  All calls on one GPU share the array: calls
+ * that overlap in time on one GPU (different streams, or different host threads) race and must
+ * be serialised by the caller; back-to-back calls on one stream are fine (each call clears the
+ * descriptors it uses with a fill kernel, never hipMemsetAsync).
+ */
+int thrust_cdna4_scan_static(int dtype, int op, int exclusive, const void* in, void* out,
+                             int64_t n, const void* init, void* stream);
+
+/*
  * Segmented prefix scan: segments are maximal runs of consecutive equal keys
  * (thrust::equal_to on adjacent keys).  Replaces inclusive_scan_by_key_n /
  * exclusive_scan_by_key_n and cub::DispatchScanByKey

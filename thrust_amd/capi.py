@@ -22,7 +22,7 @@ SYMBOLS = [
     "thrust_cdna4_fill", "thrust_cdna4_stream_synchronize", "thrust_cdna4_profile_enable",
     "thrust_cdna4_profile_count", "thrust_cdna4_profile_get",
     "thrust_cdna4_selftest_lds_atomic_order", "thrust_cdna4_set_lookback_patience",
-    "thrust_cdna4_set_test_publish_delay",
+    "thrust_cdna4_set_test_publish_delay", "thrust_cdna4_scan_static",
     "thrust_cdna4_stream_create", "thrust_cdna4_stream_destroy", "thrust_cdna4_stream_query",
     "thrust_cdna4_event_create", "thrust_cdna4_event_destroy", "thrust_cdna4_event_record", "thrust_cdna4_event_query",
     "thrust_cdna4_stream_wait_event", "thrust_cdna4_malloc_direct", "thrust_cdna4_free_direct",
@@ -58,6 +58,7 @@ def lib():
     L.thrust_cdna4_sort_keys.argtypes = [vp, psz, i32, vp, i64, i32, vp]
     L.thrust_cdna4_sort_pairs.argtypes = [vp, psz, i32, vp, i32, vp, i64, i32, vp]
     L.thrust_cdna4_scan.argtypes = [vp, psz, i32, i32, i32, vp, vp, i64, vp, vp]
+    L.thrust_cdna4_scan_static.argtypes = [i32, i32, i32, vp, vp, i64, vp, vp]
     L.thrust_cdna4_scan_by_key.argtypes = [vp, psz, i32, i32, i32, i32, vp, vp, vp, i64, vp, vp]
     L.thrust_cdna4_reduce_by_key.argtypes = [vp, psz, i32, i32, i32, vp, vp, vp, vp, vp, i64, vp]
     L.thrust_cdna4_histogram_even.argtypes = [vp, psz, i32, vp, i64, vp, i32, dbl, dbl, vp]

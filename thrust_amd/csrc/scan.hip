@@ -6,6 +6,8 @@
 // publishes the tile aggregate, obtains the prefix of all earlier tiles by look-back and
 // writes the result.  Semantics: thrust/system/detail/sequential/scan.h:47-114; replaces
 // thrust/system/cuda/detail/scan.h:57-204 (cub::DispatchScan).
+#include <mutex>
+
 #include "common.h"
 
 namespace tcd {
@@ -244,5 +246,68 @@ extern "C" int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int 
     });
   });
   (void)ok;
+  return (int)rc;
+}
+
+// ---------------------------------------------------------------------------------------
+// The same scan for callers that cannot allocate (code under HIP graph capture, serving loops,
+// harnesses that forbid hipMalloc): ticket and tile descriptors live in a fixed array in the
+// library's device image instead of caller-provided temporary storage.
+// ---------------------------------------------------------------------------------------
+namespace tcd {
+constexpr int64_t kStaticScanMaxTiles = 16384;  // 2^29 elements of up to 4 bytes, 2^28 of 8 bytes
+constexpr size_t kStaticScanScratchBytes = 256 + (size_t)kStaticScanMaxTiles * 16;  // ticket + 16 B per tile
+static __device__ __align__(256) unsigned char scratch[kStaticScanScratchBytes];
+
+// `scratch` names the host-side stand-in of the symbol; the array's device address differs per
+// GPU and is looked up once per device, with that device current.
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[kMaxDevices];
+
+static hipError_t static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> g(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return hipSuccess;
+}
+}  // namespace tcd
+
+extern "C" int thrust_cdna4_scan_static(int dtype, int op, int exclusive, const void* in, void* out,
+                                        int64_t n, const void* init, void* stream) {
+  using namespace tcd;
+  if (n < 0) return hipErrorInvalidValue;
+  // The size limit is checked first and has its own code, whatever the pointers are.
+  int64_t ntiles = -1;
+  dispatch_dtype(dtype, [&](auto t) { ntiles = ceil_div(n, ScanConfig<decltype(t)>::TILE); });
+  if (ntiles < 0) return hipErrorInvalidValue;  // unknown element type
+  if (ntiles > kStaticScanMaxTiles) return hipErrorOutOfMemory;
+  if (n > 0 && (!in || !out)) return hipErrorInvalidValue;
+  void* ptr = nullptr;
+  hipError_t rc = static_scratch(&ptr);
+  if (rc != hipSuccess) return (int)rc;
+  rc = hipErrorInvalidValue;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dispatch_dtype(dtype, [&](auto t) {
+    using T = decltype(t);
+    static_assert(TileDesc<typename ScanConfig<T>::P>::kBytesPerTile <= 16, "16 bytes of descriptor per tile");
+    dispatch_op(op, [&](auto o) {
+      using Op = decltype(o);
+      // scan_typed checks the size it needs against the bytes it is given and clears the
+      // descriptors it will use with a fill kernel before the scan kernel reads them
+      size_t bytes = kStaticScanScratchBytes;
+      rc = scan_typed<T, Op>(ptr, &bytes, exclusive, in, out, n, init, s);
+    });
+  });
   return (int)rc;
 }
