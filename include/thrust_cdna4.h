@@ -246,12 +246,25 @@ int thrust_cdna4_profile_count(void);
 int thrust_cdna4_profile_get(int index, const char** name, float* ms);
 
 /*
+ * Diagnostics; no counterpart in the reference.  Every wait of the sort's look-back is bounded: a
+ * digit's thread that polls a missing tile descriptor about 4 million times (seconds; a wait
+ * that ends takes microseconds) gives up, the kernel still runs to completion — with a wrong
+ * result — and the event is counted per device.  Blocks until the device is idle and stores the
+ * count since the process started; anything but 0 means a sort result cannot be trusted.
+ */
+int thrust_cdna4_lookback_timeouts(unsigned long long* count);
+
+/*
  * Hardware self-test.  The sort kernels rank keys with returning LDS atomics and rely on the
  * LDS unit serving the lanes of one instruction that hit the same address in lane order
  * (this is what makes the ranking stable, which cub::DeviceRadixSort obtains with warp match
  * operations, thrust/system/cuda/detail/sort.h:213-380).  Runs about 3*10^8 checked atomics
  * on the current device, waits for them, and stores the number of out-of-order results in
- * *mismatches (0 on a conforming device).  Not on any algorithm's path.
+ * *mismatches (0 on a conforming device).  The library runs a short form of it by itself (10^7
+ * atomics, about 0.1 ms): the first thrust_cdna4_sort_keys / sort_pairs call that does work on a
+ * device waits for that check once — the only time a sort call blocks; a call under stream
+ * capture leaves it to the next call — and on a device that fails it every sort returns
+ * hipErrorNotSupported (801) instead of a result that may be unstable.
  */
 int thrust_cdna4_selftest_lds_atomic_order(long long* mismatches, void* stream);
 

@@ -23,6 +23,7 @@ SYMBOLS = [
     "thrust_cdna4_profile_count", "thrust_cdna4_profile_get",
     "thrust_cdna4_selftest_lds_atomic_order", "thrust_cdna4_set_lookback_patience",
     "thrust_cdna4_set_test_publish_delay", "thrust_cdna4_scan_static",
+    "thrust_cdna4_lookback_timeouts",
     "thrust_cdna4_stream_create", "thrust_cdna4_stream_destroy", "thrust_cdna4_stream_query",
     "thrust_cdna4_event_create", "thrust_cdna4_event_destroy", "thrust_cdna4_event_record", "thrust_cdna4_event_query",
     "thrust_cdna4_stream_wait_event", "thrust_cdna4_malloc_direct", "thrust_cdna4_free_direct",
@@ -83,6 +84,7 @@ def lib():
     L.thrust_cdna4_free_direct.argtypes = [vp]
     L.thrust_cdna4_set_lookback_patience.argtypes = [i32]
     L.thrust_cdna4_set_test_publish_delay.argtypes = [i32]
+    L.thrust_cdna4_lookback_timeouts.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
     L.thrust_cdna4_profile_enable.argtypes = [i32]
     L.thrust_cdna4_selftest_lds_atomic_order.argtypes = [ctypes.POINTER(ctypes.c_longlong), vp]
     L.thrust_cdna4_profile_get.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p),

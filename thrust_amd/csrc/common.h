@@ -409,6 +409,9 @@ inline bool dispatch_op(int op, F&& f) {
   return false;
 }
 
+// Compute units of the current device (cached per device); 256 if the query fails.
+int device_cu_count();
+
 // Optional launch profiling: when enabled, every kernel launch of the library is bracketed by
 // HIP events on the launch stream and logged under its name (the counterpart of the
 // reference's THRUST_DEBUG_SYNC launch log, thrust/system/cuda/detail/core/agent_launcher.h:523-559).

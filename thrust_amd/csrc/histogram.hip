@@ -172,7 +172,7 @@ static void launch_hist(const T* samples, int64_t n, uint32_t* counts, int num_b
   if (LDS > 0)
     while (copies_log2 < 5 && ((int64_t)lds_bins << (copies_log2 + 1)) <= LDS) copies_log2++;
   int64_t blocks = ceil_div(n, (int64_t)kHistBlock * (16 / (int)sizeof(T)) * 4);
-  const int64_t cap = 256 * (int64_t)blocks_per_cu;
+  const int64_t cap = (int64_t)device_cu_count() * blocks_per_cu;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   TCD_LAUNCH("histogram_kernel", (histogram_kernel<T, LDS, MODE>), dim3((unsigned)blocks), dim3(kHistBlock), s,

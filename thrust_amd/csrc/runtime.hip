@@ -27,6 +27,22 @@ hipError_t zero_async(void* p, size_t bytes, hipStream_t stream) {
   return hipGetLastError();
 }
 
+int device_cu_count() {
+  constexpr int kMaxDev = 64;
+  static std::atomic<int> cached[kMaxDev];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 256;
+  int c = cached[dev].load(std::memory_order_relaxed);
+  if (c == 0) {
+    if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0) {
+      (void)hipGetLastError();
+      c = 256;
+    }
+    cached[dev].store(c, std::memory_order_relaxed);
+  }
+  return c;
+}
+
 // ---------------------------------------------------------------------------------------
 // Launch profiling records
 // ---------------------------------------------------------------------------------------

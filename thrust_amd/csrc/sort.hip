@@ -19,6 +19,9 @@
 // order-preserving encoding of thrust/system/detail/sequential/stable_radix_sort.inl:43-139
 // on the fly, so there are no separate encode/decode passes.  Replaces
 // thrust/system/cuda/detail/sort.h:213-380 (cub::DeviceRadixSort).
+#include <atomic>
+#include <mutex>
+
 #include "common.h"
 
 namespace tcd {
@@ -85,9 +88,6 @@ __device__ __host__ inline U decode_key(U e, U xor_mask) {
 // 8-byte keys, 32 for narrower ones.
 #ifndef TCD_SORT_HIST_UNROLL
 #define TCD_SORT_HIST_UNROLL 8  // 128-bit loads in flight per thread
-#endif
-#ifndef TCD_SORT_HIST_BLOCKS
-#define TCD_SORT_HIST_BLOCKS 256
 #endif
 constexpr int kHistThreads = 512;
 template <class U>
@@ -194,6 +194,12 @@ __device__ inline uint32_t lds_load(const uint32_t* p) {
 __device__ inline void lds_store(uint32_t* p, uint32_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
 }
+
+// Look-back polls that find nothing new before a digit's thread gives up (seconds: far beyond
+// any wait that ends).  The kernel then still runs to completion, with wrong positions that
+// stay inside the output, and counts the event in g_lookback_timeouts.
+constexpr uint32_t kLookbackSpinLimit = 1u << 22;
+__device__ unsigned int g_lookback_timeouts;
 
 template <class U, int VB, bool FLOAT, int BLOCK, int IPT, int WPE, class D>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) void onesweep_kernel(const U* __restrict__ kin, U* __restrict__ kout,
@@ -340,6 +346,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
     if (tile > 0) {
       int64_t t = tile - 1;
       bool done = false;
+      uint32_t spins = 0;
       while (!done) {
         D v[kLookW];
 #pragma unroll
@@ -356,7 +363,13 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
           }
         }
         t -= used;
-        if (used == 0) __builtin_amdgcn_s_sleep(2);
+        if (used == 0) {
+          __builtin_amdgcn_s_sleep(2);
+          if (++spins > kLookbackSpinLimit) {  // never in a working system; keeps every wait bounded
+            atomicAdd(&g_lookback_timeouts, 1u);
+            done = true;
+          }
+        }
       }
       st_agent(&desc[tile * kRadix + tid], DescWord<D>::make(kInclusive, prefix + total));
     }
@@ -532,6 +545,54 @@ __global__ __launch_bounds__(512) void lds_atomic_order_kernel(unsigned long lon
   if (bad) atomicAdd(mismatches, bad);
 }
 
+// The ranking's assumption is checked once per device, by the first sort that runs there: a
+// short run of the kernel above on the caller's stream, whose result is waited for (the only
+// time a sort call blocks).  A device that fails it gets hipErrorNotSupported from every sort
+// instead of a possibly unstable result.  A call made under stream capture cannot wait and
+// leaves the check to the next call that can.
+__device__ unsigned long long g_order_mismatches;
+constexpr int kMaxDevices = 64;
+static std::atomic<int> g_order_verdict[kMaxDevices];  // 0 not checked, 1 in order, 2 not
+static std::mutex g_order_mu;
+
+static hipError_t run_lds_order_check(hipStream_t s, int iters, unsigned long long* mismatches) {
+  void* sym = nullptr;
+  hipError_t e = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_order_mismatches));
+  if (e != hipSuccess) return e;
+  e = zero_async(sym, sizeof(unsigned long long), s);
+  if (e != hipSuccess) return e;
+  TCD_LAUNCH("lds_atomic_order_kernel", lds_atomic_order_kernel, dim3(1024), dim3(512), s,
+             static_cast<unsigned long long*>(sym), iters);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  e = hipMemcpyAsync(mismatches, sym, sizeof(*mismatches), hipMemcpyDeviceToHost, s);
+  if (e != hipSuccess) return e;
+  return hipStreamSynchronize(s);
+}
+
+static hipError_t ensure_lds_order(hipStream_t s) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  int v = g_order_verdict[dev].load(std::memory_order_acquire);
+  if (v == 1) return hipSuccess;
+  if (v == 2) return hipErrorNotSupported;
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cs) != hipSuccess) (void)hipGetLastError();
+  else if (cs != hipStreamCaptureStatusNone) return hipSuccess;
+  std::lock_guard<std::mutex> g(g_order_mu);
+  v = g_order_verdict[dev].load(std::memory_order_acquire);
+  if (v == 0) {
+    unsigned long long bad = 0;
+    e = run_lds_order_check(s, 24, &bad);  // 1.2e7 checked atomics
+    if (e != hipSuccess) return e;
+    v = bad == 0 ? 1 : 2;
+    g_order_verdict[dev].store(v, std::memory_order_release);
+  }
+  return v == 1 ? hipSuccess : hipErrorNotSupported;
+}
+
 // ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
@@ -622,6 +683,10 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   }
   if (*temp_bytes < plan.total) return hipErrorInvalidValue;
   if (n == 0) return hipSuccess;
+  {
+    const hipError_t oe = ensure_lds_order(stream);
+    if (oe != hipSuccess) return oe;
+  }
   if (n <= kTileSortMax) {  // one workgroup, one launch, nothing of `temp` is used
     TCD_LAUNCH("tile_sort_kernel", (tile_sort_kernel<U, VB, FLOAT>), dim3(1), dim3(kTileSortThreads), stream,
                static_cast<U*>(keys), values, (int)n, xor_mask);
@@ -639,7 +704,8 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
 
   const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & (sizeof(U) - 1)) == 0;  // see load16
   int64_t hblocks = ceil_div(n, kHistThreads * 64);
-  if (hblocks > TCD_SORT_HIST_BLOCKS) hblocks = TCD_SORT_HIST_BLOCKS;  // one workgroup per CU, eight loads in flight per thread: 1 % of a 2^28 sort over two with two
+  const int cus = device_cu_count();
+  if (hblocks > cus) hblocks = cus;  // one workgroup per CU, eight loads in flight per thread: 1 % of a 2^28 sort over two with two
   TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(kHistThreads), stream,
              kbuf[0], n, xor_mask, ghist, vec_ok);
   TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(P), dim3(256), stream, ghist);
@@ -724,22 +790,20 @@ extern "C" int thrust_cdna4_sort_pairs(void* temp, size_t* temp_bytes, int key_d
   return hipErrorInvalidValue;
 }
 
+extern "C" int thrust_cdna4_lookback_timeouts(unsigned long long* count) {
+  if (!count) return hipErrorInvalidValue;
+  unsigned int c = 0;
+  const hipError_t e = hipMemcpyFromSymbol(&c, HIP_SYMBOL(tcd::g_lookback_timeouts), sizeof(c));
+  *count = c;
+  return (int)e;
+}
+
 extern "C" int thrust_cdna4_selftest_lds_atomic_order(long long* mismatches, void* stream) {
   using namespace tcd;
   if (!mismatches) return hipErrorInvalidValue;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  unsigned long long* d = nullptr;
-  hipError_t e = hipMalloc(&d, sizeof(*d));
-  if (e != hipSuccess) return (int)e;
-  e = zero_async(d, sizeof(*d), s);
-  if (e == hipSuccess) {
-    TCD_LAUNCH("lds_atomic_order_kernel", lds_atomic_order_kernel, dim3(1024), dim3(512), s, d, 600);
-    e = hipGetLastError();
-  }
-  unsigned long long h = 0;
-  if (e == hipSuccess) e = hipMemcpyAsync(&h, d, sizeof(h), hipMemcpyDeviceToHost, s);
-  if (e == hipSuccess) e = hipStreamSynchronize(s);
-  hipFree(d);
-  *mismatches = (long long)h;
+  unsigned long long bad = 0;
+  std::lock_guard<std::mutex> g(g_order_mu);  // one user of the result word at a time
+  const hipError_t e = run_lds_order_check(static_cast<hipStream_t>(stream), 600, &bad);
+  *mismatches = (long long)bad;
   return (int)e;
 }
