@@ -15,30 +15,55 @@
 namespace thrust {
 
 // ---- device
+namespace detail {
+template <class K, class V, class KIn, class VIn, class KOut, class VOut, class Pred, class Op> struct reduce_by_key_has_kernel {
+  static constexpr bool value = system::cdna4::detail::dtype_of<K>::supported && system::cdna4::detail::dtype_of<V>::supported &&
+                                builtin_equal_on<Pred, K>::value && builtin_op_on<Op, V>::value &&
+                                raw_pointer_to<KIn, K>::value && raw_pointer_to<VIn, V>::value &&
+                                raw_pointer_to<KOut, K>::value && raw_pointer_to<VOut, V>::value;
+};
+template <class K, class V, class Policy, class KIn, class VIn, class KOut, class VOut, class Pred, class Op>
+std::int64_t reduce_by_key_dispatch(const Policy& exec, KIn keys, VIn vals, KOut ko, VOut vo, std::int64_t n, Pred pred, Op op, std::true_type) {
+#if defined(__HIPCC__)
+  if (n >= (std::int64_t(1) << 32))  // beyond the precompiled kernels' range
+    return system::cdna4::detail::generic_reduce_by_key<V>(exec, keys, vals, ko, vo, n, pred, op);
+#else
+  (void)pred; (void)op;  // without the kernel templates such a call fails with the C ABI's error code
+#endif
+  return system::cdna4::detail::reduce_by_key(exec, static_cast<const K*>(keys), static_cast<const V*>(vals), ko, vo, n,
+                                              typename rebind_op<Pred, K>::type(), typename rebind_op<Op, V>::type());
+}
+template <class K, class V, class Policy, class KIn, class VIn, class KOut, class VOut, class Pred, class Op>
+std::int64_t reduce_by_key_dispatch(const Policy& exec, KIn keys, VIn vals, KOut ko, VOut vo, std::int64_t n, Pred pred, Op op, std::false_type) {
+  return system::cdna4::detail::generic_reduce_by_key<V>(exec, keys, vals, ko, vo, n, pred, op);
+}
+}  // namespace detail
+
+// Raw device pointers to arithmetic types under equal_to and a built-in operator run the
+// precompiled segmented-reduction kernel; everything else (user predicates and operators, fancy
+// iterators read in place, more than 2^32 - 1 elements) the kernel templates of scan_generic.h.
 template <class D, class KIt, class VIt, class KOut, class VOut, class Pred, class Op>
 pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
-                               KOut kout, VOut vout, Pred, Op) {
-  namespace sd = system::cdna4::detail;
+                               KOut kout, VOut vout, Pred pred, Op op) {
   typedef typename detail::elem<KIt>::type K;
   typedef typename detail::elem<VIt>::type V;
+  typedef typename detail::unwrap_iterator<KIt>::type KIn;
+  typedef typename detail::unwrap_iterator<VIt>::type VIn;
+  typedef typename detail::unwrap_iterator<KOut>::type KO;
+  typedef typename detail::unwrap_iterator<VOut>::type VO;
   const std::int64_t n = (std::int64_t)(klast - kfirst);
-  sd::contiguous_input<K, typename detail::unwrap_iterator<KIt>::type> keys(exec.derived(), detail::unwrap(kfirst), n);
-  sd::contiguous_input<V, typename detail::unwrap_iterator<VIt>::type> vals(exec.derived(), detail::unwrap(vfirst), n);
-  sd::contiguous_output<K, typename detail::unwrap_iterator<KOut>::type> ko(exec.derived(), detail::unwrap(kout), n);
-  sd::contiguous_output<V, typename detail::unwrap_iterator<VOut>::type> vo(exec.derived(), detail::unwrap(vout), n);
-  const std::int64_t runs = sd::reduce_by_key(exec.derived(), keys.data(), vals.data(), ko.data(), vo.data(), n,
-                                              typename detail::rebind_op<Pred, K>::type(), typename detail::rebind_op<Op, V>::type());
-  ko.flush(exec.derived(), runs);
-  vo.flush(exec.derived(), runs);
+  const std::int64_t runs = detail::reduce_by_key_dispatch<K, V>(
+      exec.derived(), detail::unwrap(kfirst), detail::unwrap(vfirst), detail::unwrap(kout), detail::unwrap(vout), n, pred, op,
+      std::integral_constant<bool, detail::reduce_by_key_has_kernel<K, V, KIn, VIn, KO, VO, Pred, Op>::value>());
   return thrust::make_pair(kout + runs, vout + runs);
 }
 template <class D, class KIt, class VIt, class KOut, class VOut, class Pred>
 pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred p) {
-  return reduce_by_key(exec, kf, kl, vf, ko, vo, p, plus<typename detail::elem<VIt>::type>());
+  return reduce_by_key(exec, kf, kl, vf, ko, vo, p, plus<>());
 }
 template <class D, class KIt, class VIt, class KOut, class VOut>
 pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo) {
-  return reduce_by_key(exec, kf, kl, vf, ko, vo, equal_to<typename detail::elem<KIt>::type>());
+  return reduce_by_key(exec, kf, kl, vf, ko, vo, equal_to<>());
 }
 
 // ---- host

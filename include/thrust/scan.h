@@ -8,6 +8,7 @@
 #include <thrust/functional.h>
 #include <thrust/system/cdna4/detail/algorithms.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
+#include <thrust/system/cdna4/detail/scan_generic.h>
 
 namespace thrust {
 
@@ -22,44 +23,70 @@ template <template <class> class F, class T> struct rebind_op<F<void>, T> { type
 }  // namespace detail
 
 // ===================================================================== scan, device
+namespace detail {
+// The precompiled kernels serve raw device pointers to one arithmetic type under one of the four
+// built-in operators of that type (or its transparent form); everything else goes to the kernel
+// templates of scan_generic.h.
+template <class Op, class T> struct builtin_op_on { static constexpr bool value = false; };
+template <template <class> class F, class T> struct builtin_op_on<F<T>, T> {
+  static constexpr bool value = system::cdna4::detail::op_code<F<T>>::value >= 0;
+};
+template <template <class> class F, class T> struct builtin_op_on<F<void>, T> {
+  static constexpr bool value = system::cdna4::detail::op_code<F<T>>::value >= 0;
+};
+template <class P, class T> struct raw_pointer_to {
+  static constexpr bool value = std::is_pointer<P>::value &&
+      std::is_same<typename std::remove_cv<typename std::remove_pointer<P>::type>::type, T>::value;
+};
+template <class T, class In, class Out, class Op> struct scan_has_kernel {
+  static constexpr bool value = system::cdna4::detail::dtype_of<T>::supported && builtin_op_on<Op, T>::value &&
+                                raw_pointer_to<In, T>::value && raw_pointer_to<Out, T>::value;
+};
+
+template <bool EXCLUSIVE, class Policy, class T, class In, class Out, class Op>
+void scan_dispatch(const Policy& exec, In in, Out out, std::int64_t n, T init, Op, std::true_type) {
+  system::cdna4::detail::scan(exec, static_cast<const T*>(in), out, n, EXCLUSIVE, EXCLUSIVE ? &init : (const T*)nullptr,
+                              typename rebind_op<Op, T>::type());
+}
+template <bool EXCLUSIVE, class Policy, class T, class In, class Out, class Op>
+void scan_dispatch(const Policy& exec, In in, Out out, std::int64_t n, T init, Op op, std::false_type) {
+  system::cdna4::detail::generic_scan<EXCLUSIVE, T>(exec, in, out, n, init, op);
+}
+}  // namespace detail
+
+// The accumulator of an inclusive scan has the input's value type (thrust/system/cuda/detail/scan.h:63).
 template <class D, class InIt, class OutIt, class Op>
-OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, Op) {
-  namespace sd = system::cdna4::detail;
+OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, Op op) {
   typedef typename detail::elem<InIt>::type T;
+  typedef typename detail::unwrap_iterator<InIt>::type In;
+  typedef typename detail::unwrap_iterator<OutIt>::type Out;
   const std::int64_t n = (std::int64_t)(last - first);
-  sd::contiguous_input<T, typename detail::unwrap_iterator<InIt>::type> in(exec.derived(), detail::unwrap(first), n);
-  sd::contiguous_output<T, typename detail::unwrap_iterator<OutIt>::type> out(exec.derived(), detail::unwrap(result), n);
-  sd::scan(exec.derived(), in.data(), out.data(), n, false, (const T*)nullptr, typename detail::rebind_op<Op, T>::type());
-  out.flush(exec.derived(), n);
+  detail::scan_dispatch<false>(exec.derived(), detail::unwrap(first), detail::unwrap(result), n, T(), op,
+                               std::integral_constant<bool, detail::scan_has_kernel<T, In, Out, Op>::value>());
   return result + n;
 }
 template <class D, class InIt, class OutIt>
 OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result) {
-  return inclusive_scan(exec, first, last, result, plus<typename detail::elem<InIt>::type>());
+  return inclusive_scan(exec, first, last, result, plus<>());
 }
-// The accumulator of an exclusive scan has the type of `init` (thrust/system/cuda/detail/scan.h:142-154);
-// the kernels accumulate in the element type, so the two must be the same type.
+// The accumulator of an exclusive scan has the type of `init` (thrust/system/cuda/detail/scan.h:142-154).
 template <class D, class InIt, class OutIt, class T, class Op>
-OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, T init, Op) {
-  namespace sd = system::cdna4::detail;
-  typedef typename detail::elem<InIt>::type V;
-  static_assert(std::is_same<V, T>::value,
-                "cdna4 exclusive_scan: init must have the element type (it is the accumulator type)");
+OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, T init, Op op) {
+  typedef typename detail::unwrap_iterator<InIt>::type In;
+  typedef typename detail::unwrap_iterator<OutIt>::type Out;
   const std::int64_t n = (std::int64_t)(last - first);
-  sd::contiguous_input<V, typename detail::unwrap_iterator<InIt>::type> in(exec.derived(), detail::unwrap(first), n);
-  sd::contiguous_output<V, typename detail::unwrap_iterator<OutIt>::type> out(exec.derived(), detail::unwrap(result), n);
-  sd::scan(exec.derived(), in.data(), out.data(), n, true, &init, typename detail::rebind_op<Op, V>::type());
-  out.flush(exec.derived(), n);
+  detail::scan_dispatch<true>(exec.derived(), detail::unwrap(first), detail::unwrap(result), n, init, op,
+                              std::integral_constant<bool, detail::scan_has_kernel<T, In, Out, Op>::value>());
   return result + n;
 }
 template <class D, class InIt, class OutIt, class T>
 OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, T init) {
-  return exclusive_scan(exec, first, last, result, init, plus<typename detail::elem<InIt>::type>());
+  return exclusive_scan(exec, first, last, result, init, plus<>());
 }
 template <class D, class InIt, class OutIt>
 OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result) {
   typedef typename detail::elem<InIt>::type V;
-  return exclusive_scan(exec, first, last, result, V(), plus<V>());  // thrust/system/cuda/detail/scan.h:347-348
+  return exclusive_scan(exec, first, last, result, V(), plus<>());  // thrust/system/cuda/detail/scan.h:347-348
 }
 
 // ===================================================================== scan, host
@@ -126,52 +153,79 @@ template <class InIt, class OutIt, class T, class Op, detail::enable_if_host<InI
 OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init, Op op) { return exclusive_scan(host, f, l, r, init, op); }
 
 // ===================================================================== scan_by_key, device
+namespace detail {
+template <class Pred, class K> struct builtin_equal_on { static constexpr bool value = false; };
+template <class K> struct builtin_equal_on<equal_to<K>, K> { static constexpr bool value = true; };
+template <class K> struct builtin_equal_on<equal_to<void>, K> { static constexpr bool value = true; };
+template <class K, class V, class KIn, class VIn, class Out, class Pred, class Op> struct scan_by_key_has_kernel {
+  static constexpr bool value = system::cdna4::detail::dtype_of<K>::supported && system::cdna4::detail::dtype_of<V>::supported &&
+                                builtin_equal_on<Pred, K>::value && builtin_op_on<Op, V>::value &&
+                                raw_pointer_to<KIn, K>::value && raw_pointer_to<VIn, V>::value && raw_pointer_to<Out, V>::value;
+};
+template <bool EXCLUSIVE, class K, class Policy, class V, class KIn, class VIn, class Out, class Pred, class Op>
+void scan_by_key_dispatch(const Policy& exec, KIn keys, VIn vals, Out out, std::int64_t n, V init, Pred pred, Op op, std::true_type) {
+#if defined(__HIPCC__)
+  if (n >= (std::int64_t(1) << 32)) {  // beyond the precompiled kernels' range
+    system::cdna4::detail::generic_scan_by_key<EXCLUSIVE, V>(exec, keys, vals, out, n, init, pred, op);
+    return;
+  }
+#else
+  (void)pred; (void)op;  // without the kernel templates such a call fails with the C ABI's error code
+#endif
+  system::cdna4::detail::scan_by_key(exec, static_cast<const K*>(keys), static_cast<const V*>(vals), out, n, EXCLUSIVE,
+                                     EXCLUSIVE ? &init : (const V*)nullptr, typename rebind_op<Pred, K>::type(),
+                                     typename rebind_op<Op, V>::type());
+}
+template <bool EXCLUSIVE, class K, class Policy, class V, class KIn, class VIn, class Out, class Pred, class Op>
+void scan_by_key_dispatch(const Policy& exec, KIn keys, VIn vals, Out out, std::int64_t n, V init, Pred pred, Op op, std::false_type) {
+  system::cdna4::detail::generic_scan_by_key<EXCLUSIVE, V>(exec, keys, vals, out, n, init, pred, op);
+}
+}  // namespace detail
+
+// The accumulator has the value input's type for the inclusive form and the type of `init` for
+// the exclusive one (thrust/system/cuda/detail/scan_by_key.h:69-282).
 template <class D, class KIt, class VIt, class OutIt, class Pred, class Op>
 OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
-                            OutIt result, Pred, Op) {
-  namespace sd = system::cdna4::detail;
+                            OutIt result, Pred pred, Op op) {
   typedef typename detail::elem<KIt>::type K;
   typedef typename detail::elem<VIt>::type V;
+  typedef typename detail::unwrap_iterator<KIt>::type KIn;
+  typedef typename detail::unwrap_iterator<VIt>::type VIn;
+  typedef typename detail::unwrap_iterator<OutIt>::type Out;
   const std::int64_t n = (std::int64_t)(klast - kfirst);
-  sd::contiguous_input<K, typename detail::unwrap_iterator<KIt>::type> keys(exec.derived(), detail::unwrap(kfirst), n);
-  sd::contiguous_input<V, typename detail::unwrap_iterator<VIt>::type> vals(exec.derived(), detail::unwrap(vfirst), n);
-  sd::contiguous_output<V, typename detail::unwrap_iterator<OutIt>::type> out(exec.derived(), detail::unwrap(result), n);
-  sd::scan_by_key(exec.derived(), keys.data(), vals.data(), out.data(), n, false, (const V*)nullptr,
-                  typename detail::rebind_op<Pred, K>::type(), typename detail::rebind_op<Op, V>::type());
-  out.flush(exec.derived(), n);
+  detail::scan_by_key_dispatch<false, K>(exec.derived(), detail::unwrap(kfirst), detail::unwrap(vfirst), detail::unwrap(result), n,
+                                         V(), pred, op,
+                                         std::integral_constant<bool, detail::scan_by_key_has_kernel<K, V, KIn, VIn, Out, Pred, Op>::value>());
   return result + n;
 }
 template <class D, class KIt, class VIt, class OutIt, class Pred>
 OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, Pred p) {
-  return inclusive_scan_by_key(exec, kf, kl, vf, r, p, plus<typename detail::elem<VIt>::type>());
+  return inclusive_scan_by_key(exec, kf, kl, vf, r, p, plus<>());
 }
 template <class D, class KIt, class VIt, class OutIt>
 OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r) {
-  return inclusive_scan_by_key(exec, kf, kl, vf, r, equal_to<typename detail::elem<KIt>::type>());
+  return inclusive_scan_by_key(exec, kf, kl, vf, r, equal_to<>());
 }
 template <class D, class KIt, class VIt, class OutIt, class T, class Pred, class Op>
 OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
-                            OutIt result, T init, Pred, Op) {
-  namespace sd = system::cdna4::detail;
+                            OutIt result, T init, Pred pred, Op op) {
   typedef typename detail::elem<KIt>::type K;
-  typedef typename detail::elem<VIt>::type V;
-  static_assert(std::is_same<V, T>::value, "cdna4 exclusive_scan_by_key: init must have the values' element type");
+  typedef typename detail::unwrap_iterator<KIt>::type KIn;
+  typedef typename detail::unwrap_iterator<VIt>::type VIn;
+  typedef typename detail::unwrap_iterator<OutIt>::type Out;
   const std::int64_t n = (std::int64_t)(klast - kfirst);
-  sd::contiguous_input<K, typename detail::unwrap_iterator<KIt>::type> keys(exec.derived(), detail::unwrap(kfirst), n);
-  sd::contiguous_input<V, typename detail::unwrap_iterator<VIt>::type> vals(exec.derived(), detail::unwrap(vfirst), n);
-  sd::contiguous_output<V, typename detail::unwrap_iterator<OutIt>::type> out(exec.derived(), detail::unwrap(result), n);
-  sd::scan_by_key(exec.derived(), keys.data(), vals.data(), out.data(), n, true, &init,
-                  typename detail::rebind_op<Pred, K>::type(), typename detail::rebind_op<Op, V>::type());
-  out.flush(exec.derived(), n);
+  detail::scan_by_key_dispatch<true, K>(exec.derived(), detail::unwrap(kfirst), detail::unwrap(vfirst), detail::unwrap(result), n,
+                                        init, pred, op,
+                                        std::integral_constant<bool, detail::scan_by_key_has_kernel<K, T, KIn, VIn, Out, Pred, Op>::value>());
   return result + n;
 }
 template <class D, class KIt, class VIt, class OutIt, class T, class Pred>
 OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, T init, Pred p) {
-  return exclusive_scan_by_key(exec, kf, kl, vf, r, init, p, plus<typename detail::elem<VIt>::type>());
+  return exclusive_scan_by_key(exec, kf, kl, vf, r, init, p, plus<>());
 }
 template <class D, class KIt, class VIt, class OutIt, class T>
 OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, T init) {
-  return exclusive_scan_by_key(exec, kf, kl, vf, r, init, equal_to<typename detail::elem<KIt>::type>());
+  return exclusive_scan_by_key(exec, kf, kl, vf, r, init, equal_to<>());
 }
 template <class D, class KIt, class VIt, class OutIt>
 OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r) {
