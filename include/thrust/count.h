@@ -6,7 +6,7 @@
 namespace thrust {
 namespace detail {
 template <class F> struct flag_of {
-  F pred;
+  mutable F pred;
   template <class T> THRUST_CDNA4_HD std::ptrdiff_t operator()(const T& x) const { return pred(x) ? 1 : 0; }
 };
 template <class V> struct equals_value {

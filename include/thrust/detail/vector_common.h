@@ -1,0 +1,26 @@
+#pragma once
+// As in the reference, whose vector headers pull in most of the library, a translation unit that
+// includes a vector header can use the common algorithms and iterators without naming their headers.
+#include <thrust/advance.h>
+#include <thrust/copy.h>
+#include <thrust/distance.h>
+#include <thrust/equal.h>
+#include <thrust/fill.h>
+#include <thrust/for_each.h>
+#include <thrust/functional.h>
+#include <thrust/iterator/constant_iterator.h>
+#include <thrust/iterator/counting_iterator.h>
+#include <thrust/iterator/discard_iterator.h>
+#include <thrust/iterator/iterator_traits.h>
+#include <thrust/iterator/permutation_iterator.h>
+#include <thrust/iterator/reverse_iterator.h>
+#include <thrust/iterator/transform_iterator.h>
+#include <thrust/iterator/zip_iterator.h>
+#include <thrust/pair.h>
+#include <thrust/reduce.h>
+#include <thrust/sequence.h>
+#include <thrust/swap.h>
+#include <thrust/transform.h>
+#include <thrust/gather.h>
+#include <thrust/scatter.h>
+#include <thrust/tuple.h>

@@ -5,6 +5,7 @@
 #pragma once
 #include <cstddef>
 #include <iterator>
+#include <thrust/detail/hd.h>
 #include <thrust/system/cdna4/detail/core.h>
 
 namespace thrust {
@@ -15,19 +16,28 @@ template <class T>
 class device_reference {
  public:
   typedef typename std::remove_const<T>::type value_type;
-  explicit device_reference(T* p) : p_(p) {}
-  operator value_type() const {
+  THRUST_CDNA4_HD explicit device_reference(T* p) : p_(p) {}
+  // on the host one synchronous element copy; inside a kernel the element itself
+  THRUST_CDNA4_HD operator value_type() const {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *p_;
+#else
     value_type v;
     system::cdna4::detail::throw_on_error(thrust_cdna4_read_back(&v, p_, sizeof(T), nullptr), "get_value");
     return v;
+#endif
   }
-  device_reference& operator=(const value_type& v) {
+  THRUST_CDNA4_HD device_reference& operator=(const value_type& v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    *p_ = v;
+#else
     system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_htod(p_, &v, sizeof(T), nullptr), "assign_value");
     system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "assign_value");
+#endif
     return *this;
   }
-  device_reference& operator=(const device_reference& o) { return *this = static_cast<value_type>(o); }
-  device_ptr<T> operator&() const { return device_ptr<T>(p_); }
+  THRUST_CDNA4_HD device_reference& operator=(const device_reference& o) { return *this = static_cast<value_type>(o); }
+  THRUST_CDNA4_HD device_ptr<T> operator&() const { return device_ptr<T>(p_); }
 
  private:
   T* p_;
@@ -43,38 +53,38 @@ class device_ptr {
   typedef device_reference<T> reference;
   typedef system::cdna4::tag system_tag;
 
-  device_ptr() : p_(nullptr) {}
-  explicit device_ptr(T* p) : p_(p) {}
+  THRUST_CDNA4_HD device_ptr() : p_(nullptr) {}
+  THRUST_CDNA4_HD explicit device_ptr(T* p) : p_(p) {}
   template <class U, class = typename std::enable_if<std::is_convertible<U*, T*>::value>::type>
-  device_ptr(const device_ptr<U>& o) : p_(o.get()) {}
-  T* get() const { return p_; }
-  reference operator*() const { return reference(p_); }
-  reference operator[](difference_type i) const { return reference(p_ + i); }
-  device_ptr& operator++() { ++p_; return *this; }
-  device_ptr operator++(int) { device_ptr t(*this); ++p_; return t; }
-  device_ptr& operator--() { --p_; return *this; }
-  device_ptr operator--(int) { device_ptr t(*this); --p_; return t; }
-  device_ptr& operator+=(difference_type d) { p_ += d; return *this; }
-  device_ptr& operator-=(difference_type d) { p_ -= d; return *this; }
-  friend device_ptr operator+(device_ptr a, difference_type d) { return device_ptr(a.p_ + d); }
-  friend device_ptr operator+(difference_type d, device_ptr a) { return device_ptr(a.p_ + d); }
-  friend device_ptr operator-(device_ptr a, difference_type d) { return device_ptr(a.p_ - d); }
-  friend difference_type operator-(device_ptr a, device_ptr b) { return a.p_ - b.p_; }
-  friend bool operator==(device_ptr a, device_ptr b) { return a.p_ == b.p_; }
-  friend bool operator!=(device_ptr a, device_ptr b) { return a.p_ != b.p_; }
-  friend bool operator<(device_ptr a, device_ptr b) { return a.p_ < b.p_; }
-  friend bool operator>(device_ptr a, device_ptr b) { return a.p_ > b.p_; }
-  friend bool operator<=(device_ptr a, device_ptr b) { return a.p_ <= b.p_; }
-  friend bool operator>=(device_ptr a, device_ptr b) { return a.p_ >= b.p_; }
+  THRUST_CDNA4_HD device_ptr(const device_ptr<U>& o) : p_(o.get()) {}
+  THRUST_CDNA4_HD T* get() const { return p_; }
+  THRUST_CDNA4_HD reference operator*() const { return reference(p_); }
+  THRUST_CDNA4_HD reference operator[](difference_type i) const { return reference(p_ + i); }
+  THRUST_CDNA4_HD device_ptr& operator++() { ++p_; return *this; }
+  THRUST_CDNA4_HD device_ptr operator++(int) { device_ptr t(*this); ++p_; return t; }
+  THRUST_CDNA4_HD device_ptr& operator--() { --p_; return *this; }
+  THRUST_CDNA4_HD device_ptr operator--(int) { device_ptr t(*this); --p_; return t; }
+  THRUST_CDNA4_HD device_ptr& operator+=(difference_type d) { p_ += d; return *this; }
+  THRUST_CDNA4_HD device_ptr& operator-=(difference_type d) { p_ -= d; return *this; }
+  THRUST_CDNA4_HD friend device_ptr operator+(device_ptr a, difference_type d) { return device_ptr(a.p_ + d); }
+  THRUST_CDNA4_HD friend device_ptr operator+(difference_type d, device_ptr a) { return device_ptr(a.p_ + d); }
+  THRUST_CDNA4_HD friend device_ptr operator-(device_ptr a, difference_type d) { return device_ptr(a.p_ - d); }
+  THRUST_CDNA4_HD friend difference_type operator-(device_ptr a, device_ptr b) { return a.p_ - b.p_; }
+  THRUST_CDNA4_HD friend bool operator==(device_ptr a, device_ptr b) { return a.p_ == b.p_; }
+  THRUST_CDNA4_HD friend bool operator!=(device_ptr a, device_ptr b) { return a.p_ != b.p_; }
+  THRUST_CDNA4_HD friend bool operator<(device_ptr a, device_ptr b) { return a.p_ < b.p_; }
+  THRUST_CDNA4_HD friend bool operator>(device_ptr a, device_ptr b) { return a.p_ > b.p_; }
+  THRUST_CDNA4_HD friend bool operator<=(device_ptr a, device_ptr b) { return a.p_ <= b.p_; }
+  THRUST_CDNA4_HD friend bool operator>=(device_ptr a, device_ptr b) { return a.p_ >= b.p_; }
 
  private:
   T* p_;
 };
 
-template <class T> inline device_ptr<T> device_pointer_cast(T* p) { return device_ptr<T>(p); }
-template <class T> inline device_ptr<T> device_pointer_cast(device_ptr<T> p) { return p; }
-template <class T> inline T* raw_pointer_cast(device_ptr<T> p) { return p.get(); }
-template <class T> inline T* raw_pointer_cast(T* p) { return p; }
+template <class T> THRUST_CDNA4_HD inline device_ptr<T> device_pointer_cast(T* p) { return device_ptr<T>(p); }
+template <class T> THRUST_CDNA4_HD inline device_ptr<T> device_pointer_cast(device_ptr<T> p) { return p; }
+template <class T> THRUST_CDNA4_HD inline T* raw_pointer_cast(device_ptr<T> p) { return p.get(); }
+template <class T> THRUST_CDNA4_HD inline T* raw_pointer_cast(T* p) { return p; }
 
 // Cached, stream-ordered device allocation (thrust/device_malloc.h, device_free.h).
 template <class T> inline device_ptr<T> device_malloc(std::size_t n) {

@@ -62,6 +62,8 @@ class device_vector {
   const_reference operator[](size_type i) const { return const_reference(p_ + i); }
   reference front() { return (*this)[0]; }
   reference back() { return (*this)[n_ - 1]; }
+  const_reference front() const { return (*this)[0]; }
+  const_reference back() const { return (*this)[n_ - 1]; }
 
   void clear() { n_ = 0; }
   void swap(device_vector& o) noexcept { std::swap(p_, o.p_); std::swap(n_, o.n_); std::swap(cap_, o.cap_); std::swap(alloc_, o.alloc_); }
@@ -190,3 +192,5 @@ host_vector<T, A>& host_vector<T, A>::operator=(const device_vector<T, DA>& d) {
 }
 
 }  // namespace thrust
+
+#include <thrust/detail/vector_common.h>

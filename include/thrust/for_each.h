@@ -6,15 +6,31 @@
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
+namespace system { namespace cdna4 {
+// the device system's implementation, found through the policy's type
 template <class D, class It, class F>
-It for_each(const system::cdna4::execution_policy<D>& exec, It first, It last, F f) {
-  system::cdna4::detail::apply_n(exec.derived(), detail::unwrap(first), (std::int64_t)(last - first), f);
+It for_each(const execution_policy<D>& exec, It first, It last, F f) {
+  detail::apply_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)(last - first), f);
   return last;
 }
 template <class D, class It, class Size, class F>
-It for_each_n(const system::cdna4::execution_policy<D>& exec, It first, Size n, F f) {
-  system::cdna4::detail::apply_n(exec.derived(), detail::unwrap(first), (std::int64_t)n, f);
+It for_each_n(const execution_policy<D>& exec, It first, Size n, F f) {
+  detail::apply_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)n, f);
   return first + n;
+}
+}}  // namespace system::cdna4
+
+// The entry points dispatch on the policy's own type by an unqualified call, as the reference's
+// do (thrust/detail/for_each.inl:32-44): the device system's overload above is found through the
+// policy's base class, and a user's overload for a policy type derived from
+// thrust::device_execution_policy (examples/minimal_custom_backend.cu) is preferred to it.
+template <class D, class It, class F>
+It for_each(const detail::execution_policy_base<D>& exec, It first, It last, F f) {
+  return for_each(static_cast<const D&>(exec), first, last, f);
+}
+template <class D, class It, class Size, class F>
+It for_each_n(const detail::execution_policy_base<D>& exec, It first, Size n, F f) {
+  return for_each_n(static_cast<const D&>(exec), first, n, f);
 }
 template <class It, class F>
 It for_each(const system::cpp::detail::par_t&, It first, It last, F f) { std::for_each(first, last, f); return last; }

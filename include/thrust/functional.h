@@ -1,14 +1,19 @@
 // Function objects the device kernels are specialised on (thrust/functional.h).
 #pragma once
 #include <functional>
-// Callable from kernels when the translation unit is compiled by hipcc (comparison sort with
-// these functors); plain host functions under a host compiler.
-#if defined(__HIPCC__)
-#define THRUST_CDNA4_HD __host__ __device__
-#else
-#define THRUST_CDNA4_HD
-#endif
+#include <thrust/detail/hd.h>
 namespace thrust {
+// Empty bases that only carry the argument and result typedefs of an adaptable function object
+// (thrust/functional.h:66-126); user functors in existing code derive from them.
+template <class Argument, class Result> struct unary_function {
+  typedef Argument argument_type;
+  typedef Result result_type;
+};
+template <class Argument1, class Argument2, class Result> struct binary_function {
+  typedef Argument1 first_argument_type;
+  typedef Argument2 second_argument_type;
+  typedef Result result_type;
+};
 template <class T = void> struct plus { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a + b; } };
 template <class T = void> struct multiplies { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a * b; } };
 template <class T = void> struct maximum { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a < b ? b : a; } };
@@ -56,3 +61,8 @@ template <class F> struct is_equal_to { static constexpr bool value = false; };
 template <class T> struct is_equal_to<thrust::equal_to<T>> { static constexpr bool value = true; };
 }}}  // namespace system::cdna4::detail
 }  // namespace thrust
+// as in the reference, <thrust/functional.h> brings thrust::tuple and thrust::pair with it
+// (placeholder expressions are built on them there)
+#include <thrust/pair.h>
+#include <thrust/tuple.h>
+#include <thrust/detail/placeholders.h>

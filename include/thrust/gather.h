@@ -1,0 +1,71 @@
+// thrust::gather / gather_if (thrust/gather.h): result[i] = input[map[i]].
+#pragma once
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/system/cdna4/detail/index_algorithms.h>
+
+namespace thrust {
+namespace detail {
+template <class Map, class In, class Out> struct gather_body {
+  Map map; In in; Out out;
+  THRUST_CDNA4_HD void operator()(std::int64_t i) { out[i] = in[map[i]]; }
+};
+template <class Map, class S, class In, class Out, class Pred> struct gather_if_body {
+  Map map; S stencil; In in; Out out; Pred pred;
+  THRUST_CDNA4_HD void operator()(std::int64_t i) {
+    if (pred(stencil[i])) out[i] = in[map[i]];
+  }
+};
+struct truthy {
+  template <class T> THRUST_CDNA4_HD bool operator()(const T& x) const { return x ? true : false; }
+};
+}  // namespace detail
+template <class D, class Map, class In, class Out>
+Out gather(const system::cdna4::execution_policy<D>& exec, Map map_first, Map map_last, In input, Out result) {
+  const std::int64_t n = (std::int64_t)(map_last - map_first);
+  system::cdna4::detail::for_each_index(
+      exec.derived(), n,
+      detail::gather_body<typename detail::unwrap_iterator<Map>::type, typename detail::unwrap_iterator<In>::type,
+                          typename detail::unwrap_iterator<Out>::type>{detail::unwrap(map_first), detail::unwrap(input), detail::unwrap(result)},
+      "gather: failed to synchronize");
+  return result + n;
+}
+template <class Map, class In, class Out>
+Out gather(const system::cpp::detail::par_t&, Map map_first, Map map_last, In input, Out result) {
+  for (; map_first != map_last; ++map_first, ++result) *result = input[*map_first];
+  return result;
+}
+template <class D, class Map, class S, class In, class Out, class Pred>
+Out gather_if(const system::cdna4::execution_policy<D>& exec, Map map_first, Map map_last, S stencil, In input, Out result, Pred pred) {
+  const std::int64_t n = (std::int64_t)(map_last - map_first);
+  system::cdna4::detail::for_each_index(
+      exec.derived(), n,
+      detail::gather_if_body<typename detail::unwrap_iterator<Map>::type, typename detail::unwrap_iterator<S>::type,
+                             typename detail::unwrap_iterator<In>::type, typename detail::unwrap_iterator<Out>::type, Pred>{
+          detail::unwrap(map_first), detail::unwrap(stencil), detail::unwrap(input), detail::unwrap(result), pred},
+      "gather_if: failed to synchronize");
+  return result + n;
+}
+template <class Map, class S, class In, class Out, class Pred>
+Out gather_if(const system::cpp::detail::par_t&, Map map_first, Map map_last, S stencil, In input, Out result, Pred pred) {
+  for (; map_first != map_last; ++map_first, ++stencil, ++result)
+    if (pred(*stencil)) *result = input[*map_first];
+  return result;
+}
+template <class Policy, class Map, class S, class In, class Out, detail::enable_if_policy<Policy> = 0>
+Out gather_if(const Policy& exec, Map mf, Map ml, S st, In in, Out out) { return gather_if(exec, mf, ml, st, in, out, detail::truthy()); }
+
+template <class Map, class In, class Out, detail::enable_if_device<Map> = 0>
+Out gather(Map mf, Map ml, In in, Out out) { return gather(device, mf, ml, in, out); }
+template <class Map, class In, class Out, detail::enable_if_host<Map> = 0>
+Out gather(Map mf, Map ml, In in, Out out) { return gather(host, mf, ml, in, out); }
+template <class Map, class S, class In, class Out, detail::enable_if_device<Map> = 0>
+Out gather_if(Map mf, Map ml, S st, In in, Out out) { return gather_if(device, mf, ml, st, in, out); }
+template <class Map, class S, class In, class Out, detail::enable_if_host<Map> = 0>
+Out gather_if(Map mf, Map ml, S st, In in, Out out) { return gather_if(host, mf, ml, st, in, out); }
+template <class Map, class S, class In, class Out, class Pred, detail::enable_if_device<Map> = 0>
+Out gather_if(Map mf, Map ml, S st, In in, Out out, Pred p) { return gather_if(device, mf, ml, st, in, out, p); }
+template <class Map, class S, class In, class Out, class Pred, detail::enable_if_host<Map> = 0>
+Out gather_if(Map mf, Map ml, S st, In in, Out out, Pred p) { return gather_if(host, mf, ml, st, in, out, p); }
+}  // namespace thrust

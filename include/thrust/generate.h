@@ -1,0 +1,32 @@
+// thrust::generate / generate_n (thrust/generate.h): every element is assigned gen().
+#pragma once
+#include <algorithm>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/index_algorithms.h>
+
+namespace thrust {
+namespace detail {
+template <class Out, class G> struct generate_body {
+  Out out; G gen;
+  THRUST_CDNA4_HD void operator()(std::int64_t i) { out[i] = gen(); }
+};
+}  // namespace detail
+template <class D, class It, class G>
+void generate(const system::cdna4::execution_policy<D>& exec, It first, It last, G gen) {
+  typedef typename detail::unwrap_iterator<It>::type Out;
+  system::cdna4::detail::for_each_index(exec.derived(), (std::int64_t)(last - first),
+                                        detail::generate_body<Out, G>{detail::unwrap(first), gen}, "generate: failed to synchronize");
+}
+template <class It, class G>
+void generate(const system::cpp::detail::par_t&, It first, It last, G gen) { std::generate(first, last, gen); }
+template <class Policy, class It, class Size, class G, detail::enable_if_policy<Policy> = 0>
+It generate_n(const Policy& exec, It first, Size n, G gen) {
+  generate(exec, first, first + n, gen);
+  return first + n;
+}
+template <class It, class G, detail::enable_if_device<It> = 0> void generate(It f, It l, G g) { generate(device, f, l, g); }
+template <class It, class G, detail::enable_if_host<It> = 0> void generate(It f, It l, G g) { generate(host, f, l, g); }
+template <class It, class Size, class G, detail::enable_if_device<It> = 0> It generate_n(It f, Size n, G g) { return generate_n(device, f, n, g); }
+template <class It, class Size, class G, detail::enable_if_host<It> = 0> It generate_n(It f, Size n, G g) { return generate_n(host, f, n, g); }
+}  // namespace thrust

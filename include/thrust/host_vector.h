@@ -16,3 +16,4 @@ class host_vector : public std::vector<T, Alloc> {
   template <class DA> host_vector& operator=(const device_vector<T, DA>& d);
 };
 }  // namespace thrust
+#include <thrust/detail/vector_common.h>

@@ -4,8 +4,10 @@
 #include <thrust/iterator/detail/fancy_base.h>
 
 namespace thrust {
-template <class T>
-class counting_iterator : public detail::fancy_base<counting_iterator<T>, T> {
+// System, Traversal and Difference are accepted as in the reference; only a host system tag has an
+// effect (the range then counts as a host range).
+template <class T, class System = use_default, class Traversal = use_default, class Difference = use_default>
+class counting_iterator : public detail::fancy_base<counting_iterator<T, System, Traversal, Difference>, T> {
  public:
   typedef T value_type;
   typedef T reference;
@@ -19,6 +21,8 @@ class counting_iterator : public detail::fancy_base<counting_iterator<T>, T> {
 };
 template <class T> THRUST_CDNA4_HD counting_iterator<T> make_counting_iterator(T v) { return counting_iterator<T>(v); }
 namespace system { namespace cdna4 { namespace detail {
-template <class T> struct is_device_iterator<thrust::counting_iterator<T>> { static constexpr bool value = true; };
+template <class T, class S, class Tr, class D> struct is_device_iterator<thrust::counting_iterator<T, S, Tr, D>> {
+  static constexpr bool value = !std::is_same<S, thrust::system::cpp::tag>::value;
+};
 }}}
 }  // namespace thrust

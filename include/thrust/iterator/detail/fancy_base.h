@@ -5,8 +5,12 @@
 #include <cstddef>
 #include <iterator>
 #include <thrust/functional.h>
+#include <thrust/iterator/iterator_traits.h>
 
-namespace thrust { namespace detail {
+namespace thrust {
+// a template argument left to its default (thrust/iterator/detail/use_default.h)
+struct use_default {};
+namespace detail {
 template <class Derived, class Reference>
 struct fancy_base {
   typedef std::random_access_iterator_tag iterator_category;
@@ -33,4 +37,5 @@ struct fancy_base {
   THRUST_CDNA4_HD friend bool operator<=(const Derived& a, const Derived& b) { return a.distance_to(b) >= 0; }
   THRUST_CDNA4_HD friend bool operator>=(const Derived& a, const Derived& b) { return a.distance_to(b) <= 0; }
 };
-}}  // namespace thrust::detail
+}  // namespace detail
+}  // namespace thrust

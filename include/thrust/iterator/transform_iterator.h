@@ -7,13 +7,23 @@
 namespace thrust {
 namespace detail {
 template <class F, class It> struct transformed_value {
-  typedef typename std::decay<decltype(std::declval<const F&>()(std::declval<typename std::iterator_traits<It>::value_type>()))>::type type;
+  typedef typename std::decay<decltype(std::declval<F&>()(std::declval<typename std::iterator_traits<It>::reference>()))>::type type;
 };
 }  // namespace detail
-template <class F, class It>
-class transform_iterator : public detail::fancy_base<transform_iterator<F, It>, typename detail::transformed_value<F, It>::type> {
+namespace detail {
+// the element type: named by the user (third or fourth template argument, for functors whose
+// result cannot be deduced), else what the functor returns for the base's element
+template <class F, class It, class Reference, class Value> struct transform_iterator_value {
+  typedef typename std::conditional<
+      !std::is_same<Value, use_default>::value, std::decay<Value>,
+      typename std::conditional<!std::is_same<Reference, use_default>::value, std::decay<Reference>, transformed_value<F, It>>::type>::type::type type;
+};
+}  // namespace detail
+template <class F, class It, class Reference = use_default, class Value = use_default>
+class transform_iterator
+    : public detail::fancy_base<transform_iterator<F, It, Reference, Value>, typename detail::transform_iterator_value<F, It, Reference, Value>::type> {
  public:
-  typedef typename detail::transformed_value<F, It>::type value_type;
+  typedef typename detail::transform_iterator_value<F, It, Reference, Value>::type value_type;
   typedef value_type reference;
   transform_iterator() : it_(), f_() {}
   THRUST_CDNA4_HD transform_iterator(It it, F f) : it_(it), f_(f) {}
@@ -24,17 +34,17 @@ class transform_iterator : public detail::fancy_base<transform_iterator<F, It>, 
   THRUST_CDNA4_HD F functor() const { return f_; }
  private:
   It it_;
-  F f_;
+  mutable F f_;  // functors with a non-const operator() are accepted, as in the reference
 };
 template <class F, class It>
 THRUST_CDNA4_HD transform_iterator<F, It> make_transform_iterator(It it, F f) { return transform_iterator<F, It>(it, f); }
 namespace system { namespace cdna4 { namespace detail {
-template <class F, class It> struct is_device_iterator<thrust::transform_iterator<F, It>> : is_device_iterator<It> {};
+template <class F, class It, class R, class V> struct is_device_iterator<thrust::transform_iterator<F, It, R, V>> : is_device_iterator<It> {};
 }}}
 namespace detail {
-template <class F, class It> struct unwrap_iterator<thrust::transform_iterator<F, It>> {
-  typedef thrust::transform_iterator<F, typename unwrap_iterator<It>::type> type;
-  static type apply(const thrust::transform_iterator<F, It>& it) { return type(unwrap(it.base()), it.functor()); }
+template <class F, class It, class R, class V> struct unwrap_iterator<thrust::transform_iterator<F, It, R, V>> {
+  typedef thrust::transform_iterator<F, typename unwrap_iterator<It>::type, R, V> type;
+  static type apply(const thrust::transform_iterator<F, It, R, V>& it) { return type(unwrap(it.base()), it.functor()); }
 };
 }  // namespace detail
 }  // namespace thrust

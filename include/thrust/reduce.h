@@ -12,6 +12,7 @@
 #include <thrust/scan.h>
 #include <thrust/system/cdna4/detail/algorithms.h>
 
+#include <thrust/iterator/transform_iterator.h>
 namespace thrust {
 
 // ---- device

@@ -1,0 +1,66 @@
+// thrust::replace / replace_if / replace_copy / replace_copy_if (thrust/replace.h).
+#pragma once
+#include <algorithm>
+#include <thrust/count.h>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/index_algorithms.h>
+
+namespace thrust {
+namespace detail {
+// out[i] = pred(stencil[i]) ? value : in[i]
+template <class In, class S, class Out, class Pred, class T> struct replace_body {
+  In in; S stencil; Out out; Pred pred; T value;
+  THRUST_CDNA4_HD void operator()(std::int64_t i) {
+    if (pred(stencil[i])) out[i] = value;
+    else out[i] = in[i];
+  }
+};
+}  // namespace detail
+template <class D, class In, class S, class Out, class Pred, class T>
+Out replace_copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, S stencil, Out result, Pred pred, const T& value) {
+  const std::int64_t n = (std::int64_t)(last - first);
+  system::cdna4::detail::for_each_index(
+      exec.derived(), n,
+      detail::replace_body<typename detail::unwrap_iterator<In>::type, typename detail::unwrap_iterator<S>::type,
+                           typename detail::unwrap_iterator<Out>::type, Pred, T>{detail::unwrap(first), detail::unwrap(stencil), detail::unwrap(result), pred, value},
+      "replace: failed to synchronize");
+  return result + n;
+}
+template <class In, class S, class Out, class Pred, class T>
+Out replace_copy_if(const system::cpp::detail::par_t&, In first, In last, S stencil, Out result, Pred pred, const T& value) {
+  for (; first != last; ++first, ++stencil, ++result) {
+    if (pred(*stencil)) *result = value;
+    else *result = *first;
+  }
+  return result;
+}
+template <class Policy, class In, class Out, class Pred, class T, detail::enable_if_policy<Policy> = 0>
+Out replace_copy_if(const Policy& exec, In first, In last, Out result, Pred pred, const T& value) {
+  return replace_copy_if(exec, first, last, first, result, pred, value);
+}
+template <class Policy, class In, class Out, class T, detail::enable_if_policy<Policy> = 0>
+Out replace_copy(const Policy& exec, In first, In last, Out result, const T& old_value, const T& new_value) {
+  return replace_copy_if(exec, first, last, first, result, detail::equals_value<T>{old_value}, new_value);
+}
+template <class Policy, class It, class Pred, class T, detail::enable_if_policy<Policy> = 0>
+void replace_if(const Policy& exec, It first, It last, Pred pred, const T& value) { replace_copy_if(exec, first, last, first, first, pred, value); }
+template <class Policy, class It, class S, class Pred, class T, detail::enable_if_policy<Policy> = 0>
+void replace_if(const Policy& exec, It first, It last, S stencil, Pred pred, const T& value) { replace_copy_if(exec, first, last, stencil, first, pred, value); }
+template <class Policy, class It, class T, detail::enable_if_policy<Policy> = 0>
+void replace(const Policy& exec, It first, It last, const T& old_value, const T& new_value) {
+  replace_copy_if(exec, first, last, first, first, detail::equals_value<T>{old_value}, new_value);
+}
+
+#define THRUST_CDNA4_REPLACE(SYS, COND)                                                                                       \
+  template <class It, class T, COND<It> = 0> void replace(It f, It l, const T& a, const T& b) { replace(SYS, f, l, a, b); }    \
+  template <class It, class P, class T, COND<It> = 0> void replace_if(It f, It l, P p, const T& v) { replace_if(SYS, f, l, p, v); } \
+  template <class It, class S, class P, class T, COND<It> = 0, class = typename std::iterator_traits<S>::iterator_category>    \
+  void replace_if(It f, It l, S s, P p, const T& v) { replace_if(SYS, f, l, s, p, v); }                                        \
+  template <class In, class Out, class T, COND<In> = 0> Out replace_copy(In f, In l, Out o, const T& a, const T& b) { return replace_copy(SYS, f, l, o, a, b); } \
+  template <class In, class Out, class P, class T, COND<In> = 0> Out replace_copy_if(In f, In l, Out o, P p, const T& v) { return replace_copy_if(SYS, f, l, o, p, v); } \
+  template <class In, class S, class Out, class P, class T, COND<In> = 0> Out replace_copy_if(In f, In l, S s, Out o, P p, const T& v) { return replace_copy_if(SYS, f, l, s, o, p, v); }
+THRUST_CDNA4_REPLACE(device, detail::enable_if_device)
+THRUST_CDNA4_REPLACE(host, detail::enable_if_host)
+#undef THRUST_CDNA4_REPLACE
+}  // namespace thrust

@@ -1,0 +1,44 @@
+// thrust::reverse / reverse_copy (thrust/reverse.h).
+#pragma once
+#include <algorithm>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/index_algorithms.h>
+
+namespace thrust {
+namespace detail {
+template <class It> struct reverse_body {
+  It p; std::int64_t n;
+  THRUST_CDNA4_HD void operator()(std::int64_t i) {
+    typename std::iterator_traits<It>::value_type a = p[i], b = p[n - 1 - i];
+    p[i] = b;
+    p[n - 1 - i] = a;
+  }
+};
+template <class In, class Out> struct reverse_copy_body {
+  In in; Out out; std::int64_t n;
+  THRUST_CDNA4_HD void operator()(std::int64_t i) { out[i] = in[n - 1 - i]; }
+};
+}  // namespace detail
+template <class D, class It>
+void reverse(const system::cdna4::execution_policy<D>& exec, It first, It last) {
+  const std::int64_t n = (std::int64_t)(last - first);
+  system::cdna4::detail::for_each_index(exec.derived(), n / 2, detail::reverse_body<typename detail::unwrap_iterator<It>::type>{detail::unwrap(first), n},
+                                        "reverse: failed to synchronize");
+}
+template <class It> void reverse(const system::cpp::detail::par_t&, It first, It last) { std::reverse(first, last); }
+template <class D, class In, class Out>
+Out reverse_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out result) {
+  const std::int64_t n = (std::int64_t)(last - first);
+  system::cdna4::detail::for_each_index(
+      exec.derived(), n,
+      detail::reverse_copy_body<typename detail::unwrap_iterator<In>::type, typename detail::unwrap_iterator<Out>::type>{detail::unwrap(first), detail::unwrap(result), n},
+      "reverse_copy: failed to synchronize");
+  return result + n;
+}
+template <class In, class Out> Out reverse_copy(const system::cpp::detail::par_t&, In first, In last, Out result) { return std::reverse_copy(first, last, result); }
+template <class It, detail::enable_if_device<It> = 0> void reverse(It f, It l) { reverse(device, f, l); }
+template <class It, detail::enable_if_host<It> = 0> void reverse(It f, It l) { reverse(host, f, l); }
+template <class In, class Out, detail::enable_if_device<In> = 0> Out reverse_copy(In f, In l, Out o) { return reverse_copy(device, f, l, o); }
+template <class In, class Out, detail::enable_if_host<In> = 0> Out reverse_copy(In f, In l, Out o) { return reverse_copy(host, f, l, o); }
+}  // namespace thrust

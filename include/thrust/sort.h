@@ -2,6 +2,7 @@
 // Device ranges (device_vector iterators, device_ptr, or raw pointers under a device policy)
 // go to the radix-sort kernels; host ranges are sorted on the host.
 #pragma once
+#include <thrust/system/cdna4/detail/index_algorithms.h>
 #include <algorithm>
 #include <numeric>
 #include <vector>
@@ -152,4 +153,43 @@ THRUST_CDNA4_SORT_BY_KEY_DISPATCH(sort_by_key)
 THRUST_CDNA4_SORT_BY_KEY_DISPATCH(stable_sort_by_key)
 #undef THRUST_CDNA4_SORT_BY_KEY_DISPATCH
 
+
+// ---------------------------------------------------------------------------------------
+// is_sorted / is_sorted_until (thrust/sort.h:1160-): the first position whose element is before
+// its predecessor, as a minimum over such positions.
+// ---------------------------------------------------------------------------------------
+namespace detail {
+template <class It, class Compare> struct descent_index {
+  It p; mutable Compare comp; std::int64_t n;
+  THRUST_CDNA4_HD std::int64_t operator()(std::int64_t i) const { return comp(p[i + 1], p[i]) ? i + 1 : n; }
+};
+struct min_position {
+  THRUST_CDNA4_HD std::int64_t operator()(std::int64_t a, std::int64_t b) const { return a < b ? a : b; }
+};
+}  // namespace detail
+template <class D, class It, class Compare>
+It is_sorted_until(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) {
+  const std::int64_t n = (std::int64_t)(last - first);
+  if (n < 2) return last;
+  const std::int64_t at = system::cdna4::detail::reduce_index(
+      exec.derived(), n - 1, detail::descent_index<typename detail::unwrap_iterator<It>::type, Compare>{detail::unwrap(first), comp, n}, n,
+      detail::min_position());
+  return first + at;
+}
+template <class It, class Compare>
+It is_sorted_until(const system::cpp::detail::par_t&, It first, It last, Compare comp) { return std::is_sorted_until(first, last, comp); }
+template <class Policy, class It, detail::enable_if_policy<Policy> = 0>
+It is_sorted_until(const Policy& exec, It first, It last) { return is_sorted_until(exec, first, last, less<>()); }
+template <class Policy, class It, class Compare, detail::enable_if_policy<Policy> = 0>
+bool is_sorted(const Policy& exec, It first, It last, Compare comp) { return is_sorted_until(exec, first, last, comp) == last; }
+template <class Policy, class It, detail::enable_if_policy<Policy> = 0>
+bool is_sorted(const Policy& exec, It first, It last) { return is_sorted_until(exec, first, last, less<>()) == last; }
+template <class It, detail::enable_if_device<It> = 0> It is_sorted_until(It f, It l) { return is_sorted_until(device, f, l); }
+template <class It, detail::enable_if_host<It> = 0> It is_sorted_until(It f, It l) { return is_sorted_until(host, f, l); }
+template <class It, class C, detail::enable_if_device<It> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(device, f, l, c); }
+template <class It, class C, detail::enable_if_host<It> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(host, f, l, c); }
+template <class It, detail::enable_if_device<It> = 0> bool is_sorted(It f, It l) { return is_sorted(device, f, l); }
+template <class It, detail::enable_if_host<It> = 0> bool is_sorted(It f, It l) { return is_sorted(host, f, l); }
+template <class It, class C, detail::enable_if_device<It> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(device, f, l, c); }
+template <class It, class C, detail::enable_if_host<It> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(host, f, l, c); }
 }  // namespace thrust

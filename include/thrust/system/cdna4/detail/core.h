@@ -11,6 +11,7 @@
 //   thrust/detail/temporary_array.h:50-111               (algorithm-scoped temporary storage)
 #pragma once
 
+#include <cassert>
 #include <cstddef>
 #include <utility>
 #include <cstdint>
@@ -24,8 +25,32 @@
 #define THRUST_CDNA4_SYSTEM 1
 // The version of the API surface this layer mirrors (Thrust 2.2.0).
 #define THRUST_VERSION 200200
+// Device system selection, as in thrust/detail/config/device_system.h:20-43: the reference's four
+// ids keep their values, this system is the fifth and the default.  A build that names another
+// device system with -DTHRUST_DEVICE_SYSTEM=... is refused: this tree holds one.
+#define THRUST_DEVICE_SYSTEM_CUDA 1
+#define THRUST_DEVICE_SYSTEM_OMP 2
+#define THRUST_DEVICE_SYSTEM_TBB 3
+#define THRUST_DEVICE_SYSTEM_CPP 4
 #define THRUST_DEVICE_SYSTEM_CDNA4 5
+#ifndef THRUST_DEVICE_SYSTEM
 #define THRUST_DEVICE_SYSTEM THRUST_DEVICE_SYSTEM_CDNA4
+#endif
+#if THRUST_DEVICE_SYSTEM != THRUST_DEVICE_SYSTEM_CDNA4
+#error "this Thrust tree provides the cdna4 device system only: build with -DTHRUST_DEVICE_SYSTEM=THRUST_DEVICE_SYSTEM_CDNA4 (5), or leave THRUST_DEVICE_SYSTEM undefined"
+#endif
+#define __THRUST_DEVICE_SYSTEM_NAMESPACE cdna4
+#define __THRUST_DEVICE_SYSTEM_ROOT thrust/system/__THRUST_DEVICE_SYSTEM_NAMESPACE
+// the host system is the sequential one (THRUST_HOST_SYSTEM_CPP of thrust/detail/config/host_system.h)
+#define THRUST_HOST_SYSTEM_CPP 1
+#define THRUST_HOST_SYSTEM_OMP 2
+#define THRUST_HOST_SYSTEM_TBB 3
+#ifndef THRUST_HOST_SYSTEM
+#define THRUST_HOST_SYSTEM THRUST_HOST_SYSTEM_CPP
+#endif
+#if THRUST_HOST_SYSTEM != THRUST_HOST_SYSTEM_CPP
+#error "this Thrust tree provides the sequential (CPP) host system only"
+#endif
 
 namespace thrust {
 
@@ -65,6 +90,13 @@ inline const error_category& cdna4_category() {
   return cat;
 }
 
+namespace detail {
+// The root of every execution policy (thrust/detail/execution_policy.h): the public entry points
+// that dispatch to a system's implementation take it, so that an overload for a nearer base — the
+// system's own, or a user's for a policy type of their own — is the better match.
+template <class Derived> struct execution_policy_base {};
+}  // namespace detail
+
 namespace system {
 namespace cdna4 {
 
@@ -74,7 +106,7 @@ namespace cdna4 {
 struct tag {};
 
 template <class Derived>
-struct execution_policy {
+struct execution_policy : thrust::detail::execution_policy_base<Derived> {
   typedef tag tag_type;
   operator tag() const { return tag(); }
   const Derived& derived() const { return static_cast<const Derived&>(*this); }
@@ -119,6 +151,10 @@ struct execute_with_allocator : execution_policy<execute_with_allocator<Alloc>> 
 template <class Alloc> inline void* stream_of(const execute_with_allocator<Alloc>& p) { return p.stream_; }
 template <class Alloc> inline bool must_sync(const execute_with_allocator<Alloc>& p) { return p.sync_; }
 
+// a policy of the user's own, derived from execution_policy<Derived> (thrust::device_execution_policy):
+// the default stream, synchronous
+template <class Derived> inline void* stream_of(const execution_policy<Derived>&) { return nullptr; }
+template <class Derived> inline bool must_sync(const execution_policy<Derived>&) { return true; }
 inline void* stream_of(const par_t&) { return nullptr; }
 inline void* stream_of(const par_nosync_t&) { return nullptr; }
 inline void* stream_of(const execute_on_stream& p) { return p.stream_; }
@@ -258,5 +294,8 @@ struct par_t {};
 
 static const system::cdna4::detail::par_t device;
 static const system::cpp::detail::par_t host;
+// the system tags of device and host iterators (thrust/iterator/detail/device_system_tag.h:22-28)
+typedef system::cdna4::tag device_system_tag;
+typedef system::cpp::tag host_system_tag;
 
 }  // namespace thrust

@@ -44,7 +44,7 @@ template <class Out, class T> struct sequence_body {
   __device__ void operator()(std::int64_t i) { out[i] = (T)(init + (T)i * step); }
 };
 template <class In, class F, class T> struct load_transform {
-  In in; F f;
+  In in; mutable F f;
   __device__ T operator()(std::int64_t i) const { return (T)f(in[i]); }
 };
 #endif
@@ -107,7 +107,7 @@ template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
   typedef typename value_of_it<In>::type item;
   static constexpr bool rejects = false;
   static constexpr int rows = sizeof(item) <= 4 ? 64 : sizeof(item) == 8 ? 32 : generic::select_rows(sizeof(item));  // 256 KiB tiles: see select_rows_of
-  In in; Out out; Pred pred;
+  In in; Out out; mutable Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     const item x = in[i];
     keep = (bool)pred(x) != NEGATE;
@@ -119,7 +119,7 @@ template <class In, class Out, class Pred, bool NEGATE> struct keep_if_op {
 template <class In, class S, class Out, class Pred, bool NEGATE> struct keep_if_stencil_op {
   typedef typename value_of_it<In>::type item;
   static constexpr bool rejects = false;
-  In in; S stencil; Out out; Pred pred;
+  In in; S stencil; Out out; mutable Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     keep = (bool)pred(stencil[i]) != NEGATE;
     return in[i];
@@ -130,7 +130,7 @@ template <class In, class S, class Out, class Pred, bool NEGATE> struct keep_if_
 template <class In, class S, class OutT, class OutF, class Pred> struct partition_op {
   typedef typename value_of_it<In>::type item;
   static constexpr bool rejects = true;
-  In in; S stencil; OutT out_true; OutF out_false; Pred pred;
+  In in; S stencil; OutT out_true; OutF out_false; mutable Pred pred;
   __device__ item load(std::int64_t i, bool& keep) const {
     keep = (bool)pred(stencil[i]);
     return in[i];
@@ -142,7 +142,7 @@ template <class In, class S, class OutT, class OutF, class Pred> struct partitio
 template <class KIn, class KOut, class Eq> struct run_head_op {
   typedef typename value_of_it<KIn>::type item;
   static constexpr bool rejects = false;
-  KIn keys; KOut out; Eq eq;
+  KIn keys; KOut out; mutable Eq eq;
   __device__ item load(std::int64_t i, bool& keep) const {
     const item cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
     keep = (i == 0) | !(bool)eq(prev, cur);
@@ -156,7 +156,7 @@ template <class KIn, class VIn, class KOut, class VOut, class Eq> struct run_hea
   struct item { K key; V value; };
   static constexpr bool rejects = false;
   static constexpr int rows = sizeof(item) == 8 ? 32 : generic::select_rows(sizeof(item));  // 256-byte tiles per thread: see select_rows_of
-  KIn keys; VIn values; KOut kout; VOut vout; Eq eq;
+  KIn keys; VIn values; KOut kout; VOut vout; mutable Eq eq;
   __device__ item load(std::int64_t i, bool& keep) const {
     const K cur = keys[i], prev = keys[i > 0 ? i - 1 : 0];
     keep = (i == 0) | !(bool)eq(prev, cur);

@@ -1,0 +1,27 @@
+// thrust::tabulate (thrust/tabulate.h): first[i] = f(i).
+#pragma once
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/system/cdna4/detail/index_algorithms.h>
+
+namespace thrust {
+namespace detail {
+template <class Out, class F> struct tabulate_body {
+  Out out; F f;
+  THRUST_CDNA4_HD void operator()(std::int64_t i) { out[i] = f((typename std::iterator_traits<Out>::difference_type)i); }
+};
+}  // namespace detail
+template <class D, class It, class F>
+void tabulate(const system::cdna4::execution_policy<D>& exec, It first, It last, F f) {
+  typedef typename detail::unwrap_iterator<It>::type Out;
+  system::cdna4::detail::for_each_index(exec.derived(), (std::int64_t)(last - first),
+                                        detail::tabulate_body<Out, F>{detail::unwrap(first), f}, "tabulate: failed to synchronize");
+}
+template <class It, class F>
+void tabulate(const system::cpp::detail::par_t&, It first, It last, F f) {
+  typename std::iterator_traits<It>::difference_type i = 0;
+  for (; first != last; ++first, ++i) *first = f(i);
+}
+template <class It, class F, detail::enable_if_device<It> = 0> void tabulate(It f, It l, F fn) { tabulate(device, f, l, fn); }
+template <class It, class F, detail::enable_if_host<It> = 0> void tabulate(It f, It l, F fn) { tabulate(host, f, l, fn); }
+}  // namespace thrust

@@ -4,6 +4,7 @@
 #include <thrust/execution_policy.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
+#include <thrust/reduce.h>
 namespace thrust {
 template <class D, class It, class F, class T, class Op>
 T transform_reduce(const system::cdna4::execution_policy<D>& exec, It first, It last, F f, T init, Op op) {

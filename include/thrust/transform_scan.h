@@ -1,0 +1,25 @@
+// thrust::transform_inclusive_scan / transform_exclusive_scan (thrust/transform_scan.h): a scan
+// of unary_op(x) read through a transform iterator, so nothing is materialised
+// (thrust/system/cuda/detail/transform_scan.h does the same).
+#pragma once
+#include <thrust/iterator/transform_iterator.h>
+#include <thrust/scan.h>
+
+namespace thrust {
+template <class Policy, class In, class Out, class UnaryOp, class BinaryOp, detail::enable_if_policy<Policy> = 0>
+Out transform_inclusive_scan(const Policy& exec, In first, In last, Out result, UnaryOp unary_op, BinaryOp binary_op) {
+  return inclusive_scan(exec, make_transform_iterator(first, unary_op), make_transform_iterator(last, unary_op), result, binary_op);
+}
+template <class Policy, class In, class Out, class UnaryOp, class T, class BinaryOp, detail::enable_if_policy<Policy> = 0>
+Out transform_exclusive_scan(const Policy& exec, In first, In last, Out result, UnaryOp unary_op, T init, BinaryOp binary_op) {
+  return exclusive_scan(exec, make_transform_iterator(first, unary_op), make_transform_iterator(last, unary_op), result, init, binary_op);
+}
+template <class In, class Out, class U, class B, detail::enable_if_device<In> = 0>
+Out transform_inclusive_scan(In f, In l, Out o, U u, B b) { return transform_inclusive_scan(device, f, l, o, u, b); }
+template <class In, class Out, class U, class B, detail::enable_if_host<In> = 0>
+Out transform_inclusive_scan(In f, In l, Out o, U u, B b) { return transform_inclusive_scan(host, f, l, o, u, b); }
+template <class In, class Out, class U, class T, class B, detail::enable_if_device<In> = 0>
+Out transform_exclusive_scan(In f, In l, Out o, U u, T init, B b) { return transform_exclusive_scan(device, f, l, o, u, init, b); }
+template <class In, class Out, class U, class T, class B, detail::enable_if_host<In> = 0>
+Out transform_exclusive_scan(In f, In l, Out o, U u, T init, B b) { return transform_exclusive_scan(host, f, l, o, u, init, b); }
+}  // namespace thrust

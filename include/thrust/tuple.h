@@ -6,7 +6,7 @@
 #include <cstddef>
 #include <type_traits>
 #include <utility>
-#include <thrust/functional.h>
+#include <thrust/detail/hd.h>
 
 namespace thrust {
 template <class... Ts> struct tuple;

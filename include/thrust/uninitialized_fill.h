@@ -1,0 +1,21 @@
+// thrust::uninitialized_fill / uninitialized_fill_n (thrust/uninitialized_fill.h).  Device
+// ranges hold trivially copyable elements, for which construction is assignment
+// (thrust/system/detail/generic/uninitialized_fill.inl takes the same shortcut).
+#pragma once
+#include <memory>
+#include <thrust/fill.h>
+namespace thrust {
+template <class D, class It, class T>
+void uninitialized_fill(const system::cdna4::execution_policy<D>& exec, It first, It last, const T& x) { fill(exec, first, last, x); }
+template <class It, class T>
+void uninitialized_fill(const system::cpp::detail::par_t&, It first, It last, const T& x) { std::uninitialized_fill(first, last, x); }
+template <class Policy, class It, class Size, class T, detail::enable_if_policy<Policy> = 0>
+It uninitialized_fill_n(const Policy& exec, It first, Size n, const T& x) {
+  uninitialized_fill(exec, first, first + n, x);
+  return first + n;
+}
+template <class It, class T, detail::enable_if_device<It> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(device, f, l, x); }
+template <class It, class T, detail::enable_if_host<It> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(host, f, l, x); }
+template <class It, class Size, class T, detail::enable_if_device<It> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(device, f, n, x); }
+template <class It, class Size, class T, detail::enable_if_host<It> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(host, f, n, x); }
+}  // namespace thrust

@@ -124,7 +124,8 @@ int thrust_cdna4_scan_static(int dtype, int op, int exclusive, const void* in, v
  * exclusive_scan_by_key_n and cub::DispatchScanByKey
  * (thrust/system/cuda/detail/scan_by_key.h:69-282).  The exclusive form restarts from
  * `*init` at every segment head (sequential/scan_by_key.h:95-140).  `values == out` is
- * allowed.
+ * allowed.  n must be < 2^32 (32-bit head counts; the reference switches to 64-bit offsets there,
+ * thrust/system/cuda/detail/dispatch.h:29-78 — the template layer's kernel templates take over).
  */
 int thrust_cdna4_scan_by_key(void* temp, size_t* temp_bytes, int key_dtype, int value_dtype,
                              int op, int exclusive, const void* keys, const void* values,
@@ -136,7 +137,8 @@ int thrust_cdna4_scan_by_key(void* temp, size_t* temp_bytes, int key_dtype, int 
  * For each maximal run of equal consecutive keys writes the run's first key to keys_out
  * and the left-to-right reduction of its values to values_out; writes the number of runs
  * (int64) to the DEVICE location `num_runs_out`, which the caller reads back after
- * synchronising (reduce_by_key.h:1049-1052).  Outputs must not overlap inputs.
+ * synchronising (reduce_by_key.h:1049-1052).  Outputs must not overlap inputs.  n must be < 2^32
+ * (32-bit run positions; beyond, the template layer's kernel templates take over).
  */
 int thrust_cdna4_reduce_by_key(void* temp, size_t* temp_bytes, int key_dtype, int value_dtype,
                                int op, const void* keys_in, const void* values_in,
@@ -158,8 +160,9 @@ int thrust_cdna4_histogram_even(void* temp, size_t* temp_bytes, int sample_dtype
 /*
  * Temporary-storage allocator.  Replaces cuda_cub::malloc / cuda_cub::free
  * (thrust/system/cuda/detail/malloc_and_free.h:53-116), which call cudaMalloc / cudaFree on
- * every algorithm invocation.  Blocks are cached per device in power-of-two size classes
- * and handed back without a driver call; a block freed on one stream is reused on another
+ * every algorithm invocation.  Blocks are cached per device in size classes (powers of two up
+ * to 1 MiB, eight per octave above: at most 12.5 % more than asked for) and handed back without a
+ * driver call; a block freed on one stream is reused on another
  * only after an event recorded at the free has completed.
  */
 int thrust_cdna4_malloc(void** ptr, size_t bytes, void* stream);

@@ -82,6 +82,25 @@ def test_scan_by_key_i32_full_size_exact():
     assert torch.equal(got, c - before_head[keys.long()])
 
 
+def test_by_key_beyond_2p31_elements():
+    # more elements than a signed 32-bit offset holds (the reference dispatches to 64-bit offsets
+    # there, thrust/system/cuda/detail/dispatch.h:29-78); runs of 512 ones have closed forms
+    n = (1 << 31) + 777
+    keys = (torch.arange(n, dtype=torch.int64, device="cuda") >> 9).to(torch.int32)
+    vals = torch.ones(n, dtype=torch.int32, device="cuda")
+    gk, gv = thrust_amd.reduce_by_key(keys, vals)
+    r = (n + 511) // 512
+    assert gk.numel() == r
+    assert torch.equal(gk, torch.arange(r, dtype=torch.int32, device="cuda"))
+    assert bool((gv[:-1] == 512).all()) and int(gv[-1].item()) == n - 512 * (r - 1)
+    del gk, gv
+    out = thrust_amd.inclusive_scan_by_key(keys, vals)
+    assert int(out[-1].item()) == n - 512 * (r - 1) and int(out[(1 << 31) - 1].item()) == 512
+    pos = torch.arange(n - (1 << 20), n, dtype=torch.int64, device="cuda")
+    assert torch.equal(out[-(1 << 20):].long(), (pos & 511) + 1)
+    assert torch.equal(out[:1 << 20].long(), (torch.arange(1 << 20, dtype=torch.int64, device="cuda") & 511) + 1)
+
+
 # ------------------------------------------------------------------ sort_by_key u64 + u32
 def unsigned_order(k):
     """int64 whose signed order is the unsigned order of the 64-bit patterns in k."""

@@ -32,6 +32,32 @@ def test_pool_reuses_blocks_and_trims():
     capi.check(L.thrust_cdna4_free(zero, s), "free")
 
 
+def test_pool_size_classes_round_up_by_an_eighth_at_most_above_1MiB():
+    L = capi.lib()
+    s = vp(torch.cuda.current_stream().cuda_stream)
+    capi.check(L.thrust_cdna4_stream_synchronize(s), "sync")
+    capi.check(L.thrust_cdna4_pool_trim(), "trim")
+    base = L.thrust_cdna4_pool_bytes()
+    want = (1 << 30) + (21 << 20)  # the temporary storage of a 2^28-key sort: 1.02 GiB
+    p = vp()
+    capi.check(L.thrust_cdna4_malloc(ctypes.byref(p), want, s), "malloc")
+    held = L.thrust_cdna4_pool_bytes() - base
+    assert want <= held <= want + want // 8, held
+    capi.check(L.thrust_cdna4_free(p, s), "free")
+    q = vp()
+    capi.check(L.thrust_cdna4_malloc(ctypes.byref(q), want - (10 << 20), s), "malloc")  # same class: 1 GiB < x <= 1.125 GiB
+    assert q.value == p.value
+    capi.check(L.thrust_cdna4_free(q, s), "free")
+    # below 1 MiB classes are powers of two
+    small = vp()
+    capi.check(L.thrust_cdna4_malloc(ctypes.byref(small), 3000, s), "malloc")
+    assert L.thrust_cdna4_pool_bytes() - base - held == 4096
+    capi.check(L.thrust_cdna4_free(small, s), "free")
+    capi.check(L.thrust_cdna4_stream_synchronize(s), "sync")
+    capi.check(L.thrust_cdna4_pool_trim(), "trim")
+    assert L.thrust_cdna4_pool_bytes() == base
+
+
 def test_direct_allocation_copy_and_fill_roundtrip():
     L = capi.lib()
     n = 100_003

@@ -12,12 +12,15 @@ TCD_DECL(2)
 TCD_DECL(4)
 TCD_DECL(8)
 
+// head counts and run positions are 32-bit unsigned: n (hence the number of runs) must fit them
+static const int64_t kByKeyMaxN = (int64_t(1) << 32) - 1;
+
 static inline int is_float_dtype(int dt) { return dt == THRUST_CDNA4_F32 || dt == THRUST_CDNA4_F64; }
 
 extern "C" int thrust_cdna4_scan_by_key(void* temp, size_t* temp_bytes, int key_dtype, int value_dtype,
                                         int op, int exclusive, const void* keys, const void* values,
                                         void* out, int64_t n, const void* init, void* stream) {
-  if (!temp_bytes || n < 0 || n > INT32_MAX || (n > 0 && temp && (!keys || !values || !out)))
+  if (!temp_bytes || n < 0 || n > kByKeyMaxN || (n > 0 && temp && (!keys || !values || !out)))
     return hipErrorInvalidValue;
   const int fk = is_float_dtype(key_dtype);
   switch (tcd::dtype_size(key_dtype)) {
@@ -33,7 +36,7 @@ extern "C" int thrust_cdna4_reduce_by_key(void* temp, size_t* temp_bytes, int ke
                                           int op, const void* keys_in, const void* values_in,
                                           void* keys_out, void* values_out, int64_t* num_runs_out,
                                           int64_t n, void* stream) {
-  if (!temp_bytes || n < 0 || n > INT32_MAX ||
+  if (!temp_bytes || n < 0 || n > kByKeyMaxN ||
       (temp && (!num_runs_out || (n > 0 && (!keys_in || !values_in || !keys_out || !values_out)))))
     return hipErrorInvalidValue;
   const int fk = is_float_dtype(key_dtype);
