@@ -308,7 +308,22 @@ def main():
         if r.returncode == 0:
             extras.update(json.loads(r.stdout.strip().splitlines()[-1]))
 
+    def extra_api():
+        # what a caller of thrust::sort / thrust::inclusive_scan sees: header dispatch, pool,
+        # launches and synchronisation inside the timed call, the first call of a process on its
+        # own, and the user-operator engine (tests/cpp/bench_api.cpp)
+        import subprocess
+        exe = os.path.join(ROOT, "tests", "cpp", "build", "bench_api")
+        if not os.path.exists(exe):
+            return
+        r = subprocess.run([exe, str(args.log2n)], capture_output=True, text=True, timeout=600)
+        if r.returncode == 0:
+            extras.update(json.loads(r.stdout.strip().splitlines()[-1]))
+        else:
+            extras["api_error"] = r.stderr[-300:]
+
     all_extras = {
+        "api": extra_api,
         "generic": extra_generic,
         "select": extra_select,
         "merge_sort": extra_merge_sort,
@@ -350,6 +365,34 @@ def main():
             "sample": f"2^{args.log2n} uniform uint32 keys (the whole GPU workload), best of 3; oracle "
                       f"restatement of the reference OpenMP sort (per-thread radix sort + pairwise merges)",
         }
+
+        # the other algorithms of the path: the scalar oracle (the reference's sequential loops
+        # restated, 1 core) on a 2^26-element sample of the workloads of the extras above
+        if not args.no_extras and not args.only:
+            m = min(n, 1 << 26)
+            rng = np.random.default_rng(7)
+
+            def best_of(f, reps=3):
+                best = None
+                for _ in range(reps):
+                    t0 = time.perf_counter()
+                    f()
+                    dt = time.perf_counter() - t0
+                    best = dt if best is None else min(best, dt)
+                return best
+
+            xi = rng.integers(0, 16, m, dtype=np.int32)
+            keys8 = np.cumsum(rng.random(m) < 1.0 / 8, dtype=np.int32)
+            vals = rng.integers(-1000, 1001, m, dtype=np.int32)
+            zipf_w = 1.0 / np.arange(1, 4097, dtype=np.float64) ** 1.1
+            samples = np.searchsorted(np.cumsum(zipf_w / zipf_w.sum()), rng.random(m)).clip(max=4095).astype(np.float32)
+            extras["cpu_baselines"] = {
+                "kind": "port", "cores": 1, "sample": "2^%d elements, best of 3" % int(np.log2(m)),
+                "inclusive_scan_i32_gelem_per_s": round(m / best_of(lambda: oracle.scan(xi)) / 1e9, 4),
+                "reduce_by_key_i32_mean8_gelem_per_s": round(m / best_of(lambda: oracle.reduce_by_key(keys8, vals)) / 1e9, 4),
+                "inclusive_scan_by_key_i32_mean8_gelem_per_s": round(m / best_of(lambda: oracle.scan_by_key(keys8, vals)) / 1e9, 4),
+                "histogram_f32_zipf_256bins_gsamples_per_s": round(m / best_of(lambda: oracle.histogram_even(samples, 256, 0.0, 4096.0)) / 1e9, 4),
+            }
 
     out = {
         "metric": "thrust::sort throughput, 2^%d uint32 keys" % args.log2n,

@@ -57,13 +57,10 @@ OutIt copy(InIt first, InIt last, OutIt out) {
 namespace thrust {
 template <class D, class In, class Out, class Pred>
 Out copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Pred pred) {
-  typedef typename detail::value_of<In>::type V;
   return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), detail::unwrap(first), detail::unwrap(out), (std::int64_t)(last - first), pred);
 }
 template <class D, class In, class St, class Out, class Pred>
 Out copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, St stencil, Out out, Pred pred) {
-  typedef typename detail::value_of<In>::type V;
-  typedef typename detail::value_of<St>::type S;
   return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), detail::unwrap(first), detail::unwrap(stencil),
                                                             detail::unwrap(out), (std::int64_t)(last - first), pred);
 }

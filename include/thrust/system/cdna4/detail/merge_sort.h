@@ -52,18 +52,14 @@ constexpr int items_per_thread() {
 
 struct no_value {};
 
-// Pins a value that was just read from LDS into registers HERE.  A workgroup barrier does not
-// wait for LDS reads that are still in flight, and the compiler only waits for a read where its
-// result is first used; in a loop that reads LDS into registers, passes a barrier and writes
-// those registers back to LDS, a read could otherwise still be pending when another wave
-// overwrites its source after the barrier.
-template <class T>
-__device__ inline void settle(const T& x) {
-  constexpr int NW = (int)((sizeof(T) + 3) / 4);
-  std::uint32_t w[NW] = {};
-  __builtin_memcpy(w, &x, sizeof(T));
-#pragma unroll
-  for (int i = 0; i < NW; i++) asm volatile("" ::"v"(w[i]));
+// Items per thread of the tile sort: IPT, or IPT / 2 when two copies of keys and 16-bit positions
+// and one of the values do not fit the 64 KiB of static LDS at IPT.  (Half a merge tile is the
+// least the merge passes can start from: an output tile must lie within one pair of runs.)
+template <class K, class V, int IPT>
+constexpr int tile_sort_items() {
+  constexpr std::size_t per_item = 2 * sizeof(K) + 4 + (std::is_same<V, no_value>::value ? 0 : sizeof(V));
+  static_assert(per_item * kBlock * (IPT / 2) <= 65536, "cdna4 merge sort: half a tile does not fit LDS twice");
+  return per_item * kBlock * IPT <= 65536 ? IPT : IPT / 2;
 }
 
 // A thread's kIpt consecutive items as one block: when the block is a whole number of 16-byte
@@ -92,13 +88,16 @@ __device__ inline int merge_path(const K* a, int na, const K* b, int nb, int dia
 // ---------------------------------------------------------------------------------------
 // 1. Tile sort
 // ---------------------------------------------------------------------------------------
+// The rounds of the in-tile merge alternate between two LDS buffers: round r writes buffer r & 1
+// and reads only that buffer, so a round never overwrites what the round before it may still be
+// reading, and one workgroup barrier per round (between the writes and the reads) is enough.
 template <int IPT, class K, class V, class Compare>
 __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, std::int64_t n, Compare comp) {
   constexpr int kIpt = IPT, kTile = kBlock * IPT;
   static_assert((kIpt & (kIpt - 1)) == 0 && kTile <= 65536, "run widths double from kIpt; 16-bit positions in a tile");
   constexpr bool kHasValues = !std::is_same<V, no_value>::value;
-  __shared__ K s_keys[kTile];
-  __shared__ std::uint16_t s_idx[kTile];
+  __shared__ K s_keys2[2][kTile];
+  __shared__ std::uint16_t s_idx2[2][kTile];
   __shared__ typename std::conditional<kHasValues, V, char>::type s_vals[kHasValues ? kTile : 1];
 
   const int tid = threadIdx.x;
@@ -159,8 +158,10 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
   auto rounds = [&](auto whole_tag) {
     constexpr bool kWhole = decltype(whole_tag)::value;
     constexpr bool kIdx = kHasValues || !kWhole;
-    for (int width = kIpt; width < kTile; width *= 2) {
-      __syncthreads();
+    int round = 0;
+    for (int width = kIpt; width < kTile; width *= 2, round ^= 1) {
+      K* const s_keys = s_keys2[round];
+      std::uint16_t* const s_idx = s_idx2[round];
 #pragma unroll
       for (int j = 0; j < kIpt; j++) {
         s_keys[tid * kIpt + j] = k[j];
@@ -207,14 +208,6 @@ __global__ __launch_bounds__(kBlock) void block_sort_kernel(K* keys, V* values, 
           xb = take_a ? xb : xn;
         }
       }
-#pragma unroll
-      for (int j = 0; j < kIpt; j++) {  // all LDS reads of this round have landed before the next barrier
-        settle(k[j]);
-        if constexpr (kIdx) settle(idx[j]);
-      }
-      settle(ka);
-      settle(kb);
-      if constexpr (kIdx) { settle(xa); settle(xb); }
     }
   };
   if (whole) rounds(std::true_type{});
@@ -404,15 +397,21 @@ void stable_sort(void* stream_, K* keys, V* values, std::int64_t n, Compare comp
   static_assert(std::is_trivially_copyable<V>::value, "cdna4 merge sort: values must be trivially copyable");
   constexpr int IPT = items_per_thread<K, V>();
   constexpr int kTile = kBlock * IPT;
-  static_assert((sizeof(K) + sizeof(V) + 2) * kTile <= 65536, "cdna4 merge sort: a tile of keys and values must fit the 64 KiB of static LDS");
   constexpr bool kHasValues = !std::is_same<V, no_value>::value;
+  static_assert((sizeof(K) + (kHasValues ? sizeof(V) : 0) + 2) * kTile <= 65536,
+                "cdna4 merge sort: a tile of keys and values must fit the 64 KiB of static LDS");
+  // the tile sort keeps two copies of keys and positions in LDS: its tiles are those of the merge
+  // passes, or half of them where that is what fits
+  constexpr int SORT_IPT = tile_sort_items<K, V, IPT>();
+  constexpr int kSortTile = kBlock * SORT_IPT;
   if (n <= 1) return;
   hipStream_t s = static_cast<hipStream_t>(stream_);
   const std::int64_t ntiles = (n + kTile - 1) / kTile;
+  const std::int64_t nsorted = (n + kSortTile - 1) / kSortTile;
 
-  hipLaunchKernelGGL((block_sort_kernel<IPT, K, V, Compare>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, keys, values, n, comp);
+  hipLaunchKernelGGL((block_sort_kernel<SORT_IPT, K, V, Compare>), dim3((unsigned)nsorted), dim3(kBlock), 0, s, keys, values, n, comp);
   throw_on_error((int)hipGetLastError(), "merge sort: tile sort launch");
-  if (ntiles == 1) return;
+  if (nsorted == 1) return;
 
   const std::size_t kbytes = align256((std::size_t)n * sizeof(K));
   const std::size_t vbytes = kHasValues ? align256((std::size_t)n * sizeof(V)) : 0;
@@ -424,7 +423,7 @@ void stable_sort(void* stream_, K* keys, V* values, std::int64_t n, Compare comp
   std::int64_t* splits = reinterpret_cast<std::int64_t*>(t + kbytes + vbytes);
 
   int cur = 0;
-  for (std::int64_t width = kTile; width < n; width *= 2) {
+  for (std::int64_t width = kSortTile; width < n; width *= 2) {
     hipLaunchKernelGGL((merge_partition_kernel<IPT, K, Compare>), dim3((unsigned)((ntiles + 255) / 256)), dim3(256), 0, s,
                        kbuf[cur], n, width, ntiles, splits, comp);
     hipLaunchKernelGGL((merge_kernel<IPT, K, V, Compare>), dim3((unsigned)ntiles), dim3(kBlock), 0, s, kbuf[cur], vbuf[cur],

@@ -1,0 +1,330 @@
+// generate / tabulate / gather / scatter / replace / reverse / find / mismatch / equal / logical /
+// inner_product / extrema / transform_scan / swap_ranges / is_sorted / random / placeholders on
+// device ranges against the same call on host ranges, over the reference's size ladder, plus the
+// known answers of the reference's tests (testing/gather.cu:20-47, scatter.cu:19-45,
+// replace.cu:23-46, reverse.cu:8-33, find.cu:33-62, mismatch.cu:6-33, equal.cu:8-40,
+// logical.cu:9-54, inner_product.cu:10-24, min_element.cu:7-30, max_element.cu:7-30,
+// minmax_element.cu:7-30, transform_scan.cu:60-120, is_sorted.cu:7-30, tabulate.cu:48-75).
+#include <thrust/equal.h>
+#include <thrust/extrema.h>
+#include <thrust/find.h>
+#include <thrust/functional.h>
+#include <thrust/gather.h>
+#include <thrust/generate.h>
+#include <thrust/inner_product.h>
+#include <thrust/iterator/counting_iterator.h>
+#include <thrust/logical.h>
+#include <thrust/mismatch.h>
+#include <thrust/random.h>
+#include <thrust/replace.h>
+#include <thrust/reverse.h>
+#include <thrust/scatter.h>
+#include <thrust/sequence.h>
+#include <thrust/sort.h>
+#include <thrust/swap.h>
+#include <thrust/tabulate.h>
+#include <thrust/transform_scan.h>
+
+#include <random>
+
+#include "testing.h"
+
+template <class T>
+thrust::host_vector<T> hv(std::initializer_list<double> v) {
+  thrust::host_vector<T> r;
+  for (double x : v) r.push_back((T)x);
+  return r;
+}
+template <class T>
+thrust::host_vector<T> small_values(std::size_t n, std::uint64_t seed, int range) {
+  thrust::host_vector<T> v(n);
+  std::uint64_t s = seed + n;
+  for (auto& x : v) x = (T)(unittest::splitmix64(s) % (std::uint64_t)range);
+  return v;
+}
+
+// ------------------------------------------------------------------ gather / scatter
+void TestGatherScatterSimple() {
+  thrust::device_vector<int> map = hv<int>({6, 2, 1, 7, 2}), src = hv<int>({0, 1, 2, 3, 4, 5, 6, 7}), dst(5, 0);
+  thrust::gather(map.begin(), map.end(), src.begin(), dst.begin());
+  ASSERT_EQUAL(dst, hv<int>({6, 2, 1, 7, 2}));
+  thrust::device_vector<int> smap = hv<int>({6, 3, 1, 7, 2}), ssrc = hv<int>({0, 1, 2, 3, 4}), sdst(8, 0);
+  thrust::scatter(ssrc.begin(), ssrc.end(), smap.begin(), sdst.begin());
+  ASSERT_EQUAL(sdst, hv<int>({0, 2, 4, 1, 0, 0, 0, 3}));
+  thrust::device_vector<int> flags = hv<int>({0, 1, 0, 1, 0}), gdst(5, 9);
+  thrust::gather_if(map.begin(), map.end(), flags.begin(), src.begin(), gdst.begin());
+  ASSERT_EQUAL(gdst, hv<int>({9, 2, 9, 7, 9}));
+  thrust::device_vector<int> sdst2(8, 0);
+  thrust::scatter_if(ssrc.begin(), ssrc.end(), smap.begin(), flags.begin(), sdst2.begin());
+  ASSERT_EQUAL(sdst2, hv<int>({0, 0, 0, 1, 0, 0, 0, 3}));
+}
+DECLARE_UNITTEST(TestGatherScatterSimple);
+
+template <class T>
+void TestGatherScatterLadder() {
+  for (std::size_t n : unittest::sizes()) {
+    const std::size_t src_n = n ? 2 * n + 3 : 1;
+    thrust::host_vector<T> h_src = unittest::random_integers<T>(src_n);
+    thrust::host_vector<unsigned> h_map(n);
+    std::uint64_t s = 3 + n;
+    for (auto& m : h_map) m = (unsigned)(unittest::splitmix64(s) % src_n);
+    thrust::device_vector<T> d_src = h_src, d_out(n);
+    thrust::device_vector<unsigned> d_map = h_map;
+    thrust::host_vector<T> h_out(n);
+    thrust::gather(h_map.begin(), h_map.end(), h_src.begin(), h_out.begin());
+    thrust::gather(d_map.begin(), d_map.end(), d_src.begin(), d_out.begin());
+    ASSERT_EQUAL(d_out, h_out);
+    // scatter through a permutation (a map with repeated targets would race, as in the reference)
+    thrust::host_vector<unsigned> h_perm(n);
+    for (std::size_t i = 0; i < n; i++) h_perm[i] = (unsigned)((i * 7919u + 13u) % (n ? n : 1));
+    if (n % 7919 == 0 && n) continue;  // not a permutation then
+    thrust::device_vector<unsigned> d_perm = h_perm;
+    thrust::host_vector<T> h_in = unittest::random_integers<T>(n, 17), h_sc(n, T(0));
+    thrust::device_vector<T> d_in = h_in, d_sc(n, T(0));
+    thrust::scatter(h_in.begin(), h_in.end(), h_perm.begin(), h_sc.begin());
+    thrust::scatter(d_in.begin(), d_in.end(), d_perm.begin(), d_sc.begin());
+    ASSERT_EQUAL(d_sc, h_sc);
+  }
+}
+DECLARE_TYPED_UNITTEST(TestGatherScatterLadder, int32_t);
+DECLARE_TYPED_UNITTEST(TestGatherScatterLadder, int8_t);
+DECLARE_TYPED_UNITTEST(TestGatherScatterLadder, int64_t);
+
+// ------------------------------------------------------------------ replace / reverse / swap_ranges
+template <class T>
+struct less_than_five {
+  __host__ __device__ bool operator()(const T& x) const { return x < T(5); }
+};
+template <class T>
+void TestReplaceReverseSwapLadder() {
+  ASSERT_EQUAL((thrust::device_vector<T>(hv<T>({1, 2, 1, 3, 2}))).size(), std::size_t(5));
+  {
+    thrust::device_vector<T> d = hv<T>({1, 2, 1, 3, 2});
+    thrust::replace(d.begin(), d.end(), T(1), T(4));
+    thrust::replace(d.begin(), d.end(), T(2), T(5));
+    ASSERT_EQUAL(d, hv<T>({4, 5, 4, 3, 5}));  // testing/replace.cu:23-46
+    thrust::reverse(d.begin(), d.end());
+    ASSERT_EQUAL(d, hv<T>({5, 3, 4, 5, 4}));
+  }
+  for (std::size_t n : unittest::sizes()) {
+    thrust::host_vector<T> h = small_values<T>(n, 1, 10), h2 = small_values<T>(n, 2, 10), ho(n);
+    thrust::device_vector<T> d = h, d2 = h2, dout(n);
+    thrust::replace_copy_if(h.begin(), h.end(), ho.begin(), less_than_five<T>(), T(7));
+    thrust::replace_copy_if(d.begin(), d.end(), dout.begin(), less_than_five<T>(), T(7));
+    ASSERT_EQUAL(dout, ho);
+    thrust::replace_copy(h.begin(), h.end(), ho.begin(), T(3), T(9));
+    thrust::replace_copy(d.begin(), d.end(), dout.begin(), T(3), T(9));
+    ASSERT_EQUAL(dout, ho);
+    thrust::replace_if(h.begin(), h.end(), h2.begin(), less_than_five<T>(), T(0));  // stencil form
+    thrust::replace_if(d.begin(), d.end(), d2.begin(), less_than_five<T>(), T(0));
+    ASSERT_EQUAL(d, h);
+    thrust::reverse_copy(h.begin(), h.end(), ho.begin());
+    thrust::reverse_copy(d.begin(), d.end(), dout.begin());
+    ASSERT_EQUAL(dout, ho);
+    thrust::reverse(h.begin(), h.end());
+    thrust::reverse(d.begin(), d.end());
+    ASSERT_EQUAL(d, h);
+    thrust::swap_ranges(h.begin(), h.end(), h2.begin());
+    thrust::swap_ranges(d.begin(), d.end(), d2.begin());
+    ASSERT_EQUAL(d, h);
+    ASSERT_EQUAL(d2, h2);
+  }
+}
+DECLARE_TYPED_UNITTEST(TestReplaceReverseSwapLadder, int32_t);
+DECLARE_TYPED_UNITTEST(TestReplaceReverseSwapLadder, int16_t);
+DECLARE_TYPED_UNITTEST(TestReplaceReverseSwapLadder, double);
+
+// ------------------------------------------------------------------ find / mismatch / equal / logical
+template <class T>
+struct equal_to_value_pred {
+  T value;
+  __host__ __device__ bool operator()(T v) const { return v == value; }
+};
+void TestFindSimple() {  // testing/find.cu:33-62
+  thrust::device_vector<int> vec = hv<int>({1, 2, 3, 3, 5});
+  ASSERT_EQUAL(thrust::find(vec.begin(), vec.end(), 0) - vec.begin(), 5);
+  ASSERT_EQUAL(thrust::find(vec.begin(), vec.end(), 1) - vec.begin(), 0);
+  ASSERT_EQUAL(thrust::find(vec.begin(), vec.end(), 3) - vec.begin(), 2);
+  ASSERT_EQUAL(thrust::find(vec.begin(), vec.end(), 5) - vec.begin(), 4);
+  ASSERT_EQUAL(thrust::find_if(vec.begin(), vec.end(), equal_to_value_pred<int>{3}) - vec.begin(), 2);
+  ASSERT_EQUAL(thrust::find_if_not(vec.begin(), vec.end(), equal_to_value_pred<int>{1}) - vec.begin(), 1);
+  thrust::device_vector<int> a = hv<int>({1, 2, 3, 4}), b = hv<int>({1, 2, 4, 3});
+  ASSERT_EQUAL(thrust::mismatch(a.begin(), a.end(), b.begin()).first - a.begin(), 2);  // testing/mismatch.cu:6-33
+  b = a;
+  ASSERT_EQUAL(thrust::mismatch(a.begin(), a.end(), b.begin()).first - a.begin(), 4);
+  ASSERT_TRUE(thrust::equal(a.begin(), a.end(), b.begin()));
+  b[3] = 9;
+  ASSERT_TRUE(!thrust::equal(a.begin(), a.end(), b.begin()));
+  ASSERT_TRUE(thrust::equal(a.begin(), a.begin() + 3, b.begin()));
+  thrust::device_vector<int> v3 = hv<int>({1, 1, 0});  // testing/logical.cu:9-54
+  ASSERT_TRUE(thrust::all_of(v3.begin(), v3.begin(), thrust::identity<int>()));
+  ASSERT_TRUE(thrust::all_of(v3.begin(), v3.begin() + 2, thrust::identity<int>()));
+  ASSERT_TRUE(!thrust::all_of(v3.begin(), v3.end(), thrust::identity<int>()));
+  ASSERT_TRUE(thrust::any_of(v3.begin(), v3.end(), thrust::identity<int>()));
+  ASSERT_TRUE(!thrust::any_of(v3.begin() + 2, v3.end(), thrust::identity<int>()));
+  ASSERT_TRUE(thrust::none_of(v3.begin() + 2, v3.end(), thrust::identity<int>()));
+  ASSERT_TRUE(!thrust::none_of(v3.begin(), v3.end(), thrust::identity<int>()));
+}
+DECLARE_UNITTEST(TestFindSimple);
+
+template <class T>
+void TestFindMismatchLadder() {
+  for (std::size_t n : unittest::sizes()) {
+    thrust::host_vector<T> h = small_values<T>(n, 9, 1000);
+    thrust::device_vector<T> d = h;
+    for (T needle : {T(0), T(7), T(999), T(5000)}) {
+      ASSERT_EQUAL(thrust::find(d.begin(), d.end(), needle) - d.begin(), thrust::find(h.begin(), h.end(), needle) - h.begin());
+    }
+    thrust::host_vector<T> h2 = h;
+    if (n > 3) h2[n - 2] = T(h2[n - 2] + 1);
+    thrust::device_vector<T> d2 = h2;
+    ASSERT_EQUAL(thrust::mismatch(d.begin(), d.end(), d2.begin()).first - d.begin(),
+                 thrust::mismatch(h.begin(), h.end(), h2.begin()).first - h.begin());
+    ASSERT_EQUAL(thrust::equal(d.begin(), d.end(), d2.begin()), thrust::equal(h.begin(), h.end(), h2.begin()));
+    thrust::host_vector<T> hs = h;
+    std::sort(hs.begin(), hs.end());
+    thrust::device_vector<T> ds = hs;
+    ASSERT_TRUE(thrust::is_sorted(ds.begin(), ds.end()));
+    ASSERT_EQUAL(thrust::is_sorted(d.begin(), d.end()), thrust::is_sorted(h.begin(), h.end()));
+    ASSERT_EQUAL(thrust::is_sorted_until(d.begin(), d.end()) - d.begin(), thrust::is_sorted_until(h.begin(), h.end()) - h.begin());
+  }
+}
+DECLARE_TYPED_UNITTEST(TestFindMismatchLadder, int32_t);
+DECLARE_TYPED_UNITTEST(TestFindMismatchLadder, int16_t);
+
+// ------------------------------------------------------------------ inner_product / extrema
+void TestInnerProductSimple() {  // testing/inner_product.cu:10-24
+  thrust::device_vector<int> v1 = hv<int>({1, -2, 3}), v2 = hv<int>({-4, 5, 6});
+  ASSERT_EQUAL(thrust::inner_product(v1.begin(), v1.end(), v2.begin(), 3), 7);
+  ASSERT_EQUAL(thrust::inner_product(v1.begin(), v1.end(), v2.begin(), 1, thrust::multiplies<int>(), thrust::plus<int>()), 1 * -3 * 3 * 9);
+}
+DECLARE_UNITTEST(TestInnerProductSimple);
+
+template <class T>
+void TestInnerProductExtremaLadder() {
+  {  // testing/min_element.cu, max_element.cu, minmax_element.cu: the first of equal extrema
+    thrust::device_vector<T> data = hv<T>({3, 5, 1, 2, 5, 1});
+    ASSERT_EQUAL(thrust::min_element(data.begin(), data.end()) - data.begin(), 2);
+    ASSERT_EQUAL(thrust::max_element(data.begin(), data.end()) - data.begin(), 1);
+    ASSERT_EQUAL(thrust::min_element(data.begin(), data.end(), thrust::greater<T>()) - data.begin(), 1);
+    ASSERT_EQUAL(thrust::max_element(data.begin(), data.end(), thrust::greater<T>()) - data.begin(), 2);
+    auto mm = thrust::minmax_element(data.begin(), data.end());
+    ASSERT_EQUAL(mm.first - data.begin(), 2);
+    ASSERT_EQUAL(mm.second - data.begin(), 1);
+    ASSERT_TRUE(thrust::min_element(data.begin(), data.begin()) == data.begin());
+  }
+  for (std::size_t n : unittest::sizes()) {
+    thrust::host_vector<T> h1 = small_values<T>(n, 21, 50), h2 = small_values<T>(n, 22, 50);
+    thrust::device_vector<T> d1 = h1, d2 = h2;
+    ASSERT_EQUAL(thrust::inner_product(d1.begin(), d1.end(), d2.begin(), T(13)), thrust::inner_product(h1.begin(), h1.end(), h2.begin(), T(13)));
+    if (n == 0) continue;
+    ASSERT_EQUAL(thrust::min_element(d1.begin(), d1.end()) - d1.begin(), std::min_element(h1.begin(), h1.end()) - h1.begin());
+    ASSERT_EQUAL(thrust::max_element(d1.begin(), d1.end()) - d1.begin(), std::max_element(h1.begin(), h1.end()) - h1.begin());
+    auto dm = thrust::minmax_element(d1.begin(), d1.end());
+    auto hm = thrust::minmax_element(h1.begin(), h1.end());
+    ASSERT_EQUAL(dm.first - d1.begin(), hm.first - h1.begin());
+    ASSERT_EQUAL(dm.second - d1.begin(), hm.second - h1.begin());
+  }
+}
+DECLARE_TYPED_UNITTEST(TestInnerProductExtremaLadder, int32_t);
+DECLARE_TYPED_UNITTEST(TestInnerProductExtremaLadder, int64_t);
+DECLARE_TYPED_UNITTEST(TestInnerProductExtremaLadder, double);
+
+// ------------------------------------------------------------------ transform_scan / tabulate / generate
+void TestTransformScanSimple() {  // testing/transform_scan.cu:60-120
+  thrust::device_vector<int> input = hv<int>({1, 3, -2, 4, -5}), output(5);
+  thrust::transform_inclusive_scan(input.begin(), input.end(), output.begin(), thrust::negate<int>(), thrust::plus<int>());
+  ASSERT_EQUAL(output, hv<int>({-1, -4, -2, -6, -1}));
+  thrust::transform_exclusive_scan(input.begin(), input.end(), output.begin(), thrust::negate<int>(), 0, thrust::plus<int>());
+  ASSERT_EQUAL(output, hv<int>({0, -1, -4, -2, -6}));
+  thrust::transform_exclusive_scan(input.begin(), input.end(), output.begin(), thrust::negate<int>(), 3, thrust::plus<int>());
+  ASSERT_EQUAL(output, hv<int>({3, 2, -1, 1, -3}));
+  thrust::transform_inclusive_scan(input.begin(), input.end(), input.begin(), thrust::negate<int>(), thrust::plus<int>());  // in place
+  ASSERT_EQUAL(input, hv<int>({-1, -4, -2, -6, -1}));
+}
+DECLARE_UNITTEST(TestTransformScanSimple);
+
+struct constant_seven {
+  __host__ __device__ int operator()() const { return 7; }
+};
+void TestTabulateGenerateSequenceOfRandoms() {
+  using namespace thrust::placeholders;
+  thrust::device_vector<int> v(5);
+  thrust::tabulate(v.begin(), v.end(), thrust::identity<int>());
+  ASSERT_EQUAL(v, hv<int>({0, 1, 2, 3, 4}));  // testing/tabulate.cu:48-75
+  thrust::tabulate(v.begin(), v.end(), -_1);
+  ASSERT_EQUAL(v, hv<int>({0, -1, -2, -3, -4}));
+  thrust::tabulate(v.begin(), v.end(), _1 * _1 * _1);
+  ASSERT_EQUAL(v, hv<int>({0, 1, 8, 27, 64}));
+  thrust::generate(v.begin(), v.end(), constant_seven());
+  ASSERT_EQUAL(v, hv<int>({7, 7, 7, 7, 7}));
+  thrust::generate_n(v.begin(), 3, constant_seven());
+  thrust::device_vector<int> a = hv<int>({1, 2, 3, 4}), b = hv<int>({10, 20, 30, 40}), c(4);
+  thrust::transform(a.begin(), a.end(), b.begin(), c.begin(), 2 * _1 + _2);
+  ASSERT_EQUAL(c, hv<int>({12, 24, 36, 48}));
+  thrust::transform(a.begin(), a.end(), c.begin(), _1 % 2 == 0);
+  ASSERT_EQUAL(c, hv<int>({0, 1, 0, 1}));
+}
+DECLARE_UNITTEST(TestTabulateGenerateSequenceOfRandoms);
+
+// ------------------------------------------------------------------ random
+// the engines are the standard's minstd generators: the streams must agree number for number
+void TestRandomEnginesMatchTheStandardOnes() {
+  thrust::minstd_rand a;
+  std::minstd_rand b;
+  for (int i = 0; i < 1000; i++) ASSERT_EQUAL((unsigned)a(), (unsigned)b());
+  thrust::minstd_rand0 a0(12345);
+  std::minstd_rand0 b0(12345);
+  for (int i = 0; i < 1000; i++) ASSERT_EQUAL((unsigned)a0(), (unsigned)b0());
+  // the 10000th value of a default-constructed engine (C++ standard, [rand.predef])
+  thrust::minstd_rand c;
+  c.discard(9999);
+  ASSERT_EQUAL((unsigned)c(), 399268537u);
+  thrust::minstd_rand0 c0;
+  c0.discard(9999);
+  ASSERT_EQUAL((unsigned)c0(), 1043618065u);
+  // discard(z) equals z calls, also for large z (modular exponentiation)
+  thrust::minstd_rand d1(77), d2(77);
+  for (int i = 0; i < 54321; i++) d1();
+  d2.discard(54321);
+  ASSERT_TRUE(d1 == d2);
+  ASSERT_EQUAL((unsigned)thrust::minstd_rand(0)(), (unsigned)thrust::minstd_rand(1)());  // a seed of 0 becomes 1
+  thrust::default_random_engine rng;
+  thrust::uniform_int_distribution<int> dist(10, 99);
+  thrust::uniform_real_distribution<float> u01;
+  thrust::normal_distribution<double> normal(5.0, 2.0);
+  double mean = 0;
+  for (int i = 0; i < 20000; i++) {
+    const int x = dist(rng);
+    ASSERT_TRUE(x >= 10 && x <= 99);
+    const float u = u01(rng);
+    ASSERT_TRUE(u >= 0.0f && u < 1.0f);
+    mean += normal(rng);
+  }
+  mean /= 20000;
+  ASSERT_TRUE(mean > 4.9 && mean < 5.1);
+}
+DECLARE_UNITTEST(TestRandomEnginesMatchTheStandardOnes);
+
+// the same engine on the device: one value per element, each from its own position in the stream
+struct draw {
+  __host__ __device__ unsigned operator()(unsigned i) const {
+    thrust::default_random_engine rng;
+    rng.discard(i);
+    thrust::uniform_int_distribution<unsigned> dist(0, 9999);
+    return dist(rng);
+  }
+};
+void TestRandomOnDeviceMatchesHost() {
+  const unsigned n = 100000;
+  thrust::device_vector<unsigned> d(n);
+  thrust::tabulate(d.begin(), d.end(), draw());
+  thrust::host_vector<unsigned> h(n);
+  thrust::default_random_engine rng;
+  thrust::uniform_int_distribution<unsigned> dist(0, 9999);
+  for (unsigned i = 0; i < n; i++) h[i] = dist(rng);
+  ASSERT_EQUAL(d, h);
+}
+DECLARE_UNITTEST(TestRandomOnDeviceMatchesHost);
+
+int main(int argc, char** argv) { return unittest::run_all(argc, argv); }

@@ -20,9 +20,28 @@ def compile_snippet(tmp_path, body, extra=()):
 def test_cpp_tests_compile():
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    for name in ["test_sort", "test_scan", "test_by_key", "test_system", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface",
+    for name in ["test_algorithms", "test_sort", "test_scan", "test_by_key", "test_system", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface",
                  "bench_generic"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
+
+
+def test_oracle_runs_clean_under_the_sanitizers():
+    # every entry point of the CPU oracle over small inputs of every type, operator and flag, built
+    # with -fsanitize=address,undefined: the parity tests trust it as their reference
+    r = subprocess.run(["make", "-B", "-C", os.path.join(ROOT, "oracle"), "selfcheck"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    r = subprocess.run([os.path.join(ROOT, "oracle", "selfcheck")], capture_output=True, text=True,
+                       env=dict(os.environ, ASAN_OPTIONS="detect_leaks=1", UBSAN_OPTIONS="print_stacktrace=1"))
+    assert r.returncode == 0 and "selfcheck: ok" in r.stdout, r.stdout[-2000:] + r.stderr[-3000:]
+
+
+def test_host_compiled_tests_build_under_the_sanitizers():
+    # the g++ translation units once more with -fsanitize=address,undefined (run on the GPU by
+    # tests/test_cpp_api_gpu.py)
+    r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "san"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    for name in ["test_sort", "test_scan", "test_by_key", "test_system"]:
+        assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", "san", name))
 
 
 def test_existing_thrust_code_compiles_unchanged(tmp_path):

@@ -58,93 +58,23 @@ __device__ inline bool keys_differ(KU a, KU b, int float_keys) {
 
 // Both kernels are compiled for 4 wavefronts per SIMD (at most 128 VGPRs): two 512-thread
 // workgroups per CU.  Left alone, the register allocator may trade that occupancy away.
-#ifndef TCD_RBK_ATTR
-#define TCD_RBK_ATTR __attribute__((amdgpu_waves_per_eu(4)))
-#endif
-#ifndef TCD_SBK_ATTR
-#define TCD_SBK_ATTR __attribute__((amdgpu_waves_per_eu(4)))
-#endif
-template <int BYTES> struct bits_of;
-template <> struct bits_of<1> { using type = uint8_t; };
-template <> struct bits_of<2> { using type = uint16_t; };
-template <> struct bits_of<4> { using type = uint32_t; };
-template <> struct bits_of<8> { using type = uint64_t; };
-
-// N consecutive elements from a pointer aligned to min(16, N*sizeof(E)) bytes, as 128-bit
-// (or one narrower) accesses.
-template <int N, class E>
-__device__ inline void load_group(const E* p, E (&dst)[N]) {
-  constexpr int BYTES = N * (int)sizeof(E);
-  if constexpr (BYTES >= 16) {
-#pragma unroll
-    for (int q = 0; q < BYTES / 16; q++) {
-      const tcd_v4u t = load16<tcd_v4u>(reinterpret_cast<const char*>(p) + 16 * q);
-      __builtin_memcpy(reinterpret_cast<char*>(dst) + 16 * q, &t, 16);
-    }
-  } else {
-    const typename bits_of<BYTES>::type t = *reinterpret_cast<const typename bits_of<BYTES>::type*>(p);
-    __builtin_memcpy(dst, &t, BYTES);
-  }
-}
-template <int N, class E>
-__device__ inline void store_group(E* p, const E (&src)[N]) {
-  constexpr int BYTES = N * (int)sizeof(E);
-  if constexpr (BYTES >= 16) {
-#pragma unroll
-    for (int q = 0; q < BYTES / 16; q++) {
-      tcd_v4u t;
-      __builtin_memcpy(&t, reinterpret_cast<const char*>(src) + 16 * q, 16);
-      store16(reinterpret_cast<char*>(p) + 16 * q, t);
-    }
-  } else {
-    typename bits_of<BYTES>::type t;
-    __builtin_memcpy(&t, src, BYTES);
-    *reinterpret_cast<typename bits_of<BYTES>::type*>(p) = t;
-  }
-}
-
-// Tile geometry.  Two layouts exist; the blocked one is the default.  (The striped one, kept for
-// comparison with -DTCD_SEG_BLOCKED=0: a thread owns VEC consecutive elements of each of CHUNKS
-// chunks, the wider of key and value fills GROUP_BYTES per thread and chunk; 16-byte groups with
-// 8 chunks beat 32- and 64-byte groups.  On MI355X at 2^28 int32 pairs it is 2 % faster when every
-// element is a run of its own and 3-5 % slower at mean run lengths 8 and 512.)
-#ifndef TCD_SEG_BLOCKED
-#define TCD_SEG_BLOCKED 1
-#endif
-#ifndef TCD_SEG_BLOCK
-#define TCD_SEG_BLOCK 512
-#endif
-#if TCD_SEG_BLOCKED
-// Blocked tiles: a thread owns VEC consecutive elements (128 bytes of the wider of key and
-// value, at most 32 elements), a wavefront 64 * VEC consecutive ones.  Global memory is read
-// and written in wave-wide contiguous 1 KiB accesses and transposed to the blocked order through
-// a wave-private LDS buffer, so one sequential walk per thread and ONE wavefront scan per tile
-// replace a scan per 16-byte group: a third of the vector instructions of the striped layout.
-template <class T, int GROUP_BYTES, int CHUNKS_>
+#define TCD_SEG_ATTR __attribute__((amdgpu_waves_per_eu(4)))
+// Tile geometry: blocked tiles.  A thread owns VEC consecutive elements (128 bytes of the wider
+// of key and value, at most 32 elements), a wavefront 64 * VEC consecutive ones.  Global memory is
+// read and written in wave-wide contiguous 1 KiB accesses and transposed to the blocked order
+// through a wave-private LDS buffer, so one sequential walk per thread and ONE wavefront scan per
+// tile do the work.  (A striped layout, 16-byte groups of each of 8 chunks per thread with a scan
+// per group, needed three times the vector instructions; at 2^28 int32 pairs it was 2 % faster
+// when every element is a run of its own and 3-5 % slower at mean run lengths 8 and 512.)
+template <class T>
 struct SegGeom {
-  static constexpr bool BLOCKED = true;
-  static constexpr int BLOCK = TCD_SEG_BLOCK;
+  static constexpr int BLOCK = 512;
   static constexpr int WIDE = (int)(sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T));
   static constexpr int VEC = WIDE == 8 ? 16 : 32;
-  static constexpr int CHUNKS = 1;
   static constexpr int NWAVES = BLOCK / kWave;
   static constexpr int64_t TILE = (int64_t)BLOCK * VEC;
   static constexpr int XPOSE_SLOTS = 512;  // 16-byte slots of a wavefront's transpose buffer (8 KiB)
 };
-#else
-template <class T, int GROUP_BYTES, int CHUNKS_>
-struct SegGeom {
-  static constexpr bool BLOCKED = false;
-  static constexpr int BLOCK = TCD_SEG_BLOCK;
-  static constexpr int WIDE = (int)(sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T));
-  static constexpr int VEC = GROUP_BYTES / WIDE > 16 ? 16 : GROUP_BYTES / WIDE;
-  // at most 32 elements per thread: narrow types hold one element per register
-  static constexpr int CHUNKS = VEC * CHUNKS_ > 32 ? 32 / VEC : CHUNKS_;
-  static constexpr int NWAVES = BLOCK / kWave;
-  static constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
-  static constexpr int XPOSE_SLOTS = 1;
-};
-#endif
 
 // Orders a wavefront's LDS accesses around an exchange through its private buffer (the LDS
 // executes one wavefront's instructions in order; this keeps the compiler from reordering them).
@@ -250,56 +180,40 @@ __device__ inline void wave_store_blocked_partial(E* dst, const E (&src)[VEC], t
   }
   wave_lds_sync();
 }
-#ifndef TCD_SBK_GROUP
-#define TCD_SBK_GROUP 16
-#endif
-#ifndef TCD_SBK_CHUNKS
-#define TCD_SBK_CHUNKS 8
-#endif
-#ifndef TCD_RBK_GROUP
-#define TCD_RBK_GROUP 16
-#endif
-#ifndef TCD_RBK_CHUNKS
-#define TCD_RBK_CHUNKS 8
-#endif
-template <class T> using ScanByKeyGeom = SegGeom<T, TCD_SBK_GROUP, TCD_SBK_CHUNKS>;
-template <class T> using ReduceByKeyGeom = SegGeom<T, TCD_RBK_GROUP, TCD_RBK_CHUNKS>;
 
 // Loads a tile, finds the segment heads, reduces it and resolves the prefix of all earlier
-// tiles by look-back.  On return key/val hold the thread's elements, bit j of heads[c] says
-// whether element (c, j) starts a segment, and off[c] is the pair (heads seen, value of the
-// open segment) of everything before the thread's group of chunk c.  The kernels then walk
-// their elements once more from off[c]; nothing per element is kept in between.
+// tiles by look-back.  On return key/val hold the thread's VEC consecutive elements, bit j of
+// `heads` says whether element j starts a segment, and `off` is the pair (heads seen, value of the
+// open segment) of everything before the thread's first element.  The kernels then walk their
+// elements once more from `off`; nothing per element is kept in between.
 template <class T, class Op, class G>
 struct SegTile {
   using Pair = SegPair<T>;
-  static constexpr int VEC = G::VEC, CHUNKS = G::CHUNKS, NWAVES = G::NWAVES, BLOCK = G::BLOCK;
-  static_assert(CHUNKS * NWAVES <= kWave, "one wavefront scans the (chunk, wave) totals");
+  static constexpr int VEC = G::VEC, NWAVES = G::NWAVES, BLOCK = G::BLOCK;
+  static_assert(NWAVES <= kWave, "one wavefront scans the wavefronts' totals");
 
   struct Smem {
-    Pair tot[CHUNKS * NWAVES];  // inclusive total of (chunk, wave), then its prefix over the whole input
+    Pair tot[NWAVES];  // inclusive total of a wavefront, then its prefix over the whole input
     uint32_t tile;
   };
 
-  KU key[CHUNKS][VEC];
-  T val[CHUNKS][VEC];
-  uint32_t heads[CHUNKS];
-  Pair excl_w[CHUNKS];  // everything before the thread's group within its wavefront's part of chunk c
-  Pair off[CHUNKS];
+  KU key[VEC];
+  T val[VEC];
+  uint32_t heads;
+  Pair excl_w;  // everything before the thread's elements within its wavefront
+  Pair off;
   int64_t base;
   int64_t tile;
   bool full;  // every element of the tile exists, the tile is not the last one, pointers are aligned to their elements
 
-  __device__ int64_t index(int c, int j) const {
-    return base + ((int64_t)c * BLOCK + threadIdx.x) * VEC + j;
-  }
+  __device__ int64_t first_index() const { return base + (int64_t)threadIdx.x * VEC; }
 
   __device__ static Pair comb(const Pair& a, const Pair& b) { return seg_combine<T, Op>(a, b); }
 
-  // xbuf: the wavefront's transpose buffer (blocked geometry only).  TICKET: tiles are handed out
-  // by an atomic counter (every tile waited for has started; used when an output overlaps an
-  // input); otherwise a tile is the workgroup of the same index and a descriptor that stays
-  // missing after `patience` polls is recomputed from the input.
+  // xbuf: the wavefront's transpose buffer.  TICKET: tiles are handed out by an atomic counter
+  // (every tile waited for has started; used when an output overlaps an input); otherwise a tile
+  // is the workgroup of the same index and a descriptor that stays missing after `patience` polls
+  // is recomputed from the input.
   template <bool TICKET, class Meanwhile>
   __device__ void run(Smem& sm, const KU* keys, const T* vals, int64_t n, int float_keys, int vec_ok,
                       uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf, int patience, int publish_delay,
@@ -318,81 +232,59 @@ struct SegTile {
     }
     base = tile * G::TILE;
     full = vec_ok && (base + G::TILE < n);
+    const int64_t i0 = first_index();
 
     if (full) {
-      if constexpr (G::BLOCKED) {
-        const int64_t w0 = base + (int64_t)wave * (kWave * VEC);
-        wave_load_blocked<VEC>(keys + w0, key[0], xbuf, lane);
-        wave_load_blocked<VEC>(vals + w0, val[0], xbuf, lane);
-      } else {
-#pragma unroll
-        for (int c = 0; c < CHUNKS; c++) {
-          const int64_t i0 = index(c, 0);
-          load_group<VEC>(keys + i0, key[c]);
-          load_group<VEC>(vals + i0, val[c]);
-        }
-      }
-    } else if (G::BLOCKED && vec_ok) {
+      const int64_t w0 = base + (int64_t)wave * (kWave * VEC);
+      wave_load_blocked<VEC>(keys + w0, key, xbuf, lane);
+      wave_load_blocked<VEC>(vals + w0, val, xbuf, lane);
+    } else if (vec_ok) {
       // the last tile: the same contiguous accesses up to the end of the input; elements that
       // do not exist read as key 0 and the operator's identity
-      if constexpr (G::BLOCKED) {
-        const int64_t w0 = base + (int64_t)wave * (kWave * VEC);
-        wave_load_blocked_partial<VEC>(keys + w0, key[0], xbuf, lane, n - w0);
-        wave_load_blocked_partial<VEC>(vals + w0, val[0], xbuf, lane, n - w0);
-        const int64_t i0 = index(0, 0);
+      const int64_t w0 = base + (int64_t)wave * (kWave * VEC);
+      wave_load_blocked_partial<VEC>(keys + w0, key, xbuf, lane, n - w0);
+      wave_load_blocked_partial<VEC>(vals + w0, val, xbuf, lane, n - w0);
 #pragma unroll
-        for (int j = 0; j < VEC; j++)
-          if (i0 + j >= n) val[0][j] = id;
-      }
+      for (int j = 0; j < VEC; j++)
+        if (i0 + j >= n) val[j] = id;
     } else {
 #pragma unroll
-      for (int c = 0; c < CHUNKS; c++) {
-        const int64_t i0 = index(c, 0);
-#pragma unroll
-        for (int j = 0; j < VEC; j++) {
-          const int64_t idx = i0 + j;
-          key[c][j] = idx < n ? keys[idx] : KU(0);
-          val[c][j] = idx < n ? vals[idx] : id;
-        }
+      for (int j = 0; j < VEC; j++) {
+        const int64_t idx = i0 + j;
+        key[j] = idx < n ? keys[idx] : KU(0);
+        val[j] = idx < n ? vals[idx] : id;
       }
     }
-    // the key before a thread's group is the last key of the lane below (its group precedes this
-    // one in memory); only lane 0 of each wave fetches it from memory
+    // the key before a thread's elements is the last key of the lane below (its elements precede
+    // these in memory); only lane 0 of each wave fetches it from memory
     using KW = typename std::conditional<(sizeof(KU) < 4), uint32_t, KU>::type;
-    KU prev[CHUNKS];
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-      const int64_t i0 = index(c, 0);
-      KU first = KU(0);
-      if (lane == 0 && i0 > 0 && i0 < n) first = keys[i0 - 1];
-      prev[c] = (KU)wave_shift_up1((KW)key[c][VEC - 1], (KW)first);
-    }
+    KU first = KU(0);
+    if (lane == 0 && i0 > 0 && i0 < n) first = keys[i0 - 1];
+    const KU prev = (KU)wave_shift_up1((KW)key[VEC - 1], (KW)first);
 
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-      const int64_t i0 = index(c, 0);
+    {
       uint32_t h = 0;
       Pair agg = idp;
 #pragma unroll
       for (int j = 0; j < VEC; j++) {
-        const KU p = j == 0 ? prev[c] : key[c][j - 1];
-        const bool is_head = (full || i0 + j < n) && (i0 + j == 0 || keys_differ(p, key[c][j], float_keys));
+        const KU p = j == 0 ? prev : key[j - 1];
+        const bool is_head = (full || i0 + j < n) && (i0 + j == 0 || keys_differ(p, key[j], float_keys));
         h |= (is_head ? 1u : 0u) << j;
-        agg.v = is_head ? val[c][j] : Op::template apply<T>(agg.v, val[c][j]);
+        agg.v = is_head ? val[j] : Op::template apply<T>(agg.v, val[j]);
       }
-      heads[c] = h;
+      heads = h;
       agg.c = __builtin_popcount(h);
       const Pair w = wave_inclusive_scan(agg, idp, comb);
-      excl_w[c] = wave_shift_up1(w, idp);
-      if (lane == kWave - 1) sm.tot[c * NWAVES + wave] = w;
+      excl_w = wave_shift_up1(w, idp);
+      if (lane == kWave - 1) sm.tot[wave] = w;
     }
     __syncthreads();
 
-    // wave 0: scan of the (chunk, wave) totals in tile order, look-back, then each (chunk, wave)'s
+    // wave 0: scan of the wavefronts' totals in tile order, look-back, then each wavefront's
     // prefix over the whole input goes back into the table
     Pair tile_agg = idp, before = idp;
     if (wave == 0) {
-      const Pair mine = lane < CHUNKS * NWAVES ? sm.tot[lane] : idp;
+      const Pair mine = lane < NWAVES ? sm.tot[lane] : idp;
       const Pair incl = wave_inclusive_scan(mine, idp, comb);
       tile_agg = readlane(incl, kWave - 1);
       before = wave_shift_up1(incl, idp);
@@ -429,11 +321,10 @@ struct SegTile {
         }
         if (lane == 0) TileDesc<Pair>::store(desc, tile, kInclusive, comb(prefix, tile_agg));
       }
-      if (lane < CHUNKS * NWAVES) sm.tot[lane] = comb(prefix, before);
+      if (lane < NWAVES) sm.tot[lane] = comb(prefix, before);
     }
     __syncthreads();
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) off[c] = comb(sm.tot[c * NWAVES + wave], excl_w[c]);
+    off = comb(sm.tot[wave], excl_w);
   }
 };
 
@@ -441,56 +332,53 @@ struct SegTile {
 // scan_by_key
 // ---------------------------------------------------------------------------------------
 template <class T, class Op, bool TICKET>
-__global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_key_kernel(
+__global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void scan_by_key_kernel(
     const KU* keys, const T* vals, T* out, int64_t n, T init, int exclusive, int float_keys, int vec_ok,
     uint64_t* desc, uint32_t* ticket, int patience, int publish_delay) {
-  using G = ScanByKeyGeom<T>;
+  using G = SegGeom<T>;
   using ST = SegTile<T, Op, G>;
   __shared__ typename ST::Smem sm;
-  __shared__ tcd_v4u s_x[G::BLOCKED ? G::NWAVES : 1][G::XPOSE_SLOTS];
-  tcd_v4u* xbuf = s_x[G::BLOCKED ? threadIdx.x / kWave : 0];
+  __shared__ tcd_v4u s_x[G::NWAVES][G::XPOSE_SLOTS];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  tcd_v4u* xbuf = s_x[wave];
   ST t;
-  constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS;
-  // Whole tiles of the blocked layout: each wavefront scans its elements from the wavefront's
-  // own start and parks the result in its buffer (in the order of the later contiguous stores)
-  // BEFORE the look-back.  Afterwards only the elements of the run that came into the wavefront
-  // open (those before its first head, `first_head` of them) still take the value of that run
-  // so far; the four operators are commutative, so it is applied on top of the parked result.
-  constexpr int NQ = G::BLOCKED ? VEC * (int)sizeof(T) / 16 : 1;
+  constexpr int VEC = ST::VEC;
+  // Whole tiles: each wavefront scans its elements from the wavefront's own start and parks the
+  // result in its buffer (in the order of the later contiguous stores) BEFORE the look-back.
+  // Afterwards only the elements of the run that came into the wavefront open (those before its
+  // first head, `first_head` of them) still take the value of that run so far; the four operators
+  // are commutative, so it is applied on top of the parked result.
+  constexpr int NQ = VEC * (int)sizeof(T) / 16;
   constexpr int EPP = 16 / (int)sizeof(T);  // elements per 16-byte slot
   bool parked = false;
   uint32_t first_head = 0;
   t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, [&] {
-    if constexpr (G::BLOCKED) {
-      if (!t.full) return;
-      parked = true;
-      const int lane = threadIdx.x & (kWave - 1);
-      T r[VEC];
-      T open = t.excl_w[0].v;
+    if (!t.full) return;
+    parked = true;
+    T r[VEC];
+    T open = t.excl_w.v;
 #pragma unroll
-      for (int j = 0; j < VEC; j++) {
-        const bool is_head = (t.heads[0] >> j) & 1u;
-        const T x = t.val[0][j];
-        if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
-        open = is_head ? x : Op::template apply<T>(open, x);
-        if (!exclusive) r[j] = open;
-      }
-      const uint64_t has = __ballot(t.heads[0] != 0u);
-      first_head = kWave * VEC;
-      if (has) {
-        const int owner = __builtin_ctzll(has);
-        first_head = (uint32_t)(owner * VEC + __builtin_ctz((uint32_t)__builtin_amdgcn_readlane((int)t.heads[0], owner)));
-      }
+    for (int j = 0; j < VEC; j++) {
+      const bool is_head = (t.heads >> j) & 1u;
+      const T x = t.val[j];
+      if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
+      open = is_head ? x : Op::template apply<T>(open, x);
+      if (!exclusive) r[j] = open;
+    }
+    const uint64_t has = __ballot(t.heads != 0u);
+    first_head = kWave * VEC;
+    if (has) {
+      const int owner = __builtin_ctzll(has);
+      first_head = (uint32_t)(owner * VEC + __builtin_ctz((uint32_t)__builtin_amdgcn_readlane((int)t.heads, owner)));
+    }
 #pragma unroll
-      for (int i = 0; i < NQ; i++) {
-        tcd_v4u piece;
-        __builtin_memcpy(&piece, reinterpret_cast<const char*>(r) + 16 * i, 16);
-        xbuf[xpose_slot(lane * NQ + i)] = piece;
-      }
+    for (int i = 0; i < NQ; i++) {
+      tcd_v4u piece;
+      __builtin_memcpy(&piece, reinterpret_cast<const char*>(r) + 16 * i, 16);
+      xbuf[xpose_slot(lane * NQ + i)] = piece;
     }
   });
   if (parked) {
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const T carried = sm.tot[wave].v;  // the open run's value over everything before the wavefront
     char* dst = reinterpret_cast<char*>(out + t.base + (int64_t)wave * (kWave * VEC));
 #pragma unroll
@@ -508,34 +396,25 @@ __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_
     }
     return;
   }
+  // the last tile, and every tile of a call whose pointers are not aligned to their elements
+  T r[VEC];
+  T open = t.off.v;  // value of the open segment just before the element
 #pragma unroll
-  for (int c = 0; c < CHUNKS; c++) {
-    T r[VEC];
-    T open = t.off[c].v;  // value of the open segment just before the element
+  for (int j = 0; j < VEC; j++) {
+    const bool is_head = (t.heads >> j) & 1u;
+    const T x = t.val[j];
+    if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
+    open = is_head ? x : Op::template apply<T>(open, x);
+    if (!exclusive) r[j] = open;
+  }
+  if (vec_ok) {
+    const int64_t w0 = t.base + (int64_t)wave * (kWave * VEC);
+    wave_store_blocked_partial<VEC>(out + w0, r, xbuf, lane, n - w0);
+  } else {
+    const int64_t i0 = t.first_index();
 #pragma unroll
-    for (int j = 0; j < VEC; j++) {
-      const bool is_head = (t.heads[c] >> j) & 1u;
-      const T x = t.val[c][j];
-      if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
-      open = is_head ? x : Op::template apply<T>(open, x);
-      if (!exclusive) r[j] = open;
-    }
-    const int64_t i0 = t.index(c, 0);
-    if (t.full) {
-      if constexpr (G::BLOCKED)
-        wave_store_blocked<VEC>(out + t.base + (int64_t)(threadIdx.x / kWave) * (kWave * VEC), r, xbuf, threadIdx.x & (kWave - 1));
-      else
-        store_group<VEC>(out + i0, r);
-    } else if (G::BLOCKED && vec_ok) {
-      if constexpr (G::BLOCKED) {
-        const int64_t w0 = t.base + (int64_t)(threadIdx.x / kWave) * (kWave * VEC);
-        wave_store_blocked_partial<VEC>(out + w0, r, xbuf, threadIdx.x & (kWave - 1), n - w0);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < VEC; j++)
-        if (i0 + j < n) out[i0 + j] = r[j];
-    }
+    for (int j = 0; j < VEC; j++)
+      if (i0 + j < n) out[i0 + j] = r[j];
   }
 }
 
@@ -543,159 +422,116 @@ __global__ __launch_bounds__(ScanByKeyGeom<T>::BLOCK) TCD_SBK_ATTR void scan_by_
 // reduce_by_key
 // ---------------------------------------------------------------------------------------
 template <class T, class Op, bool TICKET>
-__global__ __launch_bounds__(ReduceByKeyGeom<T>::BLOCK) TCD_RBK_ATTR void reduce_by_key_kernel(
+__global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void reduce_by_key_kernel(
     const KU* keys, const T* vals, KU* keys_out, T* vals_out, int64_t* num_runs, int64_t n,
     int float_keys, int vec_ok, uint64_t* desc, uint32_t* ticket, int patience, int publish_delay) {
-  using G = ReduceByKeyGeom<T>;
+  using G = SegGeom<T>;
   using ST = SegTile<T, Op, G>;
-  constexpr int VEC = ST::VEC, CHUNKS = ST::CHUNKS, NWAVES = ST::NWAVES;
+  constexpr int VEC = ST::VEC, NWAVES = ST::NWAVES;
   __shared__ typename ST::Smem sm;
   const int lane = threadIdx.x & (kWave - 1);
-  if constexpr (G::BLOCKED) {
-    // The heads of a wavefront's 64 * VEC consecutive elements go to consecutive output slots.
-    // They are compacted in the wavefront's buffer — keys first, then, through the same 8 KiB,
-    // the values of the runs they close — and written with contiguous stores.
-    static_assert(kWave * VEC * sizeof(KU) <= G::XPOSE_SLOTS * 16 && kWave * VEC * sizeof(T) <= G::XPOSE_SLOTS * 16,
-                  "a wavefront's heads fit its buffer");
-    __shared__ tcd_v4u s_x[NWAVES][G::XPOSE_SLOTS];
-    tcd_v4u* xbuf = s_x[threadIdx.x / kWave];
-    ST t;
-    // Slot i lives at sw(i): when most elements are heads a thread's slots start VEC apart, which
-    // is one LDS bank for all lanes; the swizzle (within aligned groups of VEC slots) spreads them
-    // and the copy-out reads over all banks.
-    constexpr uint32_t kLogVec = VEC == 32 ? 5 : 4;
-    static_assert((1u << kLogVec) == (uint32_t)VEC, "VEC is 16 or 32");
-    const auto sw = [](uint32_t i) { return i ^ ((i >> kLogVec) & (uint32_t)(VEC - 1)); };
-    // A wavefront with few enough heads compacts them BEFORE the look-back, while the aggregates
-    // of earlier tiles are still on their way: keys into the lower half of its buffer, the values
-    // of the runs they close into the upper half.  Only the output position and the start of the
-    // run open at the wavefront's first element depend on earlier tiles; both are applied during
-    // the copy-out.  (Not in the last tile, which also closes the last run.)
-    constexpr uint32_t kHalfBytes = G::XPOSE_SLOTS * 16 / 2;
-    constexpr uint32_t kEarlyMax = kHalfBytes / (sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T)) - VEC;
-    KU* const early_k = reinterpret_cast<KU*>(xbuf);
-    T* const early_v = reinterpret_cast<T*>(reinterpret_cast<char*>(xbuf) + kHalfBytes);
-    bool early = false;
-    uint32_t count = 0;
-    t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, [&] {
-      count = (uint32_t)__builtin_amdgcn_readlane((int)(t.excl_w[0].c + __builtin_popcount(t.heads[0])), kWave - 1);
-      early = t.full && count <= kEarlyMax;
-      if (!early) {
-        if (t.full) {  // the keys alone always fit
-          uint32_t slot = t.excl_w[0].c;
+  // The heads of a wavefront's 64 * VEC consecutive elements go to consecutive output slots.
+  // They are compacted in the wavefront's buffer — keys first, then, through the same 8 KiB,
+  // the values of the runs they close — and written with contiguous stores.
+  static_assert(kWave * VEC * sizeof(KU) <= G::XPOSE_SLOTS * 16 && kWave * VEC * sizeof(T) <= G::XPOSE_SLOTS * 16,
+                "a wavefront's heads fit its buffer");
+  __shared__ tcd_v4u s_x[NWAVES][G::XPOSE_SLOTS];
+  tcd_v4u* xbuf = s_x[threadIdx.x / kWave];
+  ST t;
+  // Slot i lives at sw(i): when most elements are heads a thread's slots start VEC apart, which
+  // is one LDS bank for all lanes; the swizzle (within aligned groups of VEC slots) spreads them
+  // and the copy-out reads over all banks.
+  constexpr uint32_t kLogVec = VEC == 32 ? 5 : 4;
+  static_assert((1u << kLogVec) == (uint32_t)VEC, "VEC is 16 or 32");
+  const auto sw = [](uint32_t i) { return i ^ ((i >> kLogVec) & (uint32_t)(VEC - 1)); };
+  // A wavefront with few enough heads compacts them BEFORE the look-back, while the aggregates
+  // of earlier tiles are still on their way: keys into the lower half of its buffer, the values
+  // of the runs they close into the upper half.  Only the output position and the start of the
+  // run open at the wavefront's first element depend on earlier tiles; both are applied during
+  // the copy-out.  (Not in the last tile, which also closes the last run.)
+  constexpr uint32_t kHalfBytes = G::XPOSE_SLOTS * 16 / 2;
+  constexpr uint32_t kEarlyMax = kHalfBytes / (sizeof(KU) > sizeof(T) ? sizeof(KU) : sizeof(T)) - VEC;
+  KU* const early_k = reinterpret_cast<KU*>(xbuf);
+  T* const early_v = reinterpret_cast<T*>(reinterpret_cast<char*>(xbuf) + kHalfBytes);
+  bool early = false;
+  uint32_t count = 0;
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, [&] {
+    count = (uint32_t)__builtin_amdgcn_readlane((int)(t.excl_w.c + __builtin_popcount(t.heads)), kWave - 1);
+    early = t.full && count <= kEarlyMax;
+    if (!early) {
+      if (t.full) {  // the keys alone always fit
+        uint32_t slot = t.excl_w.c;
 #pragma unroll
-          for (int j = 0; j < VEC; j++)
-            if ((t.heads[0] >> j) & 1u) early_k[sw(slot++)] = t.key[0][j];
-        }
-        return;
-      }
-      uint32_t slot = t.excl_w[0].c;
-      T open = t.excl_w[0].v;  // the open run's value over the wavefront's earlier elements
-#pragma unroll
-      for (int j = 0; j < VEC; j++) {
-        if ((t.heads[0] >> j) & 1u) {
-          early_k[sw(slot)] = t.key[0][j];
-          early_v[sw(slot)] = open;
-          slot++;
-          open = t.val[0][j];
-        } else {
-          open = Op::template apply<T>(open, t.val[0][j]);
-        }
-      }
-    });
-    if (early) {
-      const SegPair<T> before_wave = sm.tot[threadIdx.x / kWave];
-      const uint32_t first = before_wave.c;
-      for (uint32_t i = lane; i < count; i += kWave) {
-        keys_out[first + i] = early_k[sw(i)];
-        T v = early_v[sw(i)];
-        if (i == 0) v = Op::template apply<T>(before_wave.v, v);  // the run came into the wavefront open
-        if (first + i) vals_out[first + i - 1] = v;
+        for (int j = 0; j < VEC; j++)
+          if ((t.heads >> j) & 1u) early_k[sw(slot++)] = t.key[j];
       }
       return;
     }
-    SegPair<T> run = t.off[0];  // (runs started so far, value of the open run) before the current element
-    const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)run.c);  // runs before this wavefront
-    const uint32_t heads = t.heads[0];
-    const uint32_t mine = run.c - first;  // slot of this thread's first head
-    const int64_t i0 = t.index(0, 0);
-    // Too many heads for both halves (or the last tile): the values go through the buffer after
-    // the keys.  A whole tile's keys were compacted before the look-back.
-    KU* sk = reinterpret_cast<KU*>(xbuf);
-    if (!t.full) {
-      uint32_t slot = mine;
+    uint32_t slot = t.excl_w.c;
+    T open = t.excl_w.v;  // the open run's value over the wavefront's earlier elements
 #pragma unroll
-      for (int j = 0; j < VEC; j++)
-        if ((heads >> j) & 1u) sk[sw(slot++)] = t.key[0][j];
-    }
-    wave_lds_sync();
-    for (uint32_t i = lane; i < count; i += kWave) keys_out[first + i] = sk[sw(i)];
-    wave_lds_sync();
-    T* sv = reinterpret_cast<T*>(xbuf);
-    {
-      uint32_t slot = mine;
-#pragma unroll
-      for (int j = 0; j < VEC; j++) {
-        const bool exists = t.full || i0 + j < n;
-        if ((heads >> j) & 1u) {
-          // a head closes the run before it and opens run number run.c
-          sv[sw(slot++)] = run.v;
-          run.c += 1;
-          run.v = t.val[0][j];
-        } else if (exists) {
-          run.v = Op::template apply<T>(run.v, t.val[0][j]);
-        }
-        if (!t.full && i0 + j == n - 1) {  // the last element closes the last run
-          vals_out[run.c - 1] = run.v;
-          *num_runs = (int64_t)run.c;
-        }
+    for (int j = 0; j < VEC; j++) {
+      if ((t.heads >> j) & 1u) {
+        early_k[sw(slot)] = t.key[j];
+        early_v[sw(slot)] = open;
+        slot++;
+        open = t.val[j];
+      } else {
+        open = Op::template apply<T>(open, t.val[j]);
       }
     }
-    wave_lds_sync();
-    for (uint32_t i = lane; i < count; i += kWave)
-      if (first + i) vals_out[first + i - 1] = sv[sw(i)];  // value of the run that ended at this head
+  });
+  if (early) {
+    const SegPair<T> before_wave = sm.tot[threadIdx.x / kWave];
+    const uint32_t first = before_wave.c;
+    for (uint32_t i = lane; i < count; i += kWave) {
+      keys_out[first + i] = early_k[sw(i)];
+      T v = early_v[sw(i)];
+      if (i == 0) v = Op::template apply<T>(before_wave.v, v);  // the run came into the wavefront open
+      if (first + i) vals_out[first + i - 1] = v;
+    }
     return;
   }
-  // Per-wave staging of one chunk's output: the heads of a wave's 64*VEC consecutive elements go
-  // to consecutive output slots, so they are compacted in LDS and written with coalesced stores
-  // (no workgroup barrier: the buffer is private to the wave).
-  __shared__ KU s_keys[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
-  __shared__ T s_vals[G::BLOCKED ? 1 : NWAVES][G::BLOCKED ? 1 : kWave * VEC];
-  ST t;
-  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, nullptr, patience, publish_delay, [] {});
-  KU* sk = s_keys[G::BLOCKED ? 0 : threadIdx.x / kWave];
-  T* sv = s_vals[G::BLOCKED ? 0 : threadIdx.x / kWave];
+  SegPair<T> run = t.off;  // (runs started so far, value of the open run) before the current element
+  const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)run.c);  // runs before this wavefront
+  const uint32_t heads = t.heads;
+  const uint32_t mine = run.c - first;  // slot of this thread's first head
+  const int64_t i0 = t.first_index();
+  // Too many heads for both halves (or the last tile): the values go through the buffer after
+  // the keys.  A whole tile's keys were compacted before the look-back.
+  KU* sk = reinterpret_cast<KU*>(xbuf);
+  if (!t.full) {
+    uint32_t slot = mine;
 #pragma unroll
-  for (int c = 0; c < CHUNKS; c++) {
-    // (runs started so far, value of the open run) before the current element
-    SegPair<T> run = t.off[c];
-    const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)run.c);  // runs before this wave's chunk
-    const int64_t i0 = t.index(c, 0);
+    for (int j = 0; j < VEC; j++)
+      if ((heads >> j) & 1u) sk[sw(slot++)] = t.key[j];
+  }
+  wave_lds_sync();
+  for (uint32_t i = lane; i < count; i += kWave) keys_out[first + i] = sk[sw(i)];
+  wave_lds_sync();
+  T* sv = reinterpret_cast<T*>(xbuf);
+  {
+    uint32_t slot = mine;
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
       const bool exists = t.full || i0 + j < n;
-      if ((t.heads[c] >> j) & 1u) {
+      if ((heads >> j) & 1u) {
         // a head closes the run before it and opens run number run.c
-        sk[run.c - first] = t.key[c][j];
-        sv[run.c - first] = run.v;
+        sv[sw(slot++)] = run.v;
         run.c += 1;
-        run.v = t.val[c][j];
+        run.v = t.val[j];
       } else if (exists) {
-        run.v = Op::template apply<T>(run.v, t.val[c][j]);
+        run.v = Op::template apply<T>(run.v, t.val[j]);
       }
       if (!t.full && i0 + j == n - 1) {  // the last element closes the last run
         vals_out[run.c - 1] = run.v;
         *num_runs = (int64_t)run.c;
       }
     }
-    const uint32_t count = (uint32_t)__builtin_amdgcn_readlane((int)run.c, kWave - 1) - first;
-    __builtin_amdgcn_wave_barrier();
-    for (uint32_t i = lane; i < count; i += kWave) {
-      keys_out[first + i] = sk[i];
-      if (first + i) vals_out[first + i - 1] = sv[i];  // value of the run that ended at this head
-    }
-    __builtin_amdgcn_wave_barrier();
   }
+  wave_lds_sync();
+  for (uint32_t i = lane; i < count; i += kWave)
+    if (first + i) vals_out[first + i - 1] = sv[sw(i)];  // value of the run that ended at this head
 }
 
 template <class T, class G>
@@ -722,11 +558,11 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
     using T = decltype(tv);
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
-      const size_t need = bykey_temp_bytes<T, ScanByKeyGeom<T>>(n);
+      const size_t need = bykey_temp_bytes<T, SegGeom<T>>(n);
       if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
       if (*temp_bytes < need) return;
       if (n == 0) { rc = hipSuccess; return; }
-      const int64_t ntiles = ceil_div(n, ScanByKeyGeom<T>::TILE);
+      const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
       // one tile consults no descriptor and reads all its input before it writes: no clearing
       // launch, no tickets
       const bool single = ntiles == 1;
@@ -743,13 +579,13 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
       const bool aliased = !single && (ranges_overlap(out, (size_t)n * sizeof(T), values, (size_t)n * sizeof(T)) ||
                            ranges_overlap(out, (size_t)n * sizeof(T), keys, (size_t)n * sizeof(KU)));
       if (aliased) {
-        TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(ScanByKeyGeom<T>::BLOCK), s,
+        TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
                            n, iv, exclusive, float_keys, vec_ok,
                            reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
                            reinterpret_cast<uint32_t*>(temp), 0, 0);
       } else {
-        TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, false>), dim3((unsigned)ntiles), dim3(ScanByKeyGeom<T>::BLOCK), s,
+        TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, false>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
                            n, iv, exclusive, float_keys, vec_ok,
                            reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
@@ -773,14 +609,14 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
     using T = decltype(tv);
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
-      const size_t need = bykey_temp_bytes<T, ReduceByKeyGeom<T>>(n);
+      const size_t need = bykey_temp_bytes<T, SegGeom<T>>(n);
       if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
       if (*temp_bytes < need) return;
       if (n == 0) {  // no runs: only the count is written
         rc = zero_async(num_runs_out, sizeof(int64_t), s);
         return;
       }
-      const int64_t ntiles = ceil_div(n, ReduceByKeyGeom<T>::TILE);
+      const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
       const bool single = ntiles == 1;  // as in scan_by_key
       if (!single) {
         rc = zero_async(temp, need, s);
@@ -795,13 +631,13 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
                            (ranges_overlap(keys_out, kb, keys_in, kb) || ranges_overlap(keys_out, kb, values_in, vb) ||
                             ranges_overlap(values_out, vb, keys_in, kb) || ranges_overlap(values_out, vb, values_in, vb));
       if (aliased) {
-        TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(ReduceByKeyGeom<T>::BLOCK), s,
+        TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
                            static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
                            vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),
                            reinterpret_cast<uint32_t*>(temp), 0, 0);
       } else {
-        TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, false>), dim3((unsigned)ntiles), dim3(ReduceByKeyGeom<T>::BLOCK), s,
+        TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, false>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
                            static_cast<KU*>(keys_out), static_cast<T*>(values_out), num_runs_out, n, float_keys,
                            vec_ok, reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256),

@@ -184,9 +184,6 @@ __device__ inline T wave_shift_up1(const T& incl, const T id) {
 // with the non-temporal hint, which keeps it from displacing other lines in the L2 (scan and
 // by-key kernels gain 3-4 %).  The sort's scattered 4- and 8-byte stores must NOT use it: they
 // rely on the L2 to merge the pieces of a line written by different waves (measured 25 % slower).
-#ifndef TCD_NT
-#define TCD_NT 3  // bit 0: stores, bit 1: loads
-#endif
 typedef unsigned int tcd_v4u __attribute__((ext_vector_type(4)));
 // The same 16 bytes at ANY address in global memory: gfx950 under the HSA ABI runs with unaligned
 // global access enabled, and the compiler emits the one 128-bit instruction for this type as it
@@ -198,8 +195,7 @@ template <class V, class E>
 __device__ inline V load16(const E* p) {
   static_assert(sizeof(V) == 16, "16-byte vector");
   tcd_v4u r;
-  if (TCD_NT & 2) r = __builtin_nontemporal_load(reinterpret_cast<const tcd_v4u_anywhere*>(p));
-  else r = *reinterpret_cast<const tcd_v4u_anywhere*>(p);
+  r = __builtin_nontemporal_load(reinterpret_cast<const tcd_v4u_anywhere*>(p));
   V v;
   __builtin_memcpy(&v, &r, 16);
   return v;
@@ -209,8 +205,7 @@ __device__ inline void store16(E* p, const V& v) {
   static_assert(sizeof(V) == 16, "16-byte vector");
   tcd_v4u r;
   __builtin_memcpy(&r, &v, 16);
-  if (TCD_NT & 1) __builtin_nontemporal_store(r, reinterpret_cast<tcd_v4u_anywhere*>(p));
-  else *reinterpret_cast<tcd_v4u_anywhere*>(p) = r;
+  __builtin_nontemporal_store(r, reinterpret_cast<tcd_v4u_anywhere*>(p));
 }
 
 // ---------------------------------------------------------------------------------------

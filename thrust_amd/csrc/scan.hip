@@ -177,17 +177,11 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 
 template <class T>
 struct ScanConfig {
-#ifndef TCD_SCAN_BLOCK
-#define TCD_SCAN_BLOCK 512
-#endif
-#ifndef TCD_SCAN_CHUNKS
-#define TCD_SCAN_CHUNKS 16
-#endif
   // 256 bytes per thread for 4- and 8-byte elements (128 KiB tiles: fewer tickets and look-backs
   // per byte; measured best on MI355X: 64 KiB tiles are 10 % slower, 192 KiB tiles 3 %); fewer
   // chunks for narrow types, which hold one element per register.
-  static constexpr int BLOCK = TCD_SCAN_BLOCK;
-  static constexpr int CHUNKS = sizeof(T) >= 4 ? TCD_SCAN_CHUNKS : (sizeof(T) == 2 ? 8 : 4);
+  static constexpr int BLOCK = 512;
+  static constexpr int CHUNKS = sizeof(T) >= 4 ? 16 : (sizeof(T) == 2 ? 8 : 4);
   static constexpr int64_t TILE = (int64_t)BLOCK * (16 / sizeof(T)) * CHUNKS;
   using P = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
 };

@@ -39,10 +39,7 @@ struct DescWord {
   __device__ static uint32_t status(D w) { return (uint32_t)(w >> kShift); }
   __device__ static uint32_t count(D w) { return (uint32_t)(w & kCountMask); }
 };
-#ifndef TCD_SORT_LOOKW
-#define TCD_SORT_LOOKW 8
-#endif
-constexpr int kLookW = TCD_SORT_LOOKW;  // look-back descriptors loaded per round trip
+constexpr int kLookW = 8;  // look-back descriptors loaded per round trip
 
 template <int BYTES>
 struct uint_of;
@@ -86,9 +83,6 @@ __device__ __host__ inline U decode_key(U e, U xor_mask) {
 // over the LDS banks whatever the keys are (random, sorted, constant) instead of meeting on
 // the few banks their digits select.  64 KiB per workgroup: 16 copies for 4-byte keys, 8 for
 // 8-byte keys, 32 for narrower ones.
-#ifndef TCD_SORT_HIST_UNROLL
-#define TCD_SORT_HIST_UNROLL 8  // 128-bit loads in flight per thread
-#endif
 constexpr int kHistThreads = 512;
 template <class U>
 struct RadixHistGeom {
@@ -102,7 +96,7 @@ __global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const U* __res
   constexpr int P = RadixHistGeom<U>::P;
   constexpr int COPIES = RadixHistGeom<U>::COPIES;
   constexpr int VEC = 16 / sizeof(U);
-  constexpr int UNROLL = TCD_SORT_HIST_UNROLL;
+  constexpr int UNROLL = 8;  // 128-bit loads in flight per thread
   __shared__ uint32_t h[P * kRadix * COPIES];
   const int tid = threadIdx.x;
   for (int i = tid; i < P * kRadix * COPIES; i += kHistThreads) h[i] = 0;
@@ -493,6 +487,10 @@ __global__ __launch_bounds__(kTileSortThreads) void tile_sort_kernel(U* keys, vo
       if (VB) s_vals[pos] = v[i];
     }
     __syncthreads();
+    // The next pass overwrites s_keys / s_vals only after three more barriers, and it uses every
+    // k[i] read here as the address of its ranking atomic before the first of them: a read of
+    // this pass cannot be outstanding when its source is rewritten.  (v[i] is read by the same
+    // instructions' neighbours and the LDS returns a wavefront's reads in order.)
 #pragma unroll
     for (int i = 0; i < IPT; i++) {
       k[i] = s_keys[slab + i * kWave];
@@ -604,50 +602,19 @@ struct SortConfig {
   // with the tile) and longer per-digit runs write fuller cache lines, so tiles are as large as
   // LDS and registers allow: one 1024-thread workgroup per CU with up to 128 VGPRs and
   // 120-155 KiB of LDS (32768 keys of up to 4 bytes, with or without values; 18432 wider ones).
-#ifndef TCD_SORT_SMALL_IPT
-#define TCD_SORT_SMALL_IPT 16
-#endif
-#ifndef TCD_SORT_A_IPT
-#define TCD_SORT_A_IPT 32
-#endif
-#ifndef TCD_SORT_A_WPE
-#define TCD_SORT_A_WPE 4
-#endif
-#ifndef TCD_SORT_P_IPT
-#define TCD_SORT_P_IPT 32
-#endif
-#ifndef TCD_SORT_P_WPE
-#define TCD_SORT_P_WPE 4
-#endif
-#ifndef TCD_SORT_B_IPT
-#define TCD_SORT_B_IPT 18
-#endif
-#ifndef TCD_SORT_B_WPE
-#define TCD_SORT_B_WPE 4
-#endif
-#ifndef TCD_SORT_C_IPT
-#define TCD_SORT_C_IPT 18
-#endif
-#ifndef TCD_SORT_C_WPE
-#define TCD_SORT_C_WPE 4
-#endif
   static constexpr int ELEM = (int)sizeof(U) > VB ? (int)sizeof(U) : VB;
   static constexpr int CLASS = ELEM <= 4 ? (VB == 0 ? 0 : 1) : (VB == 0 ? 2 : 3);  // A, P, B, C
   // Inputs too small to give every CU a few of those tiles use 512 x 16 tiles instead.
   static constexpr int BLOCK = SMALL ? 512 : 1024;
-  static constexpr int IPT = SMALL ? TCD_SORT_SMALL_IPT
-                                   : CLASS == 0 ? TCD_SORT_A_IPT : CLASS == 1 ? TCD_SORT_P_IPT : CLASS == 2 ? TCD_SORT_B_IPT : TCD_SORT_C_IPT;
+  static constexpr int IPT = SMALL ? 16 : (CLASS <= 1 ? 32 : 18);
   static constexpr int TILE = BLOCK * IPT;
   // wavefronts per SIMD the register allocation aims for
-  static constexpr int WPE = SMALL ? 4 : CLASS == 0 ? TCD_SORT_A_WPE : CLASS == 1 ? TCD_SORT_P_WPE : CLASS == 2 ? TCD_SORT_B_WPE : TCD_SORT_C_WPE;
+  static constexpr int WPE = 4;
 };
 // Below this many items the small tiles are faster (measured crossover: 2^21 keys, 2^22 pairs).
-#ifndef TCD_SORT_SMALL_LOG2N
-#define TCD_SORT_SMALL_LOG2N 21
-#endif
 // positions, digit counts and their prefix sums are 32-bit
 constexpr int64_t kSortMaxN = (int64_t(1) << 32) - 1;
-constexpr int64_t small_sort_limit(int value_bytes) { return int64_t(1) << (TCD_SORT_SMALL_LOG2N + (value_bytes ? 1 : 0)); }
+constexpr int64_t small_sort_limit(int value_bytes) { return int64_t(1) << (21 + (value_bytes ? 1 : 0)); }
 
 struct SortPlan {
   size_t keys_alt, vals_alt, hist, tickets, desc, total;
