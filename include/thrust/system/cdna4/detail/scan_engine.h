@@ -15,7 +15,8 @@
 //     upto   = before (+) load(i).
 // No identity element is needed and combine is never called with swapped arguments.
 //
-// A tile is 256 threads x ITEMS consecutive elements per thread.  Tiles take their index from a
+// A tile is 512 threads x ITEMS consecutive elements per thread (read and written in wavefront-
+// contiguous pieces and reordered through LDS).  Tiles take their index from a
 // ticket counter, so every tile a waiting tile looks back at has started and the wait ends.  A
 // tile descriptor is NW 64-bit atoms, one per 32-bit word of the accumulator, each (status << 32
 // | word), written and read with relaxed agent-scope atomics: a reader that finds the same status
@@ -34,7 +35,7 @@
 
 namespace thrust { namespace system { namespace cdna4 { namespace detail { namespace generic {
 
-constexpr int kScanBlock = 256;
+constexpr int kScanBlock = 512;
 constexpr unsigned kScanSpinLimit = 1u << 22;
 constexpr int scan_items(std::size_t acc_bytes) { return acc_bytes <= 4 ? 16 : acc_bytes <= 8 ? 8 : acc_bytes <= 16 ? 4 : 2; }
 
@@ -65,6 +66,25 @@ struct scan_desc {
   }
 };
 
+// An accumulator from `d` lanes below (undefined in lanes < d), word by word.
+template <class Acc>
+__device__ inline Acc shfl_up_acc(const Acc& a, int d) {
+  constexpr int NW = (int)((sizeof(Acc) + 3) / 4);
+  unsigned w[NW] = {};
+  __builtin_memcpy(w, &a, sizeof(Acc));
+#pragma unroll
+  for (int k = 0; k < NW; k++) w[k] = __shfl_up(w[k], (unsigned)d, 64);
+  Acc r;
+  __builtin_memcpy(&r, w, sizeof(Acc));
+  return r;
+}
+
+// Slot of element e of a tile in the staging buffer: one slot of padding after every ITEMS, so
+// that both the striped order (consecutive lanes, consecutive elements) and the blocked order
+// (consecutive lanes, ITEMS elements apart) spread over the LDS banks.
+template <int ITEMS>
+__device__ inline int staged(int e) { return e + e / ITEMS; }
+
 // words[0, tiles * NW) are the descriptors, words[tiles * NW] is the ticket counter
 template <class Op>
 __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n, Op op, unsigned long long* words, std::int64_t tiles) {
@@ -72,13 +92,21 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
   typedef scan_desc<Acc> Desc;
   constexpr int ITEMS = scan_items(sizeof(Acc));
   constexpr int TILE = kScanBlock * ITEMS;
-  __shared__ typename std::aligned_storage<sizeof(Acc), alignof(Acc)>::type raw_agg[kScanBlock], raw_look[64], raw_prefix;
+  constexpr int NWAVES = kScanBlock / 64;
+  // Global memory is touched in striped order (thread t, step j: element j * 512 + t of the tile,
+  // so a wavefront's access is one contiguous piece) while the scan wants every thread to own
+  // ITEMS consecutive elements: loaded accumulators and results change order through LDS.
+  // Accumulators too large for that buffer are loaded and stored in the threads' own order.
+  constexpr bool kStaged = sizeof(Acc) * (TILE + TILE / ITEMS) <= 40 * 1024;
+  typedef typename std::aligned_storage<sizeof(Acc), alignof(Acc)>::type Raw;
+  __shared__ Raw raw_stage[kStaged ? TILE + TILE / ITEMS : 1], raw_wave[NWAVES], raw_look[64], raw_prefix;
   __shared__ unsigned long long s_tile;
   __shared__ int s_has_prefix;
-  Acc* s_agg = reinterpret_cast<Acc*>(raw_agg);    // inclusive aggregate of threads 0..t of the tile
+  Acc* s_stage = reinterpret_cast<Acc*>(raw_stage);
+  Acc* s_wave = reinterpret_cast<Acc*>(raw_wave);  // inclusive aggregate of each wavefront's threads
   Acc* s_look = reinterpret_cast<Acc*>(raw_look);  // one look-back window
   Acc* s_prefix = reinterpret_cast<Acc*>(&raw_prefix);
-  const int tid = threadIdx.x, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   if (tid == 0) s_tile = __hip_atomic_fetch_add(&words[tiles * Desc::NW], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
@@ -88,14 +116,29 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
   const std::int64_t left = n - base;
   const int count = left >= ITEMS ? ITEMS : left > 0 ? (int)left : 0;  // this thread's elements
   const std::int64_t tile_left = n - tile_base;                         // >= 1: tile < tiles
-  const int nvalid = tile_left >= TILE ? kScanBlock : (int)((tile_left + ITEMS - 1) / ITEMS);  // threads with elements
+  const bool whole = tile_left >= TILE;
+  const int nvalid = whole ? kScanBlock : (int)((tile_left + ITEMS - 1) / ITEMS);  // threads with elements
+  const int tile_count = whole ? TILE : (int)tile_left;
 
-  // every thread loads (the last element where it has none of its own) so that the loads stay
-  // independent of each other; then the inclusive scan of the thread's own elements
+  // every thread loads ITEMS times (the last element where the tile has no more) so that the
+  // loads stay independent of each other
   Acc x[ITEMS];
-  if (tile_left >= TILE) {
+  if constexpr (kStaged) {
+    if (whole) {
 #pragma unroll
-    for (int j = 0; j < ITEMS; j++) x[j] = op.load(base + j);
+      for (int j = 0; j < ITEMS; j++) x[j] = op.load(tile_base + j * kScanBlock + tid);
+    } else {
+#pragma unroll
+      for (int j = 0; j < ITEMS; j++) {
+        const std::int64_t i = tile_base + j * kScanBlock + tid;
+        x[j] = op.load(i < n ? i : n - 1);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < ITEMS; j++) s_stage[staged<ITEMS>(j * kScanBlock + tid)] = x[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < ITEMS; j++) x[j] = s_stage[staged<ITEMS>(tid * ITEMS + j)];
   } else {
 #pragma unroll
     for (int j = 0; j < ITEMS; j++) {
@@ -103,26 +146,33 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
       x[j] = op.load(i < n ? i : n - 1);
     }
   }
+  // inclusive scan of the thread's own elements (x is only ever indexed by unrolled constants, so
+  // that it stays in registers)
+  Acc incl = x[0];
 #pragma unroll
   for (int j = 1; j < ITEMS; j++)
-    if (j < count) x[j] = op.combine(x[j - 1], x[j]);
+    if (j < count) {
+      x[j] = op.combine(x[j - 1], x[j]);
+      incl = x[j];
+    }
 
-  // inclusive scan of the threads' aggregates through LDS; threads without elements are a suffix
-  // of the tile and stay out of it
-  if (count > 0) s_agg[tid] = x[count - 1];
-  __syncthreads();
+  // inclusive scan of the threads' aggregates within each wavefront; threads without elements are
+  // a suffix of the tile and stay out of it (no identity element is assumed)
+  const bool valid = tid < nvalid;
 #pragma unroll
-  for (int d = 1; d < kScanBlock; d <<= 1) {
-    const bool take = tid >= d && tid < nvalid;
-    Acc merged;
-    if (take) merged = op.combine(s_agg[tid - d], s_agg[tid]);
-    __syncthreads();
-    if (take) s_agg[tid] = merged;
-    __syncthreads();
+  for (int d = 1; d < 64; d <<= 1) {
+    const Acc up = shfl_up_acc(incl, d);
+    if (valid && lane >= d) incl = op.combine(up, incl);
   }
+  const Acc lane_before = shfl_up_acc(incl, 1);  // aggregate of the wavefront's earlier threads (lane > 0)
+  const int last_valid = nvalid - 1;             // >= 0
+  if (valid && (lane == 63 || tid == last_valid)) s_wave[wave] = incl;
+  __syncthreads();
+  const int nwaves_valid = (last_valid >> 6) + 1;
 
-  if (tid < 64) {  // wavefront 0: publish, look back, publish again
-    const Acc tile_agg = s_agg[nvalid - 1];
+  if (wave == 0) {  // wavefront 0: publish, look back, publish again
+    Acc tile_agg = s_wave[0];
+    for (int w = 1; w < nwaves_valid; w++) tile_agg = op.combine(tile_agg, s_wave[w]);
     bool has_prefix = false;  // meaningful in lane 0
     Acc prefix = tile_agg;    // placeholder until has_prefix
     if (tile > 0) {
@@ -175,14 +225,40 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
   }
   __syncthreads();
 
-  if (count > 0) {
-    const bool tile_has = s_has_prefix != 0;
-    bool has_before = tile_has || tid > 0;
-    Acc before = x[0];  // placeholder until has_before
-    if (tid > 0) before = tile_has ? op.combine(*s_prefix, s_agg[tid - 1]) : s_agg[tid - 1];
-    else if (tile_has) before = *s_prefix;
-    const Acc thread_before = before;
-    const bool thread_has = has_before;
+  // everything before the thread's first element: tile prefix, earlier wavefronts, earlier lanes
+  const bool tile_has = s_has_prefix != 0;
+  bool thread_has = tile_has;
+  Acc thread_before = x[0];  // placeholder until thread_has
+  if (tile_has) thread_before = *s_prefix;
+  for (int w = 0; w < wave; w++) {
+    thread_before = thread_has ? op.combine(thread_before, s_wave[w]) : s_wave[w];
+    thread_has = true;
+  }
+  if (lane > 0) {
+    thread_before = thread_has ? op.combine(thread_before, lane_before) : lane_before;
+    thread_has = true;
+  }
+
+  if constexpr (kStaged) {
+    // results go to the staging buffer in the threads' order and leave it in striped order; the
+    // value before element e is the result of element e - 1 (the tile's prefix for e = 0)
+#pragma unroll
+    for (int j = 0; j < ITEMS; j++)
+      if (j < count) s_stage[staged<ITEMS>(tid * ITEMS + j)] = thread_has ? op.combine(thread_before, x[j]) : x[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < ITEMS; j++) {
+      const int e = j * kScanBlock + tid;
+      if (e < tile_count) {
+        const Acc upto = s_stage[staged<ITEMS>(e)];
+        const bool has_before = e > 0 || tile_has;
+        const Acc before = e > 0 ? s_stage[staged<ITEMS>(e - 1)] : (tile_has ? *s_prefix : upto);
+        op.store(tile_base + e, has_before, before, upto);
+      }
+    }
+  } else if (count > 0) {
+    bool has_before = thread_has;
+    Acc before = thread_before;
 #pragma unroll
     for (int j = 0; j < ITEMS; j++) {
       if (j < count) {

@@ -48,7 +48,7 @@ struct scan_by_key_body {
   // a head is an element whose key does not continue its predecessor's segment
   // (thrust/system/detail/sequential/scan_by_key.h:63-83: pred(previous key, key))
   __device__ acc load(std::int64_t i) const {
-    const bool head = i == 0 || !pred(keys[i - 1], keys[i]);
+    const bool head = (i == 0) | !pred(keys[i > 0 ? i - 1 : 0], keys[i]);  // no branch around the loads
     return acc{head ? 1u : 0u, static_cast<V>(vals[i])};
   }
   __device__ acc combine(const acc& a, const acc& b) const {
@@ -59,7 +59,7 @@ struct scan_by_key_body {
       out[i] = upto.v;
     } else {
       // init restarts at every head (sequential/scan_by_key.h:95-140)
-      const bool head = i == 0 || !pred(keys[i - 1], keys[i]);
+      const bool head = (i == 0) | !pred(keys[i > 0 ? i - 1 : 0], keys[i]);  // no branch around the loads
       out[i] = (head || !has_before) ? init : static_cast<V>(op(init, before.v));
     }
   }
@@ -70,7 +70,7 @@ struct reduce_by_key_body {
   typedef seg_acc<C, V> acc;
   KIn keys; VIn vals; KOut kout; VOut vout; long long* num_runs; std::int64_t n; Pred pred; Op op;
   __device__ acc load(std::int64_t i) const {
-    const bool head = i == 0 || !pred(keys[i - 1], keys[i]);
+    const bool head = (i == 0) | !pred(keys[i > 0 ? i - 1 : 0], keys[i]);  // no branch around the loads
     return acc{(C)(head ? 1 : 0), static_cast<V>(vals[i])};
   }
   __device__ acc combine(const acc& a, const acc& b) const {

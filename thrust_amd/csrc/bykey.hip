@@ -232,7 +232,6 @@ struct SegTile {
     }
     base = tile * G::TILE;
     full = vec_ok && (base + G::TILE < n);
-    const int64_t i0 = first_index();
 
     if (full) {
       const int64_t w0 = base + (int64_t)wave * (kWave * VEC);
@@ -244,10 +243,12 @@ struct SegTile {
       const int64_t w0 = base + (int64_t)wave * (kWave * VEC);
       wave_load_blocked_partial<VEC>(keys + w0, key, xbuf, lane, n - w0);
       wave_load_blocked_partial<VEC>(vals + w0, val, xbuf, lane, n - w0);
+      const int64_t i0 = first_index();
 #pragma unroll
       for (int j = 0; j < VEC; j++)
         if (i0 + j >= n) val[j] = id;
     } else {
+      const int64_t i0 = first_index();
 #pragma unroll
       for (int j = 0; j < VEC; j++) {
         const int64_t idx = i0 + j;
@@ -258,6 +259,9 @@ struct SegTile {
     // the key before a thread's elements is the last key of the lane below (its elements precede
     // these in memory); only lane 0 of each wave fetches it from memory
     using KW = typename std::conditional<(sizeof(KU) < 4), uint32_t, KU>::type;
+    // (the index is formed here, after the loads: held across them it costs the by-key kernels
+    // their register budget)
+    const int64_t i0 = first_index();
     KU first = KU(0);
     if (lane == 0 && i0 > 0 && i0 < n) first = keys[i0 - 1];
     const KU prev = (KU)wave_shift_up1((KW)key[VEC - 1], (KW)first);
