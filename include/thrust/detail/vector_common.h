@@ -2,6 +2,7 @@
 // As in the reference, whose vector headers pull in most of the library, a translation unit that
 // includes a vector header can use the common algorithms and iterators without naming their headers.
 #include <thrust/advance.h>
+#include <thrust/detail/minmax.h>
 #include <thrust/copy.h>
 #include <thrust/distance.h>
 #include <thrust/equal.h>

@@ -184,6 +184,19 @@ host_vector<T, A>::host_vector(const device_vector<T, DA>& d) : base(d.size()) {
   }
 }
 template <class T, class A>
+template <class U>
+host_vector<T, A>::host_vector(device_ptr<U> first, device_ptr<U> last) : base((std::size_t)(last - first)) {
+  const std::size_t n = (std::size_t)(last - first);
+  if (!n) return;
+  if (std::is_same<typename std::remove_const<U>::type, T>::value) {
+    system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_dtoh(this->data(), first.get(), n * sizeof(T), nullptr), "copy to host");
+    system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "copy to host");
+  } else {  // another element type: through a host copy of the source, converted element by element
+    host_vector<typename std::remove_const<U>::type> same(first, last);
+    for (std::size_t i = 0; i < n; i++) (*this)[i] = (T)same[i];
+  }
+}
+template <class T, class A>
 template <class DA>
 host_vector<T, A>& host_vector<T, A>::operator=(const device_vector<T, DA>& d) {
   host_vector tmp(d);

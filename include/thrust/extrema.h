@@ -6,16 +6,13 @@
 #include <thrust/detail/iterator_util.h>
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
+#include <thrust/detail/minmax.h>
 #include <thrust/pair.h>
 #include <thrust/system/cdna4/detail/index_algorithms.h>
 
 #include <thrust/reduce.h>
 #include <thrust/transform.h>
 namespace thrust {
-template <class T> THRUST_CDNA4_HD constexpr const T& min(const T& a, const T& b) { return b < a ? b : a; }
-template <class T> THRUST_CDNA4_HD constexpr const T& max(const T& a, const T& b) { return a < b ? b : a; }
-template <class T, class Compare> THRUST_CDNA4_HD constexpr const T& min(const T& a, const T& b, Compare comp) { return comp(b, a) ? b : a; }
-template <class T, class Compare> THRUST_CDNA4_HD constexpr const T& max(const T& a, const T& b, Compare comp) { return comp(a, b) ? b : a; }
 
 namespace detail {
 // position -1: no element yet

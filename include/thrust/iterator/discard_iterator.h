@@ -10,7 +10,10 @@ struct discard_proxy {
   template <class T> THRUST_CDNA4_HD const discard_proxy& operator=(const T&) const { return *this; }
 };
 }  // namespace detail
-class discard_iterator : public detail::fancy_base<discard_iterator, detail::discard_proxy> {
+// (the System parameter of the reference's template is accepted and ignored: the iterator holds
+// no data, so it serves every system)
+template <class System = use_default>
+class discard_iterator : public detail::fancy_base<discard_iterator<System>, detail::discard_proxy> {
  public:
   typedef detail::discard_proxy value_type;
   typedef detail::discard_proxy reference;
@@ -21,8 +24,8 @@ class discard_iterator : public detail::fancy_base<discard_iterator, detail::dis
  private:
   std::ptrdiff_t pos_;
 };
-THRUST_CDNA4_HD inline discard_iterator make_discard_iterator(std::ptrdiff_t pos = 0) { return discard_iterator(pos); }
+THRUST_CDNA4_HD inline discard_iterator<> make_discard_iterator(std::ptrdiff_t pos = 0) { return discard_iterator<>(pos); }
 namespace system { namespace cdna4 { namespace detail {
-template <> struct is_device_iterator<thrust::discard_iterator> { static constexpr bool value = true; };
+template <class S> struct is_device_iterator<thrust::discard_iterator<S>> { static constexpr bool value = true; };
 }}}
 }  // namespace thrust

@@ -1,4 +1,87 @@
-// <thrust/merge.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/merge.h> is not provided by the cdna4 device system"
+// thrust::merge / merge_by_key (thrust/merge.h): stable merge of two sorted ranges — of equivalent
+// elements those of the first range come first (testing/merge.cu, merge_by_key.cu).  Device ranges
+// run the merge-path kernels of system/cdna4/detail/merge_engine.h (compiled by hipcc); host ranges
+// the sequential algorithm.
+#pragma once
+#include <algorithm>
+#include <thrust/detail/iterator_util.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/pair.h>
+#include <thrust/system/cdna4/detail/generic_algorithms.h>
+#if defined(__HIPCC__)
+#include <thrust/system/cdna4/detail/merge_engine.h>
+#endif
+
+namespace thrust {
+// ---- device
+template <class D, class In1, class In2, class Out, class Comp>
+Out merge(const system::cdna4::execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  THRUST_CDNA4_NEEDS_HIPCC(Comp);
+  const std::int64_t na = (std::int64_t)(last1 - first1), nb = (std::int64_t)(last2 - first2);
+#if defined(__HIPCC__)
+  namespace m = system::cdna4::detail::merge2;
+  m::merge<false>(system::cdna4::detail::stream_of(exec.derived()), detail::unwrap(first1), na, detail::unwrap(first2), nb, system::cdna4::detail::no_values(),
+                  system::cdna4::detail::no_values(), detail::unwrap(result), system::cdna4::detail::no_values(), comp);
+  system::cdna4::detail::synchronize_optional(exec.derived(), "merge: failed to synchronize");
+#endif
+  return result + (na + nb);
+}
+template <class D, class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp>
+pair<KOut, VOut> merge_by_key(const system::cdna4::execution_policy<D>& exec, K1 kfirst1, K1 klast1, K2 kfirst2, K2 klast2, V1 vfirst1,
+                              V2 vfirst2, KOut kresult, VOut vresult, Comp comp) {
+  THRUST_CDNA4_NEEDS_HIPCC(Comp);
+  const std::int64_t na = (std::int64_t)(klast1 - kfirst1), nb = (std::int64_t)(klast2 - kfirst2);
+#if defined(__HIPCC__)
+  namespace m = system::cdna4::detail::merge2;
+  m::merge<true>(system::cdna4::detail::stream_of(exec.derived()), detail::unwrap(kfirst1), na, detail::unwrap(kfirst2), nb,
+                 detail::unwrap(vfirst1), detail::unwrap(vfirst2), detail::unwrap(kresult), detail::unwrap(vresult), comp);
+  system::cdna4::detail::synchronize_optional(exec.derived(), "merge_by_key: failed to synchronize");
+#else
+  (void)vfirst1; (void)vfirst2;
+#endif
+  return pair<KOut, VOut>(kresult + (na + nb), vresult + (na + nb));
+}
+// ---- host
+template <class In1, class In2, class Out, class Comp>
+Out merge(const system::cpp::detail::par_t&, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  return std::merge(first1, last1, first2, last2, result, comp);
+}
+template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp>
+pair<KOut, VOut> merge_by_key(const system::cpp::detail::par_t&, K1 kfirst1, K1 klast1, K2 kfirst2, K2 klast2, V1 vfirst1, V2 vfirst2,
+                              KOut kresult, VOut vresult, Comp comp) {
+  // thrust/system/detail/sequential/merge.inl: take from the second range only when its key is strictly before
+  while (kfirst1 != klast1 && kfirst2 != klast2) {
+    if (comp(*kfirst2, *kfirst1)) { *kresult = *kfirst2; *vresult = *vfirst2; ++kfirst2; ++vfirst2; }
+    else { *kresult = *kfirst1; *vresult = *vfirst1; ++kfirst1; ++vfirst1; }
+    ++kresult; ++vresult;
+  }
+  for (; kfirst1 != klast1; ++kfirst1, ++vfirst1, ++kresult, ++vresult) { *kresult = *kfirst1; *vresult = *vfirst1; }
+  for (; kfirst2 != klast2; ++kfirst2, ++vfirst2, ++kresult, ++vresult) { *kresult = *kfirst2; *vresult = *vfirst2; }
+  return pair<KOut, VOut>(kresult, vresult);
+}
+// ---- default comparison, and the forms without a policy
+template <class Policy, class In1, class In2, class Out, detail::enable_if_policy<Policy> = 0>
+Out merge(const Policy& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(exec, f1, l1, f2, l2, r, less<typename detail::value_of<In1>::type>()); }
+template <class In1, class In2, class Out, class Comp, detail::enable_if_device<In1> = 0>
+Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp c) { return merge(device, f1, l1, f2, l2, r, c); }
+template <class In1, class In2, class Out, class Comp, detail::enable_if_host<In1> = 0>
+Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp c) { return merge(host, f1, l1, f2, l2, r, c); }
+template <class In1, class In2, class Out, detail::enable_if_device<In1> = 0>
+Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(device, f1, l1, f2, l2, r); }
+template <class In1, class In2, class Out, detail::enable_if_host<In1> = 0>
+Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(host, f1, l1, f2, l2, r); }
+
+template <class Policy, class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_policy<Policy> = 0>
+pair<KOut, VOut> merge_by_key(const Policy& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) {
+  return merge_by_key(exec, kf1, kl1, kf2, kl2, v1, v2, kr, vr, less<typename detail::value_of<K1>::type>());
+}
+template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp, detail::enable_if_device<K1> = 0>
+pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp c) { return merge_by_key(device, kf1, kl1, kf2, kl2, v1, v2, kr, vr, c); }
+template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp, detail::enable_if_host<K1> = 0>
+pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp c) { return merge_by_key(host, kf1, kl1, kf2, kl2, v1, v2, kr, vr, c); }
+template <class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_device<K1> = 0>
+pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return merge_by_key(device, kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
+template <class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_host<K1> = 0>
+pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return merge_by_key(host, kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
+}  // namespace thrust

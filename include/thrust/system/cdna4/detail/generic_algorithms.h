@@ -23,6 +23,12 @@ template <class T> struct needs_hipcc { static constexpr bool value = sizeof(T) 
                 "translation unit with hipcc --offload-arch=gfx950")
 #endif
 
+// Stands for "no values" where keys-only and by-key forms share an implementation (merge, set
+// operations): indexable, never read for its content.
+struct no_values {
+  THRUST_CDNA4_HD char operator[](std::int64_t) const { return 0; }
+};
+
 // In the bodies below an "iterator" is whatever detail::unwrap gives a kernel: a raw pointer or a
 // fancy iterator over raw pointers, indexable on the device.
 #if defined(__HIPCC__)

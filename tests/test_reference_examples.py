@@ -20,10 +20,7 @@ with open(os.path.join(ROOT, "tests", "golden", "example_outputs.json")) as f:
 
 # examples this device system runs (all of the reference's examples/ but the ones named below)
 NOT_BUILT = {
-    "discrete_voronoi": "needs examples/include/timer.h of the CUDA runtime",
-    "mr_basic": "disjoint / synchronized pool resources are not provided",
-    "set_operations": "merge and the set operations are not provided",
-    "sparse_vector": "merge_by_key and the set operations are not provided",
+    "mr_basic": "disjoint / synchronized pool resources and the polymorphic adaptor are not provided",
 }
 EXAMPLES = sorted(set(GOLDEN) - set(NOT_BUILT))
 
@@ -91,7 +88,7 @@ def test_reference_examples_compile_unchanged():
 def test_a_header_that_is_not_provided_says_so(tmp_path):
     # never a silent fall-through to another Thrust on the include path (/opt/rocm/include/thrust)
     src = tmp_path / "t.cu"
-    src.write_text("#include <thrust/set_operations.h>\nint main() { return 0; }\n")
+    src.write_text("#include <thrust/shuffle.h>\nint main() { return 0; }\n")
     r = subprocess.run(["/opt/rocm/bin/hipcc", "-x", "hip", "--offload-arch=gfx950", "-fsyntax-only", "-I",
                         os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
     assert r.returncode != 0
