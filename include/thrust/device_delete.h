@@ -1,4 +1,15 @@
-// <thrust/device_delete.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/device_delete.h> is not provided by the cdna4 device system"
+// thrust::device_delete (thrust/device_delete.h): the partner of device_new — destroys n objects
+// (a no-op for the trivially destructible types device storage holds) and frees their storage.
+#pragma once
+#include <cstddef>
+#include <type_traits>
+#include <thrust/device_free.h>
+#include <thrust/device_ptr.h>
+namespace thrust {
+template <class T>
+inline void device_delete(device_ptr<T> ptr, const std::size_t n = 1) {
+  static_assert(std::is_trivially_destructible<T>::value, "cdna4: objects in device memory must be trivially destructible");
+  (void)n;
+  device_free(ptr);
+}
+}  // namespace thrust

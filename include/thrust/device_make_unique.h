@@ -1,4 +1,16 @@
-// <thrust/device_make_unique.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/device_make_unique.h> is not provided by the cdna4 device system"
+// thrust::device_make_unique (thrust/device_make_unique.h): one T(args...) in device memory from
+// thrust::device_allocator, owned by a std::unique_ptr that hands the storage back.
+#pragma once
+#include <utility>
+#include <thrust/allocate_unique.h>
+#include <thrust/device_allocator.h>
+#include <thrust/device_new.h>
+#include <thrust/device_ptr.h>
+namespace thrust {
+template <class T, class... Args>
+auto device_make_unique(Args&&... args) -> decltype(uninitialized_allocate_unique<T>(device_allocator<T>{})) {
+  auto p = uninitialized_allocate_unique<T>(device_allocator<T>{});
+  device_new<T>(device_ptr<void>(static_cast<void*>(p.get().get())), T(std::forward<Args>(args)...));
+  return p;
+}
+}  // namespace thrust

@@ -54,7 +54,13 @@ class device_ptr {
   typedef system::cdna4::tag system_tag;
 
   THRUST_CDNA4_HD device_ptr() : p_(nullptr) {}
+  THRUST_CDNA4_HD device_ptr(std::nullptr_t) : p_(nullptr) {}  // a NullablePointer, as std::unique_ptr and allocators need
   THRUST_CDNA4_HD explicit device_ptr(T* p) : p_(p) {}
+  THRUST_CDNA4_HD explicit operator bool() const { return p_ != nullptr; }
+  THRUST_CDNA4_HD friend bool operator==(device_ptr a, std::nullptr_t) { return a.p_ == nullptr; }
+  THRUST_CDNA4_HD friend bool operator==(std::nullptr_t, device_ptr a) { return a.p_ == nullptr; }
+  THRUST_CDNA4_HD friend bool operator!=(device_ptr a, std::nullptr_t) { return a.p_ != nullptr; }
+  THRUST_CDNA4_HD friend bool operator!=(std::nullptr_t, device_ptr a) { return a.p_ != nullptr; }
   template <class U, class = typename std::enable_if<std::is_convertible<U*, T*>::value>::type>
   THRUST_CDNA4_HD device_ptr(const device_ptr<U>& o) : p_(o.get()) {}
   THRUST_CDNA4_HD T* get() const { return p_; }

@@ -1,4 +1,4 @@
-// <thrust/mr/universal_memory_resource.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/mr/universal_memory_resource.h> is not provided by the cdna4 device system"
+// thrust/mr/universal_memory_resource.h: thrust::universal_memory_resource and
+// thrust::universal_host_pinned_memory_resource are the cdna4 system's.
+#pragma once
+#include <thrust/system/cdna4/memory_resource.h>

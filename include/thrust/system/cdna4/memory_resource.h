@@ -44,6 +44,30 @@ class pool_memory_resource final : public thrust::mr::memory_resource<thrust::de
  private:
   void* stream_;
 };
+// Memory that host code and device code can both address
+// (thrust/system/cuda/memory_resource.h:118-125): managed memory, or page-locked host memory that
+// the device reaches over the bus.  Pointers are device_ptr, like every pointer of this system;
+// raw_pointer_cast of one may also be dereferenced on the host.
+template <bool HOST_PINNED>
+class universal_resource final : public thrust::mr::memory_resource<thrust::device_ptr<void>> {
+ public:
+  thrust::device_ptr<void> do_allocate(std::size_t bytes, std::size_t) override {
+    void* p = nullptr;
+    const int rc = thrust_cdna4_malloc_universal(&p, bytes, HOST_PINNED ? 1 : 0);
+    if (rc != 0) throw thrust::system::detail::bad_alloc(thrust_cdna4_error_string(rc));
+    return thrust::device_ptr<void>(p);
+  }
+  void do_deallocate(thrust::device_ptr<void> p, std::size_t, std::size_t) override {
+    detail::throw_on_error(thrust_cdna4_free_universal(p.get(), HOST_PINNED ? 1 : 0), "cdna4::universal_memory_resource: free");
+  }
+  bool do_is_equal(const thrust::mr::memory_resource<thrust::device_ptr<void>>& other) const noexcept override {
+    return dynamic_cast<const universal_resource*>(&other) != nullptr;
+  }
+};
+typedef universal_resource<false> universal_memory_resource;
+typedef universal_resource<true> universal_host_pinned_memory_resource;
 }}  // namespace system::cdna4
 typedef system::cdna4::memory_resource device_memory_resource;
+typedef system::cdna4::universal_memory_resource universal_memory_resource;
+typedef system::cdna4::universal_host_pinned_memory_resource universal_host_pinned_memory_resource;
 }  // namespace thrust

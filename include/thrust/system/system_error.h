@@ -1,4 +1,8 @@
-// <thrust/system/system_error.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/system/system_error.h> is not provided by the cdna4 device system"
+// thrust::system::system_error (thrust/system/system_error.h): the exception every failed device
+// call turns into, carrying the hip error code in the cdna4 category.
+#pragma once
+#include <thrust/system/error_code.h>
+#include <thrust/system_error.h>
+namespace thrust { namespace system {
+using ::thrust::system_error;
+}}  // namespace thrust::system

@@ -1,4 +1,27 @@
-// <thrust/type_traits/is_contiguous_iterator.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/type_traits/is_contiguous_iterator.h> is not provided by the cdna4 device system"
+// thrust::is_contiguous_iterator, proclaim_contiguous_iterator and
+// THRUST_PROCLAIM_CONTIGUOUS_ITERATOR (thrust/type_traits/is_contiguous_iterator.h): iterators
+// whose elements lie next to each other in memory — raw pointers, thrust::device_ptr, the
+// iterators of std::vector / std::string / thrust::host_vector / thrust::device_vector, and
+// whatever a user proclaims.
+#pragma once
+#include <iterator>
+#include <string>
+#include <type_traits>
+#include <vector>
+#include <thrust/device_ptr.h>
+namespace thrust {
+template <class Iterator> struct proclaim_contiguous_iterator : std::false_type {};
+#define THRUST_PROCLAIM_CONTIGUOUS_ITERATOR(Iterator) \
+  namespace thrust { template <> struct proclaim_contiguous_iterator<Iterator> : std::true_type {}; }
+namespace detail {
+template <class It> struct is_contiguous_iterator_impl : proclaim_contiguous_iterator<It> {};
+template <class T> struct is_contiguous_iterator_impl<T*> : std::true_type {};
+template <class T> struct is_contiguous_iterator_impl<thrust::device_ptr<T>> : std::true_type {};
+// libstdc++'s vector and string iterators wrap a raw pointer
+template <class P, class C> struct is_contiguous_iterator_impl<__gnu_cxx::__normal_iterator<P, C>> : std::is_pointer<P> {};
+}  // namespace detail
+template <class Iterator> struct is_contiguous_iterator : detail::is_contiguous_iterator_impl<typename std::remove_cv<Iterator>::type> {};
+#if __cplusplus >= 201402L
+template <class Iterator> constexpr bool is_contiguous_iterator_v = is_contiguous_iterator<Iterator>::value;
+#endif
+}  // namespace thrust

@@ -1,4 +1,17 @@
-// <thrust/type_traits/is_operator_plus_function_object.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/type_traits/is_operator_plus_function_object.h> is not provided by the cdna4 device system"
+// thrust::is_operator_plus_function_object (thrust/type_traits/is_operator_plus_function_object.h):
+// whether a function object is known to be operator+ (thrust::plus, std::plus).
+#pragma once
+#include <functional>
+#include <type_traits>
+#include <thrust/functional.h>
+namespace thrust {
+namespace detail {
+template <class F> struct is_operator_plus_function_object_impl : std::false_type {};
+template <class T> struct is_operator_plus_function_object_impl<thrust::plus<T>> : std::true_type {};
+template <class T> struct is_operator_plus_function_object_impl<std::plus<T>> : std::true_type {};
+}  // namespace detail
+template <class F> struct is_operator_plus_function_object : detail::is_operator_plus_function_object_impl<F> {};
+#if __cplusplus >= 201402L
+template <class F> constexpr bool is_operator_plus_function_object_v = is_operator_plus_function_object<F>::value;
+#endif
+}  // namespace thrust

@@ -1,4 +1,7 @@
-// <thrust/type_traits/remove_cvref.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/type_traits/remove_cvref.h> is not provided by the cdna4 device system"
+// thrust::remove_cvref (thrust/type_traits/remove_cvref.h).
+#pragma once
+#include <type_traits>
+namespace thrust {
+template <class T> struct remove_cvref { typedef typename std::remove_cv<typename std::remove_reference<T>::type>::type type; };
+template <class T> using remove_cvref_t = typename remove_cvref<T>::type;
+}  // namespace thrust

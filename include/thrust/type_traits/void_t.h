@@ -1,4 +1,6 @@
-// <thrust/type_traits/void_t.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/type_traits/void_t.h> is not provided by the cdna4 device system"
+// thrust::void_t (thrust/type_traits/void_t.h): maps any well-formed list of types to void.
+#pragma once
+namespace thrust {
+template <class...> struct voider { typedef void type; };
+template <class... Ts> using void_t = typename voider<Ts...>::type;
+}  // namespace thrust

@@ -1,4 +1,3 @@
-// <thrust/universal_ptr.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/universal_ptr.h> is not provided by the cdna4 device system"
+// thrust::universal_ptr (thrust/universal_ptr.h): defined with universal_allocator.
+#pragma once
+#include <thrust/universal_allocator.h>

@@ -1,4 +1,9 @@
-// <thrust/universal_vector.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/universal_vector.h> is not provided by the cdna4 device system"
+// thrust::universal_vector (thrust/universal_vector.h): a device_vector whose storage host code
+// can address too (managed memory).  The algorithms treat it as a device range;
+// raw_pointer_cast(v.data()) may be read and written on the host once device work on it is done.
+#pragma once
+#include <thrust/device_vector.h>
+#include <thrust/universal_allocator.h>
+namespace thrust {
+template <class T, class Alloc = universal_allocator<T>> using universal_vector = device_vector<T, Alloc>;
+}  // namespace thrust

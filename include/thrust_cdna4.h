@@ -213,6 +213,17 @@ int thrust_cdna4_stream_wait_event(void* stream, void* event);
  */
 int thrust_cdna4_malloc_direct(void** ptr, size_t bytes);
 int thrust_cdna4_free_direct(void* ptr);
+/*
+ * Memory addressable from host and device code alike: managed memory (host_pinned = 0;
+ * thrust/system/cuda/memory_resource.h:118-121, universal_memory_resource over cudaMallocManaged)
+ * or page-locked host memory mapped into the device's address space (host_pinned = 1; :122-125,
+ * universal_host_pinned_memory_resource over cudaMallocHost).  Free with the same flag.
+ */
+int thrust_cdna4_malloc_universal(void** ptr, size_t bytes, int host_pinned);
+int thrust_cdna4_free_universal(void* ptr, int host_pinned);
+/* The device that is current for the calling thread (cudaGetDevice in
+ * thrust/system/cuda/detail/per_device_resource.h:46-62). */
+int thrust_cdna4_get_device(int* device);
 
 /*
  * Scan, scan_by_key and reduce_by_key chain their tiles by look-back.  When the output does not

@@ -20,6 +20,7 @@
 #include <thrust/reverse.h>
 #include <thrust/scatter.h>
 #include <thrust/sequence.h>
+#include <thrust/shuffle.h>
 #include <thrust/sort.h>
 #include <thrust/swap.h>
 #include <thrust/tabulate.h>
@@ -326,5 +327,74 @@ void TestRandomOnDeviceMatchesHost() {
   ASSERT_EQUAL(d, h);
 }
 DECLARE_UNITTEST(TestRandomOnDeviceMatchesHost);
+
+// the other engines: the 10000th values the reference documents (thrust/random.h:63-84,
+// thrust/random/subtract_with_carry_engine.h:226-239), and the standard's engines where the
+// definitions coincide
+void TestRandomOtherEnginesKnownAnswers() {
+  thrust::ranlux24_base a;
+  a.discard(9999);
+  ASSERT_EQUAL((unsigned long long)a(), 7937952ull);
+  thrust::ranlux48_base b;
+  b.discard(9999);
+  ASSERT_EQUAL((unsigned long long)b(), 192113843633948ull);
+  thrust::ranlux24 c;
+  c.discard(9999);
+  ASSERT_EQUAL((unsigned long long)c(), 9901578ull);
+  thrust::ranlux48 d;
+  d.discard(9999);
+  ASSERT_EQUAL((unsigned long long)d(), 88229545517833ull);
+  thrust::taus88 e;
+  e.discard(9999);
+  ASSERT_EQUAL((unsigned long long)e(), 3535848941ull);
+  ASSERT_EQUAL((unsigned long long)thrust::taus88::max, 4294967295ull);
+  thrust::ranlux24 x(77), y(77);
+  std::ranlux24 sx(77);
+  for (int i = 0; i < 1000; i++) {
+    const unsigned v = (unsigned)x();
+    ASSERT_EQUAL(v, (unsigned)sx());  // 24-bit words: the same engine as the standard's
+    ASSERT_EQUAL(v, (unsigned)y());
+  }
+  ASSERT_TRUE(x == y);
+  y();
+  ASSERT_TRUE(x != y);
+}
+DECLARE_UNITTEST(TestRandomOtherEnginesKnownAnswers);
+
+// shuffle: a permutation, the same on host and device for the same generator state
+// (testing/shuffle.cu:326-375), and the network is a bijection (:378-405)
+void TestShuffle() {
+  for (std::size_t n : {std::size_t(0), std::size_t(1), std::size_t(2), std::size_t(10), std::size_t(16), std::size_t(17), std::size_t(1000),
+                        std::size_t(4096), std::size_t(4097), std::size_t(123457), std::size_t(1 << 20)}) {
+    thrust::host_vector<int> h(n), hs(n);
+    for (std::size_t i = 0; i < n; i++) h[i] = (int)i;
+    thrust::device_vector<int> d = h, ds(n);
+    thrust::default_random_engine gh(13), gd(13);
+    thrust::shuffle_copy(h.begin(), h.end(), hs.begin(), gh);
+    thrust::shuffle_copy(d.begin(), d.end(), ds.begin(), gd);
+    ASSERT_EQUAL(ds, hs);
+    ASSERT_TRUE(gh == gd);  // both drew the same 24 keys
+    thrust::host_vector<int> sorted = hs;
+    std::sort(sorted.begin(), sorted.end());
+    ASSERT_EQUAL(sorted, h);  // a permutation
+    if (n > 100) ASSERT_TRUE(!(hs == h));
+    thrust::shuffle(d.begin(), d.end(), gd);  // in place, with the generator's next state
+    thrust::shuffle(h.begin(), h.end(), gh);
+    ASSERT_EQUAL(d, h);
+    thrust::sort(d.begin(), d.end());
+    ASSERT_EQUAL(d, sorted);
+  }
+  thrust::default_random_engine g(3);
+  thrust::detail::feistel_bijection f(1000, g);
+  ASSERT_EQUAL(f.nearest_power_of_two(), std::uint64_t(1024));
+  std::vector<std::uint64_t> image(1024);
+  for (std::uint64_t i = 0; i < 1024; i++) image[i] = f(i);
+  std::sort(image.begin(), image.end());
+  for (std::uint64_t i = 0; i < 1024; i++) ASSERT_EQUAL(image[i], i);
+  ASSERT_EQUAL(thrust::detail::feistel_bijection(17, g).nearest_power_of_two(), std::uint64_t(32));  // testing/shuffle.cu:409-424
+  ASSERT_EQUAL(thrust::detail::feistel_bijection(32, g).nearest_power_of_two(), std::uint64_t(32));
+  ASSERT_EQUAL(thrust::detail::feistel_bijection(1, g).nearest_power_of_two(), std::uint64_t(16));
+}
+DECLARE_UNITTEST(TestShuffle);
 
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }

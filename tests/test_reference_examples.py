@@ -88,7 +88,7 @@ def test_reference_examples_compile_unchanged():
 def test_a_header_that_is_not_provided_says_so(tmp_path):
     # never a silent fall-through to another Thrust on the include path (/opt/rocm/include/thrust)
     src = tmp_path / "t.cu"
-    src.write_text("#include <thrust/shuffle.h>\nint main() { return 0; }\n")
+    src.write_text("#include <thrust/system/cuda/vector.h>\nint main() { return 0; }\n")
     r = subprocess.run(["/opt/rocm/bin/hipcc", "-x", "hip", "--offload-arch=gfx950", "-fsyntax-only", "-I",
                         os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
     assert r.returncode != 0

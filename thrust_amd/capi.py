@@ -27,6 +27,7 @@ SYMBOLS = [
     "thrust_cdna4_stream_create", "thrust_cdna4_stream_destroy", "thrust_cdna4_stream_query",
     "thrust_cdna4_event_create", "thrust_cdna4_event_destroy", "thrust_cdna4_event_record", "thrust_cdna4_event_query",
     "thrust_cdna4_stream_wait_event", "thrust_cdna4_malloc_direct", "thrust_cdna4_free_direct",
+    "thrust_cdna4_malloc_universal", "thrust_cdna4_free_universal", "thrust_cdna4_get_device",
 ]
 
 
@@ -82,6 +83,9 @@ def lib():
     L.thrust_cdna4_stream_wait_event.argtypes = [vp, vp]
     L.thrust_cdna4_malloc_direct.argtypes = [ctypes.POINTER(vp), sz]
     L.thrust_cdna4_free_direct.argtypes = [vp]
+    L.thrust_cdna4_malloc_universal.argtypes = [ctypes.POINTER(vp), sz, i32]
+    L.thrust_cdna4_free_universal.argtypes = [vp, i32]
+    L.thrust_cdna4_get_device.argtypes = [ctypes.POINTER(i32)]
     L.thrust_cdna4_set_lookback_patience.argtypes = [i32]
     L.thrust_cdna4_set_test_publish_delay.argtypes = [i32]
     L.thrust_cdna4_lookback_timeouts.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]

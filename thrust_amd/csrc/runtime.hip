@@ -439,3 +439,19 @@ extern "C" int thrust_cdna4_free_direct(void* ptr) {
   if (!ptr) return hipSuccess;
   return hipFree(ptr);
 }
+// Memory that host and device code can both address: managed memory (pages move to whoever
+// touches them) or page-locked host memory that the device reaches over the bus.
+extern "C" int thrust_cdna4_malloc_universal(void** ptr, size_t bytes, int host_pinned) {
+  if (!ptr) return hipErrorInvalidValue;
+  *ptr = nullptr;
+  if (bytes == 0) return hipSuccess;
+  return host_pinned ? hipHostMalloc(ptr, bytes, hipHostMallocDefault) : hipMallocManaged(ptr, bytes, hipMemAttachGlobal);
+}
+extern "C" int thrust_cdna4_free_universal(void* ptr, int host_pinned) {
+  if (!ptr) return hipSuccess;
+  return host_pinned ? hipHostFree(ptr) : hipFree(ptr);
+}
+extern "C" int thrust_cdna4_get_device(int* device) {
+  if (!device) return hipErrorInvalidValue;
+  return hipGetDevice(device);
+}
