@@ -101,7 +101,19 @@ template <class T> inline void device_free(device_ptr<T> p) { system::cdna4::det
 namespace system { namespace cdna4 { namespace detail {
 // Contiguous device iterators are unwrapped to raw pointers before the C ABI is called
 // (thrust/type_traits/is_contiguous_iterator.h:246-, try_unwrap_contiguous_iterator).
-template <class It> struct is_device_iterator { static constexpr bool value = false; };
+// An iterator class says which memory it walks either by a partial specialisation below or by a
+// nested typedef `thrust_system_is_device` (std::true_type / std::false_type), which is what
+// thrust::iterator_facade and iterator_adaptor define; or by an iterator_category derived from one
+// of thrust's *_device_iterator_tag types.
+struct device_category_marker {};
+template <class It, class = void> struct declares_device_iterator : std::false_type {};
+template <class It> struct declares_device_iterator<It, typename std::enable_if<It::thrust_system_is_device::value || !It::thrust_system_is_device::value>::type>
+    : It::thrust_system_is_device {};
+template <class It, class = void> struct has_device_category : std::false_type {};
+template <class It> struct has_device_category<It, typename std::enable_if<std::is_base_of<device_category_marker, typename It::iterator_category>::value>::type>
+    : std::true_type {};
+template <class It> struct is_device_iterator { static constexpr bool value = declares_device_iterator<It>::value || has_device_category<It>::value; };
+template <class T> struct is_device_iterator<T*> { static constexpr bool value = false; };
 template <class T> struct is_device_iterator<thrust::device_ptr<T>> { static constexpr bool value = true; };
 }}}  // namespace system::cdna4::detail
 }  // namespace thrust

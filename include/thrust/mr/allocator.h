@@ -4,6 +4,7 @@
 #include <cstddef>
 #include <thrust/device_ptr.h>
 #include <thrust/mr/memory_resource.h>
+#include <thrust/mr/polymorphic_adaptor.h>
 
 namespace thrust { namespace mr {
 namespace detail {
@@ -54,5 +55,14 @@ class stateless_resource_allocator : public allocator<T, Upstream> {
   template <class U> struct rebind { typedef stateless_resource_allocator<U, Upstream> other; };
   stateless_resource_allocator() : allocator<T, Upstream>(get_global_resource<Upstream>()) {}
   template <class U> stateless_resource_allocator(const stateless_resource_allocator<U, Upstream>& o) : allocator<T, Upstream>(o) {}
+};
+// an allocator over a resource chosen at run time (thrust/mr/allocator.h:229-260)
+template <class T, class Pointer>
+class polymorphic_allocator : public allocator<T, polymorphic_adaptor_resource<Pointer>> {
+  typedef allocator<T, polymorphic_adaptor_resource<Pointer>> base;
+ public:
+  template <class U> struct rebind { typedef polymorphic_allocator<U, Pointer> other; };
+  polymorphic_allocator(polymorphic_adaptor_resource<Pointer>* resource) : base(resource) {}
+  template <class U> polymorphic_allocator(const polymorphic_allocator<U, Pointer>& o) : base(o) {}
 };
 }}  // namespace thrust::mr

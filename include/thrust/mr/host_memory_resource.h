@@ -1,4 +1,6 @@
-// <thrust/mr/host_memory_resource.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/mr/host_memory_resource.h> is not provided by the cdna4 device system"
+// thrust::host_memory_resource (thrust/mr/host_memory_resource.h): host memory from operator new.
+#pragma once
+#include <thrust/mr/new.h>
+namespace thrust {
+typedef mr::new_delete_resource host_memory_resource;
+}  // namespace thrust

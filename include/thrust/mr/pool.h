@@ -7,6 +7,7 @@
 // only after the work that uses the block has completed.
 #pragma once
 #include <algorithm>
+#include <memory>
 #include <cstddef>
 #include <stdexcept>
 #include <vector>
@@ -24,24 +25,33 @@ template <> struct byte_pointer<void*> {
 };
 }  // namespace detail
 
-template <class Upstream>
-class unsynchronized_pool_resource final : public memory_resource<typename Upstream::pointer> {
+namespace detail {
+// Where a pool keeps its own records (free lists, chunk table): ordinary host memory ...
+struct heap_bookkeeping {
+  template <class T> struct alloc { typedef std::allocator<T> type; };
+  template <class T> std::allocator<T> get() const { return std::allocator<T>(); }
+};
+// ... or memory of a resource the user names (the "disjoint" pools: the pooled memory itself is
+// never touched, so it may be memory the host cannot address).  Defined in <thrust/mr/disjoint_pool.h>.
+template <class Bookkeeper> struct resource_bookkeeping;
+
+template <class Upstream, class Book>
+class pool_core : public memory_resource<typename Upstream::pointer> {
  public:
   typedef typename Upstream::pointer pointer;
   static pool_options get_default_options() { return pool_options(); }
 
-  explicit unsynchronized_pool_resource(Upstream* upstream, pool_options options = get_default_options())
-      : upstream_(upstream), opt_(options) {
+  pool_core(Upstream* upstream, Book book, pool_options options)
+      : upstream_(upstream), opt_(options), book_(book), free_(book.template get<free_list>()), chunks_(book.template get<chunk>()),
+        oversized_(book.template get<big>()) {
     if (!opt_.validate()) throw std::invalid_argument("thrust::mr::pool_options: inconsistent");
     std::size_t classes = 1;
     for (std::size_t s = opt_.smallest_block_size; s < opt_.largest_block_size; s <<= 1) ++classes;
-    free_.resize(classes);
+    free_.assign(classes, free_list(book.template get<pointer>()));
   }
-  explicit unsynchronized_pool_resource(pool_options options = get_default_options())
-      : unsynchronized_pool_resource(get_global_resource<Upstream>(), options) {}
-  ~unsynchronized_pool_resource() override { release(); }
-  unsynchronized_pool_resource(const unsynchronized_pool_resource&) = delete;
-  unsynchronized_pool_resource& operator=(const unsynchronized_pool_resource&) = delete;
+  ~pool_core() override { release(); }
+  pool_core(const pool_core&) = delete;
+  pool_core& operator=(const pool_core&) = delete;
 
   // everything goes back to the upstream; blocks still handed out become invalid
   void release() {
@@ -60,7 +70,7 @@ class unsynchronized_pool_resource final : public memory_resource<typename Upstr
     if (bytes > opt_.largest_block_size) return allocate_oversized(bytes);
     std::size_t size = opt_.smallest_block_size, cls = 0;
     while (size < bytes) { size <<= 1; ++cls; }
-    std::vector<pointer>& list = free_[cls];
+    free_list& list = free_[cls];
     if (list.empty()) refill(list, size);
     pointer p = list.back();
     list.pop_back();
@@ -87,8 +97,9 @@ class unsynchronized_pool_resource final : public memory_resource<typename Upstr
  private:
   struct chunk { pointer p; std::size_t bytes; };
   struct big { pointer p; std::size_t bytes; bool in_use; };
+  typedef std::vector<pointer, typename Book::template alloc<pointer>::type> free_list;
 
-  void refill(std::vector<pointer>& list, std::size_t size) {
+  void refill(free_list& list, std::size_t size) {
     const std::size_t stride = std::max(size, opt_.alignment);  // keeps every block aligned
     std::size_t blocks = std::max(opt_.min_blocks_per_chunk, (opt_.min_bytes_per_chunk + stride - 1) / stride);
     blocks = std::min(blocks, opt_.max_blocks_per_chunk);
@@ -114,9 +125,22 @@ class unsynchronized_pool_resource final : public memory_resource<typename Upstr
 
   Upstream* upstream_;
   pool_options opt_;
-  std::vector<std::vector<pointer>> free_;
-  std::vector<chunk> chunks_;
-  std::vector<big> oversized_;
+  Book book_;
+  std::vector<free_list, typename Book::template alloc<free_list>::type> free_;
+  std::vector<chunk, typename Book::template alloc<chunk>::type> chunks_;
+  std::vector<big, typename Book::template alloc<big>::type> oversized_;
   std::size_t upstream_calls_ = 0;
+};
+}  // namespace detail
+
+template <class Upstream>
+class unsynchronized_pool_resource final : public detail::pool_core<Upstream, detail::heap_bookkeeping> {
+  typedef detail::pool_core<Upstream, detail::heap_bookkeeping> core;
+ public:
+  static pool_options get_default_options() { return pool_options(); }
+  explicit unsynchronized_pool_resource(Upstream* upstream, pool_options options = get_default_options())
+      : core(upstream, detail::heap_bookkeeping(), options) {}
+  explicit unsynchronized_pool_resource(pool_options options = get_default_options())
+      : core(get_global_resource<Upstream>(), detail::heap_bookkeeping(), options) {}
 };
 }}  // namespace thrust::mr

@@ -1,4 +1,31 @@
-// <thrust/mr/sync_pool.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/mr/sync_pool.h> is not provided by the cdna4 device system"
+// thrust::mr::synchronized_pool_resource (thrust/mr/sync_pool.h): the caching pool behind a mutex,
+// for use from several threads.
+#pragma once
+#include <mutex>
+#include <thrust/mr/pool.h>
+namespace thrust { namespace mr {
+template <class Upstream>
+class synchronized_pool_resource : public memory_resource<typename Upstream::pointer> {
+  typedef unsynchronized_pool_resource<Upstream> unsync_pool;
+ public:
+  typedef typename Upstream::pointer pointer;
+  static pool_options get_default_options() { return unsync_pool::get_default_options(); }
+  explicit synchronized_pool_resource(Upstream* upstream, pool_options options = get_default_options()) : pool_(upstream, options) {}
+  explicit synchronized_pool_resource(pool_options options = get_default_options()) : pool_(get_global_resource<Upstream>(), options) {}
+  void release() {
+    std::lock_guard<std::mutex> lock(mutex_);
+    pool_.release();
+  }
+  pointer do_allocate(std::size_t bytes, std::size_t alignment) override {
+    std::lock_guard<std::mutex> lock(mutex_);
+    return pool_.do_allocate(bytes, alignment);
+  }
+  void do_deallocate(pointer p, std::size_t bytes, std::size_t alignment) override {
+    std::lock_guard<std::mutex> lock(mutex_);
+    pool_.do_deallocate(p, bytes, alignment);
+  }
+ private:
+  std::mutex mutex_;
+  unsync_pool pool_;
+};
+}}  // namespace thrust::mr

@@ -15,6 +15,9 @@
 #include <thrust/iterator/constant_iterator.h>
 #include <thrust/iterator/counting_iterator.h>
 #include <thrust/iterator/discard_iterator.h>
+#include <thrust/iterator/iterator_adaptor.h>
+#include <thrust/iterator/iterator_facade.h>
+#include <thrust/iterator/retag.h>
 #include <thrust/iterator/permutation_iterator.h>
 #include <thrust/iterator/reverse_iterator.h>
 #include <thrust/iterator/transform_iterator.h>
@@ -397,5 +400,64 @@ void TestSortWithZipIterators() {
   }
 }
 DECLARE_UNITTEST(TestSortWithZipIterators);
+
+// A user-defined iterator from iterator_adaptor (the example of thrust/iterator/iterator_adaptor.h:
+// every element of the base range n times) and one from iterator_facade (squares of the index), used
+// as inputs of device algorithms; retag declares a raw device pointer to be a device range.
+template <class Iterator>
+class repeat_iterator : public thrust::iterator_adaptor<repeat_iterator<Iterator>, Iterator> {
+ public:
+  typedef thrust::iterator_adaptor<repeat_iterator<Iterator>, Iterator> super_t;
+  __host__ __device__ repeat_iterator(const Iterator& x, int n) : super_t(x), begin(x), n(n) {}
+  friend class thrust::iterator_core_access;
+
+ private:
+  Iterator begin;
+  int n;
+  __host__ __device__ typename super_t::reference dereference() const { return *(begin + (this->base() - begin) / n); }
+};
+class squares_iterator
+    : public thrust::iterator_facade<squares_iterator, long long, thrust::device_system_tag, thrust::random_access_traversal_tag, long long> {
+ public:
+  __host__ __device__ explicit squares_iterator(long long i = 0) : i_(i) {}
+  friend class thrust::iterator_core_access;
+
+ private:
+  long long i_;
+  __host__ __device__ long long dereference() const { return i_ * i_; }
+  __host__ __device__ bool equal(const squares_iterator& o) const { return i_ == o.i_; }
+  __host__ __device__ void increment() { ++i_; }
+  __host__ __device__ void decrement() { --i_; }
+  __host__ __device__ void advance(std::ptrdiff_t n) { i_ += n; }
+  __host__ __device__ std::ptrdiff_t distance_to(const squares_iterator& o) const { return (std::ptrdiff_t)(o.i_ - i_); }
+};
+void TestUserIteratorsFromFacadeAndAdaptor() {
+  thrust::host_vector<int> h = {1, 2, 3, 4};
+  thrust::device_vector<int> d = h;
+  typedef repeat_iterator<thrust::device_vector<int>::iterator> Rep;
+  static_assert(thrust::system::cdna4::detail::is_device_iterator<Rep>::value, "an adaptor over a device iterator is a device iterator");
+  static_assert(!thrust::system::cdna4::detail::is_device_iterator<repeat_iterator<thrust::host_vector<int>::iterator>>::value, "");
+  Rep first(d.begin(), 3), last = first + 12;
+  ASSERT_EQUAL(last - first, 12);
+  ASSERT_EQUAL(thrust::reduce(first, last), 30);
+  thrust::device_vector<int> out(12);
+  thrust::copy(first, last, out.begin());
+  ASSERT_EQUAL(out, (thrust::host_vector<int>{1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4}));
+  thrust::inclusive_scan(first, last, out.begin());
+  ASSERT_EQUAL(out, (thrust::host_vector<int>{1, 2, 3, 5, 7, 9, 12, 15, 18, 22, 26, 30}));
+  // the same adaptor over a host range runs on the host
+  repeat_iterator<thrust::host_vector<int>::iterator> hf(h.begin(), 2);
+  ASSERT_EQUAL(thrust::reduce(hf, hf + 8), 20);
+  // a facade that computes its values: sum of i^2 below n
+  const long long n = 100000;
+  ASSERT_EQUAL(thrust::reduce(squares_iterator(0), squares_iterator(n), 0ll), (n - 1) * n * (2 * n - 1) / 6);
+  ASSERT_EQUAL((long long)squares_iterator(3)[4], 49ll);
+  ASSERT_TRUE(squares_iterator(3) < squares_iterator(5) && squares_iterator(5) - squares_iterator(3) == 2);
+  // retag: a raw device pointer becomes a device range
+  int* raw = thrust::raw_pointer_cast(d.data());
+  auto tagged = thrust::retag<thrust::device_system_tag>(raw);
+  ASSERT_EQUAL(thrust::reduce(tagged, tagged + 4), 10);
+}
+DECLARE_UNITTEST(TestUserIteratorsFromFacadeAndAdaptor);
 
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }

@@ -7,11 +7,22 @@
 #include <thrust/device_vector.h>
 #include <thrust/mr/allocator.h>
 #include <thrust/mr/device_memory_resource.h>
+#include <thrust/mr/disjoint_pool.h>
+#include <thrust/mr/disjoint_sync_pool.h>
+#include <thrust/mr/disjoint_tls_pool.h>
+#include <thrust/mr/fancy_pointer_resource.h>
+#include <thrust/mr/host_memory_resource.h>
 #include <thrust/mr/new.h>
+#include <thrust/mr/polymorphic_adaptor.h>
 #include <thrust/mr/pool.h>
+#include <thrust/mr/sync_pool.h>
+#include <thrust/mr/tls_pool.h>
+#include <thrust/mr/validator.h>
 #include <thrust/reduce.h>
 #include <thrust/scan.h>
 #include <thrust/sort.h>
+
+#include <thread>
 
 #include "testing.h"
 
@@ -201,5 +212,130 @@ void TestTemporaryStorageFromUserAllocator() {
   ASSERT_TRUE(alloc.allocated_blocks.empty());
 }
 DECLARE_UNITTEST(TestTemporaryStorageFromUserAllocator);
+
+// testing/mr_disjoint_pool.cu:120-260: the same caching behaviour with the pool's records in
+// memory of a second resource, which the test sees being used
+void TestDisjointPool() {
+  thrust::mr::new_delete_resource heap;
+  tracking_resource<thrust::mr::new_delete_resource> book(&heap);
+  {
+    thrust::device_memory_resource dev;
+    tracking_resource<thrust::device_memory_resource> up(&dev);
+    typedef thrust::mr::disjoint_unsynchronized_pool_resource<tracking_resource<thrust::device_memory_resource>,
+                                                               tracking_resource<thrust::mr::new_delete_resource>> Pool;
+    thrust::mr::pool_options opt;
+    opt.smallest_block_size = 256;
+    opt.largest_block_size = 1 << 16;
+    Pool pool(&up, &book, opt);
+    ASSERT_TRUE(book.allocations > 0);  // the size-class table lives in the bookkeeper's memory
+    thrust::device_ptr<void> a = pool.allocate(1000, 256);
+    const int chunk_allocations = up.allocations;
+    ASSERT_EQUAL(chunk_allocations, 1);
+    pool.deallocate(a, 1000, 256);
+    thrust::device_ptr<void> b = pool.allocate(900, 256);  // the same class: served from the cache
+    ASSERT_TRUE(a == b);
+    ASSERT_EQUAL(up.allocations, chunk_allocations);
+    pool.deallocate(b, 900, 256);
+    thrust::device_ptr<void> big = pool.allocate(1 << 20, 256);  // oversized: straight from upstream, cached afterwards
+    pool.deallocate(big, 1 << 20, 256);
+    ASSERT_TRUE(pool.allocate(1 << 20, 256) == big);
+    pool.deallocate(big, 1 << 20, 256);
+    // a device_vector over the pool
+    typedef thrust::mr::allocator<int, Pool> Alloc;
+    thrust::device_vector<int, Alloc> v(1000, 2, Alloc(&pool));
+    ASSERT_EQUAL(thrust::reduce(v.begin(), v.end()), 2000);
+    pool.release();
+    ASSERT_EQUAL(up.allocations, up.deallocations + 0);
+  }
+  ASSERT_EQUAL(book.allocations, book.deallocations);  // the records were returned too
+  ASSERT_EQUAL(book.live_bytes, std::size_t(0));
+}
+DECLARE_UNITTEST(TestDisjointPool);
+
+// testing/mr_pool.cu (synchronized), mr_disjoint_pool.cu (synchronized): several threads on one pool
+template <class Pool>
+void hammer(Pool& pool) {
+  std::vector<std::thread> threads;
+  std::vector<int> ok(8, 0);
+  for (int t = 0; t < 8; t++)
+    threads.emplace_back([&pool, &ok, t] {
+      bool good = true;
+      for (int i = 0; i < 200; i++) {
+        const std::size_t bytes = 64 + 64 * ((i * 7 + t) % 50);
+        void* p = pool.allocate(bytes, 64);
+        good = good && p != nullptr;
+        static_cast<char*>(p)[bytes - 1] = (char)t;
+        void* q = pool.allocate(bytes, 64);
+        good = good && q != p;
+        pool.deallocate(p, bytes, 64);
+        pool.deallocate(q, bytes, 64);
+      }
+      ok[t] = good;
+    });
+  for (auto& th : threads) th.join();
+  for (int t = 0; t < 8; t++) ASSERT_TRUE(ok[t]);
+}
+void TestSynchronizedAndThreadLocalPools() {
+  thrust::mr::new_delete_resource heap;
+  thrust::mr::synchronized_pool_resource<thrust::mr::new_delete_resource> sync(&heap);
+  hammer(sync);
+  sync.release();
+  thrust::mr::disjoint_synchronized_pool_resource<thrust::mr::new_delete_resource, thrust::mr::new_delete_resource> dsync(&heap, &heap);
+  hammer(dsync);
+  // one pool per thread: the same object within a thread, another one on another thread (a
+  // thread's pool lives until the thread ends, so its upstream is the global resource object)
+  thrust::mr::new_delete_resource* global = thrust::mr::get_global_resource<thrust::mr::new_delete_resource>();
+  auto& mine = thrust::mr::tls_pool(global);
+  ASSERT_TRUE(&mine == &thrust::mr::tls_pool<thrust::mr::new_delete_resource>());
+  void* theirs = nullptr;
+  std::thread([&] { theirs = &thrust::mr::tls_pool(global); }).join();
+  ASSERT_TRUE(theirs != nullptr && theirs != (void*)&mine);
+  void* p = mine.allocate(100, 64);
+  mine.deallocate(p, 100, 64);
+  ASSERT_TRUE(mine.allocate(100, 64) == p);
+  mine.deallocate(p, 100, 64);
+  auto& dmine = thrust::mr::disjoint_tls_pool(global, global);
+  void* q = dmine.allocate(100, 64);
+  dmine.deallocate(q, 100, 64);
+}
+DECLARE_UNITTEST(TestSynchronizedAndThreadLocalPools);
+
+// examples/mr_basic.cu:38-60, testing/allocator.cu: one allocator type over resources chosen at run time
+void TestPolymorphicAdaptorAndFancyPointerResource() {
+  thrust::mr::new_delete_resource heap;
+  tracking_resource<thrust::mr::new_delete_resource> tracked(&heap);
+  thrust::mr::polymorphic_adaptor_resource<void*> adaptor(&tracked);
+  typedef thrust::mr::polymorphic_allocator<int, void*> Alloc;
+  Alloc alloc(&adaptor);
+  {
+    thrust::host_vector<int, Alloc> v(alloc);
+    for (int i = 0; i < 100; i++) v.push_back(i);
+    ASSERT_EQUAL(v.back(), 99);
+    ASSERT_TRUE(tracked.allocations > 0);
+  }
+  ASSERT_EQUAL(tracked.allocations, tracked.deallocations);
+  thrust::mr::polymorphic_adaptor_resource<void*> same(&tracked), other(&heap);
+  ASSERT_TRUE(adaptor == same);
+  ASSERT_TRUE(!(adaptor == other));
+  // device memory through the adaptor
+  thrust::device_memory_resource dev;
+  thrust::mr::polymorphic_adaptor_resource<thrust::device_ptr<void>> dadaptor(&dev);
+  typedef thrust::mr::polymorphic_allocator<int, thrust::device_ptr<void>> DAlloc;
+  thrust::device_vector<int, DAlloc> d(100, 3, DAlloc(&dadaptor));
+  ASSERT_EQUAL(thrust::reduce(d.begin(), d.end()), 300);
+  // a host resource seen through device_ptr and back
+  thrust::mr::fancy_pointer_resource<thrust::mr::new_delete_resource, thrust::device_ptr<void>> fancy(&heap);
+  thrust::device_ptr<void> fp = fancy.allocate(64, 16);
+  ASSERT_TRUE(fp.get() != nullptr);
+  fancy.deallocate(fp, 64, 16);
+  thrust::device_ptr_memory_resource<thrust::device_memory_resource> dpr;
+  thrust::device_ptr<void> dp = dpr.allocate(256, 256);
+  ASSERT_TRUE(dp.get() != nullptr);
+  dpr.deallocate(dp, 256, 256);
+  thrust::mr::validator<thrust::host_memory_resource> check1;
+  thrust::mr::validator2<thrust::device_memory_resource, thrust::mr::new_delete_resource> check2;
+  (void)check1; (void)check2;
+}
+DECLARE_UNITTEST(TestPolymorphicAdaptorAndFancyPointerResource);
 
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
