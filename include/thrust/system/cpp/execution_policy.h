@@ -1,4 +1,16 @@
-// <thrust/system/cpp/execution_policy.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/system/cpp/execution_policy.h> is not provided by the cdna4 device system"
+// thrust::system::cpp / thrust::cpp (thrust/system/cpp/execution_policy.h): the host system of this
+// build — sequential algorithms on host memory.  thrust::cpp::par is the policy object
+// thrust::host also names; thrust::cpp::tag is the system tag of host iterators.
+#pragma once
+#include <thrust/execution_policy.h>
+namespace thrust {
+namespace system { namespace cpp {
+static const detail::par_t par;
+template <class Derived> using execution_policy = thrust::host_execution_policy<Derived>;
+}}  // namespace system::cpp
+namespace cpp {
+using thrust::system::cpp::execution_policy;
+using thrust::system::cpp::par;
+using thrust::system::cpp::tag;
+}  // namespace cpp
+}  // namespace thrust

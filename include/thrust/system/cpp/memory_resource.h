@@ -1,4 +1,8 @@
-// <thrust/system/cpp/memory_resource.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/system/cpp/memory_resource.h> is not provided by the cdna4 device system"
+// Memory resources of the host system (thrust/system/cpp/memory_resource.h): operator new / delete.
+#pragma once
+#include <thrust/mr/new.h>
+namespace thrust { namespace system { namespace cpp {
+typedef thrust::mr::new_delete_resource memory_resource;
+typedef thrust::mr::new_delete_resource universal_memory_resource;
+typedef thrust::mr::new_delete_resource universal_host_pinned_memory_resource;
+}}}  // namespace thrust::system::cpp

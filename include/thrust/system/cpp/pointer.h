@@ -1,4 +1,14 @@
-// <thrust/system/cpp/pointer.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/system/cpp/pointer.h> is not provided by the cdna4 device system"
+// thrust::cpp::pointer / reference (thrust/system/cpp/pointer.h): pointers into host memory are
+// raw pointers in this build.
+#pragma once
+#include <thrust/system/cpp/execution_policy.h>
+namespace thrust {
+namespace system { namespace cpp {
+template <class T> using pointer = T*;
+template <class T> using reference = T&;
+}}  // namespace system::cpp
+namespace cpp {
+using thrust::system::cpp::pointer;
+using thrust::system::cpp::reference;
+}  // namespace cpp
+}  // namespace thrust

@@ -1,4 +1,14 @@
-// <thrust/system/cpp/vector.h> is a header of the Thrust API that the cdna4 device system does not provide.
-// The file exists so that including it stops here with a clear message instead of resolving to
-// another Thrust installation further down the include path and mixing two libraries.
-#error "<thrust/system/cpp/vector.h> is not provided by the cdna4 device system"
+// thrust::cpp::vector (thrust/system/cpp/vector.h): the host system's vector is thrust::host_vector.
+#pragma once
+#include <thrust/host_vector.h>
+#include <thrust/system/cpp/memory.h>
+namespace thrust {
+namespace system { namespace cpp {
+template <class T, class Allocator = std::allocator<T>> using vector = thrust::host_vector<T, Allocator>;
+template <class T, class Allocator = std::allocator<T>> using universal_vector = thrust::host_vector<T, Allocator>;
+}}  // namespace system::cpp
+namespace cpp {
+using thrust::system::cpp::universal_vector;
+using thrust::system::cpp::vector;
+}  // namespace cpp
+}  // namespace thrust

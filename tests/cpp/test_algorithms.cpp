@@ -15,6 +15,7 @@
 #include <thrust/iterator/counting_iterator.h>
 #include <thrust/logical.h>
 #include <thrust/mismatch.h>
+#include <thrust/optional.h>
 #include <thrust/random.h>
 #include <thrust/replace.h>
 #include <thrust/reverse.h>
@@ -396,5 +397,39 @@ void TestShuffle() {
   ASSERT_EQUAL(thrust::detail::feistel_bijection(1, g).nearest_power_of_two(), std::uint64_t(16));
 }
 DECLARE_UNITTEST(TestShuffle);
+
+// thrust::optional in device code and in device storage (trivially copyable for trivial T)
+struct checked_root {
+  __host__ __device__ thrust::optional<float> operator()(float x) const {
+    if (x < 0) return thrust::nullopt;
+    return thrust::optional<float>(x * 0.5f);
+  }
+};
+struct value_or_minus_one {
+  __host__ __device__ float operator()(const thrust::optional<float>& o) const {
+    return o.map([](float v) { return v + 1.0f; }).value_or(-1.0f);
+  }
+};
+void TestOptionalOnDevice() {
+  static_assert(std::is_trivially_copyable<thrust::optional<float>>::value, "optional of a trivial type can live in device storage");
+  const std::size_t n = 10000;
+  thrust::host_vector<float> h(n);
+  for (std::size_t i = 0; i < n; i++) h[i] = (float)((int)(i % 7) - 3);
+  thrust::device_vector<float> d = h, out(n);
+  thrust::device_vector<thrust::optional<float>> o(n);
+  thrust::transform(d.begin(), d.end(), o.begin(), checked_root());
+  thrust::transform(o.begin(), o.end(), out.begin(), value_or_minus_one());
+  thrust::host_vector<thrust::optional<float>> ho = o;
+  thrust::host_vector<float> hout = out;
+  for (std::size_t i = 0; i < n; i++) {
+    ASSERT_EQUAL(ho[i].has_value(), h[i] >= 0);
+    if (h[i] >= 0) ASSERT_EQUAL(*ho[i], h[i] * 0.5f);
+    ASSERT_EQUAL(hout[i], h[i] >= 0 ? h[i] * 0.5f + 1.0f : -1.0f);
+  }
+  thrust::optional<int> a(3), b;
+  ASSERT_TRUE(b < a && a == 3 && b == thrust::nullopt && a.value_or(0) == 3 && b.value_or(9) == 9);
+  ASSERT_THROWS(b.value(), thrust::bad_optional_access);
+}
+DECLARE_UNITTEST(TestOptionalOnDevice);
 
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
