@@ -2,6 +2,7 @@
 // Device ranges (device_vector iterators, device_ptr, or raw pointers under a device policy)
 // go to the radix-sort kernels; host ranges are sorted on the host.
 #pragma once
+#include <cstring>
 #include <thrust/system/cdna4/detail/index_algorithms.h>
 #include <algorithm>
 #include <numeric>
@@ -106,14 +107,46 @@ void sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt
 }
 
 // ---- host, explicit policy -----------------------------------------------------------
+namespace detail {
+// Floating-point keys under less / greater sort by their radix encoding, as the reference's host
+// system does (thrust/system/detail/sequential/stable_radix_sort.inl:43-139: negatives with all
+// bits flipped, the others with the sign bit flipped): a total order in which -0 comes before +0
+// and NaNs take the place of their bit patterns — `a < b` on floats is not an ordering when NaNs
+// are present and would leave -0 / +0 in input order.
+inline std::uint32_t radix_key(float f) {
+  std::uint32_t u;
+  std::memcpy(&u, &f, sizeof u);
+  return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+inline std::uint64_t radix_key(double f) {
+  std::uint64_t u;
+  std::memcpy(&u, &f, sizeof u);
+  return u ^ ((u >> 63) ? 0xFFFFFFFFFFFFFFFFull : 0x8000000000000000ull);
+}
+template <class K, class Compare, bool Encoded = std::is_floating_point<K>::value && (system::cdna4::detail::order_code<Compare>::value >= 0)>
+struct host_order {
+  Compare comp;
+  bool operator()(const K& a, const K& b) const { return comp(a, b); }
+};
+template <class K, class Compare>
+struct host_order<K, Compare, true> {
+  Compare comp;
+  bool operator()(const K& a, const K& b) const {
+    return system::cdna4::detail::order_code<Compare>::value == 0 ? radix_key(a) < radix_key(b) : radix_key(a) > radix_key(b);
+  }
+};
+}  // namespace detail
 template <class It, class Compare>
-void stable_sort(const system::cpp::detail::par_t&, It first, It last, Compare comp) { std::stable_sort(first, last, comp); }
+void stable_sort(const system::cpp::detail::par_t&, It first, It last, Compare comp) {
+  typedef typename detail::value_of<It>::type K;
+  std::stable_sort(first, last, detail::host_order<K, Compare>{comp});
+}
 template <class It>
-void stable_sort(const system::cpp::detail::par_t&, It first, It last) { std::stable_sort(first, last); }
+void stable_sort(const system::cpp::detail::par_t& e, It first, It last) { stable_sort(e, first, last, less<typename detail::value_of<It>::type>()); }
 template <class It, class Compare>
-void sort(const system::cpp::detail::par_t&, It first, It last, Compare comp) { std::stable_sort(first, last, comp); }
+void sort(const system::cpp::detail::par_t& e, It first, It last, Compare comp) { stable_sort(e, first, last, comp); }
 template <class It>
-void sort(const system::cpp::detail::par_t&, It first, It last) { std::stable_sort(first, last); }
+void sort(const system::cpp::detail::par_t& e, It first, It last) { stable_sort(e, first, last); }
 template <class KIt, class VIt, class Compare>
 void stable_sort_by_key(const system::cpp::detail::par_t&, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
   typedef typename detail::value_of<KIt>::type K;
@@ -123,7 +156,8 @@ void stable_sort_by_key(const system::cpp::detail::par_t&, KIt kfirst, KIt klast
   std::iota(idx.begin(), idx.end(), std::size_t(0));
   std::vector<K> k(kfirst, klast);
   std::vector<V> v(vfirst, vfirst + n);
-  std::stable_sort(idx.begin(), idx.end(), [&](std::size_t a, std::size_t b) { return comp(k[a], k[b]); });
+  const detail::host_order<K, Compare> order{comp};
+  std::stable_sort(idx.begin(), idx.end(), [&](std::size_t a, std::size_t b) { return order(k[a], k[b]); });
   for (std::size_t i = 0; i < n; i++) { kfirst[i] = k[idx[i]]; vfirst[i] = v[idx[i]]; }
 }
 template <class KIt, class VIt>

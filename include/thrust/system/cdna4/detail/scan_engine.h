@@ -15,8 +15,8 @@
 //     upto   = before (+) load(i).
 // No identity element is needed and combine is never called with swapped arguments.
 //
-// A tile is 512 threads x ITEMS consecutive elements per thread (read and written in wavefront-
-// contiguous pieces and reordered through LDS).  Tiles take their index from a
+// A tile is one or two parts of 512 threads x ITEMS consecutive elements per thread (read and
+// written in wavefront-contiguous pieces and reordered through LDS).  Tiles take their index from a
 // ticket counter, so every tile a waiting tile looks back at has started and the wait ends.  A
 // tile descriptor is NW 64-bit atoms, one per 32-bit word of the accumulator, each (status << 32
 // | word), written and read with relaxed agent-scope atomics: a reader that finds the same status
@@ -85,94 +85,121 @@ __device__ inline Acc shfl_up_acc(const Acc& a, int d) {
 template <int ITEMS>
 __device__ inline int staged(int e) { return e + e / ITEMS; }
 
+// Parts of a tile: a tile is SUB parts of 512 x ITEMS elements each, staged through LDS one after
+// the other, with ONE ticket, one descriptor and one look-back for all of them — the fixed costs
+// of a tile are paid per SUB x 512 x ITEMS elements while LDS holds one part.
+constexpr int scan_parts(std::size_t acc_bytes) { return acc_bytes <= 16 ? 2 : 1; }
+
+// (has_a ? a : nothing) (+) (has_b ? b : nothing), for operators without an identity
+template <class Op, class Acc>
+__device__ inline void join(const Op& op, bool& has_a, Acc& a, bool has_b, const Acc& b) {
+  if (has_b) {
+    a = has_a ? op.combine(a, b) : b;
+    has_a = true;
+  }
+}
+
 // words[0, tiles * NW) are the descriptors, words[tiles * NW] is the ticket counter
 template <class Op>
 __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n, Op op, unsigned long long* words, std::int64_t tiles) {
   typedef typename Op::acc Acc;
   typedef scan_desc<Acc> Desc;
   constexpr int ITEMS = scan_items(sizeof(Acc));
-  constexpr int TILE = kScanBlock * ITEMS;
+  constexpr int SUB = scan_parts(sizeof(Acc));
+  constexpr int PART = kScanBlock * ITEMS;
+  constexpr int TILE = SUB * PART;
   constexpr int NWAVES = kScanBlock / 64;
-  // Global memory is touched in striped order (thread t, step j: element j * 512 + t of the tile,
+  // Global memory is touched in striped order (thread t, step j: element j * 512 + t of a part,
   // so a wavefront's access is one contiguous piece) while the scan wants every thread to own
   // ITEMS consecutive elements: loaded accumulators and results change order through LDS.
   // Accumulators too large for that buffer are loaded and stored in the threads' own order.
-  constexpr bool kStaged = sizeof(Acc) * (TILE + TILE / ITEMS) <= 40 * 1024;
+  constexpr bool kStaged = sizeof(Acc) * (PART + PART / ITEMS) <= 40 * 1024;
   typedef typename std::aligned_storage<sizeof(Acc), alignof(Acc)>::type Raw;
-  __shared__ Raw raw_stage[kStaged ? TILE + TILE / ITEMS : 1], raw_wave[NWAVES], raw_look[64], raw_prefix;
+  __shared__ Raw raw_stage[kStaged ? PART + PART / ITEMS : 1], raw_wave[SUB][NWAVES], raw_part[SUB], raw_look[64], raw_prefix;
   __shared__ unsigned long long s_tile;
   __shared__ int s_has_prefix;
   Acc* s_stage = reinterpret_cast<Acc*>(raw_stage);
-  Acc* s_wave = reinterpret_cast<Acc*>(raw_wave);  // inclusive aggregate of each wavefront's threads
   Acc* s_look = reinterpret_cast<Acc*>(raw_look);  // one look-back window
   Acc* s_prefix = reinterpret_cast<Acc*>(&raw_prefix);
+  const auto s_wave = [&](int part, int w) -> Acc& { return *reinterpret_cast<Acc*>(&raw_wave[part][w]); };  // inclusive aggregate of a wavefront's threads
+  const auto s_part = [&](int part) -> Acc& { return *reinterpret_cast<Acc*>(&raw_part[part]); };           // aggregate of a part
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   if (tid == 0) s_tile = __hip_atomic_fetch_add(&words[tiles * Desc::NW], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const std::int64_t tile = (std::int64_t)s_tile;
   const std::int64_t tile_base = tile * TILE;
-  const std::int64_t base = tile_base + (std::int64_t)tid * ITEMS;
-  const std::int64_t left = n - base;
-  const int count = left >= ITEMS ? ITEMS : left > 0 ? (int)left : 0;  // this thread's elements
-  const std::int64_t tile_left = n - tile_base;                         // >= 1: tile < tiles
-  const bool whole = tile_left >= TILE;
-  const int nvalid = whole ? kScanBlock : (int)((tile_left + ITEMS - 1) / ITEMS);  // threads with elements
-  const int tile_count = whole ? TILE : (int)tile_left;
+  const bool whole = n - tile_base >= TILE;  // every element of the tile exists (n - tile_base >= 1: tile < tiles)
 
-  // every thread loads ITEMS times (the last element where the tile has no more) so that the
-  // loads stay independent of each other
-  Acc x[ITEMS];
-  if constexpr (kStaged) {
-    if (whole) {
+  // elements of part p: how many exist, how many of them are this thread's, how many threads have any
+  int part_count[SUB], count[SUB], nvalid[SUB];
 #pragma unroll
-      for (int j = 0; j < ITEMS; j++) x[j] = op.load(tile_base + j * kScanBlock + tid);
-    } else {
+  for (int p = 0; p < SUB; p++) {
+    const std::int64_t left = n - (tile_base + (std::int64_t)p * PART);
+    part_count[p] = whole ? PART : left >= PART ? PART : left > 0 ? (int)left : 0;
+    const int mine = part_count[p] - tid * ITEMS;
+    count[p] = mine >= ITEMS ? ITEMS : mine > 0 ? mine : 0;
+    nvalid[p] = (part_count[p] + ITEMS - 1) / ITEMS;
+  }
+
+  // every thread loads SUB x ITEMS times (the last element where the input has no more) so that
+  // the loads stay independent of each other
+  Acc x[SUB][ITEMS];
 #pragma unroll
-      for (int j = 0; j < ITEMS; j++) {
-        const std::int64_t i = tile_base + j * kScanBlock + tid;
-        x[j] = op.load(i < n ? i : n - 1);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < ITEMS; j++) s_stage[staged<ITEMS>(j * kScanBlock + tid)] = x[j];
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < ITEMS; j++) x[j] = s_stage[staged<ITEMS>(tid * ITEMS + j)];
-  } else {
+  for (int p = 0; p < SUB; p++) {
+    const std::int64_t part_base = tile_base + (std::int64_t)p * PART;
 #pragma unroll
     for (int j = 0; j < ITEMS; j++) {
-      const std::int64_t i = base + j;
-      x[j] = op.load(i < n ? i : n - 1);
+      const std::int64_t i = part_base + (kStaged ? j * kScanBlock + tid : tid * ITEMS + j);
+      x[p][j] = op.load(whole ? i : (i < n ? i : n - 1));
     }
   }
-  // inclusive scan of the thread's own elements (x is only ever indexed by unrolled constants, so
-  // that it stays in registers)
-  Acc incl = x[0];
-#pragma unroll
-  for (int j = 1; j < ITEMS; j++)
-    if (j < count) {
-      x[j] = op.combine(x[j - 1], x[j]);
-      incl = x[j];
-    }
 
-  // inclusive scan of the threads' aggregates within each wavefront; threads without elements are
-  // a suffix of the tile and stay out of it (no identity element is assumed)
-  const bool valid = tid < nvalid;
+  Acc lane_before[SUB];  // aggregate of the wavefront's earlier threads in part p (lane > 0)
 #pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const Acc up = shfl_up_acc(incl, d);
-    if (valid && lane >= d) incl = op.combine(up, incl);
+  for (int p = 0; p < SUB; p++) {
+    if constexpr (kStaged) {
+      if (p > 0) __syncthreads();  // the part before has been read out of the buffer
+#pragma unroll
+      for (int j = 0; j < ITEMS; j++) s_stage[staged<ITEMS>(j * kScanBlock + tid)] = x[p][j];
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < ITEMS; j++) x[p][j] = s_stage[staged<ITEMS>(tid * ITEMS + j)];
+    }
+    // inclusive scan of the thread's own elements (x is only ever indexed by unrolled constants,
+    // so that it stays in registers)
+    Acc incl = x[p][0];
+#pragma unroll
+    for (int j = 1; j < ITEMS; j++)
+      if (j < count[p]) {
+        x[p][j] = op.combine(x[p][j - 1], x[p][j]);
+        incl = x[p][j];
+      }
+    // inclusive scan of the threads' aggregates within each wavefront; threads without elements
+    // are a suffix of the part and stay out of it (no identity element is assumed)
+    const bool valid = tid < nvalid[p];
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const Acc up = shfl_up_acc(incl, d);
+      if (valid && lane >= d) incl = op.combine(up, incl);
+    }
+    lane_before[p] = shfl_up_acc(incl, 1);
+    if (valid && (lane == 63 || tid == nvalid[p] - 1)) s_wave(p, wave) = incl;
   }
-  const Acc lane_before = shfl_up_acc(incl, 1);  // aggregate of the wavefront's earlier threads (lane > 0)
-  const int last_valid = nvalid - 1;             // >= 0
-  if (valid && (lane == 63 || tid == last_valid)) s_wave[wave] = incl;
   __syncthreads();
-  const int nwaves_valid = (last_valid >> 6) + 1;
 
-  if (wave == 0) {  // wavefront 0: publish, look back, publish again
-    Acc tile_agg = s_wave[0];
-    for (int w = 1; w < nwaves_valid; w++) tile_agg = op.combine(tile_agg, s_wave[w]);
+  if (wave == 0) {  // wavefront 0: aggregates of the parts and of the tile, publish, look back, publish again
+    bool has_agg = false;
+    Acc tile_agg = x[0][0];  // placeholder until has_agg (part 0 is never empty)
+#pragma unroll
+    for (int p = 0; p < SUB; p++) {
+      const int nw = (nvalid[p] + 63) >> 6;  // wavefronts with elements in part p
+      bool has = false;
+      Acc agg = tile_agg;
+      for (int w = 0; w < nw; w++) join(op, has, agg, true, s_wave(p, w));
+      if (has && lane == 0) s_part(p) = agg;
+      join(op, has_agg, tile_agg, has, agg);
+    }
     bool has_prefix = false;  // meaningful in lane 0
     Acc prefix = tile_agg;    // placeholder until has_prefix
     if (tile > 0) {
@@ -225,48 +252,53 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
   }
   __syncthreads();
 
-  // everything before the thread's first element: tile prefix, earlier wavefronts, earlier lanes
-  const bool tile_has = s_has_prefix != 0;
-  bool thread_has = tile_has;
-  Acc thread_before = x[0];  // placeholder until thread_has
-  if (tile_has) thread_before = *s_prefix;
-  for (int w = 0; w < wave; w++) {
-    thread_before = thread_has ? op.combine(thread_before, s_wave[w]) : s_wave[w];
-    thread_has = true;
-  }
-  if (lane > 0) {
-    thread_before = thread_has ? op.combine(thread_before, lane_before) : lane_before;
-    thread_has = true;
-  }
-
-  if constexpr (kStaged) {
-    // results go to the staging buffer in the threads' order and leave it in striped order; the
-    // value before element e is the result of element e - 1 (the tile's prefix for e = 0)
+  // everything before part p: the tile's prefix and the parts before it
+  bool part_has = s_has_prefix != 0;
+  Acc part_before = x[0][0];  // placeholder until part_has
+  if (part_has) part_before = *s_prefix;
 #pragma unroll
-    for (int j = 0; j < ITEMS; j++)
-      if (j < count) s_stage[staged<ITEMS>(tid * ITEMS + j)] = thread_has ? op.combine(thread_before, x[j]) : x[j];
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < ITEMS; j++) {
-      const int e = j * kScanBlock + tid;
-      if (e < tile_count) {
-        const Acc upto = s_stage[staged<ITEMS>(e)];
-        const bool has_before = e > 0 || tile_has;
-        const Acc before = e > 0 ? s_stage[staged<ITEMS>(e - 1)] : (tile_has ? *s_prefix : upto);
-        op.store(tile_base + e, has_before, before, upto);
+  for (int p = 0; p < SUB; p++) {
+    if (part_count[p] > 0) {
+      // everything before the thread's first element of the part: earlier wavefronts, earlier lanes
+      bool thread_has = part_has;
+      Acc thread_before = part_before;
+      if (count[p] > 0) {  // (a thread without elements has no use for it, and the wavefronts before it may have none either)
+        for (int w = 0; w < wave; w++) join(op, thread_has, thread_before, true, s_wave(p, w));
+        join(op, thread_has, thread_before, lane > 0, lane_before[p]);
       }
-    }
-  } else if (count > 0) {
-    bool has_before = thread_has;
-    Acc before = thread_before;
+      const std::int64_t part_base = tile_base + (std::int64_t)p * PART;
+      if constexpr (kStaged) {
+        // results go to the staging buffer in the threads' order and leave it in striped order;
+        // the value before element e is the result of element e - 1 (the part's prefix for e = 0)
+        __syncthreads();  // the buffer is free: the loads of the last part, or the stores of the part before, are done
 #pragma unroll
-    for (int j = 0; j < ITEMS; j++) {
-      if (j < count) {
-        const Acc upto = thread_has ? op.combine(thread_before, x[j]) : x[j];
-        op.store(base + j, has_before, before, upto);
-        before = upto;
-        has_before = true;
+        for (int j = 0; j < ITEMS; j++)
+          if (j < count[p]) s_stage[staged<ITEMS>(tid * ITEMS + j)] = thread_has ? op.combine(thread_before, x[p][j]) : x[p][j];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < ITEMS; j++) {
+          const int e = j * kScanBlock + tid;
+          if (e < part_count[p]) {
+            const Acc upto = s_stage[staged<ITEMS>(e)];
+            const bool has_before = e > 0 || part_has;
+            const Acc before = e > 0 ? s_stage[staged<ITEMS>(e - 1)] : (part_has ? part_before : upto);
+            op.store(part_base + e, has_before, before, upto);
+          }
+        }
+      } else if (count[p] > 0) {
+        bool has_before = thread_has;
+        Acc before = thread_before;
+#pragma unroll
+        for (int j = 0; j < ITEMS; j++) {
+          if (j < count[p]) {
+            const Acc upto = thread_has ? op.combine(thread_before, x[p][j]) : x[p][j];
+            op.store(part_base + tid * ITEMS + j, has_before, before, upto);
+            before = upto;
+            has_before = true;
+          }
+        }
       }
+      if (p + 1 < SUB) join(op, part_has, part_before, true, s_part(p));
     }
   }
 }
@@ -277,7 +309,7 @@ void scan_engine(void* stream_, std::int64_t n, Op op) {
   static_assert(std::is_trivially_copyable<Acc>::value, "cdna4 scan: the accumulator type must be trivially copyable");
   if (n <= 0) return;
   hipStream_t s = static_cast<hipStream_t>(stream_);
-  constexpr std::int64_t kTile = (std::int64_t)kScanBlock * scan_items(sizeof(Acc));
+  constexpr std::int64_t kTile = (std::int64_t)kScanBlock * scan_items(sizeof(Acc)) * scan_parts(sizeof(Acc));
   const std::int64_t tiles = (n + kTile - 1) / kTile;
   const std::int64_t nwords = tiles * scan_desc<Acc>::NW + 1;
   temporary_storage tmp((std::size_t)nwords * sizeof(unsigned long long), stream_);

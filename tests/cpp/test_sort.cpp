@@ -168,4 +168,59 @@ void TestSortRawPointersAndSubrange() {
 }
 DECLARE_UNITTEST(TestSortRawPointersAndSubrange);
 
+// Floating-point keys: host and device ranges give the same order bit for bit — the total order of
+// the reference's radix encoding (thrust/system/detail/sequential/stable_radix_sort.inl:43-139):
+// -NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN, equal keys in input order; descending is the
+// stable mirror image.
+template <class T, class U>
+void TestSortFloatTotalOrderHostAndDevice() {
+  const T nan = std::numeric_limits<T>::quiet_NaN(), inf = std::numeric_limits<T>::infinity(), tiny = std::numeric_limits<T>::denorm_min();
+  const T specials[] = {T(0), -T(0), nan, -nan, inf, -inf, tiny, -tiny, T(1), T(-1)};
+  const std::size_t n = 100000;
+  thrust::host_vector<T> h(n);
+  std::uint64_t s = 5;
+  for (std::size_t i = 0; i < n; i++) {
+    const std::uint64_t r = unittest::splitmix64(s);
+    h[i] = (r & 3) == 0 ? specials[(r >> 2) % 10] : (T)((double)(r >> 11) / 9007199254740992.0 * 8.0 - 4.0);
+  }
+  thrust::host_vector<int> hv(n);
+  for (std::size_t i = 0; i < n; i++) hv[i] = (int)i;
+  auto bits = [](const thrust::host_vector<T>& v) {
+    thrust::host_vector<U> b(v.size());
+    std::memcpy(b.data(), v.data(), v.size() * sizeof(T));
+    return b;
+  };
+  for (int descending = 0; descending < 2; descending++) {
+    thrust::host_vector<T> hk = h;
+    thrust::host_vector<int> hvals = hv;
+    thrust::device_vector<T> dk = h;
+    thrust::device_vector<int> dvals = hv;
+    if (descending) {
+      thrust::sort_by_key(hk.begin(), hk.end(), hvals.begin(), thrust::greater<T>());
+      thrust::sort_by_key(dk.begin(), dk.end(), dvals.begin(), thrust::greater<T>());
+    } else {
+      thrust::sort_by_key(hk.begin(), hk.end(), hvals.begin());
+      thrust::sort_by_key(dk.begin(), dk.end(), dvals.begin());
+    }
+    ASSERT_EQUAL(bits(thrust::host_vector<T>(dk)), bits(hk));
+    ASSERT_EQUAL(dvals, hvals);
+    thrust::host_vector<T> hs = h;
+    thrust::device_vector<T> ds = h;
+    if (descending) {
+      thrust::sort(hs.begin(), hs.end(), thrust::greater<T>());
+      thrust::sort(ds.begin(), ds.end(), thrust::greater<T>());
+    } else {
+      thrust::sort(hs.begin(), hs.end());
+      thrust::sort(ds.begin(), ds.end());
+    }
+    ASSERT_EQUAL(bits(thrust::host_vector<T>(ds)), bits(hs));
+    ASSERT_TRUE(std::signbit(hs[descending ? n - 1 : 0]) && std::isnan(hs[descending ? n - 1 : 0]));  // -NaN at the low end
+  }
+}
+void TestSortFloatTotalOrder() {
+  TestSortFloatTotalOrderHostAndDevice<float, std::uint32_t>();
+  TestSortFloatTotalOrderHostAndDevice<double, std::uint64_t>();
+}
+DECLARE_UNITTEST(TestSortFloatTotalOrder);
+
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
