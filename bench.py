@@ -158,6 +158,16 @@ def main():
         ms = timed(fn, restore, 5, 1)
         assert torch.equal(k0[v.long()], k), "sort_by_key: values are not the permutation of the keys"
         add_extra("sort_by_key_u64_u32", n, ms, 200.0 * n, "Gkeys/s")
+        # the same call on keys whose upper bytes are all alike (64-bit keys that hold 32-bit numbers;
+        # all keys equal): places where every key has the same digit are skipped on the device
+        for label, keys in (("keys_below_2^32", k0 & 0xFFFFFFFF), ("all_keys_equal", torch.full_like(k0, 42))):
+            def restore_low(keys=keys):
+                k.copy_(keys)
+                v.copy_(v0)
+            ms = timed(fn, restore_low, 5, 1)
+            assert torch.equal(keys[v.long()], k) and bool((k[1:] >= k[:-1]).all())
+            extras[f"sort_by_key_u64_u32_{label}"] = {"value": round(n / float(np.median(ms)) / 1e6, 3), "unit": "Gkeys/s",
+                                                      "ms": round(float(np.median(ms)), 4)}
 
     def extra_scan(dtype_name):
         if dtype_name == "i32":

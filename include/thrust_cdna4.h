@@ -72,6 +72,8 @@ const char* thrust_cdna4_error_string(int code);
  * (sequential/stable_radix_sort.inl:43-139) — for floating-point keys that is the total
  * order -NaN < -inf < ... < -0 < +0 < ... < +inf < +NaN.  `descending != 0` gives the
  * order of thrust::greater (sequential/sort.inl:54-75).  n must be < 2^32 - 1.
+ * A pass over a digit place at which all keys agree (64-bit keys holding small numbers, constant
+ * fields, all keys equal) is skipped on the device; the result is the same, the call is faster.
  */
 int thrust_cdna4_sort_keys(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
                            int64_t n, int descending, void* stream);

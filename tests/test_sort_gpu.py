@@ -226,3 +226,42 @@ def test_sort_beyond_2p30_items():
     assert bool((k[1:] >= k[:-1]).all())
     assert bool(((k[1:] > k[:-1]) | (v[1:] > v[:-1])).all())  # equal keys keep their input order
     assert bool((src[v.long()] == k).all())
+
+
+# Places where every key has the same digit are skipped on the device (the identity for a stable
+# sort), and the number of passes that run stays even so that the result ends in the caller's
+# buffer.  Every pattern of constant and varying bytes must give the oracle's result, for keys and
+# for pairs, in both tile configurations (n below and above the small-tile limit).
+def _masked_keys(seed, n, dtype, vary_mask, constant):
+    k = random_ints(seed, n, dtype).astype(dtype)
+    u = k.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[k.dtype.itemsize])
+    u &= u.dtype.type(vary_mask)
+    u |= u.dtype.type(constant & ~vary_mask & (2 ** (8 * u.dtype.itemsize) - 1))
+    return u.view(dtype)
+
+
+@pytest.mark.parametrize("dtype,patterns", [
+    (np.uint32, [(0x000000FF, 0), (0x0000FFFF, 0xAB000000), (0xFF00FFFF, 0x00CD0000), (0xFF000000, 0x00123456),
+                 (0x00FFFF00, 0), (0x00000000, 0xDEADBEEF), (0x00FF0000, 0x11000022)]),
+    (np.int32, [(0x000000FF, 0), (0x000000FF, 0xFFFFFF00), (0x800000FF, 0), (0x00FF00FF, 0x7F000000)]),
+    (np.uint64, [(0x00000000000FFFFF, 0), (0x00000000FFFFFFFF, 0), (0xFFFF00000000FFFF, 0x0000ABCDEF000000),
+                 (0x0000000000000000, 42), (0x00000000000000FF, 0x0100000000000000), (0xFF00FF00FF00FF00, 0x0011002200330044)]),
+    (np.int64, [(0x00000000000FFFFF, 0), (0x80000000000000FF, 0), (0x00000000000000FF, 0xFFFFFFFFFFFFFF00)]),
+    (np.uint16, [(0x00FF, 0x1200), (0xFF00, 0x0034), (0x0000, 0x5678)]),
+    (np.float32, [(0x007FFFFF, 0x3F800000), (0x80000000, 0x3F800000), (0x000000FF, 0xBF800000)]),
+])
+def test_sort_skips_places_where_all_keys_agree(dtype, patterns):
+    for n in [4097, 70001, (1 << 21) + 77, (1 << 22) + 5]:
+        for vary, const in patterns:
+            for descending in (False, True):
+                k = _masked_keys(n + (vary & 0xFFFF), n, dtype, vary, const)
+                d = dev(k)
+                thrust_amd.sort(d, descending)
+                assert same_bits(host(d), oracle.sort_keys(k, descending)), (n, hex(vary), hex(const), descending)
+            # pairs: stability shows in the values
+            k = _masked_keys(n + 1, n, dtype, vary, const)
+            v = np.arange(n, dtype=np.uint32)
+            dk, dv = dev(k), dev(v)
+            thrust_amd.sort_by_key(dk, dv)
+            ek, ev = oracle.sort_pairs(k, v)
+            assert same_bits(host(dk), ek) and same_bits(host(dv), ev), (n, hex(vary), hex(const))

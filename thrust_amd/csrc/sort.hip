@@ -149,18 +149,50 @@ __global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const U* __res
 // ---------------------------------------------------------------------------------------
 // 2. Exclusive scan of the 256 bins of each digit place (one workgroup per place)
 // ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void radix_bins_kernel(uint32_t* ghist) {
+// One workgroup handles all P places, and then decides which passes run.  A place where every
+// key has the same digit is the identity permutation for a stable sort, so its pass is skipped
+// (64-bit keys that hold small numbers, keys with constant fields, all-equal keys).  The number of
+// passes that run is kept even, so that the result ends in the caller's buffer without a copy: if
+// an odd number of places need their pass, one of the skippable ones runs as well.  The decision
+// travels in the pass's ticket counter, which every workgroup of the pass reads anyway: the
+// counter starts at kPassSkipped for a pass that does not run and at kPassReadsAlt for one whose
+// input is the alternate buffer; the tile number is in the low bits.  With skipping off every
+// pass runs (places = 1: the caller copies the result back).
+constexpr uint32_t kPassSkipped = 0x80000000u, kPassReadsAlt = 0x40000000u, kTicketMask = 0x3FFFFFFFu;
+__global__ __launch_bounds__(256) void radix_bins_kernel(uint32_t* ghist, int places, uint32_t n, uint32_t* tickets, int skipping) {
   __shared__ uint32_t s_w[4];
+  __shared__ uint32_t s_same[8];  // places is at most 8
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  uint32_t* h = ghist + (size_t)blockIdx.x * kRadix;
-  const uint32_t c = h[tid];
-  uint32_t incl = wave_inclusive_scan(c, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-  if (lane == 63) s_w[wave] = incl;
+  if (tid < 8) s_same[tid] = 0;
+  for (int p = 0; p < places; p++) {
+    __syncthreads();
+    uint32_t* h = ghist + (size_t)p * kRadix;
+    const uint32_t c = h[tid];
+    if (c == n) s_same[p] = 1;  // all keys in one bin
+    uint32_t incl = wave_inclusive_scan(c, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+    if (lane == 63) s_w[wave] = incl;
+    __syncthreads();
+    uint32_t base = 0;
+    for (int w = 0; w < wave; w++) base += s_w[w];
+    h[tid] = base + incl - c;
+  }
   __syncthreads();
-  uint32_t base = 0;
-  for (int w = 0; w < wave; w++) base += s_w[w];
-  h[tid] = base + incl - c;
+  if (tid == 0) {
+    int needed = 0;
+    for (int p = 0; p < places; p++) needed += s_same[p] ? 0 : 1;
+    bool one_more = skipping && (needed & 1);  // keep the number of passes even
+    uint32_t reads_alt = 0;
+    for (int p = 0; p < places; p++) {
+      bool runs = !skipping || !s_same[p];
+      if (!runs && one_more) {
+        runs = true;
+        one_more = false;
+      }
+      tickets[p] = runs ? reads_alt : kPassSkipped;
+      if (runs) reads_alt ^= kPassReadsAlt;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -196,8 +228,7 @@ constexpr uint32_t kLookbackSpinLimit = 1u << 22;
 __device__ unsigned int g_lookback_timeouts;
 
 template <class U, int VB, bool FLOAT, int BLOCK, int IPT, int WPE, class D>
-__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) void onesweep_kernel(const U* __restrict__ kin, U* __restrict__ kout,
-                                                         const void* __restrict__ vin_, void* __restrict__ vout_,
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) void onesweep_kernel(U* kmain, U* kalt, void* vmain, void* valt,
                                                          int64_t n, U xor_mask, int shift,
                                                          const uint32_t* __restrict__ gbase,
                                                          D* desc, uint32_t* ticket) {
@@ -208,9 +239,6 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
   __shared__ OnesweepSmem<U, VB, BLOCK, IPT> sm;
   U* s_keys = reinterpret_cast<U*>(sm.exch);
   V* s_vals = reinterpret_cast<V*>(sm.exch);
-  const V* vin = static_cast<const V*>(vin_);
-  V* vout = static_cast<V*>(vout_);
-
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
@@ -221,7 +249,14 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
     for (int w = 0; w < NWAVES; w++) reinterpret_cast<uint32_t*>(sm.wave_cnt[w])[tid] = 0;
   }
   __syncthreads();
-  const int64_t tile = sm.tile;
+  const uint32_t ticket_word = sm.tile;  // tile number, and what radix_bins_kernel decided about this pass
+  if (ticket_word & kPassSkipped) return;  // every key has the same digit here
+  const bool from_alt = (ticket_word & kPassReadsAlt) != 0;
+  const U* __restrict__ kin = from_alt ? kalt : kmain;
+  U* __restrict__ kout = from_alt ? kmain : kalt;
+  const V* __restrict__ vin = static_cast<const V*>(from_alt ? valt : vmain);
+  V* __restrict__ vout = static_cast<V*>(from_alt ? vmain : valt);
+  const int64_t tile = ticket_word & kTicketMask;
   const int64_t base = tile * TILE;
   const int valid = (int)((n - base) < (int64_t)TILE ? (n - base) : (int64_t)TILE);
   const bool full = valid == TILE;
@@ -675,17 +710,18 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   if (hblocks > cus) hblocks = cus;  // one workgroup per CU, eight loads in flight per thread: 1 % of a 2^28 sort over two with two
   TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(kHistThreads), stream,
              kbuf[0], n, xor_mask, ghist, vec_ok);
-  TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(P), dim3(256), stream, ghist);
-  int cur = 0;
+  // passes over places where all keys agree are skipped on the device; with an even number of
+  // places the passes that run are an even number too and the result ends in the caller's buffer
+  constexpr int kSkipping = (P % 2 == 0) ? 1 : 0;
+  TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(1), dim3(256), stream, ghist, P, (uint32_t)n, tickets, kSkipping);
   for (int p = 0; p < P; p++) {
     TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT, C::WPE, D>), dim3((unsigned)plan.ntiles),
-               dim3(C::BLOCK), stream, kbuf[cur], kbuf[cur ^ 1], vbuf[cur], vbuf[cur ^ 1], n, xor_mask, 8 * p,
+               dim3(C::BLOCK), stream, kbuf[0], kbuf[1], static_cast<void*>(vbuf[0]), static_cast<void*>(vbuf[1]), n, xor_mask, 8 * p,
                ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix, tickets + p);
-    cur ^= 1;
   }
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  if (cur == 1) {  // odd number of passes: bring the result home
+  if (P % 2 == 1) {  // an odd number of passes, none skipped: bring the result home
     e = copy_async(kbuf[0], kbuf[1], (size_t)n * sizeof(U), stream);
     if (e != hipSuccess) return e;
     if (VB) e = copy_async(vbuf[0], vbuf[1], (size_t)n * VB, stream);
