@@ -74,6 +74,7 @@ const char* thrust_cdna4_error_string(int code);
  * order of thrust::greater (sequential/sort.inl:54-75).  n must be < 2^32 - 1.
  * A pass over a digit place at which all keys agree (64-bit keys holding small numbers, constant
  * fields, all keys equal) is skipped on the device; the result is the same, the call is faster.
+ * One-byte keys are not moved at all: the sorted sequence is written from their histogram.
  */
 int thrust_cdna4_sort_keys(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
                            int64_t n, int descending, void* stream);
@@ -109,9 +110,9 @@ int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int op, int exc
  * arguments, results and kernels as thrust_cdna4_scan without `temp` / `temp_bytes`: the tile
  * descriptors live in a fixed 256 KiB array inside the library's device image (one copy per GPU,
  * held until the process ends), whose device address is looked up on the first call on each
- * device; no call allocates or frees memory.  Limit: at most 16384 tiles, i.e.
- * n <= 2^29 elements of 1, 2 or 4 bytes (32768 per tile) and n <= 2^28 elements of 8 bytes
- * (16384 per tile); a larger n returns hipErrorOutOfMemory (2) before anything else is looked
+ * device; no call allocates or frees memory.  Limit: at most 16384 tiles of 128 KiB, i.e. 2 GiB
+ * of input (n <= 2^31 elements of 1 byte, 2^30 of 2 bytes, 2^29 of 4 bytes, 2^28 of 8 bytes);
+ * a larger n returns hipErrorOutOfMemory (2) before anything else is looked
  * at, and launches nothing.  All calls on one GPU share the array: calls
  * that overlap in time on one GPU (different streams, or different host threads) race and must
  * be serialised by the caller; back-to-back calls on one stream are fine (each call clears the

@@ -78,7 +78,7 @@ def test_bad_arguments_return_an_error_code(bad):
 
 def test_scan_static_refuses_sizes_beyond_its_array_before_it_touches_a_device():
     L = capi.lib()
-    for code, limit in [(capi.I32, 1 << 29), (capi.U8, 1 << 29), (capi.I16, 1 << 29), (capi.F32, 1 << 29),
+    for code, limit in [(capi.I32, 1 << 29), (capi.U8, 1 << 31), (capi.I16, 1 << 30), (capi.F32, 1 << 29),
                         (capi.I64, 1 << 28), (capi.F64, 1 << 28)]:
         assert L.thrust_cdna4_scan_static(code, capi.PLUS, 0, None, None, limit + 1, None, None) == 2
         assert L.thrust_cdna4_scan_static(code, capi.PLUS, 0, None, None, limit, None, None) == 1  # NULL ranges

@@ -265,3 +265,29 @@ def test_sort_skips_places_where_all_keys_agree(dtype, patterns):
             thrust_amd.sort_by_key(dk, dv)
             ek, ev = oracle.sort_pairs(k, v)
             assert same_bits(host(dk), ek) and same_bits(host(dv), ev), (n, hex(vary), hex(const))
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.int8])
+def test_sort_one_byte_keys_by_counting(dtype):
+    """One-byte keys without values are written from their histogram (no key moves): all run shapes
+    — uniform, few distinct values with empty bins between them, one value, the extreme values, ends
+    of the input inside a 16-byte piece — at any alignment, both directions, against the oracle."""
+    info = np.iinfo(dtype)
+    for n in [4097, 4111, 70001, (1 << 21) + 77, (1 << 22) + 13]:
+        rng = np.random.default_rng(n)
+        cases = {
+            "uniform": rng.integers(info.min, info.max + 1, n).astype(dtype),
+            "three values": rng.choice(np.array([info.min, 7, info.max], dtype=dtype), n),
+            "one value": np.full(n, info.max, dtype=dtype),
+            "short runs at the ends": np.concatenate([np.full(n - 9, 5), np.arange(9) + info.min]).astype(dtype),
+            "skewed": np.minimum(rng.geometric(0.3, n), info.max).astype(dtype),
+        }
+        for name, k in cases.items():
+            for descending in (False, True):
+                for shift in (0, 1, 7):
+                    buf = torch.zeros(n + 32, dtype=torch.int8 if dtype == np.int8 else torch.uint8, device="cuda")
+                    view = buf[shift:shift + n]
+                    view.copy_(dev(k))
+                    thrust_amd.sort(view, descending)
+                    assert np.array_equal(host(view), oracle.sort_keys(k, descending)), (n, name, descending, shift)
+                    assert int(buf[:shift].sum()) == 0 and int(buf[shift + n:].sum()) == 0, "wrote outside the range"

@@ -64,7 +64,7 @@ def test_rejects_sizes_beyond_the_array_and_allocates_nothing():
     # One tile more than the array holds is refused with its own code before anything else is
     # looked at.  The calls pass NULL ranges, so nothing could be launched even if the size check
     # were wrong: they would then fail with code 1 instead of 2.
-    for code, limit in [(capi.I32, 1 << 29), (capi.U8, 1 << 29), (capi.I16, 1 << 29), (capi.F32, 1 << 29),
+    for code, limit in [(capi.I32, 1 << 29), (capi.U8, 1 << 31), (capi.I16, 1 << 30), (capi.F32, 1 << 29),
                         (capi.I64, 1 << 28), (capi.F64, 1 << 28)]:
         assert L.thrust_cdna4_scan_static(code, capi.PLUS, 0, None, None, limit + 1, None, _stream()) == 2
         assert L.thrust_cdna4_scan_static(code, capi.PLUS, 0, None, None, limit, None, _stream()) == 1

@@ -175,13 +175,206 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// The same scan for 1- and 2-byte elements.  Above, every element has a register of its own,
+// which holds narrow types to 64 elements per thread and a tile to 32 KiB: too little per ticket
+// and look-back.  Here the tile stays PACKED in registers (4 dwords per 16-byte chunk, 16 chunks
+// per thread: 256 bytes, as for the wide types); an element is unpacked where it is used — once
+// for the totals, once more when the results are formed and packed for the store.  The arithmetic
+// is a few operations per element and far below the memory time.
+// ---------------------------------------------------------------------------------------
+template <class T>
+__device__ inline T packed_get(const uint32_t (&r)[4], int j) {  // j is a constant after unrolling
+  constexpr int PER = 4 / (int)sizeof(T);
+  using U = typename unsigned_of<T>::type;
+  return (T)(U)(r[j / PER] >> ((j % PER) * 8 * (int)sizeof(T)));
+}
+template <class T>
+__device__ inline void packed_put(uint32_t (&r)[4], int j, T v) {
+  constexpr int PER = 4 / (int)sizeof(T);
+  using U = typename unsigned_of<T>::type;
+  const uint32_t w = (uint32_t)(U)v << ((j % PER) * 8 * (int)sizeof(T));
+  r[j / PER] = (j % PER) == 0 ? w : (r[j / PER] | w);
+}
+
+template <class T, class Op, int BLOCK, int CHUNKS, bool TICKET>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void scan_packed_kernel(const T* in, T* out, int64_t n, T init,
+                                                     int exclusive, uint64_t* desc,
+                                                     uint32_t* ticket, int vec_ok, int patience, int publish_delay) {
+  static_assert(sizeof(T) < 4, "1- and 2-byte elements");
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int NWAVES = BLOCK / kWave;
+  constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
+  using W = uint32_t;  // cross-lane traffic, LDS and descriptors carry a dword container
+  using U = typename unsigned_of<T>::type;
+
+  __shared__ W s_tot[CHUNKS * NWAVES];  // inclusive total of (chunk, wave), then its exclusive offset
+  __shared__ uint32_t s_tile;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const T id = Op::template identity<T>();
+  auto op = [](T a, T b) { return Op::template apply<T>(a, b); };
+  auto toW = [](T a) { return (W)(U)a; };
+  auto opW = [&](W a, W b) { return (W)(U)op((T)a, (T)b); };
+  const W idW = toW(id);
+
+  int64_t tile = blockIdx.x;
+  if constexpr (TICKET) {
+    if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+    __syncthreads();
+    tile = s_tile;
+  }
+  const int64_t base = tile * TILE;
+  // 128-bit accesses need no alignment here, so only the tile that the input ends in is special
+  (void)vec_ok;
+  const bool fast = base + TILE <= n;
+  const T* tin = in + base + (int64_t)tid * VEC;
+  T* tout = out + base + (int64_t)tid * VEC;
+
+  // The chunk that the input ends in is put together element by element (a loop with a computed
+  // shift, not unrolled: it runs once per call); chunks past the end hold the identity.
+  const uint32_t id_word = (uint32_t)(U)id * (sizeof(T) == 1 ? 0x01010101u : 0x00010001u);
+  auto load_tail = [&](const T* p, int count) {
+    uint64_t half[2] = {((uint64_t)id_word << 32) | id_word, ((uint64_t)id_word << 32) | id_word};
+#pragma unroll 1
+    for (int j = 0; j < count; j++) {
+      const int bit = j * 8 * (int)sizeof(T);
+      const uint64_t mask = (uint64_t)(U)~U(0) << (bit & 63);
+      const uint64_t e = (uint64_t)(U)p[j] << (bit & 63);
+      if (bit < 64) half[0] = (half[0] & ~mask) | e;
+      else half[1] = (half[1] & ~mask) | e;
+    }
+    tcd_v4u v;
+    v.x = (uint32_t)half[0]; v.y = (uint32_t)(half[0] >> 32); v.z = (uint32_t)half[1]; v.w = (uint32_t)(half[1] >> 32);
+    return v;
+  };
+  uint32_t x[CHUNKS][4];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; c++) {
+    tcd_v4u v;
+    if (fast) {
+      v = load16<tcd_v4u>(tin + c * BLOCK * VEC);
+    } else {
+      const int64_t left = n - (base + ((int64_t)c * BLOCK + tid) * VEC);  // elements from this chunk's first to the end
+      v.x = v.y = v.z = v.w = id_word;
+      if (left >= VEC) v = load16<tcd_v4u>(tin + c * BLOCK * VEC);
+      else if (left > 0) v = load_tail(tin + c * BLOCK * VEC, (int)left);
+    }
+    x[c][0] = v.x; x[c][1] = v.y; x[c][2] = v.z; x[c][3] = v.w;
+  }
+
+  // total of each 16-byte group, then a wave scan of the group totals
+  T excl[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; c++) {
+    T acc = packed_get<T>(x[c], 0);
+#pragma unroll
+    for (int j = 1; j < VEC; j++) acc = op(acc, packed_get<T>(x[c], j));
+    const W incl = wave_inclusive_scan(toW(acc), idW, opW);
+    excl[c] = (T)wave_shift_up1(incl, idW);
+    if (lane == kWave - 1) s_tot[c * NWAVES + wave] = incl;
+  }
+  __syncthreads();
+
+  // wave 0: exclusive scan of the (chunk, wave) totals in tile order, then the look-back
+  if (wave == 0) {
+    constexpr int NTOT = CHUNKS * NWAVES;
+    constexpr int PER = (NTOT + kWave - 1) / kWave;
+    W mine[PER];
+#pragma unroll
+    for (int q = 0; q < PER; q++) {
+      const int idx = lane * PER + q;
+      mine[q] = idx < NTOT ? s_tot[idx] : idW;
+      if (q > 0) mine[q] = opW(mine[q - 1], mine[q]);
+    }
+    const W incl = wave_inclusive_scan(mine[PER - 1], idW, opW);
+    const W tile_agg = readlane(incl, kWave - 1);
+    const W before = wave_shift_up1(incl, idW);  // totals of the lanes below
+    // descriptors carry sums of INPUT elements only; `init` is applied by every tile to its own prefix
+    W prefix = idW;
+    if (tile == 0) {
+      for (int i = 0; i < publish_delay; i++) __builtin_amdgcn_s_sleep(127);  // test knob, 0 in normal use
+      if (lane == 0) TileDesc<W>::store(desc, 0, kInclusive, tile_agg);
+    } else {
+      if (lane == 0) TileDesc<W>::store(desc, tile, kPartial, tile_agg);
+      if constexpr (TICKET) {
+        prefix = wave_lookback<W>(desc, tile, idW, opW);
+      } else {
+        // the aggregate of an earlier tile (always a whole one), straight from the input
+        const auto aggregate_of = [&](int64_t t) -> W {
+          const T* p = in + t * TILE + lane;
+          T acc = p[0];
+#pragma unroll 8
+          for (int k = 1; k < (int)(TILE / kWave); k++) acc = op(acc, p[(int64_t)k * kWave]);
+          return readlane(wave_inclusive_scan(toW(acc), idW, opW), kWave - 1);
+        };
+        prefix = wave_lookback_or_compute<W>(desc, tile, idW, opW, patience, aggregate_of);
+      }
+      if (lane == 0) TileDesc<W>::store(desc, tile, kInclusive, opW(prefix, tile_agg));
+    }
+    if (exclusive) prefix = opW(toW(init), prefix);
+    const W base_w = opW(prefix, before);
+#pragma unroll
+    for (int q = 0; q < PER; q++) {
+      const int idx = lane * PER + q;
+      if (idx < NTOT) s_tot[idx] = q == 0 ? base_w : opW(base_w, mine[q - 1]);
+    }
+  }
+  __syncthreads();
+
+  // results: the running value starts at the offset of the element's group and walks the group.
+  // (The packed words pass through an empty asm first: the elements are unpacked again here, not
+  // kept in registers of their own since the totals were formed.)
+#pragma unroll
+  for (int c = 0; c < CHUNKS; c++) {
+    T run = op((T)s_tot[c * NWAVES + wave], excl[c]);
+    uint32_t src[4], r[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      src[q] = x[c][q];
+      asm volatile("" : "+v"(src[q]));
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+      const T e = packed_get<T>(src, j);
+      if (exclusive) {
+        packed_put<T>(r, j, run);
+        run = op(run, e);
+      } else {
+        run = op(run, e);
+        packed_put<T>(r, j, run);
+      }
+    }
+    tcd_v4u v;
+    v.x = r[0]; v.y = r[1]; v.z = r[2]; v.w = r[3];
+    if (fast) {
+      store16(tout + c * BLOCK * VEC, v);
+    } else {
+      const int64_t left = n - (base + ((int64_t)c * BLOCK + tid) * VEC);
+      if (left >= VEC) {
+        store16(tout + c * BLOCK * VEC, v);
+      } else if (left > 0) {
+        const uint64_t half[2] = {((uint64_t)r[1] << 32) | r[0], ((uint64_t)r[3] << 32) | r[2]};
+        T* p = tout + c * BLOCK * VEC;
+#pragma unroll 1
+        for (int j = 0; j < (int)left; j++) {
+          const int bit = j * 8 * (int)sizeof(T);
+          p[j] = (T)(U)((bit < 64 ? half[0] : half[1]) >> (bit & 63));
+        }
+      }
+    }
+  }
+}
+
 template <class T>
 struct ScanConfig {
-  // 256 bytes per thread for 4- and 8-byte elements (128 KiB tiles: fewer tickets and look-backs
-  // per byte; measured best on MI355X: 64 KiB tiles are 10 % slower, 192 KiB tiles 3 %); fewer
-  // chunks for narrow types, which hold one element per register.
+  // 256 bytes per thread (128 KiB tiles: fewer tickets and look-backs per byte; measured best on
+  // MI355X: 64 KiB tiles are 10 % slower, 192 KiB tiles 3 %); 1- and 2-byte elements stay packed
+  // in their registers (scan_packed_kernel).
   static constexpr int BLOCK = 512;
-  static constexpr int CHUNKS = sizeof(T) >= 4 ? 16 : (sizeof(T) == 2 ? 8 : 4);
+  static constexpr int CHUNKS = 16;
   static constexpr int64_t TILE = (int64_t)BLOCK * (16 / sizeof(T)) * CHUNKS;
   using P = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
 };
@@ -211,14 +404,18 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   uint64_t* desc = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256);
   // 128-bit accesses need no more than the elements' own alignment (see load16)
   const int vec_ok = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & (sizeof(T) - 1)) == 0;
-  if (!single && ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T))) {
-    TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS, true>), dim3((unsigned)ntiles), dim3(C::BLOCK),
-               stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
-               desc, ticket, vec_ok, 0, 0);
+  const bool ticketed = !single && ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T));
+  const int patience = ticketed ? 0 : lookback_patience(), delay = ticketed ? 0 : lookback_test_publish_delay();
+  auto launch = [&](auto kernel) {
+    TCD_LAUNCH("scan_kernel", kernel, dim3((unsigned)ntiles), dim3(C::BLOCK), stream, static_cast<const T*>(in),
+               static_cast<T*>(out), n, iv, exclusive, desc, ticket, vec_ok, patience, delay);
+  };
+  if constexpr (sizeof(T) < 4) {
+    if (ticketed) launch(scan_packed_kernel<T, Op, C::BLOCK, C::CHUNKS, true>);
+    else launch(scan_packed_kernel<T, Op, C::BLOCK, C::CHUNKS, false>);
   } else {
-    TCD_LAUNCH("scan_kernel", (scan_kernel<T, Op, C::BLOCK, C::CHUNKS, false>), dim3((unsigned)ntiles), dim3(C::BLOCK),
-               stream, static_cast<const T*>(in), static_cast<T*>(out), n, iv, exclusive,
-               desc, ticket, vec_ok, lookback_patience(), lookback_test_publish_delay());
+    if (ticketed) launch(scan_kernel<T, Op, C::BLOCK, C::CHUNKS, true>);
+    else launch(scan_kernel<T, Op, C::BLOCK, C::CHUNKS, false>);
   }
   return hipGetLastError();
 }
@@ -249,7 +446,7 @@ extern "C" int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int 
 // library's device image instead of caller-provided temporary storage.
 // ---------------------------------------------------------------------------------------
 namespace tcd {
-constexpr int64_t kStaticScanMaxTiles = 16384;  // 2^29 elements of up to 4 bytes, 2^28 of 8 bytes
+constexpr int64_t kStaticScanMaxTiles = 16384;  // tiles of 128 KiB: 2 GiB of input
 constexpr size_t kStaticScanScratchBytes = 256 + (size_t)kStaticScanMaxTiles * 16;  // ticket + 16 B per tile
 static __device__ __align__(256) unsigned char scratch[kStaticScanScratchBytes];
 

@@ -657,18 +657,52 @@ struct SortPlan {
   int64_t ntiles;
 };
 
+// One-byte keys without values are not moved at all: their sorted sequence is the 256 runs that the
+// histogram describes.  Thread t writes 16 output bytes at a time; the digit of its first byte is
+// found by bisection over the 256 run starts, and nearly every 16-byte piece lies inside one run.
+constexpr int kFillThreads = 256;
+__global__ __launch_bounds__(kFillThreads) void counting_fill_kernel(uint8_t* out, int64_t n, uint8_t xor_mask,
+                                                                   const uint32_t* __restrict__ gbase) {
+  __shared__ uint32_t s_start[kRadix + 1];
+  s_start[threadIdx.x] = gbase[threadIdx.x];
+  if (threadIdx.x == 0) s_start[kRadix] = (uint32_t)n;  // n < 2^32 - 1
+  __syncthreads();
+  const int64_t pieces = (n + 15) / 16;
+  for (int64_t c = (int64_t)blockIdx.x * kFillThreads + threadIdx.x; c < pieces; c += (int64_t)gridDim.x * kFillThreads) {
+    const int64_t p0 = c * 16;
+    int d = 0;  // the last digit whose run starts at or before p0 (empty runs before it share its start)
+#pragma unroll
+    for (int step = kRadix / 2; step > 0; step >>= 1)
+      if ((int64_t)s_start[d + step] <= p0) d += step;
+    if ((int64_t)s_start[d + 1] >= p0 + 16) {  // one run covers the piece (and the piece lies inside the output)
+      const uint32_t w = (uint32_t)(uint8_t)(d ^ xor_mask) * 0x01010101u;
+      tcd_v4u v;
+      v.x = v.y = v.z = v.w = w;
+      store16(out + p0, v);
+    } else {
+      const int count = (int)(n - p0 < 16 ? n - p0 : 16);
+#pragma unroll 1
+      for (int j = 0; j < count; j++) {
+        while ((int64_t)s_start[d + 1] <= p0 + j) d++;  // ends: s_start[256] = n > p0 + j
+        out[p0 + j] = (uint8_t)(d ^ xor_mask);
+      }
+    }
+  }
+}
+
 template <class U, int VB, class C, class D>
 static SortPlan make_plan(int64_t n) {
   constexpr int P = sizeof(U);
   SortPlan p{};
   p.ntiles = ceil_div(n, C::TILE);
   size_t off = 0;
-  p.keys_alt = off; off += align_up((size_t)n * sizeof(U), 256);
+  constexpr bool kCounting = sizeof(U) == 1 && VB == 0;  // histogram and fill: no alternate buffer, no descriptors
+  p.keys_alt = off; off += kCounting ? 0 : align_up((size_t)n * sizeof(U), 256);
   p.vals_alt = off; off += align_up((size_t)n * VB, 256);
   p.zero_begin = off;
   p.hist = off; off += align_up((size_t)P * kRadix * 4, 256);
   p.tickets = off; off += 256;
-  p.desc = off; off += align_up((size_t)P * p.ntiles * kRadix * sizeof(D), 256);
+  p.desc = off; off += kCounting ? 0 : align_up((size_t)P * p.ntiles * kRadix * sizeof(D), 256);
   p.zero_bytes = off - p.zero_begin;
   p.total = off;
   return p;
@@ -714,6 +748,13 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   // places the passes that run are an even number too and the result ends in the caller's buffer
   constexpr int kSkipping = (P % 2 == 0) ? 1 : 0;
   TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(1), dim3(256), stream, ghist, P, (uint32_t)n, tickets, kSkipping);
+  if constexpr (sizeof(U) == 1 && VB == 0) {
+    int64_t fblocks = ceil_div(n, (int64_t)kFillThreads * 16 * 4);
+    if (fblocks > (int64_t)cus * 8) fblocks = (int64_t)cus * 8;
+    TCD_LAUNCH("counting_fill_kernel", counting_fill_kernel, dim3((unsigned)fblocks), dim3(kFillThreads), stream,
+               reinterpret_cast<uint8_t*>(kbuf[0]), n, (uint8_t)xor_mask, ghist);
+    return hipGetLastError();
+  }
   for (int p = 0; p < P; p++) {
     TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT, C::WPE, D>), dim3((unsigned)plan.ntiles),
                dim3(C::BLOCK), stream, kbuf[0], kbuf[1], static_cast<void*>(vbuf[0]), static_cast<void*>(vbuf[1]), n, xor_mask, 8 * p,
