@@ -25,4 +25,15 @@ template <class P> struct is_policy {
   static constexpr bool value = std::is_base_of<system::cdna4::execution_policy<P>, P>::value || std::is_same<P, system::cpp::detail::par_t>::value;
 };
 template <class P> using enable_if_policy = typename std::enable_if<is_policy<P>::value, int>::type;
+// The policy an algorithm called WITHOUT one runs under, from its first iterator's system
+// (thrust/detail/sort.inl:202-215: `System system; sort(select_system(system), ...)`): the device
+// system's default policy — or, for an iterator retagged with a user's policy type
+// (thrust::retag<my_tag>(it), my_tag derived from thrust::device_execution_policy<my_tag>), a
+// default-constructed object of that type, so that the user's overloads for it are found.
+template <class Iterator, class Tag> class tagged_iterator;
+template <class It> struct implicit_policy { typedef system::cdna4::detail::par_t type; };
+template <class I, class Tag> struct implicit_policy<tagged_iterator<I, Tag>> {
+  typedef typename std::conditional<std::is_base_of<system::cdna4::execution_policy<Tag>, Tag>::value, Tag,
+                                    system::cdna4::detail::par_t>::type type;
+};
 }}  // namespace thrust::detail

@@ -54,15 +54,17 @@ void scan_dispatch(const Policy& exec, In in, Out out, std::int64_t n, T init, O
 }
 }  // namespace detail
 
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 // The accumulator of an inclusive scan has the input's value type (thrust/system/cuda/detail/scan.h:63).
 template <class D, class InIt, class OutIt, class Op>
 OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, Op op) {
-  typedef typename detail::elem<InIt>::type T;
-  typedef typename detail::unwrap_iterator<InIt>::type In;
-  typedef typename detail::unwrap_iterator<OutIt>::type Out;
+  typedef typename thrust::detail::elem<InIt>::type T;
+  typedef typename thrust::detail::unwrap_iterator<InIt>::type In;
+  typedef typename thrust::detail::unwrap_iterator<OutIt>::type Out;
   const std::int64_t n = (std::int64_t)(last - first);
-  detail::scan_dispatch<false>(exec.derived(), detail::unwrap(first), detail::unwrap(result), n, T(), op,
-                               std::integral_constant<bool, detail::scan_has_kernel<T, In, Out, Op>::value>());
+  thrust::detail::scan_dispatch<false>(exec.derived(), thrust::detail::unwrap(first), thrust::detail::unwrap(result), n, T(), op,
+                               std::integral_constant<bool, thrust::detail::scan_has_kernel<T, In, Out, Op>::value>());
   return result + n;
 }
 template <class D, class InIt, class OutIt>
@@ -72,11 +74,11 @@ OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first,
 // The accumulator of an exclusive scan has the type of `init` (thrust/system/cuda/detail/scan.h:142-154).
 template <class D, class InIt, class OutIt, class T, class Op>
 OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, T init, Op op) {
-  typedef typename detail::unwrap_iterator<InIt>::type In;
-  typedef typename detail::unwrap_iterator<OutIt>::type Out;
+  typedef typename thrust::detail::unwrap_iterator<InIt>::type In;
+  typedef typename thrust::detail::unwrap_iterator<OutIt>::type Out;
   const std::int64_t n = (std::int64_t)(last - first);
-  detail::scan_dispatch<true>(exec.derived(), detail::unwrap(first), detail::unwrap(result), n, init, op,
-                              std::integral_constant<bool, detail::scan_has_kernel<T, In, Out, Op>::value>());
+  thrust::detail::scan_dispatch<true>(exec.derived(), thrust::detail::unwrap(first), thrust::detail::unwrap(result), n, init, op,
+                              std::integral_constant<bool, thrust::detail::scan_has_kernel<T, In, Out, Op>::value>());
   return result + n;
 }
 template <class D, class InIt, class OutIt, class T>
@@ -85,8 +87,32 @@ OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first,
 }
 template <class D, class InIt, class OutIt>
 OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result) {
-  typedef typename detail::elem<InIt>::type V;
+  typedef typename thrust::detail::elem<InIt>::type V;
   return exclusive_scan(exec, first, last, result, V(), plus<>());  // thrust/system/cuda/detail/scan.h:347-348
+}
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/scan.inl:35-48):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class InIt, class OutIt, class Op>
+OutIt inclusive_scan(const detail::execution_policy_base<D>& exec, InIt first, InIt last, OutIt result, Op op) {
+  return inclusive_scan(detail::derived_cast(detail::strip_const(exec)), first, last, result, op);
+}
+template <class D, class InIt, class OutIt>
+OutIt inclusive_scan(const detail::execution_policy_base<D>& exec, InIt first, InIt last, OutIt result) {
+  return inclusive_scan(detail::derived_cast(detail::strip_const(exec)), first, last, result);
+}
+template <class D, class InIt, class OutIt, class T, class Op>
+OutIt exclusive_scan(const detail::execution_policy_base<D>& exec, InIt first, InIt last, OutIt result, T init, Op op) {
+  return exclusive_scan(detail::derived_cast(detail::strip_const(exec)), first, last, result, init, op);
+}
+template <class D, class InIt, class OutIt, class T>
+OutIt exclusive_scan(const detail::execution_policy_base<D>& exec, InIt first, InIt last, OutIt result, T init) {
+  return exclusive_scan(detail::derived_cast(detail::strip_const(exec)), first, last, result, init);
+}
+template <class D, class InIt, class OutIt>
+OutIt exclusive_scan(const detail::execution_policy_base<D>& exec, InIt first, InIt last, OutIt result) {
+  return exclusive_scan(detail::derived_cast(detail::strip_const(exec)), first, last, result);
 }
 
 // ===================================================================== scan, host
@@ -131,20 +157,20 @@ OutIt exclusive_scan(const system::cpp::detail::par_t& e, InIt first, InIt last,
 
 // ===================================================================== scan, no policy
 template <class InIt, class OutIt, detail::enable_if_device<InIt> = 0>
-OutIt inclusive_scan(InIt f, InIt l, OutIt r) { return inclusive_scan(device, f, l, r); }
+OutIt inclusive_scan(InIt f, InIt l, OutIt r) { return inclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r); }
 template <class InIt, class OutIt, class Op, detail::enable_if_device<InIt> = 0>
-OutIt inclusive_scan(InIt f, InIt l, OutIt r, Op op) { return inclusive_scan(device, f, l, r, op); }
+OutIt inclusive_scan(InIt f, InIt l, OutIt r, Op op) { return inclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r, op); }
 template <class InIt, class OutIt, detail::enable_if_host<InIt> = 0>
 OutIt inclusive_scan(InIt f, InIt l, OutIt r) { return inclusive_scan(host, f, l, r); }
 template <class InIt, class OutIt, class Op, detail::enable_if_host<InIt> = 0>
 OutIt inclusive_scan(InIt f, InIt l, OutIt r, Op op) { return inclusive_scan(host, f, l, r, op); }
 
 template <class InIt, class OutIt, detail::enable_if_device<InIt> = 0>
-OutIt exclusive_scan(InIt f, InIt l, OutIt r) { return exclusive_scan(device, f, l, r); }
+OutIt exclusive_scan(InIt f, InIt l, OutIt r) { return exclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r); }
 template <class InIt, class OutIt, class T, detail::enable_if_device<InIt> = 0>
-OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init) { return exclusive_scan(device, f, l, r, init); }
+OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init) { return exclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r, init); }
 template <class InIt, class OutIt, class T, class Op, detail::enable_if_device<InIt> = 0>
-OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init, Op op) { return exclusive_scan(device, f, l, r, init, op); }
+OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init, Op op) { return exclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r, init, op); }
 template <class InIt, class OutIt, detail::enable_if_host<InIt> = 0>
 OutIt exclusive_scan(InIt f, InIt l, OutIt r) { return exclusive_scan(host, f, l, r); }
 template <class InIt, class OutIt, class T, detail::enable_if_host<InIt> = 0>
@@ -182,20 +208,22 @@ void scan_by_key_dispatch(const Policy& exec, KIn keys, VIn vals, Out out, std::
 }
 }  // namespace detail
 
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 // The accumulator has the value input's type for the inclusive form and the type of `init` for
 // the exclusive one (thrust/system/cuda/detail/scan_by_key.h:69-282).
 template <class D, class KIt, class VIt, class OutIt, class Pred, class Op>
 OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
                             OutIt result, Pred pred, Op op) {
-  typedef typename detail::elem<KIt>::type K;
-  typedef typename detail::elem<VIt>::type V;
-  typedef typename detail::unwrap_iterator<KIt>::type KIn;
-  typedef typename detail::unwrap_iterator<VIt>::type VIn;
-  typedef typename detail::unwrap_iterator<OutIt>::type Out;
+  typedef typename thrust::detail::elem<KIt>::type K;
+  typedef typename thrust::detail::elem<VIt>::type V;
+  typedef typename thrust::detail::unwrap_iterator<KIt>::type KIn;
+  typedef typename thrust::detail::unwrap_iterator<VIt>::type VIn;
+  typedef typename thrust::detail::unwrap_iterator<OutIt>::type Out;
   const std::int64_t n = (std::int64_t)(klast - kfirst);
-  detail::scan_by_key_dispatch<false, K>(exec.derived(), detail::unwrap(kfirst), detail::unwrap(vfirst), detail::unwrap(result), n,
+  thrust::detail::scan_by_key_dispatch<false, K>(exec.derived(), thrust::detail::unwrap(kfirst), thrust::detail::unwrap(vfirst), thrust::detail::unwrap(result), n,
                                          V(), pred, op,
-                                         std::integral_constant<bool, detail::scan_by_key_has_kernel<K, V, KIn, VIn, Out, Pred, Op>::value>());
+                                         std::integral_constant<bool, thrust::detail::scan_by_key_has_kernel<K, V, KIn, VIn, Out, Pred, Op>::value>());
   return result + n;
 }
 template <class D, class KIt, class VIt, class OutIt, class Pred>
@@ -209,14 +237,14 @@ OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt 
 template <class D, class KIt, class VIt, class OutIt, class T, class Pred, class Op>
 OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
                             OutIt result, T init, Pred pred, Op op) {
-  typedef typename detail::elem<KIt>::type K;
-  typedef typename detail::unwrap_iterator<KIt>::type KIn;
-  typedef typename detail::unwrap_iterator<VIt>::type VIn;
-  typedef typename detail::unwrap_iterator<OutIt>::type Out;
+  typedef typename thrust::detail::elem<KIt>::type K;
+  typedef typename thrust::detail::unwrap_iterator<KIt>::type KIn;
+  typedef typename thrust::detail::unwrap_iterator<VIt>::type VIn;
+  typedef typename thrust::detail::unwrap_iterator<OutIt>::type Out;
   const std::int64_t n = (std::int64_t)(klast - kfirst);
-  detail::scan_by_key_dispatch<true, K>(exec.derived(), detail::unwrap(kfirst), detail::unwrap(vfirst), detail::unwrap(result), n,
+  thrust::detail::scan_by_key_dispatch<true, K>(exec.derived(), thrust::detail::unwrap(kfirst), thrust::detail::unwrap(vfirst), thrust::detail::unwrap(result), n,
                                         init, pred, op,
-                                        std::integral_constant<bool, detail::scan_by_key_has_kernel<K, T, KIn, VIn, Out, Pred, Op>::value>());
+                                        std::integral_constant<bool, thrust::detail::scan_by_key_has_kernel<K, T, KIn, VIn, Out, Pred, Op>::value>());
   return result + n;
 }
 template <class D, class KIt, class VIt, class OutIt, class T, class Pred>
@@ -229,7 +257,39 @@ OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt 
 }
 template <class D, class KIt, class VIt, class OutIt>
 OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r) {
-  return exclusive_scan_by_key(exec, kf, kl, vf, r, typename detail::elem<VIt>::type());
+  return exclusive_scan_by_key(exec, kf, kl, vf, r, typename thrust::detail::elem<VIt>::type());
+}
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/scan.inl:35-48):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class KIt, class VIt, class OutIt, class Pred, class Op>
+OutIt inclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kfirst, KIt klast, VIt vfirst, OutIt result, Pred pred, Op op) {
+  return inclusive_scan_by_key(detail::derived_cast(detail::strip_const(exec)), kfirst, klast, vfirst, result, pred, op);
+}
+template <class D, class KIt, class VIt, class OutIt, class Pred>
+OutIt inclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, Pred p) {
+  return inclusive_scan_by_key(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, r, p);
+}
+template <class D, class KIt, class VIt, class OutIt>
+OutIt inclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r) {
+  return inclusive_scan_by_key(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, r);
+}
+template <class D, class KIt, class VIt, class OutIt, class T, class Pred, class Op>
+OutIt exclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kfirst, KIt klast, VIt vfirst, OutIt result, T init, Pred pred, Op op) {
+  return exclusive_scan_by_key(detail::derived_cast(detail::strip_const(exec)), kfirst, klast, vfirst, result, init, pred, op);
+}
+template <class D, class KIt, class VIt, class OutIt, class T, class Pred>
+OutIt exclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, T init, Pred p) {
+  return exclusive_scan_by_key(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, r, init, p);
+}
+template <class D, class KIt, class VIt, class OutIt, class T>
+OutIt exclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, T init) {
+  return exclusive_scan_by_key(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, r, init);
+}
+template <class D, class KIt, class VIt, class OutIt>
+OutIt exclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r) {
+  return exclusive_scan_by_key(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, r);
 }
 
 // ===================================================================== scan_by_key, host
@@ -299,9 +359,9 @@ OutIt exclusive_scan_by_key(const system::cpp::detail::par_t& e, KIt kf, KIt kl,
   template <class K, class V, class O, class A, COND<K> = 0> O NAME(K kf, K kl, V vf, O r, A a) { return NAME(SYS, kf, kl, vf, r, a); } \
   template <class K, class V, class O, class A, class B, COND<K> = 0> O NAME(K kf, K kl, V vf, O r, A a, B b) { return NAME(SYS, kf, kl, vf, r, a, b); } \
   template <class K, class V, class O, class A, class B, class C, COND<K> = 0> O NAME(K kf, K kl, V vf, O r, A a, B b, C c) { return NAME(SYS, kf, kl, vf, r, a, b, c); }
-THRUST_CDNA4_SBK(inclusive_scan_by_key, device, detail::enable_if_device)
+THRUST_CDNA4_SBK(inclusive_scan_by_key, typename detail::implicit_policy<K>::type(), detail::enable_if_device)
 THRUST_CDNA4_SBK(inclusive_scan_by_key, host, detail::enable_if_host)
-THRUST_CDNA4_SBK(exclusive_scan_by_key, device, detail::enable_if_device)
+THRUST_CDNA4_SBK(exclusive_scan_by_key, typename detail::implicit_policy<K>::type(), detail::enable_if_device)
 THRUST_CDNA4_SBK(exclusive_scan_by_key, host, detail::enable_if_host)
 #undef THRUST_CDNA4_SBK
 

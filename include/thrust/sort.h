@@ -74,36 +74,83 @@ void sort_pairs_range(const Policy& exec, KIt kfirst, KIt klast, VIt vfirst, Com
 }
 }  // namespace detail
 
+template <class D, class It, class Compare> void stable_sort(const detail::execution_policy_base<D>& exec, It first, It last, Compare comp);
+template <class D, class It> void stable_sort(const detail::execution_policy_base<D>& exec, It first, It last);
+template <class D, class KIt, class VIt, class Compare>
+void stable_sort_by_key(const detail::execution_policy_base<D>& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp);
+template <class D, class KIt, class VIt> void stable_sort_by_key(const detail::execution_policy_base<D>& exec, KIt kfirst, KIt klast, VIt vfirst);
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 template <class D, class It, class Compare>
 void stable_sort(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) {
-  detail::sort_range(exec.derived(), first, last, comp, typename detail::is_contiguous_device<It>::type());
+  thrust::detail::sort_range(exec.derived(), first, last, comp, typename thrust::detail::is_contiguous_device<It>::type());
 }
 template <class D, class It>
 void stable_sort(const system::cdna4::execution_policy<D>& exec, It first, It last) {
-  stable_sort(exec, first, last, less<typename detail::value_of<It>::type>());
+  stable_sort(exec, first, last, less<typename thrust::detail::value_of<It>::type>());
 }
 // sort forwards to stable_sort, as the generic layer does (thrust/system/detail/generic/sort.inl:56-62)
 template <class D, class It, class Compare>
-void sort(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) { stable_sort(exec, first, last, comp); }
+void sort(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) {
+  thrust::stable_sort(thrust::detail::derived_cast(thrust::detail::strip_const(exec)), first, last, comp);
+}
 template <class D, class It>
-void sort(const system::cdna4::execution_policy<D>& exec, It first, It last) { stable_sort(exec, first, last); }
+void sort(const system::cdna4::execution_policy<D>& exec, It first, It last) {
+  thrust::stable_sort(thrust::detail::derived_cast(thrust::detail::strip_const(exec)), first, last);
+}
 
 template <class D, class KIt, class VIt, class Compare>
 void stable_sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
-  detail::sort_pairs_range(exec.derived(), kfirst, klast, vfirst, comp,
-                           std::integral_constant<bool, detail::is_contiguous_device<KIt>::value && detail::is_contiguous_device<VIt>::value>());
+  thrust::detail::sort_pairs_range(exec.derived(), kfirst, klast, vfirst, comp,
+                           std::integral_constant<bool, thrust::detail::is_contiguous_device<KIt>::value && thrust::detail::is_contiguous_device<VIt>::value>());
 }
 template <class D, class KIt, class VIt>
 void stable_sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst) {
-  stable_sort_by_key(exec, kfirst, klast, vfirst, less<typename detail::value_of<KIt>::type>());
+  stable_sort_by_key(exec, kfirst, klast, vfirst, less<typename thrust::detail::value_of<KIt>::type>());
 }
 template <class D, class KIt, class VIt, class Compare>
 void sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
-  stable_sort_by_key(exec, kfirst, klast, vfirst, comp);
+  thrust::stable_sort_by_key(thrust::detail::derived_cast(thrust::detail::strip_const(exec)), kfirst, klast, vfirst, comp);
 }
 template <class D, class KIt, class VIt>
 void sort_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst) {
-  stable_sort_by_key(exec, kfirst, klast, vfirst);
+  thrust::stable_sort_by_key(thrust::detail::derived_cast(thrust::detail::strip_const(exec)), kfirst, klast, vfirst);
+}
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/sort.inl:32-44, :84-100):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class It, class Compare>
+void stable_sort(const detail::execution_policy_base<D>& exec, It first, It last, Compare comp) {
+  stable_sort(detail::derived_cast(detail::strip_const(exec)), first, last, comp);
+}
+template <class D, class It>
+void stable_sort(const detail::execution_policy_base<D>& exec, It first, It last) {
+  stable_sort(detail::derived_cast(detail::strip_const(exec)), first, last);
+}
+template <class D, class It, class Compare>
+void sort(const detail::execution_policy_base<D>& exec, It first, It last, Compare comp) {
+  sort(detail::derived_cast(detail::strip_const(exec)), first, last, comp);
+}
+template <class D, class It>
+void sort(const detail::execution_policy_base<D>& exec, It first, It last) {
+  sort(detail::derived_cast(detail::strip_const(exec)), first, last);
+}
+template <class D, class KIt, class VIt, class Compare>
+void stable_sort_by_key(const detail::execution_policy_base<D>& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
+  stable_sort_by_key(detail::derived_cast(detail::strip_const(exec)), kfirst, klast, vfirst, comp);
+}
+template <class D, class KIt, class VIt>
+void stable_sort_by_key(const detail::execution_policy_base<D>& exec, KIt kfirst, KIt klast, VIt vfirst) {
+  stable_sort_by_key(detail::derived_cast(detail::strip_const(exec)), kfirst, klast, vfirst);
+}
+template <class D, class KIt, class VIt, class Compare>
+void sort_by_key(const detail::execution_policy_base<D>& exec, KIt kfirst, KIt klast, VIt vfirst, Compare comp) {
+  sort_by_key(detail::derived_cast(detail::strip_const(exec)), kfirst, klast, vfirst, comp);
+}
+template <class D, class KIt, class VIt>
+void sort_by_key(const detail::execution_policy_base<D>& exec, KIt kfirst, KIt klast, VIt vfirst) {
+  sort_by_key(detail::derived_cast(detail::strip_const(exec)), kfirst, klast, vfirst);
 }
 
 // ---- host, explicit policy -----------------------------------------------------------
@@ -171,16 +218,16 @@ void sort_by_key(const system::cpp::detail::par_t& e, KIt kfirst, KIt klast, VIt
 
 // ---- no policy: the iterator's system decides (thrust/detail/sort.inl:202-339) --------
 #define THRUST_CDNA4_SORT_DISPATCH(NAME)                                                                         \
-  template <class It, detail::enable_if_device<It> = 0> void NAME(It f, It l) { NAME(device, f, l); }              \
-  template <class It, class C, detail::enable_if_device<It> = 0> void NAME(It f, It l, C c) { NAME(device, f, l, c); } \
+  template <class It, detail::enable_if_device<It> = 0> void NAME(It f, It l) { NAME(typename detail::implicit_policy<It>::type(), f, l); }              \
+  template <class It, class C, detail::enable_if_device<It> = 0> void NAME(It f, It l, C c) { NAME(typename detail::implicit_policy<It>::type(), f, l, c); } \
   template <class It, detail::enable_if_host<It> = 0> void NAME(It f, It l) { NAME(host, f, l); }                  \
   template <class It, class C, detail::enable_if_host<It> = 0> void NAME(It f, It l, C c) { NAME(host, f, l, c); }
 THRUST_CDNA4_SORT_DISPATCH(sort)
 THRUST_CDNA4_SORT_DISPATCH(stable_sort)
 #undef THRUST_CDNA4_SORT_DISPATCH
 #define THRUST_CDNA4_SORT_BY_KEY_DISPATCH(NAME)                                                                  \
-  template <class K, class V, detail::enable_if_device<K> = 0> void NAME(K f, K l, V v) { NAME(device, f, l, v); }  \
-  template <class K, class V, class C, detail::enable_if_device<K> = 0> void NAME(K f, K l, V v, C c) { NAME(device, f, l, v, c); } \
+  template <class K, class V, detail::enable_if_device<K> = 0> void NAME(K f, K l, V v) { NAME(typename detail::implicit_policy<K>::type(), f, l, v); }  \
+  template <class K, class V, class C, detail::enable_if_device<K> = 0> void NAME(K f, K l, V v, C c) { NAME(typename detail::implicit_policy<K>::type(), f, l, v, c); } \
   template <class K, class V, detail::enable_if_host<K> = 0> void NAME(K f, K l, V v) { NAME(host, f, l, v); }      \
   template <class K, class V, class C, detail::enable_if_host<K> = 0> void NAME(K f, K l, V v, C c) { NAME(host, f, l, v, c); }
 THRUST_CDNA4_SORT_BY_KEY_DISPATCH(sort_by_key)

@@ -95,6 +95,13 @@ namespace detail {
 // that dispatch to a system's implementation take it, so that an overload for a nearer base — the
 // system's own, or a user's for a policy type of their own — is the better match.
 template <class Derived> struct execution_policy_base {};
+// the policy as its own type, and without const: user overloads take their policy by reference
+// (thrust/detail/execution_policy.h:50-75)
+template <class Derived> inline execution_policy_base<Derived>& strip_const(const execution_policy_base<Derived>& x) {
+  return const_cast<execution_policy_base<Derived>&>(x);
+}
+template <class Derived> inline Derived& derived_cast(execution_policy_base<Derived>& x) { return static_cast<Derived&>(x); }
+template <class Derived> inline const Derived& derived_cast(const execution_policy_base<Derived>& x) { return static_cast<const Derived&>(x); }
 }  // namespace detail
 
 namespace system {
