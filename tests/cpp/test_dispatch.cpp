@@ -5,11 +5,15 @@
 // testing/stable_sort.cu, sort_by_key.cu, stable_sort_by_key.cu, scan.cu:19-90, scan_by_key.inclusive.cu,
 // scan_by_key.exclusive.cu, reduce_by_key.cu and reduce.cu, with my_system / my_tag of
 // testing/unittest/special_types.h:135-170.  Compiled by hipcc (retagged iterators are fancy iterators: kernel templates).
+#include <thrust/copy.h>
 #include <thrust/execution_policy.h>
+#include <thrust/fill.h>
 #include <thrust/iterator/retag.h>
 #include <thrust/reduce.h>
 #include <thrust/scan.h>
 #include <thrust/sort.h>
+#include <thrust/transform.h>
+#include <thrust/transform_reduce.h>
 
 #include "testing.h"
 
@@ -51,6 +55,15 @@ thrust::pair<KO, VO> reduce_by_key(my_tag, K, K, V, KO ko, VO vo) { *ko = 13; re
 template <class It> int reduce(my_system& s, It, It) { s.validate_dispatch(); return 13; }
 template <class It> int reduce(my_tag, It, It) { return 13; }
 
+template <class In, class Out> Out copy(my_system& s, In, In, Out r) { s.validate_dispatch(); return r; }
+template <class In, class Out> Out copy(my_tag, In, In, Out r) { *r = 13; return r; }
+template <class In, class Out, class P> Out copy_if(my_system& s, In, In, Out r, P) { s.validate_dispatch(); return r; }
+template <class In, class Out, class P> Out copy_if(my_system& s, In, In, In, Out r, P) { s.validate_dispatch(); return r; }
+template <class It, class T> void fill(my_system& s, It, It, const T&) { s.validate_dispatch(); }
+template <class In, class Out, class F> Out transform(my_system& s, In, In, Out r, F) { s.validate_dispatch(); return r; }
+template <class In, class Out, class F> Out transform(my_system& s, In, In, In, Out r, F) { s.validate_dispatch(); return r; }
+template <class In, class F, class T, class Op> T transform_reduce(my_system& s, In, In, F, T init, Op) { s.validate_dispatch(); return init; }
+
 #define EXPLICIT(NAME, ...)                    \
   void Test_##NAME##_DispatchExplicit() {      \
     thrust::device_vector<int> vec(1);         \
@@ -88,6 +101,27 @@ IMPLICIT(exclusive_scan_by_key, T, T, T, T);
 EXPLICIT(reduce_by_key, B, B, B, B, B);
 IMPLICIT(reduce_by_key, T, T, T, T, T);
 EXPLICIT(reduce, B, B);
+
+EXPLICIT(copy, B, B, B);
+IMPLICIT(copy, T, T, T);
+EXPLICIT(copy_if, B, B, B, thrust::identity<int>());
+void TestCopyIfStencilDispatchExplicit() {
+  thrust::device_vector<int> vec(1);
+  my_system sys(0);
+  thrust::copy_if(sys, B, B, B, B, thrust::identity<int>());
+  ASSERT_EQUAL(true, sys.is_valid());
+}
+DECLARE_UNITTEST(TestCopyIfStencilDispatchExplicit);
+EXPLICIT(fill, B, B, 0);
+EXPLICIT(transform, B, B, B, thrust::negate<int>());
+void TestBinaryTransformDispatchExplicit() {
+  thrust::device_vector<int> vec(1);
+  my_system sys(0);
+  thrust::transform(sys, B, B, B, B, thrust::plus<int>());
+  ASSERT_EQUAL(true, sys.is_valid());
+}
+DECLARE_UNITTEST(TestBinaryTransformDispatchExplicit);
+EXPLICIT(transform_reduce, B, B, thrust::negate<int>(), 0, thrust::plus<int>());
 
 void TestReduceDispatchImplicit() {
   thrust::device_vector<int> vec(1);
