@@ -28,10 +28,24 @@ template <class Pred> struct negated {
   template <class T> THRUST_CDNA4_HD bool operator()(const T& x) const { return !pred(x); }
 };
 }  // namespace detail
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 template <class D, class It, class Pred>
-It find_if(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) { return detail::find_first<false>(exec.derived(), first, last, pred); }
+It find_if(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) { return thrust::detail::find_first<false>(exec.derived(), first, last, pred); }
 template <class D, class It, class Pred>
-It find_if_not(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) { return detail::find_first<true>(exec.derived(), first, last, pred); }
+It find_if_not(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) { return thrust::detail::find_first<true>(exec.derived(), first, last, pred); }
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/find.inl):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class It, class Pred>
+It find_if(const detail::execution_policy_base<D>& exec, It first, It last, Pred pred) {
+  return find_if(detail::derived_cast(detail::strip_const(exec)), first, last, pred);
+}
+template <class D, class It, class Pred>
+It find_if_not(const detail::execution_policy_base<D>& exec, It first, It last, Pred pred) {
+  return find_if_not(detail::derived_cast(detail::strip_const(exec)), first, last, pred);
+}
 template <class It, class Pred> It find_if(const system::cpp::detail::par_t&, It first, It last, Pred pred) { return std::find_if(first, last, pred); }
 template <class It, class Pred> It find_if_not(const system::cpp::detail::par_t&, It first, It last, Pred pred) { return std::find_if_not(first, last, pred); }
 template <class Policy, class It, class T, detail::enable_if_policy<Policy> = 0>

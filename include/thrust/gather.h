@@ -21,31 +21,51 @@ struct truthy {
   template <class T> THRUST_CDNA4_HD bool operator()(const T& x) const { return x ? true : false; }
 };
 }  // namespace detail
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 template <class D, class Map, class In, class Out>
 Out gather(const system::cdna4::execution_policy<D>& exec, Map map_first, Map map_last, In input, Out result) {
   const std::int64_t n = (std::int64_t)(map_last - map_first);
   system::cdna4::detail::for_each_index(
       exec.derived(), n,
-      detail::gather_body<typename detail::unwrap_iterator<Map>::type, typename detail::unwrap_iterator<In>::type,
-                          typename detail::unwrap_iterator<Out>::type>{detail::unwrap(map_first), detail::unwrap(input), detail::unwrap(result)},
+      thrust::detail::gather_body<typename thrust::detail::unwrap_iterator<Map>::type, typename thrust::detail::unwrap_iterator<In>::type,
+                          typename thrust::detail::unwrap_iterator<Out>::type>{thrust::detail::unwrap(map_first), thrust::detail::unwrap(input), thrust::detail::unwrap(result)},
       "gather: failed to synchronize");
   return result + n;
+}
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/gather.inl):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class Map, class In, class Out>
+Out gather(const detail::execution_policy_base<D>& exec, Map map_first, Map map_last, In input, Out result) {
+  return gather(detail::derived_cast(detail::strip_const(exec)), map_first, map_last, input, result);
 }
 template <class Map, class In, class Out>
 Out gather(const system::cpp::detail::par_t&, Map map_first, Map map_last, In input, Out result) {
   for (; map_first != map_last; ++map_first, ++result) *result = input[*map_first];
   return result;
 }
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 template <class D, class Map, class S, class In, class Out, class Pred>
 Out gather_if(const system::cdna4::execution_policy<D>& exec, Map map_first, Map map_last, S stencil, In input, Out result, Pred pred) {
   const std::int64_t n = (std::int64_t)(map_last - map_first);
   system::cdna4::detail::for_each_index(
       exec.derived(), n,
-      detail::gather_if_body<typename detail::unwrap_iterator<Map>::type, typename detail::unwrap_iterator<S>::type,
-                             typename detail::unwrap_iterator<In>::type, typename detail::unwrap_iterator<Out>::type, Pred>{
-          detail::unwrap(map_first), detail::unwrap(stencil), detail::unwrap(input), detail::unwrap(result), pred},
+      thrust::detail::gather_if_body<typename thrust::detail::unwrap_iterator<Map>::type, typename thrust::detail::unwrap_iterator<S>::type,
+                             typename thrust::detail::unwrap_iterator<In>::type, typename thrust::detail::unwrap_iterator<Out>::type, Pred>{
+          thrust::detail::unwrap(map_first), thrust::detail::unwrap(stencil), thrust::detail::unwrap(input), thrust::detail::unwrap(result), pred},
       "gather_if: failed to synchronize");
   return result + n;
+}
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/gather.inl):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class Map, class S, class In, class Out, class Pred>
+Out gather_if(const detail::execution_policy_base<D>& exec, Map map_first, Map map_last, S stencil, In input, Out result, Pred pred) {
+  return gather_if(detail::derived_cast(detail::strip_const(exec)), map_first, map_last, stencil, input, result, pred);
 }
 template <class Map, class S, class In, class Out, class Pred>
 Out gather_if(const system::cpp::detail::par_t&, Map map_first, Map map_last, S stencil, In input, Out result, Pred pred) {

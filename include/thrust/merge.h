@@ -14,6 +14,8 @@
 #endif
 
 namespace thrust {
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 // ---- device
 template <class D, class In1, class In2, class Out, class Comp>
 Out merge(const system::cdna4::execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
@@ -21,8 +23,8 @@ Out merge(const system::cdna4::execution_policy<D>& exec, In1 first1, In1 last1,
   const std::int64_t na = (std::int64_t)(last1 - first1), nb = (std::int64_t)(last2 - first2);
 #if defined(__HIPCC__)
   namespace m = system::cdna4::detail::merge2;
-  m::merge<false>(system::cdna4::detail::stream_of(exec.derived()), detail::unwrap(first1), na, detail::unwrap(first2), nb, system::cdna4::detail::no_values(),
-                  system::cdna4::detail::no_values(), detail::unwrap(result), system::cdna4::detail::no_values(), comp);
+  m::merge<false>(system::cdna4::detail::stream_of(exec.derived()), thrust::detail::unwrap(first1), na, thrust::detail::unwrap(first2), nb, system::cdna4::detail::no_values(),
+                  system::cdna4::detail::no_values(), thrust::detail::unwrap(result), system::cdna4::detail::no_values(), comp);
   system::cdna4::detail::synchronize_optional(exec.derived(), "merge: failed to synchronize");
 #endif
   return result + (na + nb);
@@ -34,13 +36,25 @@ pair<KOut, VOut> merge_by_key(const system::cdna4::execution_policy<D>& exec, K1
   const std::int64_t na = (std::int64_t)(klast1 - kfirst1), nb = (std::int64_t)(klast2 - kfirst2);
 #if defined(__HIPCC__)
   namespace m = system::cdna4::detail::merge2;
-  m::merge<true>(system::cdna4::detail::stream_of(exec.derived()), detail::unwrap(kfirst1), na, detail::unwrap(kfirst2), nb,
-                 detail::unwrap(vfirst1), detail::unwrap(vfirst2), detail::unwrap(kresult), detail::unwrap(vresult), comp);
+  m::merge<true>(system::cdna4::detail::stream_of(exec.derived()), thrust::detail::unwrap(kfirst1), na, thrust::detail::unwrap(kfirst2), nb,
+                 thrust::detail::unwrap(vfirst1), thrust::detail::unwrap(vfirst2), thrust::detail::unwrap(kresult), thrust::detail::unwrap(vresult), comp);
   system::cdna4::detail::synchronize_optional(exec.derived(), "merge_by_key: failed to synchronize");
 #else
   (void)vfirst1; (void)vfirst2;
 #endif
   return pair<KOut, VOut>(kresult + (na + nb), vresult + (na + nb));
+}
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/merge.inl):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class In1, class In2, class Out, class Comp>
+Out merge(const detail::execution_policy_base<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  return merge(detail::derived_cast(detail::strip_const(exec)), first1, last1, first2, last2, result, comp);
+}
+template <class D, class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp>
+pair<KOut, VOut> merge_by_key(const detail::execution_policy_base<D>& exec, K1 kfirst1, K1 klast1, K2 kfirst2, K2 klast2, V1 vfirst1, V2 vfirst2, KOut kresult, VOut vresult, Comp comp) {
+  return merge_by_key(detail::derived_cast(detail::strip_const(exec)), kfirst1, klast1, kfirst2, klast2, vfirst1, vfirst2, kresult, vresult, comp);
 }
 // ---- host
 template <class In1, class In2, class Out, class Comp>

@@ -20,21 +20,41 @@ template <class In, class Out> struct reverse_copy_body {
   THRUST_CDNA4_HD void operator()(std::int64_t i) { out[i] = in[n - 1 - i]; }
 };
 }  // namespace detail
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 template <class D, class It>
 void reverse(const system::cdna4::execution_policy<D>& exec, It first, It last) {
   const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::for_each_index(exec.derived(), n / 2, detail::reverse_body<typename detail::unwrap_iterator<It>::type>{detail::unwrap(first), n},
+  system::cdna4::detail::for_each_index(exec.derived(), n / 2, thrust::detail::reverse_body<typename thrust::detail::unwrap_iterator<It>::type>{thrust::detail::unwrap(first), n},
                                         "reverse: failed to synchronize");
 }
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/reverse.inl):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class It>
+void reverse(const detail::execution_policy_base<D>& exec, It first, It last) {
+  reverse(detail::derived_cast(detail::strip_const(exec)), first, last);
+}
 template <class It> void reverse(const system::cpp::detail::par_t&, It first, It last) { std::reverse(first, last); }
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 template <class D, class In, class Out>
 Out reverse_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out result) {
   const std::int64_t n = (std::int64_t)(last - first);
   system::cdna4::detail::for_each_index(
       exec.derived(), n,
-      detail::reverse_copy_body<typename detail::unwrap_iterator<In>::type, typename detail::unwrap_iterator<Out>::type>{detail::unwrap(first), detail::unwrap(result), n},
+      thrust::detail::reverse_copy_body<typename thrust::detail::unwrap_iterator<In>::type, typename thrust::detail::unwrap_iterator<Out>::type>{thrust::detail::unwrap(first), thrust::detail::unwrap(result), n},
       "reverse_copy: failed to synchronize");
   return result + n;
+}
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/reverse.inl):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class In, class Out>
+Out reverse_copy(const detail::execution_policy_base<D>& exec, In first, In last, Out result) {
+  return reverse_copy(detail::derived_cast(detail::strip_const(exec)), first, last, result);
 }
 template <class In, class Out> Out reverse_copy(const system::cpp::detail::par_t&, In first, In last, Out result) { return std::reverse_copy(first, last, result); }
 template <class It, detail::enable_if_device<It> = 0> void reverse(It f, It l) { reverse(device, f, l); }

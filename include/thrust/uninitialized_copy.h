@@ -4,8 +4,18 @@
 #include <memory>
 #include <thrust/copy.h>
 namespace thrust {
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
 template <class D, class In, class Out>
 Out uninitialized_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out result) { return copy(exec, first, last, result); }
+}}  // namespace system::cdna4
+// The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/uninitialized_copy.inl):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
+template <class D, class In, class Out>
+Out uninitialized_copy(const detail::execution_policy_base<D>& exec, In first, In last, Out result) {
+  return uninitialized_copy(detail::derived_cast(detail::strip_const(exec)), first, last, result);
+}
 template <class In, class Out>
 Out uninitialized_copy(const system::cpp::detail::par_t&, In first, In last, Out result) { return std::uninitialized_copy(first, last, result); }
 template <class Policy, class In, class Size, class Out, detail::enable_if_policy<Policy> = 0>

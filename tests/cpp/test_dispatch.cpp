@@ -5,6 +5,27 @@
 // testing/stable_sort.cu, sort_by_key.cu, stable_sort_by_key.cu, scan.cu:19-90, scan_by_key.inclusive.cu,
 // scan_by_key.exclusive.cu, reduce_by_key.cu and reduce.cu, with my_system / my_tag of
 // testing/unittest/special_types.h:135-170.  Compiled by hipcc (retagged iterators are fancy iterators: kernel templates).
+#include <thrust/adjacent_difference.h>
+#include <thrust/extrema.h>
+#include <thrust/find.h>
+#include <thrust/gather.h>
+#include <thrust/generate.h>
+#include <thrust/inner_product.h>
+#include <thrust/merge.h>
+#include <thrust/mismatch.h>
+#include <thrust/partition.h>
+#include <thrust/random.h>
+#include <thrust/remove.h>
+#include <thrust/replace.h>
+#include <thrust/reverse.h>
+#include <thrust/scatter.h>
+#include <thrust/sequence.h>
+#include <thrust/shuffle.h>
+#include <thrust/swap.h>
+#include <thrust/tabulate.h>
+#include <thrust/uninitialized_copy.h>
+#include <thrust/uninitialized_fill.h>
+#include <thrust/unique.h>
 #include <thrust/copy.h>
 #include <thrust/execution_policy.h>
 #include <thrust/fill.h>
@@ -79,49 +100,127 @@ template <class In, class F, class T, class Op> T transform_reduce(my_system& s,
     ASSERT_EQUAL(13, (int)vec.front());        \
   }                                            \
   DECLARE_UNITTEST(Test_##NAME##_DispatchImplicit)
-#define B vec.begin()
-#define T thrust::retag<my_tag>(vec.begin())
+#define BEGIN_ vec.begin()
+#define TAGGED_ thrust::retag<my_tag>(vec.begin())
 
-EXPLICIT(sort, B, B);
-IMPLICIT(sort, T, T);
-EXPLICIT(stable_sort, B, B);
-IMPLICIT(stable_sort, T, T);
-EXPLICIT(sort_by_key, B, B, B);
-IMPLICIT(sort_by_key, T, T, T);
-EXPLICIT(stable_sort_by_key, B, B, B);
-IMPLICIT(stable_sort_by_key, T, T, T);
-EXPLICIT(inclusive_scan, B, B, B);
-IMPLICIT(inclusive_scan, T, T, T);
-EXPLICIT(exclusive_scan, B, B, B);
-IMPLICIT(exclusive_scan, T, T, T);
-EXPLICIT(inclusive_scan_by_key, B, B, B, B);
-IMPLICIT(inclusive_scan_by_key, T, T, T, T);
-EXPLICIT(exclusive_scan_by_key, B, B, B, B);
-IMPLICIT(exclusive_scan_by_key, T, T, T, T);
-EXPLICIT(reduce_by_key, B, B, B, B, B);
-IMPLICIT(reduce_by_key, T, T, T, T, T);
-EXPLICIT(reduce, B, B);
+EXPLICIT(sort, BEGIN_, BEGIN_);
+IMPLICIT(sort, TAGGED_, TAGGED_);
+EXPLICIT(stable_sort, BEGIN_, BEGIN_);
+IMPLICIT(stable_sort, TAGGED_, TAGGED_);
+EXPLICIT(sort_by_key, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(sort_by_key, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(stable_sort_by_key, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(stable_sort_by_key, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(inclusive_scan, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(inclusive_scan, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(exclusive_scan, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(exclusive_scan, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(inclusive_scan_by_key, BEGIN_, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(inclusive_scan_by_key, TAGGED_, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(exclusive_scan_by_key, BEGIN_, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(exclusive_scan_by_key, TAGGED_, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(reduce_by_key, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(reduce_by_key, TAGGED_, TAGGED_, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(reduce, BEGIN_, BEGIN_);
 
-EXPLICIT(copy, B, B, B);
-IMPLICIT(copy, T, T, T);
-EXPLICIT(copy_if, B, B, B, thrust::identity<int>());
+EXPLICIT(copy, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(copy, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(copy_if, BEGIN_, BEGIN_, BEGIN_, thrust::identity<int>());
 void TestCopyIfStencilDispatchExplicit() {
   thrust::device_vector<int> vec(1);
   my_system sys(0);
-  thrust::copy_if(sys, B, B, B, B, thrust::identity<int>());
+  thrust::copy_if(sys, BEGIN_, BEGIN_, BEGIN_, BEGIN_, thrust::identity<int>());
   ASSERT_EQUAL(true, sys.is_valid());
 }
 DECLARE_UNITTEST(TestCopyIfStencilDispatchExplicit);
-EXPLICIT(fill, B, B, 0);
-EXPLICIT(transform, B, B, B, thrust::negate<int>());
+EXPLICIT(fill, BEGIN_, BEGIN_, 0);
+EXPLICIT(transform, BEGIN_, BEGIN_, BEGIN_, thrust::negate<int>());
 void TestBinaryTransformDispatchExplicit() {
   thrust::device_vector<int> vec(1);
   my_system sys(0);
-  thrust::transform(sys, B, B, B, B, thrust::plus<int>());
+  thrust::transform(sys, BEGIN_, BEGIN_, BEGIN_, BEGIN_, thrust::plus<int>());
   ASSERT_EQUAL(true, sys.is_valid());
 }
 DECLARE_UNITTEST(TestBinaryTransformDispatchExplicit);
-EXPLICIT(transform_reduce, B, B, thrust::negate<int>(), 0, thrust::plus<int>());
+EXPLICIT(transform_reduce, BEGIN_, BEGIN_, thrust::negate<int>(), 0, thrust::plus<int>());
+
+
+// ---- the other algorithms: the form that names every operator dispatches on the policy type (the
+//      shorter forms supply the default operator and call it) --------------------------------
+#define V(x) s.validate_dispatch(); return x
+template <class In, class Out, class Op> Out adjacent_difference(my_system& s, In, In, Out r, Op) { V(r); }
+template <class It, class C> It min_element(my_system& s, It f, It, C) { V(f); }
+template <class It, class C> It max_element(my_system& s, It f, It, C) { V(f); }
+template <class It, class C> thrust::pair<It, It> minmax_element(my_system& s, It f, It, C) { V(thrust::make_pair(f, f)); }
+template <class It, class P> It find_if(my_system& s, It f, It, P) { V(f); }
+template <class It, class P> It find_if_not(my_system& s, It f, It, P) { V(f); }
+template <class M, class In, class Out> Out gather(my_system& s, M, M, In, Out r) { V(r); }
+template <class M, class S, class In, class Out, class P> Out gather_if(my_system& s, M, M, S, In, Out r, P) { V(r); }
+template <class It, class G> void generate(my_system& s, It, It, G) { s.validate_dispatch(); }
+template <class A, class Bi, class T, class O1, class O2> T inner_product(my_system& s, A, A, Bi, T init, O1, O2) { V(init); }
+template <class A, class Bi, class Out, class C> Out merge(my_system& s, A, A, Bi, Bi, Out r, C) { V(r); }
+template <class A, class Bi, class VA, class VBB, class KO, class VO, class C>
+thrust::pair<KO, VO> merge_by_key(my_system& s, A, A, Bi, Bi, VA, VBB, KO ko, VO vo, C) { V(thrust::make_pair(ko, vo)); }
+template <class A, class Bi, class P> thrust::pair<A, Bi> mismatch(my_system& s, A a, A, Bi b, P) { V(thrust::make_pair(a, b)); }
+template <class It, class P> It stable_partition(my_system& s, It f, It, P) { V(f); }
+template <class In, class O1, class O2, class P> thrust::pair<O1, O2> stable_partition_copy(my_system& s, In, In, O1 a, O2 b, P) { V(thrust::make_pair(a, b)); }
+template <class In, class Out, class P> Out remove_copy_if(my_system& s, In, In, Out r, P) { V(r); }
+template <class It, class P> It remove_if(my_system& s, It f, It, P) { V(f); }
+template <class In, class S, class Out, class P, class T> Out replace_copy_if(my_system& s, In, In, S, Out r, P, const T&) { V(r); }
+template <class It> void reverse(my_system& s, It, It) { s.validate_dispatch(); }
+template <class In, class Out> Out reverse_copy(my_system& s, In, In, Out r) { V(r); }
+template <class In, class M, class Out> void scatter(my_system& s, In, In, M, Out) { s.validate_dispatch(); }
+template <class In, class M, class S, class Out, class P> void scatter_if(my_system& s, In, In, M, S, Out, P) { s.validate_dispatch(); }
+template <class It, class T> void sequence(my_system& s, It, It, T, T) { s.validate_dispatch(); }
+template <class It, class G> void shuffle(my_system& s, It, It, G&&) { s.validate_dispatch(); }
+template <class In, class Out, class G> void shuffle_copy(my_system& s, In, In, Out, G&&) { s.validate_dispatch(); }
+template <class A, class Bi> Bi swap_ranges(my_system& s, A, A, Bi b) { V(b); }
+template <class It, class F> void tabulate(my_system& s, It, It, F) { s.validate_dispatch(); }
+template <class In, class Out> Out uninitialized_copy(my_system& s, In, In, Out r) { V(r); }
+template <class It, class T> void uninitialized_fill(my_system& s, It, It, const T&) { s.validate_dispatch(); }
+template <class It, class E> It unique(my_system& s, It f, It, E) { V(f); }
+template <class In, class Out, class E> Out unique_copy(my_system& s, In, In, Out r, E) { V(r); }
+template <class K, class Vi, class E> thrust::pair<K, Vi> unique_by_key(my_system& s, K k, K, Vi v, E) { V(thrust::make_pair(k, v)); }
+template <class K, class Vi, class KO, class VO, class E>
+thrust::pair<KO, VO> unique_by_key_copy(my_system& s, K, K, Vi, KO ko, VO vo, E) { V(thrust::make_pair(ko, vo)); }
+#undef V
+
+typedef thrust::less<int> L;
+typedef thrust::equal_to<int> E;
+typedef thrust::identity<int> I;
+EXPLICIT(adjacent_difference, BEGIN_, BEGIN_, BEGIN_, thrust::minus<int>());
+EXPLICIT(min_element, BEGIN_, BEGIN_, L());
+EXPLICIT(max_element, BEGIN_, BEGIN_, L());
+EXPLICIT(minmax_element, BEGIN_, BEGIN_, L());
+EXPLICIT(find_if, BEGIN_, BEGIN_, I());
+EXPLICIT(find_if_not, BEGIN_, BEGIN_, I());
+EXPLICIT(gather, BEGIN_, BEGIN_, BEGIN_, BEGIN_);
+EXPLICIT(gather_if, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, I());
+EXPLICIT(generate, BEGIN_, BEGIN_, thrust::default_random_engine());
+EXPLICIT(inner_product, BEGIN_, BEGIN_, BEGIN_, 0, thrust::plus<int>(), thrust::multiplies<int>());
+EXPLICIT(merge, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, L());
+EXPLICIT(merge_by_key, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, L());
+EXPLICIT(mismatch, BEGIN_, BEGIN_, BEGIN_, E());
+EXPLICIT(stable_partition, BEGIN_, BEGIN_, I());
+EXPLICIT(stable_partition_copy, BEGIN_, BEGIN_, BEGIN_, BEGIN_, I());
+EXPLICIT(remove_copy_if, BEGIN_, BEGIN_, BEGIN_, I());
+EXPLICIT(remove_if, BEGIN_, BEGIN_, I());
+EXPLICIT(replace_copy_if, BEGIN_, BEGIN_, BEGIN_, BEGIN_, I(), 0);
+EXPLICIT(reverse, BEGIN_, BEGIN_);
+EXPLICIT(reverse_copy, BEGIN_, BEGIN_, BEGIN_);
+EXPLICIT(scatter, BEGIN_, BEGIN_, BEGIN_, BEGIN_);
+EXPLICIT(scatter_if, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, I());
+EXPLICIT(sequence, BEGIN_, BEGIN_, 0, 1);
+EXPLICIT(shuffle, BEGIN_, BEGIN_, thrust::default_random_engine());
+EXPLICIT(shuffle_copy, BEGIN_, BEGIN_, BEGIN_, thrust::default_random_engine());
+EXPLICIT(swap_ranges, BEGIN_, BEGIN_, BEGIN_);
+EXPLICIT(tabulate, BEGIN_, BEGIN_, I());
+EXPLICIT(uninitialized_copy, BEGIN_, BEGIN_, BEGIN_);
+EXPLICIT(uninitialized_fill, BEGIN_, BEGIN_, 0);
+EXPLICIT(unique, BEGIN_, BEGIN_, E());
+EXPLICIT(unique_copy, BEGIN_, BEGIN_, BEGIN_, E());
+EXPLICIT(unique_by_key, BEGIN_, BEGIN_, BEGIN_, E());
+EXPLICIT(unique_by_key_copy, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, E());
 
 void TestReduceDispatchImplicit() {
   thrust::device_vector<int> vec(1);
