@@ -22,7 +22,7 @@
 // | word), written and read with relaxed agent-scope atomics: a reader that finds the same status
 // in all NW atoms has a consistent value, so no fence is needed (each atom is written once per
 // status).  One wavefront looks back 64 tiles at a time; because combine need not commute, the
-// window is folded in tile order by one lane.
+// window is folded in tile order (a suffix reduction over the lanes).
 #pragma once
 #if !defined(__HIPCC__)
 #error "thrust/system/cdna4/detail/scan_engine.h holds device kernel templates: compile with hipcc"
@@ -79,6 +79,19 @@ __device__ inline Acc shfl_up_acc(const Acc& a, int d) {
   return r;
 }
 
+// An accumulator from `d` lanes above (undefined in lanes >= 64 - d), word by word.
+template <class Acc>
+__device__ inline Acc shfl_down_acc(const Acc& a, int d) {
+  constexpr int NW = (int)((sizeof(Acc) + 3) / 4);
+  unsigned w[NW] = {};
+  __builtin_memcpy(w, &a, sizeof(Acc));
+#pragma unroll
+  for (int k = 0; k < NW; k++) w[k] = __shfl_down(w[k], (unsigned)d, 64);
+  Acc r;
+  __builtin_memcpy(&r, w, sizeof(Acc));
+  return r;
+}
+
 // Slot of element e of a tile in the staging buffer: one slot of padding after every ITEMS, so
 // that both the striped order (consecutive lanes, consecutive elements) and the blocked order
 // (consecutive lanes, ITEMS elements apart) spread over the LDS banks.
@@ -115,11 +128,10 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
   // Accumulators too large for that buffer are loaded and stored in the threads' own order.
   constexpr bool kStaged = sizeof(Acc) * (PART + PART / ITEMS) <= 40 * 1024;
   typedef typename std::aligned_storage<sizeof(Acc), alignof(Acc)>::type Raw;
-  __shared__ Raw raw_stage[kStaged ? PART + PART / ITEMS : 1], raw_wave[SUB][NWAVES], raw_part[SUB], raw_look[64], raw_prefix;
+  __shared__ Raw raw_stage[kStaged ? PART + PART / ITEMS : 1], raw_wave[SUB][NWAVES], raw_part[SUB], raw_prefix;
   __shared__ unsigned long long s_tile;
   __shared__ int s_has_prefix;
   Acc* s_stage = reinterpret_cast<Acc*>(raw_stage);
-  Acc* s_look = reinterpret_cast<Acc*>(raw_look);  // one look-back window
   Acc* s_prefix = reinterpret_cast<Acc*>(&raw_prefix);
   const auto s_wave = [&](int part, int w) -> Acc& { return *reinterpret_cast<Acc*>(&raw_wave[part][w]); };  // inclusive aggregate of a wavefront's threads
   const auto s_part = [&](int part) -> Acc& { return *reinterpret_cast<Acc*>(&raw_part[part]); };           // aggregate of a part
@@ -221,25 +233,21 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
           __builtin_amdgcn_s_sleep(1);
           continue;
         }
-        s_look[lane] = val;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        if (lane == 0) {
-          const int last = full ? __builtin_ctzll(full) : 63;  // the farthest lane that counts
-          bool has = false;
-          Acc a = tile_agg;
-          for (int l = last; l >= 0; l--) {  // in tile order: far to near
-            if (nearest - l < 0) continue;   // the virtual tile before tile 0
-            a = has ? op.combine(a, s_look[l]) : s_look[l];
-            has = true;
-          }
-          if (has) {
-            prefix = has_prefix ? op.combine(a, prefix) : a;
-            has_prefix = true;
-          }
+        // The window is folded in tile order — far to near, combine need not commute — by a
+        // suffix reduction over the lanes: after step d lane l holds lanes l + 2d - 1 ... l.
+        // Lanes beyond the nearest complete descriptor, and the virtual tiles before tile 0, stay out.
+        int last = full ? __builtin_ctzll(full) : 63;  // the farthest lane that counts
+        if ((std::int64_t)last > nearest) last = (int)nearest;
+        Acc a = val;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const Acc farther = shfl_down_acc(a, d);
+          if (lane + d <= last) a = op.combine(farther, a);
         }
-        __builtin_amdgcn_wave_barrier();
+        if (lane == 0 && last >= 0) {
+          prefix = has_prefix ? op.combine(a, prefix) : a;
+          has_prefix = true;
+        }
         if (full) break;
         nearest -= 64;
       }
