@@ -55,18 +55,9 @@ OutIt copy(InIt first, InIt last, OutIt out) {
 #include <thrust/detail/iterator_util.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Out, class Pred>
-Out copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Pred pred) {
-  return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), thrust::detail::unwrap(first), thrust::detail::unwrap(out), (std::int64_t)(last - first), pred);
-}
-template <class D, class In, class St, class Out, class Pred>
-Out copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, St stencil, Out out, Pred pred) {
-  return out + system::cdna4::detail::copy_flagged_n<false>(exec.derived(), thrust::detail::unwrap(first), thrust::detail::unwrap(stencil),
-                                                            thrust::detail::unwrap(out), (std::int64_t)(last - first), pred);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/copy_if.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/copy.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.
@@ -100,25 +91,9 @@ namespace detail {
 template <class It> struct is_fancy_device_iterator { static constexpr bool value = system::cdna4::detail::is_device_iterator<It>::value; };
 template <class T> struct is_fancy_device_iterator<device_ptr<T>> { static constexpr bool value = false; };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Out>
-Out copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out) {
-  const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::transform_n(exec.derived(), thrust::detail::unwrap(first), thrust::detail::unwrap(out), n, identity<typename thrust::detail::value_of<In>::type>());
-  return out + n;
-}
-// contiguous device ranges of one type: a stream-ordered memcpy, no kernel template
-template <class D, class T>
-device_ptr<typename std::remove_const<T>::type> copy(const system::cdna4::execution_policy<D>& exec, device_ptr<T> first, device_ptr<T> last,
-                                                     device_ptr<typename std::remove_const<T>::type> out) {
-  namespace sd = system::cdna4::detail;
-  const std::size_t n = (std::size_t)(last - first);
-  if (n) sd::throw_on_error(thrust_cdna4_memcpy_dtod(out.get(), first.get(), n * sizeof(T), sd::stream_of(exec.derived())), "copy");
-  sd::synchronize_optional(exec.derived(), "copy: failed to synchronize");
-  return out + n;
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/copy.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/copy.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -46,25 +46,9 @@ extremum<typename value_of<It>::type> extrema_of(const Policy& exec, It first, I
                                              extremum<V>{V(), -1, V(), -1}, extremum_merge<V, Compare>{comp});
 }
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It, class Compare>
-It min_element(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) {
-  if (first == last) return last;
-  return first + thrust::detail::extrema_of(exec.derived(), first, last, comp).lo_at;
-}
-template <class D, class It, class Compare>
-It max_element(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) {
-  if (first == last) return last;
-  return first + thrust::detail::extrema_of(exec.derived(), first, last, comp).hi_at;
-}
-template <class D, class It, class Compare>
-pair<It, It> minmax_element(const system::cdna4::execution_policy<D>& exec, It first, It last, Compare comp) {
-  if (first == last) return thrust::make_pair(last, last);
-  const auto e = thrust::detail::extrema_of(exec.derived(), first, last, comp);
-  return thrust::make_pair(first + e.lo_at, first + e.hi_at);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/extrema.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/extrema.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

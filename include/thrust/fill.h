@@ -35,13 +35,9 @@ void fill_device(const Policy& exec, Out first, std::int64_t n, const V& value) 
 }
 }  // namespace detail
 
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It, class V>
-void fill(const system::cdna4::execution_policy<D>& exec, It first, It last, const V& value) {
-  thrust::detail::fill_device(exec.derived(), first, (std::int64_t)(last - first), value);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/fill.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/fill.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -28,13 +28,9 @@ template <class Pred> struct negated {
   template <class T> THRUST_CDNA4_HD bool operator()(const T& x) const { return !pred(x); }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It, class Pred>
-It find_if(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) { return thrust::detail::find_first<false>(exec.derived(), first, last, pred); }
-template <class D, class It, class Pred>
-It find_if_not(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) { return thrust::detail::find_first<true>(exec.derived(), first, last, pred); }
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/find.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/find.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -6,19 +6,9 @@
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementation, found through the policy's type
-template <class D, class It, class F>
-It for_each(const execution_policy<D>& exec, It first, It last, F f) {
-  detail::apply_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)(last - first), f);
-  return last;
-}
-template <class D, class It, class Size, class F>
-It for_each_n(const execution_policy<D>& exec, It first, Size n, F f) {
-  detail::apply_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)n, f);
-  return first + n;
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/for_each.h>
+namespace thrust {
 
 // The entry points dispatch on the policy's own type by an unqualified call, as the reference's
 // do (thrust/detail/for_each.inl:32-44): the device system's overload above is found through the

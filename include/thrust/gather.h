@@ -21,19 +21,9 @@ struct truthy {
   template <class T> THRUST_CDNA4_HD bool operator()(const T& x) const { return x ? true : false; }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class Map, class In, class Out>
-Out gather(const system::cdna4::execution_policy<D>& exec, Map map_first, Map map_last, In input, Out result) {
-  const std::int64_t n = (std::int64_t)(map_last - map_first);
-  system::cdna4::detail::for_each_index(
-      exec.derived(), n,
-      thrust::detail::gather_body<typename thrust::detail::unwrap_iterator<Map>::type, typename thrust::detail::unwrap_iterator<In>::type,
-                          typename thrust::detail::unwrap_iterator<Out>::type>{thrust::detail::unwrap(map_first), thrust::detail::unwrap(input), thrust::detail::unwrap(result)},
-      "gather: failed to synchronize");
-  return result + n;
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/gather.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/gather.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.
@@ -46,20 +36,9 @@ Out gather(const system::cpp::detail::par_t&, Map map_first, Map map_last, In in
   for (; map_first != map_last; ++map_first, ++result) *result = input[*map_first];
   return result;
 }
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class Map, class S, class In, class Out, class Pred>
-Out gather_if(const system::cdna4::execution_policy<D>& exec, Map map_first, Map map_last, S stencil, In input, Out result, Pred pred) {
-  const std::int64_t n = (std::int64_t)(map_last - map_first);
-  system::cdna4::detail::for_each_index(
-      exec.derived(), n,
-      thrust::detail::gather_if_body<typename thrust::detail::unwrap_iterator<Map>::type, typename thrust::detail::unwrap_iterator<S>::type,
-                             typename thrust::detail::unwrap_iterator<In>::type, typename thrust::detail::unwrap_iterator<Out>::type, Pred>{
-          thrust::detail::unwrap(map_first), thrust::detail::unwrap(stencil), thrust::detail::unwrap(input), thrust::detail::unwrap(result), pred},
-      "gather_if: failed to synchronize");
-  return result + n;
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/gather_if.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/gather.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

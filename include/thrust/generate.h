@@ -12,15 +12,9 @@ template <class Out, class G> struct generate_body {
   THRUST_CDNA4_HD void operator()(std::int64_t i) { out[i] = gen(); }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It, class G>
-void generate(const system::cdna4::execution_policy<D>& exec, It first, It last, G gen) {
-  typedef typename thrust::detail::unwrap_iterator<It>::type Out;
-  system::cdna4::detail::for_each_index(exec.derived(), (std::int64_t)(last - first),
-                                        thrust::detail::generate_body<Out, G>{thrust::detail::unwrap(first), gen}, "generate: failed to synchronize");
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/generate.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/generate.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -14,17 +14,9 @@ template <class A, class B, class Op2, class T> struct product_at {
   THRUST_CDNA4_HD T operator()(std::int64_t i) const { return (T)op2(a[i], b[i]); }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It1, class It2, class T, class Op1, class Op2>
-T inner_product(const system::cdna4::execution_policy<D>& exec, It1 first1, It1 last1, It2 first2, T init, Op1 op1, Op2 op2) {
-  return system::cdna4::detail::reduce_index(
-      exec.derived(), (std::int64_t)(last1 - first1),
-      thrust::detail::product_at<typename thrust::detail::unwrap_iterator<It1>::type, typename thrust::detail::unwrap_iterator<It2>::type, Op2, T>{
-          thrust::detail::unwrap(first1), thrust::detail::unwrap(first2), op2},
-      init, op1);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/inner_product.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/inner_product.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

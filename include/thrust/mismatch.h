@@ -14,19 +14,9 @@ template <class A, class B, class Pred> struct differ_index {
   THRUST_CDNA4_HD std::int64_t operator()(std::int64_t i) const { return pred(a[i], b[i]) ? n : i; }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It1, class It2, class Pred>
-pair<It1, It2> mismatch(const system::cdna4::execution_policy<D>& exec, It1 first1, It1 last1, It2 first2, Pred pred) {
-  const std::int64_t n = (std::int64_t)(last1 - first1);
-  const std::int64_t at = system::cdna4::detail::reduce_index(
-      exec.derived(), n,
-      thrust::detail::differ_index<typename thrust::detail::unwrap_iterator<It1>::type, typename thrust::detail::unwrap_iterator<It2>::type, Pred>{
-          thrust::detail::unwrap(first1), thrust::detail::unwrap(first2), pred, n},
-      n, thrust::detail::min_index());
-  return thrust::make_pair(first1 + at, first2 + at);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/mismatch.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/mismatch.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -40,35 +40,9 @@ std::int64_t reduce_by_key_dispatch(const Policy& exec, KIn keys, VIn vals, KOut
 }
 }  // namespace detail
 
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-// Raw device pointers to arithmetic types under equal_to and a built-in operator run the
-// precompiled segmented-reduction kernel; everything else (user predicates and operators, fancy
-// iterators read in place, more than 2^32 - 1 elements) the kernel templates of scan_generic.h.
-template <class D, class KIt, class VIt, class KOut, class VOut, class Pred, class Op>
-pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
-                               KOut kout, VOut vout, Pred pred, Op op) {
-  typedef typename thrust::detail::elem<KIt>::type K;
-  typedef typename thrust::detail::elem<VIt>::type V;
-  typedef typename thrust::detail::unwrap_iterator<KIt>::type KIn;
-  typedef typename thrust::detail::unwrap_iterator<VIt>::type VIn;
-  typedef typename thrust::detail::unwrap_iterator<KOut>::type KO;
-  typedef typename thrust::detail::unwrap_iterator<VOut>::type VO;
-  const std::int64_t n = (std::int64_t)(klast - kfirst);
-  const std::int64_t runs = thrust::detail::reduce_by_key_dispatch<K, V>(
-      exec.derived(), thrust::detail::unwrap(kfirst), thrust::detail::unwrap(vfirst), thrust::detail::unwrap(kout), thrust::detail::unwrap(vout), n, pred, op,
-      std::integral_constant<bool, thrust::detail::reduce_by_key_has_kernel<K, V, KIn, VIn, KO, VO, Pred, Op>::value>());
-  return thrust::make_pair(kout + runs, vout + runs);
-}
-template <class D, class KIt, class VIt, class KOut, class VOut, class Pred>
-pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred p) {
-  return reduce_by_key(exec, kf, kl, vf, ko, vo, p, plus<>());
-}
-template <class D, class KIt, class VIt, class KOut, class VOut>
-pair<KOut, VOut> reduce_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo) {
-  return reduce_by_key(exec, kf, kl, vf, ko, vo, equal_to<>());
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/reduce_by_key.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/reduce.inl:33-44, :112-130):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.
@@ -132,25 +106,9 @@ THRUST_CDNA4_RBK(host, detail::enable_if_host)
 #undef THRUST_CDNA4_RBK
 
 
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-// ---------------------------------------------------------------------------------------
-// reduce
-// ---------------------------------------------------------------------------------------
-template <class D, class It, class T, class Op>
-T reduce(const system::cdna4::execution_policy<D>& exec, It first, It last, T init, Op op) {
-  typedef typename thrust::detail::value_of<It>::type V;
-  return system::cdna4::detail::transform_reduce_n(exec.derived(), thrust::detail::unwrap(first),
-                                                   (std::int64_t)(last - first), identity<V>(), init, op);
-}
-template <class D, class It, class T>
-T reduce(const system::cdna4::execution_policy<D>& exec, It first, It last, T init) { return reduce(exec, first, last, init, plus<T>()); }
-template <class D, class It>
-typename thrust::detail::value_of<It>::type reduce(const system::cdna4::execution_policy<D>& exec, It first, It last) {
-  typedef typename thrust::detail::value_of<It>::type V;
-  return reduce(exec, first, last, V(0), plus<V>());
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/reduce.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/reduce.inl:33-44, :112-130):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -8,22 +8,9 @@
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Out, class Pred>
-Out remove_copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Pred pred) {
-  typedef typename thrust::detail::value_of<In>::type V;
-  const V* in = thrust::detail::unwrap(first);
-  return out + system::cdna4::detail::copy_flagged_n<true>(exec.derived(), in, thrust::detail::unwrap(out), (std::int64_t)(last - first), pred);
-}
-template <class D, class In, class Pred>
-In remove_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Pred pred) {
-  typedef typename thrust::detail::value_of<In>::type V;
-  const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::scratch_copy<V> tmp((const V*)thrust::detail::unwrap(first), n, system::cdna4::detail::stream_of(exec.derived()));
-  return first + system::cdna4::detail::copy_flagged_n<true>(exec.derived(), tmp.data(), thrust::detail::unwrap(first), n, pred);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/remove.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/remove.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -17,19 +17,9 @@ template <class In, class S, class Out, class Pred, class T> struct replace_body
   }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class S, class Out, class Pred, class T>
-Out replace_copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, S stencil, Out result, Pred pred, const T& value) {
-  const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::for_each_index(
-      exec.derived(), n,
-      thrust::detail::replace_body<typename thrust::detail::unwrap_iterator<In>::type, typename thrust::detail::unwrap_iterator<S>::type,
-                           typename thrust::detail::unwrap_iterator<Out>::type, Pred, T>{thrust::detail::unwrap(first), thrust::detail::unwrap(stencil), thrust::detail::unwrap(result), pred, value},
-      "replace: failed to synchronize");
-  return result + n;
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/replace.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/replace.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -20,15 +20,9 @@ template <class In, class Out> struct reverse_copy_body {
   THRUST_CDNA4_HD void operator()(std::int64_t i) { out[i] = in[n - 1 - i]; }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It>
-void reverse(const system::cdna4::execution_policy<D>& exec, It first, It last) {
-  const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::for_each_index(exec.derived(), n / 2, thrust::detail::reverse_body<typename thrust::detail::unwrap_iterator<It>::type>{thrust::detail::unwrap(first), n},
-                                        "reverse: failed to synchronize");
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/reverse.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/reverse.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.
@@ -37,18 +31,9 @@ void reverse(const detail::execution_policy_base<D>& exec, It first, It last) {
   reverse(detail::derived_cast(detail::strip_const(exec)), first, last);
 }
 template <class It> void reverse(const system::cpp::detail::par_t&, It first, It last) { std::reverse(first, last); }
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Out>
-Out reverse_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out result) {
-  const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::for_each_index(
-      exec.derived(), n,
-      thrust::detail::reverse_copy_body<typename thrust::detail::unwrap_iterator<In>::type, typename thrust::detail::unwrap_iterator<Out>::type>{thrust::detail::unwrap(first), thrust::detail::unwrap(result), n},
-      "reverse_copy: failed to synchronize");
-  return result + n;
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/reverse_copy.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/reverse.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

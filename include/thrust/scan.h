@@ -54,43 +54,9 @@ void scan_dispatch(const Policy& exec, In in, Out out, std::int64_t n, T init, O
 }
 }  // namespace detail
 
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-// The accumulator of an inclusive scan has the input's value type (thrust/system/cuda/detail/scan.h:63).
-template <class D, class InIt, class OutIt, class Op>
-OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, Op op) {
-  typedef typename thrust::detail::elem<InIt>::type T;
-  typedef typename thrust::detail::unwrap_iterator<InIt>::type In;
-  typedef typename thrust::detail::unwrap_iterator<OutIt>::type Out;
-  const std::int64_t n = (std::int64_t)(last - first);
-  thrust::detail::scan_dispatch<false>(exec.derived(), thrust::detail::unwrap(first), thrust::detail::unwrap(result), n, T(), op,
-                               std::integral_constant<bool, thrust::detail::scan_has_kernel<T, In, Out, Op>::value>());
-  return result + n;
-}
-template <class D, class InIt, class OutIt>
-OutIt inclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result) {
-  return inclusive_scan(exec, first, last, result, plus<>());
-}
-// The accumulator of an exclusive scan has the type of `init` (thrust/system/cuda/detail/scan.h:142-154).
-template <class D, class InIt, class OutIt, class T, class Op>
-OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, T init, Op op) {
-  typedef typename thrust::detail::unwrap_iterator<InIt>::type In;
-  typedef typename thrust::detail::unwrap_iterator<OutIt>::type Out;
-  const std::int64_t n = (std::int64_t)(last - first);
-  thrust::detail::scan_dispatch<true>(exec.derived(), thrust::detail::unwrap(first), thrust::detail::unwrap(result), n, init, op,
-                              std::integral_constant<bool, thrust::detail::scan_has_kernel<T, In, Out, Op>::value>());
-  return result + n;
-}
-template <class D, class InIt, class OutIt, class T>
-OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result, T init) {
-  return exclusive_scan(exec, first, last, result, init, plus<>());
-}
-template <class D, class InIt, class OutIt>
-OutIt exclusive_scan(const system::cdna4::execution_policy<D>& exec, InIt first, InIt last, OutIt result) {
-  typedef typename thrust::detail::elem<InIt>::type V;
-  return exclusive_scan(exec, first, last, result, V(), plus<>());  // thrust/system/cuda/detail/scan.h:347-348
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/scan.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/scan.inl:35-48):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.
@@ -208,58 +174,9 @@ void scan_by_key_dispatch(const Policy& exec, KIn keys, VIn vals, Out out, std::
 }
 }  // namespace detail
 
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-// The accumulator has the value input's type for the inclusive form and the type of `init` for
-// the exclusive one (thrust/system/cuda/detail/scan_by_key.h:69-282).
-template <class D, class KIt, class VIt, class OutIt, class Pred, class Op>
-OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
-                            OutIt result, Pred pred, Op op) {
-  typedef typename thrust::detail::elem<KIt>::type K;
-  typedef typename thrust::detail::elem<VIt>::type V;
-  typedef typename thrust::detail::unwrap_iterator<KIt>::type KIn;
-  typedef typename thrust::detail::unwrap_iterator<VIt>::type VIn;
-  typedef typename thrust::detail::unwrap_iterator<OutIt>::type Out;
-  const std::int64_t n = (std::int64_t)(klast - kfirst);
-  thrust::detail::scan_by_key_dispatch<false, K>(exec.derived(), thrust::detail::unwrap(kfirst), thrust::detail::unwrap(vfirst), thrust::detail::unwrap(result), n,
-                                         V(), pred, op,
-                                         std::integral_constant<bool, thrust::detail::scan_by_key_has_kernel<K, V, KIn, VIn, Out, Pred, Op>::value>());
-  return result + n;
-}
-template <class D, class KIt, class VIt, class OutIt, class Pred>
-OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, Pred p) {
-  return inclusive_scan_by_key(exec, kf, kl, vf, r, p, plus<>());
-}
-template <class D, class KIt, class VIt, class OutIt>
-OutIt inclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r) {
-  return inclusive_scan_by_key(exec, kf, kl, vf, r, equal_to<>());
-}
-template <class D, class KIt, class VIt, class OutIt, class T, class Pred, class Op>
-OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kfirst, KIt klast, VIt vfirst,
-                            OutIt result, T init, Pred pred, Op op) {
-  typedef typename thrust::detail::elem<KIt>::type K;
-  typedef typename thrust::detail::unwrap_iterator<KIt>::type KIn;
-  typedef typename thrust::detail::unwrap_iterator<VIt>::type VIn;
-  typedef typename thrust::detail::unwrap_iterator<OutIt>::type Out;
-  const std::int64_t n = (std::int64_t)(klast - kfirst);
-  thrust::detail::scan_by_key_dispatch<true, K>(exec.derived(), thrust::detail::unwrap(kfirst), thrust::detail::unwrap(vfirst), thrust::detail::unwrap(result), n,
-                                        init, pred, op,
-                                        std::integral_constant<bool, thrust::detail::scan_by_key_has_kernel<K, T, KIn, VIn, Out, Pred, Op>::value>());
-  return result + n;
-}
-template <class D, class KIt, class VIt, class OutIt, class T, class Pred>
-OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, T init, Pred p) {
-  return exclusive_scan_by_key(exec, kf, kl, vf, r, init, p, plus<>());
-}
-template <class D, class KIt, class VIt, class OutIt, class T>
-OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r, T init) {
-  return exclusive_scan_by_key(exec, kf, kl, vf, r, init, equal_to<>());
-}
-template <class D, class KIt, class VIt, class OutIt>
-OutIt exclusive_scan_by_key(const system::cdna4::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, OutIt r) {
-  return exclusive_scan_by_key(exec, kf, kl, vf, r, typename thrust::detail::elem<VIt>::type());
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/scan_by_key.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/scan.inl:35-48):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -18,17 +18,9 @@ template <class In, class Map, class S, class Out, class Pred> struct scatter_if
   }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Map, class Out>
-void scatter(const system::cdna4::execution_policy<D>& exec, In first, In last, Map map, Out output) {
-  system::cdna4::detail::for_each_index(
-      exec.derived(), (std::int64_t)(last - first),
-      thrust::detail::scatter_body<typename thrust::detail::unwrap_iterator<In>::type, typename thrust::detail::unwrap_iterator<Map>::type,
-                           typename thrust::detail::unwrap_iterator<Out>::type>{thrust::detail::unwrap(first), thrust::detail::unwrap(map), thrust::detail::unwrap(output)},
-      "scatter: failed to synchronize");
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/scatter.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/scatter.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.
@@ -40,18 +32,9 @@ template <class In, class Map, class Out>
 void scatter(const system::cpp::detail::par_t&, In first, In last, Map map, Out output) {
   for (; first != last; ++first, ++map) output[*map] = *first;
 }
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Map, class S, class Out, class Pred>
-void scatter_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Map map, S stencil, Out output, Pred pred) {
-  system::cdna4::detail::for_each_index(
-      exec.derived(), (std::int64_t)(last - first),
-      thrust::detail::scatter_if_body<typename thrust::detail::unwrap_iterator<In>::type, typename thrust::detail::unwrap_iterator<Map>::type,
-                              typename thrust::detail::unwrap_iterator<S>::type, typename thrust::detail::unwrap_iterator<Out>::type, Pred>{
-          thrust::detail::unwrap(first), thrust::detail::unwrap(map), thrust::detail::unwrap(stencil), thrust::detail::unwrap(output), pred},
-      "scatter_if: failed to synchronize");
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/scatter_if.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/scatter.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

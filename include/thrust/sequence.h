@@ -5,14 +5,9 @@
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It, class T>
-void sequence(const system::cdna4::execution_policy<D>& exec, It first, It last, T init, T step) {
-  typedef typename thrust::detail::value_of<It>::type V;
-  system::cdna4::detail::sequence_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)(last - first), (V)init, (V)step);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/sequence.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/sequence.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -66,24 +66,9 @@ template <class In, class Out> struct shuffle_op {
 #endif
 }  // namespace detail
 
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Out, class URBG>
-void shuffle_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out result, URBG&& g) {
-  THRUST_CDNA4_NEEDS_HIPCC(In);
-  const std::uint64_t m = (std::uint64_t)(last - first);
-  if (m == 0) return;
-  thrust::detail::feistel_bijection bijection(m, g);
-#if defined(__HIPCC__)
-  typedef typename thrust::detail::unwrap_iterator<In>::type RawIn;
-  typedef typename thrust::detail::unwrap_iterator<Out>::type RawOut;
-  system::cdna4::detail::generic::select(system::cdna4::detail::stream_of(exec.derived()), (std::int64_t)bijection.nearest_power_of_two(),
-                                         thrust::detail::shuffle_op<RawIn, RawOut>{thrust::detail::unwrap(first), thrust::detail::unwrap(result), m, bijection});
-#else
-  (void)exec; (void)result;
-#endif
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/shuffle_copy.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/shuffle.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.
@@ -105,16 +90,9 @@ void shuffle_copy(const system::cpp::detail::par_t&, In first, In last, Out resu
     }
   }
 }
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-// in place: shuffle a copy back into the range
-template <class D, class It, class URBG>
-void shuffle(const system::cdna4::execution_policy<D>& exec, It first, It last, URBG&& g) {
-  typedef typename std::iterator_traits<It>::value_type T;
-  thrust::device_vector<T> copy(first, last);
-  shuffle_copy(exec, copy.begin(), copy.end(), first, g);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/shuffle.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/shuffle.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

@@ -22,18 +22,9 @@ template <class A, class B> struct swap_body {
   }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It1, class It2>
-It2 swap_ranges(const system::cdna4::execution_policy<D>& exec, It1 first1, It1 last1, It2 first2) {
-  const std::int64_t n = (std::int64_t)(last1 - first1);
-  system::cdna4::detail::for_each_index(
-      exec.derived(), n,
-      thrust::detail::swap_body<typename thrust::detail::unwrap_iterator<It1>::type, typename thrust::detail::unwrap_iterator<It2>::type>{thrust::detail::unwrap(first1), thrust::detail::unwrap(first2)},
-      "swap_ranges: failed to synchronize");
-  return first2 + n;
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/swap_ranges.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/swap.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

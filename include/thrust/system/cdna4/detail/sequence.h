@@ -1,0 +1,15 @@
+// The cdna4 device system's sequence (the counterpart of thrust/system/cuda/detail/sequence.h): free functions
+// in the policy's namespace, found by the unqualified calls of the entry points in <thrust/sequence.h>,
+// which includes this file where the helpers it uses have been declared.
+#pragma once
+#include <thrust/sequence.h>
+namespace thrust {
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
+template <class D, class It, class T>
+void sequence(const system::cdna4::execution_policy<D>& exec, It first, It last, T init, T step) {
+  typedef typename thrust::detail::value_of<It>::type V;
+  system::cdna4::detail::sequence_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)(last - first), (V)init, (V)step);
+}
+}}  // namespace system::cdna4
+}  // namespace thrust

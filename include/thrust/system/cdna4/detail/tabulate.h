@@ -1,0 +1,16 @@
+// The cdna4 device system's tabulate (the counterpart of thrust/system/cuda/detail/tabulate.h): free functions
+// in the policy's namespace, found by the unqualified calls of the entry points in <thrust/tabulate.h>,
+// which includes this file where the helpers it uses have been declared.
+#pragma once
+#include <thrust/tabulate.h>
+namespace thrust {
+namespace system { namespace cdna4 {
+// the device system's implementations, found through the policy's type
+template <class D, class It, class F>
+void tabulate(const system::cdna4::execution_policy<D>& exec, It first, It last, F f) {
+  typedef typename thrust::detail::unwrap_iterator<It>::type Out;
+  system::cdna4::detail::for_each_index(exec.derived(), (std::int64_t)(last - first),
+                                        thrust::detail::tabulate_body<Out, F>{thrust::detail::unwrap(first), f}, "tabulate: failed to synchronize");
+}
+}}  // namespace system::cdna4
+}  // namespace thrust

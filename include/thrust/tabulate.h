@@ -11,15 +11,9 @@ template <class Out, class F> struct tabulate_body {
   THRUST_CDNA4_HD void operator()(std::int64_t i) { out[i] = f((typename std::iterator_traits<Out>::difference_type)i); }
 };
 }  // namespace detail
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It, class F>
-void tabulate(const system::cdna4::execution_policy<D>& exec, It first, It last, F f) {
-  typedef typename thrust::detail::unwrap_iterator<It>::type Out;
-  system::cdna4::detail::for_each_index(exec.derived(), (std::int64_t)(last - first),
-                                        thrust::detail::tabulate_body<Out, F>{thrust::detail::unwrap(first), f}, "tabulate: failed to synchronize");
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/tabulate.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/tabulate.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

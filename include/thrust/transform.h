@@ -6,23 +6,9 @@
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Out, class F>
-Out transform(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, F f) {
-  const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::transform_n(exec.derived(), thrust::detail::unwrap(first),
-                                     thrust::detail::unwrap(out), n, f);
-  return out + n;
-}
-template <class D, class In1, class In2, class Out, class F>
-Out transform(const system::cdna4::execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out out, F f) {
-  const std::int64_t n = (std::int64_t)(last1 - first1);
-  system::cdna4::detail::transform_n(exec.derived(), thrust::detail::unwrap(first1),
-                                     thrust::detail::unwrap(first2), thrust::detail::unwrap(out), n, f);
-  return out + n;
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/transform.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/transform.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

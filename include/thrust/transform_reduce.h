@@ -6,14 +6,9 @@
 
 #include <thrust/reduce.h>
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It, class F, class T, class Op>
-T transform_reduce(const system::cdna4::execution_policy<D>& exec, It first, It last, F f, T init, Op op) {
-  return system::cdna4::detail::transform_reduce_n(exec.derived(), thrust::detail::unwrap(first),
-                                                   (std::int64_t)(last - first), f, init, op);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/transform_reduce.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/transform_reduce.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

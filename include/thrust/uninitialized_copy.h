@@ -4,11 +4,9 @@
 #include <memory>
 #include <thrust/copy.h>
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class In, class Out>
-Out uninitialized_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out result) { return copy(exec, first, last, result); }
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/uninitialized_copy.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/uninitialized_copy.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

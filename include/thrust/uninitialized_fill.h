@@ -5,11 +5,9 @@
 #include <memory>
 #include <thrust/fill.h>
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-template <class D, class It, class T>
-void uninitialized_fill(const system::cdna4::execution_policy<D>& exec, It first, It last, const T& x) { fill(exec, first, last, x); }
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/uninitialized_fill.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/uninitialized_fill.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

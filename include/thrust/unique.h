@@ -10,45 +10,9 @@
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
-namespace system { namespace cdna4 {
-// the device system's implementations, found through the policy's type
-// ---- device
-template <class D, class In, class Out, class Eq>
-Out unique_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Eq eq) {
-  typedef typename thrust::detail::value_of<In>::type V;
-  return out + system::cdna4::detail::unique_copy_n(exec.derived(), thrust::detail::unwrap(first), thrust::detail::unwrap(out),
-                                                    (std::int64_t)(last - first), eq);
-}
-template <class D, class In, class Eq>
-In unique(const system::cdna4::execution_policy<D>& exec, In first, In last, Eq eq) {
-  typedef typename thrust::detail::value_of<In>::type V;
-  const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::scratch_copy<V> tmp((const V*)thrust::detail::unwrap(first), n, system::cdna4::detail::stream_of(exec.derived()));
-  return first + system::cdna4::detail::unique_copy_n(exec.derived(), tmp.data(), thrust::detail::unwrap(first), n, eq);
-}
-template <class D, class KIn, class VIn, class KOut, class VOut, class Eq>
-pair<KOut, VOut> unique_by_key_copy(const system::cdna4::execution_policy<D>& exec, KIn kfirst, KIn klast, VIn vfirst,
-                                    KOut kout, VOut vout, Eq eq) {
-  typedef typename thrust::detail::value_of<KIn>::type K;
-  typedef typename thrust::detail::value_of<VIn>::type V;
-  const std::int64_t c = system::cdna4::detail::unique_by_key_copy_n(
-      exec.derived(), thrust::detail::unwrap(kfirst), thrust::detail::unwrap(vfirst), thrust::detail::unwrap(kout),
-      thrust::detail::unwrap(vout), (std::int64_t)(klast - kfirst), eq);
-  return thrust::make_pair(kout + c, vout + c);
-}
-template <class D, class KIn, class VIn, class Eq>
-pair<KIn, VIn> unique_by_key(const system::cdna4::execution_policy<D>& exec, KIn kfirst, KIn klast, VIn vfirst, Eq eq) {
-  typedef typename thrust::detail::value_of<KIn>::type K;
-  typedef typename thrust::detail::value_of<VIn>::type V;
-  const std::int64_t n = (std::int64_t)(klast - kfirst);
-  void* s = system::cdna4::detail::stream_of(exec.derived());
-  system::cdna4::detail::scratch_copy<K> tk((const K*)thrust::detail::unwrap(kfirst), n, s);
-  system::cdna4::detail::scratch_copy<V> tv((const V*)thrust::detail::unwrap(vfirst), n, s);
-  const std::int64_t c = system::cdna4::detail::unique_by_key_copy_n(exec.derived(), tk.data(), tv.data(), thrust::detail::unwrap(kfirst),
-                                                                     thrust::detail::unwrap(vfirst), n, eq);
-  return thrust::make_pair(kfirst + c, vfirst + c);
-}
-}}  // namespace system::cdna4
+}  // namespace thrust
+#include <thrust/system/cdna4/detail/unique.h>
+namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/unique.inl):
 // a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
 // the device system's, which is found through the policy's base class.

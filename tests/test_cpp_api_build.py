@@ -20,7 +20,7 @@ def compile_snippet(tmp_path, body, extra=()):
 def test_cpp_tests_compile():
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    for name in ["test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface",
+    for name in ["test_system_dir", "test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface",
                  "bench_generic"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
 
@@ -214,3 +214,30 @@ def test_every_public_header_compiles_on_its_own(tmp_path):
     for h in headers:  # and each one alone
         r = compile_snippet(tmp_path, '#include <%s>\nint main() { return 0; }\n' % os.path.relpath(h, INC))
         assert r.returncode == 0, (h, r.stderr[-2000:])
+
+
+# the per-algorithm headers a device system's directory holds: one for every name under the
+# reference's thrust/system/detail/adl/ (each adl/<name>.h includes <system root>/detail/<name>.h)
+SYSTEM_DETAIL_NAMES = """adjacent_difference assign_value binary_search copy copy_if count equal extrema fill find for_each
+gather generate get_value inner_product iter_swap logical malloc_and_free merge mismatch partition per_device_resource
+reduce reduce_by_key remove replace reverse scan scan_by_key scatter sequence set_operations sort swap_ranges tabulate
+temporary_buffer transform transform_reduce transform_scan uninitialized_copy uninitialized_fill unique unique_by_key""".split()
+
+
+def test_the_system_directory_has_the_reference_layout(tmp_path):
+    """thrust/system/cdna4/ holds what the reference asks of a device system's directory
+    (thrust/system/cuda/: execution_policy.h, memory.h, memory_resource.h, pointer.h, vector.h,
+    detail/execution_policy.h, detail/par.h and one detail/<algorithm>.h per name of
+    thrust/system/detail/adl/), and each of these headers compiles when it is the first one included."""
+    root = os.path.join(INC, "thrust", "system", "cdna4")
+    assert len(SYSTEM_DETAIL_NAMES) == 43
+    names = (["execution_policy.h", "memory.h", "memory_resource.h", "pointer.h", "vector.h", "detail/execution_policy.h", "detail/par.h"]
+             + ["detail/%s.h" % n for n in SYSTEM_DETAIL_NAMES])
+    for n in names:
+        assert os.path.exists(os.path.join(root, n)), n
+    ref = "/root/reference/thrust/system/detail/adl"
+    if os.path.isdir(ref):  # the list above is the reference's
+        assert sorted(f[:-2] for f in os.listdir(ref) if f.endswith(".h")) == sorted(SYSTEM_DETAIL_NAMES)
+    for n in names:
+        r = compile_snippet(tmp_path, '#include <thrust/system/cdna4/%s>\nint main() { return 0; }\n' % n)
+        assert r.returncode == 0, (n, r.stderr[-2000:])
