@@ -204,6 +204,30 @@ def main():
             sweep[f"2^{lg}"] = round(m / float(np.median(ms)) / 1e6, 2)
         extras["inclusive_scan_i32_sweep_gelem_per_s"] = sweep
 
+    def extra_narrow():
+        # 1- and 2-byte elements: the scan keeps them packed in registers, and one-byte keys without
+        # values are sorted by histogram and fill (no key moves: 2 bytes of traffic per key)
+        for tname, tdt, code in (("i8", torch.int8, capi.I8), ("i16", torch.int16, capi.I16)):
+            x = torch.randint(-3, 4, (n,), dtype=tdt, device=dev, generator=gen(31))
+            out = torch.empty_like(x)
+            call = lambda t, nb: L.thrust_cdna4_scan(t, ctypes.byref(nb), code, capi.PLUS, 0, ctypes.c_void_p(x.data_ptr()),
+                                                      ctypes.c_void_p(out.data_ptr()), n, None, sp)
+            tmp, nb = two_phase(call)
+            tp = ctypes.c_void_p(tmp.data_ptr())
+            ms = timed(lambda: capi.check(call(tp, nb), "scan"), lambda: None, 10, 2)
+            assert torch.equal(out[-1000:], torch.cumsum(x.to(torch.int32), 0, dtype=torch.int32)[-1000:].to(tdt))
+            add_extra(f"inclusive_scan_{tname}", n, ms, 2.0 * x.element_size() * n, "Gelem/s")
+            del x, out
+        src = torch.randint(0, 256, (n,), dtype=torch.uint8, device=dev, generator=gen(32))
+        k = torch.empty_like(src)
+        call = lambda t, nb: L.thrust_cdna4_sort_keys(t, ctypes.byref(nb), capi.U8, ctypes.c_void_p(k.data_ptr()), n, 0, sp)
+        tmp, nb = two_phase(call)
+        tp = ctypes.c_void_p(tmp.data_ptr())
+        ms = timed(lambda: capi.check(call(tp, nb), "sort_keys"), lambda: k.copy_(src), 10, 2)
+        assert torch.equal(torch.bincount(k.to(torch.int64), minlength=256), torch.bincount(src.to(torch.int64), minlength=256))
+        assert bool((k[1:] >= k[:-1]).all())
+        add_extra("sort_u8_keys", n, ms, 2.0 * n, "Gkeys/s")
+
     def extra_rbk(mean):
         if mean == 1:
             keys = torch.arange(n, dtype=torch.int32, device=dev)
@@ -341,6 +365,7 @@ def main():
         "scan_i32": lambda: extra_scan("i32"),
         "scan_f32": lambda: extra_scan("f32"),
         "scan_sweep": extra_scan_sweep,
+        "narrow": extra_narrow,
         "rbk1": lambda: extra_rbk(1),
         "rbk8": lambda: extra_rbk(8),
         "rbk512": lambda: extra_rbk(512),
