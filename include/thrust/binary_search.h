@@ -7,6 +7,7 @@
 #include <thrust/device_vector.h>
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
+#include <thrust/pair.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 namespace thrust {
@@ -94,4 +95,21 @@ bool binary_search(const Policy& exec, Hay first, Hay last, const T& value) {
 }
 template <class Hay, class T, detail::enable_if_device<Hay> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(device, f, l, v); }
 template <class Hay, class T, detail::enable_if_host<Hay> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(host, f, l, v); }
+
+// ---- equal_range (thrust/binary_search.h:727-1017): the pair (lower_bound, upper_bound) of one value
+template <class Policy, class Hay, class T, class Comp, detail::enable_if_policy<Policy> = 0>
+pair<Hay, Hay> equal_range(const Policy& exec, Hay first, Hay last, const T& value, Comp comp) {
+  const Hay lo = thrust::lower_bound(exec, first, last, value, comp);
+  return pair<Hay, Hay>(lo, thrust::upper_bound(exec, lo, last, value, comp));
+}
+template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>
+pair<Hay, Hay> equal_range(const Policy& exec, Hay first, Hay last, const T& value) {
+  return equal_range(exec, first, last, value, less<T>());
+}
+template <class Hay, class T, detail::enable_if_device<Hay> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(device, f, l, v); }
+template <class Hay, class T, detail::enable_if_host<Hay> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(host, f, l, v); }
+template <class Hay, class T, class Comp, detail::enable_if_device<Hay> = 0, typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>
+pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v, Comp c) { return equal_range(device, f, l, v, c); }
+template <class Hay, class T, class Comp, detail::enable_if_host<Hay> = 0, typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>
+pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v, Comp c) { return equal_range(host, f, l, v, c); }
 }  // namespace thrust

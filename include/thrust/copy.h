@@ -54,8 +54,6 @@ OutIt copy(InIt first, InIt last, OutIt out) {
 #include <thrust/execution_policy.h>
 #include <thrust/detail/iterator_util.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/copy_if.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/copy.inl):

@@ -11,8 +11,41 @@
 #include <vector>
 #include <thrust/execution_policy.h>
 #include <thrust/system/cdna4/detail/core.h>
+#include <thrust/system/error_code.h>
 
 namespace thrust {
+// The errors of events and futures (thrust/detail/event_error.h:33-157): an operation on a handle
+// without a stream (default constructed, moved from, consumed) raises event_error(no_state), one that
+// needs a value on a future without one event_error(no_content).
+enum class event_errc { unknown_event_error, no_state, no_content, last_event_error };
+struct event_error_category : std::error_category {
+  const char* name() const noexcept override { return "event"; }
+  std::string message(int ev) const override {
+    switch (static_cast<event_errc>(ev)) {
+      case event_errc::no_state:
+        return "no_state: an operation that requires an event or future to have a stream or content has been performed on an "
+               "event or future without either, e.g. a moved-from or default constructed one";
+      case event_errc::no_content:
+        return "no_content: an operation that requires a future to have content has been performed on a future without any";
+      default: return "unknown_event_error: an unknown error with a future object has occurred";
+    }
+  }
+};
+inline const std::error_category& event_category() {
+  static const event_error_category result;
+  return result;
+}
+inline std::error_code make_error_code(event_errc e) { return std::error_code(static_cast<int>(e), event_category()); }
+inline std::error_condition make_error_condition(event_errc e) { return std::error_condition(static_cast<int>(e), event_category()); }
+struct event_error : std::logic_error {
+  explicit event_error(std::error_code ec) : std::logic_error(ec.message()), ec_(ec) {}
+  explicit event_error(event_errc e) : event_error(make_error_code(e)) {}
+  const std::error_code& code() const noexcept { return ec_; }
+ private:
+  std::error_code ec_;
+};
+inline bool operator==(const event_error& a, const event_error& b) noexcept { return a.code() == b.code(); }
+inline bool operator<(const event_error& a, const event_error& b) noexcept { return a.code() < b.code(); }
 namespace system { namespace cdna4 { namespace detail {
 // The state shared by an event and the events that depend on it: a stream of its own, plus
 // whatever must stay alive until the stream's work is done.
@@ -90,7 +123,7 @@ class device_event {
   const std::shared_ptr<system::cdna4::detail::async_signal>& signal() const { return signal_; }
  protected:
   system::cdna4::detail::async_signal& state() const {
-    if (!signal_) throw std::logic_error("thrust::device_event: no state");
+    if (!signal_) throw event_error(event_errc::no_state);
     return *signal_;
   }
   std::shared_ptr<system::cdna4::detail::async_signal> signal_;
@@ -110,7 +143,7 @@ class device_future : public device_event {
   // waits for the work, reads the value back (once) and returns it
   T get() {
     if (!have_) {
-      if (!data_) throw std::logic_error("thrust::device_future: no state");
+      if (!data_) throw event_error(signal_ ? event_errc::no_content : event_errc::no_state);
       wait();
       system::cdna4::detail::throw_on_error(thrust_cdna4_read_back(&value_, data_, sizeof(T), stream()), "future: read back");
       have_ = true;
@@ -130,6 +163,13 @@ class device_future : public device_event {
   T value_;
   bool have_;
 };
+
+// the reference's names for the same handles (thrust/future.h:70-116): an event or future of a system
+// is that system's unique eager one, and this build has one device system
+template <class System> using unique_eager_event = device_event;
+template <class T, class System> using unique_eager_future = device_future<T>;
+typedef device_event device_unique_eager_event;
+template <class T> using device_unique_eager_future = device_future<T>;
 
 namespace system { namespace cdna4 { namespace detail {
 // thrust::device.after(events...): the next asynchronous algorithm starts after these

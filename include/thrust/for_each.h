@@ -5,8 +5,6 @@
 #include <thrust/execution_policy.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/for_each.h>
 namespace thrust {
 

@@ -14,36 +14,101 @@ template <class Argument1, class Argument2, class Result> struct binary_function
   typedef Argument2 second_argument_type;
   typedef Result result_type;
 };
-template <class T = void> struct plus { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a + b; } };
-template <class T = void> struct multiplies { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a * b; } };
-template <class T = void> struct maximum { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a < b ? b : a; } };
-template <class T = void> struct minimum { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a < b ? a : b; } };
-template <class T = void> struct less { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a < b; } };
-template <class T = void> struct greater { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a > b; } };
-template <class T = void> struct equal_to { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a == b; } };
-template <class T = void> struct minus { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a - b; } };
-template <class T = void> struct divides { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a / b; } };
-template <class T = void> struct modulus { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a % b; } };
-template <class T = void> struct negate { THRUST_CDNA4_HD constexpr T operator()(const T& a) const { return -a; } };
-template <class T = void> struct not_equal_to { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a != b; } };
-template <class T = void> struct less_equal { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a <= b; } };
-template <class T = void> struct greater_equal { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a >= b; } };
-template <class T = void> struct logical_and { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a && b; } };
-template <class T = void> struct logical_or { THRUST_CDNA4_HD constexpr bool operator()(const T& a, const T& b) const { return a || b; } };
-template <class T = void> struct logical_not { THRUST_CDNA4_HD constexpr bool operator()(const T& a) const { return !a; } };
-template <class T = void> struct bit_and { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a & b; } };
-template <class T = void> struct bit_or { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a | b; } };
-template <class T = void> struct bit_xor { THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a ^ b; } };
-template <class T = void> struct identity { THRUST_CDNA4_HD constexpr const T& operator()(const T& a) const { return a; } };
-
-// transparent forms (thrust::plus<> etc.)
-template <> struct plus<void> { template <class A, class B> THRUST_CDNA4_HD constexpr auto operator()(const A& a, const B& b) const -> decltype(a + b) { return a + b; } };
-template <> struct multiplies<void> { template <class A, class B> THRUST_CDNA4_HD constexpr auto operator()(const A& a, const B& b) const -> decltype(a * b) { return a * b; } };
-template <> struct maximum<void> { template <class A> THRUST_CDNA4_HD constexpr A operator()(const A& a, const A& b) const { return a < b ? b : a; } };
-template <> struct minimum<void> { template <class A> THRUST_CDNA4_HD constexpr A operator()(const A& a, const A& b) const { return a < b ? a : b; } };
-template <> struct less<void> { template <class A, class B> THRUST_CDNA4_HD constexpr bool operator()(const A& a, const B& b) const { return a < b; } };
-template <> struct greater<void> { template <class A, class B> THRUST_CDNA4_HD constexpr bool operator()(const A& a, const B& b) const { return a > b; } };
-template <> struct equal_to<void> { template <class A, class B> THRUST_CDNA4_HD constexpr bool operator()(const A& a, const B& b) const { return a == b; } };
+// The arithmetic, comparison, logical and bitwise function objects (thrust/functional.h:129-1130), each
+// with the argument / result typedefs of an adaptable function object and a transparent form
+// (thrust::plus<> etc.) that deduces its types per call.
+#define THRUST_CDNA4_BINARY_FUNCTOR(NAME, RESULT, EXPR)                                                                   \
+  template <class T = void> struct NAME {                                                                                \
+    typedef T first_argument_type;                                                                                       \
+    typedef T second_argument_type;                                                                                      \
+    typedef RESULT result_type;                                                                                          \
+    THRUST_CDNA4_HD constexpr RESULT operator()(const T& a, const T& b) const { return EXPR; }                            \
+  };                                                                                                                     \
+  template <> struct NAME<void> {                                                                                        \
+    typedef void is_transparent;                                                                                         \
+    template <class A, class B> THRUST_CDNA4_HD constexpr auto operator()(const A& a, const B& b) const -> decltype(EXPR) { return EXPR; } \
+  };
+#define THRUST_CDNA4_UNARY_FUNCTOR(NAME, RESULT, EXPR)                                                                    \
+  template <class T = void> struct NAME {                                                                                \
+    typedef T argument_type;                                                                                             \
+    typedef RESULT result_type;                                                                                          \
+    THRUST_CDNA4_HD constexpr RESULT operator()(const T& a) const { return EXPR; }                                        \
+  };                                                                                                                     \
+  template <> struct NAME<void> {                                                                                        \
+    typedef void is_transparent;                                                                                         \
+    template <class A> THRUST_CDNA4_HD constexpr auto operator()(const A& a) const -> decltype(EXPR) { return EXPR; }      \
+  };
+THRUST_CDNA4_BINARY_FUNCTOR(plus, T, a + b)
+THRUST_CDNA4_BINARY_FUNCTOR(minus, T, a - b)
+THRUST_CDNA4_BINARY_FUNCTOR(multiplies, T, a * b)
+THRUST_CDNA4_BINARY_FUNCTOR(divides, T, a / b)
+THRUST_CDNA4_BINARY_FUNCTOR(modulus, T, a % b)
+THRUST_CDNA4_UNARY_FUNCTOR(negate, T, -a)
+THRUST_CDNA4_UNARY_FUNCTOR(square, T, a * a)
+THRUST_CDNA4_BINARY_FUNCTOR(equal_to, bool, a == b)
+THRUST_CDNA4_BINARY_FUNCTOR(not_equal_to, bool, a != b)
+THRUST_CDNA4_BINARY_FUNCTOR(greater, bool, a > b)
+THRUST_CDNA4_BINARY_FUNCTOR(less, bool, a < b)
+THRUST_CDNA4_BINARY_FUNCTOR(greater_equal, bool, a >= b)
+THRUST_CDNA4_BINARY_FUNCTOR(less_equal, bool, a <= b)
+THRUST_CDNA4_BINARY_FUNCTOR(logical_and, bool, a && b)
+THRUST_CDNA4_BINARY_FUNCTOR(logical_or, bool, a || b)
+THRUST_CDNA4_UNARY_FUNCTOR(logical_not, bool, !a)
+THRUST_CDNA4_BINARY_FUNCTOR(bit_and, T, a & b)
+THRUST_CDNA4_BINARY_FUNCTOR(bit_or, T, a | b)
+THRUST_CDNA4_BINARY_FUNCTOR(bit_xor, T, a ^ b)
+#undef THRUST_CDNA4_BINARY_FUNCTOR
+#undef THRUST_CDNA4_UNARY_FUNCTOR
+// maximum / minimum return one of their arguments (thrust/functional.h:1196-1284): the first of two
+// equivalent ones for minimum, the first for maximum as well (a < b ? b : a)
+template <class T = void> struct maximum {
+  typedef T first_argument_type; typedef T second_argument_type; typedef T result_type;
+  THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a < b ? b : a; }
+};
+template <class T = void> struct minimum {
+  typedef T first_argument_type; typedef T second_argument_type; typedef T result_type;
+  THRUST_CDNA4_HD constexpr T operator()(const T& a, const T& b) const { return a < b ? a : b; }
+};
+template <> struct maximum<void> { typedef void is_transparent; template <class A> THRUST_CDNA4_HD constexpr A operator()(const A& a, const A& b) const { return a < b ? b : a; } };
+template <> struct minimum<void> { typedef void is_transparent; template <class A> THRUST_CDNA4_HD constexpr A operator()(const A& a, const A& b) const { return a < b ? a : b; } };
+template <class T = void> struct identity {
+  typedef T argument_type; typedef T result_type;
+  THRUST_CDNA4_HD constexpr const T& operator()(const T& a) const { return a; }
+};
+template <> struct identity<void> { typedef void is_transparent; template <class A> THRUST_CDNA4_HD constexpr const A& operator()(const A& a) const { return a; } };
+// project1st / project2nd return one of their two arguments (thrust/functional.h:1303-1396)
+template <class T1 = void, class T2 = void> struct project1st {
+  typedef T1 first_argument_type; typedef T2 second_argument_type; typedef T1 result_type;
+  THRUST_CDNA4_HD constexpr const T1& operator()(const T1& a, const T2&) const { return a; }
+};
+template <> struct project1st<void, void> { typedef void is_transparent; template <class A, class B> THRUST_CDNA4_HD constexpr const A& operator()(const A& a, const B&) const { return a; } };
+template <class T1 = void, class T2 = void> struct project2nd {
+  typedef T1 first_argument_type; typedef T2 second_argument_type; typedef T2 result_type;
+  THRUST_CDNA4_HD constexpr const T2& operator()(const T1&, const T2& b) const { return b; }
+};
+template <> struct project2nd<void, void> { typedef void is_transparent; template <class A, class B> THRUST_CDNA4_HD constexpr const B& operator()(const A&, const B& b) const { return b; } };
+// negators (thrust/functional.h:1411-1529): unary_negate / not1 and binary_negate / not2 for adaptable
+// predicates, not_fn for any callable
+template <class Predicate> struct unary_negate : unary_function<typename Predicate::argument_type, bool> {
+  THRUST_CDNA4_HD explicit unary_negate(Predicate p) : pred(p) {}
+  THRUST_CDNA4_HD bool operator()(const typename Predicate::argument_type& x) { return !pred(x); }
+  Predicate pred;
+};
+template <class Predicate> THRUST_CDNA4_HD unary_negate<Predicate> not1(const Predicate& pred) { return unary_negate<Predicate>(pred); }
+template <class Predicate> struct binary_negate : binary_function<typename Predicate::first_argument_type, typename Predicate::second_argument_type, bool> {
+  THRUST_CDNA4_HD explicit binary_negate(Predicate p) : pred(p) {}
+  THRUST_CDNA4_HD bool operator()(const typename Predicate::first_argument_type& x, const typename Predicate::second_argument_type& y) { return !pred(x, y); }
+  Predicate pred;
+};
+template <class Predicate> THRUST_CDNA4_HD binary_negate<Predicate> not2(const Predicate& pred) { return binary_negate<Predicate>(pred); }
+namespace detail {
+template <class F> struct not_fun_t {
+  F f;
+  template <class... Ts> THRUST_CDNA4_HD auto operator()(Ts&&... ts) -> decltype(!f(static_cast<Ts&&>(ts)...)) { return !f(static_cast<Ts&&>(ts)...); }
+  template <class... Ts> THRUST_CDNA4_HD auto operator()(Ts&&... ts) const -> decltype(!f(static_cast<Ts&&>(ts)...)) { return !f(static_cast<Ts&&>(ts)...); }
+};
+}  // namespace detail
+template <class F> THRUST_CDNA4_HD detail::not_fun_t<F> not_fn(F f) { return detail::not_fun_t<F>{f}; }
 
 namespace system { namespace cdna4 { namespace detail {
 // C-ABI operator code of a functor type, or -1 when no kernel exists for it.

@@ -13,8 +13,6 @@
 #include <thrust/system/cdna4/detail/merge_engine.h>
 #endif
 
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/merge.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/merge.inl):

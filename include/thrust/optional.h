@@ -12,6 +12,11 @@
 
 namespace thrust {
 
+// the value type of an optional that only says whether it is engaged (thrust/optional.h:171)
+class monostate {};
+THRUST_CDNA4_HD constexpr bool operator==(monostate, monostate) noexcept { return true; }
+THRUST_CDNA4_HD constexpr bool operator!=(monostate, monostate) noexcept { return false; }
+THRUST_CDNA4_HD constexpr bool operator<(monostate, monostate) noexcept { return false; }
 struct nullopt_t {
   struct do_not_use {};
   THRUST_CDNA4_HD constexpr explicit nullopt_t(do_not_use, do_not_use) noexcept {}

@@ -8,11 +8,11 @@
 #include <vector>
 #include <thrust/detail/iterator_util.h>
 #include <thrust/execution_policy.h>
+#include <thrust/find.h>
+#include <thrust/logical.h>
 #include <thrust/pair.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/partition.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/partition.inl):
@@ -103,4 +103,17 @@ THRUST_CDNA4_PARTITION_NO_POLICY(stable_partition)
 THRUST_CDNA4_PARTITION_COPY_NO_POLICY(partition_copy)
 THRUST_CDNA4_PARTITION_COPY_NO_POLICY(stable_partition_copy)
 #undef THRUST_CDNA4_PARTITION_COPY_NO_POLICY
+
+// ---- partition_point / is_partitioned (thrust/partition.h:1311-1435), on find_if_not and none_of as
+//      the reference's generic layer has them (thrust/system/detail/generic/partition.inl:203-238)
+template <class Policy, class It, class Pred, detail::enable_if_policy<Policy> = 0>
+It partition_point(const Policy& exec, It first, It last, Pred pred) { return thrust::find_if_not(exec, first, last, pred); }
+template <class Policy, class It, class Pred, detail::enable_if_policy<Policy> = 0>
+bool is_partitioned(const Policy& exec, It first, It last, Pred pred) {
+  return thrust::none_of(exec, thrust::find_if_not(exec, first, last, pred), last, pred);
+}
+template <class It, class Pred, detail::enable_if_device<It> = 0> It partition_point(It f, It l, Pred p) { return partition_point(device, f, l, p); }
+template <class It, class Pred, detail::enable_if_host<It> = 0> It partition_point(It f, It l, Pred p) { return partition_point(host, f, l, p); }
+template <class It, class Pred, detail::enable_if_device<It> = 0> bool is_partitioned(It f, It l, Pred p) { return is_partitioned(device, f, l, p); }
+template <class It, class Pred, detail::enable_if_host<It> = 0> bool is_partitioned(It f, It l, Pred p) { return is_partitioned(host, f, l, p); }
 }  // namespace thrust

@@ -7,8 +7,6 @@
 #include <thrust/execution_policy.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/remove.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/remove.inl):

@@ -4,8 +4,6 @@
 #include <thrust/execution_policy.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/sequence.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/sequence.inl):

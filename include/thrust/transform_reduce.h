@@ -5,8 +5,6 @@
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
 #include <thrust/reduce.h>
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/transform_reduce.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/transform_reduce.inl):

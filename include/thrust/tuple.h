@@ -10,6 +10,9 @@
 
 namespace thrust {
 template <class... Ts> struct tuple;
+// the type the reference's ten-parameter tuple pads itself with (thrust/tuple.h:50); this tuple is
+// variadic and has no use for it beyond existing code that names it
+struct null_type {};
 
 namespace detail {
 template <std::size_t I, class T> struct tuple_leaf {

@@ -3,8 +3,6 @@
 #pragma once
 #include <memory>
 #include <thrust/copy.h>
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/uninitialized_copy.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/uninitialized_copy.inl):

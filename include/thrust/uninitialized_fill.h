@@ -4,8 +4,6 @@
 #pragma once
 #include <memory>
 #include <thrust/fill.h>
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/uninitialized_fill.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/uninitialized_fill.inl):

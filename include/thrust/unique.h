@@ -7,10 +7,10 @@
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
 #include <thrust/pair.h>
+#include <thrust/iterator/counting_iterator.h>
+#include <thrust/transform_reduce.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 
-namespace thrust {
-}  // namespace thrust
 #include <thrust/system/cdna4/detail/unique.h>
 namespace thrust {
 // The entry points dispatch on the policy's own type by an unqualified call (thrust/detail/unique.inl):
@@ -89,4 +89,34 @@ template <class K, class V, class KO, class VO, detail::enable_if_device<K> = 0>
 pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(device, f, l, v, ko, vo); }
 template <class K, class V, class KO, class VO, detail::enable_if_host<K> = 0>
 pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(host, f, l, v, ko, vo); }
+
+// ---- unique_count (thrust/unique.h:1022-1176): the number of runs of consecutive equivalent
+//      elements, i.e. how many elements unique would keep — one plus the positions whose element is
+//      not equivalent to the one before it, counted by a reduction over the positions
+namespace detail {
+template <class It, class Eq>
+struct starts_a_run {
+  It p; Eq eq;
+  template <class Index> THRUST_CDNA4_HD std::int64_t operator()(Index i) { return eq(p[i], p[i + 1]) ? 0 : 1; }
+};
+}  // namespace detail
+template <class Policy, class It, class Eq, detail::enable_if_policy<Policy> = 0>
+typename std::iterator_traits<It>::difference_type unique_count(const Policy& exec, It first, It last, Eq eq) {
+  typedef typename std::iterator_traits<It>::difference_type D;
+  const std::int64_t n = (std::int64_t)(last - first);
+  if (n <= 0) return D(0);
+  typedef detail::starts_a_run<typename detail::unwrap_iterator<It>::type, Eq> F;
+  return D(1 + thrust::transform_reduce(exec, counting_iterator<std::int64_t>(0), counting_iterator<std::int64_t>(n - 1),
+                                        F{detail::unwrap(first), eq}, std::int64_t(0), plus<std::int64_t>()));
+}
+template <class Policy, class It, detail::enable_if_policy<Policy> = 0>
+typename std::iterator_traits<It>::difference_type unique_count(const Policy& exec, It first, It last) {
+  return unique_count(exec, first, last, equal_to<typename detail::value_of<It>::type>());
+}
+template <class It, detail::enable_if_device<It> = 0> typename std::iterator_traits<It>::difference_type unique_count(It f, It l) { return unique_count(device, f, l); }
+template <class It, detail::enable_if_host<It> = 0> typename std::iterator_traits<It>::difference_type unique_count(It f, It l) { return unique_count(host, f, l); }
+template <class It, class Eq, detail::enable_if_device<It> = 0, typename std::enable_if<!detail::is_policy<It>::value, int>::type = 0>
+typename std::iterator_traits<It>::difference_type unique_count(It f, It l, Eq eq) { return unique_count(device, f, l, eq); }
+template <class It, class Eq, detail::enable_if_host<It> = 0, typename std::enable_if<!detail::is_policy<It>::value, int>::type = 0>
+typename std::iterator_traits<It>::difference_type unique_count(It f, It l, Eq eq) { return unique_count(host, f, l, eq); }
 }  // namespace thrust

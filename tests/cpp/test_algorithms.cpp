@@ -16,6 +16,10 @@
 #include <thrust/logical.h>
 #include <thrust/mismatch.h>
 #include <thrust/optional.h>
+#include <thrust/partition.h>
+#include <thrust/binary_search.h>
+#include <thrust/transform.h>
+#include <thrust/unique.h>
 #include <thrust/random.h>
 #include <thrust/replace.h>
 #include <thrust/reverse.h>
@@ -431,5 +435,146 @@ void TestOptionalOnDevice() {
   ASSERT_THROWS(b.value(), thrust::bad_optional_access);
 }
 DECLARE_UNITTEST(TestOptionalOnDevice);
+
+// ---- transform_if, partition_point, is_partitioned, equal_range, unique_count, and the function
+//      objects they are tested with — after testing/transform.cu:169-194, :339-369,
+//      partition_point.cu:14-48, is_partitioned.cu:14-60, binary_search.cu:217-249, unique.cu:143-147
+template <class Vector>
+void TestTransformIfSimple() {
+  typedef typename Vector::value_type T;
+  Vector input(3), input2(3), stencil(3), output(3), result(3);
+  input[0] = 1; input[1] = -2; input[2] = 3;
+  output[0] = 1; output[1] = 2; output[2] = 3;
+  stencil[0] = 1; stencil[1] = 0; stencil[2] = 1;
+  result[0] = -1; result[1] = 2; result[2] = -3;
+  typename Vector::iterator iter = thrust::transform_if(input.begin(), input.end(), stencil.begin(), output.begin(), thrust::negate<T>(), thrust::identity<T>());
+  ASSERT_EQUAL((std::size_t)(iter - output.begin()), input.size());
+  ASSERT_EQUAL(output, result);
+  // the predicate on the element itself
+  output[0] = 7; output[1] = 8; output[2] = 9;
+  iter = thrust::transform_if(input.begin(), input.end(), output.begin(), thrust::negate<T>(), thrust::not1(thrust::identity<T>()));
+  result[0] = 7; result[1] = 8; result[2] = 9;  // no element is zero: nothing is written
+  ASSERT_EQUAL(output, result);
+  // binary, through a negated stencil
+  input2[0] = -4; input2[1] = 5; input2[2] = 6;
+  stencil[0] = 0; stencil[1] = 1; stencil[2] = 0;
+  output[0] = 1; output[1] = 2; output[2] = 3;
+  result[0] = 5; result[1] = 2; result[2] = -3;
+  iter = thrust::transform_if(input.begin(), input.end(), input2.begin(), stencil.begin(), output.begin(), thrust::minus<T>(), thrust::not1(thrust::identity<T>()));
+  ASSERT_EQUAL((std::size_t)(iter - output.begin()), input.size());
+  ASSERT_EQUAL(output, result);
+}
+void TestTransformIfSimpleHost() { TestTransformIfSimple<thrust::host_vector<int>>(); }
+void TestTransformIfSimpleDevice() { TestTransformIfSimple<thrust::device_vector<int>>(); }
+DECLARE_UNITTEST(TestTransformIfSimpleHost);
+DECLARE_UNITTEST(TestTransformIfSimpleDevice);
+
+struct is_even_int { __host__ __device__ bool operator()(int x) const { return (x & 1) == 0; } };
+void TestTransformIfLarge() {
+  const int n = (1 << 18) + 5;
+  thrust::host_vector<int> h(n), expect(n);
+  for (int i = 0; i < n; i++) { h[i] = (i * 2654435761u) >> 20; expect[i] = (h[i] & 1) ? -7 : h[i] * 3; }
+  thrust::device_vector<int> d = h, out(n, -7);
+  thrust::transform_if(thrust::device, d.begin(), d.end(), out.begin(), [] __host__ __device__(int x) { return x * 3; }, is_even_int());
+  ASSERT_EQUAL(thrust::host_vector<int>(out), expect);
+}
+DECLARE_UNITTEST(TestTransformIfLarge);
+
+template <class Vector>
+void TestPartitionPointAndIsPartitioned() {
+  typedef typename Vector::value_type T;
+  Vector v(4);
+  v[0] = 1; v[1] = 1; v[2] = 1; v[3] = 0;
+  ASSERT_TRUE(thrust::partition_point(v.begin(), v.end(), thrust::identity<T>()) == v.begin() + 3);
+  ASSERT_TRUE(thrust::partition_point(v.begin(), v.begin() + 3, thrust::identity<T>()) == v.begin() + 3);
+  ASSERT_EQUAL(true, thrust::is_partitioned(v.begin(), v.begin(), thrust::identity<T>()));      // empty
+  ASSERT_EQUAL(true, thrust::is_partitioned(v.begin(), v.begin() + 1, thrust::identity<T>()));  // one true element
+  ASSERT_EQUAL(true, thrust::is_partitioned(v.begin(), v.begin() + 2, thrust::identity<T>()));
+  ASSERT_EQUAL(true, thrust::is_partitioned(v.begin(), v.end(), thrust::identity<T>()));
+  ASSERT_EQUAL(true, thrust::is_partitioned(v.begin() + 3, v.end(), thrust::identity<T>()));    // one false element
+  v[0] = 1; v[1] = 0; v[2] = 1; v[3] = 1;
+  ASSERT_EQUAL(false, thrust::is_partitioned(v.begin(), v.end(), thrust::identity<T>()));
+  const int n = (1 << 16) + 13;
+  thrust::host_vector<int> h(n);
+  for (int i = 0; i < n; i++) h[i] = (i * 2654435761u) >> 12;
+  Vector big(h.begin(), h.end());
+  ASSERT_EQUAL(false, thrust::is_partitioned(big.begin(), big.end(), is_even_int()));
+  typename Vector::iterator ref = thrust::stable_partition(big.begin(), big.end(), is_even_int());
+  ASSERT_EQUAL((long)(ref - big.begin()), (long)(thrust::partition_point(big.begin(), big.end(), is_even_int()) - big.begin()));
+  ASSERT_EQUAL(true, thrust::is_partitioned(big.begin(), big.end(), is_even_int()));
+}
+void TestPartitionPointHost() { TestPartitionPointAndIsPartitioned<thrust::host_vector<int>>(); }
+void TestPartitionPointDevice() { TestPartitionPointAndIsPartitioned<thrust::device_vector<int>>(); }
+DECLARE_UNITTEST(TestPartitionPointHost);
+DECLARE_UNITTEST(TestPartitionPointDevice);
+
+template <class Vector>
+void TestScalarEqualRangeSimple() {
+  Vector vec(5);
+  vec[0] = 0; vec[1] = 2; vec[2] = 5; vec[3] = 7; vec[4] = 8;
+  const int first[10] = {0, 1, 1, 2, 2, 2, 3, 3, 4, 5}, second[10] = {1, 1, 2, 2, 2, 3, 3, 4, 5, 5};
+  for (int x = 0; x < 10; x++) {
+    ASSERT_EQUAL((int)(thrust::equal_range(vec.begin(), vec.end(), x).first - vec.begin()), first[x]);
+    ASSERT_EQUAL((int)(thrust::equal_range(vec.begin(), vec.end(), x).second - vec.begin()), second[x]);
+  }
+  // descending order under greater
+  Vector desc(6);
+  desc[0] = 9; desc[1] = 7; desc[2] = 7; desc[3] = 7; desc[4] = 3; desc[5] = 1;
+  auto r = thrust::equal_range(desc.begin(), desc.end(), 7, thrust::greater<int>());
+  ASSERT_EQUAL((int)(r.first - desc.begin()), 1);
+  ASSERT_EQUAL((int)(r.second - desc.begin()), 4);
+}
+void TestScalarEqualRangeHost() { TestScalarEqualRangeSimple<thrust::host_vector<int>>(); }
+void TestScalarEqualRangeDevice() { TestScalarEqualRangeSimple<thrust::device_vector<int>>(); }
+DECLARE_UNITTEST(TestScalarEqualRangeHost);
+DECLARE_UNITTEST(TestScalarEqualRangeDevice);
+
+struct is_equal_div_10 { __host__ __device__ bool operator()(int x, int y) const { return x / 10 == y / 10; } };
+template <class Vector>
+void TestUniqueCount() {
+  Vector data(10);
+  const int raw[10] = {11, 11, 12, 20, 29, 21, 21, 31, 31, 37};
+  for (int i = 0; i < 10; i++) data[i] = raw[i];
+  ASSERT_EQUAL((int)thrust::unique_count(data.begin(), data.end()), 7);
+  ASSERT_EQUAL((int)thrust::unique_count(data.begin(), data.end(), is_equal_div_10()), 3);
+  ASSERT_EQUAL((int)thrust::unique_count(data.begin(), data.begin()), 0);
+  ASSERT_EQUAL((int)thrust::unique_count(data.begin(), data.begin() + 1), 1);
+  const int n = (1 << 17) + 3;
+  thrust::host_vector<int> h(n);
+  for (int i = 0; i < n; i++) h[i] = ((i * 2654435761u) >> 28) / 3;
+  Vector big(h.begin(), h.end());
+  const long expect = (long)(std::unique(h.begin(), h.end()) - h.begin());
+  ASSERT_EQUAL((long)thrust::unique_count(big.begin(), big.end()), expect);
+  ASSERT_EQUAL((long)(thrust::unique(big.begin(), big.end()) - big.begin()), expect);
+}
+void TestUniqueCountHost() { TestUniqueCount<thrust::host_vector<int>>(); }
+void TestUniqueCountDevice() { TestUniqueCount<thrust::device_vector<int>>(); }
+DECLARE_UNITTEST(TestUniqueCountHost);
+DECLARE_UNITTEST(TestUniqueCountDevice);
+
+void TestFunctionObjects() {
+  // adaptable typedefs, transparent forms, negators, projections (thrust/functional.h:129-1529)
+  static_assert(std::is_same<thrust::plus<int>::result_type, int>::value && std::is_same<thrust::less<float>::result_type, bool>::value, "");
+  static_assert(std::is_same<thrust::negate<int>::argument_type, int>::value && std::is_same<thrust::minus<long>::first_argument_type, long>::value, "");
+  ASSERT_EQUAL(thrust::square<int>()(7), 49);
+  ASSERT_EQUAL(thrust::square<>()(1.5), 2.25);
+  ASSERT_EQUAL(thrust::minus<>()(7, 2.5), 4.5);
+  ASSERT_EQUAL(thrust::bit_xor<>()(6, 3), 5);
+  ASSERT_EQUAL(thrust::logical_not<>()(0), true);
+  ASSERT_EQUAL((thrust::project1st<int, double>()(3, 4.5)), 3);
+  ASSERT_EQUAL((thrust::project2nd<int, double>()(3, 4.5)), 4.5);
+  ASSERT_EQUAL(thrust::project1st<>()(3, 4.5), 3);
+  ASSERT_EQUAL(thrust::not1(thrust::identity<int>())(0), true);
+  ASSERT_EQUAL(thrust::not2(thrust::less<int>())(1, 2), false);
+  ASSERT_EQUAL(thrust::not_fn(is_even_int())(3), true);
+  thrust::device_vector<int> v(100), sq(100);
+  thrust::sequence(v.begin(), v.end());
+  thrust::transform(v.begin(), v.end(), sq.begin(), thrust::square<int>());
+  ASSERT_EQUAL((int)sq[9], 81);
+  ASSERT_EQUAL((int)thrust::count_if(v.begin(), v.end(), thrust::not_fn(is_even_int())), 50);
+  thrust::transform(v.begin(), v.end(), sq.begin(), sq.begin(), thrust::project1st<int, int>());
+  ASSERT_EQUAL((int)sq[9], 9);
+}
+DECLARE_UNITTEST(TestFunctionObjects);
 
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }

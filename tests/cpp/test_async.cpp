@@ -162,6 +162,18 @@ void TestAsyncDependencyChain() {
   thrust::device_event none;
   ASSERT_TRUE(!none.valid_stream() && !none.ready());
   ASSERT_THROWS(none.wait(), std::logic_error);
+  // the error carries the reference's code (testing/event.cu:39-50, testing/async_reduce.cu:797-821)
+  try {
+    none.wait();
+    ASSERT_TRUE(false);
+  } catch (const thrust::event_error& e) {
+    ASSERT_TRUE(e == thrust::event_error(thrust::event_errc::no_state));
+    ASSERT_TRUE(e.code().category() == thrust::event_category());
+  }
+  thrust::device_future<int> empty;
+  ASSERT_THROWS(empty.get(), thrust::event_error);
+  static_assert(std::is_same<thrust::device_unique_eager_event, thrust::device_event>::value, "");
+  static_assert(std::is_same<thrust::unique_eager_future<int, thrust::device_system_tag>, thrust::device_future<int>>::value, "");
 }
 DECLARE_UNITTEST(TestAsyncDependencyChain);
 
