@@ -12,6 +12,8 @@
 #include <thrust/device_allocator.h>
 #include <thrust/device_ptr.h>
 #include <thrust/host_vector.h>
+#include <thrust/iterator/reverse_iterator.h>
+#include <stdexcept>
 
 namespace thrust {
 
@@ -28,6 +30,10 @@ class device_vector {
   typedef device_ptr<T> pointer;
   typedef device_reference<T> reference;
   typedef device_reference<const T> const_reference;
+  typedef std::ptrdiff_t difference_type;
+  typedef device_ptr<const T> const_pointer;
+  typedef thrust::reverse_iterator<iterator> reverse_iterator;
+  typedef thrust::reverse_iterator<const_iterator> const_reverse_iterator;
 
   device_vector() : p_(nullptr), n_(0), cap_(0), alloc_() {}
   explicit device_vector(const Alloc& alloc) : p_(nullptr), n_(0), cap_(0), alloc_(alloc) {}
@@ -53,6 +59,12 @@ class device_vector {
   const_iterator end() const { return const_iterator(p_ + n_); }
   const_iterator cbegin() const { return begin(); }
   const_iterator cend() const { return end(); }
+  reverse_iterator rbegin() { return reverse_iterator(end()); }
+  reverse_iterator rend() { return reverse_iterator(begin()); }
+  const_reverse_iterator rbegin() const { return const_reverse_iterator(end()); }
+  const_reverse_iterator rend() const { return const_reverse_iterator(begin()); }
+  const_reverse_iterator crbegin() const { return rbegin(); }
+  const_reverse_iterator crend() const { return rend(); }
   pointer data() { return pointer(p_); }
   device_ptr<const T> data() const { return device_ptr<const T>(p_); }
   size_type size() const { return n_; }
@@ -60,6 +72,10 @@ class device_vector {
   bool empty() const { return n_ == 0; }
   reference operator[](size_type i) { return reference(p_ + i); }
   const_reference operator[](size_type i) const { return const_reference(p_ + i); }
+  // checked access (thrust/detail/vector_base.h: at() throws std::out_of_range)
+  reference at(size_type i) { if (i >= n_) throw std::out_of_range("thrust::device_vector::at"); return (*this)[i]; }
+  const_reference at(size_type i) const { if (i >= n_) throw std::out_of_range("thrust::device_vector::at"); return (*this)[i]; }
+  size_type max_size() const { return static_cast<size_type>(-1) / sizeof(T); }
   reference front() { return (*this)[0]; }
   reference back() { return (*this)[n_ - 1]; }
   const_reference front() const { return (*this)[0]; }

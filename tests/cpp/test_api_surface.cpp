@@ -182,4 +182,23 @@ void TestSearchOverloads() {
 }
 DECLARE_UNITTEST(TestSearchOverloads);
 
+// the rest of the vector's container interface (thrust/detail/vector_base.h:240-470)
+void TestDeviceVectorReverseIterationAndCheckedAccess() {
+  thrust::device_vector<int> v(5);
+  for (int i = 0; i < 5; i++) v[i] = i * i;
+  ASSERT_EQUAL((int)v.at(3), 9);
+  ASSERT_THROWS(v.at(5), std::out_of_range);
+  ASSERT_EQUAL((int)*v.rbegin(), 16);
+  ASSERT_EQUAL((int)(v.rend() - v.rbegin()), 5);
+  thrust::host_vector<int> back(v.rbegin(), v.rend());
+  ASSERT_EQUAL(back[0], 16);
+  ASSERT_EQUAL(back[4], 0);
+  const thrust::device_vector<int>& c = v;
+  ASSERT_EQUAL((int)*c.crbegin(), 16);
+  ASSERT_EQUAL((int)c.at(1), 1);
+  ASSERT_TRUE(v.max_size() >= v.size());
+  static_assert(std::is_same<thrust::device_vector<int>::difference_type, std::ptrdiff_t>::value, "");
+}
+DECLARE_UNITTEST(TestDeviceVectorReverseIterationAndCheckedAccess);
+
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
