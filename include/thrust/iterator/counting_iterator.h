@@ -16,6 +16,7 @@ class counting_iterator : public detail::fancy_base<counting_iterator<T, System,
   THRUST_CDNA4_HD T at(std::ptrdiff_t n) const { return (T)(v_ + (T)n); }
   THRUST_CDNA4_HD void advance(std::ptrdiff_t n) { v_ = (T)(v_ + (T)n); }
   THRUST_CDNA4_HD std::ptrdiff_t distance_to(const counting_iterator& o) const { return (std::ptrdiff_t)(o.v_ - v_); }
+  THRUST_CDNA4_HD const T& base() const { return v_; }  // the counter (thrust/iterator/iterator_adaptor.h:178)
  private:
   T v_;
 };

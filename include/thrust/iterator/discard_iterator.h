@@ -2,6 +2,7 @@
 // assigned to it.
 #pragma once
 #include <thrust/detail/iterator_util.h>
+#include <thrust/iterator/counting_iterator.h>
 #include <thrust/iterator/detail/fancy_base.h>
 
 namespace thrust {
@@ -21,6 +22,7 @@ class discard_iterator : public detail::fancy_base<discard_iterator<System>, det
   THRUST_CDNA4_HD detail::discard_proxy at(std::ptrdiff_t) const { return detail::discard_proxy(); }
   THRUST_CDNA4_HD void advance(std::ptrdiff_t n) { pos_ += n; }
   THRUST_CDNA4_HD std::ptrdiff_t distance_to(const discard_iterator& o) const { return o.pos_ - pos_; }
+  THRUST_CDNA4_HD counting_iterator<std::ptrdiff_t> base() const { return counting_iterator<std::ptrdiff_t>(pos_); }  // its position
  private:
   std::ptrdiff_t pos_;
 };

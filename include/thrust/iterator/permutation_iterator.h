@@ -17,6 +17,7 @@ class permutation_iterator : public detail::fancy_base<permutation_iterator<Elem
   THRUST_CDNA4_HD std::ptrdiff_t distance_to(const permutation_iterator& o) const { return o.i_ - i_; }
   THRUST_CDNA4_HD ElementIt elements() const { return e_; }
   THRUST_CDNA4_HD IndexIt indices() const { return i_; }
+  THRUST_CDNA4_HD IndexIt base() const { return i_; }  // the adapted iterator is the index iterator (thrust/iterator/permutation_iterator.h:130)
  private:
   ElementIt e_;
   IndexIt i_;

@@ -460,4 +460,25 @@ void TestUserIteratorsFromFacadeAndAdaptor() {
 }
 DECLARE_UNITTEST(TestUserIteratorsFromFacadeAndAdaptor);
 
+// the accessors of the fancy iterators (base(), value(), functor(), get_iterator_tuple())
+void TestIteratorAccessors() {
+  thrust::counting_iterator<int> c(7);
+  ASSERT_EQUAL((c + 3).base(), 10);
+  thrust::constant_iterator<float> k(2.5f);
+  ASSERT_EQUAL((k + 4).value(), 2.5f);
+  ASSERT_EQUAL((int)*(k + 4).base(), 4);
+  thrust::device_vector<int> data(4), idx(4);
+  auto perm = thrust::make_permutation_iterator(data.begin(), idx.begin());
+  ASSERT_TRUE((perm + 2).base() == idx.begin() + 2);
+  auto d = thrust::make_discard_iterator(3);
+  ASSERT_EQUAL((int)*(d + 2).base(), 5);
+  auto r = thrust::make_reverse_iterator(data.end());
+  ASSERT_TRUE((r + 1).base() == data.end() - 1);
+  auto t = thrust::make_transform_iterator(data.begin(), thrust::negate<int>());
+  ASSERT_TRUE((t + 1).base() == data.begin() + 1);
+  auto z = thrust::make_zip_iterator(thrust::make_tuple(data.begin(), idx.begin()));
+  ASSERT_TRUE(thrust::get<1>((z + 3).get_iterator_tuple()) == idx.begin() + 3);
+}
+DECLARE_UNITTEST(TestIteratorAccessors);
+
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
