@@ -226,6 +226,18 @@ def test_sort_beyond_2p30_items():
     assert bool((k[1:] >= k[:-1]).all())
     assert bool(((k[1:] > k[:-1]) | (v[1:] > v[:-1])).all())  # equal keys keep their input order
     assert bool((src[v.long()] == k).all())
+    del src, k, v
+    torch.cuda.empty_cache()
+    # one-byte keys at the largest size the entry point takes (2^32 - 2): run starts near 2^32
+    n = (1 << 32) - 2
+    k = torch.randint(0, 4, (n,), dtype=torch.uint8, device="cuda", generator=g) * 85
+    step = 1 << 30
+    counts = sum(torch.bincount(k[a:a + step].to(torch.int32), minlength=256) for a in range(0, n, step))
+    thrust_amd.sort(k, descending=True)
+    for a in range(0, n, step):
+        c = k[a:a + step]
+        assert bool((c[1:] <= c[:-1]).all()) and (a == 0 or bool(k[a] <= k[a - 1]))
+    assert torch.equal(counts, sum(torch.bincount(k[a:a + step].to(torch.int32), minlength=256) for a in range(0, n, step)))
 
 
 # Places where every key has the same digit are skipped on the device (the identity for a stable
