@@ -285,6 +285,24 @@ int thrust_cdna4_lookback_timeouts(unsigned long long* count);
  */
 int thrust_cdna4_selftest_lds_atomic_order(long long* mismatches, void* stream);
 
+/*
+ * Hardware self-test of what the sort's tile assignment relies on for speed.  Consecutive tiles of a
+ * pass write the ends of their per-digit runs into the same cache lines; when one XCD processes
+ * groups of consecutive tiles its L2 puts those lines together, which is worth 10 % of a pair sort.
+ * That form is only used on a device where workgroup i runs on XCD i mod 8 and every XCD starts its
+ * next workgroup independently of the others — otherwise a tile could wait for one that cannot start.
+ * This call runs the probe that the library runs by itself before its first large sort on a device
+ * (about 0.2 ms, workgroups that wait on nothing but the clock) and stores 1 in *grouped when the
+ * device behaves that way, else 0 (the sort then hands tiles out from one counter in index order, the
+ * form that depends on nothing).  A sort call under stream capture never runs the probe.
+ * The reference has no counterpart.
+ */
+int thrust_cdna4_selftest_xcd_dispatch(int* grouped, void* stream);
+
+/* Test knob: non-zero makes every later sort hand its tiles out from one counter (the form used on
+ * devices that fail the probe above); returns the previous setting. */
+int thrust_cdna4_set_test_sort_plain_tickets(int on);
+
 #ifdef __cplusplus
 }
 #endif

@@ -161,6 +161,42 @@ def test_lds_atomic_order_selftest():
     assert bad.value == 0
 
 
+def test_xcd_dispatch_selftest_and_both_tile_assignments():
+    """Large sorts hand consecutive tiles to one XCD in groups (its L2 then merges the run ends that
+    two tiles write into one cache line) on a device that passes the library's dispatch probe; MI355X
+    does.  Both forms of the tile assignment — grouped, and one counter in index order — must give the
+    oracle's result, for keys and pairs, at sizes with partial last groups."""
+    import ctypes
+
+    from thrust_amd import capi
+    L = capi.lib()
+    grouped = ctypes.c_int(-1)
+    rc = L.thrust_cdna4_selftest_xcd_dispatch(ctypes.byref(grouped), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    assert grouped.value == 1
+    before = ctypes.c_ulonglong(0)
+    L.thrust_cdna4_lookback_timeouts(ctypes.byref(before))
+    for plain in (0, 1):
+        prev = L.thrust_cdna4_set_test_sort_plain_tickets(plain)
+        try:
+            for n in [(1 << 23) + 1, 256 * 32768, 257 * 32768 + 5, (1 << 24) - 3]:
+                k = random_ints(n, n, np.uint32)
+                d = dev(k)
+                thrust_amd.sort(d)
+                assert same_bits(host(d), oracle.sort_keys(k)), (plain, n)
+                k64 = random_ints(n + 1, n // 2, np.uint64) & np.uint64(0xFFFFFF)
+                v = np.arange(n // 2, dtype=np.uint32)
+                dk, dv = dev(k64), dev(v)
+                thrust_amd.sort_by_key(dk, dv, descending=True)
+                ek, ev = oracle.sort_pairs(k64, v, descending=True)
+                assert same_bits(host(dk), ek) and same_bits(host(dv), ev), (plain, n)
+        finally:
+            L.thrust_cdna4_set_test_sort_plain_tickets(prev)
+    after = ctypes.c_ulonglong(0)
+    L.thrust_cdna4_lookback_timeouts(ctypes.byref(after))
+    assert after.value == before.value
+
+
 def test_sort_skewed_digits_stability():
     """Keys whose digits are heavily skewed (most lanes of a wavefront share a digit) take the
     careful ranking loop; pairs must stay stable."""

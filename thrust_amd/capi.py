@@ -28,6 +28,7 @@ SYMBOLS = [
     "thrust_cdna4_event_create", "thrust_cdna4_event_destroy", "thrust_cdna4_event_record", "thrust_cdna4_event_query",
     "thrust_cdna4_stream_wait_event", "thrust_cdna4_malloc_direct", "thrust_cdna4_free_direct",
     "thrust_cdna4_malloc_universal", "thrust_cdna4_free_universal", "thrust_cdna4_get_device",
+    "thrust_cdna4_selftest_xcd_dispatch", "thrust_cdna4_set_test_sort_plain_tickets",
 ]
 
 
@@ -91,6 +92,8 @@ def lib():
     L.thrust_cdna4_lookback_timeouts.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
     L.thrust_cdna4_profile_enable.argtypes = [i32]
     L.thrust_cdna4_selftest_lds_atomic_order.argtypes = [ctypes.POINTER(ctypes.c_longlong), vp]
+    L.thrust_cdna4_selftest_xcd_dispatch.argtypes = [ctypes.POINTER(i32), vp]
+    L.thrust_cdna4_set_test_sort_plain_tickets.argtypes = [i32]
     L.thrust_cdna4_profile_get.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p),
                                            ctypes.POINTER(ctypes.c_float)]
     _lib = L

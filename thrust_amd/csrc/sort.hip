@@ -22,6 +22,8 @@
 #include <atomic>
 #include <mutex>
 
+#include <vector>
+
 #include "common.h"
 
 namespace tcd {
@@ -40,6 +42,12 @@ struct DescWord {
   __device__ static uint32_t count(D w) { return (uint32_t)(w & kCountMask); }
 };
 constexpr int kLookW = 8;  // look-back descriptors loaded per round trip
+// Consecutive tiles write the ends of their per-digit runs into the same cache lines.  Groups of
+// this many consecutive tiles are processed by one XCD, so that seven of eight such lines are put
+// together in that XCD's L2 instead of being written to memory in two pieces (see take_tile).
+constexpr int kXcdGroup = 8;
+constexpr int kXcds = 8;             // the scheme is used on devices that spread workgroup i to XCD i mod 8
+constexpr int kXcdCounterStride = 32;  // words: each XCD's counter in a cache line of its own
 
 template <int BYTES>
 struct uint_of;
@@ -227,11 +235,44 @@ __device__ inline void lds_store(uint32_t* p, uint32_t v) {
 constexpr uint32_t kLookbackSpinLimit = 1u << 22;
 __device__ unsigned int g_lookback_timeouts;
 
+// The tile a workgroup processes, with the pass's flags in the top bits.  Plain form (xcd == nullptr):
+// the next ticket of the pass's counter — tiles start in index order, so every tile that a look-back
+// waits for is running.  Grouped form: workgroup i runs on XCD i mod 8 (checked on the device before
+// this form is used); the workgroups of an XCD take the tiles of the XCD's current group of kXcdGroup
+// consecutive tiles in order, and the one that takes the first tile of a group claims the group from
+// the pass's counter and leaves its number for the others.  An XCD's tiles are still started in index
+// order and groups are claimed in index order, so the lowest tile that has not started belongs to an
+// XCD all of whose running tiles are lower — they need nothing from it and finish —, and that XCD
+// starts its next workgroup whatever the other XCDs are doing (also checked): every wait ends.
+__device__ inline uint32_t take_tile(uint32_t* ticket, uint32_t* xcd, int xcd_slots) {
+  if (xcd == nullptr) return atomicAdd(ticket, 1u);
+  const uint32_t x = blockIdx.x % kXcds;
+  const uint32_t idx = atomicAdd(&xcd[x * kXcdCounterStride], 1u);
+  const uint32_t slot = idx / kXcdGroup, within = idx % kXcdGroup;
+  uint32_t* cell = &xcd[kXcds * kXcdCounterStride + x * xcd_slots + slot];
+  uint32_t group_word;
+  if (within == 0) {
+    group_word = atomicAdd(ticket, 1u);
+    st_agent(cell, group_word + 1u);  // never 0: the cell starts at 0
+  } else {
+    // the workgroup that took the group's first tile started before this one and writes the cell
+    // right after its own atomic; the poll limit only makes sure that the loop ends
+    uint32_t v = ld_agent(cell), spins = 0;
+    while (v == 0u && ++spins < kLookbackSpinLimit) {
+      __builtin_amdgcn_s_sleep(1);
+      v = ld_agent(cell);
+    }
+    if (v == 0u) atomicAdd(&g_lookback_timeouts, 1u);
+    group_word = v - 1u;
+  }
+  return (group_word & ~kTicketMask) | ((group_word & kTicketMask) * kXcdGroup + within);
+}
+
 template <class U, int VB, bool FLOAT, int BLOCK, int IPT, int WPE, class D>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) void onesweep_kernel(U* kmain, U* kalt, void* vmain, void* valt,
                                                          int64_t n, U xor_mask, int shift,
                                                          const uint32_t* __restrict__ gbase,
-                                                         D* desc, uint32_t* ticket) {
+                                                         D* desc, uint32_t* ticket, uint32_t* xcd, int xcd_slots) {
   static_assert(BLOCK % 256 == 0, "one thread per digit needs at least 256 threads");
   using V = typename value_of<VB>::type;
   constexpr int NWAVES = BLOCK / kWave;
@@ -243,7 +284,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
 
-  if (tid == 0) sm.tile = atomicAdd(ticket, 1u);
+  if (tid == 0) sm.tile = take_tile(ticket, xcd, xcd_slots);
   if (tid < kRadix / 2) {
 #pragma unroll
     for (int w = 0; w < NWAVES; w++) reinterpret_cast<uint32_t*>(sm.wave_cnt[w])[tid] = 0;
@@ -257,6 +298,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
   const V* __restrict__ vin = static_cast<const V*>(from_alt ? valt : vmain);
   V* __restrict__ vout = static_cast<V*>(from_alt ? vmain : valt);
   const int64_t tile = ticket_word & kTicketMask;
+  if (tile * TILE >= n) return;  // a workgroup of the padding that makes every XCD's share whole groups
   const int64_t base = tile * TILE;
   const int valid = (int)((n - base) < (int64_t)TILE ? (n - base) : (int64_t)TILE);
   const bool full = valid == TILE;
@@ -627,6 +669,94 @@ static hipError_t ensure_lds_order(hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------
+// Which form of take_tile a device gets.  The grouped form needs two things of the device:
+// workgroup i runs on XCD i mod 8, and an XCD starts its next workgroup as soon as it has room,
+// whether or not the other XCDs have.  Both are observed once per device by a probe whose
+// workgroups wait on nothing but the clock: one workgroup per CU (they ask for 125 KiB of LDS),
+// three rounds of them per XCD; those of class 0 (index 0 mod 8) stay for 60 us each, the others
+// leave at once.  Every workgroup notes its XCD and when it started.  On a device of the expected
+// kind the classes 1..7 are through their three rounds while class 0 is still in its first.
+// Anything else — another XCD count, another partition mode, a dispatcher that serves the XCDs in
+// turn — selects the plain tickets.
+constexpr int kProbeMax = 4096;
+__device__ unsigned long long g_probe_start[kProbeMax];
+__device__ unsigned int g_probe_xcd[kProbeMax];
+__global__ __launch_bounds__(1024) void xcd_dispatch_probe_kernel(unsigned long long* start, unsigned int* xcd_of, int slow_ticks) {
+  __shared__ uint32_t occupy[125 * 256];  // 125 KiB: one workgroup per CU
+  const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();  // 100 MHz
+  if (threadIdx.x == 0) {
+    start[blockIdx.x] = t0;
+    xcd_of[blockIdx.x] = __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 15u;  // XCC_ID, bits 3:0
+    occupy[blockIdx.x % (125 * 256)] = 1u;
+  }
+  if (blockIdx.x % kXcds == 0)
+    while (__builtin_amdgcn_s_memrealtime() - t0 < (unsigned long long)slow_ticks) __builtin_amdgcn_s_sleep(32);
+  if (threadIdx.x == 1 && occupy[1] == 0xdeadbeefu) start[0] = 0;  // keeps the array
+}
+static std::atomic<int> g_xcd_verdict[kMaxDevices];  // 0 not probed, 1 grouped tiles, 2 plain tickets
+static std::atomic<int> g_force_plain_tickets{0};    // test knob
+static std::mutex g_xcd_mu;
+
+static hipError_t run_xcd_dispatch_probe(hipStream_t s, bool* grouped_ok) {
+  *grouped_ok = false;
+  const int per_xcd = device_cu_count() / kXcds;
+  const int wgs = kXcds * 3 * per_xcd;
+  if (per_xcd < 1 || device_cu_count() % kXcds != 0 || wgs > kProbeMax) return hipSuccess;
+  void *d_start = nullptr, *d_xcd = nullptr;
+  hipError_t e = hipGetSymbolAddress(&d_start, HIP_SYMBOL(g_probe_start));
+  if (e != hipSuccess) return e;
+  e = hipGetSymbolAddress(&d_xcd, HIP_SYMBOL(g_probe_xcd));
+  if (e != hipSuccess) return e;
+  TCD_LAUNCH("xcd_dispatch_probe_kernel", xcd_dispatch_probe_kernel, dim3(wgs), dim3(1024), s,
+             static_cast<unsigned long long*>(d_start), static_cast<unsigned int*>(d_xcd), 6000);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  std::vector<unsigned long long> start(wgs);
+  std::vector<unsigned int> xcd_of(wgs);
+  e = hipMemcpyAsync(start.data(), d_start, sizeof(unsigned long long) * wgs, hipMemcpyDeviceToHost, s);
+  if (e != hipSuccess) return e;
+  e = hipMemcpyAsync(xcd_of.data(), d_xcd, sizeof(unsigned int) * wgs, hipMemcpyDeviceToHost, s);
+  if (e != hipSuccess) return e;
+  e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return e;
+  for (int i = 0; i < wgs; i++)
+    if (xcd_of[i] != (unsigned)(i % kXcds)) return hipSuccess;  // another mapping of workgroups to XCDs
+  // class 0's first workgroup of the second round starts when one of its first round has left
+  const unsigned long long second_round_of_slow = start[(size_t)per_xcd * kXcds];
+  for (int c = 1; c < kXcds; c++)
+    if (start[(size_t)(3 * per_xcd - 1) * kXcds + c] >= second_round_of_slow) return hipSuccess;  // the XCDs are not served independently
+  *grouped_ok = true;
+  return hipSuccess;
+}
+
+// true: the grouped form may be used by this call
+static hipError_t xcd_groups_usable(hipStream_t s, bool* usable) {
+  *usable = false;
+  if (g_force_plain_tickets.load(std::memory_order_relaxed)) return hipSuccess;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipSuccess;
+  int v = g_xcd_verdict[dev].load(std::memory_order_acquire);
+  if (v == 0) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cs) != hipSuccess) (void)hipGetLastError();
+    else if (cs != hipStreamCaptureStatusNone) return hipSuccess;  // the probe blocks: a later call runs it
+    std::lock_guard<std::mutex> g(g_xcd_mu);
+    v = g_xcd_verdict[dev].load(std::memory_order_acquire);
+    if (v == 0) {
+      bool ok = false;
+      e = run_xcd_dispatch_probe(s, &ok);
+      if (e != hipSuccess) return e;
+      v = ok ? 1 : 2;
+      g_xcd_verdict[dev].store(v, std::memory_order_release);
+    }
+  }
+  *usable = v == 1;
+  return hipSuccess;
+}
+
+// ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
 template <class U, int VB, bool SMALL>
@@ -652,7 +782,8 @@ constexpr int64_t kSortMaxN = (int64_t(1) << 32) - 1;
 constexpr int64_t small_sort_limit(int value_bytes) { return int64_t(1) << (21 + (value_bytes ? 1 : 0)); }
 
 struct SortPlan {
-  size_t keys_alt, vals_alt, hist, tickets, desc, total;
+  size_t keys_alt, vals_alt, hist, tickets, xcd, desc, total;
+  int xcd_slots;  // groups an XCD may take in one pass
   size_t zero_begin, zero_bytes;
   int64_t ntiles;
 };
@@ -690,6 +821,7 @@ __global__ __launch_bounds__(kFillThreads) void counting_fill_kernel(uint8_t* ou
   }
 }
 
+static constexpr size_t xcd_words_per_pass(int slots) { return (size_t)kXcds * kXcdCounterStride + (size_t)kXcds * (size_t)slots; }
 template <class U, int VB, class C, class D>
 static SortPlan make_plan(int64_t n) {
   constexpr int P = sizeof(U);
@@ -702,6 +834,9 @@ static SortPlan make_plan(int64_t n) {
   p.zero_begin = off;
   p.hist = off; off += align_up((size_t)P * kRadix * 4, 256);
   p.tickets = off; off += 256;
+  // per pass: a counter per XCD (a cache line each) and the numbers of the groups each XCD took
+  p.xcd_slots = (int)ceil_div(p.ntiles, (int64_t)kXcds * kXcdGroup);
+  p.xcd = off; off += kCounting ? 0 : align_up((size_t)P * xcd_words_per_pass(p.xcd_slots) * 4, 256);
   p.desc = off; off += kCounting ? 0 : align_up((size_t)P * p.ntiles * kRadix * sizeof(D), 256);
   p.zero_bytes = off - p.zero_begin;
   p.total = off;
@@ -755,10 +890,19 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
                reinterpret_cast<uint8_t*>(kbuf[0]), n, (uint8_t)xor_mask, ghist);
     return hipGetLastError();
   }
+  // tiles in groups per XCD where the device was seen to allow it and every XCD has several groups to
+  // take; the grid is then padded so that each XCD's share of the workgroups is whole groups
+  bool grouped = false;
+  if (plan.ntiles >= (int64_t)kXcds * kXcdGroup * 4) {
+    e = xcd_groups_usable(stream, &grouped);
+    if (e != hipSuccess) return e;
+  }
+  const int64_t grid = grouped ? (int64_t)kXcds * kXcdGroup * plan.xcd_slots : plan.ntiles;
   for (int p = 0; p < P; p++) {
-    TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT, C::WPE, D>), dim3((unsigned)plan.ntiles),
+    uint32_t* xcd = grouped ? reinterpret_cast<uint32_t*>(t + plan.xcd) + (size_t)p * xcd_words_per_pass(plan.xcd_slots) : nullptr;
+    TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT, C::WPE, D>), dim3((unsigned)grid),
                dim3(C::BLOCK), stream, kbuf[0], kbuf[1], static_cast<void*>(vbuf[0]), static_cast<void*>(vbuf[1]), n, xor_mask, 8 * p,
-               ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix, tickets + p);
+               ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix, tickets + p, xcd, plan.xcd_slots);
   }
   e = hipGetLastError();
   if (e != hipSuccess) return e;
@@ -832,6 +976,18 @@ extern "C" int thrust_cdna4_sort_pairs(void* temp, size_t* temp_bytes, int key_d
     case 8: return (int)tcd::sort_dispatch<8>(temp, temp_bytes, key_dtype, keys, values, n, descending, s);
   }
   return hipErrorInvalidValue;
+}
+
+extern "C" int thrust_cdna4_set_test_sort_plain_tickets(int on) {
+  return tcd::g_force_plain_tickets.exchange(on ? 1 : 0);
+}
+
+extern "C" int thrust_cdna4_selftest_xcd_dispatch(int* grouped, void* stream) {
+  if (!grouped) return hipErrorInvalidValue;
+  bool ok = false;
+  const hipError_t e = tcd::run_xcd_dispatch_probe(static_cast<hipStream_t>(stream), &ok);
+  *grouped = ok ? 1 : 0;
+  return (int)e;
 }
 
 extern "C" int thrust_cdna4_lookback_timeouts(unsigned long long* count) {
