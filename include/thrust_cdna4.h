@@ -293,8 +293,9 @@ int thrust_cdna4_selftest_lds_atomic_order(long long* mismatches, void* stream);
  * next workgroup independently of the others — otherwise a tile could wait for one that cannot start.
  * This call runs the probe that the library runs by itself before its first large sort on a device
  * (about 0.2 ms, workgroups that wait on nothing but the clock) and stores 1 in *grouped when the
- * device behaves that way, else 0 (the sort then hands tiles out from one counter in index order, the
- * form that depends on nothing).  A sort call under stream capture never runs the probe.
+ * device behaves that way, else 0 (its workgroups are not spread over 8 XCDs by index), -1 (the XCDs
+ * were not seen to be served independently) or -2 (a CU count the probe does not fit); the sort then
+ * hands tiles out from one counter in index order, the form that depends on nothing.  A sort call under stream capture never runs the probe.
  * The reference has no counterpart.
  */
 int thrust_cdna4_selftest_xcd_dispatch(int* grouped, void* stream);

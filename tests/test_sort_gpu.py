@@ -170,10 +170,15 @@ def test_xcd_dispatch_selftest_and_both_tile_assignments():
 
     from thrust_amd import capi
     L = capi.lib()
-    grouped = ctypes.c_int(-1)
-    rc = L.thrust_cdna4_selftest_xcd_dispatch(ctypes.byref(grouped), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-    assert rc == 0
-    assert grouped.value == 1
+    torch.cuda.synchronize()
+    verdicts = []
+    for _ in range(3):  # 1: the device qualifies; 0 / -1 / -2: why not (the probe times workgroups: it is conservative under load)
+        grouped = ctypes.c_int(-9)
+        rc = L.thrust_cdna4_selftest_xcd_dispatch(ctypes.byref(grouped), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0
+        verdicts.append(grouped.value)
+    print("xcd dispatch probe:", verdicts)
+    assert 1 in verdicts, verdicts
     before = ctypes.c_ulonglong(0)
     L.thrust_cdna4_lookback_timeouts(ctypes.byref(before))
     for plain in (0, 1):

@@ -697,8 +697,13 @@ static std::atomic<int> g_xcd_verdict[kMaxDevices];  // 0 not probed, 1 grouped 
 static std::atomic<int> g_force_plain_tickets{0};    // test knob
 static std::mutex g_xcd_mu;
 
-static hipError_t run_xcd_dispatch_probe(hipStream_t s, bool* grouped_ok) {
+// *why: 1 the device qualifies; 0 its workgroups are not spread over 8 XCDs by index; -1 the XCDs
+// were not seen to be served independently; -2 the CU count does not fit the probe
+static hipError_t run_xcd_dispatch_probe(hipStream_t s, bool* grouped_ok, int* why = nullptr) {
   *grouped_ok = false;
+  int why_local = 0;
+  if (!why) why = &why_local;
+  *why = -2;
   const int per_xcd = device_cu_count() / kXcds;
   const int wgs = kXcds * 3 * per_xcd;
   if (per_xcd < 1 || device_cu_count() % kXcds != 0 || wgs > kProbeMax) return hipSuccess;
@@ -719,13 +724,19 @@ static hipError_t run_xcd_dispatch_probe(hipStream_t s, bool* grouped_ok) {
   if (e != hipSuccess) return e;
   e = hipStreamSynchronize(s);
   if (e != hipSuccess) return e;
+  // workgroup i on XCD (i + first) mod 8, with one `first` for the whole launch: the workgroups of an
+  // index class then share an XCD, which is all that the groups need
+  *why = 0;
+  const unsigned first = xcd_of[0];
   for (int i = 0; i < wgs; i++)
-    if (xcd_of[i] != (unsigned)(i % kXcds)) return hipSuccess;  // another mapping of workgroups to XCDs
+    if (xcd_of[i] >= (unsigned)kXcds || xcd_of[i] != (first + (unsigned)i) % kXcds) return hipSuccess;
+  *why = -1;
   // class 0's first workgroup of the second round starts when one of its first round has left
   const unsigned long long second_round_of_slow = start[(size_t)per_xcd * kXcds];
   for (int c = 1; c < kXcds; c++)
     if (start[(size_t)(3 * per_xcd - 1) * kXcds + c] >= second_round_of_slow) return hipSuccess;  // the XCDs are not served independently
   *grouped_ok = true;
+  *why = 1;
   return hipSuccess;
 }
 
@@ -985,8 +996,9 @@ extern "C" int thrust_cdna4_set_test_sort_plain_tickets(int on) {
 extern "C" int thrust_cdna4_selftest_xcd_dispatch(int* grouped, void* stream) {
   if (!grouped) return hipErrorInvalidValue;
   bool ok = false;
-  const hipError_t e = tcd::run_xcd_dispatch_probe(static_cast<hipStream_t>(stream), &ok);
-  *grouped = ok ? 1 : 0;
+  int why = 0;
+  const hipError_t e = tcd::run_xcd_dispatch_probe(static_cast<hipStream_t>(stream), &ok, &why);
+  *grouped = why;
   return (int)e;
 }
 
