@@ -21,7 +21,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # measured HBM traffic of one onesweep launch over 2^28 uint32 keys
 # (profiles/onesweep_u32_sort_2p28_and_extras.md)
-ONESWEEP_U32_TRAFFIC_BYTES = 2.243e9
+ONESWEEP_U32_TRAFFIC_BYTES = 2.213e9
 
 
 def parse():
