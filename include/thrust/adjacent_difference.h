@@ -31,12 +31,12 @@ template <class Policy, class In, class Out, detail::enable_if_policy<Policy> = 
 Out adjacent_difference(const Policy& exec, In first, In last, Out out) {
   return adjacent_difference(exec, first, last, out, minus<typename detail::value_of<In>::type>());
 }
-template <class In, class Out, detail::enable_if_device<In> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(device, f, l, o); }
-template <class In, class Out, detail::enable_if_host<In> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(host, f, l, o); }
-template <class In, class Out, class Op, detail::enable_if_device<In> = 0,
+template <class In, class Out, detail::enable_if_device<In, Out> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(device, f, l, o); }
+template <class In, class Out, detail::enable_if_host<In, Out> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(host, f, l, o); }
+template <class In, class Out, class Op, detail::enable_if_device<In, Out, Op> = 0,
           class = typename std::iterator_traits<Out>::iterator_category>
 Out adjacent_difference(In f, In l, Out o, Op op) { return adjacent_difference(device, f, l, o, op); }
-template <class In, class Out, class Op, detail::enable_if_host<In> = 0,
+template <class In, class Out, class Op, detail::enable_if_host<In, Out, Op> = 0,
           class = typename std::iterator_traits<Out>::iterator_category>
 Out adjacent_difference(In f, In l, Out o, Op op) { return adjacent_difference(host, f, l, o, op); }
 }  // namespace thrust

@@ -74,12 +74,12 @@ Out copy_if(const system::cpp::detail::par_t&, In first, In last, St stencil, Ou
   for (; first != last; ++first, ++stencil) if (pred(*stencil)) { *out = *first; ++out; }
   return out;
 }
-template <class In, class Out, class Pred, detail::enable_if_device<In> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(device, f, l, o, p); }
-template <class In, class Out, class Pred, detail::enable_if_host<In> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(host, f, l, o, p); }
-template <class In, class St, class Out, class Pred, detail::enable_if_device<In> = 0,
+template <class In, class Out, class Pred, detail::enable_if_device<In, Out, Pred> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(device, f, l, o, p); }
+template <class In, class Out, class Pred, detail::enable_if_host<In, Out, Pred> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(host, f, l, o, p); }
+template <class In, class St, class Out, class Pred, detail::enable_if_device<In, St, Out, Pred> = 0,
           class = typename std::iterator_traits<St>::iterator_category>
 Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(device, f, l, s, o, p); }
-template <class In, class St, class Out, class Pred, detail::enable_if_host<In> = 0,
+template <class In, class St, class Out, class Pred, detail::enable_if_host<In, St, Out, Pred> = 0,
           class = typename std::iterator_traits<St>::iterator_category>
 Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(host, f, l, s, o, p); }
 

@@ -1,0 +1,3 @@
+// <thrust/detail/cpp14_required.h>: every compiler these headers build with is C++14 or later.
+#pragma once
+#include <thrust/detail/config.h>

@@ -18,8 +18,11 @@ template <class T> struct unwrap_iterator<thrust::device_ptr<T>> {
 };
 template <class It> inline typename unwrap_iterator<It>::type unwrap(It it) { return unwrap_iterator<It>::apply(it); }
 template <class It> struct value_of { typedef typename std::iterator_traits<It>::value_type type; };
-template <class It> using enable_if_device = typename std::enable_if<system::cdna4::detail::is_device_iterator<It>::value, int>::type;
-template <class It> using enable_if_host = typename std::enable_if<!system::cdna4::detail::is_device_iterator<It>::value, int>::type;
+// Which overload of an algorithm called without a policy applies, from the types of its arguments:
+// the first iterator that walks memory decides (counting / constant / discard iterators and
+// arguments that are no iterators do not); with none, the device.
+template <class... Args> using enable_if_device = typename std::enable_if<system::cdna4::detail::runs_on_device<Args...>::value, int>::type;
+template <class... Args> using enable_if_host = typename std::enable_if<!system::cdna4::detail::runs_on_device<Args...>::value, int>::type;
 // an execution policy of either system (tells policy-first overloads from iterator-first ones)
 template <class P> struct is_policy {
   static constexpr bool value = std::is_base_of<system::cdna4::execution_policy<P>, P>::value || std::is_same<P, system::cpp::detail::par_t>::value;

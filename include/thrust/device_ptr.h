@@ -115,5 +115,21 @@ template <class It> struct has_device_category<It, typename std::enable_if<std::
 template <class It> struct is_device_iterator { static constexpr bool value = declares_device_iterator<It>::value || has_device_category<It>::value; };
 template <class T> struct is_device_iterator<T*> { static constexpr bool value = false; };
 template <class T> struct is_device_iterator<thrust::device_ptr<T>> { static constexpr bool value = true; };
+// Iterators that walk no memory — counting, constant, discard, and adaptors over nothing else —
+// belong to any system (thrust/iterator/detail/any_system_tag.h:27-38): they count as device
+// iterators, and next to a range in memory they follow that range's system.
+template <class It> struct is_any_system_iterator : std::false_type {};
+template <class T, bool = std::is_pointer<T>::value, class = void> struct is_iterator_type : std::false_type {};
+template <class T> struct is_iterator_type<T, true, void> : std::is_object<typename std::remove_pointer<T>::type> {};
+template <class T> struct is_iterator_type<T, false, typename std::conditional<false, typename std::iterator_traits<T>::iterator_category, void>::type> : std::true_type {};
+// The system that an algorithm called without a policy runs on, from all of its argument types
+// (thrust/detail/generic/select_system.inl:60-170): arguments that are no iterators, and iterators
+// of any system, have no say; the first other iterator decides; with none, the device.
+template <class... Ts> struct runs_on_device : std::true_type {};
+template <class T, class... R> struct runs_on_device<T, R...>
+    : std::conditional<!is_iterator_type<T>::value || is_any_system_iterator<T>::value, runs_on_device<R...>,
+                       std::integral_constant<bool, is_device_iterator<T>::value>>::type {};
+template <class... Ts> struct all_any_system : std::true_type {};
+template <class T, class... R> struct all_any_system<T, R...> : std::integral_constant<bool, is_any_system_iterator<T>::value && all_any_system<R...>::value> {};
 }}}  // namespace system::cdna4::detail
 }  // namespace thrust

@@ -19,7 +19,12 @@ namespace thrust {
 
 template <class T, class Alloc>
 class device_vector {
-  static_assert(std::is_trivially_copyable<T>::value, "device_vector of the cdna4 system holds trivially copyable types");
+  // Elements travel between host and device, and within the device, as bytes — what the reference
+  // does for the types it holds to be trivially relocatable (thrust/type_traits/is_trivially_relocatable.h).
+  // A copy constructor or assignment operator written out by the user (a number-like struct with
+  // __host__ __device__ members, say) is accepted and not run; a destructor with effects is refused.
+  static_assert(detail::is_bytewise_movable<T>::value,
+                "device_vector of the cdna4 system holds types that can be moved as bytes");
 
  public:
   typedef T value_type;

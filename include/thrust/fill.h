@@ -52,8 +52,8 @@ It fill_n(const Policy& exec, It first, Size n, const V& value) {
   fill(exec, first, first + n, value);
   return first + n;
 }
-template <class It, class V, detail::enable_if_device<It> = 0> void fill(It f, It l, const V& v) { fill(device, f, l, v); }
-template <class It, class V, detail::enable_if_host<It> = 0> void fill(It f, It l, const V& v) { fill(host, f, l, v); }
-template <class It, class Size, class V, detail::enable_if_device<It> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(device, f, n, v); }
-template <class It, class Size, class V, detail::enable_if_host<It> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(host, f, n, v); }
+template <class It, class V, detail::enable_if_device<It, V> = 0> void fill(It f, It l, const V& v) { fill(device, f, l, v); }
+template <class It, class V, detail::enable_if_host<It, V> = 0> void fill(It f, It l, const V& v) { fill(host, f, l, v); }
+template <class It, class Size, class V, detail::enable_if_device<It, Size, V> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(device, f, n, v); }
+template <class It, class Size, class V, detail::enable_if_host<It, Size, V> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(host, f, n, v); }
 }  // namespace thrust

@@ -47,10 +47,10 @@ template <class It, class Pred> It find_if_not(const system::cpp::detail::par_t&
 template <class Policy, class It, class T, detail::enable_if_policy<Policy> = 0>
 It find(const Policy& exec, It first, It last, const T& value) { return find_if(exec, first, last, detail::equals_value<T>{value}); }
 
-template <class It, class T, detail::enable_if_device<It> = 0> It find(It f, It l, const T& v) { return find(device, f, l, v); }
-template <class It, class T, detail::enable_if_host<It> = 0> It find(It f, It l, const T& v) { return find(host, f, l, v); }
-template <class It, class P, detail::enable_if_device<It> = 0> It find_if(It f, It l, P p) { return find_if(device, f, l, p); }
-template <class It, class P, detail::enable_if_host<It> = 0> It find_if(It f, It l, P p) { return find_if(host, f, l, p); }
-template <class It, class P, detail::enable_if_device<It> = 0> It find_if_not(It f, It l, P p) { return find_if_not(device, f, l, p); }
-template <class It, class P, detail::enable_if_host<It> = 0> It find_if_not(It f, It l, P p) { return find_if_not(host, f, l, p); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> It find(It f, It l, const T& v) { return find(device, f, l, v); }
+template <class It, class T, detail::enable_if_host<It, T> = 0> It find(It f, It l, const T& v) { return find(host, f, l, v); }
+template <class It, class P, detail::enable_if_device<It, P> = 0> It find_if(It f, It l, P p) { return find_if(device, f, l, p); }
+template <class It, class P, detail::enable_if_host<It, P> = 0> It find_if(It f, It l, P p) { return find_if(host, f, l, p); }
+template <class It, class P, detail::enable_if_device<It, P> = 0> It find_if_not(It f, It l, P p) { return find_if_not(device, f, l, p); }
+template <class It, class P, detail::enable_if_host<It, P> = 0> It find_if_not(It f, It l, P p) { return find_if_not(host, f, l, p); }
 }  // namespace thrust

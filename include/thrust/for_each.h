@@ -14,19 +14,19 @@ namespace thrust {
 // thrust::device_execution_policy (examples/minimal_custom_backend.cu) is preferred to it.
 template <class D, class It, class F>
 It for_each(const detail::execution_policy_base<D>& exec, It first, It last, F f) {
-  return for_each(static_cast<const D&>(exec), first, last, f);
+  return for_each(detail::derived_cast(detail::strip_const(exec)), first, last, f);
 }
 template <class D, class It, class Size, class F>
 It for_each_n(const detail::execution_policy_base<D>& exec, It first, Size n, F f) {
-  return for_each_n(static_cast<const D&>(exec), first, n, f);
+  return for_each_n(detail::derived_cast(detail::strip_const(exec)), first, n, f);
 }
 template <class It, class F>
 It for_each(const system::cpp::detail::par_t&, It first, It last, F f) { std::for_each(first, last, f); return last; }
 template <class It, class Size, class F>
 It for_each_n(const system::cpp::detail::par_t&, It first, Size n, F f) { std::for_each(first, first + n, f); return first + n; }
 
-template <class It, class F, detail::enable_if_device<It> = 0> It for_each(It f, It l, F fn) { return for_each(device, f, l, fn); }
-template <class It, class F, detail::enable_if_host<It> = 0> It for_each(It f, It l, F fn) { return for_each(host, f, l, fn); }
-template <class It, class Size, class F, detail::enable_if_device<It> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(device, f, n, fn); }
-template <class It, class Size, class F, detail::enable_if_host<It> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(host, f, n, fn); }
+template <class It, class F, detail::enable_if_device<It, F> = 0> It for_each(It f, It l, F fn) { return for_each(device, f, l, fn); }
+template <class It, class F, detail::enable_if_host<It, F> = 0> It for_each(It f, It l, F fn) { return for_each(host, f, l, fn); }
+template <class It, class Size, class F, detail::enable_if_device<It, Size, F> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(device, f, n, fn); }
+template <class It, class Size, class F, detail::enable_if_host<It, Size, F> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(host, f, n, fn); }
 }  // namespace thrust

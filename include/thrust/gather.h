@@ -55,16 +55,16 @@ Out gather_if(const system::cpp::detail::par_t&, Map map_first, Map map_last, S 
 template <class Policy, class Map, class S, class In, class Out, detail::enable_if_policy<Policy> = 0>
 Out gather_if(const Policy& exec, Map mf, Map ml, S st, In in, Out out) { return gather_if(exec, mf, ml, st, in, out, detail::truthy()); }
 
-template <class Map, class In, class Out, detail::enable_if_device<Map> = 0>
+template <class Map, class In, class Out, detail::enable_if_device<Map, In, Out> = 0>
 Out gather(Map mf, Map ml, In in, Out out) { return gather(device, mf, ml, in, out); }
-template <class Map, class In, class Out, detail::enable_if_host<Map> = 0>
+template <class Map, class In, class Out, detail::enable_if_host<Map, In, Out> = 0>
 Out gather(Map mf, Map ml, In in, Out out) { return gather(host, mf, ml, in, out); }
-template <class Map, class S, class In, class Out, detail::enable_if_device<Map> = 0>
+template <class Map, class S, class In, class Out, detail::enable_if_device<Map, S, In, Out> = 0>
 Out gather_if(Map mf, Map ml, S st, In in, Out out) { return gather_if(device, mf, ml, st, in, out); }
-template <class Map, class S, class In, class Out, detail::enable_if_host<Map> = 0>
+template <class Map, class S, class In, class Out, detail::enable_if_host<Map, S, In, Out> = 0>
 Out gather_if(Map mf, Map ml, S st, In in, Out out) { return gather_if(host, mf, ml, st, in, out); }
-template <class Map, class S, class In, class Out, class Pred, detail::enable_if_device<Map> = 0>
+template <class Map, class S, class In, class Out, class Pred, detail::enable_if_device<Map, S, In, Out, Pred> = 0>
 Out gather_if(Map mf, Map ml, S st, In in, Out out, Pred p) { return gather_if(device, mf, ml, st, in, out, p); }
-template <class Map, class S, class In, class Out, class Pred, detail::enable_if_host<Map> = 0>
+template <class Map, class S, class In, class Out, class Pred, detail::enable_if_host<Map, S, In, Out, Pred> = 0>
 Out gather_if(Map mf, Map ml, S st, In in, Out out, Pred p) { return gather_if(host, mf, ml, st, in, out, p); }
 }  // namespace thrust

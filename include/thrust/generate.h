@@ -29,8 +29,8 @@ It generate_n(const Policy& exec, It first, Size n, G gen) {
   generate(exec, first, first + n, gen);
   return first + n;
 }
-template <class It, class G, detail::enable_if_device<It> = 0> void generate(It f, It l, G g) { generate(device, f, l, g); }
-template <class It, class G, detail::enable_if_host<It> = 0> void generate(It f, It l, G g) { generate(host, f, l, g); }
-template <class It, class Size, class G, detail::enable_if_device<It> = 0> It generate_n(It f, Size n, G g) { return generate_n(device, f, n, g); }
-template <class It, class Size, class G, detail::enable_if_host<It> = 0> It generate_n(It f, Size n, G g) { return generate_n(host, f, n, g); }
+template <class It, class G, detail::enable_if_device<It, G> = 0> void generate(It f, It l, G g) { generate(device, f, l, g); }
+template <class It, class G, detail::enable_if_host<It, G> = 0> void generate(It f, It l, G g) { generate(host, f, l, g); }
+template <class It, class Size, class G, detail::enable_if_device<It, Size, G> = 0> It generate_n(It f, Size n, G g) { return generate_n(device, f, n, g); }
+template <class It, class Size, class G, detail::enable_if_host<It, Size, G> = 0> It generate_n(It f, Size n, G g) { return generate_n(host, f, n, g); }
 }  // namespace thrust

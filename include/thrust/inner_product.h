@@ -30,10 +30,10 @@ T inner_product(const system::cpp::detail::par_t&, It1 first1, It1 last1, It2 fi
 }
 template <class Policy, class It1, class It2, class T, detail::enable_if_policy<Policy> = 0>
 T inner_product(const Policy& exec, It1 f1, It1 l1, It2 f2, T init) { return inner_product(exec, f1, l1, f2, init, plus<T>(), multiplies<T>()); }
-template <class It1, class It2, class T, detail::enable_if_device<It1> = 0> T inner_product(It1 f1, It1 l1, It2 f2, T init) { return inner_product(device, f1, l1, f2, init); }
-template <class It1, class It2, class T, detail::enable_if_host<It1> = 0> T inner_product(It1 f1, It1 l1, It2 f2, T init) { return inner_product(host, f1, l1, f2, init); }
-template <class It1, class It2, class T, class O1, class O2, detail::enable_if_device<It1> = 0>
+template <class It1, class It2, class T, detail::enable_if_device<It1, It2, T> = 0> T inner_product(It1 f1, It1 l1, It2 f2, T init) { return inner_product(device, f1, l1, f2, init); }
+template <class It1, class It2, class T, detail::enable_if_host<It1, It2, T> = 0> T inner_product(It1 f1, It1 l1, It2 f2, T init) { return inner_product(host, f1, l1, f2, init); }
+template <class It1, class It2, class T, class O1, class O2, detail::enable_if_device<It1, It2, T, O1, O2> = 0>
 T inner_product(It1 f1, It1 l1, It2 f2, T init, O1 o1, O2 o2) { return inner_product(device, f1, l1, f2, init, o1, o2); }
-template <class It1, class It2, class T, class O1, class O2, detail::enable_if_host<It1> = 0>
+template <class It1, class It2, class T, class O1, class O2, detail::enable_if_host<It1, It2, T, O1, O2> = 0>
 T inner_product(It1 f1, It1 l1, It2 f2, T init, O1 o1, O2 o2) { return inner_product(host, f1, l1, f2, init, o1, o2); }
 }  // namespace thrust

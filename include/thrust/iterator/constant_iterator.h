@@ -24,5 +24,6 @@ class constant_iterator : public detail::fancy_base<constant_iterator<T>, T> {
 template <class T> THRUST_CDNA4_HD constant_iterator<T> make_constant_iterator(T v) { return constant_iterator<T>(v); }
 namespace system { namespace cdna4 { namespace detail {
 template <class T> struct is_device_iterator<thrust::constant_iterator<T>> { static constexpr bool value = true; };
+template <class T> struct is_any_system_iterator<thrust::constant_iterator<T>> : std::true_type {};
 }}}
 }  // namespace thrust

@@ -25,5 +25,6 @@ namespace system { namespace cdna4 { namespace detail {
 template <class T, class S, class Tr, class D> struct is_device_iterator<thrust::counting_iterator<T, S, Tr, D>> {
   static constexpr bool value = !std::is_same<S, thrust::system::cpp::tag>::value;
 };
+template <class T, class Tr, class D> struct is_any_system_iterator<thrust::counting_iterator<T, use_default, Tr, D>> : std::true_type {};
 }}}
 }  // namespace thrust

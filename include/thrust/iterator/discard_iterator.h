@@ -29,5 +29,6 @@ class discard_iterator : public detail::fancy_base<discard_iterator<System>, det
 THRUST_CDNA4_HD inline discard_iterator<> make_discard_iterator(std::ptrdiff_t pos = 0) { return discard_iterator<>(pos); }
 namespace system { namespace cdna4 { namespace detail {
 template <class S> struct is_device_iterator<thrust::discard_iterator<S>> { static constexpr bool value = true; };
+template <class S> struct is_any_system_iterator<thrust::discard_iterator<S>> : std::true_type {};
 }}}
 }  // namespace thrust

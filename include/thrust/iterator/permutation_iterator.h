@@ -27,7 +27,8 @@ THRUST_CDNA4_HD permutation_iterator<ElementIt, IndexIt> make_permutation_iterat
   return permutation_iterator<ElementIt, IndexIt>(e, i);
 }
 namespace system { namespace cdna4 { namespace detail {
-template <class E, class I> struct is_device_iterator<thrust::permutation_iterator<E, I>> : is_device_iterator<E> {};
+template <class E, class I> struct is_device_iterator<thrust::permutation_iterator<E, I>> : runs_on_device<E, I> {};
+template <class E, class I> struct is_any_system_iterator<thrust::permutation_iterator<E, I>> : all_any_system<E, I> {};
 }}}
 namespace detail {
 template <class E, class I> struct unwrap_iterator<thrust::permutation_iterator<E, I>> {

@@ -21,6 +21,7 @@ class reverse_iterator : public detail::fancy_base<reverse_iterator<It>, typenam
 template <class It> THRUST_CDNA4_HD reverse_iterator<It> make_reverse_iterator(It it) { return reverse_iterator<It>(it); }
 namespace system { namespace cdna4 { namespace detail {
 template <class It> struct is_device_iterator<thrust::reverse_iterator<It>> : is_device_iterator<It> {};
+template <class It> struct is_any_system_iterator<thrust::reverse_iterator<It>> : is_any_system_iterator<It> {};
 }}}
 namespace detail {
 template <class It> struct unwrap_iterator<thrust::reverse_iterator<It>> {

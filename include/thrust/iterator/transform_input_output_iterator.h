@@ -45,6 +45,7 @@ THRUST_CDNA4_HD transform_input_output_iterator<InF, OutF, It> make_transform_in
 }
 namespace system { namespace cdna4 { namespace detail {
 template <class InF, class OutF, class It> struct is_device_iterator<thrust::transform_input_output_iterator<InF, OutF, It>> : is_device_iterator<It> {};
+template <class InF, class OutF, class It> struct is_any_system_iterator<thrust::transform_input_output_iterator<InF, OutF, It>> : is_any_system_iterator<It> {};
 }}}
 namespace detail {
 template <class InF, class OutF, class It> struct unwrap_iterator<thrust::transform_input_output_iterator<InF, OutF, It>> {

@@ -40,6 +40,7 @@ template <class F, class It>
 THRUST_CDNA4_HD transform_iterator<F, It> make_transform_iterator(It it, F f) { return transform_iterator<F, It>(it, f); }
 namespace system { namespace cdna4 { namespace detail {
 template <class F, class It, class R, class V> struct is_device_iterator<thrust::transform_iterator<F, It, R, V>> : is_device_iterator<It> {};
+template <class F, class It, class R, class V> struct is_any_system_iterator<thrust::transform_iterator<F, It, R, V>> : is_any_system_iterator<It> {};
 }}}
 namespace detail {
 template <class F, class It, class R, class V> struct unwrap_iterator<thrust::transform_iterator<F, It, R, V>> {

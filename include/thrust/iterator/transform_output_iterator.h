@@ -34,6 +34,7 @@ template <class F, class It>
 THRUST_CDNA4_HD transform_output_iterator<F, It> make_transform_output_iterator(It it, F f) { return transform_output_iterator<F, It>(it, f); }
 namespace system { namespace cdna4 { namespace detail {
 template <class F, class It> struct is_device_iterator<thrust::transform_output_iterator<F, It>> : is_device_iterator<It> {};
+template <class F, class It> struct is_any_system_iterator<thrust::transform_output_iterator<F, It>> : is_any_system_iterator<It> {};
 }}}
 namespace detail {
 template <class F, class It> struct unwrap_iterator<thrust::transform_output_iterator<F, It>> {

@@ -34,7 +34,8 @@ THRUST_CDNA4_HD zip_iterator<tuple<Its...>> make_zip_iterator(const tuple<Its...
 template <class... Its, class = typename std::enable_if<(sizeof...(Its) > 1)>::type>
 THRUST_CDNA4_HD zip_iterator<tuple<Its...>> make_zip_iterator(Its... its) { return zip_iterator<tuple<Its...>>(tuple<Its...>(its...)); }
 namespace system { namespace cdna4 { namespace detail {
-template <class It, class... Its> struct is_device_iterator<thrust::zip_iterator<thrust::tuple<It, Its...>>> : is_device_iterator<It> {};
+template <class It, class... Its> struct is_device_iterator<thrust::zip_iterator<thrust::tuple<It, Its...>>> : runs_on_device<It, Its...> {};
+template <class... Its> struct is_any_system_iterator<thrust::zip_iterator<thrust::tuple<Its...>>> : all_any_system<Its...> {};
 }}}
 namespace detail {
 template <class... Its> struct unwrap_iterator<thrust::zip_iterator<thrust::tuple<Its...>>> {

@@ -11,8 +11,8 @@ bool any_of(const Policy& exec, It first, It last, Pred pred) { return find_if(e
 template <class Policy, class It, class Pred, detail::enable_if_policy<Policy> = 0>
 bool none_of(const Policy& exec, It first, It last, Pred pred) { return !any_of(exec, first, last, pred); }
 #define THRUST_CDNA4_LOGICAL(NAME)                                                                                   \
-  template <class It, class P, detail::enable_if_device<It> = 0> bool NAME(It f, It l, P p) { return NAME(device, f, l, p); } \
-  template <class It, class P, detail::enable_if_host<It> = 0> bool NAME(It f, It l, P p) { return NAME(host, f, l, p); }
+  template <class It, class P, detail::enable_if_device<It, P> = 0> bool NAME(It f, It l, P p) { return NAME(device, f, l, p); } \
+  template <class It, class P, detail::enable_if_host<It, P> = 0> bool NAME(It f, It l, P p) { return NAME(host, f, l, p); }
 THRUST_CDNA4_LOGICAL(all_of)
 THRUST_CDNA4_LOGICAL(any_of)
 THRUST_CDNA4_LOGICAL(none_of)

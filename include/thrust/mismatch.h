@@ -31,8 +31,8 @@ pair<It1, It2> mismatch(const system::cpp::detail::par_t&, It1 first1, It1 last1
 }
 template <class Policy, class It1, class It2, detail::enable_if_policy<Policy> = 0>
 pair<It1, It2> mismatch(const Policy& exec, It1 f1, It1 l1, It2 f2) { return mismatch(exec, f1, l1, f2, equal_to<>()); }
-template <class It1, class It2, detail::enable_if_device<It1> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2) { return mismatch(device, f1, l1, f2); }
-template <class It1, class It2, detail::enable_if_host<It1> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2) { return mismatch(host, f1, l1, f2); }
-template <class It1, class It2, class P, detail::enable_if_device<It1> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2, P p) { return mismatch(device, f1, l1, f2, p); }
-template <class It1, class It2, class P, detail::enable_if_host<It1> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2, P p) { return mismatch(host, f1, l1, f2, p); }
+template <class It1, class It2, detail::enable_if_device<It1, It2> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2) { return mismatch(device, f1, l1, f2); }
+template <class It1, class It2, detail::enable_if_host<It1, It2> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2) { return mismatch(host, f1, l1, f2); }
+template <class It1, class It2, class P, detail::enable_if_device<It1, It2, P> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2, P p) { return mismatch(device, f1, l1, f2, p); }
+template <class It1, class It2, class P, detail::enable_if_host<It1, It2, P> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2, P p) { return mismatch(host, f1, l1, f2, p); }
 }  // namespace thrust

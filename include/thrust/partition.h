@@ -76,28 +76,28 @@ pair<OutT, OutF> partition_copy(const Policy& exec, In first, In last, St stenci
 }
 // ---- no policy
 #define THRUST_CDNA4_PARTITION_NO_POLICY(NAME)                                                                          \
-  template <class It, class Pred, detail::enable_if_device<It> = 0>                                                     \
+  template <class It, class Pred, detail::enable_if_device<It, Pred> = 0>                                                     \
   It NAME(It f, It l, Pred p) { return NAME(device, f, l, p); }                                                         \
-  template <class It, class Pred, detail::enable_if_host<It> = 0>                                                       \
+  template <class It, class Pred, detail::enable_if_host<It, Pred> = 0>                                                       \
   It NAME(It f, It l, Pred p) { return NAME(host, f, l, p); }                                                           \
-  template <class It, class St, class Pred, detail::enable_if_device<It> = 0,                                           \
+  template <class It, class St, class Pred, detail::enable_if_device<It, St, Pred> = 0,                                           \
             class = typename std::iterator_traits<St>::iterator_category>                                               \
   It NAME(It f, It l, St s, Pred p) { return NAME(device, f, l, s, p); }                                                \
-  template <class It, class St, class Pred, detail::enable_if_host<It> = 0,                                             \
+  template <class It, class St, class Pred, detail::enable_if_host<It, St, Pred> = 0,                                             \
             class = typename std::iterator_traits<St>::iterator_category>                                               \
   It NAME(It f, It l, St s, Pred p) { return NAME(host, f, l, s, p); }
 THRUST_CDNA4_PARTITION_NO_POLICY(partition)
 THRUST_CDNA4_PARTITION_NO_POLICY(stable_partition)
 #undef THRUST_CDNA4_PARTITION_NO_POLICY
 #define THRUST_CDNA4_PARTITION_COPY_NO_POLICY(NAME)                                                                     \
-  template <class In, class OutT, class OutF, class Pred, detail::enable_if_device<In> = 0>                             \
+  template <class In, class OutT, class OutF, class Pred, detail::enable_if_device<In, OutT, OutF, Pred> = 0>                             \
   pair<OutT, OutF> NAME(In f, In l, OutT t, OutF o, Pred p) { return NAME(device, f, l, t, o, p); }                     \
-  template <class In, class OutT, class OutF, class Pred, detail::enable_if_host<In> = 0>                               \
+  template <class In, class OutT, class OutF, class Pred, detail::enable_if_host<In, OutT, OutF, Pred> = 0>                               \
   pair<OutT, OutF> NAME(In f, In l, OutT t, OutF o, Pred p) { return NAME(host, f, l, t, o, p); }                       \
-  template <class In, class St, class OutT, class OutF, class Pred, detail::enable_if_device<In> = 0,                   \
+  template <class In, class St, class OutT, class OutF, class Pred, detail::enable_if_device<In, St, OutT, OutF, Pred> = 0,                   \
             class = typename std::iterator_traits<OutF>::iterator_category>                                             \
   pair<OutT, OutF> NAME(In f, In l, St s, OutT t, OutF o, Pred p) { return NAME(device, f, l, s, t, o, p); }            \
-  template <class In, class St, class OutT, class OutF, class Pred, detail::enable_if_host<In> = 0,                     \
+  template <class In, class St, class OutT, class OutF, class Pred, detail::enable_if_host<In, St, OutT, OutF, Pred> = 0,                     \
             class = typename std::iterator_traits<OutF>::iterator_category>                                             \
   pair<OutT, OutF> NAME(In f, In l, St s, OutT t, OutF o, Pred p) { return NAME(host, f, l, s, t, o, p); }
 THRUST_CDNA4_PARTITION_COPY_NO_POLICY(partition_copy)
@@ -112,8 +112,8 @@ template <class Policy, class It, class Pred, detail::enable_if_policy<Policy> =
 bool is_partitioned(const Policy& exec, It first, It last, Pred pred) {
   return thrust::none_of(exec, thrust::find_if_not(exec, first, last, pred), last, pred);
 }
-template <class It, class Pred, detail::enable_if_device<It> = 0> It partition_point(It f, It l, Pred p) { return partition_point(device, f, l, p); }
-template <class It, class Pred, detail::enable_if_host<It> = 0> It partition_point(It f, It l, Pred p) { return partition_point(host, f, l, p); }
-template <class It, class Pred, detail::enable_if_device<It> = 0> bool is_partitioned(It f, It l, Pred p) { return is_partitioned(device, f, l, p); }
-template <class It, class Pred, detail::enable_if_host<It> = 0> bool is_partitioned(It f, It l, Pred p) { return is_partitioned(host, f, l, p); }
+template <class It, class Pred, detail::enable_if_device<It, Pred> = 0> It partition_point(It f, It l, Pred p) { return partition_point(device, f, l, p); }
+template <class It, class Pred, detail::enable_if_host<It, Pred> = 0> It partition_point(It f, It l, Pred p) { return partition_point(host, f, l, p); }
+template <class It, class Pred, detail::enable_if_device<It, Pred> = 0> bool is_partitioned(It f, It l, Pred p) { return is_partitioned(device, f, l, p); }
+template <class It, class Pred, detail::enable_if_host<It, Pred> = 0> bool is_partitioned(It f, It l, Pred p) { return is_partitioned(host, f, l, p); }
 }  // namespace thrust

@@ -135,9 +135,9 @@ typename detail::value_of<It>::type reduce(const system::cpp::detail::par_t&, It
 }
 template <class It, detail::enable_if_device<It> = 0> typename detail::value_of<It>::type reduce(It f, It l) { return reduce(typename detail::implicit_policy<It>::type(), f, l); }
 template <class It, detail::enable_if_host<It> = 0> typename detail::value_of<It>::type reduce(It f, It l) { return reduce(host, f, l); }
-template <class It, class T, detail::enable_if_device<It> = 0> T reduce(It f, It l, T init) { return reduce(typename detail::implicit_policy<It>::type(), f, l, init); }
-template <class It, class T, detail::enable_if_host<It> = 0> T reduce(It f, It l, T init) { return reduce(host, f, l, init); }
-template <class It, class T, class Op, detail::enable_if_device<It> = 0> T reduce(It f, It l, T init, Op op) { return reduce(typename detail::implicit_policy<It>::type(), f, l, init, op); }
-template <class It, class T, class Op, detail::enable_if_host<It> = 0> T reduce(It f, It l, T init, Op op) { return reduce(host, f, l, init, op); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> T reduce(It f, It l, T init) { return reduce(typename detail::implicit_policy<It>::type(), f, l, init); }
+template <class It, class T, detail::enable_if_host<It, T> = 0> T reduce(It f, It l, T init) { return reduce(host, f, l, init); }
+template <class It, class T, class Op, detail::enable_if_device<It, T, Op> = 0> T reduce(It f, It l, T init, Op op) { return reduce(typename detail::implicit_policy<It>::type(), f, l, init, op); }
+template <class It, class T, class Op, detail::enable_if_host<It, T, Op> = 0> T reduce(It f, It l, T init, Op op) { return reduce(host, f, l, init, op); }
 
 }  // namespace thrust

@@ -122,26 +122,26 @@ OutIt exclusive_scan(const system::cpp::detail::par_t& e, InIt first, InIt last,
 }
 
 // ===================================================================== scan, no policy
-template <class InIt, class OutIt, detail::enable_if_device<InIt> = 0>
+template <class InIt, class OutIt, detail::enable_if_device<InIt, OutIt> = 0>
 OutIt inclusive_scan(InIt f, InIt l, OutIt r) { return inclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r); }
-template <class InIt, class OutIt, class Op, detail::enable_if_device<InIt> = 0>
+template <class InIt, class OutIt, class Op, detail::enable_if_device<InIt, OutIt, Op> = 0>
 OutIt inclusive_scan(InIt f, InIt l, OutIt r, Op op) { return inclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r, op); }
-template <class InIt, class OutIt, detail::enable_if_host<InIt> = 0>
+template <class InIt, class OutIt, detail::enable_if_host<InIt, OutIt> = 0>
 OutIt inclusive_scan(InIt f, InIt l, OutIt r) { return inclusive_scan(host, f, l, r); }
-template <class InIt, class OutIt, class Op, detail::enable_if_host<InIt> = 0>
+template <class InIt, class OutIt, class Op, detail::enable_if_host<InIt, OutIt, Op> = 0>
 OutIt inclusive_scan(InIt f, InIt l, OutIt r, Op op) { return inclusive_scan(host, f, l, r, op); }
 
-template <class InIt, class OutIt, detail::enable_if_device<InIt> = 0>
+template <class InIt, class OutIt, detail::enable_if_device<InIt, OutIt> = 0>
 OutIt exclusive_scan(InIt f, InIt l, OutIt r) { return exclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r); }
-template <class InIt, class OutIt, class T, detail::enable_if_device<InIt> = 0>
+template <class InIt, class OutIt, class T, detail::enable_if_device<InIt, OutIt, T> = 0>
 OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init) { return exclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r, init); }
-template <class InIt, class OutIt, class T, class Op, detail::enable_if_device<InIt> = 0>
+template <class InIt, class OutIt, class T, class Op, detail::enable_if_device<InIt, OutIt, T, Op> = 0>
 OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init, Op op) { return exclusive_scan(typename detail::implicit_policy<InIt>::type(), f, l, r, init, op); }
-template <class InIt, class OutIt, detail::enable_if_host<InIt> = 0>
+template <class InIt, class OutIt, detail::enable_if_host<InIt, OutIt> = 0>
 OutIt exclusive_scan(InIt f, InIt l, OutIt r) { return exclusive_scan(host, f, l, r); }
-template <class InIt, class OutIt, class T, detail::enable_if_host<InIt> = 0>
+template <class InIt, class OutIt, class T, detail::enable_if_host<InIt, OutIt, T> = 0>
 OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init) { return exclusive_scan(host, f, l, r, init); }
-template <class InIt, class OutIt, class T, class Op, detail::enable_if_host<InIt> = 0>
+template <class InIt, class OutIt, class T, class Op, detail::enable_if_host<InIt, OutIt, T, Op> = 0>
 OutIt exclusive_scan(InIt f, InIt l, OutIt r, T init, Op op) { return exclusive_scan(host, f, l, r, init, op); }
 
 // ===================================================================== scan_by_key, device

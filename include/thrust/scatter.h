@@ -50,12 +50,12 @@ void scatter_if(const system::cpp::detail::par_t&, In first, In last, Map map, S
 template <class Policy, class In, class Map, class S, class Out, detail::enable_if_policy<Policy> = 0>
 void scatter_if(const Policy& exec, In f, In l, Map m, S st, Out o) { scatter_if(exec, f, l, m, st, o, detail::truthy()); }
 
-template <class In, class Map, class Out, detail::enable_if_device<In> = 0> void scatter(In f, In l, Map m, Out o) { scatter(device, f, l, m, o); }
-template <class In, class Map, class Out, detail::enable_if_host<In> = 0> void scatter(In f, In l, Map m, Out o) { scatter(host, f, l, m, o); }
-template <class In, class Map, class S, class Out, detail::enable_if_device<In> = 0> void scatter_if(In f, In l, Map m, S st, Out o) { scatter_if(device, f, l, m, st, o); }
-template <class In, class Map, class S, class Out, detail::enable_if_host<In> = 0> void scatter_if(In f, In l, Map m, S st, Out o) { scatter_if(host, f, l, m, st, o); }
-template <class In, class Map, class S, class Out, class Pred, detail::enable_if_device<In> = 0>
+template <class In, class Map, class Out, detail::enable_if_device<In, Map, Out> = 0> void scatter(In f, In l, Map m, Out o) { scatter(device, f, l, m, o); }
+template <class In, class Map, class Out, detail::enable_if_host<In, Map, Out> = 0> void scatter(In f, In l, Map m, Out o) { scatter(host, f, l, m, o); }
+template <class In, class Map, class S, class Out, detail::enable_if_device<In, Map, S, Out> = 0> void scatter_if(In f, In l, Map m, S st, Out o) { scatter_if(device, f, l, m, st, o); }
+template <class In, class Map, class S, class Out, detail::enable_if_host<In, Map, S, Out> = 0> void scatter_if(In f, In l, Map m, S st, Out o) { scatter_if(host, f, l, m, st, o); }
+template <class In, class Map, class S, class Out, class Pred, detail::enable_if_device<In, Map, S, Out, Pred> = 0>
 void scatter_if(In f, In l, Map m, S st, Out o, Pred p) { scatter_if(device, f, l, m, st, o, p); }
-template <class In, class Map, class S, class Out, class Pred, detail::enable_if_host<In> = 0>
+template <class In, class Map, class S, class Out, class Pred, detail::enable_if_host<In, Map, S, Out, Pred> = 0>
 void scatter_if(In f, In l, Map m, S st, Out o, Pred p) { scatter_if(host, f, l, m, st, o, p); }
 }  // namespace thrust

@@ -29,8 +29,8 @@ void sequence(const Policy& exec, It first, It last) {
 
 template <class It, detail::enable_if_device<It> = 0> void sequence(It f, It l) { sequence(device, f, l); }
 template <class It, detail::enable_if_host<It> = 0> void sequence(It f, It l) { sequence(host, f, l); }
-template <class It, class T, detail::enable_if_device<It> = 0> void sequence(It f, It l, T init) { sequence(device, f, l, init); }
-template <class It, class T, detail::enable_if_host<It> = 0> void sequence(It f, It l, T init) { sequence(host, f, l, init); }
-template <class It, class T, detail::enable_if_device<It> = 0> void sequence(It f, It l, T init, T step) { sequence(device, f, l, init, step); }
-template <class It, class T, detail::enable_if_host<It> = 0> void sequence(It f, It l, T init, T step) { sequence(host, f, l, init, step); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> void sequence(It f, It l, T init) { sequence(device, f, l, init); }
+template <class It, class T, detail::enable_if_host<It, T> = 0> void sequence(It f, It l, T init) { sequence(host, f, l, init); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> void sequence(It f, It l, T init, T step) { sequence(device, f, l, init, step); }
+template <class It, class T, detail::enable_if_host<It, T> = 0> void sequence(It f, It l, T init, T step) { sequence(host, f, l, init, step); }
 }  // namespace thrust

@@ -184,17 +184,17 @@ void sort_by_key(const system::cpp::detail::par_t& e, KIt kfirst, KIt klast, VIt
 // ---- no policy: the iterator's system decides (thrust/detail/sort.inl:202-339) --------
 #define THRUST_CDNA4_SORT_DISPATCH(NAME)                                                                         \
   template <class It, detail::enable_if_device<It> = 0> void NAME(It f, It l) { NAME(typename detail::implicit_policy<It>::type(), f, l); }              \
-  template <class It, class C, detail::enable_if_device<It> = 0> void NAME(It f, It l, C c) { NAME(typename detail::implicit_policy<It>::type(), f, l, c); } \
+  template <class It, class C, detail::enable_if_device<It, C> = 0> void NAME(It f, It l, C c) { NAME(typename detail::implicit_policy<It>::type(), f, l, c); } \
   template <class It, detail::enable_if_host<It> = 0> void NAME(It f, It l) { NAME(host, f, l); }                  \
-  template <class It, class C, detail::enable_if_host<It> = 0> void NAME(It f, It l, C c) { NAME(host, f, l, c); }
+  template <class It, class C, detail::enable_if_host<It, C> = 0> void NAME(It f, It l, C c) { NAME(host, f, l, c); }
 THRUST_CDNA4_SORT_DISPATCH(sort)
 THRUST_CDNA4_SORT_DISPATCH(stable_sort)
 #undef THRUST_CDNA4_SORT_DISPATCH
 #define THRUST_CDNA4_SORT_BY_KEY_DISPATCH(NAME)                                                                  \
-  template <class K, class V, detail::enable_if_device<K> = 0> void NAME(K f, K l, V v) { NAME(typename detail::implicit_policy<K>::type(), f, l, v); }  \
-  template <class K, class V, class C, detail::enable_if_device<K> = 0> void NAME(K f, K l, V v, C c) { NAME(typename detail::implicit_policy<K>::type(), f, l, v, c); } \
-  template <class K, class V, detail::enable_if_host<K> = 0> void NAME(K f, K l, V v) { NAME(host, f, l, v); }      \
-  template <class K, class V, class C, detail::enable_if_host<K> = 0> void NAME(K f, K l, V v, C c) { NAME(host, f, l, v, c); }
+  template <class K, class V, detail::enable_if_device<K, V> = 0> void NAME(K f, K l, V v) { NAME(typename detail::implicit_policy<K>::type(), f, l, v); }  \
+  template <class K, class V, class C, detail::enable_if_device<K, V, C> = 0> void NAME(K f, K l, V v, C c) { NAME(typename detail::implicit_policy<K>::type(), f, l, v, c); } \
+  template <class K, class V, detail::enable_if_host<K, V> = 0> void NAME(K f, K l, V v) { NAME(host, f, l, v); }      \
+  template <class K, class V, class C, detail::enable_if_host<K, V, C> = 0> void NAME(K f, K l, V v, C c) { NAME(host, f, l, v, c); }
 THRUST_CDNA4_SORT_BY_KEY_DISPATCH(sort_by_key)
 THRUST_CDNA4_SORT_BY_KEY_DISPATCH(stable_sort_by_key)
 #undef THRUST_CDNA4_SORT_BY_KEY_DISPATCH
@@ -232,10 +232,10 @@ template <class Policy, class It, detail::enable_if_policy<Policy> = 0>
 bool is_sorted(const Policy& exec, It first, It last) { return is_sorted_until(exec, first, last, less<>()) == last; }
 template <class It, detail::enable_if_device<It> = 0> It is_sorted_until(It f, It l) { return is_sorted_until(device, f, l); }
 template <class It, detail::enable_if_host<It> = 0> It is_sorted_until(It f, It l) { return is_sorted_until(host, f, l); }
-template <class It, class C, detail::enable_if_device<It> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(device, f, l, c); }
-template <class It, class C, detail::enable_if_host<It> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(host, f, l, c); }
+template <class It, class C, detail::enable_if_device<It, C> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(device, f, l, c); }
+template <class It, class C, detail::enable_if_host<It, C> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(host, f, l, c); }
 template <class It, detail::enable_if_device<It> = 0> bool is_sorted(It f, It l) { return is_sorted(device, f, l); }
 template <class It, detail::enable_if_host<It> = 0> bool is_sorted(It f, It l) { return is_sorted(host, f, l); }
-template <class It, class C, detail::enable_if_device<It> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(device, f, l, c); }
-template <class It, class C, detail::enable_if_host<It> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(host, f, l, c); }
+template <class It, class C, detail::enable_if_device<It, C> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(device, f, l, c); }
+template <class It, class C, detail::enable_if_host<It, C> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(host, f, l, c); }
 }  // namespace thrust

@@ -75,7 +75,7 @@ void sort_pairs_impl(const Policy& exec, K* keys, V* values, std::int64_t n, Com
 
 template <class Policy, class K, class V, class Compare>
 void sort_pairs(const Policy& exec, K* keys, V* values, std::int64_t n, Compare comp) {
-  static_assert(std::is_trivially_copyable<V>::value, "cdna4 sort_by_key: values must be trivially copyable");
+  static_assert(thrust::detail::is_bytewise_movable<V>::value, "cdna4 sort_by_key: values must be movable as bytes");
   if (n <= 0) return;
   constexpr bool radix_value = sizeof(V) == 1 || sizeof(V) == 2 || sizeof(V) == 4 || sizeof(V) == 8;
   sort_pairs_impl(exec, keys, values, n, comp,

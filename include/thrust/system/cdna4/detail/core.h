@@ -91,6 +91,14 @@ inline const error_category& cdna4_category() {
 }
 
 namespace detail {
+// The element, key, value and accumulator types the device algorithms accept: those that may be
+// moved as bytes between host and device and through kernel arguments.  A trivially copyable type
+// is one; so is a number-like struct whose copy operations are written out but whose destructor is
+// trivial (the reference's own tests use such a type, testing/unittest/testframework.h:128-232):
+// its copy operations run where a kernel copies an element, and not where bytes are moved.
+template <class T> struct is_bytewise_movable
+    : std::integral_constant<bool, std::is_trivially_copyable<T>::value || std::is_trivially_destructible<T>::value> {};
+
 // The root of every execution policy (thrust/detail/execution_policy.h): the public entry points
 // that dispatch to a system's implementation take it, so that an overload for a nearer base — the
 // system's own, or a user's for a policy type of their own — is the better match.

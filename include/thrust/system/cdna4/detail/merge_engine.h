@@ -147,8 +147,8 @@ template <bool HAS_VALUES, class KA, class KB, class VA, class VB, class KO, cla
 void merge(void* stream_, KA a, std::int64_t na, KB b, std::int64_t nb, VA va, VB vb, KO kout, VO vout, Compare comp) {
   typedef typename std::iterator_traits<KA>::value_type K;
   typedef typename std::conditional<HAS_VALUES, typename std::iterator_traits<typename std::conditional<HAS_VALUES, VA, KA>::type>::value_type, char>::type V;
-  static_assert(std::is_trivially_copyable<K>::value && std::is_trivially_copyable<V>::value,
-                "cdna4 merge: keys and values must be trivially copyable");
+  static_assert(thrust::detail::is_bytewise_movable<K>::value && thrust::detail::is_bytewise_movable<V>::value,
+                "cdna4 merge: keys and values must be movable as bytes");
   constexpr int IPT = items_per_thread<K, HAS_VALUES ? sizeof(V) : 0>();
   constexpr int kTile = kBlock * IPT;
   static_assert((sizeof(K) + (HAS_VALUES ? sizeof(V) : 0)) * kTile <= 65536, "cdna4 merge: an item is too large for a tile in LDS");

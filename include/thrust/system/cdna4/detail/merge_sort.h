@@ -393,8 +393,8 @@ inline std::size_t align256(std::size_t x) { return (x + 255) & ~std::size_t(255
 
 template <class K, class V, class Compare>
 void stable_sort(void* stream_, K* keys, V* values, std::int64_t n, Compare comp) {
-  static_assert(std::is_trivially_copyable<K>::value, "cdna4 merge sort: keys must be trivially copyable");
-  static_assert(std::is_trivially_copyable<V>::value, "cdna4 merge sort: values must be trivially copyable");
+  static_assert(thrust::detail::is_bytewise_movable<K>::value, "cdna4 merge sort: keys must be movable as bytes");
+  static_assert(thrust::detail::is_bytewise_movable<V>::value, "cdna4 merge sort: values must be movable as bytes");
   constexpr int IPT = items_per_thread<K, V>();
   constexpr int kTile = kBlock * IPT;
   constexpr bool kHasValues = !std::is_same<V, no_value>::value;

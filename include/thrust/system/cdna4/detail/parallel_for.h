@@ -104,7 +104,7 @@ __global__ __launch_bounds__(kBlock) void reduce_final_kernel(const T* partial, 
 // without waiting (the asynchronous reductions; n == 0 stores init).
 template <class T, class Unary, class Op>
 void transform_reduce_into(void* stream_, std::int64_t n, Unary unary, T init, Op op, T* out) {
-  static_assert(std::is_trivially_copyable<T>::value, "cdna4 reduce: the result type must be trivially copyable");
+  static_assert(thrust::detail::is_bytewise_movable<T>::value, "cdna4 reduce: the result type must be movable as bytes");
   hipStream_t s = static_cast<hipStream_t>(stream_);
   std::int64_t blocks = (n + kBlock - 1) / kBlock;
   const std::int64_t enough = 2048;
@@ -121,7 +121,7 @@ void transform_reduce_into(void* stream_, std::int64_t n, Unary unary, T init, O
 // (thrust/system/cuda/detail/reduce.h:947-971 does the same).
 template <class T, class Unary, class Op>
 T transform_reduce(void* stream_, std::int64_t n, Unary unary, T init, Op op) {
-  static_assert(std::is_trivially_copyable<T>::value, "cdna4 reduce: the result type must be trivially copyable");
+  static_assert(thrust::detail::is_bytewise_movable<T>::value, "cdna4 reduce: the result type must be movable as bytes");
   if (n <= 0) return init;
   hipStream_t s = static_cast<hipStream_t>(stream_);
   std::int64_t blocks = (n + kBlock - 1) / kBlock;  // every workgroup gets at least one index

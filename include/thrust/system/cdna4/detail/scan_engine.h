@@ -314,7 +314,7 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
 template <class Op>
 void scan_engine(void* stream_, std::int64_t n, Op op) {
   typedef typename Op::acc Acc;
-  static_assert(std::is_trivially_copyable<Acc>::value, "cdna4 scan: the accumulator type must be trivially copyable");
+  static_assert(thrust::detail::is_bytewise_movable<Acc>::value, "cdna4 scan: the accumulator type must be movable as bytes");
   if (n <= 0) return;
   hipStream_t s = static_cast<hipStream_t>(stream_);
   constexpr std::int64_t kTile = (std::int64_t)kScanBlock * scan_items(sizeof(Acc)) * scan_parts(sizeof(Acc));

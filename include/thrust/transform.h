@@ -27,14 +27,14 @@ Out transform(const system::cpp::detail::par_t&, In1 first1, In1 last1, In2 firs
   return std::transform(first1, last1, first2, out, f);
 }
 
-template <class In, class Out, class F, detail::enable_if_device<In> = 0>
+template <class In, class Out, class F, detail::enable_if_device<In, Out, F> = 0>
 Out transform(In f, In l, Out o, F fn) { return transform(device, f, l, o, fn); }
-template <class In, class Out, class F, detail::enable_if_host<In> = 0>
+template <class In, class Out, class F, detail::enable_if_host<In, Out, F> = 0>
 Out transform(In f, In l, Out o, F fn) { return transform(host, f, l, o, fn); }
-template <class In1, class In2, class Out, class F, detail::enable_if_device<In1> = 0,
+template <class In1, class In2, class Out, class F, detail::enable_if_device<In1, In2, Out, F> = 0,
           class = typename std::iterator_traits<In2>::iterator_category>
 Out transform(In1 f, In1 l, In2 f2, Out o, F fn) { return transform(device, f, l, f2, o, fn); }
-template <class In1, class In2, class Out, class F, detail::enable_if_host<In1> = 0,
+template <class In1, class In2, class Out, class F, detail::enable_if_host<In1, In2, Out, F> = 0,
           class = typename std::iterator_traits<In2>::iterator_category>
 Out transform(In1 f, In1 l, In2 f2, Out o, F fn) { return transform(host, f, l, f2, o, fn); }
 

@@ -14,12 +14,12 @@ template <class Policy, class In, class Out, class UnaryOp, class T, class Binar
 Out transform_exclusive_scan(const Policy& exec, In first, In last, Out result, UnaryOp unary_op, T init, BinaryOp binary_op) {
   return exclusive_scan(exec, make_transform_iterator(first, unary_op), make_transform_iterator(last, unary_op), result, init, binary_op);
 }
-template <class In, class Out, class U, class B, detail::enable_if_device<In> = 0>
+template <class In, class Out, class U, class B, detail::enable_if_device<In, Out, U, B> = 0>
 Out transform_inclusive_scan(In f, In l, Out o, U u, B b) { return transform_inclusive_scan(device, f, l, o, u, b); }
-template <class In, class Out, class U, class B, detail::enable_if_host<In> = 0>
+template <class In, class Out, class U, class B, detail::enable_if_host<In, Out, U, B> = 0>
 Out transform_inclusive_scan(In f, In l, Out o, U u, B b) { return transform_inclusive_scan(host, f, l, o, u, b); }
-template <class In, class Out, class U, class T, class B, detail::enable_if_device<In> = 0>
+template <class In, class Out, class U, class T, class B, detail::enable_if_device<In, Out, U, T, B> = 0>
 Out transform_exclusive_scan(In f, In l, Out o, U u, T init, B b) { return transform_exclusive_scan(device, f, l, o, u, init, b); }
-template <class In, class Out, class U, class T, class B, detail::enable_if_host<In> = 0>
+template <class In, class Out, class U, class T, class B, detail::enable_if_host<In, Out, U, T, B> = 0>
 Out transform_exclusive_scan(In f, In l, Out o, U u, T init, B b) { return transform_exclusive_scan(host, f, l, o, u, init, b); }
 }  // namespace thrust

@@ -102,6 +102,70 @@ THRUST_CDNA4_HD constexpr tuple<typename std::decay<Ts>::type...> make_tuple(con
 }
 template <class... Ts>
 THRUST_CDNA4_HD constexpr tuple<Ts&...> tie(Ts&... vs) { return tuple<Ts&...>(vs...); }
+// The same two for a fixed number of arguments (thrust/tuple.h:190-260 declares them that way).
+// Called unqualified under `using namespace thrust` with arguments of std types — a host_vector's
+// iterators —, std::make_tuple and std::tie are candidates too; a function template without a
+// parameter pack is the more specialised one and is chosen.
+template <class T0>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type> make_tuple(T0&& v0) {
+  return tuple<typename std::decay<T0>::type>(static_cast<T0&&>(v0));
+}
+template <class T0, class T1>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type> make_tuple(T0&& v0, T1&& v1) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1));
+}
+template <class T0, class T1, class T2>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type> make_tuple(T0&& v0, T1&& v1, T2&& v2) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1), static_cast<T2&&>(v2));
+}
+template <class T0, class T1, class T2, class T3>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type> make_tuple(T0&& v0, T1&& v1, T2&& v2, T3&& v3) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1), static_cast<T2&&>(v2), static_cast<T3&&>(v3));
+}
+template <class T0, class T1, class T2, class T3, class T4>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type> make_tuple(T0&& v0, T1&& v1, T2&& v2, T3&& v3, T4&& v4) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1), static_cast<T2&&>(v2), static_cast<T3&&>(v3), static_cast<T4&&>(v4));
+}
+template <class T0, class T1, class T2, class T3, class T4, class T5>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type> make_tuple(T0&& v0, T1&& v1, T2&& v2, T3&& v3, T4&& v4, T5&& v5) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1), static_cast<T2&&>(v2), static_cast<T3&&>(v3), static_cast<T4&&>(v4), static_cast<T5&&>(v5));
+}
+template <class T0, class T1, class T2, class T3, class T4, class T5, class T6>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type, typename std::decay<T6>::type> make_tuple(T0&& v0, T1&& v1, T2&& v2, T3&& v3, T4&& v4, T5&& v5, T6&& v6) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type, typename std::decay<T6>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1), static_cast<T2&&>(v2), static_cast<T3&&>(v3), static_cast<T4&&>(v4), static_cast<T5&&>(v5), static_cast<T6&&>(v6));
+}
+template <class T0, class T1, class T2, class T3, class T4, class T5, class T6, class T7>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type, typename std::decay<T6>::type, typename std::decay<T7>::type> make_tuple(T0&& v0, T1&& v1, T2&& v2, T3&& v3, T4&& v4, T5&& v5, T6&& v6, T7&& v7) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type, typename std::decay<T6>::type, typename std::decay<T7>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1), static_cast<T2&&>(v2), static_cast<T3&&>(v3), static_cast<T4&&>(v4), static_cast<T5&&>(v5), static_cast<T6&&>(v6), static_cast<T7&&>(v7));
+}
+template <class T0, class T1, class T2, class T3, class T4, class T5, class T6, class T7, class T8>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type, typename std::decay<T6>::type, typename std::decay<T7>::type, typename std::decay<T8>::type> make_tuple(T0&& v0, T1&& v1, T2&& v2, T3&& v3, T4&& v4, T5&& v5, T6&& v6, T7&& v7, T8&& v8) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type, typename std::decay<T6>::type, typename std::decay<T7>::type, typename std::decay<T8>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1), static_cast<T2&&>(v2), static_cast<T3&&>(v3), static_cast<T4&&>(v4), static_cast<T5&&>(v5), static_cast<T6&&>(v6), static_cast<T7&&>(v7), static_cast<T8&&>(v8));
+}
+template <class T0, class T1, class T2, class T3, class T4, class T5, class T6, class T7, class T8, class T9>
+THRUST_CDNA4_HD constexpr tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type, typename std::decay<T6>::type, typename std::decay<T7>::type, typename std::decay<T8>::type, typename std::decay<T9>::type> make_tuple(T0&& v0, T1&& v1, T2&& v2, T3&& v3, T4&& v4, T5&& v5, T6&& v6, T7&& v7, T8&& v8, T9&& v9) {
+  return tuple<typename std::decay<T0>::type, typename std::decay<T1>::type, typename std::decay<T2>::type, typename std::decay<T3>::type, typename std::decay<T4>::type, typename std::decay<T5>::type, typename std::decay<T6>::type, typename std::decay<T7>::type, typename std::decay<T8>::type, typename std::decay<T9>::type>(static_cast<T0&&>(v0), static_cast<T1&&>(v1), static_cast<T2&&>(v2), static_cast<T3&&>(v3), static_cast<T4&&>(v4), static_cast<T5&&>(v5), static_cast<T6&&>(v6), static_cast<T7&&>(v7), static_cast<T8&&>(v8), static_cast<T9&&>(v9));
+}
+template <class T0>
+THRUST_CDNA4_HD constexpr tuple<T0&> tie(T0& v0) { return tuple<T0&>(v0); }
+template <class T0, class T1>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&> tie(T0& v0, T1& v1) { return tuple<T0&, T1&>(v0, v1); }
+template <class T0, class T1, class T2>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&> tie(T0& v0, T1& v1, T2& v2) { return tuple<T0&, T1&, T2&>(v0, v1, v2); }
+template <class T0, class T1, class T2, class T3>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&> tie(T0& v0, T1& v1, T2& v2, T3& v3) { return tuple<T0&, T1&, T2&, T3&>(v0, v1, v2, v3); }
+template <class T0, class T1, class T2, class T3, class T4>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&> tie(T0& v0, T1& v1, T2& v2, T3& v3, T4& v4) { return tuple<T0&, T1&, T2&, T3&, T4&>(v0, v1, v2, v3, v4); }
+template <class T0, class T1, class T2, class T3, class T4, class T5>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&, T5&> tie(T0& v0, T1& v1, T2& v2, T3& v3, T4& v4, T5& v5) { return tuple<T0&, T1&, T2&, T3&, T4&, T5&>(v0, v1, v2, v3, v4, v5); }
+template <class T0, class T1, class T2, class T3, class T4, class T5, class T6>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&> tie(T0& v0, T1& v1, T2& v2, T3& v3, T4& v4, T5& v5, T6& v6) { return tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&>(v0, v1, v2, v3, v4, v5, v6); }
+template <class T0, class T1, class T2, class T3, class T4, class T5, class T6, class T7>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&> tie(T0& v0, T1& v1, T2& v2, T3& v3, T4& v4, T5& v5, T6& v6, T7& v7) { return tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&>(v0, v1, v2, v3, v4, v5, v6, v7); }
+template <class T0, class T1, class T2, class T3, class T4, class T5, class T6, class T7, class T8>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&> tie(T0& v0, T1& v1, T2& v2, T3& v3, T4& v4, T5& v5, T6& v6, T7& v7, T8& v8) { return tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&>(v0, v1, v2, v3, v4, v5, v6, v7, v8); }
+template <class T0, class T1, class T2, class T3, class T4, class T5, class T6, class T7, class T8, class T9>
+THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&, T9&> tie(T0& v0, T1& v1, T2& v2, T3& v3, T4& v4, T5& v5, T6& v6, T7& v7, T8& v8, T9& v9) { return tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&, T9&>(v0, v1, v2, v3, v4, v5, v6, v7, v8, v9); }
 
 template <class... Ts, class... Us>
 THRUST_CDNA4_HD constexpr bool operator==(const tuple<Ts...>& a, const tuple<Us...>& b) {

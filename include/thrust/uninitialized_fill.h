@@ -20,8 +20,8 @@ It uninitialized_fill_n(const Policy& exec, It first, Size n, const T& x) {
   uninitialized_fill(exec, first, first + n, x);
   return first + n;
 }
-template <class It, class T, detail::enable_if_device<It> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(device, f, l, x); }
-template <class It, class T, detail::enable_if_host<It> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(host, f, l, x); }
-template <class It, class Size, class T, detail::enable_if_device<It> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(device, f, n, x); }
-template <class It, class Size, class T, detail::enable_if_host<It> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(host, f, n, x); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(device, f, l, x); }
+template <class It, class T, detail::enable_if_host<It, T> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(host, f, l, x); }
+template <class It, class Size, class T, detail::enable_if_device<It, Size, T> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(device, f, n, x); }
+template <class It, class Size, class T, detail::enable_if_host<It, Size, T> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(host, f, n, x); }
 }  // namespace thrust

@@ -69,25 +69,25 @@ pair<KOut, VOut> unique_by_key_copy(const Policy& exec, KIn kfirst, KIn klast, V
 // ---- no policy
 template <class In, detail::enable_if_device<In> = 0> In unique(In f, In l) { return unique(device, f, l); }
 template <class In, detail::enable_if_host<In> = 0> In unique(In f, In l) { return unique(host, f, l); }
-template <class In, class Eq, detail::enable_if_device<In> = 0> In unique(In f, In l, Eq eq) { return unique(device, f, l, eq); }
-template <class In, class Eq, detail::enable_if_host<In> = 0> In unique(In f, In l, Eq eq) { return unique(host, f, l, eq); }
-template <class In, class Out, detail::enable_if_device<In> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(device, f, l, o); }
-template <class In, class Out, detail::enable_if_host<In> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(host, f, l, o); }
-template <class K, class V, detail::enable_if_device<K> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(device, f, l, v); }
-template <class K, class V, detail::enable_if_host<K> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(host, f, l, v); }
-template <class In, class Out, class Eq, detail::enable_if_device<In> = 0, class = typename std::iterator_traits<Out>::iterator_category>
+template <class In, class Eq, detail::enable_if_device<In, Eq> = 0> In unique(In f, In l, Eq eq) { return unique(device, f, l, eq); }
+template <class In, class Eq, detail::enable_if_host<In, Eq> = 0> In unique(In f, In l, Eq eq) { return unique(host, f, l, eq); }
+template <class In, class Out, detail::enable_if_device<In, Out> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(device, f, l, o); }
+template <class In, class Out, detail::enable_if_host<In, Out> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(host, f, l, o); }
+template <class K, class V, detail::enable_if_device<K, V> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(device, f, l, v); }
+template <class K, class V, detail::enable_if_host<K, V> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(host, f, l, v); }
+template <class In, class Out, class Eq, detail::enable_if_device<In, Out, Eq> = 0, class = typename std::iterator_traits<Out>::iterator_category>
 Out unique_copy(In f, In l, Out o, Eq eq) { return unique_copy(device, f, l, o, eq); }
-template <class In, class Out, class Eq, detail::enable_if_host<In> = 0, class = typename std::iterator_traits<Out>::iterator_category>
+template <class In, class Out, class Eq, detail::enable_if_host<In, Out, Eq> = 0, class = typename std::iterator_traits<Out>::iterator_category>
 Out unique_copy(In f, In l, Out o, Eq eq) { return unique_copy(host, f, l, o, eq); }
-template <class K, class V, class Eq, detail::enable_if_device<K> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(device, f, l, v, eq); }
-template <class K, class V, class Eq, detail::enable_if_host<K> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(host, f, l, v, eq); }
-template <class K, class V, class KO, class VO, class Eq, detail::enable_if_device<K> = 0>
+template <class K, class V, class Eq, detail::enable_if_device<K, V, Eq> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(device, f, l, v, eq); }
+template <class K, class V, class Eq, detail::enable_if_host<K, V, Eq> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(host, f, l, v, eq); }
+template <class K, class V, class KO, class VO, class Eq, detail::enable_if_device<K, V, KO, VO, Eq> = 0>
 pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo, Eq eq) { return unique_by_key_copy(device, f, l, v, ko, vo, eq); }
-template <class K, class V, class KO, class VO, class Eq, detail::enable_if_host<K> = 0>
+template <class K, class V, class KO, class VO, class Eq, detail::enable_if_host<K, V, KO, VO, Eq> = 0>
 pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo, Eq eq) { return unique_by_key_copy(host, f, l, v, ko, vo, eq); }
-template <class K, class V, class KO, class VO, detail::enable_if_device<K> = 0>
+template <class K, class V, class KO, class VO, detail::enable_if_device<K, V, KO, VO> = 0>
 pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(device, f, l, v, ko, vo); }
-template <class K, class V, class KO, class VO, detail::enable_if_host<K> = 0>
+template <class K, class V, class KO, class VO, detail::enable_if_host<K, V, KO, VO> = 0>
 pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(host, f, l, v, ko, vo); }
 
 // ---- unique_count (thrust/unique.h:1022-1176): the number of runs of consecutive equivalent
@@ -115,8 +115,8 @@ typename std::iterator_traits<It>::difference_type unique_count(const Policy& ex
 }
 template <class It, detail::enable_if_device<It> = 0> typename std::iterator_traits<It>::difference_type unique_count(It f, It l) { return unique_count(device, f, l); }
 template <class It, detail::enable_if_host<It> = 0> typename std::iterator_traits<It>::difference_type unique_count(It f, It l) { return unique_count(host, f, l); }
-template <class It, class Eq, detail::enable_if_device<It> = 0, typename std::enable_if<!detail::is_policy<It>::value, int>::type = 0>
+template <class It, class Eq, detail::enable_if_device<It, Eq> = 0, typename std::enable_if<!detail::is_policy<It>::value, int>::type = 0>
 typename std::iterator_traits<It>::difference_type unique_count(It f, It l, Eq eq) { return unique_count(device, f, l, eq); }
-template <class It, class Eq, detail::enable_if_host<It> = 0, typename std::enable_if<!detail::is_policy<It>::value, int>::type = 0>
+template <class It, class Eq, detail::enable_if_host<It, Eq> = 0, typename std::enable_if<!detail::is_policy<It>::value, int>::type = 0>
 typename std::iterator_traits<It>::difference_type unique_count(It f, It l, Eq eq) { return unique_count(host, f, l, eq); }
 }  // namespace thrust
