@@ -27,15 +27,25 @@ template <class In, class Out, class Op>
 Out adjacent_difference(const system::cpp::detail::par_t&, In first, In last, Out out, Op op) {
   return std::adjacent_difference(first, last, out, op);
 }
-template <class Policy, class In, class Out, detail::enable_if_policy<Policy> = 0>
-Out adjacent_difference(const Policy& exec, In first, In last, Out out) {
+namespace detail {
+template <class Policy, class In, class Out>
+Out composed_adjacent_difference(const Policy& exec, In first, In last, Out out) {
   return adjacent_difference(exec, first, last, out, minus<typename detail::value_of<In>::type>());
 }
-template <class In, class Out, detail::enable_if_device<In, Out> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(device, f, l, o); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In, class Out>
+Out adjacent_difference(execution_policy<D_>& exec, In first, In last, Out out) { return thrust::detail::composed_adjacent_difference(exec, first, last, out); }
+}}  // namespace system::cdna4
+template <class D_, class In, class Out>
+Out adjacent_difference(const detail::execution_policy_base<D_>& exec, In first, In last, Out out) { return adjacent_difference(detail::derived_cast(detail::strip_const(exec)), first, last, out); }
+template <class In, class Out>
+Out adjacent_difference(const system::cpp::detail::par_t& exec, In first, In last, Out out) { return detail::composed_adjacent_difference(exec, first, last, out); }
+template <class In, class Out, detail::enable_if_device<In, Out> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(typename detail::implicit_policy<In, Out>::type(), f, l, o); }
 template <class In, class Out, detail::enable_if_host<In, Out> = 0> Out adjacent_difference(In f, In l, Out o) { return adjacent_difference(host, f, l, o); }
 template <class In, class Out, class Op, detail::enable_if_device<In, Out, Op> = 0,
           class = typename std::iterator_traits<Out>::iterator_category>
-Out adjacent_difference(In f, In l, Out o, Op op) { return adjacent_difference(device, f, l, o, op); }
+Out adjacent_difference(In f, In l, Out o, Op op) { return adjacent_difference(typename detail::implicit_policy<In, Out, Op>::type(), f, l, o, op); }
 template <class In, class Out, class Op, detail::enable_if_host<In, Out, Op> = 0,
           class = typename std::iterator_traits<Out>::iterator_category>
 Out adjacent_difference(In f, In l, Out o, Op op) { return adjacent_difference(host, f, l, o, op); }

@@ -55,13 +55,13 @@ std::ptrdiff_t scalar_search(const system::cpp::detail::par_t&, Hay first, Hay l
   }                                                                                                                      \
   template <class Hay, class Needles, class Out, detail::enable_if_device<Hay, Needles, Out> = 0,                                      \
             class = typename std::iterator_traits<Out>::iterator_category>                                               \
-  Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o) { return NAME(device, f, l, vf, vl, o); }                        \
+  Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o) { return NAME(typename detail::implicit_policy<Hay, Needles, Out>::type(), f, l, vf, vl, o); }                        \
   template <class Hay, class Needles, class Out, detail::enable_if_host<Hay, Needles, Out> = 0,                                        \
             class = typename std::iterator_traits<Out>::iterator_category>                                               \
   Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o) { return NAME(host, f, l, vf, vl, o); }                          \
   template <class Hay, class Needles, class Out, class Comp, detail::enable_if_device<Hay, Needles, Out, Comp> = 0,                          \
             class = typename std::iterator_traits<Out>::iterator_category>                                               \
-  Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o, Comp c) { return NAME(device, f, l, vf, vl, o, c); }             \
+  Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o, Comp c) { return NAME(typename detail::implicit_policy<Hay, Needles, Out, Comp>::type(), f, l, vf, vl, o, c); }             \
   template <class Hay, class Needles, class Out, class Comp, detail::enable_if_host<Hay, Needles, Out, Comp> = 0,                            \
             class = typename std::iterator_traits<Out>::iterator_category>                                               \
   Out NAME(Hay f, Hay l, Needles vf, Needles vl, Out o, Comp c) { return NAME(host, f, l, vf, vl, o, c); }
@@ -80,7 +80,7 @@ THRUST_CDNA4_SEARCH(binary_search, 2)
   Hay NAME(const Policy& exec, Hay first, Hay last, const T& value) {                                                    \
     return first + detail::scalar_search<MODE>(exec, first, last, value, less<T>());                                     \
   }                                                                                                                      \
-  template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(device, f, l, v); } \
+  template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(typename detail::implicit_policy<Hay, T>::type(), f, l, v); } \
   template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(host, f, l, v); }
 THRUST_CDNA4_SCALAR_BOUND(lower_bound, 0)
 THRUST_CDNA4_SCALAR_BOUND(upper_bound, 1)
@@ -93,7 +93,7 @@ template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0
 bool binary_search(const Policy& exec, Hay first, Hay last, const T& value) {
   return detail::scalar_search<2>(exec, first, last, value, less<T>()) != 0;
 }
-template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(device, f, l, v); }
+template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(typename detail::implicit_policy<Hay, T>::type(), f, l, v); }
 template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(host, f, l, v); }
 
 // ---- equal_range (thrust/binary_search.h:727-1017): the pair (lower_bound, upper_bound) of one value
@@ -106,10 +106,10 @@ template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0
 pair<Hay, Hay> equal_range(const Policy& exec, Hay first, Hay last, const T& value) {
   return equal_range(exec, first, last, value, less<T>());
 }
-template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(device, f, l, v); }
+template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(typename detail::implicit_policy<Hay, T>::type(), f, l, v); }
 template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(host, f, l, v); }
 template <class Hay, class T, class Comp, detail::enable_if_device<Hay, T, Comp> = 0, typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>
-pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v, Comp c) { return equal_range(device, f, l, v, c); }
+pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v, Comp c) { return equal_range(typename detail::implicit_policy<Hay, T, Comp>::type(), f, l, v, c); }
 template <class Hay, class T, class Comp, detail::enable_if_host<Hay, T, Comp> = 0, typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>
 pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v, Comp c) { return equal_range(host, f, l, v, c); }
 }  // namespace thrust

@@ -74,11 +74,11 @@ Out copy_if(const system::cpp::detail::par_t&, In first, In last, St stencil, Ou
   for (; first != last; ++first, ++stencil) if (pred(*stencil)) { *out = *first; ++out; }
   return out;
 }
-template <class In, class Out, class Pred, detail::enable_if_device<In, Out, Pred> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(device, f, l, o, p); }
+template <class In, class Out, class Pred, detail::enable_if_device<In, Out, Pred> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(typename detail::implicit_policy<In, Out, Pred>::type(), f, l, o, p); }
 template <class In, class Out, class Pred, detail::enable_if_host<In, Out, Pred> = 0> Out copy_if(In f, In l, Out o, Pred p) { return copy_if(host, f, l, o, p); }
 template <class In, class St, class Out, class Pred, detail::enable_if_device<In, St, Out, Pred> = 0,
           class = typename std::iterator_traits<St>::iterator_category>
-Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(device, f, l, s, o, p); }
+Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(typename detail::implicit_policy<In, St, Out, Pred>::type(), f, l, s, o, p); }
 template <class In, class St, class Out, class Pred, detail::enable_if_host<In, St, Out, Pred> = 0,
           class = typename std::iterator_traits<St>::iterator_category>
 Out copy_if(In f, In l, St s, Out o, Pred p) { return copy_if(host, f, l, s, o, p); }
@@ -121,8 +121,18 @@ Out copy(In first, In last, Out out) {
   system::cdna4::detail::copy_bytes(host.data(), tmp, n * sizeof(V), 1);
   return std::copy(host.begin(), host.end(), out);
 }
-template <class Policy, class In, class Size, class Out, detail::enable_if_policy<Policy> = 0>
-Out copy_n(const Policy& exec, In first, Size n, Out out) { return thrust::copy(exec, first, first + n, out); }
+namespace detail {
+template <class Policy, class In, class Size, class Out>
+Out composed_copy_n(const Policy& exec, In first, Size n, Out out) { return thrust::copy(exec, first, first + n, out); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In, class Size, class Out>
+Out copy_n(execution_policy<D_>& exec, In first, Size n, Out out) { return thrust::detail::composed_copy_n(exec, first, n, out); }
+}}  // namespace system::cdna4
+template <class D_, class In, class Size, class Out>
+Out copy_n(const detail::execution_policy_base<D_>& exec, In first, Size n, Out out) { return copy_n(detail::derived_cast(detail::strip_const(exec)), first, n, out); }
+template <class In, class Size, class Out>
+Out copy_n(const system::cpp::detail::par_t& exec, In first, Size n, Out out) { return detail::composed_copy_n(exec, first, n, out); }
 template <class In, class Size, class Out, typename std::enable_if<!detail::is_policy<In>::value, int>::type = 0>
 Out copy_n(In first, Size n, Out out) { return thrust::copy(first, first + n, out); }
 }  // namespace thrust

@@ -22,8 +22,8 @@ template <class Policy, class It, class V, class = typename std::iterator_traits
 std::ptrdiff_t count(const Policy& exec, It first, It last, const V& value) {
   return count_if(exec, first, last, detail::equals_value<V>{value});
 }
-template <class It, class Pred, detail::enable_if_device<It, Pred> = 0> std::ptrdiff_t count_if(It f, It l, Pred p) { return count_if(device, f, l, p); }
+template <class It, class Pred, detail::enable_if_device<It, Pred> = 0> std::ptrdiff_t count_if(It f, It l, Pred p) { return count_if(typename detail::implicit_policy<It, Pred>::type(), f, l, p); }
 template <class It, class Pred, detail::enable_if_host<It, Pred> = 0> std::ptrdiff_t count_if(It f, It l, Pred p) { return count_if(host, f, l, p); }
-template <class It, class V, detail::enable_if_device<It, V> = 0> std::ptrdiff_t count(It f, It l, const V& v) { return count(device, f, l, v); }
+template <class It, class V, detail::enable_if_device<It, V> = 0> std::ptrdiff_t count(It f, It l, const V& v) { return count(typename detail::implicit_policy<It, V>::type(), f, l, v); }
 template <class It, class V, detail::enable_if_host<It, V> = 0> std::ptrdiff_t count(It f, It l, const V& v) { return count(host, f, l, v); }
 }  // namespace thrust

@@ -34,9 +34,10 @@ template <class P> using enable_if_policy = typename std::enable_if<is_policy<P>
 // (thrust::retag<my_tag>(it), my_tag derived from thrust::device_execution_policy<my_tag>), a
 // default-constructed object of that type, so that the user's overloads for it are found.
 template <class Iterator, class Tag> class tagged_iterator;
-template <class It> struct implicit_policy { typedef system::cdna4::detail::par_t type; };
-template <class I, class Tag> struct implicit_policy<tagged_iterator<I, Tag>> {
+template <class... Args> struct implicit_policy { typedef system::cdna4::detail::par_t type; };
+template <class A, class... R> struct implicit_policy<A, R...> : implicit_policy<R...> {};
+template <class I, class Tag, class... R> struct implicit_policy<tagged_iterator<I, Tag>, R...> {
   typedef typename std::conditional<std::is_base_of<system::cdna4::execution_policy<Tag>, Tag>::value, Tag,
-                                    system::cdna4::detail::par_t>::type type;
+                                    typename implicit_policy<R...>::type>::type type;
 };
 }}  // namespace thrust::detail

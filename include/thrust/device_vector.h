@@ -48,7 +48,15 @@ class device_vector {
   device_vector(size_type n, const T& v) : device_vector() { assign(n, v); }
   device_vector(const device_vector& o) : device_vector(o.alloc_) { assign_device(o.p_, o.n_); }
   device_vector(device_vector&& o) noexcept : p_(o.p_), n_(o.n_), cap_(o.cap_), alloc_(o.alloc_) { o.p_ = nullptr; o.n_ = o.cap_ = 0; }
-  template <class A> device_vector(const std::vector<T, A>& h) : device_vector() { assign_host(h.data(), h.size()); }
+  // from a vector of either system, of this or a convertible element type
+  template <class U, class A> device_vector(const std::vector<U, A>& h) : device_vector() { assign(h.begin(), h.end()); }
+  template <class U, class A> device_vector(const host_vector<U, A>& h) : device_vector() { assign(h.begin(), h.end()); }
+  template <class U, class A> device_vector(const device_vector<U, A>& d) : device_vector() { assign(d.begin(), d.end()); }
+  device_vector(const device_vector& o, const Alloc& alloc) : device_vector(alloc) { assign_device(o.p_, o.n_); }
+  device_vector(std::initializer_list<T> il, const Alloc& alloc) : device_vector(alloc) { assign_host(il.begin(), il.size()); }
+  template <class It, class = typename std::iterator_traits<It>::iterator_category>
+  device_vector(It first, It last, const Alloc& alloc) : device_vector(alloc) { assign(first, last); }
+  device_vector(size_type n, const Alloc& alloc) : device_vector(alloc) { resize(n); }
   device_vector(std::initializer_list<T> il) : device_vector() { assign_host(il.begin(), il.size()); }
   template <class It, class = typename std::iterator_traits<It>::iterator_category>
   device_vector(It first, It last) : device_vector() { assign(first, last); }
@@ -56,7 +64,10 @@ class device_vector {
 
   device_vector& operator=(const device_vector& o) { if (this != &o) assign_device(o.p_, o.n_); return *this; }
   device_vector& operator=(device_vector&& o) noexcept { swap(o); return *this; }
-  template <class A> device_vector& operator=(const std::vector<T, A>& h) { assign_host(h.data(), h.size()); return *this; }
+  template <class U, class A> device_vector& operator=(const std::vector<U, A>& h) { assign(h.begin(), h.end()); return *this; }
+  template <class U, class A> device_vector& operator=(const host_vector<U, A>& h) { assign(h.begin(), h.end()); return *this; }
+  template <class U, class A> device_vector& operator=(const device_vector<U, A>& d) { assign(d.begin(), d.end()); return *this; }
+  device_vector& operator=(std::initializer_list<T> il) { assign_host(il.begin(), il.size()); return *this; }
 
   iterator begin() { return iterator(p_); }
   iterator end() { return iterator(p_ + n_); }
@@ -97,7 +108,9 @@ class device_vector {
   }
   void assign(size_type n, const T& v) { n_ = 0; if (n > cap_) regrow(n); fill_raw(p_, n, v); n_ = n; }
   template <class It, class = typename std::iterator_traits<It>::iterator_category>
-  void assign(It first, It last) { assign_range(first, last, typename std::is_same<It, iterator>::type()); }
+  void assign(It first, It last) {
+    assign_range(first, last, std::integral_constant<bool, std::is_same<It, iterator>::value || std::is_same<It, const_iterator>::value>());
+  }
   void pop_back() { --n_; }
   void shrink_to_fit() {
     if (n_ == cap_) return;
@@ -136,9 +149,11 @@ class device_vector {
     n_ = total;
     return begin() + at;
   }
-  iterator insert(iterator pos, const T& v) {
-    const T one[1] = {v};
-    return insert(pos, one, one + 1);
+  iterator insert(iterator pos, const T& v) { return insert(pos, (size_type)1, v); }
+  iterator insert(iterator pos, size_type n, const T& v) {
+    const size_type at = (size_type)(pos - begin());
+    device_vector added(n, v, alloc_);
+    return insert(begin() + at, added.begin(), added.end());
   }
   void push_back(const T& v) {
     if (n_ == cap_) regrow(cap_ ? 2 * cap_ : 16);
@@ -146,10 +161,6 @@ class device_vector {
     ++n_;
   }
 
-  friend bool operator==(const device_vector& a, const device_vector& b) {
-    return host_vector<T>(a) == host_vector<T>(b);
-  }
-  friend bool operator!=(const device_vector& a, const device_vector& b) { return !(a == b); }
 
  private:
   static void check(int rc, const char* what) { system::cdna4::detail::throw_on_error(rc, what); }
@@ -167,7 +178,7 @@ class device_vector {
     if (sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8) {
       check(thrust_cdna4_fill(dst, &v, (int)sizeof(T), (int64_t)n, nullptr), "device_vector: fill");
     } else {  // other element sizes (user structs): staged through the host
-      const std::vector<T> tmp(n, v);
+      const host_vector<T> tmp(n, v);
       check(thrust_cdna4_memcpy_htod(dst, tmp.data(), n * sizeof(T), nullptr), "device_vector: fill");
     }
     sync();
@@ -185,8 +196,10 @@ class device_vector {
     n_ = n;
   }
   template <class It> void assign_range(It first, It last, std::true_type) { assign_device(first.get(), (size_type)(last - first)); }
+  // any other range, in host or in device memory, of this or a convertible element type: through
+  // a host_vector, which reads a device range by the device system's copy
   template <class It> void assign_range(It first, It last, std::false_type) {
-    std::vector<T> tmp(first, last);
+    const host_vector<T> tmp(first, last);
     assign_host(tmp.data(), tmp.size());
   }
 
@@ -195,35 +208,28 @@ class device_vector {
   Alloc alloc_;
 };
 
-template <class T, class A>
-template <class DA>
-host_vector<T, A>::host_vector(const device_vector<T, DA>& d) : base(d.size()) {
-  if (d.size()) {
-    system::cdna4::detail::throw_on_error(
-        thrust_cdna4_memcpy_dtoh(this->data(), d.begin().get(), d.size() * sizeof(T), nullptr), "copy to host");
-    system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "copy to host");
-  }
-}
-template <class T, class A>
-template <class U>
-host_vector<T, A>::host_vector(device_ptr<U> first, device_ptr<U> last) : base((std::size_t)(last - first)) {
-  const std::size_t n = (std::size_t)(last - first);
-  if (!n) return;
-  if (std::is_same<typename std::remove_const<U>::type, T>::value) {
-    system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_dtoh(this->data(), first.get(), n * sizeof(T), nullptr), "copy to host");
-    system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "copy to host");
-  } else {  // another element type: through a host copy of the source, converted element by element
-    host_vector<typename std::remove_const<U>::type> same(first, last);
-    for (std::size_t i = 0; i < n; i++) (*this)[i] = (T)same[i];
-  }
-}
-template <class T, class A>
-template <class DA>
-host_vector<T, A>& host_vector<T, A>::operator=(const device_vector<T, DA>& d) {
-  host_vector tmp(d);
-  this->swap(tmp);
-  return *this;
-}
+// equality across the two vector kinds, element types and allocators (thrust/detail/vector_base.h:588-622)
+template <class T1, class A1, class T2, class A2>
+bool operator==(const device_vector<T1, A1>& a, const device_vector<T2, A2>& b) { return host_vector<T1>(a) == host_vector<T2>(b); }
+template <class T1, class A1, class T2, class A2>
+bool operator==(const device_vector<T1, A1>& a, const host_vector<T2, A2>& b) { return host_vector<T1>(a) == b; }
+template <class T1, class A1, class T2, class A2>
+bool operator==(const host_vector<T1, A1>& a, const device_vector<T2, A2>& b) { return a == host_vector<T2>(b); }
+template <class T1, class A1, class T2, class A2>
+bool operator==(const device_vector<T1, A1>& a, const std::vector<T2, A2>& b) { return host_vector<T1>(a) == b; }
+template <class T1, class A1, class T2, class A2>
+bool operator==(const std::vector<T1, A1>& a, const device_vector<T2, A2>& b) { return a == host_vector<T2>(b); }
+template <class T1, class A1, class T2, class A2>
+bool operator!=(const device_vector<T1, A1>& a, const device_vector<T2, A2>& b) { return !(a == b); }
+template <class T1, class A1, class T2, class A2>
+bool operator!=(const device_vector<T1, A1>& a, const host_vector<T2, A2>& b) { return !(a == b); }
+template <class T1, class A1, class T2, class A2>
+bool operator!=(const host_vector<T1, A1>& a, const device_vector<T2, A2>& b) { return !(a == b); }
+template <class T1, class A1, class T2, class A2>
+bool operator!=(const device_vector<T1, A1>& a, const std::vector<T2, A2>& b) { return !(a == b); }
+template <class T1, class A1, class T2, class A2>
+bool operator!=(const std::vector<T1, A1>& a, const device_vector<T2, A2>& b) { return !(a == b); }
+template <class T, class A> void swap(device_vector<T, A>& a, device_vector<T, A>& b) noexcept { a.swap(b); }
 
 }  // namespace thrust
 

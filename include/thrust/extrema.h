@@ -72,9 +72,9 @@ pair<It, It> minmax_element(const system::cpp::detail::par_t&, It first, It last
 }
 #define THRUST_CDNA4_EXTREMA(NAME, RET)                                                                                     \
   template <class Policy, class It, detail::enable_if_policy<Policy> = 0> RET NAME(const Policy& exec, It f, It l) { return NAME(exec, f, l, less<>()); } \
-  template <class It, detail::enable_if_device<It> = 0> RET NAME(It f, It l) { return NAME(device, f, l); }                    \
+  template <class It, detail::enable_if_device<It> = 0> RET NAME(It f, It l) { return NAME(typename detail::implicit_policy<It>::type(), f, l); }                    \
   template <class It, detail::enable_if_host<It> = 0> RET NAME(It f, It l) { return NAME(host, f, l); }                        \
-  template <class It, class C, detail::enable_if_device<It, C> = 0> RET NAME(It f, It l, C c) { return NAME(device, f, l, c); }  \
+  template <class It, class C, detail::enable_if_device<It, C> = 0> RET NAME(It f, It l, C c) { return NAME(typename detail::implicit_policy<It, C>::type(), f, l, c); }  \
   template <class It, class C, detail::enable_if_host<It, C> = 0> RET NAME(It f, It l, C c) { return NAME(host, f, l, c); }
 THRUST_CDNA4_EXTREMA(min_element, It)
 THRUST_CDNA4_EXTREMA(max_element, It)

@@ -47,13 +47,23 @@ void fill(const detail::execution_policy_base<D>& exec, It first, It last, const
 }
 template <class It, class V>
 void fill(const system::cpp::detail::par_t&, It first, It last, const V& value) { std::fill(first, last, value); }
-template <class Policy, class It, class Size, class V, detail::enable_if_policy<Policy> = 0>
-It fill_n(const Policy& exec, It first, Size n, const V& value) {
+namespace detail {
+template <class Policy, class It, class Size, class V>
+It composed_fill_n(const Policy& exec, It first, Size n, const V& value) {
   fill(exec, first, first + n, value);
   return first + n;
 }
-template <class It, class V, detail::enable_if_device<It, V> = 0> void fill(It f, It l, const V& v) { fill(device, f, l, v); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class Size, class V>
+It fill_n(execution_policy<D_>& exec, It first, Size n, const V& value) { return thrust::detail::composed_fill_n(exec, first, n, value); }
+}}  // namespace system::cdna4
+template <class D_, class It, class Size, class V>
+It fill_n(const detail::execution_policy_base<D_>& exec, It first, Size n, const V& value) { return fill_n(detail::derived_cast(detail::strip_const(exec)), first, n, value); }
+template <class It, class Size, class V>
+It fill_n(const system::cpp::detail::par_t& exec, It first, Size n, const V& value) { return detail::composed_fill_n(exec, first, n, value); }
+template <class It, class V, detail::enable_if_device<It, V> = 0> void fill(It f, It l, const V& v) { fill(typename detail::implicit_policy<It, V>::type(), f, l, v); }
 template <class It, class V, detail::enable_if_host<It, V> = 0> void fill(It f, It l, const V& v) { fill(host, f, l, v); }
-template <class It, class Size, class V, detail::enable_if_device<It, Size, V> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(device, f, n, v); }
+template <class It, class Size, class V, detail::enable_if_device<It, Size, V> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(typename detail::implicit_policy<It, Size, V>::type(), f, n, v); }
 template <class It, class Size, class V, detail::enable_if_host<It, Size, V> = 0> It fill_n(It f, Size n, const V& v) { return fill_n(host, f, n, v); }
 }  // namespace thrust

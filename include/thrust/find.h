@@ -44,13 +44,23 @@ It find_if_not(const detail::execution_policy_base<D>& exec, It first, It last, 
 }
 template <class It, class Pred> It find_if(const system::cpp::detail::par_t&, It first, It last, Pred pred) { return std::find_if(first, last, pred); }
 template <class It, class Pred> It find_if_not(const system::cpp::detail::par_t&, It first, It last, Pred pred) { return std::find_if_not(first, last, pred); }
-template <class Policy, class It, class T, detail::enable_if_policy<Policy> = 0>
-It find(const Policy& exec, It first, It last, const T& value) { return find_if(exec, first, last, detail::equals_value<T>{value}); }
+namespace detail {
+template <class Policy, class It, class T>
+It composed_find(const Policy& exec, It first, It last, const T& value) { return find_if(exec, first, last, detail::equals_value<T>{value}); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class T>
+It find(execution_policy<D_>& exec, It first, It last, const T& value) { return thrust::detail::composed_find(exec, first, last, value); }
+}}  // namespace system::cdna4
+template <class D_, class It, class T>
+It find(const detail::execution_policy_base<D_>& exec, It first, It last, const T& value) { return find(detail::derived_cast(detail::strip_const(exec)), first, last, value); }
+template <class It, class T>
+It find(const system::cpp::detail::par_t& exec, It first, It last, const T& value) { return detail::composed_find(exec, first, last, value); }
 
-template <class It, class T, detail::enable_if_device<It, T> = 0> It find(It f, It l, const T& v) { return find(device, f, l, v); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> It find(It f, It l, const T& v) { return find(typename detail::implicit_policy<It, T>::type(), f, l, v); }
 template <class It, class T, detail::enable_if_host<It, T> = 0> It find(It f, It l, const T& v) { return find(host, f, l, v); }
-template <class It, class P, detail::enable_if_device<It, P> = 0> It find_if(It f, It l, P p) { return find_if(device, f, l, p); }
+template <class It, class P, detail::enable_if_device<It, P> = 0> It find_if(It f, It l, P p) { return find_if(typename detail::implicit_policy<It, P>::type(), f, l, p); }
 template <class It, class P, detail::enable_if_host<It, P> = 0> It find_if(It f, It l, P p) { return find_if(host, f, l, p); }
-template <class It, class P, detail::enable_if_device<It, P> = 0> It find_if_not(It f, It l, P p) { return find_if_not(device, f, l, p); }
+template <class It, class P, detail::enable_if_device<It, P> = 0> It find_if_not(It f, It l, P p) { return find_if_not(typename detail::implicit_policy<It, P>::type(), f, l, p); }
 template <class It, class P, detail::enable_if_host<It, P> = 0> It find_if_not(It f, It l, P p) { return find_if_not(host, f, l, p); }
 }  // namespace thrust

@@ -25,8 +25,8 @@ It for_each(const system::cpp::detail::par_t&, It first, It last, F f) { std::fo
 template <class It, class Size, class F>
 It for_each_n(const system::cpp::detail::par_t&, It first, Size n, F f) { std::for_each(first, first + n, f); return first + n; }
 
-template <class It, class F, detail::enable_if_device<It, F> = 0> It for_each(It f, It l, F fn) { return for_each(device, f, l, fn); }
+template <class It, class F, detail::enable_if_device<It, F> = 0> It for_each(It f, It l, F fn) { return for_each(typename detail::implicit_policy<It, F>::type(), f, l, fn); }
 template <class It, class F, detail::enable_if_host<It, F> = 0> It for_each(It f, It l, F fn) { return for_each(host, f, l, fn); }
-template <class It, class Size, class F, detail::enable_if_device<It, Size, F> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(device, f, n, fn); }
+template <class It, class Size, class F, detail::enable_if_device<It, Size, F> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(typename detail::implicit_policy<It, Size, F>::type(), f, n, fn); }
 template <class It, class Size, class F, detail::enable_if_host<It, Size, F> = 0> It for_each_n(It f, Size n, F fn) { return for_each_n(host, f, n, fn); }
 }  // namespace thrust

@@ -52,19 +52,29 @@ Out gather_if(const system::cpp::detail::par_t&, Map map_first, Map map_last, S 
     if (pred(*stencil)) *result = input[*map_first];
   return result;
 }
-template <class Policy, class Map, class S, class In, class Out, detail::enable_if_policy<Policy> = 0>
-Out gather_if(const Policy& exec, Map mf, Map ml, S st, In in, Out out) { return gather_if(exec, mf, ml, st, in, out, detail::truthy()); }
+namespace detail {
+template <class Policy, class Map, class S, class In, class Out>
+Out composed_gather_if(const Policy& exec, Map mf, Map ml, S st, In in, Out out) { return gather_if(exec, mf, ml, st, in, out, detail::truthy()); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class Map, class S, class In, class Out>
+Out gather_if(execution_policy<D_>& exec, Map mf, Map ml, S st, In in, Out out) { return thrust::detail::composed_gather_if(exec, mf, ml, st, in, out); }
+}}  // namespace system::cdna4
+template <class D_, class Map, class S, class In, class Out>
+Out gather_if(const detail::execution_policy_base<D_>& exec, Map mf, Map ml, S st, In in, Out out) { return gather_if(detail::derived_cast(detail::strip_const(exec)), mf, ml, st, in, out); }
+template <class Map, class S, class In, class Out>
+Out gather_if(const system::cpp::detail::par_t& exec, Map mf, Map ml, S st, In in, Out out) { return detail::composed_gather_if(exec, mf, ml, st, in, out); }
 
 template <class Map, class In, class Out, detail::enable_if_device<Map, In, Out> = 0>
-Out gather(Map mf, Map ml, In in, Out out) { return gather(device, mf, ml, in, out); }
+Out gather(Map mf, Map ml, In in, Out out) { return gather(typename detail::implicit_policy<Map, In, Out>::type(), mf, ml, in, out); }
 template <class Map, class In, class Out, detail::enable_if_host<Map, In, Out> = 0>
 Out gather(Map mf, Map ml, In in, Out out) { return gather(host, mf, ml, in, out); }
 template <class Map, class S, class In, class Out, detail::enable_if_device<Map, S, In, Out> = 0>
-Out gather_if(Map mf, Map ml, S st, In in, Out out) { return gather_if(device, mf, ml, st, in, out); }
+Out gather_if(Map mf, Map ml, S st, In in, Out out) { return gather_if(typename detail::implicit_policy<Map, S, In, Out>::type(), mf, ml, st, in, out); }
 template <class Map, class S, class In, class Out, detail::enable_if_host<Map, S, In, Out> = 0>
 Out gather_if(Map mf, Map ml, S st, In in, Out out) { return gather_if(host, mf, ml, st, in, out); }
 template <class Map, class S, class In, class Out, class Pred, detail::enable_if_device<Map, S, In, Out, Pred> = 0>
-Out gather_if(Map mf, Map ml, S st, In in, Out out, Pred p) { return gather_if(device, mf, ml, st, in, out, p); }
+Out gather_if(Map mf, Map ml, S st, In in, Out out, Pred p) { return gather_if(typename detail::implicit_policy<Map, S, In, Out, Pred>::type(), mf, ml, st, in, out, p); }
 template <class Map, class S, class In, class Out, class Pred, detail::enable_if_host<Map, S, In, Out, Pred> = 0>
 Out gather_if(Map mf, Map ml, S st, In in, Out out, Pred p) { return gather_if(host, mf, ml, st, in, out, p); }
 }  // namespace thrust

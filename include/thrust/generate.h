@@ -24,13 +24,23 @@ void generate(const detail::execution_policy_base<D>& exec, It first, It last, G
 }
 template <class It, class G>
 void generate(const system::cpp::detail::par_t&, It first, It last, G gen) { std::generate(first, last, gen); }
-template <class Policy, class It, class Size, class G, detail::enable_if_policy<Policy> = 0>
-It generate_n(const Policy& exec, It first, Size n, G gen) {
+namespace detail {
+template <class Policy, class It, class Size, class G>
+It composed_generate_n(const Policy& exec, It first, Size n, G gen) {
   generate(exec, first, first + n, gen);
   return first + n;
 }
-template <class It, class G, detail::enable_if_device<It, G> = 0> void generate(It f, It l, G g) { generate(device, f, l, g); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class Size, class G>
+It generate_n(execution_policy<D_>& exec, It first, Size n, G gen) { return thrust::detail::composed_generate_n(exec, first, n, gen); }
+}}  // namespace system::cdna4
+template <class D_, class It, class Size, class G>
+It generate_n(const detail::execution_policy_base<D_>& exec, It first, Size n, G gen) { return generate_n(detail::derived_cast(detail::strip_const(exec)), first, n, gen); }
+template <class It, class Size, class G>
+It generate_n(const system::cpp::detail::par_t& exec, It first, Size n, G gen) { return detail::composed_generate_n(exec, first, n, gen); }
+template <class It, class G, detail::enable_if_device<It, G> = 0> void generate(It f, It l, G g) { generate(typename detail::implicit_policy<It, G>::type(), f, l, g); }
 template <class It, class G, detail::enable_if_host<It, G> = 0> void generate(It f, It l, G g) { generate(host, f, l, g); }
-template <class It, class Size, class G, detail::enable_if_device<It, Size, G> = 0> It generate_n(It f, Size n, G g) { return generate_n(device, f, n, g); }
+template <class It, class Size, class G, detail::enable_if_device<It, Size, G> = 0> It generate_n(It f, Size n, G g) { return generate_n(typename detail::implicit_policy<It, Size, G>::type(), f, n, g); }
 template <class It, class Size, class G, detail::enable_if_host<It, Size, G> = 0> It generate_n(It f, Size n, G g) { return generate_n(host, f, n, g); }
 }  // namespace thrust

@@ -45,27 +45,47 @@ pair<KOut, VOut> merge_by_key(const system::cpp::detail::par_t&, K1 kfirst1, K1 
   return pair<KOut, VOut>(kresult, vresult);
 }
 // ---- default comparison, and the forms without a policy
-template <class Policy, class In1, class In2, class Out, detail::enable_if_policy<Policy> = 0>
-Out merge(const Policy& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(exec, f1, l1, f2, l2, r, less<typename detail::value_of<In1>::type>()); }
+namespace detail {
+template <class Policy, class In1, class In2, class Out>
+Out composed_merge(const Policy& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(exec, f1, l1, f2, l2, r, less<typename detail::value_of<In1>::type>()); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In1, class In2, class Out>
+Out merge(execution_policy<D_>& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return thrust::detail::composed_merge(exec, f1, l1, f2, l2, r); }
+}}  // namespace system::cdna4
+template <class D_, class In1, class In2, class Out>
+Out merge(const detail::execution_policy_base<D_>& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(detail::derived_cast(detail::strip_const(exec)), f1, l1, f2, l2, r); }
+template <class In1, class In2, class Out>
+Out merge(const system::cpp::detail::par_t& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return detail::composed_merge(exec, f1, l1, f2, l2, r); }
 template <class In1, class In2, class Out, class Comp, detail::enable_if_device<In1, In2, Out, Comp> = 0>
-Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp c) { return merge(device, f1, l1, f2, l2, r, c); }
+Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp c) { return merge(typename detail::implicit_policy<In1, In2, Out, Comp>::type(), f1, l1, f2, l2, r, c); }
 template <class In1, class In2, class Out, class Comp, detail::enable_if_host<In1, In2, Out, Comp> = 0>
 Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp c) { return merge(host, f1, l1, f2, l2, r, c); }
 template <class In1, class In2, class Out, detail::enable_if_device<In1, In2, Out> = 0>
-Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(device, f1, l1, f2, l2, r); }
+Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(typename detail::implicit_policy<In1, In2, Out>::type(), f1, l1, f2, l2, r); }
 template <class In1, class In2, class Out, detail::enable_if_host<In1, In2, Out> = 0>
 Out merge(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return merge(host, f1, l1, f2, l2, r); }
 
-template <class Policy, class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_policy<Policy> = 0>
-pair<KOut, VOut> merge_by_key(const Policy& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) {
+namespace detail {
+template <class Policy, class K1, class K2, class V1, class V2, class KOut, class VOut>
+pair<KOut, VOut> composed_merge_by_key(const Policy& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) {
   return merge_by_key(exec, kf1, kl1, kf2, kl2, v1, v2, kr, vr, less<typename detail::value_of<K1>::type>());
 }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class K1, class K2, class V1, class V2, class KOut, class VOut>
+pair<KOut, VOut> merge_by_key(execution_policy<D_>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return thrust::detail::composed_merge_by_key(exec, kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
+}}  // namespace system::cdna4
+template <class D_, class K1, class K2, class V1, class V2, class KOut, class VOut>
+pair<KOut, VOut> merge_by_key(const detail::execution_policy_base<D_>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return merge_by_key(detail::derived_cast(detail::strip_const(exec)), kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
+template <class K1, class K2, class V1, class V2, class KOut, class VOut>
+pair<KOut, VOut> merge_by_key(const system::cpp::detail::par_t& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return detail::composed_merge_by_key(exec, kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
 template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp, detail::enable_if_device<K1, K2, V1, V2, KOut, VOut, Comp> = 0>
-pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp c) { return merge_by_key(device, kf1, kl1, kf2, kl2, v1, v2, kr, vr, c); }
+pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp c) { return merge_by_key(typename detail::implicit_policy<K1, K2, V1, V2, KOut, VOut, Comp>::type(), kf1, kl1, kf2, kl2, v1, v2, kr, vr, c); }
 template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp, detail::enable_if_host<K1, K2, V1, V2, KOut, VOut, Comp> = 0>
 pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp c) { return merge_by_key(host, kf1, kl1, kf2, kl2, v1, v2, kr, vr, c); }
 template <class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_device<K1, K2, V1, V2, KOut, VOut> = 0>
-pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return merge_by_key(device, kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
+pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return merge_by_key(typename detail::implicit_policy<K1, K2, V1, V2, KOut, VOut>::type(), kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
 template <class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_host<K1, K2, V1, V2, KOut, VOut> = 0>
 pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return merge_by_key(host, kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
 }  // namespace thrust

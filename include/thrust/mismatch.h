@@ -29,10 +29,20 @@ pair<It1, It2> mismatch(const system::cpp::detail::par_t&, It1 first1, It1 last1
   auto r = std::mismatch(first1, last1, first2, pred);
   return thrust::make_pair(r.first, r.second);
 }
-template <class Policy, class It1, class It2, detail::enable_if_policy<Policy> = 0>
-pair<It1, It2> mismatch(const Policy& exec, It1 f1, It1 l1, It2 f2) { return mismatch(exec, f1, l1, f2, equal_to<>()); }
-template <class It1, class It2, detail::enable_if_device<It1, It2> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2) { return mismatch(device, f1, l1, f2); }
+namespace detail {
+template <class Policy, class It1, class It2>
+pair<It1, It2> composed_mismatch(const Policy& exec, It1 f1, It1 l1, It2 f2) { return mismatch(exec, f1, l1, f2, equal_to<>()); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It1, class It2>
+pair<It1, It2> mismatch(execution_policy<D_>& exec, It1 f1, It1 l1, It2 f2) { return thrust::detail::composed_mismatch(exec, f1, l1, f2); }
+}}  // namespace system::cdna4
+template <class D_, class It1, class It2>
+pair<It1, It2> mismatch(const detail::execution_policy_base<D_>& exec, It1 f1, It1 l1, It2 f2) { return mismatch(detail::derived_cast(detail::strip_const(exec)), f1, l1, f2); }
+template <class It1, class It2>
+pair<It1, It2> mismatch(const system::cpp::detail::par_t& exec, It1 f1, It1 l1, It2 f2) { return detail::composed_mismatch(exec, f1, l1, f2); }
+template <class It1, class It2, detail::enable_if_device<It1, It2> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2) { return mismatch(typename detail::implicit_policy<It1, It2>::type(), f1, l1, f2); }
 template <class It1, class It2, detail::enable_if_host<It1, It2> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2) { return mismatch(host, f1, l1, f2); }
-template <class It1, class It2, class P, detail::enable_if_device<It1, It2, P> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2, P p) { return mismatch(device, f1, l1, f2, p); }
+template <class It1, class It2, class P, detail::enable_if_device<It1, It2, P> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2, P p) { return mismatch(typename detail::implicit_policy<It1, It2, P>::type(), f1, l1, f2, p); }
 template <class It1, class It2, class P, detail::enable_if_host<It1, It2, P> = 0> pair<It1, It2> mismatch(It1 f1, It1 l1, It2 f2, P p) { return mismatch(host, f1, l1, f2, p); }
 }  // namespace thrust

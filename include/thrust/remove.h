@@ -32,10 +32,10 @@ Out remove_copy(const Policy& exec, In first, In last, Out out, const V& value) 
 template <class Policy, class In, class V, class = typename std::iterator_traits<In>::iterator_category>
 In remove(const Policy& exec, In first, In last, const V& value) { return remove_if(exec, first, last, detail::equals_value<V>{value}); }
 
-template <class In, class Out, class Pred, detail::enable_if_device<In, Out, Pred> = 0> Out remove_copy_if(In f, In l, Out o, Pred p) { return remove_copy_if(device, f, l, o, p); }
+template <class In, class Out, class Pred, detail::enable_if_device<In, Out, Pred> = 0> Out remove_copy_if(In f, In l, Out o, Pred p) { return remove_copy_if(typename detail::implicit_policy<In, Out, Pred>::type(), f, l, o, p); }
 template <class In, class Out, class Pred, detail::enable_if_host<In, Out, Pred> = 0> Out remove_copy_if(In f, In l, Out o, Pred p) { return remove_copy_if(host, f, l, o, p); }
-template <class In, class Pred, detail::enable_if_device<In, Pred> = 0> In remove_if(In f, In l, Pred p) { return remove_if(device, f, l, p); }
+template <class In, class Pred, detail::enable_if_device<In, Pred> = 0> In remove_if(In f, In l, Pred p) { return remove_if(typename detail::implicit_policy<In, Pred>::type(), f, l, p); }
 template <class In, class Pred, detail::enable_if_host<In, Pred> = 0> In remove_if(In f, In l, Pred p) { return remove_if(host, f, l, p); }
-template <class In, class V, detail::enable_if_device<In, V> = 0> In remove(In f, In l, const V& v) { return remove(device, f, l, v); }
+template <class In, class V, detail::enable_if_device<In, V> = 0> In remove(In f, In l, const V& v) { return remove(typename detail::implicit_policy<In, V>::type(), f, l, v); }
 template <class In, class V, detail::enable_if_host<In, V> = 0> In remove(In f, In l, const V& v) { return remove(host, f, l, v); }
 }  // namespace thrust

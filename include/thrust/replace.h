@@ -35,22 +35,72 @@ Out replace_copy_if(const system::cpp::detail::par_t&, In first, In last, S sten
   }
   return result;
 }
-template <class Policy, class In, class Out, class Pred, class T, detail::enable_if_policy<Policy> = 0>
-Out replace_copy_if(const Policy& exec, In first, In last, Out result, Pred pred, const T& value) {
+namespace detail {
+template <class Policy, class In, class Out, class Pred, class T>
+Out composed_replace_copy_if(const Policy& exec, In first, In last, Out result, Pred pred, const T& value) {
   return replace_copy_if(exec, first, last, first, result, pred, value);
 }
-template <class Policy, class In, class Out, class T, detail::enable_if_policy<Policy> = 0>
-Out replace_copy(const Policy& exec, In first, In last, Out result, const T& old_value, const T& new_value) {
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In, class Out, class Pred, class T>
+Out replace_copy_if(execution_policy<D_>& exec, In first, In last, Out result, Pred pred, const T& value) { return thrust::detail::composed_replace_copy_if(exec, first, last, result, pred, value); }
+}}  // namespace system::cdna4
+template <class D_, class In, class Out, class Pred, class T>
+Out replace_copy_if(const detail::execution_policy_base<D_>& exec, In first, In last, Out result, Pred pred, const T& value) { return replace_copy_if(detail::derived_cast(detail::strip_const(exec)), first, last, result, pred, value); }
+template <class In, class Out, class Pred, class T>
+Out replace_copy_if(const system::cpp::detail::par_t& exec, In first, In last, Out result, Pred pred, const T& value) { return detail::composed_replace_copy_if(exec, first, last, result, pred, value); }
+namespace detail {
+template <class Policy, class In, class Out, class T>
+Out composed_replace_copy(const Policy& exec, In first, In last, Out result, const T& old_value, const T& new_value) {
   return replace_copy_if(exec, first, last, first, result, detail::equals_value<T>{old_value}, new_value);
 }
-template <class Policy, class It, class Pred, class T, detail::enable_if_policy<Policy> = 0>
-void replace_if(const Policy& exec, It first, It last, Pred pred, const T& value) { replace_copy_if(exec, first, last, first, first, pred, value); }
-template <class Policy, class It, class S, class Pred, class T, detail::enable_if_policy<Policy> = 0>
-void replace_if(const Policy& exec, It first, It last, S stencil, Pred pred, const T& value) { replace_copy_if(exec, first, last, stencil, first, pred, value); }
-template <class Policy, class It, class T, detail::enable_if_policy<Policy> = 0>
-void replace(const Policy& exec, It first, It last, const T& old_value, const T& new_value) {
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In, class Out, class T>
+Out replace_copy(execution_policy<D_>& exec, In first, In last, Out result, const T& old_value, const T& new_value) { return thrust::detail::composed_replace_copy(exec, first, last, result, old_value, new_value); }
+}}  // namespace system::cdna4
+template <class D_, class In, class Out, class T>
+Out replace_copy(const detail::execution_policy_base<D_>& exec, In first, In last, Out result, const T& old_value, const T& new_value) { return replace_copy(detail::derived_cast(detail::strip_const(exec)), first, last, result, old_value, new_value); }
+template <class In, class Out, class T>
+Out replace_copy(const system::cpp::detail::par_t& exec, In first, In last, Out result, const T& old_value, const T& new_value) { return detail::composed_replace_copy(exec, first, last, result, old_value, new_value); }
+namespace detail {
+template <class Policy, class It, class Pred, class T>
+void composed_replace_if(const Policy& exec, It first, It last, Pred pred, const T& value) { replace_copy_if(exec, first, last, first, first, pred, value); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class Pred, class T>
+void replace_if(execution_policy<D_>& exec, It first, It last, Pred pred, const T& value) { return thrust::detail::composed_replace_if(exec, first, last, pred, value); }
+}}  // namespace system::cdna4
+template <class D_, class It, class Pred, class T>
+void replace_if(const detail::execution_policy_base<D_>& exec, It first, It last, Pred pred, const T& value) { return replace_if(detail::derived_cast(detail::strip_const(exec)), first, last, pred, value); }
+template <class It, class Pred, class T>
+void replace_if(const system::cpp::detail::par_t& exec, It first, It last, Pred pred, const T& value) { return detail::composed_replace_if(exec, first, last, pred, value); }
+namespace detail {
+template <class Policy, class It, class S, class Pred, class T>
+void composed_replace_if(const Policy& exec, It first, It last, S stencil, Pred pred, const T& value) { replace_copy_if(exec, first, last, stencil, first, pred, value); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class S, class Pred, class T>
+void replace_if(execution_policy<D_>& exec, It first, It last, S stencil, Pred pred, const T& value) { return thrust::detail::composed_replace_if(exec, first, last, stencil, pred, value); }
+}}  // namespace system::cdna4
+template <class D_, class It, class S, class Pred, class T>
+void replace_if(const detail::execution_policy_base<D_>& exec, It first, It last, S stencil, Pred pred, const T& value) { return replace_if(detail::derived_cast(detail::strip_const(exec)), first, last, stencil, pred, value); }
+template <class It, class S, class Pred, class T>
+void replace_if(const system::cpp::detail::par_t& exec, It first, It last, S stencil, Pred pred, const T& value) { return detail::composed_replace_if(exec, first, last, stencil, pred, value); }
+namespace detail {
+template <class Policy, class It, class T>
+void composed_replace(const Policy& exec, It first, It last, const T& old_value, const T& new_value) {
   replace_copy_if(exec, first, last, first, first, detail::equals_value<T>{old_value}, new_value);
 }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class T>
+void replace(execution_policy<D_>& exec, It first, It last, const T& old_value, const T& new_value) { return thrust::detail::composed_replace(exec, first, last, old_value, new_value); }
+}}  // namespace system::cdna4
+template <class D_, class It, class T>
+void replace(const detail::execution_policy_base<D_>& exec, It first, It last, const T& old_value, const T& new_value) { return replace(detail::derived_cast(detail::strip_const(exec)), first, last, old_value, new_value); }
+template <class It, class T>
+void replace(const system::cpp::detail::par_t& exec, It first, It last, const T& old_value, const T& new_value) { return detail::composed_replace(exec, first, last, old_value, new_value); }
 
 #define THRUST_CDNA4_REPLACE(SYS, COND)                                                                                       \
   template <class It, class T, COND<It> = 0> void replace(It f, It l, const T& a, const T& b) { replace(SYS, f, l, a, b); }    \

@@ -42,8 +42,8 @@ Out reverse_copy(const detail::execution_policy_base<D>& exec, In first, In last
   return reverse_copy(detail::derived_cast(detail::strip_const(exec)), first, last, result);
 }
 template <class In, class Out> Out reverse_copy(const system::cpp::detail::par_t&, In first, In last, Out result) { return std::reverse_copy(first, last, result); }
-template <class It, detail::enable_if_device<It> = 0> void reverse(It f, It l) { reverse(device, f, l); }
+template <class It, detail::enable_if_device<It> = 0> void reverse(It f, It l) { reverse(typename detail::implicit_policy<It>::type(), f, l); }
 template <class It, detail::enable_if_host<It> = 0> void reverse(It f, It l) { reverse(host, f, l); }
-template <class In, class Out, detail::enable_if_device<In, Out> = 0> Out reverse_copy(In f, In l, Out o) { return reverse_copy(device, f, l, o); }
+template <class In, class Out, detail::enable_if_device<In, Out> = 0> Out reverse_copy(In f, In l, Out o) { return reverse_copy(typename detail::implicit_policy<In, Out>::type(), f, l, o); }
 template <class In, class Out, detail::enable_if_host<In, Out> = 0> Out reverse_copy(In f, In l, Out o) { return reverse_copy(host, f, l, o); }
 }  // namespace thrust

@@ -47,15 +47,25 @@ void scatter_if(const system::cpp::detail::par_t&, In first, In last, Map map, S
   for (; first != last; ++first, ++map, ++stencil)
     if (pred(*stencil)) output[*map] = *first;
 }
-template <class Policy, class In, class Map, class S, class Out, detail::enable_if_policy<Policy> = 0>
-void scatter_if(const Policy& exec, In f, In l, Map m, S st, Out o) { scatter_if(exec, f, l, m, st, o, detail::truthy()); }
+namespace detail {
+template <class Policy, class In, class Map, class S, class Out>
+void composed_scatter_if(const Policy& exec, In f, In l, Map m, S st, Out o) { scatter_if(exec, f, l, m, st, o, detail::truthy()); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In, class Map, class S, class Out>
+void scatter_if(execution_policy<D_>& exec, In f, In l, Map m, S st, Out o) { return thrust::detail::composed_scatter_if(exec, f, l, m, st, o); }
+}}  // namespace system::cdna4
+template <class D_, class In, class Map, class S, class Out>
+void scatter_if(const detail::execution_policy_base<D_>& exec, In f, In l, Map m, S st, Out o) { return scatter_if(detail::derived_cast(detail::strip_const(exec)), f, l, m, st, o); }
+template <class In, class Map, class S, class Out>
+void scatter_if(const system::cpp::detail::par_t& exec, In f, In l, Map m, S st, Out o) { return detail::composed_scatter_if(exec, f, l, m, st, o); }
 
-template <class In, class Map, class Out, detail::enable_if_device<In, Map, Out> = 0> void scatter(In f, In l, Map m, Out o) { scatter(device, f, l, m, o); }
+template <class In, class Map, class Out, detail::enable_if_device<In, Map, Out> = 0> void scatter(In f, In l, Map m, Out o) { scatter(typename detail::implicit_policy<In, Map, Out>::type(), f, l, m, o); }
 template <class In, class Map, class Out, detail::enable_if_host<In, Map, Out> = 0> void scatter(In f, In l, Map m, Out o) { scatter(host, f, l, m, o); }
-template <class In, class Map, class S, class Out, detail::enable_if_device<In, Map, S, Out> = 0> void scatter_if(In f, In l, Map m, S st, Out o) { scatter_if(device, f, l, m, st, o); }
+template <class In, class Map, class S, class Out, detail::enable_if_device<In, Map, S, Out> = 0> void scatter_if(In f, In l, Map m, S st, Out o) { scatter_if(typename detail::implicit_policy<In, Map, S, Out>::type(), f, l, m, st, o); }
 template <class In, class Map, class S, class Out, detail::enable_if_host<In, Map, S, Out> = 0> void scatter_if(In f, In l, Map m, S st, Out o) { scatter_if(host, f, l, m, st, o); }
 template <class In, class Map, class S, class Out, class Pred, detail::enable_if_device<In, Map, S, Out, Pred> = 0>
-void scatter_if(In f, In l, Map m, S st, Out o, Pred p) { scatter_if(device, f, l, m, st, o, p); }
+void scatter_if(In f, In l, Map m, S st, Out o, Pred p) { scatter_if(typename detail::implicit_policy<In, Map, S, Out, Pred>::type(), f, l, m, st, o, p); }
 template <class In, class Map, class S, class Out, class Pred, detail::enable_if_host<In, Map, S, Out, Pred> = 0>
 void scatter_if(In f, In l, Map m, S st, Out o, Pred p) { scatter_if(host, f, l, m, st, o, p); }
 }  // namespace thrust

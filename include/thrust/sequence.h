@@ -27,10 +27,10 @@ void sequence(const Policy& exec, It first, It last) {
   sequence(exec, first, last, V(0), V(1));
 }
 
-template <class It, detail::enable_if_device<It> = 0> void sequence(It f, It l) { sequence(device, f, l); }
+template <class It, detail::enable_if_device<It> = 0> void sequence(It f, It l) { sequence(typename detail::implicit_policy<It>::type(), f, l); }
 template <class It, detail::enable_if_host<It> = 0> void sequence(It f, It l) { sequence(host, f, l); }
-template <class It, class T, detail::enable_if_device<It, T> = 0> void sequence(It f, It l, T init) { sequence(device, f, l, init); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> void sequence(It f, It l, T init) { sequence(typename detail::implicit_policy<It, T>::type(), f, l, init); }
 template <class It, class T, detail::enable_if_host<It, T> = 0> void sequence(It f, It l, T init) { sequence(host, f, l, init); }
-template <class It, class T, detail::enable_if_device<It, T> = 0> void sequence(It f, It l, T init, T step) { sequence(device, f, l, init, step); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> void sequence(It f, It l, T init, T step) { sequence(typename detail::implicit_policy<It, T>::type(), f, l, init, step); }
 template <class It, class T, detail::enable_if_host<It, T> = 0> void sequence(It f, It l, T init, T step) { sequence(host, f, l, init, step); }
 }  // namespace thrust

@@ -121,11 +121,11 @@ std::int64_t set_operation(const system::cpp::detail::par_t&, K1 k1, K1 l1, K2 k
     return NAME(exec, f1, l1, f2, l2, r, less<typename detail::value_of<In1>::type>());                                               \
   }                                                                                                                                   \
   template <class In1, class In2, class Out, class Comp, detail::enable_if_device<In1, In2, Out, Comp> = 0>                                           \
-  Out NAME(In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp c) { return NAME(device, f1, l1, f2, l2, r, c); }                              \
+  Out NAME(In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp c) { return NAME(typename detail::implicit_policy<In1, In2, Out, Comp>::type(), f1, l1, f2, l2, r, c); }                              \
   template <class In1, class In2, class Out, class Comp, detail::enable_if_host<In1, In2, Out, Comp> = 0>                                             \
   Out NAME(In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp c) { return NAME(host, f1, l1, f2, l2, r, c); }                                \
   template <class In1, class In2, class Out, detail::enable_if_device<In1, In2, Out> = 0>                                                       \
-  Out NAME(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return NAME(device, f1, l1, f2, l2, r); }                                         \
+  Out NAME(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return NAME(typename detail::implicit_policy<In1, In2, Out>::type(), f1, l1, f2, l2, r); }                                         \
   template <class In1, class In2, class Out, detail::enable_if_host<In1, In2, Out> = 0>                                                         \
   Out NAME(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return NAME(host, f1, l1, f2, l2, r); }
 THRUST_CDNA4_SET_OPERATION(set_difference, detail::set_difference_mode)
@@ -147,11 +147,11 @@ THRUST_CDNA4_SET_OPERATION(set_union, detail::set_union_mode)
     return NAME(exec, kf1, kl1, kf2, kl2, v1, v2, kr, vr, less<typename detail::value_of<K1>::type>());                               \
   }                                                                                                                                   \
   template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp, detail::enable_if_device<K1, K2, V1, V2, KOut, VOut, Comp> = 0>             \
-  pair<KOut, VOut> NAME(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp c) { return NAME(device, kf1, kl1, kf2, kl2, v1, v2, kr, vr, c); } \
+  pair<KOut, VOut> NAME(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp c) { return NAME(typename detail::implicit_policy<K1, K2, V1, V2, KOut, VOut, Comp>::type(), kf1, kl1, kf2, kl2, v1, v2, kr, vr, c); } \
   template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp, detail::enable_if_host<K1, K2, V1, V2, KOut, VOut, Comp> = 0>               \
   pair<KOut, VOut> NAME(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp c) { return NAME(host, kf1, kl1, kf2, kl2, v1, v2, kr, vr, c); } \
   template <class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_device<K1, K2, V1, V2, KOut, VOut> = 0>                         \
-  pair<KOut, VOut> NAME(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return NAME(device, kf1, kl1, kf2, kl2, v1, v2, kr, vr); } \
+  pair<KOut, VOut> NAME(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return NAME(typename detail::implicit_policy<K1, K2, V1, V2, KOut, VOut>::type(), kf1, kl1, kf2, kl2, v1, v2, kr, vr); } \
   template <class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_host<K1, K2, V1, V2, KOut, VOut> = 0>                           \
   pair<KOut, VOut> NAME(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return NAME(host, kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
 THRUST_CDNA4_SET_OPERATION_BY_KEY(set_difference_by_key, detail::set_difference_mode)
@@ -170,11 +170,11 @@ pair<KOut, VOut> set_intersection_by_key(const Policy& exec, K1 kf1, K1 kl1, K2 
   return set_intersection_by_key(exec, kf1, kl1, kf2, kl2, v1, kr, vr, less<typename detail::value_of<K1>::type>());
 }
 template <class K1, class K2, class V1, class KOut, class VOut, class Comp, detail::enable_if_device<K1, K2, V1, KOut, VOut, Comp> = 0>
-pair<KOut, VOut> set_intersection_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr, Comp c) { return set_intersection_by_key(device, kf1, kl1, kf2, kl2, v1, kr, vr, c); }
+pair<KOut, VOut> set_intersection_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr, Comp c) { return set_intersection_by_key(typename detail::implicit_policy<K1, K2, V1, KOut, VOut, Comp>::type(), kf1, kl1, kf2, kl2, v1, kr, vr, c); }
 template <class K1, class K2, class V1, class KOut, class VOut, class Comp, detail::enable_if_host<K1, K2, V1, KOut, VOut, Comp> = 0>
 pair<KOut, VOut> set_intersection_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr, Comp c) { return set_intersection_by_key(host, kf1, kl1, kf2, kl2, v1, kr, vr, c); }
 template <class K1, class K2, class V1, class KOut, class VOut, detail::enable_if_device<K1, K2, V1, KOut, VOut> = 0>
-pair<KOut, VOut> set_intersection_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr) { return set_intersection_by_key(device, kf1, kl1, kf2, kl2, v1, kr, vr); }
+pair<KOut, VOut> set_intersection_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr) { return set_intersection_by_key(typename detail::implicit_policy<K1, K2, V1, KOut, VOut>::type(), kf1, kl1, kf2, kl2, v1, kr, vr); }
 template <class K1, class K2, class V1, class KOut, class VOut, detail::enable_if_host<K1, K2, V1, KOut, VOut> = 0>
 pair<KOut, VOut> set_intersection_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr) { return set_intersection_by_key(host, kf1, kl1, kf2, kl2, v1, kr, vr); }
 }  // namespace thrust

@@ -106,8 +106,8 @@ void shuffle(const system::cpp::detail::par_t& exec, It first, It last, URBG&& g
   std::vector<T> copy(first, last);
   shuffle_copy(exec, copy.begin(), copy.end(), first, g);
 }
-template <class It, class URBG, detail::enable_if_device<It, URBG> = 0> void shuffle(It first, It last, URBG&& g) { shuffle(device, first, last, g); }
+template <class It, class URBG, detail::enable_if_device<It, URBG> = 0> void shuffle(It first, It last, URBG&& g) { shuffle(typename detail::implicit_policy<It, URBG>::type(), first, last, g); }
 template <class It, class URBG, detail::enable_if_host<It, URBG> = 0> void shuffle(It first, It last, URBG&& g) { shuffle(host, first, last, g); }
-template <class In, class Out, class URBG, detail::enable_if_device<In, Out, URBG> = 0> void shuffle_copy(In first, In last, Out result, URBG&& g) { shuffle_copy(device, first, last, result, g); }
+template <class In, class Out, class URBG, detail::enable_if_device<In, Out, URBG> = 0> void shuffle_copy(In first, In last, Out result, URBG&& g) { shuffle_copy(typename detail::implicit_policy<In, Out, URBG>::type(), first, last, result, g); }
 template <class In, class Out, class URBG, detail::enable_if_host<In, Out, URBG> = 0> void shuffle_copy(In first, In last, Out result, URBG&& g) { shuffle_copy(host, first, last, result, g); }
 }  // namespace thrust

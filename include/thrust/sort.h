@@ -224,18 +224,48 @@ It is_sorted_until(const system::cdna4::execution_policy<D>& exec, It first, It 
 }
 template <class It, class Compare>
 It is_sorted_until(const system::cpp::detail::par_t&, It first, It last, Compare comp) { return std::is_sorted_until(first, last, comp); }
-template <class Policy, class It, detail::enable_if_policy<Policy> = 0>
-It is_sorted_until(const Policy& exec, It first, It last) { return is_sorted_until(exec, first, last, less<>()); }
-template <class Policy, class It, class Compare, detail::enable_if_policy<Policy> = 0>
-bool is_sorted(const Policy& exec, It first, It last, Compare comp) { return is_sorted_until(exec, first, last, comp) == last; }
-template <class Policy, class It, detail::enable_if_policy<Policy> = 0>
-bool is_sorted(const Policy& exec, It first, It last) { return is_sorted_until(exec, first, last, less<>()) == last; }
-template <class It, detail::enable_if_device<It> = 0> It is_sorted_until(It f, It l) { return is_sorted_until(device, f, l); }
+namespace detail {
+template <class Policy, class It>
+It composed_is_sorted_until(const Policy& exec, It first, It last) { return is_sorted_until(exec, first, last, less<>()); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It>
+It is_sorted_until(execution_policy<D_>& exec, It first, It last) { return thrust::detail::composed_is_sorted_until(exec, first, last); }
+}}  // namespace system::cdna4
+template <class D_, class It>
+It is_sorted_until(const detail::execution_policy_base<D_>& exec, It first, It last) { return is_sorted_until(detail::derived_cast(detail::strip_const(exec)), first, last); }
+template <class It>
+It is_sorted_until(const system::cpp::detail::par_t& exec, It first, It last) { return detail::composed_is_sorted_until(exec, first, last); }
+namespace detail {
+template <class Policy, class It, class Compare>
+bool composed_is_sorted(const Policy& exec, It first, It last, Compare comp) { return is_sorted_until(exec, first, last, comp) == last; }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class Compare>
+bool is_sorted(execution_policy<D_>& exec, It first, It last, Compare comp) { return thrust::detail::composed_is_sorted(exec, first, last, comp); }
+}}  // namespace system::cdna4
+template <class D_, class It, class Compare>
+bool is_sorted(const detail::execution_policy_base<D_>& exec, It first, It last, Compare comp) { return is_sorted(detail::derived_cast(detail::strip_const(exec)), first, last, comp); }
+template <class It, class Compare>
+bool is_sorted(const system::cpp::detail::par_t& exec, It first, It last, Compare comp) { return detail::composed_is_sorted(exec, first, last, comp); }
+namespace detail {
+template <class Policy, class It>
+bool composed_is_sorted(const Policy& exec, It first, It last) { return is_sorted_until(exec, first, last, less<>()) == last; }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It>
+bool is_sorted(execution_policy<D_>& exec, It first, It last) { return thrust::detail::composed_is_sorted(exec, first, last); }
+}}  // namespace system::cdna4
+template <class D_, class It>
+bool is_sorted(const detail::execution_policy_base<D_>& exec, It first, It last) { return is_sorted(detail::derived_cast(detail::strip_const(exec)), first, last); }
+template <class It>
+bool is_sorted(const system::cpp::detail::par_t& exec, It first, It last) { return detail::composed_is_sorted(exec, first, last); }
+template <class It, detail::enable_if_device<It> = 0> It is_sorted_until(It f, It l) { return is_sorted_until(typename detail::implicit_policy<It>::type(), f, l); }
 template <class It, detail::enable_if_host<It> = 0> It is_sorted_until(It f, It l) { return is_sorted_until(host, f, l); }
-template <class It, class C, detail::enable_if_device<It, C> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(device, f, l, c); }
+template <class It, class C, detail::enable_if_device<It, C> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(typename detail::implicit_policy<It, C>::type(), f, l, c); }
 template <class It, class C, detail::enable_if_host<It, C> = 0> It is_sorted_until(It f, It l, C c) { return is_sorted_until(host, f, l, c); }
-template <class It, detail::enable_if_device<It> = 0> bool is_sorted(It f, It l) { return is_sorted(device, f, l); }
+template <class It, detail::enable_if_device<It> = 0> bool is_sorted(It f, It l) { return is_sorted(typename detail::implicit_policy<It>::type(), f, l); }
 template <class It, detail::enable_if_host<It> = 0> bool is_sorted(It f, It l) { return is_sorted(host, f, l); }
-template <class It, class C, detail::enable_if_device<It, C> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(device, f, l, c); }
+template <class It, class C, detail::enable_if_device<It, C> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(typename detail::implicit_policy<It, C>::type(), f, l, c); }
 template <class It, class C, detail::enable_if_host<It, C> = 0> bool is_sorted(It f, It l, C c) { return is_sorted(host, f, l, c); }
 }  // namespace thrust

@@ -33,6 +33,6 @@ It2 swap_ranges(const detail::execution_policy_base<D>& exec, It1 first1, It1 la
   return swap_ranges(detail::derived_cast(detail::strip_const(exec)), first1, last1, first2);
 }
 template <class It1, class It2> It2 swap_ranges(const system::cpp::detail::par_t&, It1 f1, It1 l1, It2 f2) { return std::swap_ranges(f1, l1, f2); }
-template <class It1, class It2, detail::enable_if_device<It1, It2> = 0> It2 swap_ranges(It1 f1, It1 l1, It2 f2) { return swap_ranges(device, f1, l1, f2); }
+template <class It1, class It2, detail::enable_if_device<It1, It2> = 0> It2 swap_ranges(It1 f1, It1 l1, It2 f2) { return swap_ranges(typename detail::implicit_policy<It1, It2>::type(), f1, l1, f2); }
 template <class It1, class It2, detail::enable_if_host<It1, It2> = 0> It2 swap_ranges(It1 f1, It1 l1, It2 f2) { return swap_ranges(host, f1, l1, f2); }
 }  // namespace thrust

@@ -26,6 +26,6 @@ void tabulate(const system::cpp::detail::par_t&, It first, It last, F f) {
   typename std::iterator_traits<It>::difference_type i = 0;
   for (; first != last; ++first, ++i) *first = f(i);
 }
-template <class It, class F, detail::enable_if_device<It, F> = 0> void tabulate(It f, It l, F fn) { tabulate(device, f, l, fn); }
+template <class It, class F, detail::enable_if_device<It, F> = 0> void tabulate(It f, It l, F fn) { tabulate(typename detail::implicit_policy<It, F>::type(), f, l, fn); }
 template <class It, class F, detail::enable_if_host<It, F> = 0> void tabulate(It f, It l, F fn) { tabulate(host, f, l, fn); }
 }  // namespace thrust

@@ -28,12 +28,12 @@ Out transform(const system::cpp::detail::par_t&, In1 first1, In1 last1, In2 firs
 }
 
 template <class In, class Out, class F, detail::enable_if_device<In, Out, F> = 0>
-Out transform(In f, In l, Out o, F fn) { return transform(device, f, l, o, fn); }
+Out transform(In f, In l, Out o, F fn) { return transform(typename detail::implicit_policy<In, Out, F>::type(), f, l, o, fn); }
 template <class In, class Out, class F, detail::enable_if_host<In, Out, F> = 0>
 Out transform(In f, In l, Out o, F fn) { return transform(host, f, l, o, fn); }
 template <class In1, class In2, class Out, class F, detail::enable_if_device<In1, In2, Out, F> = 0,
           class = typename std::iterator_traits<In2>::iterator_category>
-Out transform(In1 f, In1 l, In2 f2, Out o, F fn) { return transform(device, f, l, f2, o, fn); }
+Out transform(In1 f, In1 l, In2 f2, Out o, F fn) { return transform(typename detail::implicit_policy<In1, In2, Out, F>::type(), f, l, f2, o, fn); }
 template <class In1, class In2, class Out, class F, detail::enable_if_host<In1, In2, Out, F> = 0,
           class = typename std::iterator_traits<In2>::iterator_category>
 Out transform(In1 f, In1 l, In2 f2, Out o, F fn) { return transform(host, f, l, f2, o, fn); }
@@ -59,18 +59,48 @@ Out transform_if_n(const Policy& exec, In1 a, In2 b, St stencil, Out out, std::i
   return out + n;
 }
 }  // namespace detail
-template <class Policy, class In, class Out, class Op, class Pred, detail::enable_if_policy<Policy> = 0>
-Out transform_if(const Policy& exec, In first, In last, Out result, Op op, Pred pred) {
+namespace detail {
+template <class Policy, class In, class Out, class Op, class Pred>
+Out composed_transform_if(const Policy& exec, In first, In last, Out result, Op op, Pred pred) {
   return detail::transform_if_n<1, false>(exec, first, first, first, result, (std::int64_t)(last - first), op, pred);
 }
-template <class Policy, class In, class St, class Out, class Op, class Pred, detail::enable_if_policy<Policy> = 0>
-Out transform_if(const Policy& exec, In first, In last, St stencil, Out result, Op op, Pred pred) {
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In, class Out, class Op, class Pred>
+Out transform_if(execution_policy<D_>& exec, In first, In last, Out result, Op op, Pred pred) { return thrust::detail::composed_transform_if(exec, first, last, result, op, pred); }
+}}  // namespace system::cdna4
+template <class D_, class In, class Out, class Op, class Pred>
+Out transform_if(const detail::execution_policy_base<D_>& exec, In first, In last, Out result, Op op, Pred pred) { return transform_if(detail::derived_cast(detail::strip_const(exec)), first, last, result, op, pred); }
+template <class In, class Out, class Op, class Pred>
+Out transform_if(const system::cpp::detail::par_t& exec, In first, In last, Out result, Op op, Pred pred) { return detail::composed_transform_if(exec, first, last, result, op, pred); }
+namespace detail {
+template <class Policy, class In, class St, class Out, class Op, class Pred>
+Out composed_transform_if(const Policy& exec, In first, In last, St stencil, Out result, Op op, Pred pred) {
   return detail::transform_if_n<1, true>(exec, first, first, stencil, result, (std::int64_t)(last - first), op, pred);
 }
-template <class Policy, class In1, class In2, class St, class Out, class Op, class Pred, detail::enable_if_policy<Policy> = 0>
-Out transform_if(const Policy& exec, In1 first1, In1 last1, In2 first2, St stencil, Out result, Op op, Pred pred) {
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In, class St, class Out, class Op, class Pred>
+Out transform_if(execution_policy<D_>& exec, In first, In last, St stencil, Out result, Op op, Pred pred) { return thrust::detail::composed_transform_if(exec, first, last, stencil, result, op, pred); }
+}}  // namespace system::cdna4
+template <class D_, class In, class St, class Out, class Op, class Pred>
+Out transform_if(const detail::execution_policy_base<D_>& exec, In first, In last, St stencil, Out result, Op op, Pred pred) { return transform_if(detail::derived_cast(detail::strip_const(exec)), first, last, stencil, result, op, pred); }
+template <class In, class St, class Out, class Op, class Pred>
+Out transform_if(const system::cpp::detail::par_t& exec, In first, In last, St stencil, Out result, Op op, Pred pred) { return detail::composed_transform_if(exec, first, last, stencil, result, op, pred); }
+namespace detail {
+template <class Policy, class In1, class In2, class St, class Out, class Op, class Pred>
+Out composed_transform_if(const Policy& exec, In1 first1, In1 last1, In2 first2, St stencil, Out result, Op op, Pred pred) {
   return detail::transform_if_n<2, true>(exec, first1, first2, stencil, result, (std::int64_t)(last1 - first1), op, pred);
 }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In1, class In2, class St, class Out, class Op, class Pred>
+Out transform_if(execution_policy<D_>& exec, In1 first1, In1 last1, In2 first2, St stencil, Out result, Op op, Pred pred) { return thrust::detail::composed_transform_if(exec, first1, last1, first2, stencil, result, op, pred); }
+}}  // namespace system::cdna4
+template <class D_, class In1, class In2, class St, class Out, class Op, class Pred>
+Out transform_if(const detail::execution_policy_base<D_>& exec, In1 first1, In1 last1, In2 first2, St stencil, Out result, Op op, Pred pred) { return transform_if(detail::derived_cast(detail::strip_const(exec)), first1, last1, first2, stencil, result, op, pred); }
+template <class In1, class In2, class St, class Out, class Op, class Pred>
+Out transform_if(const system::cpp::detail::par_t& exec, In1 first1, In1 last1, In2 first2, St stencil, Out result, Op op, Pred pred) { return detail::composed_transform_if(exec, first1, last1, first2, stencil, result, op, pred); }
 #define THRUST_CDNA4_TRANSFORM_IF_NO_POLICY(SYS, COND)                                                                         \
   template <class In, class Out, class Op, class Pred, COND<In> = 0>                                                           \
   Out transform_if(In first, In last, Out result, Op op, Pred pred) { return transform_if(SYS, first, last, result, op, pred); } \

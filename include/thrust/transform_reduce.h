@@ -20,7 +20,7 @@ T transform_reduce(const system::cpp::detail::par_t&, It first, It last, F f, T 
   return init;
 }
 template <class It, class F, class T, class Op, detail::enable_if_device<It, F, T, Op> = 0>
-T transform_reduce(It f, It l, F fn, T init, Op op) { return transform_reduce(device, f, l, fn, init, op); }
+T transform_reduce(It f, It l, F fn, T init, Op op) { return transform_reduce(typename detail::implicit_policy<It, F, T, Op>::type(), f, l, fn, init, op); }
 template <class It, class F, class T, class Op, detail::enable_if_host<It, F, T, Op> = 0>
 T transform_reduce(It f, It l, F fn, T init, Op op) { return transform_reduce(host, f, l, fn, init, op); }
 }  // namespace thrust

@@ -9,6 +9,7 @@
 #include <type_traits>
 #include <vector>
 #include <thrust/device_ptr.h>
+#include <thrust/iterator/detail/normal_iterator.h>
 namespace thrust {
 template <class Iterator> struct proclaim_contiguous_iterator : std::false_type {};
 #define THRUST_PROCLAIM_CONTIGUOUS_ITERATOR(Iterator) \
@@ -19,6 +20,8 @@ template <class T> struct is_contiguous_iterator_impl<T*> : std::true_type {};
 template <class T> struct is_contiguous_iterator_impl<thrust::device_ptr<T>> : std::true_type {};
 // libstdc++'s vector and string iterators wrap a raw pointer
 template <class P, class C> struct is_contiguous_iterator_impl<__gnu_cxx::__normal_iterator<P, C>> : std::is_pointer<P> {};
+// thrust::host_vector's iterators wrap a raw pointer too
+template <class P> struct is_contiguous_iterator_impl<normal_iterator<P>> : std::is_pointer<P> {};
 }  // namespace detail
 template <class Iterator> struct is_contiguous_iterator : detail::is_contiguous_iterator_impl<typename std::remove_cv<Iterator>::type> {};
 #if __cplusplus >= 201402L

@@ -14,8 +14,18 @@ Out uninitialized_copy(const detail::execution_policy_base<D>& exec, In first, I
 }
 template <class In, class Out>
 Out uninitialized_copy(const system::cpp::detail::par_t&, In first, In last, Out result) { return std::uninitialized_copy(first, last, result); }
-template <class Policy, class In, class Size, class Out, detail::enable_if_policy<Policy> = 0>
-Out uninitialized_copy_n(const Policy& exec, In first, Size n, Out result) { return uninitialized_copy(exec, first, first + n, result); }
+namespace detail {
+template <class Policy, class In, class Size, class Out>
+Out composed_uninitialized_copy_n(const Policy& exec, In first, Size n, Out result) { return uninitialized_copy(exec, first, first + n, result); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class In, class Size, class Out>
+Out uninitialized_copy_n(execution_policy<D_>& exec, In first, Size n, Out result) { return thrust::detail::composed_uninitialized_copy_n(exec, first, n, result); }
+}}  // namespace system::cdna4
+template <class D_, class In, class Size, class Out>
+Out uninitialized_copy_n(const detail::execution_policy_base<D_>& exec, In first, Size n, Out result) { return uninitialized_copy_n(detail::derived_cast(detail::strip_const(exec)), first, n, result); }
+template <class In, class Size, class Out>
+Out uninitialized_copy_n(const system::cpp::detail::par_t& exec, In first, Size n, Out result) { return detail::composed_uninitialized_copy_n(exec, first, n, result); }
 template <class In, class Out> Out uninitialized_copy(In f, In l, Out o) { return copy(f, l, o); }
 template <class In, class Size, class Out, class = typename std::iterator_traits<In>::iterator_category>
 Out uninitialized_copy_n(In f, Size n, Out o) { return copy(f, f + n, o); }

@@ -15,13 +15,23 @@ void uninitialized_fill(const detail::execution_policy_base<D>& exec, It first, 
 }
 template <class It, class T>
 void uninitialized_fill(const system::cpp::detail::par_t&, It first, It last, const T& x) { std::uninitialized_fill(first, last, x); }
-template <class Policy, class It, class Size, class T, detail::enable_if_policy<Policy> = 0>
-It uninitialized_fill_n(const Policy& exec, It first, Size n, const T& x) {
+namespace detail {
+template <class Policy, class It, class Size, class T>
+It composed_uninitialized_fill_n(const Policy& exec, It first, Size n, const T& x) {
   uninitialized_fill(exec, first, first + n, x);
   return first + n;
 }
-template <class It, class T, detail::enable_if_device<It, T> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(device, f, l, x); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class Size, class T>
+It uninitialized_fill_n(execution_policy<D_>& exec, It first, Size n, const T& x) { return thrust::detail::composed_uninitialized_fill_n(exec, first, n, x); }
+}}  // namespace system::cdna4
+template <class D_, class It, class Size, class T>
+It uninitialized_fill_n(const detail::execution_policy_base<D_>& exec, It first, Size n, const T& x) { return uninitialized_fill_n(detail::derived_cast(detail::strip_const(exec)), first, n, x); }
+template <class It, class Size, class T>
+It uninitialized_fill_n(const system::cpp::detail::par_t& exec, It first, Size n, const T& x) { return detail::composed_uninitialized_fill_n(exec, first, n, x); }
+template <class It, class T, detail::enable_if_device<It, T> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(typename detail::implicit_policy<It, T>::type(), f, l, x); }
 template <class It, class T, detail::enable_if_host<It, T> = 0> void uninitialized_fill(It f, It l, const T& x) { uninitialized_fill(host, f, l, x); }
-template <class It, class Size, class T, detail::enable_if_device<It, Size, T> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(device, f, n, x); }
+template <class It, class Size, class T, detail::enable_if_device<It, Size, T> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(typename detail::implicit_policy<It, Size, T>::type(), f, n, x); }
 template <class It, class Size, class T, detail::enable_if_host<It, Size, T> = 0> It uninitialized_fill_n(It f, Size n, const T& x) { return uninitialized_fill_n(host, f, n, x); }
 }  // namespace thrust

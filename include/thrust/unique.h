@@ -67,26 +67,26 @@ pair<KOut, VOut> unique_by_key_copy(const Policy& exec, KIn kfirst, KIn klast, V
   return unique_by_key_copy(exec, kfirst, klast, vfirst, kout, vout, equal_to<typename detail::value_of<KIn>::type>());
 }
 // ---- no policy
-template <class In, detail::enable_if_device<In> = 0> In unique(In f, In l) { return unique(device, f, l); }
+template <class In, detail::enable_if_device<In> = 0> In unique(In f, In l) { return unique(typename detail::implicit_policy<In>::type(), f, l); }
 template <class In, detail::enable_if_host<In> = 0> In unique(In f, In l) { return unique(host, f, l); }
-template <class In, class Eq, detail::enable_if_device<In, Eq> = 0> In unique(In f, In l, Eq eq) { return unique(device, f, l, eq); }
+template <class In, class Eq, detail::enable_if_device<In, Eq> = 0> In unique(In f, In l, Eq eq) { return unique(typename detail::implicit_policy<In, Eq>::type(), f, l, eq); }
 template <class In, class Eq, detail::enable_if_host<In, Eq> = 0> In unique(In f, In l, Eq eq) { return unique(host, f, l, eq); }
-template <class In, class Out, detail::enable_if_device<In, Out> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(device, f, l, o); }
+template <class In, class Out, detail::enable_if_device<In, Out> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(typename detail::implicit_policy<In, Out>::type(), f, l, o); }
 template <class In, class Out, detail::enable_if_host<In, Out> = 0> Out unique_copy(In f, In l, Out o) { return unique_copy(host, f, l, o); }
-template <class K, class V, detail::enable_if_device<K, V> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(device, f, l, v); }
+template <class K, class V, detail::enable_if_device<K, V> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(typename detail::implicit_policy<K, V>::type(), f, l, v); }
 template <class K, class V, detail::enable_if_host<K, V> = 0> pair<K, V> unique_by_key(K f, K l, V v) { return unique_by_key(host, f, l, v); }
 template <class In, class Out, class Eq, detail::enable_if_device<In, Out, Eq> = 0, class = typename std::iterator_traits<Out>::iterator_category>
-Out unique_copy(In f, In l, Out o, Eq eq) { return unique_copy(device, f, l, o, eq); }
+Out unique_copy(In f, In l, Out o, Eq eq) { return unique_copy(typename detail::implicit_policy<In, Out, Eq>::type(), f, l, o, eq); }
 template <class In, class Out, class Eq, detail::enable_if_host<In, Out, Eq> = 0, class = typename std::iterator_traits<Out>::iterator_category>
 Out unique_copy(In f, In l, Out o, Eq eq) { return unique_copy(host, f, l, o, eq); }
-template <class K, class V, class Eq, detail::enable_if_device<K, V, Eq> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(device, f, l, v, eq); }
+template <class K, class V, class Eq, detail::enable_if_device<K, V, Eq> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(typename detail::implicit_policy<K, V, Eq>::type(), f, l, v, eq); }
 template <class K, class V, class Eq, detail::enable_if_host<K, V, Eq> = 0> pair<K, V> unique_by_key(K f, K l, V v, Eq eq) { return unique_by_key(host, f, l, v, eq); }
 template <class K, class V, class KO, class VO, class Eq, detail::enable_if_device<K, V, KO, VO, Eq> = 0>
-pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo, Eq eq) { return unique_by_key_copy(device, f, l, v, ko, vo, eq); }
+pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo, Eq eq) { return unique_by_key_copy(typename detail::implicit_policy<K, V, KO, VO, Eq>::type(), f, l, v, ko, vo, eq); }
 template <class K, class V, class KO, class VO, class Eq, detail::enable_if_host<K, V, KO, VO, Eq> = 0>
 pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo, Eq eq) { return unique_by_key_copy(host, f, l, v, ko, vo, eq); }
 template <class K, class V, class KO, class VO, detail::enable_if_device<K, V, KO, VO> = 0>
-pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(device, f, l, v, ko, vo); }
+pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(typename detail::implicit_policy<K, V, KO, VO>::type(), f, l, v, ko, vo); }
 template <class K, class V, class KO, class VO, detail::enable_if_host<K, V, KO, VO> = 0>
 pair<KO, VO> unique_by_key_copy(K f, K l, V v, KO ko, VO vo) { return unique_by_key_copy(host, f, l, v, ko, vo); }
 
@@ -100,8 +100,9 @@ struct starts_a_run {
   template <class Index> THRUST_CDNA4_HD std::int64_t operator()(Index i) { return eq(p[i], p[i + 1]) ? 0 : 1; }
 };
 }  // namespace detail
-template <class Policy, class It, class Eq, detail::enable_if_policy<Policy> = 0>
-typename std::iterator_traits<It>::difference_type unique_count(const Policy& exec, It first, It last, Eq eq) {
+namespace detail {
+template <class Policy, class It, class Eq>
+typename std::iterator_traits<It>::difference_type composed_unique_count(const Policy& exec, It first, It last, Eq eq) {
   typedef typename std::iterator_traits<It>::difference_type D;
   const std::int64_t n = (std::int64_t)(last - first);
   if (n <= 0) return D(0);
@@ -109,14 +110,33 @@ typename std::iterator_traits<It>::difference_type unique_count(const Policy& ex
   return D(1 + thrust::transform_reduce(exec, counting_iterator<std::int64_t>(0), counting_iterator<std::int64_t>(n - 1),
                                         F{detail::unwrap(first), eq}, std::int64_t(0), plus<std::int64_t>()));
 }
-template <class Policy, class It, detail::enable_if_policy<Policy> = 0>
-typename std::iterator_traits<It>::difference_type unique_count(const Policy& exec, It first, It last) {
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It, class Eq>
+typename std::iterator_traits<It>::difference_type unique_count(execution_policy<D_>& exec, It first, It last, Eq eq) { return thrust::detail::composed_unique_count(exec, first, last, eq); }
+}}  // namespace system::cdna4
+template <class D_, class It, class Eq>
+typename std::iterator_traits<It>::difference_type unique_count(const detail::execution_policy_base<D_>& exec, It first, It last, Eq eq) { return unique_count(detail::derived_cast(detail::strip_const(exec)), first, last, eq); }
+template <class It, class Eq>
+typename std::iterator_traits<It>::difference_type unique_count(const system::cpp::detail::par_t& exec, It first, It last, Eq eq) { return detail::composed_unique_count(exec, first, last, eq); }
+namespace detail {
+template <class Policy, class It>
+typename std::iterator_traits<It>::difference_type composed_unique_count(const Policy& exec, It first, It last) {
   return unique_count(exec, first, last, equal_to<typename detail::value_of<It>::type>());
 }
-template <class It, detail::enable_if_device<It> = 0> typename std::iterator_traits<It>::difference_type unique_count(It f, It l) { return unique_count(device, f, l); }
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D_, class It>
+typename std::iterator_traits<It>::difference_type unique_count(execution_policy<D_>& exec, It first, It last) { return thrust::detail::composed_unique_count(exec, first, last); }
+}}  // namespace system::cdna4
+template <class D_, class It>
+typename std::iterator_traits<It>::difference_type unique_count(const detail::execution_policy_base<D_>& exec, It first, It last) { return unique_count(detail::derived_cast(detail::strip_const(exec)), first, last); }
+template <class It>
+typename std::iterator_traits<It>::difference_type unique_count(const system::cpp::detail::par_t& exec, It first, It last) { return detail::composed_unique_count(exec, first, last); }
+template <class It, detail::enable_if_device<It> = 0> typename std::iterator_traits<It>::difference_type unique_count(It f, It l) { return unique_count(typename detail::implicit_policy<It>::type(), f, l); }
 template <class It, detail::enable_if_host<It> = 0> typename std::iterator_traits<It>::difference_type unique_count(It f, It l) { return unique_count(host, f, l); }
 template <class It, class Eq, detail::enable_if_device<It, Eq> = 0, typename std::enable_if<!detail::is_policy<It>::value, int>::type = 0>
-typename std::iterator_traits<It>::difference_type unique_count(It f, It l, Eq eq) { return unique_count(device, f, l, eq); }
+typename std::iterator_traits<It>::difference_type unique_count(It f, It l, Eq eq) { return unique_count(typename detail::implicit_policy<It, Eq>::type(), f, l, eq); }
 template <class It, class Eq, detail::enable_if_host<It, Eq> = 0, typename std::enable_if<!detail::is_policy<It>::value, int>::type = 0>
 typename std::iterator_traits<It>::difference_type unique_count(It f, It l, Eq eq) { return unique_count(host, f, l, eq); }
 }  // namespace thrust

@@ -60,8 +60,8 @@ auto printable(const T& x) -> decltype(+x) { return +x; }
 template <class T, typename std::enable_if<!std::is_arithmetic<T>::value, int>::type = 0>
 const T& printable(const T& x) { return x; }
 
-template <class T, class U>
-void assert_equal_vec(const std::vector<T>& a, const std::vector<U>& b, const char* expr, const char* file, int line) {
+template <class T, class U, class VecA, class VecB>
+void assert_equal_vec(const VecA& a, const VecB& b, const char* expr, const char* file, int line) {
   if (a.size() != b.size()) {
     std::ostringstream os;
     os << expr << " failed: sizes " << a.size() << " vs " << b.size();
