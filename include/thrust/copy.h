@@ -3,6 +3,7 @@
 #pragma once
 #include <algorithm>
 #include <iterator>
+#include <memory>
 #include <vector>
 #include <thrust/device_ptr.h>
 
@@ -29,20 +30,24 @@ device_ptr<U> copy(device_ptr<T> first, device_ptr<T> last, device_ptr<U> out) {
 template <class T, class OutIt, class = typename std::enable_if<!system::cdna4::detail::is_device_iterator<OutIt>::value>::type>
 OutIt copy(device_ptr<T> first, device_ptr<T> last, OutIt out) {
   typedef typename std::remove_const<T>::type V;
-  std::vector<V> tmp(last - first);
-  system::cdna4::detail::copy_bytes(tmp.data(), first.get(), tmp.size() * sizeof(V), 1);
-  return std::copy(tmp.begin(), tmp.end(), out);
+  const std::size_t n = (std::size_t)(last - first);
+  std::unique_ptr<V[]> tmp(new V[n]);
+  system::cdna4::detail::copy_bytes(tmp.get(), first.get(), n * sizeof(V), 1);
+  return std::copy(tmp.get(), tmp.get() + n, out);
 }
 // host -> device
 template <class InIt, class U, class = typename std::enable_if<!system::cdna4::detail::is_device_iterator<InIt>::value>::type>
 device_ptr<U> copy(InIt first, InIt last, device_ptr<U> out) {
-  std::vector<U> tmp(first, last);
-  system::cdna4::detail::copy_bytes(out.get(), tmp.data(), tmp.size() * sizeof(U), 0);
-  return out + tmp.size();
+  const std::size_t n = (std::size_t)std::distance(first, last);
+  std::unique_ptr<U[]> tmp(new U[n]);  // (not std::vector: its bool specialisation is no array)
+  std::copy(first, last, tmp.get());
+  system::cdna4::detail::copy_bytes(out.get(), tmp.get(), n * sizeof(U), 0);
+  return out + n;
 }
 // host -> host
 template <class InIt, class OutIt,
-          class = typename std::enable_if<!system::cdna4::detail::is_device_iterator<InIt>::value &&
+          class = typename std::enable_if<(!system::cdna4::detail::is_device_iterator<InIt>::value ||
+                                           system::cdna4::detail::is_any_system_iterator<InIt>::value) &&
                                           !system::cdna4::detail::is_device_iterator<OutIt>::value>::type>
 OutIt copy(InIt first, InIt last, OutIt out) {
   return std::copy(first, last, out);
@@ -110,16 +115,41 @@ template <class In, class Out,
           typename std::enable_if<detail::is_fancy_device_iterator<In>::value && system::cdna4::detail::is_device_iterator<Out>::value, int>::type = 0>
 Out copy(In first, In last, Out out) { return copy(typename detail::implicit_policy<In>::type(), first, last, out); }
 template <class In, class Out,
-          typename std::enable_if<detail::is_fancy_device_iterator<In>::value && !system::cdna4::detail::is_device_iterator<Out>::value, long>::type = 0>
+          typename std::enable_if<detail::is_fancy_device_iterator<In>::value && !system::cdna4::detail::is_any_system_iterator<In>::value &&
+                                      !system::cdna4::detail::is_device_iterator<Out>::value, long>::type = 0>
 Out copy(In first, In last, Out out) {
   typedef typename detail::value_of<In>::type V;
   const std::size_t n = (std::size_t)(last - first);
   system::cdna4::detail::temporary_storage staging(n * sizeof(V), static_cast<void*>(nullptr));
   V* tmp = static_cast<V*>(staging.data());
   copy(device, first, last, device_ptr<V>(tmp));
-  std::vector<V> host(n);
-  system::cdna4::detail::copy_bytes(host.data(), tmp, n * sizeof(V), 1);
-  return std::copy(host.begin(), host.end(), out);
+  std::unique_ptr<V[]> host(new V[n]);
+  system::cdna4::detail::copy_bytes(host.get(), tmp, n * sizeof(V), 1);
+  return std::copy(host.get(), host.get() + n, out);
+}
+// The remaining pairs of systems without a policy.  A contiguous device range into a device output
+// that is no plain pointer (a zip or transform-output iterator over device memory, a discard
+// iterator): the device system's copy.
+template <class T, class Out,
+          typename std::enable_if<system::cdna4::detail::is_device_iterator<Out>::value, char>::type = 0>
+Out copy(device_ptr<T> first, device_ptr<T> last, Out out) { return copy(typename detail::implicit_policy<device_ptr<T>, Out>::type(), first, last, out); }
+// A host range (or a counting / constant range) into such an output: a discard iterator drops it on
+// the host; otherwise the elements are staged in device memory and copied there.
+template <class In, class Out,
+          typename std::enable_if<(!system::cdna4::detail::is_device_iterator<In>::value) &&
+                                      system::cdna4::detail::is_device_iterator<Out>::value, short>::type = 0>
+Out copy(In first, In last, Out out) {
+  typedef typename detail::value_of<In>::type V;
+  const std::size_t n = (std::size_t)std::distance(first, last);
+  if (system::cdna4::detail::is_any_system_iterator<Out>::value || n == 0) return out + n;
+  std::unique_ptr<V[]> host(new V[n]);
+  std::copy(first, last, host.get());
+  system::cdna4::detail::temporary_storage staging(n * sizeof(V), static_cast<void*>(nullptr));
+  V* tmp = static_cast<V*>(staging.data());
+  system::cdna4::detail::copy_bytes(tmp, host.get(), n * sizeof(V), 0);
+  Out end = copy(device, device_ptr<V>(tmp), device_ptr<V>(tmp + n), out);
+  system::cdna4::detail::throw_on_error(thrust_cdna4_stream_synchronize(nullptr), "copy");
+  return end;
 }
 namespace detail {
 template <class Policy, class In, class Size, class Out>

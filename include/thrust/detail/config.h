@@ -139,7 +139,23 @@
   noexcept(noexcept(__VA_ARGS__)) -> typename ::std::enable_if<condition, decltype(__VA_ARGS__)>::type \
   { return (__VA_ARGS__); }
 
+// deprecation brackets (thrust/detail/config/deprecated.h:24-60)
+#if defined(__clang__)
+#define THRUST_SUPPRESS_DEPRECATED_PUSH _Pragma("clang diagnostic push") _Pragma("clang diagnostic ignored \"-Wdeprecated-declarations\"")
+#define THRUST_SUPPRESS_DEPRECATED_POP _Pragma("clang diagnostic pop")
+#elif defined(__GNUC__)
+#define THRUST_SUPPRESS_DEPRECATED_PUSH _Pragma("GCC diagnostic push") _Pragma("GCC diagnostic ignored \"-Wdeprecated-declarations\"")
+#define THRUST_SUPPRESS_DEPRECATED_POP _Pragma("GCC diagnostic pop")
+#else
+#define THRUST_SUPPRESS_DEPRECATED_PUSH
+#define THRUST_SUPPRESS_DEPRECATED_POP
+#endif
+
 // alignment of allocations made by the memory resources (thrust/mr/memory_resource.h:36-38)
 #ifndef THRUST_MR_DEFAULT_ALIGNMENT
 #define THRUST_MR_DEFAULT_ALIGNMENT alignof(::std::max_align_t)
 #endif
+
+// the token-pasting and argument-counting macros come with the configuration
+#include <thrust/detail/preprocessor.h>
+#include <thrust/detail/static_assert.h>

@@ -41,3 +41,7 @@ template <class I, class Tag, class... R> struct implicit_policy<tagged_iterator
                                     typename implicit_policy<R...>::type>::type type;
 };
 }}  // namespace thrust::detail
+// For macros that stamp out the no-policy forms of an algorithm for both systems: the policy
+// object of the form, from the types of its iterator arguments.
+#define THRUST_CDNA4_DEVICE_SYS(...) typename ::thrust::detail::implicit_policy<__VA_ARGS__>::type()
+#define THRUST_CDNA4_HOST_SYS(...) ::thrust::host

@@ -3,6 +3,8 @@
 // device_reference is one synchronous element copy, as in the reference
 // (thrust/system/cuda/detail/get_value.h:47-58, assign_value.h).
 #pragma once
+#include <ostream>
+#include <utility>
 #include <cstddef>
 #include <iterator>
 #include <thrust/detail/hd.h>
@@ -37,7 +39,34 @@ class device_reference {
     return *this;
   }
   THRUST_CDNA4_HD device_reference& operator=(const device_reference& o) { return *this = static_cast<value_type>(o); }
+  // from the pointer to the element, and from a reference to an element of a convertible type
+  // (thrust/device_reference.h:224-260)
+  template <class P, class = decltype(static_cast<T*>(std::declval<const P&>().get()))>
+  THRUST_CDNA4_HD explicit device_reference(const P& ptr) : p_(ptr.get()) {}
+  template <class U, class = typename std::enable_if<std::is_convertible<U*, T*>::value && !std::is_same<U, T>::value>::type>
+  THRUST_CDNA4_HD device_reference(const device_reference<U>& o) : p_((&o).get()) {}
+  template <class U, class = typename std::enable_if<!std::is_same<U, T>::value>::type>
+  THRUST_CDNA4_HD device_reference& operator=(const device_reference<U>& o) { return *this = static_cast<value_type>(static_cast<typename device_reference<U>::value_type>(o)); }
   THRUST_CDNA4_HD device_ptr<T> operator&() const { return device_ptr<T>(p_); }
+  // read-modify-write forms (thrust/detail/reference.h:160-420)
+  THRUST_CDNA4_HD device_reference& operator++() { value_type t = *this; ++t; return *this = t; }
+  THRUST_CDNA4_HD value_type operator++(int) { value_type t = *this, old = t; ++t; *this = t; return old; }
+  THRUST_CDNA4_HD device_reference& operator--() { value_type t = *this; --t; return *this = t; }
+  THRUST_CDNA4_HD value_type operator--(int) { value_type t = *this, old = t; --t; *this = t; return old; }
+#define THRUST_CDNA4_REFERENCE_COMPOUND(OP) \
+  template <class U> THRUST_CDNA4_HD device_reference& operator OP(const U& r) { value_type t = *this; t OP r; return *this = t; }
+  THRUST_CDNA4_REFERENCE_COMPOUND(+=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(-=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(*=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(/=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(%=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(<<=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(>>=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(&=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(|=)
+  THRUST_CDNA4_REFERENCE_COMPOUND(^=)
+#undef THRUST_CDNA4_REFERENCE_COMPOUND
+  THRUST_CDNA4_HD void swap(device_reference& o) { value_type a = *this, b = o; *this = b; o = a; }
 
  private:
   T* p_;
@@ -87,6 +116,16 @@ class device_ptr {
   T* p_;
 };
 
+template <class T> THRUST_CDNA4_HD inline void swap(device_reference<T> a, device_reference<T> b) { a.swap(b); }
+// streamed as the element's value and as the raw address (thrust/device_reference.h:975, thrust/device_ptr.h:170)
+template <class Ch, class Tr, class T>
+std::basic_ostream<Ch, Tr>& operator<<(std::basic_ostream<Ch, Tr>& os, const device_reference<T>& r) {
+  return os << static_cast<typename device_reference<T>::value_type>(r);
+}
+template <class Ch, class Tr, class T>
+std::basic_ostream<Ch, Tr>& operator<<(std::basic_ostream<Ch, Tr>& os, const device_ptr<T>& p) {
+  return os << static_cast<const void*>(p.get());
+}
 template <class T> THRUST_CDNA4_HD inline device_ptr<T> device_pointer_cast(T* p) { return device_ptr<T>(p); }
 template <class T> THRUST_CDNA4_HD inline device_ptr<T> device_pointer_cast(device_ptr<T> p) { return p; }
 template <class T> THRUST_CDNA4_HD inline T* raw_pointer_cast(device_ptr<T> p) { return p.get(); }

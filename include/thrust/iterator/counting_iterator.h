@@ -13,6 +13,9 @@ class counting_iterator : public detail::fancy_base<counting_iterator<T, System,
   typedef T reference;
   counting_iterator() : v_() {}
   THRUST_CDNA4_HD explicit counting_iterator(T v) : v_(v) {}
+  // the same counter under another system, traversal or difference parameter
+  template <class S2, class Tr2, class D2>
+  THRUST_CDNA4_HD counting_iterator(const counting_iterator<T, S2, Tr2, D2>& o) : v_(o.base()) {}
   THRUST_CDNA4_HD T at(std::ptrdiff_t n) const { return (T)(v_ + (T)n); }
   THRUST_CDNA4_HD void advance(std::ptrdiff_t n) { v_ = (T)(v_ + (T)n); }
   THRUST_CDNA4_HD std::ptrdiff_t distance_to(const counting_iterator& o) const { return (std::ptrdiff_t)(o.v_ - v_); }

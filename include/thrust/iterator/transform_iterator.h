@@ -6,8 +6,12 @@
 
 namespace thrust {
 namespace detail {
+// a functor that hands its argument back (thrust::identity<>) returns the base's proxy reference:
+// the element type is then what the proxy stands for
+template <class T> struct unproxied { typedef T type; };
+template <class U> struct unproxied<thrust::device_reference<U>> { typedef typename std::remove_const<U>::type type; };
 template <class F, class It> struct transformed_value {
-  typedef typename std::decay<decltype(std::declval<F&>()(std::declval<typename std::iterator_traits<It>::reference>()))>::type type;
+  typedef typename unproxied<typename std::decay<decltype(std::declval<F&>()(std::declval<typename std::iterator_traits<It>::reference>()))>::type>::type type;
 };
 }  // namespace detail
 namespace detail {

@@ -103,14 +103,14 @@ template <class It, class T>
 void replace(const system::cpp::detail::par_t& exec, It first, It last, const T& old_value, const T& new_value) { return detail::composed_replace(exec, first, last, old_value, new_value); }
 
 #define THRUST_CDNA4_REPLACE(SYS, COND)                                                                                       \
-  template <class It, class T, COND<It> = 0> void replace(It f, It l, const T& a, const T& b) { replace(SYS, f, l, a, b); }    \
-  template <class It, class P, class T, COND<It> = 0> void replace_if(It f, It l, P p, const T& v) { replace_if(SYS, f, l, p, v); } \
-  template <class It, class S, class P, class T, COND<It> = 0, class = typename std::iterator_traits<S>::iterator_category>    \
-  void replace_if(It f, It l, S s, P p, const T& v) { replace_if(SYS, f, l, s, p, v); }                                        \
-  template <class In, class Out, class T, COND<In> = 0> Out replace_copy(In f, In l, Out o, const T& a, const T& b) { return replace_copy(SYS, f, l, o, a, b); } \
-  template <class In, class Out, class P, class T, COND<In> = 0> Out replace_copy_if(In f, In l, Out o, P p, const T& v) { return replace_copy_if(SYS, f, l, o, p, v); } \
-  template <class In, class S, class Out, class P, class T, COND<In> = 0> Out replace_copy_if(In f, In l, S s, Out o, P p, const T& v) { return replace_copy_if(SYS, f, l, s, o, p, v); }
-THRUST_CDNA4_REPLACE(device, detail::enable_if_device)
-THRUST_CDNA4_REPLACE(host, detail::enable_if_host)
+  template <class It, class T, COND<It, T> = 0> void replace(It f, It l, const T& a, const T& b) { replace(SYS(It, T), f, l, a, b); }    \
+  template <class It, class P, class T, COND<It, P, T> = 0> void replace_if(It f, It l, P p, const T& v) { replace_if(SYS(It, P, T), f, l, p, v); } \
+  template <class It, class S, class P, class T, COND<It, S, P, T> = 0, class = typename std::iterator_traits<S>::iterator_category>    \
+  void replace_if(It f, It l, S s, P p, const T& v) { replace_if(SYS(It, S, P, T), f, l, s, p, v); }                                        \
+  template <class In, class Out, class T, COND<In, Out, T> = 0> Out replace_copy(In f, In l, Out o, const T& a, const T& b) { return replace_copy(SYS(In, Out, T), f, l, o, a, b); } \
+  template <class In, class Out, class P, class T, COND<In, Out, P, T> = 0> Out replace_copy_if(In f, In l, Out o, P p, const T& v) { return replace_copy_if(SYS(In, Out, P, T), f, l, o, p, v); } \
+  template <class In, class S, class Out, class P, class T, COND<In, S, Out, P, T> = 0> Out replace_copy_if(In f, In l, S s, Out o, P p, const T& v) { return replace_copy_if(SYS(In, S, Out, P, T), f, l, s, o, p, v); }
+THRUST_CDNA4_REPLACE(THRUST_CDNA4_DEVICE_SYS, detail::enable_if_device)
+THRUST_CDNA4_REPLACE(THRUST_CDNA4_HOST_SYS, detail::enable_if_host)
 #undef THRUST_CDNA4_REPLACE
 }  // namespace thrust

@@ -137,7 +137,7 @@ inline std::uint64_t radix_key(double f) {
 }
 template <class K, class Compare, bool Encoded = std::is_floating_point<K>::value && (system::cdna4::detail::order_code<Compare>::value >= 0)>
 struct host_order {
-  Compare comp;
+  mutable Compare comp;
   bool operator()(const K& a, const K& b) const { return comp(a, b); }
 };
 template <class K, class Compare>

@@ -24,7 +24,7 @@ namespace thrust { namespace system { namespace cdna4 { namespace detail {
 template <class In, class Out, class Acc, class Op, bool EXCLUSIVE>
 struct scan_body {
   typedef Acc acc;
-  In in; Out out; Acc init; Op op;
+  In in; Out out; Acc init; mutable Op op;
   __device__ Acc load(std::int64_t i) const { return static_cast<Acc>(in[i]); }
   __device__ Acc combine(const Acc& a, const Acc& b) const { return static_cast<Acc>(op(a, b)); }
   __device__ void store(std::int64_t i, bool has_before, const Acc& before, const Acc& upto) const {
@@ -44,7 +44,7 @@ struct seg_acc {
 template <class KIn, class VIn, class Out, class V, class Pred, class Op, bool EXCLUSIVE>
 struct scan_by_key_body {
   typedef seg_acc<unsigned, V> acc;
-  KIn keys; VIn vals; Out out; V init; Pred pred; Op op;
+  KIn keys; VIn vals; Out out; V init; mutable Pred pred; mutable Op op;
   // a head is an element whose key does not continue its predecessor's segment
   // (thrust/system/detail/sequential/scan_by_key.h:63-83: pred(previous key, key))
   __device__ acc load(std::int64_t i) const {
@@ -68,7 +68,7 @@ struct scan_by_key_body {
 template <class C, class KIn, class VIn, class KOut, class VOut, class V, class Pred, class Op>
 struct reduce_by_key_body {
   typedef seg_acc<C, V> acc;
-  KIn keys; VIn vals; KOut kout; VOut vout; long long* num_runs; std::int64_t n; Pred pred; Op op;
+  KIn keys; VIn vals; KOut kout; VOut vout; long long* num_runs; std::int64_t n; mutable Pred pred; mutable Op op;
   __device__ acc load(std::int64_t i) const {
     const bool head = (i == 0) | !pred(keys[i > 0 ? i - 1 : 0], keys[i]);  // no branch around the loads
     return acc{(C)(head ? 1 : 0), static_cast<V>(vals[i])};

@@ -102,17 +102,17 @@ Out transform_if(const detail::execution_policy_base<D_>& exec, In1 first1, In1 
 template <class In1, class In2, class St, class Out, class Op, class Pred>
 Out transform_if(const system::cpp::detail::par_t& exec, In1 first1, In1 last1, In2 first2, St stencil, Out result, Op op, Pred pred) { return detail::composed_transform_if(exec, first1, last1, first2, stencil, result, op, pred); }
 #define THRUST_CDNA4_TRANSFORM_IF_NO_POLICY(SYS, COND)                                                                         \
-  template <class In, class Out, class Op, class Pred, COND<In> = 0>                                                           \
-  Out transform_if(In first, In last, Out result, Op op, Pred pred) { return transform_if(SYS, first, last, result, op, pred); } \
-  template <class In, class St, class Out, class Op, class Pred, COND<In> = 0>                                                 \
+  template <class In, class Out, class Op, class Pred, COND<In, Out, Op, Pred> = 0>                                                           \
+  Out transform_if(In first, In last, Out result, Op op, Pred pred) { return transform_if(SYS(In, Out, Op, Pred), first, last, result, op, pred); } \
+  template <class In, class St, class Out, class Op, class Pred, COND<In, St, Out, Op, Pred> = 0>                                                 \
   Out transform_if(In first, In last, St stencil, Out result, Op op, Pred pred) {                                              \
-    return transform_if(SYS, first, last, stencil, result, op, pred);                                                          \
+    return transform_if(SYS(In, St, Out, Op, Pred), first, last, stencil, result, op, pred);                                                          \
   }                                                                                                                            \
-  template <class In1, class In2, class St, class Out, class Op, class Pred, COND<In1> = 0>                                    \
+  template <class In1, class In2, class St, class Out, class Op, class Pred, COND<In1, In2, St, Out, Op, Pred> = 0>                                    \
   Out transform_if(In1 first1, In1 last1, In2 first2, St stencil, Out result, Op op, Pred pred) {                              \
-    return transform_if(SYS, first1, last1, first2, stencil, result, op, pred);                                                \
+    return transform_if(SYS(In1, In2, St, Out, Op, Pred), first1, last1, first2, stencil, result, op, pred);                                                \
   }
-THRUST_CDNA4_TRANSFORM_IF_NO_POLICY(device, detail::enable_if_device)
-THRUST_CDNA4_TRANSFORM_IF_NO_POLICY(host, detail::enable_if_host)
+THRUST_CDNA4_TRANSFORM_IF_NO_POLICY(THRUST_CDNA4_DEVICE_SYS, detail::enable_if_device)
+THRUST_CDNA4_TRANSFORM_IF_NO_POLICY(THRUST_CDNA4_HOST_SYS, detail::enable_if_host)
 #undef THRUST_CDNA4_TRANSFORM_IF_NO_POLICY
 }  // namespace thrust

@@ -40,7 +40,7 @@ struct tuple_impl<std::index_sequence<Is...>, Ts...> : tuple_leaf<Is, Ts>... {
   THRUST_CDNA4_HD constexpr tuple_impl(const Ts&... vs) : tuple_leaf<Is, Ts>{vs}... {}
   template <class... Us>
   THRUST_CDNA4_HD constexpr tuple_impl(const tuple_impl<std::index_sequence<Is...>, Us...>& o)
-      : tuple_leaf<Is, Ts>{static_cast<const tuple_leaf<Is, Us>&>(o).value}... {}
+      : tuple_leaf<Is, Ts>{static_cast<Ts>(static_cast<const tuple_leaf<Is, Us>&>(o).value)}... {}
   template <class... Us>
   THRUST_CDNA4_HD void assign(const tuple_impl<std::index_sequence<Is...>, Us...>& o) {
     int unused[] = {0, ((void)(static_cast<tuple_leaf<Is, Ts>&>(*this).value = static_cast<const tuple_leaf<Is, Us>&>(o).value), 0)...};
@@ -188,4 +188,10 @@ template <class... Ts, class... Us>
 THRUST_CDNA4_HD constexpr bool operator<(const tuple<Ts...>& a, const tuple<Us...>& b) {
   return detail::tuple_less<0, sizeof...(Ts)>::run(a, b);
 }
+template <class... Ts, class... Us>
+THRUST_CDNA4_HD constexpr bool operator>(const tuple<Ts...>& a, const tuple<Us...>& b) { return b < a; }
+template <class... Ts, class... Us>
+THRUST_CDNA4_HD constexpr bool operator<=(const tuple<Ts...>& a, const tuple<Us...>& b) { return !(b < a); }
+template <class... Ts, class... Us>
+THRUST_CDNA4_HD constexpr bool operator>=(const tuple<Ts...>& a, const tuple<Us...>& b) { return !(a < b); }
 }  // namespace thrust
