@@ -38,6 +38,8 @@ struct alignas(2 * sizeof(T)) complex {
   THRUST_CDNA4_HD T imag() const volatile { return data_[1]; }
   THRUST_CDNA4_HD void real(T re) { data_[0] = re; }
   THRUST_CDNA4_HD void imag(T im) { data_[1] = im; }
+  THRUST_CDNA4_HD void real(T re) volatile { data_[0] = re; }
+  THRUST_CDNA4_HD void imag(T im) volatile { data_[1] = im; }
   operator std::complex<T>() const { return std::complex<T>(real(), imag()); }
 
   template <class U> THRUST_CDNA4_HD complex& operator+=(const complex<U>& z) { data_[0] += T(z.real()); data_[1] += T(z.imag()); return *this; }

@@ -20,11 +20,20 @@ inline void copy_bytes(void* dst, const void* src, std::size_t bytes, int kind) 
 }}}  // namespace system::cdna4::detail
 
 // device -> device
+namespace detail {
 template <class T, class U>
-device_ptr<U> copy(device_ptr<T> first, device_ptr<T> last, device_ptr<U> out) {
-  static_assert(std::is_same<typename std::remove_const<T>::type, U>::value, "element types must match");
+device_ptr<U> copy_device_range(device_ptr<T> first, device_ptr<T> last, device_ptr<U> out, std::true_type) {
   system::cdna4::detail::copy_bytes(out.get(), first.get(), (last - first) * sizeof(U), 2);
   return out + (last - first);
+}
+// another element type: converted element by element on the device (defined below, once the device
+// system's copy is declared)
+template <class T, class U>
+device_ptr<U> copy_device_range(device_ptr<T> first, device_ptr<T> last, device_ptr<U> out, std::false_type);
+}  // namespace detail
+template <class T, class U>
+device_ptr<U> copy(device_ptr<T> first, device_ptr<T> last, device_ptr<U> out) {
+  return detail::copy_device_range(first, last, out, std::is_same<typename std::remove_const<T>::type, U>());
 }
 // device -> host (contiguous host output: raw pointer or vector iterator)
 template <class T, class OutIt, class = typename std::enable_if<!system::cdna4::detail::is_device_iterator<OutIt>::value>::type>
@@ -127,6 +136,12 @@ Out copy(In first, In last, Out out) {
   system::cdna4::detail::copy_bytes(host.get(), tmp, n * sizeof(V), 1);
   return std::copy(host.get(), host.get() + n, out);
 }
+namespace detail {
+template <class T, class U>
+device_ptr<U> copy_device_range(device_ptr<T> first, device_ptr<T> last, device_ptr<U> out, std::false_type) {
+  return copy(device, first, last, out);
+}
+}  // namespace detail
 // The remaining pairs of systems without a policy.  A contiguous device range into a device output
 // that is no plain pointer (a zip or transform-output iterator over device memory, a discard
 // iterator): the device system's copy.

@@ -78,10 +78,17 @@ THRUST_CDNA4_PH_BINARY_OP(op_mod_assign, a %= b)
 THRUST_CDNA4_PH_BINARY_OP(op_and_assign, a &= b)
 THRUST_CDNA4_PH_BINARY_OP(op_or_assign, a |= b)
 THRUST_CDNA4_PH_BINARY_OP(op_xor_assign, a ^= b)
+THRUST_CDNA4_PH_BINARY_OP(op_shl_assign, a <<= b)
+THRUST_CDNA4_PH_BINARY_OP(op_shr_assign, a >>= b)
 #undef THRUST_CDNA4_PH_BINARY_OP
 struct op_negate { template <class A> THRUST_CDNA4_HD constexpr decltype(auto) operator()(A&& a) const { return -a; } };
 struct op_not { template <class A> THRUST_CDNA4_HD constexpr decltype(auto) operator()(A&& a) const { return !a; } };
 struct op_bit_not { template <class A> THRUST_CDNA4_HD constexpr decltype(auto) operator()(A&& a) const { return ~a; } };
+struct op_unary_plus { template <class A> THRUST_CDNA4_HD constexpr decltype(auto) operator()(A&& a) const { return +a; } };
+struct op_pre_inc { template <class A> THRUST_CDNA4_HD constexpr decltype(auto) operator()(A&& a) const { return ++a; } };
+struct op_pre_dec { template <class A> THRUST_CDNA4_HD constexpr decltype(auto) operator()(A&& a) const { return --a; } };
+struct op_post_inc { template <class A> THRUST_CDNA4_HD constexpr decltype(auto) operator()(A&& a) const { return a++; } };
+struct op_post_dec { template <class A> THRUST_CDNA4_HD constexpr decltype(auto) operator()(A&& a) const { return a--; } };
 
 template <class E>
 struct actor : E {
@@ -101,6 +108,8 @@ struct actor : E {
   THRUST_CDNA4_PH_ASSIGN(&=, op_and_assign)
   THRUST_CDNA4_PH_ASSIGN(|=, op_or_assign)
   THRUST_CDNA4_PH_ASSIGN(^=, op_xor_assign)
+  THRUST_CDNA4_PH_ASSIGN(<<=, op_shl_assign)
+  THRUST_CDNA4_PH_ASSIGN(>>=, op_shr_assign)
 #undef THRUST_CDNA4_PH_ASSIGN
 };
 
@@ -135,6 +144,11 @@ THRUST_CDNA4_PH_OPERATOR(>>, op_shr)
 template <class E> THRUST_CDNA4_HD constexpr actor<unary_expr<op_negate, E>> operator-(const actor<E>& e) { return actor<unary_expr<op_negate, E>>(unary_expr<op_negate, E>{e}); }
 template <class E> THRUST_CDNA4_HD constexpr actor<unary_expr<op_not, E>> operator!(const actor<E>& e) { return actor<unary_expr<op_not, E>>(unary_expr<op_not, E>{e}); }
 template <class E> THRUST_CDNA4_HD constexpr actor<unary_expr<op_bit_not, E>> operator~(const actor<E>& e) { return actor<unary_expr<op_bit_not, E>>(unary_expr<op_bit_not, E>{e}); }
+template <class E> THRUST_CDNA4_HD constexpr actor<unary_expr<op_unary_plus, E>> operator+(const actor<E>& e) { return actor<unary_expr<op_unary_plus, E>>(unary_expr<op_unary_plus, E>{e}); }
+template <class E> THRUST_CDNA4_HD constexpr actor<unary_expr<op_pre_inc, E>> operator++(const actor<E>& e) { return actor<unary_expr<op_pre_inc, E>>(unary_expr<op_pre_inc, E>{e}); }
+template <class E> THRUST_CDNA4_HD constexpr actor<unary_expr<op_pre_dec, E>> operator--(const actor<E>& e) { return actor<unary_expr<op_pre_dec, E>>(unary_expr<op_pre_dec, E>{e}); }
+template <class E> THRUST_CDNA4_HD constexpr actor<unary_expr<op_post_inc, E>> operator++(const actor<E>& e, int) { return actor<unary_expr<op_post_inc, E>>(unary_expr<op_post_inc, E>{e}); }
+template <class E> THRUST_CDNA4_HD constexpr actor<unary_expr<op_post_dec, E>> operator--(const actor<E>& e, int) { return actor<unary_expr<op_post_dec, E>>(unary_expr<op_post_dec, E>{e}); }
 
 }}  // namespace detail::functional
 

@@ -93,6 +93,8 @@ class device_ptr {
   template <class U, class = typename std::enable_if<std::is_convertible<U*, T*>::value>::type>
   THRUST_CDNA4_HD device_ptr(const device_ptr<U>& o) : p_(o.get()) {}
   THRUST_CDNA4_HD T* get() const { return p_; }
+  // member access: in a kernel, and on the host for memory the host can address (universal memory)
+  THRUST_CDNA4_HD T* operator->() const { return p_; }
   THRUST_CDNA4_HD reference operator*() const { return reference(p_); }
   THRUST_CDNA4_HD reference operator[](difference_type i) const { return reference(p_ + i); }
   THRUST_CDNA4_HD device_ptr& operator++() { ++p_; return *this; }

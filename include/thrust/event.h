@@ -168,6 +168,9 @@ class device_future : public device_event {
 // is that system's unique eager one, and this build has one device system
 template <class System> using unique_eager_event = device_event;
 template <class T, class System> using unique_eager_future = device_future<T>;
+// the default event and future of a system (thrust/event.h:21-26, thrust/future.h:150-160)
+template <class System> using event = unique_eager_event<System>;
+template <class T, class System> using future = unique_eager_future<T, System>;
 typedef device_event device_unique_eager_event;
 template <class T> using device_unique_eager_future = device_future<T>;
 

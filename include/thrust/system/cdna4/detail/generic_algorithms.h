@@ -47,7 +47,10 @@ template <class In1, class In2, class Out, class F> struct transform2_body {
 };
 template <class Out, class T> struct sequence_body {
   Out out; T init, step;
-  __device__ void operator()(std::int64_t i) { out[i] = (T)(init + (T)i * step); }
+  __device__ void operator()(std::int64_t i) { out[i] = at(i, std::is_arithmetic<T>()); }
+  __device__ T at(std::int64_t i, std::true_type) const { return (T)(init + (T)i * step); }
+  // a number-like class: init + step * i with the index as it is (thrust/system/detail/generic/sequence.inl:36-60)
+  __device__ T at(std::int64_t i, std::false_type) const { return init + step * (std::size_t)i; }
 };
 template <class In, class F, class T> struct load_transform {
   In in; mutable F f;

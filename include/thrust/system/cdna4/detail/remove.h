@@ -6,18 +6,36 @@
 namespace thrust {
 namespace system { namespace cdna4 {
 // the device system's implementations, found through the policy's type
+namespace detail {
+// a contiguous input is read through a pointer to const; any other iterator as it is
+template <class T> inline const T* as_input(T* p) { return p; }
+template <class It> inline It as_input(It it) { return it; }
+template <class Policy, class In, class Pred>
+In remove_if_in_place(const Policy& exec, In first, In last, Pred pred, std::true_type /* contiguous */) {
+  typedef typename thrust::detail::value_of<In>::type V;
+  const std::int64_t n = (std::int64_t)(last - first);
+  scratch_copy<V> tmp((const V*)thrust::detail::unwrap(first), n, stream_of(exec));
+  return first + copy_flagged_n<true>(exec, tmp.data(), thrust::detail::unwrap(first), n, pred);
+}
+// a range that is no array (a zip of arrays, say): its elements are gathered into a temporary first
+template <class Policy, class In, class Pred>
+In remove_if_in_place(const Policy& exec, In first, In last, Pred pred, std::false_type) {
+  typedef typename thrust::detail::value_of<In>::type V;
+  const std::int64_t n = (std::int64_t)(last - first);
+  temporary_storage buf((std::size_t)n * sizeof(V), exec);
+  V* tmp = static_cast<V*>(buf.data());
+  thrust::copy(exec, first, last, thrust::device_ptr<V>(tmp));
+  return first + copy_flagged_n<true>(exec, (const V*)tmp, thrust::detail::unwrap(first), n, pred);
+}
+}  // namespace detail
 template <class D, class In, class Out, class Pred>
 Out remove_copy_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out, Pred pred) {
-  typedef typename thrust::detail::value_of<In>::type V;
-  const V* in = thrust::detail::unwrap(first);
-  return out + system::cdna4::detail::copy_flagged_n<true>(exec.derived(), in, thrust::detail::unwrap(out), (std::int64_t)(last - first), pred);
+  return out + system::cdna4::detail::copy_flagged_n<true>(exec.derived(), detail::as_input(thrust::detail::unwrap(first)), thrust::detail::unwrap(out),
+                                                           (std::int64_t)(last - first), pred);
 }
 template <class D, class In, class Pred>
 In remove_if(const system::cdna4::execution_policy<D>& exec, In first, In last, Pred pred) {
-  typedef typename thrust::detail::value_of<In>::type V;
-  const std::int64_t n = (std::int64_t)(last - first);
-  system::cdna4::detail::scratch_copy<V> tmp((const V*)thrust::detail::unwrap(first), n, system::cdna4::detail::stream_of(exec.derived()));
-  return first + system::cdna4::detail::copy_flagged_n<true>(exec.derived(), tmp.data(), thrust::detail::unwrap(first), n, pred);
+  return detail::remove_if_in_place(exec.derived(), first, last, pred, std::is_pointer<typename thrust::detail::unwrap_iterator<In>::type>());
 }
 }}  // namespace system::cdna4
 }  // namespace thrust

@@ -84,9 +84,13 @@ template <> struct tuple<> {};
 template <std::size_t I, class T> struct tuple_element;
 template <std::size_t I, class... Ts> struct tuple_element<I, tuple<Ts...>> { typedef typename detail::nth_type<I, Ts...>::type type; };
 template <std::size_t I, class T> struct tuple_element<I, const T> { typedef typename std::add_const<typename tuple_element<I, T>::type>::type type; };
+template <std::size_t I, class T> struct tuple_element<I, volatile T> { typedef typename std::add_volatile<typename tuple_element<I, T>::type>::type type; };
+template <std::size_t I, class T> struct tuple_element<I, const volatile T> { typedef typename std::add_cv<typename tuple_element<I, T>::type>::type type; };
 template <class T> struct tuple_size;
 template <class... Ts> struct tuple_size<tuple<Ts...>> : std::integral_constant<std::size_t, sizeof...(Ts)> {};
 template <class T> struct tuple_size<const T> : tuple_size<T> {};
+template <class T> struct tuple_size<volatile T> : tuple_size<T> {};
+template <class T> struct tuple_size<const volatile T> : tuple_size<T> {};
 
 template <std::size_t I, class... Ts>
 THRUST_CDNA4_HD constexpr typename detail::nth_type<I, Ts...>::type& get(tuple<Ts...>& t) {

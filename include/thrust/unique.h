@@ -34,7 +34,18 @@ pair<KIn, VIn> unique_by_key(const detail::execution_policy_base<D>& exec, KIn k
 }
 // ---- host
 template <class In, class Out, class Eq>
-Out unique_copy(const system::cpp::detail::par_t&, In first, In last, Out out, Eq eq) { return std::unique_copy(first, last, out, eq); }
+Out unique_copy(const system::cpp::detail::par_t&, In first, In last, Out out, Eq eq) {
+  // the last element kept is held in a variable, so that the output is only ever written
+  // (thrust/system/detail/sequential/unique.h:38-66) — it may be a discard iterator
+  if (first == last) return out;
+  typename std::iterator_traits<In>::value_type kept = *first;
+  *out = kept; ++out;
+  for (++first; first != last; ++first) {
+    typename std::iterator_traits<In>::value_type x = *first;
+    if (!eq(kept, x)) { kept = x; *out = kept; ++out; }
+  }
+  return out;
+}
 template <class In, class Eq>
 In unique(const system::cpp::detail::par_t&, In first, In last, Eq eq) { return std::unique(first, last, eq); }
 template <class KIn, class VIn, class KOut, class VOut, class Eq>
