@@ -167,8 +167,13 @@ Out copy(In first, In last, Out out) {
   return end;
 }
 namespace detail {
+// first + n, also for iterators that only step (a std::list's)
+template <class It, class N> inline auto plus_n(It it, N n, int) -> decltype(It(it + n)) { return it + n; }
+template <class It, class N> inline It plus_n(It it, N n, long) { std::advance(it, n); return it; }
+}  // namespace detail
+namespace detail {
 template <class Policy, class In, class Size, class Out>
-Out composed_copy_n(const Policy& exec, In first, Size n, Out out) { return thrust::copy(exec, first, first + n, out); }
+Out composed_copy_n(const Policy& exec, In first, Size n, Out out) { return thrust::copy(exec, first, detail::plus_n(first, n, 0), out); }
 }  // namespace detail
 namespace system { namespace cdna4 {
 template <class D_, class In, class Size, class Out>
@@ -179,5 +184,5 @@ Out copy_n(const detail::execution_policy_base<D_>& exec, In first, Size n, Out 
 template <class In, class Size, class Out>
 Out copy_n(const system::cpp::detail::par_t& exec, In first, Size n, Out out) { return detail::composed_copy_n(exec, first, n, out); }
 template <class In, class Size, class Out, typename std::enable_if<!detail::is_policy<In>::value, int>::type = 0>
-Out copy_n(In first, Size n, Out out) { return thrust::copy(first, first + n, out); }
+Out copy_n(In first, Size n, Out out) { return thrust::copy(first, detail::plus_n(first, n, 0), out); }
 }  // namespace thrust

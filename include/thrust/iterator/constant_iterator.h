@@ -27,6 +27,12 @@ class constant_iterator : public detail::fancy_base<constant_iterator<T, Increme
   T v_;
   index_type pos_;
 };
+// positions subtract across index and system parameters
+template <class T1, class I1, class S1, class T2, class I2, class S2,
+          class = typename std::enable_if<!std::is_same<constant_iterator<T1, I1, S1>, constant_iterator<T2, I2, S2>>::value>::type>
+THRUST_CDNA4_HD std::ptrdiff_t operator-(const constant_iterator<T1, I1, S1>& a, const constant_iterator<T2, I2, S2>& b) {
+  return (std::ptrdiff_t)*a.base() - (std::ptrdiff_t)*b.base();
+}
 template <class T> THRUST_CDNA4_HD constant_iterator<T> make_constant_iterator(T v) { return constant_iterator<T>(v); }
 template <class T, class I> THRUST_CDNA4_HD constant_iterator<T, I> make_constant_iterator(T v, I pos) { return constant_iterator<T, I>(v, pos); }
 namespace system { namespace cdna4 { namespace detail {

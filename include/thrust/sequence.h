@@ -13,11 +13,15 @@ template <class D, class It, class T>
 void sequence(const detail::execution_policy_base<D>& exec, It first, It last, T init, T step) {
   sequence(detail::derived_cast(detail::strip_const(exec)), first, last, init, step);
 }
+namespace detail {
+// element i, computed in the type of init and step (thrust/system/detail/generic/sequence.inl:36-60)
+template <class T> inline T sequence_value(const T& init, const T& step, std::size_t i, std::true_type) { return (T)(init + (T)i * step); }
+template <class T> inline T sequence_value(const T& init, const T& step, std::size_t i, std::false_type) { return init + step * i; }
+}  // namespace detail
 template <class It, class T>
 void sequence(const system::cpp::detail::par_t&, It first, It last, T init, T step) {
-  typedef typename detail::value_of<It>::type V;
   std::size_t i = 0;
-  for (; first != last; ++first, ++i) *first = (V)((V)init + (V)i * (V)step);
+  for (; first != last; ++first, ++i) *first = detail::sequence_value(init, step, i, std::is_arithmetic<T>());
 }
 template <class Policy, class It, class T>
 void sequence(const Policy& exec, It first, It last, T init) { sequence(exec, first, last, init, T(1)); }

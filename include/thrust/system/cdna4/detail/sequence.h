@@ -8,8 +8,9 @@ namespace system { namespace cdna4 {
 // the device system's implementations, found through the policy's type
 template <class D, class It, class T>
 void sequence(const system::cdna4::execution_policy<D>& exec, It first, It last, T init, T step) {
-  typedef typename thrust::detail::value_of<It>::type V;
-  system::cdna4::detail::sequence_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)(last - first), (V)init, (V)step);
+  // computed in the type of init and step, converted where it is stored
+  // (thrust/system/detail/generic/sequence.inl:36-90)
+  system::cdna4::detail::sequence_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)(last - first), init, step);
 }
 }}  // namespace system::cdna4
 }  // namespace thrust

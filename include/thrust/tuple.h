@@ -10,6 +10,7 @@
 
 namespace thrust {
 template <class... Ts> struct tuple;
+template <class T1, class T2> struct pair;
 // the type the reference's ten-parameter tuple pads itself with (thrust/tuple.h:50); this tuple is
 // variadic and has no use for it beyond existing code that names it
 struct null_type {};
@@ -70,6 +71,20 @@ struct tuple : detail::tuple_impl<std::index_sequence_for<Ts...>, Ts...> {
   template <class... Us>
   THRUST_CDNA4_HD tuple& operator=(const tuple<Us...>& o) {
     base::assign(static_cast<const typename tuple<Us...>::base&>(o));
+    return *this;
+  }
+  // a tuple of two from and to a pair (thrust/tuple.h: tuple<T0, T1>::operator=(const pair<U1, U2>&))
+  template <class U1, class U2, class = typename std::enable_if<sizeof...(Ts) == 2 && (sizeof(U1) > 0)>::type>
+  THRUST_CDNA4_HD constexpr tuple(const pair<U1, U2>& p) : base(p.first, p.second) {}
+  template <class U1, class U2>
+  THRUST_CDNA4_HD tuple& operator=(const pair<U1, U2>& p) {
+    static_cast<detail::tuple_leaf<0, typename detail::nth_type<0, Ts...>::type>&>(*this).value = p.first;
+    static_cast<detail::tuple_leaf<1, typename detail::nth_type<1, Ts...>::type>&>(*this).value = p.second;
+    return *this;
+  }
+  template <class U1, class U2>
+  THRUST_CDNA4_HD const tuple& operator=(const pair<U1, U2>& p) const {
+    *const_cast<tuple*>(this) = p;
     return *this;
   }
   // a tuple of references assigns through them, also when it is a temporary
@@ -170,6 +185,25 @@ template <class T0, class T1, class T2, class T3, class T4, class T5, class T6, 
 THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&> tie(T0& v0, T1& v1, T2& v2, T3& v3, T4& v4, T5& v5, T6& v6, T7& v7, T8& v8) { return tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&>(v0, v1, v2, v3, v4, v5, v6, v7, v8); }
 template <class T0, class T1, class T2, class T3, class T4, class T5, class T6, class T7, class T8, class T9>
 THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&, T9&> tie(T0& v0, T1& v1, T2& v2, T3& v3, T4& v4, T5& v5, T6& v6, T7& v7, T8& v8, T9& v9) { return tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&, T9&>(v0, v1, v2, v3, v4, v5, v6, v7, v8, v9); }
+
+// swap: element by element; tuples of references (what a zip_iterator yields) are taken by value
+// and swap what they refer to
+namespace detail {
+template <std::size_t I, std::size_t N> struct tuple_swap {
+  template <class A, class B> THRUST_CDNA4_HD static void run(A& a, B& b) {
+    using std::swap;
+    swap(get<I>(a), get<I>(b));
+    tuple_swap<I + 1, N>::run(a, b);
+  }
+};
+template <std::size_t N> struct tuple_swap<N, N> {
+  template <class A, class B> THRUST_CDNA4_HD static void run(A&, B&) {}
+};
+}  // namespace detail
+template <class... Ts>
+THRUST_CDNA4_HD void swap(tuple<Ts...>& a, tuple<Ts...>& b) { detail::tuple_swap<0, sizeof...(Ts)>::run(a, b); }
+template <class... Ts>
+THRUST_CDNA4_HD void swap(tuple<Ts&...>&& a, tuple<Ts&...>&& b) { detail::tuple_swap<0, sizeof...(Ts)>::run(a, b); }
 
 template <class... Ts, class... Us>
 THRUST_CDNA4_HD constexpr bool operator==(const tuple<Ts...>& a, const tuple<Us...>& b) {
