@@ -28,6 +28,7 @@
 #include <cstdint>
 #include <type_traits>
 #include <thrust/system/cdna4/detail/core.h>
+#include <thrust/system/cdna4/detail/parallel_for.h>
 
 namespace thrust { namespace system { namespace cdna4 { namespace detail { namespace merge {
 
@@ -391,10 +392,77 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(const K* kin, const V* vi
 // ---------------------------------------------------------------------------------------
 inline std::size_t align256(std::size_t x) { return (x + 255) & ~std::size_t(255); }
 
+// Whether tiles of K (and V) can live in the static LDS arrays of the kernels above: half a sort
+// tile and a whole merge tile must fit 64 KiB, and LDS arrays cannot hold a type whose default
+// constructor or destructor does anything.
+template <class K, class V>
+constexpr bool tiles_fit_lds() {
+  constexpr bool has_values = !std::is_same<V, no_value>::value;
+  constexpr std::size_t vsize = has_values ? sizeof(V) : 0;
+  constexpr int IPT = items_per_thread<K, V>();
+  return std::is_trivially_default_constructible<K>::value && std::is_trivially_destructible<K>::value &&
+         std::is_trivially_default_constructible<V>::value && std::is_trivially_destructible<V>::value &&
+         (sizeof(K) + vsize + 2) * kBlock * IPT <= 65536 && (2 * sizeof(K) + 4 + vsize) * kBlock * (IPT / 2) <= 65536;
+}
+
+template <class K, class V, class Compare>
+void stable_sort_tiles(void* stream_, K* keys, V* values, std::int64_t n, Compare comp);
+
+// Wide or non-trivial elements (the reference sorts keys and values of 8 KiB each,
+// testing/stable_sort_by_key_large_keys_and_values.cu): their positions are sorted instead, under
+// a comparison that reads the keys where they lie, and keys and values are then gathered once.
+// Positions of equivalent keys stay in their order, so the sort is stable.
+template <class I, class K, class Compare> struct compare_at {
+  const K* keys; mutable Compare comp;
+  __device__ bool operator()(I a, I b) const { return comp(keys[a], keys[b]); }
+};
+template <class I> struct iota_body {
+  I* out;
+  __device__ void operator()(std::int64_t i) const { out[i] = (I)i; }
+};
+template <class I, class T> struct gather_body {
+  const T* in; const I* at; T* out;
+  __device__ void operator()(std::int64_t i) const { out[i] = in[at[i]]; }
+};
+template <class I, class K, class V, class Compare>
+void stable_sort_positions(void* stream_, K* keys, V* values, std::int64_t n, Compare comp) {
+  constexpr bool kHasValues = !std::is_same<V, no_value>::value;
+  const std::size_t ibytes = align256((std::size_t)n * sizeof(I));
+  const std::size_t kbytes = align256((std::size_t)n * sizeof(K));
+  const std::size_t vbytes = kHasValues ? align256((std::size_t)n * sizeof(V)) : 0;
+  temporary_storage tmp(ibytes + kbytes + vbytes, stream_);
+  char* t = static_cast<char*>(tmp.data());
+  I* at = reinterpret_cast<I*>(t);
+  K* kcopy = reinterpret_cast<K*>(t + ibytes);
+  V* vcopy = reinterpret_cast<V*>(t + ibytes + kbytes);
+  generic::parallel_for(stream_, n, iota_body<I>{at});
+  stable_sort_tiles<I, no_value>(stream_, at, static_cast<no_value*>(nullptr), n, compare_at<I, K, Compare>{keys, comp});
+  generic::parallel_for(stream_, n, gather_body<I, K>{keys, at, kcopy});
+  throw_on_error(thrust_cdna4_memcpy_dtod(keys, kcopy, (std::size_t)n * sizeof(K), stream_), "merge sort: copy back");
+  if (kHasValues) {
+    generic::parallel_for(stream_, n, gather_body<I, V>{values, at, vcopy});
+    throw_on_error(thrust_cdna4_memcpy_dtod(values, vcopy, (std::size_t)n * sizeof(V), stream_), "merge sort: copy back");
+  }
+}
+template <class K, class V, class Compare>
+void stable_sort_dispatch(void* stream_, K* keys, V* values, std::int64_t n, Compare comp, std::true_type /* tiles fit */) {
+  stable_sort_tiles(stream_, keys, values, n, comp);
+}
+template <class K, class V, class Compare>
+void stable_sort_dispatch(void* stream_, K* keys, V* values, std::int64_t n, Compare comp, std::false_type) {
+  if (n <= 1) return;
+  if (n <= (std::int64_t)0xFFFFFFFFll) stable_sort_positions<std::uint32_t>(stream_, keys, values, n, comp);
+  else stable_sort_positions<std::uint64_t>(stream_, keys, values, n, comp);
+}
 template <class K, class V, class Compare>
 void stable_sort(void* stream_, K* keys, V* values, std::int64_t n, Compare comp) {
   static_assert(thrust::detail::is_bytewise_movable<K>::value, "cdna4 merge sort: keys must be movable as bytes");
   static_assert(thrust::detail::is_bytewise_movable<V>::value, "cdna4 merge sort: values must be movable as bytes");
+  stable_sort_dispatch(stream_, keys, values, n, comp, std::integral_constant<bool, tiles_fit_lds<K, V>()>());
+}
+
+template <class K, class V, class Compare>
+void stable_sort_tiles(void* stream_, K* keys, V* values, std::int64_t n, Compare comp) {
   constexpr int IPT = items_per_thread<K, V>();
   constexpr int kTile = kBlock * IPT;
   constexpr bool kHasValues = !std::is_same<V, no_value>::value;

@@ -232,4 +232,88 @@ DECLARE_TYPED_UNITTEST(TestStableSortOffsetRanges, uint16_t);
 DECLARE_TYPED_UNITTEST(TestStableSortOffsetRanges, unsigned);
 DECLARE_TYPED_UNITTEST(TestStableSortOffsetRanges, int64_t);
 
+// testing/stable_sort_large.cu, stable_sort_by_key_large_keys.cu, ..._large_keys_and_values.cu:
+// keys and values of N ints, ordered by their first; N up to 2048 ints (8 KiB) an element.  Wider
+// than an LDS tile allows, so positions are sorted and the elements gathered.
+template <int N>
+struct fixed_vector {
+  int v[N];
+  __host__ __device__ fixed_vector() { for (int i = 0; i < N; i++) v[i] = 0; }
+  __host__ __device__ explicit fixed_vector(int x) { for (int i = 0; i < N; i++) v[i] = x; }
+  __host__ __device__ bool operator<(const fixed_vector& o) const { return v[0] < o.v[0]; }
+  __host__ __device__ bool operator==(const fixed_vector& o) const {
+    for (int i = 0; i < N; i++) if (v[i] != o.v[i]) return false;
+    return true;
+  }
+};
+template <int N> inline std::ostream& operator<<(std::ostream& os, const fixed_vector<N>& f) { return os << "fixed_vector(" << f.v[0] << ")"; }
+template <int N>
+void TestStableSortWideKeysAndValues() {
+  const std::size_t n = (128 * 1024) / sizeof(fixed_vector<N>) + 3;
+  thrust::host_vector<fixed_vector<N>> hk(n), hv(n);
+  thrust::host_vector<int> r = unittest::random_integers<int>(n);
+  for (std::size_t i = 0; i < n; i++) { hk[i] = fixed_vector<N>((r[i] & 0x7fffffff) % 97); hv[i] = fixed_vector<N>((int)i); }
+  std::vector<std::size_t> idx(n);
+  std::iota(idx.begin(), idx.end(), std::size_t(0));
+  std::stable_sort(idx.begin(), idx.end(), [&](std::size_t a, std::size_t b) { return hk[a] < hk[b]; });
+  thrust::host_vector<fixed_vector<N>> rk(n), rv(n);
+  for (std::size_t i = 0; i < n; i++) { rk[i] = hk[idx[i]]; rv[i] = hv[idx[i]]; }
+  {  // keys only
+    thrust::device_vector<fixed_vector<N>> dk = hk;
+    thrust::stable_sort(dk.begin(), dk.end());
+    ASSERT_EQUAL(dk == rk, true);
+  }
+  {  // wide keys, int values
+    thrust::device_vector<fixed_vector<N>> dk = hk;
+    thrust::device_vector<int> dv(n);
+    thrust::sequence(dv.begin(), dv.end());
+    thrust::stable_sort_by_key(dk.begin(), dk.end(), dv.begin());
+    ASSERT_EQUAL(dk == rk, true);
+    thrust::host_vector<int> ri(n);
+    for (std::size_t i = 0; i < n; i++) ri[i] = (int)idx[i];
+    ASSERT_EQUAL(dv, ri);
+  }
+  {  // wide keys and wide values
+    thrust::device_vector<fixed_vector<N>> dk = hk, dv = hv;
+    thrust::stable_sort_by_key(dk.begin(), dk.end(), dv.begin());
+    ASSERT_EQUAL(dk == rk, true);
+    ASSERT_EQUAL(dv == rv, true);
+  }
+}
+void TestStableSortWide16() { TestStableSortWideKeysAndValues<16>(); }
+void TestStableSortWide33() { TestStableSortWideKeysAndValues<33>(); }
+void TestStableSortWide256() { TestStableSortWideKeysAndValues<256>(); }
+void TestStableSortWide2048() { TestStableSortWideKeysAndValues<2048>(); }
+DECLARE_UNITTEST(TestStableSortWide16);
+DECLARE_UNITTEST(TestStableSortWide33);
+DECLARE_UNITTEST(TestStableSortWide256);
+DECLARE_UNITTEST(TestStableSortWide2048);
+
+// a 4-byte key whose default constructor is written out (LDS arrays cannot hold it): the same path,
+// over the size ladder and under a comparator of the user's
+struct counted_key {
+  int x;
+  __host__ __device__ counted_key() : x(-1) {}
+  __host__ __device__ explicit counted_key(int y) : x(y) {}
+  __host__ __device__ bool operator==(const counted_key& o) const { return x == o.x; }
+};
+inline std::ostream& operator<<(std::ostream& os, const counted_key& k) { return os << k.x; }
+struct counted_key_tens {
+  __host__ __device__ bool operator()(const counted_key& a, const counted_key& b) const { return a.x / 10 < b.x / 10; }
+};
+void TestStableSortKeysWithConstructors() {
+  for (std::size_t n : unittest::sizes()) {
+    if (n > 300000) continue;
+    thrust::host_vector<int> r = unittest::random_integers<int>(n);
+    thrust::host_vector<counted_key> h(n);
+    for (std::size_t i = 0; i < n; i++) h[i] = counted_key((r[i] & 0x7fffffff) % 1000);
+    thrust::device_vector<counted_key> d = h;
+    thrust::stable_sort(d.begin(), d.end(), counted_key_tens());
+    std::vector<counted_key> ref(h.begin(), h.end());
+    std::stable_sort(ref.begin(), ref.end(), counted_key_tens());
+    ASSERT_EQUAL(d == thrust::host_vector<counted_key>(ref.begin(), ref.end()), true);
+  }
+}
+DECLARE_UNITTEST(TestStableSortKeysWithConstructors);
+
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
