@@ -103,6 +103,13 @@ class uniform_real_distribution {
   THRUST_CDNA4_HD result_type(max)() const { return b(); }
   THRUST_CDNA4_HD friend bool operator==(const uniform_real_distribution& l, const uniform_real_distribution& r) { return l.param_ == r.param_; }
   THRUST_CDNA4_HD friend bool operator!=(const uniform_real_distribution& l, const uniform_real_distribution& r) { return !(l == r); }
+  // saved and restored as its two parameters (thrust/random/detail/uniform_real_distribution.inl: stream_out, stream_in)
+  template <class Ch, class Tr> friend std::basic_ostream<Ch, Tr>& operator<<(std::basic_ostream<Ch, Tr>& os, const uniform_real_distribution& d) {
+    return os << d.param_.first << os.widen(' ') << d.param_.second;
+  }
+  template <class Ch, class Tr> friend std::basic_istream<Ch, Tr>& operator>>(std::basic_istream<Ch, Tr>& is, uniform_real_distribution& d) {
+    return is >> d.param_.first >> d.param_.second;
+  }
 
  private:
   param_type param_;
@@ -130,6 +137,13 @@ class uniform_int_distribution {
   THRUST_CDNA4_HD result_type(max)() const { return b(); }
   THRUST_CDNA4_HD friend bool operator==(const uniform_int_distribution& l, const uniform_int_distribution& r) { return l.param_ == r.param_; }
   THRUST_CDNA4_HD friend bool operator!=(const uniform_int_distribution& l, const uniform_int_distribution& r) { return !(l == r); }
+  // saved and restored as its two parameters (thrust/random/detail/uniform_int_distribution.inl: stream_out, stream_in)
+  template <class Ch, class Tr> friend std::basic_ostream<Ch, Tr>& operator<<(std::basic_ostream<Ch, Tr>& os, const uniform_int_distribution& d) {
+    return os << d.param_.first << os.widen(' ') << d.param_.second;
+  }
+  template <class Ch, class Tr> friend std::basic_istream<Ch, Tr>& operator>>(std::basic_istream<Ch, Tr>& is, uniform_int_distribution& d) {
+    return is >> d.param_.first >> d.param_.second;
+  }
 
  private:
   param_type param_;
@@ -167,6 +181,15 @@ class normal_distribution {
   THRUST_CDNA4_HD void param(const param_type& p) { param_ = p; }
   THRUST_CDNA4_HD result_type(min)() const { return -std::numeric_limits<RealType>::max(); }
   THRUST_CDNA4_HD result_type(max)() const { return std::numeric_limits<RealType>::max(); }
+  THRUST_CDNA4_HD friend bool operator==(const normal_distribution& l, const normal_distribution& r) { return l.param_ == r.param_; }
+  THRUST_CDNA4_HD friend bool operator!=(const normal_distribution& l, const normal_distribution& r) { return !(l == r); }
+  // saved and restored as mean and standard deviation (thrust/random/detail/normal_distribution.inl:206-231)
+  template <class Ch, class Tr> friend std::basic_ostream<Ch, Tr>& operator<<(std::basic_ostream<Ch, Tr>& os, const normal_distribution& d) {
+    return os << d.param_.first << os.widen(' ') << d.param_.second;
+  }
+  template <class Ch, class Tr> friend std::basic_istream<Ch, Tr>& operator>>(std::basic_istream<Ch, Tr>& is, normal_distribution& d) {
+    return is >> d.param_.first >> d.param_.second;
+  }
 
  private:
   param_type param_;

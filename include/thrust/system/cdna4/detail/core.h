@@ -139,12 +139,16 @@ struct execute_on_stream : execution_policy<execute_on_stream> {
 // returns after it has completed (thrust/system/cuda/detail/util.h:46-55, :113-140).
 struct execute_after;  // thrust/event.h
 template <class Alloc> struct execute_with_allocator;
+template <class Alloc> struct execute_with_owned_allocator;
 struct par_t : execution_policy<par_t> {
   execute_on_stream on(void* stream) const { return execute_on_stream(stream, true); }
   // thrust::device.after(events...): policy of an asynchronous algorithm that starts after them
   // (defined in thrust/event.h)
   template <class... Events> execute_after after(Events&&... events) const;
   template <class Alloc> execute_with_allocator<Alloc> operator()(Alloc& alloc) const;
+  // an allocator passed as a temporary or a constant is copied into the policy
+  // (thrust/detail/execute_with_allocator.h: the by-value form)
+  template <class Alloc> execute_with_owned_allocator<Alloc> operator()(const Alloc& alloc) const;
 };
 // par_nosync: the call may return before the work has completed, except where a result has
 // to be read back (thrust/system/cuda/detail/par.h:102-107, :181-186).
@@ -162,6 +166,15 @@ struct execute_with_allocator : execution_policy<execute_with_allocator<Alloc>> 
   bool sync_;
   execute_with_allocator(Alloc& a, void* s, bool sync) : alloc_(a), stream_(s), sync_(sync) {}
   execute_with_allocator on(void* stream) const { return execute_with_allocator(alloc_, stream, sync_); }
+};
+template <class Alloc> struct owned_allocator { mutable Alloc owned_; explicit owned_allocator(const Alloc& a) : owned_(a) {} };
+template <class Alloc>
+struct execute_with_owned_allocator : private owned_allocator<Alloc>, execute_with_allocator<Alloc> {
+  execute_with_owned_allocator(const Alloc& a, void* s, bool sync)
+      : owned_allocator<Alloc>(a), execute_with_allocator<Alloc>(this->owned_, s, sync) {}
+  execute_with_owned_allocator(const execute_with_owned_allocator& o)
+      : owned_allocator<Alloc>(o.owned_), execute_with_allocator<Alloc>(this->owned_, o.stream_, o.sync_) {}
+  execute_with_owned_allocator on(void* stream) const { return execute_with_owned_allocator(this->owned_, stream, this->sync_); }
 };
 template <class Alloc> inline void* stream_of(const execute_with_allocator<Alloc>& p) { return p.stream_; }
 template <class Alloc> inline bool must_sync(const execute_with_allocator<Alloc>& p) { return p.sync_; }
@@ -234,6 +247,17 @@ inline void free_bytes(void* p, void* stream) noexcept { (void)thrust_cdna4_free
 
 template <class Alloc>
 execute_with_allocator<Alloc> par_t::operator()(Alloc& alloc) const { return execute_with_allocator<Alloc>(alloc, nullptr, true); }
+template <class Alloc>
+execute_with_owned_allocator<Alloc> par_t::operator()(const Alloc& alloc) const { return execute_with_owned_allocator<Alloc>(alloc, nullptr, true); }
+// an allocator of void hands out bytes through its rebound form
+template <class Alloc, class V = typename Alloc::value_type> struct storage_allocator {
+  typedef Alloc type;
+  static Alloc& get(Alloc& a) { return a; }
+};
+template <class Alloc> struct storage_allocator<Alloc, void> {
+  typedef typename std::allocator_traits<Alloc>::template rebind_alloc<char> type;
+  static type get(Alloc& a) { return type(a); }
+};
 
 // raw address of what an allocator returned (a raw pointer or a pointer-like object with get())
 template <class T> inline void* address_of_allocation(T* p) { return const_cast<typename std::remove_const<T>::type*>(p); }
@@ -251,15 +275,16 @@ class temporary_storage {
   template <class Alloc>
   temporary_storage(std::size_t bytes, const execute_with_allocator<Alloc>& exec)
       : stream_(exec.stream_), bytes_(bytes), ptr_(nullptr), user_(&exec.alloc_), release_(nullptr) {
-    typedef typename Alloc::value_type V;
+    typedef typename storage_allocator<Alloc>::type A;
+    typedef typename A::value_type V;
     if (bytes_) {
       const std::size_t count = (bytes_ + sizeof(V) - 1) / sizeof(V);
-      ptr_ = address_of_allocation(exec.alloc_.allocate(count));
+      ptr_ = address_of_allocation(storage_allocator<Alloc>::get(exec.alloc_).allocate(count));
       release_ = [](void* alloc, void* p, std::size_t n, void* stream) {
         // the allocator may hand the block out again at once: wait for the work that uses it
         (void)thrust_cdna4_stream_synchronize(stream);
-        typedef decltype(std::declval<Alloc&>().allocate(1)) pointer;
-        static_cast<Alloc*>(alloc)->deallocate(pointer(static_cast<V*>(p)), (n + sizeof(V) - 1) / sizeof(V));
+        typedef decltype(std::declval<A&>().allocate(1)) pointer;
+        storage_allocator<Alloc>::get(*static_cast<Alloc*>(alloc)).deallocate(pointer(static_cast<V*>(p)), (n + sizeof(V) - 1) / sizeof(V));
       };
     }
   }

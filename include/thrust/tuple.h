@@ -102,6 +102,17 @@ template <std::size_t I, class T> struct tuple_element<I, const T> { typedef typ
 template <std::size_t I, class T> struct tuple_element<I, volatile T> { typedef typename std::add_volatile<typename tuple_element<I, T>::type>::type type; };
 template <std::size_t I, class T> struct tuple_element<I, const volatile T> { typedef typename std::add_cv<typename tuple_element<I, T>::type>::type type; };
 template <class T> struct tuple_size;
+// how an element of a tuple is handed out (thrust/tuple.h: access_traits, from the boost tuple)
+template <class T> struct access_traits {
+  typedef const T& const_type;
+  typedef T& non_const_type;
+  typedef const typename std::remove_cv<T>::type& parameter_type;
+};
+template <class T> struct access_traits<T&> {
+  typedef T& const_type;
+  typedef T& non_const_type;
+  typedef T& parameter_type;
+};
 template <class... Ts> struct tuple_size<tuple<Ts...>> : std::integral_constant<std::size_t, sizeof...(Ts)> {};
 template <class T> struct tuple_size<const T> : tuple_size<T> {};
 template <class T> struct tuple_size<volatile T> : tuple_size<T> {};
