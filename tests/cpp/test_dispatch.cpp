@@ -6,6 +6,12 @@
 // scan_by_key.exclusive.cu, reduce_by_key.cu and reduce.cu, with my_system / my_tag of
 // testing/unittest/special_types.h:135-170.  Compiled by hipcc (retagged iterators are fancy iterators: kernel templates).
 #include <thrust/adjacent_difference.h>
+#include <thrust/iterator/constant_iterator.h>
+#include <thrust/iterator/counting_iterator.h>
+#include <thrust/equal.h>
+#include <thrust/for_each.h>
+#include <thrust/transform_scan.h>
+#include <thrust/logical.h>
 #include <thrust/extrema.h>
 #include <thrust/find.h>
 #include <thrust/gather.h>
@@ -221,6 +227,121 @@ EXPLICIT(unique, BEGIN_, BEGIN_, E());
 EXPLICIT(unique_copy, BEGIN_, BEGIN_, BEGIN_, E());
 EXPLICIT(unique_by_key, BEGIN_, BEGIN_, BEGIN_, E());
 EXPLICIT(unique_by_key_copy, BEGIN_, BEGIN_, BEGIN_, BEGIN_, BEGIN_, E());
+
+// ---- algorithms composed from others dispatch on the policy's own type too, and every form
+//      without a policy takes the policy of retagged iterators (testing/{partition_point,
+//      is_partitioned,logical,generate,replace,transform,transform_scan,remove,for_each,equal,find}.cu)
+#define V(x) s.validate_dispatch(); return x
+template <class It, class P> It partition_point(my_system& s, It f, It, P) { V(f); }
+template <class It, class P> It partition_point(my_tag, It f, It, P) { *f = 13; return f; }
+template <class It, class P> bool is_partitioned(my_system& s, It, It, P) { V(false); }
+template <class It, class P> bool is_partitioned(my_tag, It f, It, P) { *f = 13; return false; }
+template <class It, class P> bool all_of(my_system& s, It, It, P) { V(false); }
+template <class It, class P> bool all_of(my_tag, It f, It, P) { *f = 13; return false; }
+template <class It, class P> bool any_of(my_system& s, It, It, P) { V(false); }
+template <class It, class P> bool none_of(my_system& s, It, It, P) { V(false); }
+template <class It, class N, class G> It generate_n(my_system& s, It f, N, G) { V(f); }
+template <class It, class N, class G> It generate_n(my_tag, It f, N, G) { *f = 13; return f; }
+template <class It, class G> void generate(my_tag, It f, It, G) { *f = 13; }
+template <class It, class P, class T> void replace_if(my_system& s, It, It, P, const T&) { s.validate_dispatch(); }
+template <class It, class P, class T> void replace_if(my_tag, It f, It, P, const T&) { *f = 13; }
+template <class It, class T> void replace(my_system& s, It, It, const T&, const T&) { s.validate_dispatch(); }
+template <class In, class Out, class F, class P> Out transform_if(my_system& s, In, In, Out r, F, P) { V(r); }
+template <class In, class Out, class F, class P> Out transform_if(my_tag, In, In, Out r, F, P) { *r = 13; return r; }
+template <class In, class St, class Out, class F, class P> Out transform_if(my_system& s, In, In, St, Out r, F, P) { V(r); }
+template <class In, class Out, class F, class Op> Out transform_inclusive_scan(my_system& s, In, In, Out r, F, Op) { V(r); }
+template <class In, class Out, class F, class Op> Out transform_inclusive_scan(my_tag, In, In, Out r, F, Op) { *r = 13; return r; }
+template <class In, class Out, class F, class T, class Op> Out transform_exclusive_scan(my_system& s, In, In, Out r, F, T, Op) { V(r); }
+template <class It, class T> It remove(my_system& s, It f, It, const T&) { V(f); }
+template <class It, class T> It remove(my_tag, It f, It, const T&) { *f = 13; return f; }
+template <class In, class Out, class T> Out remove_copy(my_system& s, In, In, Out r, const T&) { V(r); }
+template <class It, class St, class P> It remove_if(my_system& s, It f, It, St, P) { V(f); }
+template <class It, class F> It for_each(my_system& s, It f, It, F) { V(f); }
+template <class It, class F> It for_each(my_tag, It f, It, F) { *f = 13; return f; }
+template <class It, class N, class F> It for_each_n(my_system& s, It f, N, F) { V(f); }
+template <class A, class Bi> bool equal(my_system& s, A, A, Bi) { V(false); }
+template <class A, class Bi> bool equal(my_tag, A f, A, Bi) { *f = 13; return false; }
+template <class It, class T> It find(my_system& s, It f, It, const T&) { V(f); }
+template <class In, class N, class Out> Out copy_n(my_system& s, In, N, Out r) { V(r); }
+template <class It, class P> It remove_if(my_tag, It f, It, P) { *f = 13; return f; }
+template <class In, class Out, class F> Out transform(my_tag, In, In, Out r, F) { *r = 13; return r; }
+template <class It, class T> void fill(my_tag, It f, It, const T&) { *f = 13; }
+template <class It, class T> void sequence(my_tag, It f, It, T, T) { *f = 13; }
+template <class It, class E_> It unique(my_tag, It f, It, E_) { *f = 13; return f; }
+#undef V
+EXPLICIT(partition_point, BEGIN_, BEGIN_, I());
+IMPLICIT(partition_point, TAGGED_, TAGGED_, I());
+EXPLICIT(is_partitioned, BEGIN_, BEGIN_, I());
+IMPLICIT(is_partitioned, TAGGED_, TAGGED_, I());
+EXPLICIT(all_of, BEGIN_, BEGIN_, I());
+IMPLICIT(all_of, TAGGED_, TAGGED_, I());
+EXPLICIT(any_of, BEGIN_, BEGIN_, I());
+EXPLICIT(none_of, BEGIN_, BEGIN_, I());
+EXPLICIT(generate_n, BEGIN_, 1, thrust::default_random_engine());
+IMPLICIT(generate_n, TAGGED_, 1, thrust::default_random_engine());
+IMPLICIT(generate, TAGGED_, TAGGED_, thrust::default_random_engine());
+EXPLICIT(replace_if, BEGIN_, BEGIN_, I(), 0);
+IMPLICIT(replace_if, TAGGED_, TAGGED_, I(), 0);
+EXPLICIT(replace, BEGIN_, BEGIN_, 0, 1);
+EXPLICIT(transform_if, BEGIN_, BEGIN_, BEGIN_, thrust::negate<int>(), I());
+IMPLICIT(transform_if, TAGGED_, TAGGED_, TAGGED_, thrust::negate<int>(), I());
+void TestTransformIfStencilDispatchExplicit() {
+  thrust::device_vector<int> vec(1);
+  my_system sys(0);
+  thrust::transform_if(sys, BEGIN_, BEGIN_, BEGIN_, BEGIN_, thrust::negate<int>(), I());
+  ASSERT_EQUAL(true, sys.is_valid());
+}
+DECLARE_UNITTEST(TestTransformIfStencilDispatchExplicit);
+EXPLICIT(transform_inclusive_scan, BEGIN_, BEGIN_, BEGIN_, thrust::negate<int>(), thrust::plus<int>());
+IMPLICIT(transform_inclusive_scan, TAGGED_, TAGGED_, TAGGED_, thrust::negate<int>(), thrust::plus<int>());
+EXPLICIT(transform_exclusive_scan, BEGIN_, BEGIN_, BEGIN_, thrust::negate<int>(), 0, thrust::plus<int>());
+EXPLICIT(remove, BEGIN_, BEGIN_, 0);
+IMPLICIT(remove, TAGGED_, TAGGED_, 0);
+EXPLICIT(remove_copy, BEGIN_, BEGIN_, BEGIN_, 0);
+void TestRemoveIfStencilDispatchExplicit() {
+  thrust::device_vector<int> vec(1);
+  my_system sys(0);
+  thrust::remove_if(sys, BEGIN_, BEGIN_, BEGIN_, I());
+  ASSERT_EQUAL(true, sys.is_valid());
+}
+DECLARE_UNITTEST(TestRemoveIfStencilDispatchExplicit);
+EXPLICIT(for_each, BEGIN_, BEGIN_, I());
+IMPLICIT(for_each, TAGGED_, TAGGED_, I());
+EXPLICIT(for_each_n, BEGIN_, 1, I());
+EXPLICIT(equal, BEGIN_, BEGIN_, BEGIN_);
+IMPLICIT(equal, TAGGED_, TAGGED_, TAGGED_);
+EXPLICIT(find, BEGIN_, BEGIN_, 0);
+EXPLICIT(copy_n, BEGIN_, 1, BEGIN_);
+IMPLICIT(remove_if, TAGGED_, TAGGED_, I());
+IMPLICIT(transform, TAGGED_, TAGGED_, TAGGED_, thrust::negate<int>());
+IMPLICIT(fill, TAGGED_, TAGGED_, 0);
+IMPLICIT(sequence, TAGGED_, TAGGED_, 0, 1);
+IMPLICIT(unique, TAGGED_, TAGGED_, E());
+
+// a counting range next to a host range runs on the host (it belongs to any system); next to a
+// device range, and alone, on the device
+struct times_two { __host__ __device__ int operator()(int x) const { return 2 * x; } };
+void TestAnySystemIteratorsFollowTheOtherRange() {
+  thrust::host_vector<int> h(5);
+  thrust::transform(thrust::counting_iterator<int>(0), thrust::counting_iterator<int>(5), h.begin(), times_two());
+  for (int i = 0; i < 5; i++) ASSERT_EQUAL(h[i], 2 * i);
+  thrust::device_vector<int> d(5);
+  thrust::transform(thrust::counting_iterator<int>(0), thrust::counting_iterator<int>(5), d.begin(), times_two());
+  ASSERT_EQUAL(d, h);
+  ASSERT_EQUAL(thrust::reduce(thrust::counting_iterator<int>(0), thrust::counting_iterator<int>(5)), 10);
+  thrust::host_vector<int> c(3);
+  thrust::copy(thrust::constant_iterator<int>(7), thrust::constant_iterator<int>(7) + 3, c.begin());
+  ASSERT_EQUAL(c[2], 7);
+  // sequence computes in the type of init and converts where it stores
+  thrust::device_vector<int> q(4);
+  thrust::sequence(q.begin(), q.end(), 0.5f, 1.5f);
+  thrust::host_vector<int> hq = q;
+  ASSERT_EQUAL(hq[0], 0); ASSERT_EQUAL(hq[1], 2); ASSERT_EQUAL(hq[2], 3); ASSERT_EQUAL(hq[3], 5);
+  thrust::host_vector<int> hs(4);
+  thrust::sequence(hs.begin(), hs.end(), 0.5f, 1.5f);
+  ASSERT_EQUAL(hs, hq);
+}
+DECLARE_UNITTEST(TestAnySystemIteratorsFollowTheOtherRange);
 
 void TestReduceDispatchImplicit() {
   thrust::device_vector<int> vec(1);

@@ -20,7 +20,7 @@ def compile_snippet(tmp_path, body, extra=()):
 def test_cpp_tests_compile():
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    for name in ["test_system_dir", "test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface",
+    for name in ["test_system_dir", "test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_host_vector", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface",
                  "bench_generic", "bench_api", "bench_store_pattern"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
 
@@ -40,8 +40,19 @@ def test_host_compiled_tests_build_under_the_sanitizers():
     # tests/test_cpp_api_gpu.py)
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "san"], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    for name in ["test_sort", "test_scan", "test_by_key", "test_system"]:
+    for name in ["test_sort", "test_scan", "test_by_key", "test_system", "test_host_vector"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", "san", name))
+
+
+def test_host_vector_container_on_the_cpu():
+    # thrust::host_vector is host code only: its tests run here, plain and under the sanitizers
+    for sub in ("", "san"):
+        path = os.path.join(ROOT, "tests", "cpp", "build", sub, "test_host_vector")
+        if not os.path.exists(path):
+            subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp"), os.path.join("build", sub, "test_host_vector")], check=True)
+        r = subprocess.run([path], capture_output=True, text=True, timeout=300,
+                           env=dict(os.environ, ASAN_OPTIONS="detect_leaks=1", UBSAN_OPTIONS="print_stacktrace=1"))
+        assert r.returncode == 0 and "0 failed" in r.stdout, r.stdout[-2000:] + r.stderr[-3000:]
 
 
 def test_existing_thrust_code_compiles_unchanged(tmp_path):
