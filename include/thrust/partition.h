@@ -4,6 +4,7 @@
 // accepts and the ones it rejects, each in input order.  The in-place forms read a temporary
 // copy and collect the rejected elements in a second temporary before appending them.
 #pragma once
+#include <thrust/copy.h>
 #include <algorithm>
 #include <vector>
 #include <thrust/detail/iterator_util.h>

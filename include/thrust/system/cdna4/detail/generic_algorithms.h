@@ -198,6 +198,9 @@ std::int64_t copy_flagged_n(const Policy& exec, In in, S stencil, Out out, std::
 #endif
 }
 // stable two-way split by pred(stencil[i]); returns the number that went to out_true
+// a contiguous input is read through a pointer to const; any other iterator as it is
+template <class T> inline const T* as_input(T* p) { return p; }
+template <class It> inline It as_input(It it) { return it; }
 template <class Policy, class In, class S, class OutT, class OutF, class Pred>
 std::int64_t partition_copy_n(const Policy& exec, In in, S stencil, OutT out_true, OutF out_false, std::int64_t n, Pred pred) {
   THRUST_CDNA4_NEEDS_HIPCC(Pred);

@@ -21,7 +21,34 @@ template <class D, class In, class OutT, class OutF, class Pred, class = typenam
 pair<OutT, OutF> stable_partition_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, OutT out_true, OutF out_false, Pred pred) {
   return stable_partition_copy(exec, first, last, first, out_true, out_false, pred);
 }
-template <class D, class It, class St, class Pred, class = typename std::iterator_traits<St>::iterator_category>
+namespace detail {
+// In place over a range that is no array (a zip of arrays, say): the elements are gathered into a
+// temporary, partitioned from there into the range and a second temporary, and the rejected ones
+// copied behind the accepted.  STENCIL_IS_INPUT: the predicate reads the elements themselves.
+template <bool STENCIL_IS_INPUT, class Policy, class It, class St, class Pred>
+It stable_partition_gathered(const Policy& exec, It first, It last, St stencil, Pred pred) {
+  typedef typename thrust::detail::value_of<It>::type V;
+  const std::int64_t n = (std::int64_t)(last - first);
+  if (n <= 0) return first;
+  temporary_storage gathered((std::size_t)n * sizeof(V), exec), rejected((std::size_t)n * sizeof(V), exec);
+  V* in = static_cast<V*>(gathered.data());
+  V* rej = static_cast<V*>(rejected.data());
+  thrust::copy(exec, first, last, thrust::device_ptr<V>(in));
+  std::int64_t c;
+  if constexpr (STENCIL_IS_INPUT) c = partition_copy_n(exec, (const V*)in, (const V*)in, thrust::detail::unwrap(first), rej, n, pred);
+  else c = partition_copy_n(exec, (const V*)in, as_input(thrust::detail::unwrap(stencil)), thrust::detail::unwrap(first), rej, n, pred);
+  thrust::copy(exec, thrust::device_ptr<V>(rej), thrust::device_ptr<V>(rej + (n - c)), first + c);
+  return first + c;
+}
+template <class It> struct unwraps_to_pointer : std::is_pointer<typename thrust::detail::unwrap_iterator<It>::type> {};
+}  // namespace detail
+template <class D, class It, class St, class Pred, class = typename std::iterator_traits<St>::iterator_category,
+          typename std::enable_if<!(detail::unwraps_to_pointer<It>::value && detail::unwraps_to_pointer<St>::value), int>::type = 0>
+It stable_partition(const system::cdna4::execution_policy<D>& exec, It first, It last, St stencil, Pred pred) {
+  return detail::stable_partition_gathered<false>(exec.derived(), first, last, stencil, pred);
+}
+template <class D, class It, class St, class Pred, class = typename std::iterator_traits<St>::iterator_category,
+          typename std::enable_if<detail::unwraps_to_pointer<It>::value && detail::unwraps_to_pointer<St>::value, int>::type = 0>
 It stable_partition(const system::cdna4::execution_policy<D>& exec, It first, It last, St stencil, Pred pred) {
   namespace sd = system::cdna4::detail;
   typedef typename thrust::detail::value_of<It>::type V;
@@ -40,9 +67,13 @@ It stable_partition(const system::cdna4::execution_policy<D>& exec, It first, It
   }
   return first + c;
 }
-template <class D, class It, class Pred>
+template <class D, class It, class Pred, typename std::enable_if<detail::unwraps_to_pointer<It>::value, int>::type = 0>
 It stable_partition(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) {
   return stable_partition(exec, first, last, first, pred);
+}
+template <class D, class It, class Pred, typename std::enable_if<!detail::unwraps_to_pointer<It>::value, int>::type = 0>
+It stable_partition(const system::cdna4::execution_policy<D>& exec, It first, It last, Pred pred) {
+  return detail::stable_partition_gathered<true>(exec.derived(), first, last, first, pred);
 }
 }}  // namespace system::cdna4
 }  // namespace thrust

@@ -7,9 +7,6 @@ namespace thrust {
 namespace system { namespace cdna4 {
 // the device system's implementations, found through the policy's type
 namespace detail {
-// a contiguous input is read through a pointer to const; any other iterator as it is
-template <class T> inline const T* as_input(T* p) { return p; }
-template <class It> inline It as_input(It it) { return it; }
 template <class Policy, class In, class Pred>
 In remove_if_in_place(const Policy& exec, In first, In last, Pred pred, std::true_type /* contiguous */) {
   typedef typename thrust::detail::value_of<In>::type V;

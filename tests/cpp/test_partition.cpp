@@ -4,7 +4,10 @@
 #include <algorithm>
 
 #include <thrust/functional.h>
+#include <thrust/iterator/zip_iterator.h>
 #include <thrust/partition.h>
+#include <thrust/remove.h>
+#include <thrust/tuple.h>
 #include <thrust/sequence.h>
 
 #include "testing.h"
@@ -155,5 +158,72 @@ void TestStablePartitionLarge() {
   ASSERT_EQUAL(h, d);
 }
 DECLARE_UNITTEST(TestStablePartitionLarge);
+
+// testing/partition.cu:760-860 (TestPartitionZipIterator, TestStablePartitionZipIterator) and
+// testing/remove.cu: in place over a zipped pair of device arrays, with and without a stencil;
+// remove_if / remove_copy_if with a stencil and remove_copy of a value
+struct first_is_even {
+  __host__ __device__ bool operator()(const thrust::tuple<int, int>& t) const { return (thrust::get<0>(t) & 1) == 0; }
+};
+struct is_odd_int { __host__ __device__ bool operator()(int x) const { return (x & 1) != 0; } };
+void TestPartitionAndRemoveOverZippedRanges() {
+  for (std::size_t n : {std::size_t(0), std::size_t(1), std::size_t(5), std::size_t(1000), std::size_t(70001)}) {
+    thrust::host_vector<int> ha(n), hb(n), hs(n);
+    for (std::size_t i = 0; i < n; i++) { ha[i] = (int)((i * 2654435761u) >> 7) % 1000; hb[i] = (int)i; hs[i] = (int)(i % 3); }
+    std::vector<std::pair<int, int>> ref(n);
+    for (std::size_t i = 0; i < n; i++) ref[i] = {ha[i], hb[i]};
+    {  // stable_partition of zip(a, b) by a's parity
+      thrust::device_vector<int> a = ha, b = hb;
+      auto zb = thrust::make_zip_iterator(thrust::make_tuple(a.begin(), b.begin()));
+      auto mid = thrust::stable_partition(zb, zb + n, first_is_even());
+      auto r = ref;
+      auto rm = std::stable_partition(r.begin(), r.end(), [](const std::pair<int, int>& p) { return (p.first & 1) == 0; });
+      ASSERT_EQUAL((std::size_t)(mid - zb), (std::size_t)(rm - r.begin()));
+      thrust::host_vector<int> ra(n), rb(n);
+      for (std::size_t i = 0; i < n; i++) { ra[i] = r[i].first; rb[i] = r[i].second; }
+      ASSERT_EQUAL(a, ra);
+      ASSERT_EQUAL(b, rb);
+    }
+    {  // the same with a stencil: element i is accepted when stencil[i] is odd
+      thrust::device_vector<int> a = ha, b = hb, st = hs;
+      auto zb = thrust::make_zip_iterator(thrust::make_tuple(a.begin(), b.begin()));
+      auto mid = thrust::stable_partition(zb, zb + n, st.begin(), is_odd_int());
+      thrust::host_vector<int> ra, rb;
+      for (std::size_t i = 0; i < n; i++) if (hs[i] & 1) { ra.push_back(ha[i]); rb.push_back(hb[i]); }
+      const std::size_t c = ra.size();
+      for (std::size_t i = 0; i < n; i++) if (!(hs[i] & 1)) { ra.push_back(ha[i]); rb.push_back(hb[i]); }
+      ASSERT_EQUAL((std::size_t)(mid - zb), c);
+      ASSERT_EQUAL(a, ra);
+      ASSERT_EQUAL(b, rb);
+    }
+    {  // remove_if over the zip
+      thrust::device_vector<int> a = ha, b = hb;
+      auto zb = thrust::make_zip_iterator(thrust::make_tuple(a.begin(), b.begin()));
+      auto end = thrust::remove_if(zb, zb + n, first_is_even());
+      thrust::host_vector<int> ra, rb;
+      for (std::size_t i = 0; i < n; i++) if (ha[i] & 1) { ra.push_back(ha[i]); rb.push_back(hb[i]); }
+      ASSERT_EQUAL((std::size_t)(end - zb), ra.size());
+      a.resize(ra.size()); b.resize(rb.size());
+      ASSERT_EQUAL(a, ra);
+      ASSERT_EQUAL(b, rb);
+    }
+    {  // remove_if and remove_copy_if with a stencil, remove_copy of a value
+      thrust::device_vector<int> a = ha, st = hs, out(n), out2(n);
+      auto e1 = thrust::remove_copy_if(a.begin(), a.end(), st.begin(), out.begin(), is_odd_int());
+      auto e2 = thrust::remove_copy(a.begin(), a.end(), out2.begin(), n ? ha[0] : 0);
+      auto e0 = thrust::remove_if(a.begin(), a.end(), st.begin(), is_odd_int());
+      thrust::host_vector<int> r1, r2;
+      for (std::size_t i = 0; i < n; i++) { if (!(hs[i] & 1)) r1.push_back(ha[i]); if (ha[i] != ha[0]) r2.push_back(ha[i]); }
+      ASSERT_EQUAL((std::size_t)(e1 - out.begin()), r1.size());
+      ASSERT_EQUAL((std::size_t)(e0 - a.begin()), r1.size());
+      ASSERT_EQUAL((std::size_t)(e2 - out2.begin()), r2.size());
+      out.resize(r1.size()); a.resize(r1.size()); out2.resize(r2.size());
+      ASSERT_EQUAL(out, r1);
+      ASSERT_EQUAL(a, r1);
+      ASSERT_EQUAL(out2, r2);
+    }
+  }
+}
+DECLARE_UNITTEST(TestPartitionAndRemoveOverZippedRanges);
 
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
