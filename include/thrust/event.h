@@ -119,7 +119,14 @@ class device_event {
   bool valid_stream() const { return bool(signal_); }
   bool ready() const { return valid_stream() && signal_->ready(); }
   void wait() const { state().wait(); }
-  void* stream() const { return state().stream(); }  // the native stream handle
+  // the stream the event's work was queued on: converts to the native handle, which
+  // native_handle() names as the reference's unique_stream does (thrust/system/cuda/detail/future.inl)
+  struct stream_reference {
+    void* handle;
+    void* native_handle() const { return handle; }
+    operator void*() const { return handle; }
+  };
+  stream_reference stream() const { return stream_reference{state().stream()}; }
   const std::shared_ptr<system::cdna4::detail::async_signal>& signal() const { return signal_; }
  protected:
   system::cdna4::detail::async_signal& state() const {
@@ -131,7 +138,7 @@ class device_event {
 
 template <class T>
 class device_future : public device_event {
-  static_assert(std::is_trivially_copyable<T>::value, "device_future: the value type must be trivially copyable");
+  static_assert(detail::is_bytewise_movable<T>::value, "device_future: the value type must be movable as bytes");
  public:
   typedef T value_type;
   device_future() : data_(nullptr), have_(false) {}
@@ -167,10 +174,10 @@ class device_future : public device_event {
 // the reference's names for the same handles (thrust/future.h:70-116): an event or future of a system
 // is that system's unique eager one, and this build has one device system
 template <class System> using unique_eager_event = device_event;
-template <class T, class System> using unique_eager_future = device_future<T>;
+template <class System, class T> using unique_eager_future = device_future<T>;
 // the default event and future of a system (thrust/event.h:21-26, thrust/future.h:150-160)
 template <class System> using event = unique_eager_event<System>;
-template <class T, class System> using future = unique_eager_future<T, System>;
+template <class System, class T> using future = unique_eager_future<System, T>;
 typedef device_event device_unique_eager_event;
 template <class T> using device_unique_eager_future = device_future<T>;
 

@@ -5,6 +5,7 @@
 #include <thrust/device_free.h>
 #include <thrust/device_malloc.h>
 #include <thrust/device_ptr.h>
+#include <thrust/detail/pointer.h>
 #include <cstdlib>
 #include <thrust/pair.h>
 #include <thrust/system/cdna4/detail/malloc_and_free.h>

@@ -173,7 +173,7 @@ void TestAsyncDependencyChain() {
   thrust::device_future<int> empty;
   ASSERT_THROWS(empty.get(), thrust::event_error);
   static_assert(std::is_same<thrust::device_unique_eager_event, thrust::device_event>::value, "");
-  static_assert(std::is_same<thrust::unique_eager_future<int, thrust::device_system_tag>, thrust::device_future<int>>::value, "");
+  static_assert(std::is_same<thrust::unique_eager_future<thrust::device_system_tag, int>, thrust::device_future<int>>::value, "");
 }
 DECLARE_UNITTEST(TestAsyncDependencyChain);
 
