@@ -2,7 +2,17 @@
 // without a policy on device and host ranges.  Mostly a compile check of the overload sets
 // (templates that no other test instantiates); each call's result is also compared between the
 // host and the device range.  Compiled by hipcc.
+#include <list>
+#include <numeric>
+#include <sstream>
 #include <thrust/adjacent_difference.h>
+#include <thrust/iterator/counting_iterator.h>
+#include <thrust/iterator/discard_iterator.h>
+#include <thrust/iterator/transform_iterator.h>
+#include <thrust/iterator/zip_iterator.h>
+#include <thrust/memory.h>
+#include <thrust/swap.h>
+#include <thrust/universal_vector.h>
 #include <thrust/binary_search.h>
 #include <thrust/copy.h>
 #include <thrust/count.h>
@@ -200,5 +210,168 @@ void TestDeviceVectorReverseIterationAndCheckedAccess() {
   static_assert(std::is_same<thrust::device_vector<int>::difference_type, std::ptrdiff_t>::value, "");
 }
 DECLARE_UNITTEST(TestDeviceVectorReverseIterationAndCheckedAccess);
+
+// ---- vectors convert between systems, element types and allocators (thrust/detail/vector_base.h:153-185)
+void TestVectorConversions() {
+  thrust::host_vector<int> hi(100);
+  for (int i = 0; i < 100; i++) hi[i] = i - 50;
+  thrust::device_vector<float> df(hi);            // host int -> device float
+  thrust::device_vector<double> dd(df);           // device float -> device double
+  thrust::host_vector<long> hl(dd);               // device double -> host long
+  for (int i = 0; i < 100; i++) ASSERT_EQUAL(hl[i], (long)(i - 50));
+  std::vector<short> sv{1, 2, 3};
+  thrust::device_vector<int> ds(sv);
+  ASSERT_EQUAL(ds == (thrust::host_vector<int>{1, 2, 3}), true);
+  ASSERT_EQUAL(ds == (std::vector<long>{1, 2, 3}), true);
+  ASSERT_EQUAL((thrust::host_vector<int>{1, 2, 4}) != ds, true);
+  ds = hi;                                        // assignment across systems
+  ASSERT_EQUAL(ds.size(), std::size_t(100));
+  ASSERT_EQUAL((int)ds[99], 49);
+  df = ds;                                        // and across element types
+  ASSERT_EQUAL((float)df[0], -50.0f);
+  thrust::host_vector<bool> hb(9, false);
+  hb[4] = true;
+  thrust::device_vector<bool> db = hb;            // bool elements are bytes on both sides
+  thrust::host_vector<bool> back = db;
+  ASSERT_EQUAL(back == hb, true);
+  ASSERT_EQUAL((bool)db[4], true);
+  thrust::host_vector<int> from_fancy(thrust::make_transform_iterator(ds.begin(), thrust::negate<int>()),
+                                      thrust::make_transform_iterator(ds.end(), thrust::negate<int>()));
+  ASSERT_EQUAL(from_fancy[0], 50);
+  thrust::host_vector<int> from_counting(thrust::counting_iterator<int>(3), thrust::counting_iterator<int>(6));
+  ASSERT_EQUAL(from_counting == (std::vector<int>{3, 4, 5}), true);
+  ds.insert(ds.begin() + 1, 3, 7);
+  ASSERT_EQUAL((int)ds[1], 7); ASSERT_EQUAL((int)ds[3], 7); ASSERT_EQUAL((int)ds[4], -49);
+  ASSERT_EQUAL(ds.size(), std::size_t(103));
+}
+DECLARE_UNITTEST(TestVectorConversions);
+
+// ---- thrust::copy between every pair of systems and iterator kinds, without a policy
+void TestCopyBetweenEveryPairOfSystems() {
+  const int n = 1000;
+  thrust::host_vector<int> h(n);
+  for (int i = 0; i < n; i++) h[i] = 3 * i;
+  thrust::device_vector<int> d(n), d2(n);
+  thrust::copy(h.begin(), h.end(), d.begin());                          // host -> device
+  thrust::copy(d.begin(), d.end(), d2.begin());                         // device -> device
+  thrust::device_vector<float> df(n);
+  thrust::copy(d.begin(), d.end(), df.begin());                         // device -> device, converting
+  ASSERT_EQUAL((float)df[n - 1], 3.0f * (n - 1));
+  thrust::host_vector<int> back(n);
+  thrust::copy(d2.begin(), d2.end(), back.begin());                     // device -> host
+  ASSERT_EQUAL(back, h);
+  thrust::device_vector<int> da(n), db(n);
+  thrust::host_vector<thrust::tuple<int, int>> aos(n);
+  for (int i = 0; i < n; i++) aos[i] = thrust::make_tuple(i, -i);
+  thrust::copy(aos.begin(), aos.end(), thrust::make_zip_iterator(thrust::make_tuple(da.begin(), db.begin())));  // host -> zipped device
+  ASSERT_EQUAL((int)da[7], 7); ASSERT_EQUAL((int)db[7], -7);
+  thrust::device_vector<int> dc(n), dd(n);
+  thrust::copy(thrust::make_zip_iterator(thrust::make_tuple(da.begin(), db.begin())),
+               thrust::make_zip_iterator(thrust::make_tuple(da.end(), db.end())),
+               thrust::make_zip_iterator(thrust::make_tuple(dc.begin(), dd.begin())));                          // zipped device -> zipped device
+  ASSERT_EQUAL(dc, da); ASSERT_EQUAL(dd, db);
+  auto e1 = thrust::copy(h.begin(), h.end(), thrust::make_discard_iterator());                                  // host -> nowhere
+  auto e2 = thrust::copy(d.begin(), d.end(), thrust::make_discard_iterator());                                  // device -> nowhere
+  ASSERT_EQUAL((int)(e1 - thrust::make_discard_iterator()), n);
+  ASSERT_EQUAL((int)(e2 - thrust::make_discard_iterator()), n);
+  thrust::host_vector<int> hc(5);
+  thrust::copy(thrust::counting_iterator<int>(10), thrust::counting_iterator<int>(15), hc.begin());             // counting -> host, on the host
+  ASSERT_EQUAL(hc[4], 14);
+  thrust::copy_n(thrust::counting_iterator<int>(10), 5, d.begin());                                             // counting -> device
+  ASSERT_EQUAL((int)d[4], 14);
+  std::list<int> l{5, 6, 7};
+  thrust::copy_n(l.begin(), 3, d.begin());                                                                      // a stepping host iterator
+  ASSERT_EQUAL((int)d[2], 7);
+}
+DECLARE_UNITTEST(TestCopyBetweenEveryPairOfSystems);
+
+// ---- device_reference behaves like the element (thrust/device_reference.h:224-970)
+void TestDeviceReferenceArithmetic() {
+  thrust::device_vector<int> v(2, 10);
+  thrust::device_reference<int> r = v[0];
+  r += 5; ASSERT_EQUAL((int)v[0], 15);
+  r -= 1; r *= 2; ASSERT_EQUAL((int)v[0], 28);
+  r /= 7; r %= 3; ASSERT_EQUAL((int)v[0], 1);
+  r <<= 4; r |= 1; r ^= 3; r &= 0xfe; r >>= 1; ASSERT_EQUAL((int)v[0], 9);
+  ++r; ASSERT_EQUAL((int)r, 10);
+  ASSERT_EQUAL(r++, 10); ASSERT_EQUAL((int)r, 11);
+  --r; r--; ASSERT_EQUAL((int)v[0], 9);
+  thrust::device_reference<int> q(v.data() + 1);
+  q = r;
+  ASSERT_EQUAL((int)v[1], 9);
+  v[1] = 4;
+  thrust::swap(r, q);
+  ASSERT_EQUAL((int)v[0], 4); ASSERT_EQUAL((int)v[1], 9);
+  thrust::device_reference<const int> c = v[1];
+  ASSERT_EQUAL((int)c, 9);
+  std::ostringstream os;
+  os << r << ' ' << (v.data() != thrust::device_ptr<int>());
+  ASSERT_EQUAL(os.str() == std::string("4 1"), true);
+}
+DECLARE_UNITTEST(TestDeviceReferenceArithmetic);
+
+// ---- thrust::pointer carries its system; universal_vector is a class of its own
+struct tagged_policy : thrust::device_execution_policy<tagged_policy> {};
+template <class T> int which_vector(const thrust::device_vector<T>&) { return 1; }
+template <class T> int which_vector(const thrust::universal_vector<T>&) { return 2; }
+void TestTaggedPointerAndUniversalVector() {
+  thrust::device_vector<int> v(100);
+  thrust::pointer<int, thrust::device_system_tag> p(thrust::raw_pointer_cast(v.data()));
+  thrust::sequence(p, p + 100);
+  ASSERT_EQUAL(thrust::reduce(p, p + 100), 4950);
+  ASSERT_EQUAL((int)p[7], 7);
+  *p = 3;
+  ASSERT_EQUAL((int)v[0], 3);
+  thrust::pointer<int, tagged_policy> t(thrust::raw_pointer_cast(v.data()));
+  thrust::fill(t, t + 100, 2);  // runs on the device under the user's (overload-free) policy type
+  ASSERT_EQUAL(thrust::reduce(v.begin(), v.end()), 200);
+  int host_array[4] = {4, 3, 2, 1};
+  thrust::pointer<int, thrust::host_system_tag> hp(host_array);
+  thrust::sort(hp, hp + 4);
+  ASSERT_EQUAL(host_array[0], 1); ASSERT_EQUAL(*hp, 1);
+  thrust::universal_vector<int> u(10, 1);
+  thrust::device_vector<int> d(10, 1);
+  ASSERT_EQUAL(which_vector(u), 2);
+  ASSERT_EQUAL(which_vector(d), 1);
+  ASSERT_EQUAL(thrust::reduce(u.begin(), u.end()), 10);
+  u = d;
+  thrust::universal_vector<int> u2 = u;
+  ASSERT_EQUAL(u2.size(), std::size_t(10));
+}
+DECLARE_UNITTEST(TestTaggedPointerAndUniversalVector);
+
+// ---- a number-like struct with written-out copy operations as an element
+// (custom_numeric of testing/unittest/testframework.h:128-232)
+struct numberlike {
+  int v[2];
+  __host__ __device__ numberlike() { v[0] = v[1] = 0; }
+  __host__ __device__ numberlike(int x) { v[0] = v[1] = x; }
+  __host__ __device__ numberlike(const numberlike& o) { v[0] = o.v[0]; v[1] = o.v[1]; }
+  __host__ __device__ numberlike& operator=(const numberlike& o) { v[0] = o.v[0]; v[1] = o.v[1]; return *this; }
+  __host__ __device__ numberlike operator+(const numberlike& o) const { return numberlike(v[0] + o.v[0]); }
+  __host__ __device__ numberlike operator*(const numberlike& o) const { return numberlike(v[0] * o.v[0]); }
+  __host__ __device__ bool operator<(const numberlike& o) const { return v[0] < o.v[0]; }
+  __host__ __device__ bool operator==(const numberlike& o) const { return v[0] == o.v[0] && v[1] == o.v[1]; }
+};
+inline std::ostream& operator<<(std::ostream& os, const numberlike& x) { return os << x.v[0]; }
+void TestNumberLikeStructElements() {
+  const int n = 5000;
+  thrust::host_vector<numberlike> h(n);
+  for (int i = 0; i < n; i++) h[i] = numberlike((i * 7919) % 1000);
+  thrust::device_vector<numberlike> d = h, out(n);
+  ASSERT_EQUAL(thrust::reduce(d.begin(), d.end(), numberlike(0), thrust::plus<numberlike>()) ==
+                   std::accumulate(h.begin(), h.end(), numberlike(0), thrust::plus<numberlike>()), true);
+  thrust::inclusive_scan(d.begin(), d.end(), out.begin(), thrust::plus<numberlike>());
+  thrust::host_vector<numberlike> hs(n);
+  std::partial_sum(h.begin(), h.end(), hs.begin(), thrust::plus<numberlike>());
+  ASSERT_EQUAL(out == hs, true);
+  thrust::sort(d.begin(), d.end());
+  std::stable_sort(h.begin(), h.end());
+  ASSERT_EQUAL(d == h, true);
+  thrust::device_vector<numberlike> seq(8);
+  thrust::sequence(seq.begin(), seq.end(), numberlike(1), numberlike(2));
+  ASSERT_EQUAL(((numberlike)seq[3]).v[0], 7);
+}
+DECLARE_UNITTEST(TestNumberLikeStructElements);
 
 int main(int argc, char** argv) { return unittest::run_all(argc, argv); }
