@@ -63,7 +63,15 @@ class device_vector {
   ~device_vector() { release(); }
 
   device_vector& operator=(const device_vector& o) { if (this != &o) assign_device(o.p_, o.n_); return *this; }
-  device_vector& operator=(device_vector&& o) noexcept { swap(o); return *this; }
+  // the source is left empty (testing/vector.cu:814-826)
+  device_vector& operator=(device_vector&& o) noexcept {
+    if (this != &o) {
+      release();
+      p_ = o.p_; n_ = o.n_; cap_ = o.cap_; alloc_ = o.alloc_;
+      o.p_ = nullptr; o.n_ = o.cap_ = 0;
+    }
+    return *this;
+  }
   template <class U, class A> device_vector& operator=(const std::vector<U, A>& h) { assign(h.begin(), h.end()); return *this; }
   template <class U, class A> device_vector& operator=(const host_vector<U, A>& h) { assign(h.begin(), h.end()); return *this; }
   template <class U, class A> device_vector& operator=(const device_vector<U, A>& d) { assign(d.begin(), d.end()); return *this; }

@@ -62,7 +62,15 @@ class host_vector {
   ~host_vector() { release(); }
 
   host_vector& operator=(const host_vector& o) { if (this != &o) assign_range(o.p_, o.p_ + o.n_); return *this; }
-  host_vector& operator=(host_vector&& o) noexcept { swap(o); return *this; }
+  // the source is left empty (thrust/detail/vector_base.inl: move assignment; testing/vector.cu:814-826)
+  host_vector& operator=(host_vector&& o) noexcept {
+    if (this != &o) {
+      release();
+      p_ = o.p_; n_ = o.n_; cap_ = o.cap_; alloc_ = std::move(o.alloc_);
+      o.p_ = nullptr; o.n_ = o.cap_ = 0;
+    }
+    return *this;
+  }
   host_vector& operator=(std::initializer_list<T> il) { assign_range(il.begin(), il.end()); return *this; }
   template <class U, class A2> host_vector& operator=(const host_vector<U, A2>& o) { assign_range(o.begin(), o.end()); return *this; }
   template <class U, class A2> host_vector& operator=(const std::vector<U, A2>& o) { assign_range(o.begin(), o.end()); return *this; }

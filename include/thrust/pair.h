@@ -15,7 +15,8 @@ struct pair {
   T1 first;
   T2 second;
 
-  pair() = default;
+  // the members are value-initialised (thrust/pair.h:82-85; testing/pair.cu:13-16)
+  THRUST_CDNA4_HD constexpr pair() : first(), second() {}
   THRUST_CDNA4_HD constexpr pair(const T1& x, const T2& y) : first(x), second(y) {}
   template <class U1, class U2, class = typename std::enable_if<std::is_convertible<const U1&, T1>::value && std::is_convertible<const U2&, T2>::value>::type>
   THRUST_CDNA4_HD constexpr pair(const pair<U1, U2>& p) : first(p.first), second(p.second) {}

@@ -243,6 +243,14 @@ void TestVectorConversions() {
   ds.insert(ds.begin() + 1, 3, 7);
   ASSERT_EQUAL((int)ds[1], 7); ASSERT_EQUAL((int)ds[3], 7); ASSERT_EQUAL((int)ds[4], -49);
   ASSERT_EQUAL(ds.size(), std::size_t(103));
+  // move assignment hands the storage over and leaves the source empty (testing/vector.cu:814-826)
+  thrust::device_vector<int> m1(3, 1), m2(2, 2);
+  const int* held = thrust::raw_pointer_cast(m1.data());
+  m2 = std::move(m1);
+  ASSERT_EQUAL(m1.empty(), true);
+  ASSERT_EQUAL(m2.size(), std::size_t(3));
+  ASSERT_EQUAL(thrust::raw_pointer_cast(m2.data()) == held, true);
+  ASSERT_EQUAL((int)m2[2], 1);
 }
 DECLARE_UNITTEST(TestVectorConversions);
 

@@ -87,6 +87,25 @@ void TestHostVectorAssignment() {
 }
 DECLARE_UNITTEST(TestHostVectorAssignment);
 
+// testing/vector.cu:780-840: a moved-from vector is empty and the target has its storage
+void TestHostVectorMove() {
+  thrust::host_vector<int> v1{0, 1, 2};
+  const int* p1 = v1.data();
+  thrust::host_vector<int> v2(std::move(v1));
+  ASSERT_EQUAL(v1.empty(), true);
+  ASSERT_EQUAL(v2.data() == p1, true);
+  thrust::host_vector<int> v3{3, 4, 5};
+  const int* p3 = v3.data();
+  v2 = std::move(v3);
+  ASSERT_EQUAL(v3.empty(), true);
+  ASSERT_EQUAL(v2.data() == p3, true);
+  ASSERT_EQUAL(v2[2], 5);
+  thrust::pair<int, float> z;
+  ASSERT_EQUAL(z.first, 0);
+  ASSERT_EQUAL(z.second, 0.0f);
+}
+DECLARE_UNITTEST(TestHostVectorMove);
+
 void TestHostVectorGrowthAndShrinking() {
   thrust::host_vector<int> h;
   std::vector<int> v;

@@ -39,3 +39,34 @@ def test_reference_unit_tests_compile_unchanged():
     assert not broken, broken
     leaked = {name: foreign for name, _, _, foreign in results if foreign}
     assert not leaked, leaked
+
+
+# Reference test files whose host-vector variants (test names ending in "Host") run here on the
+# CPU; the few of those that move data to or from a device vector need a device and are left out.
+CORE = ["sort", "stable_sort", "sort_by_key", "stable_sort_by_key", "scan_by_key.inclusive", "scan_by_key.exclusive",
+        "reduce_by_key", "reduce", "vector", "vector_insert", "vector_manipulation", "unique", "unique_by_key", "merge",
+        "set_union", "partition_point", "remove", "replace", "transform", "gather", "scatter", "tuple", "pair"]
+NEEDS_A_DEVICE = {"TestVectorAssignFromDeviceVectorHost", "TestVectorToAndFromDeviceVectorHost", "TestTupleSwap", "TestTupleTie",
+                  "TestPairSwap"}
+DEVICE_FREE_FILES = {"tuple", "pair"}  # every other test of these files runs on the CPU
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_TESTING) or not os.path.exists(HIPCC), reason="needs the reference tree and hipcc")
+def test_reference_host_vector_tests_pass_on_the_cpu():
+    """The reference's unit tests, built unchanged by `make -C oracle ref_tests`, run their
+    host-vector variants: the host system of this header layer (thrust::host_vector, the sequential
+    algorithm forms, tuple, pair, dispatch on host iterators) against the reference's own checks."""
+    r = subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "ref_tests", "-j8"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    ran = 0
+    for name in CORE:
+        exe = os.path.join(ROOT, "oracle", "_ref", "testing", name)
+        listed = subprocess.run([exe, "--list"], stdout=subprocess.PIPE, text=True).stdout.split()
+        names = [t for t in listed if t not in NEEDS_A_DEVICE] if name in DEVICE_FREE_FILES else [
+            t for t in listed if (t.endswith("Host") or t.endswith("<thrust::host_vector>")) and t not in NEEDS_A_DEVICE]
+        if not names:  # a file whose tests all use the device
+            continue
+        p = subprocess.run([exe] + names, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+        assert p.returncode == 0 and "0 failures, 0 known failures, 0 errors" in p.stdout, name + "\n" + p.stdout[-3000:]
+        ran += len(names)
+    assert ran >= 80, ran
