@@ -17,10 +17,10 @@ struct allocator_traits : std::allocator_traits<Alloc> {
   typedef typename base::value_type& reference;
   typedef const typename base::value_type& const_reference;
   template <class U> using rebind_alloc = typename base::template rebind_alloc<U>;
-  // (the traits of the rebound allocator, also under the reference's nested name `other`)
-  template <class U> struct rebind_traits : allocator_traits<typename base::template rebind_alloc<U>> {
-    typedef allocator_traits<typename base::template rebind_alloc<U>> other;
-  };
+  // the traits of the rebound allocator; `other` names a traits class itself, so that both
+  // rebind_traits<U> and the older spelling rebind_traits<U>::other give it
+  template <class U> using rebind_traits = allocator_traits<typename base::template rebind_alloc<U>>;
+  typedef allocator_traits other;
   // the allocator as it should be passed on: a reference when it has state, else a fresh object
   typedef typename std::conditional<std::is_empty<Alloc>::value, Alloc, Alloc&>::type get_result_type;
   static get_result_type get(Alloc& a) { return a; }

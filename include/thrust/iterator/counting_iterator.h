@@ -18,7 +18,11 @@ class counting_iterator : public detail::fancy_base<counting_iterator<T, System,
   THRUST_CDNA4_HD counting_iterator(const counting_iterator<T, S2, Tr2, D2>& o) : v_(o.base()) {}
   THRUST_CDNA4_HD T at(std::ptrdiff_t n) const { return (T)(v_ + (T)n); }
   THRUST_CDNA4_HD void advance(std::ptrdiff_t n) { v_ = (T)(v_ + (T)n); }
-  THRUST_CDNA4_HD std::ptrdiff_t distance_to(const counting_iterator& o) const { return (std::ptrdiff_t)(o.v_ - v_); }
+  // signed also for an unsigned counter (thrust/iterator/counting_iterator.h: the difference type of an
+  // unsigned counter is a wider signed integer)
+  THRUST_CDNA4_HD std::ptrdiff_t distance_to(const counting_iterator& o) const { return distance(o.v_, v_, std::is_integral<T>()); }
+  THRUST_CDNA4_HD static std::ptrdiff_t distance(const T& to, const T& from, std::true_type) { return (std::ptrdiff_t)to - (std::ptrdiff_t)from; }
+  THRUST_CDNA4_HD static std::ptrdiff_t distance(const T& to, const T& from, std::false_type) { return (std::ptrdiff_t)(to - from); }
   THRUST_CDNA4_HD const T& base() const { return v_; }  // the counter (thrust/iterator/iterator_adaptor.h:178)
  private:
   T v_;

@@ -17,7 +17,7 @@ template <class Upstream, class Bookkeeper>
 class disjoint_unsynchronized_pool_resource final : public detail::pool_core<Upstream, detail::resource_bookkeeping<Bookkeeper>> {
   typedef detail::pool_core<Upstream, detail::resource_bookkeeping<Bookkeeper>> core;
  public:
-  static pool_options get_default_options() { return pool_options(); }
+  static pool_options get_default_options() { return detail::default_pool_options(); }
   disjoint_unsynchronized_pool_resource(Upstream* upstream, Bookkeeper* bookkeeper, pool_options options = get_default_options())
       : core(upstream, detail::resource_bookkeeping<Bookkeeper>{bookkeeper}, options) {}
   explicit disjoint_unsynchronized_pool_resource(pool_options options = get_default_options())

@@ -39,12 +39,13 @@ template <class Upstream, class Book>
 class pool_core : public memory_resource<typename Upstream::pointer> {
  public:
   typedef typename Upstream::pointer pointer;
-  static pool_options get_default_options() { return pool_options(); }
+  static pool_options get_default_options() { return detail::default_pool_options(); }
 
   pool_core(Upstream* upstream, Book book, pool_options options)
       : upstream_(upstream), opt_(options), book_(book), free_(book.template get<free_list>()), chunks_(book.template get<chunk>()),
         oversized_(book.template get<big>()) {
     if (!opt_.validate()) throw std::invalid_argument("thrust::mr::pool_options: inconsistent");
+    if (opt_.alignment == 0) opt_.alignment = alignof(std::max_align_t);  // left unset by the caller
     std::size_t classes = 1;
     for (std::size_t s = opt_.smallest_block_size; s < opt_.largest_block_size; s <<= 1) ++classes;
     free_.assign(classes, free_list(book.template get<pointer>()));
@@ -114,7 +115,7 @@ class pool_core : public memory_resource<typename Upstream::pointer> {
     if (opt_.cache_oversized) {
       big* best = nullptr;
       for (auto& o : oversized_)
-        if (!o.in_use && o.bytes >= bytes && o.bytes / opt_.cached_size_cutoff_factor <= bytes && (!best || o.bytes < best->bytes)) best = &o;
+        if (!o.in_use && o.bytes >= bytes && (opt_.cached_size_cutoff_factor == 0 || o.bytes / opt_.cached_size_cutoff_factor <= bytes) && (!best || o.bytes < best->bytes)) best = &o;
       if (best) { best->in_use = true; return best->p; }
     }
     pointer p = upstream_->allocate(bytes, opt_.alignment);
@@ -137,7 +138,7 @@ template <class Upstream>
 class unsynchronized_pool_resource final : public detail::pool_core<Upstream, detail::heap_bookkeeping> {
   typedef detail::pool_core<Upstream, detail::heap_bookkeeping> core;
  public:
-  static pool_options get_default_options() { return pool_options(); }
+  static pool_options get_default_options() { return detail::default_pool_options(); }
   explicit unsynchronized_pool_resource(Upstream* upstream, pool_options options = get_default_options())
       : core(upstream, detail::heap_bookkeeping(), options) {}
   explicit unsynchronized_pool_resource(pool_options options = get_default_options())

@@ -66,7 +66,7 @@ template <class Upstream>
 void pool_behaviour(Upstream* upstream) {
   tracking_resource<Upstream> tracker(upstream);
   {
-    thrust::mr::pool_options opt;
+    thrust::mr::pool_options opt = thrust::mr::unsynchronized_pool_resource<thrust::mr::new_delete_resource>::get_default_options();
     opt.smallest_block_size = 256;
     opt.largest_block_size = 1 << 16;
     opt.min_blocks_per_chunk = 4;
@@ -223,7 +223,7 @@ void TestDisjointPool() {
     tracking_resource<thrust::device_memory_resource> up(&dev);
     typedef thrust::mr::disjoint_unsynchronized_pool_resource<tracking_resource<thrust::device_memory_resource>,
                                                                tracking_resource<thrust::mr::new_delete_resource>> Pool;
-    thrust::mr::pool_options opt;
+    thrust::mr::pool_options opt = thrust::mr::unsynchronized_pool_resource<thrust::mr::new_delete_resource>::get_default_options();
     opt.smallest_block_size = 256;
     opt.largest_block_size = 1 << 16;
     Pool pool(&up, &book, opt);
