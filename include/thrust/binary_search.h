@@ -44,6 +44,8 @@ std::ptrdiff_t scalar_search(const system::cpp::detail::par_t&, Hay first, Hay l
 }
 }  // namespace detail
 
+// Without a comparator the elements and the values are compared as they are, by the transparent
+// less (thrust/system/detail/generic/binary_search.inl: `_1 < _2`), not converted to one type first.
 #define THRUST_CDNA4_SEARCH(NAME, MODE)                                                                                  \
   template <class Policy, class Hay, class Needles, class Out, class Comp, detail::enable_if_policy<Policy> = 0>         \
   Out NAME(const Policy& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out, Comp comp) {                 \
@@ -51,7 +53,7 @@ std::ptrdiff_t scalar_search(const system::cpp::detail::par_t&, Hay first, Hay l
   }                                                                                                                      \
   template <class Policy, class Hay, class Needles, class Out, detail::enable_if_policy<Policy> = 0>                     \
   Out NAME(const Policy& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out) {                            \
-    return detail::vector_search<MODE>(exec, first, last, vfirst, vlast, out, less<typename detail::value_of<Hay>::type>()); \
+    return detail::vector_search<MODE>(exec, first, last, vfirst, vlast, out, less<>()); \
   }                                                                                                                      \
   template <class Hay, class Needles, class Out, detail::enable_if_device<Hay, Needles, Out> = 0,                                      \
             class = typename std::iterator_traits<Out>::iterator_category>                                               \
@@ -78,10 +80,16 @@ THRUST_CDNA4_SEARCH(binary_search, 2)
   }                                                                                                                      \
   template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>                                      \
   Hay NAME(const Policy& exec, Hay first, Hay last, const T& value) {                                                    \
-    return first + detail::scalar_search<MODE>(exec, first, last, value, less<T>());                                     \
+    return first + detail::scalar_search<MODE>(exec, first, last, value, less<>());                                     \
   }                                                                                                                      \
   template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(typename detail::implicit_policy<Hay, T>::type(), f, l, v); } \
-  template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(host, f, l, v); }
+  template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(host, f, l, v); } \
+  template <class Hay, class T, class Comp, detail::enable_if_device<Hay, T> = 0,                                        \
+            typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>                                     \
+  Hay NAME(Hay f, Hay l, const T& v, Comp c) { return NAME(typename detail::implicit_policy<Hay, T>::type(), f, l, v, c); } \
+  template <class Hay, class T, class Comp, detail::enable_if_host<Hay, T> = 0,                                          \
+            typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>                                     \
+  Hay NAME(Hay f, Hay l, const T& v, Comp c) { return NAME(host, f, l, v, c); }
 THRUST_CDNA4_SCALAR_BOUND(lower_bound, 0)
 THRUST_CDNA4_SCALAR_BOUND(upper_bound, 1)
 #undef THRUST_CDNA4_SCALAR_BOUND
@@ -91,10 +99,14 @@ bool binary_search(const Policy& exec, Hay first, Hay last, const T& value, Comp
 }
 template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>
 bool binary_search(const Policy& exec, Hay first, Hay last, const T& value) {
-  return detail::scalar_search<2>(exec, first, last, value, less<T>()) != 0;
+  return detail::scalar_search<2>(exec, first, last, value, less<>()) != 0;
 }
 template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(typename detail::implicit_policy<Hay, T>::type(), f, l, v); }
 template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(host, f, l, v); }
+template <class Hay, class T, class Comp, detail::enable_if_device<Hay, T> = 0, typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>
+bool binary_search(Hay f, Hay l, const T& v, Comp c) { return binary_search(typename detail::implicit_policy<Hay, T>::type(), f, l, v, c); }
+template <class Hay, class T, class Comp, detail::enable_if_host<Hay, T> = 0, typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>
+bool binary_search(Hay f, Hay l, const T& v, Comp c) { return binary_search(host, f, l, v, c); }
 
 // ---- equal_range (thrust/binary_search.h:727-1017): the pair (lower_bound, upper_bound) of one value
 template <class Policy, class Hay, class T, class Comp, detail::enable_if_policy<Policy> = 0>
@@ -104,7 +116,7 @@ pair<Hay, Hay> equal_range(const Policy& exec, Hay first, Hay last, const T& val
 }
 template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>
 pair<Hay, Hay> equal_range(const Policy& exec, Hay first, Hay last, const T& value) {
-  return equal_range(exec, first, last, value, less<T>());
+  return equal_range(exec, first, last, value, less<>());
 }
 template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(typename detail::implicit_policy<Hay, T>::type(), f, l, v); }
 template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(host, f, l, v); }
