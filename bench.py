@@ -356,14 +356,6 @@ def main():
         else:
             extras["api_error"] = r.stderr[-300:]
 
-    def extra_store_probe():
-        # what bounds a radix pass of this shape (tests/cpp/bench_store_pattern.cpp): a copy with the
-        # pass's store pattern and tile assignments; only on request (--only store_probe)
-        import subprocess
-        exe = os.path.join(ROOT, "tests", "cpp", "build", "bench_store_pattern")
-        r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
-        extras["store_pattern_probe"] = r.stdout.strip().splitlines() if r.returncode == 0 else r.stderr[-300:]
-
     all_extras = {
         "api": extra_api,
         "generic": extra_generic,
@@ -382,8 +374,6 @@ def main():
         "copy": extra_copy_ceiling,
     }
     if not args.no_extras:
-        if args.only == "store_probe":
-            extra_store_probe()
         for name, f in all_extras.items():
             if args.only and name != args.only:
                 continue

@@ -107,10 +107,12 @@ int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int op, int exc
  * thrust_cdna4_scan for callers that cannot allocate: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference, whose scan
  * always takes caller-provided temporary storage (thrust/system/cuda/detail/scan.h:80-117).  Same
- * arguments, results and kernels as thrust_cdna4_scan without `temp` / `temp_bytes`: the tile
- * descriptors live in a fixed 256 KiB array inside the library's device image (one copy per GPU,
- * held until the process ends), whose device address is looked up on the first call on each
- * device; no call allocates or frees memory.  Limit: at most 16384 tiles of 128 KiB, i.e. 2 GiB
+ * arguments, results and kernels as thrust_cdna4_scan without `temp` / `temp_bytes`: the ticket
+ * and the tile descriptors live in a fixed array of 256 B + 256 KiB inside the library's device
+ * image (one copy per GPU, held until the process ends), whose device address is looked up on the
+ * first call on each device; no call allocates or frees memory.  That first call must be made
+ * outside a stream capture: under capture on a device whose address is not known yet the call
+ * returns hipErrorStreamCaptureUnsupported (900) and launches nothing.  Limit: at most 16384 tiles of 128 KiB, i.e. 2 GiB
  * of input (n <= 2^31 elements of 1 byte, 2^30 of 2 bytes, 2^29 of 4 bytes, 2^28 of 8 bytes);
  * a larger n returns hipErrorOutOfMemory (2) before anything else is looked
  * at, and launches nothing.  All calls on one GPU share the array: calls

@@ -21,7 +21,7 @@ def test_cpp_tests_compile():
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
     for name in ["test_system_dir", "test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_host_vector", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface",
-                 "bench_generic", "bench_api", "bench_store_pattern"]:
+                 "bench_generic", "bench_api"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
 
 

@@ -21,7 +21,7 @@ with open(os.path.join(ROOT, "tests", "golden", "reference_unit_tests.json")) as
 
 def _check(name):
     cmd = [HIPCC, "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-fsyntax-only", "-w", "-H", "-ferror-limit=3",
-           "-I" + os.path.join(ROOT, "include"), "-I" + REF_TESTING, os.path.join(REF_TESTING, name + ".cu")]
+           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "tests", "shim"), "-I" + REF_TESTING, os.path.join(REF_TESTING, name + ".cu")]
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
     foreign = sorted({ln.split()[-1] for ln in p.stderr.splitlines()
                       if ln.startswith(".") and "/include/thrust/" in ln and not ln.split()[-1].startswith((ROOT, REF_TESTING))})

@@ -456,13 +456,20 @@ constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mu;
 static void* g_scratch_ptr[kMaxDevices];
 
-static hipError_t static_scratch(void** out) {
+static hipError_t static_scratch(void** out, hipStream_t stream) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
   std::lock_guard<std::mutex> g(g_scratch_mu);
   if (!g_scratch_ptr[dev]) {
+    // the look-up is not something to do while the caller records a graph
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) != hipSuccess) {
+      (void)hipGetLastError();
+      return hipErrorStreamCaptureUnsupported;
+    }
+    if (cs != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return e;
@@ -484,11 +491,11 @@ extern "C" int thrust_cdna4_scan_static(int dtype, int op, int exclusive, const 
   if (ntiles < 0) return hipErrorInvalidValue;  // unknown element type
   if (ntiles > kStaticScanMaxTiles) return hipErrorOutOfMemory;
   if (n > 0 && (!in || !out)) return hipErrorInvalidValue;
+  hipStream_t s = static_cast<hipStream_t>(stream);
   void* ptr = nullptr;
-  hipError_t rc = static_scratch(&ptr);
+  hipError_t rc = static_scratch(&ptr, s);
   if (rc != hipSuccess) return (int)rc;
   rc = hipErrorInvalidValue;
-  hipStream_t s = static_cast<hipStream_t>(stream);
   dispatch_dtype(dtype, [&](auto t) {
     using T = decltype(t);
     static_assert(TileDesc<typename ScanConfig<T>::P>::kBytesPerTile <= 16, "16 bytes of descriptor per tile");

@@ -653,9 +653,14 @@ static hipError_t ensure_lds_order(hipStream_t s) {
   int v = g_order_verdict[dev].load(std::memory_order_acquire);
   if (v == 1) return hipSuccess;
   if (v == 2) return hipErrorNotSupported;
+  // The check blocks, so it is left to a later call when this one may be recorded into a graph.
+  // A query that fails (the legacy stream while another thread captures) counts as capturing.
   hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(s, &cs) != hipSuccess) (void)hipGetLastError();
-  else if (cs != hipStreamCaptureStatusNone) return hipSuccess;
+  if (hipStreamIsCapturing(s, &cs) != hipSuccess) {
+    (void)hipGetLastError();
+    return hipSuccess;
+  }
+  if (cs != hipStreamCaptureStatusNone) return hipSuccess;
   std::lock_guard<std::mutex> g(g_order_mu);
   v = g_order_verdict[dev].load(std::memory_order_acquire);
   if (v == 0) {
@@ -750,9 +755,13 @@ static hipError_t xcd_groups_usable(hipStream_t s, bool* usable) {
   if (dev < 0 || dev >= kMaxDevices) return hipSuccess;
   int v = g_xcd_verdict[dev].load(std::memory_order_acquire);
   if (v == 0) {
+    // the probe blocks: a later call runs it (a failing query counts as capturing, as above)
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &cs) != hipSuccess) (void)hipGetLastError();
-    else if (cs != hipStreamCaptureStatusNone) return hipSuccess;  // the probe blocks: a later call runs it
+    if (hipStreamIsCapturing(s, &cs) != hipSuccess) {
+      (void)hipGetLastError();
+      return hipSuccess;
+    }
+    if (cs != hipStreamCaptureStatusNone) return hipSuccess;
     std::lock_guard<std::mutex> g(g_xcd_mu);
     v = g_xcd_verdict[dev].load(std::memory_order_acquire);
     if (v == 0) {
@@ -997,6 +1006,7 @@ extern "C" int thrust_cdna4_selftest_xcd_dispatch(int* grouped, void* stream) {
   if (!grouped) return hipErrorInvalidValue;
   bool ok = false;
   int why = 0;
+  std::lock_guard<std::mutex> g(tcd::g_xcd_mu);  // the probe's device arrays have one user at a time
   const hipError_t e = tcd::run_xcd_dispatch_probe(static_cast<hipStream_t>(stream), &ok, &why);
   *grouped = why;
   return (int)e;
