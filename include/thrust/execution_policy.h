@@ -1,6 +1,7 @@
 // thrust::device, thrust::host and the cdna4 stream policies (thrust/execution_policy.h:295, :344).
 #pragma once
 #include <thrust/system/cdna4/detail/core.h>
+#include <thrust/detail/seq.h>
 
 namespace thrust {
 // Bases for user-defined policies and tags (thrust/execution_policy.h:63-, :171-): an algorithm

@@ -11,6 +11,7 @@
 #include <thrust/pair.h>
 #include <thrust/scan.h>
 #include <thrust/system/cdna4/detail/algorithms.h>
+#include <thrust/system/detail/sequential/algorithms.h>
 
 #include <thrust/iterator/transform_iterator.h>
 namespace thrust {

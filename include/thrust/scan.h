@@ -9,6 +9,7 @@
 #include <thrust/system/cdna4/detail/algorithms.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
 #include <thrust/system/cdna4/detail/scan_generic.h>
+#include <thrust/system/detail/sequential/algorithms.h>
 
 namespace thrust {
 

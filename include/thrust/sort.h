@@ -12,6 +12,7 @@
 #include <thrust/functional.h>
 #include <thrust/system/cdna4/detail/algorithms.h>
 #include <thrust/system/cdna4/detail/generic_algorithms.h>
+#include <thrust/system/detail/sequential/algorithms.h>
 
 namespace thrust {
 

@@ -31,6 +31,9 @@ void sort_keys_impl(const Policy& exec, K* keys, std::int64_t n, Compare, std::t
   temporary_storage tmp(bytes, exec);
   throw_on_error(thrust_cdna4_sort_keys(tmp.data(), &bytes, dtype_of<K>::value, keys, n, order_code<Compare>::value, s),
                  "sort: launch");
+  // a synchronous call waits here and learns whether every wait inside the sort ended
+  // (thrust/system/cuda/detail/util.h:207-292); par_nosync leaves that to the caller
+  if (must_sync(exec)) throw_on_error(thrust_cdna4_sort_status(tmp.data(), n, s), "sort: a wait inside the sort did not end");
 }
 template <class Policy, class K, class Compare>
 void sort_keys_impl(const Policy& exec, K* keys, std::int64_t n, Compare comp, std::false_type) {
@@ -60,6 +63,7 @@ void sort_pairs_impl(const Policy& exec, K* keys, V* values, std::int64_t n, Com
   temporary_storage tmp(bytes, exec);
   throw_on_error(thrust_cdna4_sort_pairs(tmp.data(), &bytes, dtype_of<K>::value, keys, (int)sizeof(V), values, n,
                                          order_code<Compare>::value, s), "sort_by_key: launch");
+  if (must_sync(exec)) throw_on_error(thrust_cdna4_sort_status(tmp.data(), n, s), "sort_by_key: a wait inside the sort did not end");
 }
 template <class Policy, class K, class V, class Compare>
 void sort_pairs_impl(const Policy& exec, K* keys, V* values, std::int64_t n, Compare comp, std::false_type) {

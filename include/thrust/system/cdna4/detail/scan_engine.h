@@ -114,7 +114,7 @@ __device__ inline void join(const Op& op, bool& has_a, Acc& a, bool has_b, const
 
 // words[0, tiles * NW) are the descriptors, words[tiles * NW] is the ticket counter
 template <class Op>
-__global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n, Op op, unsigned long long* words, std::int64_t tiles) {
+__global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n, Op op, unsigned long long* words, std::int64_t tiles, unsigned* timeouts) {
   typedef typename Op::acc Acc;
   typedef scan_desc<Acc> Desc;
   constexpr int ITEMS = scan_items(sizeof(Acc));
@@ -229,9 +229,14 @@ __global__ __launch_bounds__(kScanBlock) void scan_engine_kernel(std::int64_t n,
         const unsigned long long use = full ? ((full & (0ull - full)) << 1) - 1ull : ~0ull;
         // (the tiles waited for hold earlier tickets, so they are running and will publish; the
         // poll limit — seconds — only makes sure that this loop ends whatever happens)
-        if ((empty & use) && ++spins < kScanSpinLimit) {
-          __builtin_amdgcn_s_sleep(1);
-          continue;
+        if (empty & use) {
+          if (++spins < kScanSpinLimit) {
+            __builtin_amdgcn_s_sleep(1);
+            continue;
+          }
+          // gives up and carries on with what it has; counted where the sort's time-outs are
+          // (thrust_cdna4_lookback_timeouts)
+          if (lane == 0 && timeouts) atomicAdd(timeouts, 1u);
         }
         // The window is folded in tile order — far to near, combine need not commute — by a
         // suffix reduction over the lanes: after step d lane l holds lanes l + 2d - 1 ... l.
@@ -323,7 +328,10 @@ void scan_engine(void* stream_, std::int64_t n, Op op) {
   temporary_storage tmp((std::size_t)nwords * sizeof(unsigned long long), stream_);
   unsigned long long* words = static_cast<unsigned long long*>(tmp.data());
   hipLaunchKernelGGL((select_init_kernel<unsigned long long>), dim3((unsigned)((nwords + 255) / 256)), dim3(256), 0, s, words, nwords);
-  hipLaunchKernelGGL((scan_engine_kernel<Op>), dim3((unsigned)tiles), dim3(kScanBlock), 0, s, n, op, words, tiles);
+  void* timeouts = nullptr;  // the library's per-device counter of waits that did not end
+  throw_on_error(thrust_cdna4_lookback_timeout_counter(&timeouts), "scan: time-out counter");
+  hipLaunchKernelGGL((scan_engine_kernel<Op>), dim3((unsigned)tiles), dim3(kScanBlock), 0, s, n, op, words, tiles,
+                     static_cast<unsigned*>(timeouts));
   throw_on_error((int)hipGetLastError(), "scan: launch");
 }
 

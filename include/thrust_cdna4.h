@@ -244,7 +244,7 @@ int thrust_cdna4_get_device(int* device);
 int thrust_cdna4_set_lookback_patience(int polls);
 /*
  * Test knob for that recomputation path; no counterpart in the reference.  Tile 0 of the
- * ticketless scan, scan_by_key and reduce_by_key kernels sleeps `sleeps` times (a few
+ * ticketless scan, scan_by_key and reduce_by_key kernels and of every pass of the sort sleeps `sleeps` times (a few
  * microseconds each, clamped to 100000) before it publishes its descriptor, so that with
  * patience 0 every later tile deterministically finds it missing, also at the second look.
  * Every kernel still runs to completion.  Returns the previous value; 0 (the default) switches
@@ -265,13 +265,45 @@ int thrust_cdna4_profile_count(void);
 int thrust_cdna4_profile_get(int index, const char** name, float* ms);
 
 /*
- * Diagnostics; no counterpart in the reference.  Every wait of the sort's look-back is bounded: a
- * digit's thread that polls a missing tile descriptor about 4 million times (seconds; a wait
- * that ends takes microseconds) gives up, the kernel still runs to completion — with a wrong
- * result — and the event is counted per device.  Blocks until the device is idle and stores the
- * count since the process started; anything but 0 means a sort result cannot be trusted.
+ * The outcome of the sort whose temporary storage was `temp` (n items, enqueued on `stream`):
+ * waits for the stream and returns hipSuccess, the stream's error, or hipErrorLaunchTimeOut (702)
+ * when a wait inside the sort did not end.  Replaces the error path of the reference's
+ * synchronous sort, which turns every runtime failure of its kernels into thrust::system_error
+ * (thrust/system/cuda/detail/util.h:207-292, throw_on_error after cuda_cub::synchronize).
+ *
+ * Every wait of the sort's look-back is bounded: a thread that polls a missing tile descriptor
+ * about 4 million times (seconds; a wait that ends takes microseconds) gives up and the kernels
+ * still run to completion, with keys at wrong positions inside the output.  The sort records
+ * that in the first word of its temporary storage, which this call reads; `temp` must still be
+ * the storage the sort was given (call this before handing it to anything else).  After a
+ * time-out, sorts on that device hand their tiles out from a single counter (the form whose
+ * waits rest on nothing but running workgroups) for the rest of the process.
+ *
+ * The synchronous policies of the template layer (thrust::device, par, par.on(stream)) and
+ * thrust_amd.sort call it in place of their synchronisation and throw.  A caller that does not
+ * synchronise (par_nosync, or this C ABI used directly) calls it when it does, or reads
+ * thrust_cdna4_lookback_timeouts: without one of the two a timed-out sort goes unnoticed.
+ * Sorts of up to 4096 items are one workgroup, have no such wait, and use nothing of `temp`.
+ */
+int thrust_cdna4_sort_status(const void* temp, int64_t n, void* stream);
+/*
+ * Diagnostics; no counterpart in the reference.  Counts the waits that did not end (see
+ * thrust_cdna4_sort_status) per device: blocks until the device is idle and stores the count
+ * since the process started; anything but 0 means that some sort's result cannot be trusted.
  */
 int thrust_cdna4_lookback_timeouts(unsigned long long* count);
+/* The device address of that counter (a 32-bit unsigned word) on the current device, for kernels
+ * built outside the library (the template layer's kernel templates add to it when one of their
+ * own bounded waits gives up). */
+int thrust_cdna4_lookback_timeout_counter(void** device_address);
+/*
+ * Test knob for that error path; no counterpart in the reference.  The number of polls after
+ * which a wait inside the sort gives up (negative: the default, about 4 million); returns the
+ * previous value.  With 0 and thrust_cdna4_set_test_publish_delay, tile 0 of a pass publishes
+ * late, the tiles that look for it give up at once, every kernel still runs to completion, and
+ * thrust_cdna4_sort_status reports the time-out.
+ */
+int thrust_cdna4_set_test_sort_spin_limit(long long polls);
 
 /*
  * Hardware self-test.  The sort kernels rank keys with returning LDS atomics and rely on the
@@ -305,6 +337,11 @@ int thrust_cdna4_selftest_xcd_dispatch(int* grouped, void* stream);
 /* Test knob: non-zero makes every later sort hand its tiles out from one counter (the form used on
  * devices that fail the probe above); returns the previous setting. */
 int thrust_cdna4_set_test_sort_plain_tickets(int on);
+/* Which form the library has settled on for the current device: 0 not decided yet (no large sort
+ * has run outside a stream capture), 1 groups of consecutive tiles per XCD, 2 the single counter
+ * (the probe failed, or a wait timed out).  The probe's own verdict is asked for up to three times
+ * when it rests on timing alone. */
+int thrust_cdna4_sort_tile_assignment(int* form);
 
 #ifdef __cplusplus
 }

@@ -20,9 +20,17 @@ def compile_snippet(tmp_path, body, extra=()):
 def test_cpp_tests_compile():
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    for name in ["test_system_dir", "test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_host_vector", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface",
+    for name in ["test_system_dir", "test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_host_vector", "test_scan_generic", "test_merge_sort", "bench_merge_sort", "test_generic", "test_select", "bench_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface", "test_seq",
                  "bench_generic", "bench_api"]:
         assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "build", name))
+
+
+def test_seq_algorithms_on_the_cpu():
+    # thrust::seq on host ranges: the sequential sort (in place, by rotations), scans and
+    # reduce_by_key that kernels call as well; the kernel half of the file runs on the GPU
+    path = os.path.join(ROOT, "tests", "cpp", "build", "test_seq")
+    r = subprocess.run([path, "Host"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "2 tests, 0 failed" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
 
 def test_oracle_runs_clean_under_the_sanitizers():

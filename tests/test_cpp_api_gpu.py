@@ -11,7 +11,7 @@ from conftest import ROOT
 
 BIN_DIR = os.path.join(ROOT, "tests", "cpp", "build")
 # test_scan_generic, test_merge_sort, test_generic and test_select instantiate kernel templates with user functors and are compiled by hipcc
-BINARIES = ["test_system_dir", "test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_host_vector", "test_scan_generic", "test_merge_sort", "test_generic", "test_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface"]
+BINARIES = ["test_system_dir", "test_dispatch", "test_algorithms", "test_complex", "test_merge_set", "test_memory", "test_sort", "test_scan", "test_by_key", "test_system", "test_host_vector", "test_scan_generic", "test_merge_sort", "test_generic", "test_select", "test_partition", "test_iterators", "test_async", "test_mr", "test_api_surface", "test_seq"]
 
 
 @pytest.mark.gpu

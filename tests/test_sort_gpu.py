@@ -195,6 +195,12 @@ def test_xcd_dispatch_selftest_and_both_tile_assignments():
                 thrust_amd.sort_by_key(dk, dv, descending=True)
                 ek, ev = oracle.sort_pairs(k64, v, descending=True)
                 assert same_bits(host(dk), ek) and same_bits(host(dv), ev), (plain, n)
+            if plain == 0:
+                # the leg above really ran the grouped form: the library's own cached verdict
+                # (its probe is repeated when it rests on timing alone) says so
+                form = ctypes.c_int(-1)
+                assert L.thrust_cdna4_sort_tile_assignment(ctypes.byref(form)) == 0
+                assert form.value == 1, form.value
         finally:
             L.thrust_cdna4_set_test_sort_plain_tickets(prev)
     after = ctypes.c_ulonglong(0)

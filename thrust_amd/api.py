@@ -74,6 +74,8 @@ def sort(keys, descending=False):
     tmp = _temp(nb.value, keys.device)
     capi.check(L.thrust_cdna4_sort_keys(_ptr(tmp), ctypes.byref(nb), code, _ptr(keys), n,
                                         int(descending), _stream()), "sort_keys")
+    # thrust::sort(thrust::device, ...) returns when the work is done and throws if it failed
+    capi.check(L.thrust_cdna4_sort_status(_ptr(tmp), n, _stream()), "sort_keys: a wait inside the sort did not end")
     return keys
 
 
@@ -94,6 +96,7 @@ def sort_by_key(keys, values, descending=False):
     capi.check(L.thrust_cdna4_sort_pairs(_ptr(tmp), ctypes.byref(nb), code, _ptr(keys), vb,
                                          _ptr(values), n, int(descending), _stream()),
                "sort_pairs")
+    capi.check(L.thrust_cdna4_sort_status(_ptr(tmp), n, _stream()), "sort_pairs: a wait inside the sort did not end")
     return keys, values
 
 

@@ -29,6 +29,8 @@ SYMBOLS = [
     "thrust_cdna4_stream_wait_event", "thrust_cdna4_malloc_direct", "thrust_cdna4_free_direct",
     "thrust_cdna4_malloc_universal", "thrust_cdna4_free_universal", "thrust_cdna4_get_device",
     "thrust_cdna4_selftest_xcd_dispatch", "thrust_cdna4_set_test_sort_plain_tickets",
+    "thrust_cdna4_sort_status", "thrust_cdna4_set_test_sort_spin_limit", "thrust_cdna4_sort_tile_assignment",
+    "thrust_cdna4_lookback_timeout_counter",
 ]
 
 
@@ -60,6 +62,10 @@ def lib():
     L.thrust_cdna4_error_string.argtypes = [i32]
     L.thrust_cdna4_sort_keys.argtypes = [vp, psz, i32, vp, i64, i32, vp]
     L.thrust_cdna4_sort_pairs.argtypes = [vp, psz, i32, vp, i32, vp, i64, i32, vp]
+    L.thrust_cdna4_sort_status.argtypes = [vp, i64, vp]
+    L.thrust_cdna4_set_test_sort_spin_limit.argtypes = [ctypes.c_longlong]
+    L.thrust_cdna4_sort_tile_assignment.argtypes = [ctypes.POINTER(i32)]
+    L.thrust_cdna4_lookback_timeout_counter.argtypes = [ctypes.POINTER(vp)]
     L.thrust_cdna4_scan.argtypes = [vp, psz, i32, i32, i32, vp, vp, i64, vp, vp]
     L.thrust_cdna4_scan_static.argtypes = [i32, i32, i32, vp, vp, i64, vp, vp]
     L.thrust_cdna4_scan_by_key.argtypes = [vp, psz, i32, i32, i32, i32, vp, vp, vp, i64, vp, vp]

@@ -231,9 +231,15 @@ __device__ inline void lds_store(uint32_t* p, uint32_t v) {
 
 // Look-back polls that find nothing new before a digit's thread gives up (seconds: far beyond
 // any wait that ends).  The kernel then still runs to completion, with wrong positions that
-// stay inside the output, and counts the event in g_lookback_timeouts.
+// stay inside the output; the event is recorded in the status word of the sort call (the first
+// word of its temporary storage, read by thrust_cdna4_sort_status) and counted per device in
+// g_lookback_timeouts.
 constexpr uint32_t kLookbackSpinLimit = 1u << 22;
 __device__ unsigned int g_lookback_timeouts;
+__device__ inline void note_timeout(uint32_t* status) {
+  atomicOr(status, 1u);
+  atomicAdd(&g_lookback_timeouts, 1u);
+}
 
 // The tile a workgroup processes, with the pass's flags in the top bits.  Plain form (xcd == nullptr):
 // the next ticket of the pass's counter — tiles start in index order, so every tile that a look-back
@@ -244,7 +250,7 @@ __device__ unsigned int g_lookback_timeouts;
 // order and groups are claimed in index order, so the lowest tile that has not started belongs to an
 // XCD all of whose running tiles are lower — they need nothing from it and finish —, and that XCD
 // starts its next workgroup whatever the other XCDs are doing (also checked): every wait ends.
-__device__ inline uint32_t take_tile(uint32_t* ticket, uint32_t* xcd, int xcd_slots) {
+__device__ inline uint32_t take_tile(uint32_t* ticket, uint32_t* xcd, int xcd_slots, uint32_t spin_limit, uint32_t* status) {
   if (xcd == nullptr) return atomicAdd(ticket, 1u);
   const uint32_t x = blockIdx.x % kXcds;
   const uint32_t idx = atomicAdd(&xcd[x * kXcdCounterStride], 1u);
@@ -258,11 +264,16 @@ __device__ inline uint32_t take_tile(uint32_t* ticket, uint32_t* xcd, int xcd_sl
     // the workgroup that took the group's first tile started before this one and writes the cell
     // right after its own atomic; the poll limit only makes sure that the loop ends
     uint32_t v = ld_agent(cell), spins = 0;
-    while (v == 0u && ++spins < kLookbackSpinLimit) {
+    while (v == 0u && ++spins < spin_limit) {
       __builtin_amdgcn_s_sleep(1);
       v = ld_agent(cell);
     }
-    if (v == 0u) atomicAdd(&g_lookback_timeouts, 1u);
+    if (v == 0u) {
+      // no group number: the workgroup leaves (as for a skipped pass); the tile it would have
+      // taken is never published, the tiles after it time out as well, and the call reports it
+      note_timeout(status);
+      return kPassSkipped;
+    }
     group_word = v - 1u;
   }
   return (group_word & ~kTicketMask) | ((group_word & kTicketMask) * kXcdGroup + within);
@@ -272,7 +283,8 @@ template <class U, int VB, bool FLOAT, int BLOCK, int IPT, int WPE, class D>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) void onesweep_kernel(U* kmain, U* kalt, void* vmain, void* valt,
                                                          int64_t n, U xor_mask, int shift,
                                                          const uint32_t* __restrict__ gbase,
-                                                         D* desc, uint32_t* ticket, uint32_t* xcd, int xcd_slots) {
+                                                         D* desc, uint32_t* ticket, uint32_t* xcd, int xcd_slots,
+                                                         uint32_t* status, uint32_t spin_limit, int publish_delay) {
   static_assert(BLOCK % 256 == 0, "one thread per digit needs at least 256 threads");
   using V = typename value_of<VB>::type;
   constexpr int NWAVES = BLOCK / kWave;
@@ -284,7 +296,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
 
-  if (tid == 0) sm.tile = take_tile(ticket, xcd, xcd_slots);
+  if (tid == 0) sm.tile = take_tile(ticket, xcd, xcd_slots, spin_limit, status);
   if (tid < kRadix / 2) {
 #pragma unroll
     for (int w = 0; w < NWAVES; w++) reinterpret_cast<uint32_t*>(sm.wave_cnt[w])[tid] = 0;
@@ -384,6 +396,8 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
 #pragma unroll
     for (int w = 0; w < NWAVES; w++) total += sm.wave_cnt[w][tid];
     const uint32_t st = (tile == 0) ? kInclusive : kPartial;
+    if (tile == 0)
+      for (int i = 0; i < publish_delay; i++) __builtin_amdgcn_s_sleep(127);  // test knob, 0 in normal use
     st_agent(&desc[tile * kRadix + tid], DescWord<D>::make(st, total));
     const uint32_t incl = wave_inclusive_scan(total, 0u, [](uint32_t a, uint32_t b) { return a + b; });
     if (lane == 63) sm.wave_tot[wave] = incl;
@@ -436,8 +450,8 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
         t -= used;
         if (used == 0) {
           __builtin_amdgcn_s_sleep(2);
-          if (++spins > kLookbackSpinLimit) {  // never in a working system; keeps every wait bounded
-            atomicAdd(&g_lookback_timeouts, 1u);
+          if (++spins > spin_limit) {  // never in a working system; keeps every wait bounded
+            note_timeout(status);
             done = true;
           }
         }
@@ -765,9 +779,15 @@ static hipError_t xcd_groups_usable(hipStream_t s, bool* usable) {
     std::lock_guard<std::mutex> g(g_xcd_mu);
     v = g_xcd_verdict[dev].load(std::memory_order_acquire);
     if (v == 0) {
+      // a verdict that rests on timing (-1) is asked for up to three times before it is believed:
+      // it stays for the life of the process and costs a pair sort 10 %
       bool ok = false;
-      e = run_xcd_dispatch_probe(s, &ok);
-      if (e != hipSuccess) return e;
+      int why = 0;
+      for (int attempt = 0; attempt < 3 && !ok; attempt++) {
+        e = run_xcd_dispatch_probe(s, &ok, &why);
+        if (e != hipSuccess) return e;
+        if (why != -1) break;
+      }
       v = ok ? 1 : 2;
       g_xcd_verdict[dev].store(v, std::memory_order_release);
     }
@@ -802,7 +822,7 @@ constexpr int64_t kSortMaxN = (int64_t(1) << 32) - 1;
 constexpr int64_t small_sort_limit(int value_bytes) { return int64_t(1) << (21 + (value_bytes ? 1 : 0)); }
 
 struct SortPlan {
-  size_t keys_alt, vals_alt, hist, tickets, xcd, desc, total;
+  size_t status, keys_alt, vals_alt, hist, tickets, xcd, desc, total;
   int xcd_slots;  // groups an XCD may take in one pass
   size_t zero_begin, zero_bytes;
   int64_t ntiles;
@@ -841,6 +861,8 @@ __global__ __launch_bounds__(kFillThreads) void counting_fill_kernel(uint8_t* ou
   }
 }
 
+constexpr size_t kSortStatusOffset = 0;  // of the status word in a sort call's temporary storage
+static std::atomic<uint32_t> g_test_spin_limit{kLookbackSpinLimit};  // test knob
 static constexpr size_t xcd_words_per_pass(int slots) { return (size_t)kXcds * kXcdCounterStride + (size_t)kXcds * (size_t)slots; }
 template <class U, int VB, class C, class D>
 static SortPlan make_plan(int64_t n) {
@@ -849,9 +871,9 @@ static SortPlan make_plan(int64_t n) {
   p.ntiles = ceil_div(n, C::TILE);
   size_t off = 0;
   constexpr bool kCounting = sizeof(U) == 1 && VB == 0;  // histogram and fill: no alternate buffer, no descriptors
-  p.keys_alt = off; off += kCounting ? 0 : align_up((size_t)n * sizeof(U), 256);
-  p.vals_alt = off; off += align_up((size_t)n * VB, 256);
+  // what starts at zero comes first; its first word is the call's status (kSortStatusOffset)
   p.zero_begin = off;
+  p.status = off; off += 256;
   p.hist = off; off += align_up((size_t)P * kRadix * 4, 256);
   p.tickets = off; off += 256;
   // per pass: a counter per XCD (a cache line each) and the numbers of the groups each XCD took
@@ -859,6 +881,8 @@ static SortPlan make_plan(int64_t n) {
   p.xcd = off; off += kCounting ? 0 : align_up((size_t)P * xcd_words_per_pass(p.xcd_slots) * 4, 256);
   p.desc = off; off += kCounting ? 0 : align_up((size_t)P * p.ntiles * kRadix * sizeof(D), 256);
   p.zero_bytes = off - p.zero_begin;
+  p.keys_alt = off; off += kCounting ? 0 : align_up((size_t)n * sizeof(U), 256);
+  p.vals_alt = off; off += align_up((size_t)n * VB, 256);
   p.total = off;
   return p;
 }
@@ -889,6 +913,10 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   uint32_t* ghist = reinterpret_cast<uint32_t*>(t + plan.hist);
   uint32_t* tickets = reinterpret_cast<uint32_t*>(t + plan.tickets);
   D* desc = reinterpret_cast<D*>(t + plan.desc);
+  static_assert(kSortStatusOffset == 0, "thrust_cdna4_sort_status reads the first word");
+  uint32_t* status = reinterpret_cast<uint32_t*>(t + plan.status);
+  const uint32_t spin_limit = g_test_spin_limit.load(std::memory_order_relaxed);
+  const int publish_delay = lookback_test_publish_delay();
 
   hipError_t e = zero_async(t + plan.zero_begin, plan.zero_bytes, stream);
   if (e != hipSuccess) return e;
@@ -922,7 +950,8 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
     uint32_t* xcd = grouped ? reinterpret_cast<uint32_t*>(t + plan.xcd) + (size_t)p * xcd_words_per_pass(plan.xcd_slots) : nullptr;
     TCD_LAUNCH("onesweep_kernel", (onesweep_kernel<U, VB, FLOAT, C::BLOCK, C::IPT, C::WPE, D>), dim3((unsigned)grid),
                dim3(C::BLOCK), stream, kbuf[0], kbuf[1], static_cast<void*>(vbuf[0]), static_cast<void*>(vbuf[1]), n, xor_mask, 8 * p,
-               ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix, tickets + p, xcd, plan.xcd_slots);
+               ghist + p * kRadix, desc + (size_t)p * plan.ntiles * kRadix, tickets + p, xcd, plan.xcd_slots,
+               status, spin_limit, publish_delay);
   }
   e = hipGetLastError();
   if (e != hipSuccess) return e;
@@ -1010,6 +1039,45 @@ extern "C" int thrust_cdna4_selftest_xcd_dispatch(int* grouped, void* stream) {
   const hipError_t e = tcd::run_xcd_dispatch_probe(static_cast<hipStream_t>(stream), &ok, &why);
   *grouped = why;
   return (int)e;
+}
+
+extern "C" int thrust_cdna4_sort_tile_assignment(int* form) {
+  if (!form) return hipErrorInvalidValue;
+  int dev = 0;
+  const hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  *form = (dev >= 0 && dev < tcd::kMaxDevices) ? tcd::g_xcd_verdict[dev].load(std::memory_order_acquire) : 2;
+  return hipSuccess;
+}
+
+extern "C" int thrust_cdna4_set_test_sort_spin_limit(long long polls) {
+  const uint32_t v = polls < 0 ? tcd::kLookbackSpinLimit : (uint32_t)(polls > 0xffffffffLL ? 0xffffffffLL : polls);
+  return (int)tcd::g_test_spin_limit.exchange(v, std::memory_order_relaxed);
+}
+
+extern "C" int thrust_cdna4_sort_status(const void* temp, int64_t n, void* stream) {
+  using namespace tcd;
+  if (n < 0 || (n > kTileSortMax && !temp)) return hipErrorInvalidValue;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipError_t e;
+  uint32_t word = 0;
+  if (n > kTileSortMax) {  // smaller sorts are one workgroup: no look-back, and nothing of `temp` is used
+    e = hipMemcpyAsync(&word, static_cast<const char*>(temp) + kSortStatusOffset, sizeof(word), hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) return (int)e;
+  }
+  e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return (int)e;
+  if (word == 0) return hipSuccess;
+  // a wait that did not end: whatever the reason, later sorts on this device hand their tiles
+  // out from the single counter, whose waits depend on nothing the probe had to observe
+  int dev = 0;
+  if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices) g_xcd_verdict[dev].store(2, std::memory_order_release);
+  return hipErrorLaunchTimeOut;
+}
+
+extern "C" int thrust_cdna4_lookback_timeout_counter(void** device_address) {
+  if (!device_address) return hipErrorInvalidValue;
+  return (int)hipGetSymbolAddress(device_address, HIP_SYMBOL(tcd::g_lookback_timeouts));
 }
 
 extern "C" int thrust_cdna4_lookback_timeouts(unsigned long long* count) {
