@@ -98,7 +98,14 @@ int thrust_cdna4_sort_pairs(void* temp, size_t* temp_bytes, int key_dtype, void*
  * `init` is a HOST pointer to one element of `dtype` (NULL = value-initialised, the
  * reference's default, scan.h:347-348).  `in == out` is allowed
  * (testing/scan.cu:86-105).  Integer results are bit-exact (two's-complement wraparound);
- * floating-point results are a reassociation of the serial left fold.
+ * floating-point sums and products are a reassociation of the serial left fold: they differ from
+ * it, and from one run to the next (which tile's look-back sees which neighbour's aggregate
+ * first depends on timing, and with it the grouping), by rounding only.  Floating-point
+ * maximum and minimum select an input value and are bit-exact; maximum (a < b ? b : a) is so
+ * with NaNs as well — the serial fold keeps a NaN that starts it (element 0, or *init) and
+ * skips NaNs met later, and so do scan, scan_by_key (per segment) and reduce_by_key (per run).
+ * minimum (a < b ? a : b) with NaN inputs is NOT the serial fold, in which every NaN restarts
+ * the fold: here the results around a NaN depend on the grouping.
  */
 int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int op, int exclusive,
                       const void* in, void* out, int64_t n, const void* init, void* stream);

@@ -262,3 +262,54 @@ def test_by_key_mixed_run_lengths_match_oracle(kd, vd):
             assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op=op)), oracle.scan_by_key(k, v, op=op)), (n, op)
         assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=3)),
                          oracle.scan_by_key(k, v, exclusive=True, init=3)), n
+
+
+@pytest.mark.parametrize("vd", [np.float32, np.float64])
+def test_float_maximum_by_key_with_nans_is_the_serial_fold(vd):
+    """thrust::maximum is a < b ? b : a: in the serial folds (thrust/system/detail/sequential/
+    scan_by_key.h:46-142, reduce_by_key.h:43-95) a NaN at the head of a segment stays for the whole
+    segment, a NaN inside one is skipped, and the exclusive form — whose folds start from `init` —
+    skips every NaN unless `init` is one.  Same bits from the kernels, over several tiles."""
+    rng = np.random.default_rng(21)
+    for n in (1, 2, 9, 2049, 16385, 50021, 200003):
+        for mean in (1, 3, 300):
+            k = runs(n + mean, n, mean)
+            head = np.ones(n, bool)
+            head[1:] = k[1:] != k[:-1]
+            for where in ("none", "heads", "inside", "both", "all"):
+                v = rng.uniform(-5, 5, n).astype(vd)
+                v[rng.random(n) < 0.05] = vd(-np.inf)
+                if where in ("heads", "both"):
+                    v[head & (rng.random(n) < 0.5)] = np.nan
+                if where in ("inside", "both"):
+                    v[~head & (rng.random(n) < 0.3)] = np.nan
+                if where == "all":
+                    v[:] = np.nan
+                dk, dv = dev(k), dev(v)
+                assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op="maximum")),
+                                 oracle.scan_by_key(k, v, op="maximum")), (n, mean, where)
+                for init in (vd(1.5), vd(np.nan)):
+                    assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=init, op="maximum")),
+                                     oracle.scan_by_key(k, v, op="maximum", exclusive=True, init=init)), (n, mean, where, init)
+                ko, vo = thrust_amd.reduce_by_key(dk, dv, op="maximum")
+                ek, ev = oracle.reduce_by_key(k, v, op="maximum")
+                assert same_bits(host(ko), ek) and same_bits(host(vo), ev), (n, mean, where)
+                y = dev(v)
+                thrust_amd.inclusive_scan_by_key(dk, y, out=y, op="maximum")  # in place: tiles by ticket
+                assert same_bits(host(y), oracle.scan_by_key(k, v, op="maximum")), (n, mean, where, "in place")
+
+
+def test_float_maximum_by_key_with_nans_on_the_recompute_path(no_patience, tile0_publishes_late):
+    rng = np.random.default_rng(22)
+    n = 16384 * 3 + 5
+    for mean in (1, 40):
+        k = runs(n + mean, n, mean)
+        v = rng.uniform(-5, 5, n).astype(np.float32)
+        v[rng.random(n) < 0.3] = np.nan
+        dk, dv = dev(k), dev(v)
+        assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op="maximum")), oracle.scan_by_key(k, v, op="maximum")), mean
+        assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=np.float32(0.25), op="maximum")),
+                         oracle.scan_by_key(k, v, op="maximum", exclusive=True, init=np.float32(0.25))), mean
+        ko, vo = thrust_amd.reduce_by_key(dk, dv, op="maximum")
+        ek, ev = oracle.reduce_by_key(k, v, op="maximum")
+        assert same_bits(host(ko), ek) and same_bits(host(vo), ev), mean

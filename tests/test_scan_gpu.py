@@ -184,3 +184,55 @@ def test_scan_in_place_takes_the_ticket_path_and_out_of_place_does_not():
     dst = buf[:x.size]  # starts 256 bytes before the input
     thrust_amd.inclusive_scan(src, out=dst)
     assert same_bits(host(dst), ref)
+
+
+def _with_nans(rng, n, where, dt):
+    x = rng.uniform(-5, 5, n).astype(dt)
+    x[rng.random(n) < 0.05] = dt(-np.inf)
+    if where == "first":
+        x[0] = np.nan
+    elif where == "middle" and n > 2:
+        x[n // 2] = np.nan
+        x[1] = np.nan
+    elif where == "many":
+        x[rng.random(n) < 0.3] = np.nan
+        x[0] = dt(1.0)
+    elif where == "many_and_first":
+        x[rng.random(n) < 0.3] = np.nan
+        x[0] = np.nan
+    elif where == "all":
+        x[:] = np.nan
+    return x
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_float_maximum_scans_with_nans_are_the_serial_fold(dt):
+    """thrust::maximum is a < b ? b : a: the serial fold (thrust/system/detail/sequential/scan.h:54-72)
+    keeps a NaN that starts it and skips NaNs met later.  The kernel must give the same bits whatever
+    its grouping: NaN first, in the middle, scattered, everywhere; a NaN `init`; several tiles; in place."""
+    rng = np.random.default_rng(11)
+    for n in (1, 2, 5, 4097, 70001, 300007):
+        for where in ("none", "first", "middle", "many", "many_and_first", "all"):
+            x = _with_nans(rng, n, where, dt)
+            d = dev(x)
+            assert same_bits(host(thrust_amd.inclusive_scan(d, op="maximum")), oracle.scan(x, op="maximum")), (n, where)
+            for init in (dt(0.5), dt(np.nan), dt(-np.inf)):
+                assert same_bits(host(thrust_amd.exclusive_scan(d, init=init, op="maximum")),
+                                 oracle.scan(x, op="maximum", exclusive=True, init=init)), (n, where, init)
+            y = dev(x)
+            thrust_amd.inclusive_scan(y, out=y, op="maximum")  # in place: tiles by ticket
+            assert same_bits(host(y), oracle.scan(x, op="maximum")), (n, where, "in place")
+            y = dev(x)
+            thrust_amd.exclusive_scan(y, out=y, init=dt(np.nan), op="maximum")
+            assert same_bits(host(y), oracle.scan(x, op="maximum", exclusive=True, init=dt(np.nan))), (n, where, "in place, NaN init")
+
+
+def test_float_maximum_scan_with_nans_on_the_recompute_path(no_patience, tile0_publishes_late):
+    rng = np.random.default_rng(12)
+    n = 32768 * 3 + 77
+    for where in ("first", "many", "many_and_first"):
+        x = _with_nans(rng, n, where, np.float32)
+        d = dev(x)
+        assert same_bits(host(thrust_amd.inclusive_scan(d, op="maximum")), oracle.scan(x, op="maximum")), where
+        assert same_bits(host(thrust_amd.exclusive_scan(d, init=np.float32(2.0), op="maximum")),
+                         oracle.scan(x, op="maximum", exclusive=True, init=np.float32(2.0))), where

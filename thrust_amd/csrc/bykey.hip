@@ -214,10 +214,19 @@ struct SegTile {
   // (every tile waited for has started; used when an output overlaps an input); otherwise a tile
   // is the workgroup of the same index and a descriptor that stays missing after `patience` polls
   // is recomputed from the input.
+  // maximum(a, b) = a < b ? b : a over floating-point values with NaNs is not associative: the
+  // serial fold keeps a NaN that STARTS it (NaN < x is false) and skips a NaN met later
+  // (acc < NaN is false too).  A NaN that cannot start a fold is therefore replaced by the
+  // identity as the elements are classified — every NaN but those of segment heads; and those
+  // too when `folds_start_from_init` (exclusive_scan_by_key, whose folds start from `init`).  What
+  // is left is associative, and a NaN only ever appears as the operator's LEFT operand, where it
+  // is kept.  Nothing of this is compiled for other types and operators.
+  static constexpr bool kNanAware = std::is_floating_point<T>::value && std::is_same<Op, OpMaximum>::value;
+
   template <bool TICKET, class Meanwhile>
   __device__ void run(Smem& sm, const KU* keys, const T* vals, int64_t n, int float_keys, int vec_ok,
                       uint64_t* desc, uint32_t* ticket, tcd_v4u* xbuf, int patience, int publish_delay,
-                      Meanwhile meanwhile) {
+                      bool folds_start_from_init, Meanwhile meanwhile) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -273,6 +282,9 @@ struct SegTile {
       for (int j = 0; j < VEC; j++) {
         const KU p = j == 0 ? prev : key[j - 1];
         const bool is_head = (full || i0 + j < n) && (i0 + j == 0 || keys_differ(p, key[j], float_keys));
+        if constexpr (kNanAware) {
+          if ((folds_start_from_init || !is_head) && __builtin_isnan(val[j])) val[j] = id;
+        }
         h |= (is_head ? 1u : 0u) << j;
         agg.v = is_head ? val[j] : Op::template apply<T>(agg.v, val[j]);
       }
@@ -313,8 +325,11 @@ struct SegTile {
             Pair a = idp;
             for (int k = 0; k < PIECE; k++) {
               const KU kk = keys[start + k];
-              const T vv = vals[start + k];
+              T vv = vals[start + k];
               const bool is_head = start + k == 0 || keys_differ(before, kk, float_keys);
+              if constexpr (kNanAware) {
+                if ((folds_start_from_init || !is_head) && __builtin_isnan(vv)) vv = Op::template identity<T>();
+              }
               a.c += is_head ? 1u : 0u;
               a.v = is_head ? vv : Op::template apply<T>(a.v, vv);
               before = kk;
@@ -356,7 +371,7 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void scan_by_key_ke
   constexpr int EPP = 16 / (int)sizeof(T);  // elements per 16-byte slot
   bool parked = false;
   uint32_t first_head = 0;
-  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, [&] {
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, exclusive != 0, [&] {
     if (!t.full) return;
     parked = true;
     T r[VEC];
@@ -393,7 +408,12 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void scan_by_key_ke
         __builtin_memcpy(x, &piece, 16);
 #pragma unroll
         for (int e = 0; e < EPP; e++)
-          if ((uint32_t)((q * kWave + lane) * EPP + e) < first_head) x[e] = Op::template apply<T>(carried, x[e]);
+          if ((uint32_t)((q * kWave + lane) * EPP + e) < first_head) {
+            // the run's value so far goes in front of what the wavefront folded; the exclusive
+            // form has `init` in front of both, inside x[e] (the operands commute unless one
+            // is a NaN, which — see kNanAware — can only be the first in fold order)
+            x[e] = exclusive ? Op::template apply<T>(x[e], carried) : Op::template apply<T>(carried, x[e]);
+          }
         __builtin_memcpy(&piece, x, 16);
       }
       store16(dst + (q * kWave + lane) * 16, piece);
@@ -459,7 +479,7 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void reduce_by_key_
   T* const early_v = reinterpret_cast<T*>(reinterpret_cast<char*>(xbuf) + kHalfBytes);
   bool early = false;
   uint32_t count = 0;
-  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, [&] {
+  t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, false, [&] {
     count = (uint32_t)__builtin_amdgcn_readlane((int)(t.excl_w.c + __builtin_popcount(t.heads)), kWave - 1);
     early = t.full && count <= kEarlyMax;
     if (!early) {

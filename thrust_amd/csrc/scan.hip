@@ -60,6 +60,17 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
   const T* tin = in + base + (int64_t)tid * VEC;
   T* tout = out + base + (int64_t)tid * VEC;
 
+  // maximum(a, b) = a < b ? b : a over floating-point values with NaNs is not associative: the
+  // serial fold keeps a NaN that STARTS it (NaN < x is false) and skips a NaN met later
+  // (acc < NaN is false too).  So every NaN is replaced by the identity as it is loaded, which
+  // leaves an associative fold, and the one NaN that the serial fold would have kept — the first
+  // value of the fold: element 0, or `init` of an exclusive scan — is handled apart: all results
+  // are then that NaN.  (An in-place scan may already have overwritten element 0: with the same
+  // bits.)  Nothing of this is compiled for other types and operators.
+  constexpr bool kNanAware = std::is_floating_point<T>::value && std::is_same<Op, OpMaximum>::value;
+  T lead = id;
+  if constexpr (kNanAware) lead = exclusive ? init : in[0];
+
   T x[CHUNKS][VEC];
   if (fast) {
 #pragma unroll
@@ -78,6 +89,12 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         x[c][j] = idx < n ? got : id;
       }
     }
+  }
+  if constexpr (kNanAware) {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++)
+#pragma unroll
+      for (int j = 0; j < VEC; j++) x[c][j] = __builtin_isnan(x[c][j]) ? id : x[c][j];
   }
 
   // thread-local inclusive scan of each 16-byte group, then a wave scan of the group sums
@@ -122,9 +139,14 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         // the aggregate of an earlier tile (always a whole one), straight from the input
         const auto aggregate_of = [&](int64_t t) -> W {
           const T* p = in + t * TILE + lane;
-          T acc = p[0];
+          const auto element = [&](int k) {
+            const T e = p[(int64_t)k * kWave];
+            if constexpr (kNanAware) return __builtin_isnan(e) ? id : e;
+            else return e;
+          };
+          T acc = element(0);
 #pragma unroll 8
-          for (int k = 1; k < (int)(TILE / kWave); k++) acc = op(acc, p[(int64_t)k * kWave]);
+          for (int k = 1; k < (int)(TILE / kWave); k++) acc = op(acc, element(k));
           return readlane(wave_inclusive_scan(toW(acc), idW, opW), kWave - 1);
         };
         prefix = wave_lookback_or_compute<W>(desc, tile, idW, opW, patience, aggregate_of);
@@ -153,6 +175,14 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
     } else {
 #pragma unroll
       for (int j = 0; j < VEC; j++) x[c][j] = op(off, x[c][j]);
+    }
+  }
+  if constexpr (kNanAware) {
+    if (__builtin_isnan(lead)) {
+#pragma unroll
+      for (int c = 0; c < CHUNKS; c++)
+#pragma unroll
+        for (int j = 0; j < VEC; j++) x[c][j] = lead;
     }
   }
   if (fast) {
