@@ -398,7 +398,8 @@ def main():
         cpu = {
             "value": round(m / best / 1e9, 4), "unit": "Gkeys/s", "cores": threads, "kind": "port",
             "sample": f"2^{args.log2n} uniform uint32 keys (the whole GPU workload), best of 3; oracle "
-                      f"restatement of the reference OpenMP sort (per-thread radix sort + pairwise merges)",
+                      f"restatement of the reference OpenMP sort (per-thread radix sort with the reference's "
+                      f"digit widths, 4 bits for these tiles, + pairwise merges)",
         }
 
         # the other algorithms of the path: the scalar oracle (the reference's sequential loops

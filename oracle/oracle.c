@@ -60,9 +60,19 @@ static int dtype_enc(int dt) {
 /* One histogram pass over all digits (:262-271), exclusive scan per digit with the    */
 /* "one bin holds everything" skip (:274-289), then one stable scatter per digit       */
 /* (:292-323), ping-ponging between the two buffers, and a final copy back (:326-).    */
-/* The reference picks 3/4/8-bit digits by key size and N (:443-515); the digit width   */
-/* does not change the result of a stable LSD sort, so 8 bits are used throughout.     */
+/* The digit width is the reference's choice by key size, values and N                  */
+/* (radix_sort_dispatcher, :345-515): it does not change the result of a stable LSD     */
+/* sort, but it is what the timed CPU baseline pays for (eight 4-bit passes over 2^24   */
+/* four-byte keys per thread, not four 8-bit ones).                                     */
 /* ---------------------------------------------------------------------------------- */
+static int reference_radix_bits(int key_bytes, int has_values, size_t n) {
+  switch (key_bytes) {
+    case 1: return 8;                                                   /* :345-372 */
+    case 2: return n < ((size_t)1 << (has_values ? 15 : 16)) ? 8 : 16;  /* :375-428 */
+    case 4: return n < ((size_t)1 << 22) ? 8 : (has_values ? 3 : 4);    /* :431-473 */
+    default: return n < ((size_t)1 << 21) ? 8 : (has_values ? 3 : 4);   /* :476-518 */
+  }
+}
 
 #define DEFINE_RADIX(W, UT)                                                              \
   static inline UT encode_##W(UT x, int enc) {                                           \
@@ -73,21 +83,24 @@ static int dtype_enc(int dt) {
   }                                                                                      \
   static int radix_sort_##W(UT* keys1, UT* keys2, unsigned char* vals1,                  \
                             unsigned char* vals2, int vb, size_t n, int enc) {           \
-    enum { NH = W / 8 };                                                                 \
-    size_t(*hist)[256] = calloc(NH, sizeof(size_t[256]));                                \
-    int skip[NH];                                                                        \
+    const int bits = reference_radix_bits(W / 8, vb != 0, n);                            \
+    const int NH = (W + bits - 1) / bits; /* digits per key (:240) */                    \
+    const size_t NB = (size_t)1 << bits;  /* bins per digit */                           \
+    const UT mask = (UT)(NB - 1);                                                        \
+    size_t* hist = calloc((size_t)NH * NB, sizeof(size_t));                              \
+    int skip[64];                                                                        \
     if (!hist) return 1;                                                                 \
     for (size_t i = 0; i < n; i++) {                                                     \
       UT x = encode_##W(keys1[i], enc);                                                  \
-      for (int j = 0; j < NH; j++) hist[j][(x >> (8 * j)) & 0xff]++;                     \
+      for (int j = 0; j < NH; j++) hist[(size_t)j * NB + ((x >> (bits * j)) & mask)]++;  \
     }                                                                                    \
     for (int j = 0; j < NH; j++) {                                                       \
       size_t sum = 0;                                                                    \
       skip[j] = 0;                                                                       \
-      for (int b = 0; b < 256; b++) {                                                    \
-        size_t c = hist[j][b];                                                           \
+      for (size_t b = 0; b < NB; b++) {                                                  \
+        size_t c = hist[(size_t)j * NB + b];                                             \
         if (c == n) skip[j] = 1;                                                         \
-        hist[j][b] = sum;                                                                \
+        hist[(size_t)j * NB + b] = sum;                                                  \
         sum += c;                                                                        \
       }                                                                                  \
     }                                                                                    \
@@ -98,10 +111,10 @@ static int dtype_enc(int dt) {
       UT* dst = flip ? keys1 : keys2;                                                    \
       const unsigned char* vsrc = flip ? vals2 : vals1;                                  \
       unsigned char* vdst = flip ? vals1 : vals2;                                        \
-      size_t* h = hist[j];                                                               \
+      size_t* h = hist + (size_t)j * NB;                                                 \
       for (size_t i = 0; i < n; i++) {                                                   \
         UT k = src[i];                                                                   \
-        size_t pos = h[(encode_##W(k, enc) >> (8 * j)) & 0xff]++;                        \
+        size_t pos = h[(encode_##W(k, enc) >> (bits * j)) & mask]++;                     \
         dst[pos] = k;                                                                    \
         switch (vb) {                                                                    \
           case 0: break;                                                                 \
