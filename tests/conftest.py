@@ -10,8 +10,59 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+# THRUST_CDNA4_EMULATED=1 runs the GPU parity tests WITHOUT a GPU: the C ABI is served by the host
+# build of the same kernel sources under the lockstep emulator (tests/emu), "device" tensors are CPU
+# tensors, and the harness's device checks are relaxed here, in the tests, never in the package.
+# tests/test_emulated_kernels.py starts such sessions; nothing else sets the variable.
+EMULATED = os.environ.get("THRUST_CDNA4_EMULATED") == "1"
+EMU_LIB = os.path.join(ROOT, "tests", "emu", "build", "libthrust_cdna4_emu.so")
+if EMULATED:
+    os.environ["THRUST_CDNA4_LIB"] = EMU_LIB
+
+
+def _enter_emulated_session():
+    import ctypes
+
+    import torch
+
+    import gpu_util
+    import thrust_amd.api as api
+
+    def need_contiguous(*ts):
+        for t in ts:
+            if t is not None and not t.is_contiguous():
+                raise ValueError("contiguous tensors required")
+
+    api._need_cuda = need_contiguous
+    api._stream = lambda: ctypes.c_void_p(0)
+    # THRUST_CDNA4_EMULATED_RESIDENT="k" or "k:seed": workgroups in flight (default 1, one after the other)
+    k, _, seed = os.environ.get("THRUST_CDNA4_EMULATED_RESIDENT", "1").partition(":")
+    emu = ctypes.CDLL(EMU_LIB)
+    emu.emu_set_resident_workgroups.argtypes = [ctypes.c_int, ctypes.c_uint64]
+    emu.emu_set_resident_workgroups(int(k), int(seed or 1))
+    gpu_util.DEVICE = "cpu"
+    gpu_util.dev = lambda a: torch.from_numpy(np.array(a, copy=True, order="C"))
+    gpu_util.host = lambda t: t.numpy().copy()
+    gpu_util.stream_handle = lambda: ctypes.c_void_p(0)
+    gpu_util.synchronize = lambda: None
+    gpu_util.empty_cache = lambda: None
+    gpu_util.memory_allocated = lambda: 0
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    config.addinivalue_line("markers", "needs_device: a gpu test that the emulated session cannot run")
+    if EMULATED:
+        _enter_emulated_session()
+
+
+def pytest_collection_modifyitems(config, items):
+    if not EMULATED:
+        return
+    skip = pytest.mark.skip(reason="needs the device itself (full-size input, graphs, streams, timing)")
+    for item in items:
+        if "needs_device" in item.keywords:
+            item.add_marker(skip)
 
 
 @pytest.fixture(scope="session")

@@ -1,0 +1,193 @@
+// Stand-in for <hip/hip_runtime.h> that lets the kernel sources of thrust_amd/csrc be compiled for
+// the HOST and run there, lane by lane, by the lockstep emulator in tests/emu/emu.cpp.
+//
+// TEST INFRASTRUCTURE ONLY.  Nothing of the product includes or links this; the library that it
+// builds (tests/emu/build/libthrust_cdna4_emu.so) is loaded by tests/test_emulated_kernels.py alone,
+// to run the very kernel code on the CPU — one workgroup after the other, every wavefront in
+// lockstep — where no GPU is at hand.  It checks what a kernel computes (indexing, layouts, the
+// order of combinations, edge tiles), not how workgroups interleave on the device.
+//
+// What a kernel sees here:
+//   * threadIdx / blockIdx / blockDim / gridDim of the lane that is running;
+//   * __shared__ as thread-local static storage (a workgroup in flight has a thread of its own);
+//   * __syncthreads / s_barrier as a rendezvous of the workgroup's lanes;
+//   * the cross-lane operations (DPP moves, ds_bpermute, readlane, readfirstlane, ballot) and every
+//     atomicAdd / atomicOr as a rendezvous of the wavefront's lanes that execute it, served in lane
+//     order — which is also the order the LDS unit serves same-address atomics of one instruction in,
+//     the property the sort's ranking relies on;
+//   * agent-scope atomic loads and stores as plain accesses (one host thread runs everything).
+#pragma once
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#define __global__
+#define __device__
+#define __host__
+#define __shared__ static thread_local
+#define __launch_bounds__(...)
+#define __forceinline__ inline __attribute__((always_inline))
+#define __align__(n) __attribute__((aligned(n)))
+
+// ---- the error codes and handle types the sources name ----
+typedef int hipError_t;
+enum : int {
+  hipSuccess = 0,
+  hipErrorInvalidValue = 1,
+  hipErrorOutOfMemory = 2,
+  hipErrorInvalidSymbol = 13,
+  hipErrorInvalidDevice = 101,
+  hipErrorLaunchTimeOut = 702,
+  hipErrorNotSupported = 801,
+  hipErrorStreamCaptureUnsupported = 900,
+};
+typedef void* hipStream_t;
+enum hipStreamCaptureStatus { hipStreamCaptureStatusNone = 0, hipStreamCaptureStatusActive = 1 };
+enum hipMemcpyKind { hipMemcpyHostToDevice = 1, hipMemcpyDeviceToHost = 2, hipMemcpyDeviceToDevice = 3 };
+
+struct dim3 {
+  unsigned x, y, z;
+  dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
+};
+
+namespace emu {
+struct Index3 { unsigned x, y, z; };
+struct LaneView {  // what the running lane reads through threadIdx & co.
+  Index3 thread, block, block_dim, grid_dim;
+};
+LaneView& view();
+
+// rendezvous operations of a wavefront; each blocks the calling lane until the wavefront's lanes
+// that execute the same operation have arrived, and returns the lane's result
+int dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl);
+int bpermute(int byte_address, int src);
+int readlane(int v, int lane);
+int readfirstlane(int v);
+uint64_t ballot(bool pred);
+void wave_barrier();
+void workgroup_barrier();
+void sleep();  // s_sleep: the wavefront steps aside until the others have had a turn
+// atomics: all lanes of the wavefront that execute the instruction, served in lane order
+uint32_t atomic_add_u32(uint32_t* p, uint32_t v);
+uint64_t atomic_add_u64(uint64_t* p, uint64_t v);
+uint32_t atomic_or_u32(uint32_t* p, uint32_t v);
+uint64_t lockstep_load(const void* p, int bytes);
+void lockstep_store(void* p, uint64_t v, int bytes);
+int lane();  // 0..63
+uint64_t clock();
+
+void launch(dim3 grid, dim3 block, void (*trampoline)(void*), void* closure);
+template <class F>
+inline void launch_closure(dim3 grid, dim3 block, const F& f) {
+  launch(grid, block, [](void* c) { (*static_cast<const F*>(c))(); }, const_cast<F*>(&f));
+}
+}  // namespace emu
+
+#define threadIdx (::emu::view().thread)
+#define blockIdx (::emu::view().block)
+#define blockDim (::emu::view().block_dim)
+#define gridDim (::emu::view().grid_dim)
+
+// ---- launches: synchronous, one workgroup after the other ----
+#define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) \
+  ::emu::launch_closure(dim3(grid), dim3(block), [=]() { kernel(__VA_ARGS__); })
+
+// ---- the host API the sources call ----
+inline hipError_t hipGetLastError() { return hipSuccess; }
+inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+inline hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus* s) { *s = hipStreamCaptureStatusNone; return hipSuccess; }
+inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+inline hipError_t hipMemcpyAsync(void* dst, const void* src, size_t n, hipMemcpyKind, hipStream_t) { memcpy(dst, src, n); return hipSuccess; }
+#define HIP_SYMBOL(x) (&(x))
+template <class T> inline hipError_t hipGetSymbolAddress(void** p, T* sym) { *p = (void*)sym; return hipSuccess; }
+template <class T> inline hipError_t hipMemcpyFromSymbol(void* dst, T* sym, size_t n) { memcpy(dst, (const void*)sym, n); return hipSuccess; }
+// device memory is host memory; events complete at once
+enum { hipDeviceAttributeMultiprocessorCount = 63, hipEventDisableTiming = 2, hipHostMallocDefault = 0, hipMemAttachGlobal = 1 };
+enum : int { hipErrorNotReady = 600 };
+inline hipError_t hipDeviceGetAttribute(int* v, int, int) { *v = 256; return hipSuccess; }
+enum { hipHostMallocPortable = 1, hipStreamNonBlocking = 1 };
+inline const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "no error" : "error (emulated runtime)"; }
+inline hipError_t hipStreamCreateWithFlags(hipStream_t* s, unsigned) { *s = malloc(1); return hipSuccess; }
+inline hipError_t hipStreamDestroy(hipStream_t s) { free(s); return hipSuccess; }
+inline hipError_t hipStreamQuery(hipStream_t) { return hipSuccess; }
+struct emu_event {};
+typedef emu_event* hipEvent_t;
+inline hipError_t hipEventCreate(hipEvent_t* e) { *e = new emu_event; return hipSuccess; }
+inline hipError_t hipEventCreateWithFlags(hipEvent_t* e, unsigned) { *e = new emu_event; return hipSuccess; }
+inline hipError_t hipEventDestroy(hipEvent_t e) { delete e; return hipSuccess; }
+inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
+inline hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
+inline hipError_t hipEventQuery(hipEvent_t) { return hipSuccess; }
+inline hipError_t hipEventElapsedTime(float* ms, hipEvent_t, hipEvent_t) { *ms = 0.f; return hipSuccess; }
+inline hipError_t hipStreamWaitEvent(hipStream_t, hipEvent_t, unsigned) { return hipSuccess; }
+inline hipError_t hipMalloc(void** p, size_t n) { *p = aligned_alloc(256, (n + 255) / 256 * 256 + 256); return *p ? hipSuccess : hipErrorOutOfMemory; }
+inline hipError_t hipFree(void* p) { free(p); return hipSuccess; }
+inline hipError_t hipHostMalloc(void** p, size_t n, unsigned) { return hipMalloc(p, n); }
+inline hipError_t hipMallocManaged(void** p, size_t n, unsigned) { return hipMalloc(p, n); }
+inline hipError_t hipHostFree(void* p) { free(p); return hipSuccess; }
+template <class K> inline hipError_t hipOccupancyMaxActiveBlocksPerMultiprocessor(int* nb, K, int, size_t) { *nb = 2; return hipSuccess; }
+
+// ---- memory scopes and ordered accesses ----
+#define __HIP_MEMORY_SCOPE_WAVEFRONT 1
+#define __HIP_MEMORY_SCOPE_WORKGROUP 2
+#define __HIP_MEMORY_SCOPE_AGENT 3
+// An ordered access of WAVEFRONT scope says that the kernel counts on the wavefront's lanes executing
+// it together (all lanes load before any lane runs the store that follows): a rendezvous here.  Wider
+// scopes talk to other wavefronts and are plain accesses.
+template <class T>
+inline T emu_ordered_load(const T* p, int scope) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit");
+  if (scope != __HIP_MEMORY_SCOPE_WAVEFRONT) return __atomic_load_n(p, __ATOMIC_RELAXED);
+  const uint64_t r = ::emu::lockstep_load(p, (int)sizeof(T));
+  return (T)r;
+}
+template <class T, class V>
+inline void emu_ordered_store(T* p, V v, int scope) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit");
+  if (scope != __HIP_MEMORY_SCOPE_WAVEFRONT) __atomic_store_n(p, (T)v, __ATOMIC_RELAXED);
+  else ::emu::lockstep_store(p, (uint64_t)(T)v, (int)sizeof(T));
+}
+#define __hip_atomic_load(p, order, scope) emu_ordered_load((p), (scope))
+#define __hip_atomic_store(p, v, order, scope) emu_ordered_store((p), (v), (scope))
+inline uint32_t emu_fetch_add(uint32_t* p, uint32_t v) { return ::emu::atomic_add_u32(p, v); }
+inline uint64_t emu_fetch_add(uint64_t* p, uint64_t v) { return ::emu::atomic_add_u64(p, v); }
+inline unsigned long long emu_fetch_add(unsigned long long* p, unsigned long long v) { return ::emu::atomic_add_u64((uint64_t*)p, v); }
+#define __hip_atomic_fetch_add(p, v, order, scope) emu_fetch_add((p), (v))
+inline uint32_t atomicAdd(uint32_t* p, uint32_t v) { return ::emu::atomic_add_u32(p, v); }
+inline unsigned long long atomicAdd(unsigned long long* p, unsigned long long v) { return ::emu::atomic_add_u64((uint64_t*)p, v); }
+inline uint32_t atomicOr(uint32_t* p, uint32_t v) { return ::emu::atomic_or_u32(p, v); }
+
+// ---- gfx950 builtins ----
+#define __popcll(x) __builtin_popcountll(x)
+#define __popc(x) __builtin_popcount(x)
+#define __syncthreads() ::emu::workgroup_barrier()
+#define __ballot(pred) ::emu::ballot((pred) != 0)
+inline unsigned emu_mbcnt_lo(unsigned mask, unsigned base) {
+  const int l = ::emu::lane();
+  const unsigned below = l >= 32 ? 0xffffffffu : ((1u << l) - 1u);
+  return base + (unsigned)__builtin_popcount(mask & below);
+}
+inline unsigned emu_mbcnt_hi(unsigned mask, unsigned base) {
+  const int l = ::emu::lane();
+  const unsigned below = l <= 32 ? 0u : ((1u << (l - 32)) - 1u);
+  return base + (unsigned)__builtin_popcount(mask & below);
+}
+#define __builtin_amdgcn_mbcnt_lo(mask, base) emu_mbcnt_lo((mask), (base))
+#define __builtin_amdgcn_mbcnt_hi(mask, base) emu_mbcnt_hi((mask), (base))
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound) ::emu::dpp((old), (src), (ctrl), (row_mask), (bank_mask), (bound))
+#define __builtin_amdgcn_ds_bpermute(addr, src) ::emu::bpermute((addr), (src))
+#define __builtin_amdgcn_readlane(v, l) ::emu::readlane((v), (l))
+#define __builtin_amdgcn_readfirstlane(v) ::emu::readfirstlane((v))
+#define __builtin_amdgcn_ballot_w64(pred) ::emu::ballot((pred))
+#define __builtin_amdgcn_wave_barrier() ::emu::wave_barrier()
+#define __builtin_amdgcn_s_barrier() ::emu::workgroup_barrier()
+#define __builtin_amdgcn_fence(...) ((void)0)
+#define __builtin_amdgcn_s_sleep(n) ::emu::sleep()
+#define __builtin_amdgcn_s_setprio(n) ((void)0)
+#define __builtin_amdgcn_sched_barrier(n) ((void)0)
+#define __builtin_amdgcn_s_memtime() ::emu::clock()
+#define __builtin_amdgcn_s_memrealtime() ::emu::clock()
+#define __builtin_amdgcn_s_getreg(x) 0u

@@ -6,6 +6,7 @@ import torch
 import oracle
 import thrust_amd
 from conftest import SMALL_SIZES, random_ints, same_bits
+import gpu_util
 from gpu_util import dev, host
 
 pytestmark = pytest.mark.gpu
@@ -146,18 +147,19 @@ def test_reduce_by_key_ops_and_float_keys():
     assert same_bits(host(gk), rk) and host(gv).tolist() == [1, 2, 3, 4, 11]
 
 
+@pytest.mark.needs_device
 def test_reduce_by_key_empty_and_full_size_closed_form():
-    gk, gv = thrust_amd.reduce_by_key(torch.empty(0, dtype=torch.int32, device="cuda"),
-                                      torch.empty(0, dtype=torch.int32, device="cuda"))
+    gk, gv = thrust_amd.reduce_by_key(torch.empty(0, dtype=torch.int32, device=gpu_util.DEVICE),
+                                      torch.empty(0, dtype=torch.int32, device=gpu_util.DEVICE))
     assert gk.numel() == 0 and gv.numel() == 0
     # 2^28 elements, keys = i // 512, values = 1: every run sums to 512
     # (closed form, cf. testing/cuda/reduce_by_key.cu:339-400)
     n = 1 << 28
-    keys = torch.arange(n, dtype=torch.int32, device="cuda") // 512
-    vals = torch.ones(n, dtype=torch.int32, device="cuda")
+    keys = torch.arange(n, dtype=torch.int32, device=gpu_util.DEVICE) // 512
+    vals = torch.ones(n, dtype=torch.int32, device=gpu_util.DEVICE)
     gk, gv = thrust_amd.reduce_by_key(keys, vals)
     assert gk.numel() == n // 512
-    assert torch.equal(gk, torch.arange(n // 512, dtype=torch.int32, device="cuda"))
+    assert torch.equal(gk, torch.arange(n // 512, dtype=torch.int32, device=gpu_util.DEVICE))
     assert bool((gv == 512).all())
 
 

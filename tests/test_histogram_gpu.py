@@ -6,6 +6,7 @@ import torch
 import oracle
 import thrust_amd
 from conftest import ALL_DTYPES, same_bits
+import gpu_util
 from gpu_util import dev, host
 
 pytestmark = pytest.mark.gpu
@@ -60,9 +61,10 @@ def test_histogram_all_types_general_ranges(dtype):
         assert same_bits(got, oracle.histogram_even(s, bins, lo, hi)), (bins, lo, hi)
 
 
+@pytest.mark.needs_device
 def test_histogram_full_size_closed_form():
     # 2^30 u8 samples i % 256: every bin holds exactly 2^22
     n = 1 << 30
-    s = (torch.arange(n, dtype=torch.int32, device="cuda") & 255).to(torch.uint8)
+    s = (torch.arange(n, dtype=torch.int32, device=gpu_util.DEVICE) & 255).to(torch.uint8)
     got = counts(thrust_amd.histogram_even(s, 256, 0, 256))
     assert (got == (1 << 22)).all()

@@ -8,6 +8,7 @@ import torch
 import oracle
 import thrust_amd
 from conftest import INT_DTYPES, SIZES, random_ints, same_bits
+import gpu_util
 from gpu_util import dev, host
 
 pytestmark = pytest.mark.gpu
@@ -83,17 +84,18 @@ def test_scan_unaligned_in_place():
     assert host(d)[0] == x[0]
 
 
+@pytest.mark.needs_device
 def test_scan_full_size_closed_forms():
     # 2^28 elements (benchmark configuration 2): constants have closed-form scans
     n = 1 << 28
-    ones = torch.ones(n, dtype=torch.int32, device="cuda")
+    ones = torch.ones(n, dtype=torch.int32, device=gpu_util.DEVICE)
     out = thrust_amd.inclusive_scan(ones)
-    assert torch.equal(out, torch.arange(1, n + 1, dtype=torch.int32, device="cuda"))
+    assert torch.equal(out, torch.arange(1, n + 1, dtype=torch.int32, device=gpu_util.DEVICE))
     thrust_amd.exclusive_scan(ones, out=ones, init=0)  # in place
-    assert torch.equal(ones, torch.arange(0, n, dtype=torch.int32, device="cuda"))
+    assert torch.equal(ones, torch.arange(0, n, dtype=torch.int32, device=gpu_util.DEVICE))
     del ones, out
-    g = torch.Generator(device="cuda").manual_seed(5)
-    x = torch.randint(0, 16, (n,), dtype=torch.int32, device="cuda", generator=g)
+    g = torch.Generator(device=gpu_util.DEVICE).manual_seed(5)
+    x = torch.randint(0, 16, (n,), dtype=torch.int32, device=gpu_util.DEVICE, generator=g)
     incl = thrust_amd.inclusive_scan(x)
     excl = thrust_amd.exclusive_scan(x, init=0)
     assert torch.equal(incl - excl, x)  # inclusive[i] - exclusive[i] == x[i]
@@ -162,9 +164,10 @@ def test_scan_recompute_path_matches_oracle(no_patience):
     assert (np.abs(got - ref) <= FP_RTOL * np.cumsum(np.abs(f.astype(np.float64)))).all()
 
 
+@pytest.mark.needs_device
 def test_scan_full_size_recompute_path(no_patience):
     n = 1 << 28
-    x = torch.ones(n, dtype=torch.int32, device="cuda")
+    x = torch.ones(n, dtype=torch.int32, device=gpu_util.DEVICE)
     out = thrust_amd.inclusive_scan(x)
     assert int(out[-1].item()) == n and int(out[12345678].item()) == 12345679
     assert bool((out[1:] - out[:-1] == 1).all())
@@ -178,7 +181,7 @@ def test_scan_in_place_takes_the_ticket_path_and_out_of_place_does_not():
     assert same_bits(host(thrust_amd.inclusive_scan(d)), ref)
     thrust_amd.inclusive_scan(d, out=d)
     assert same_bits(host(d), ref)
-    buf = torch.empty(x.size + 64, dtype=torch.int32, device="cuda")
+    buf = torch.empty(x.size + 64, dtype=torch.int32, device=gpu_util.DEVICE)
     src = buf[64:]
     src.copy_(dev(x))
     dst = buf[:x.size]  # starts 256 bytes before the input

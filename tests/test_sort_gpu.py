@@ -7,6 +7,7 @@ import oracle
 import thrust_amd
 from conftest import (FLOAT_DTYPES, INT_DTYPES, SIZES, SMALL_SIZES, encoded, random_floats, random_ints,
                       same_bits, splitmix64)
+import gpu_util
 from gpu_util import dev, host
 
 pytestmark = pytest.mark.gpu
@@ -131,11 +132,12 @@ def test_sort_unaligned_views_and_repeat_determinism():
         assert got == first
 
 
+@pytest.mark.needs_device
 def test_sort_full_size_properties():
     # 2^28 u32 keys: sortedness + multiset preserved (checksums), no oracle at this size
     n = 1 << 28
-    g = torch.Generator(device="cuda").manual_seed(1337)
-    k = torch.randint(-2**31, 2**31, (n,), dtype=torch.int32, device="cuda", generator=g)
+    g = torch.Generator(device=gpu_util.DEVICE).manual_seed(1337)
+    k = torch.randint(-2**31, 2**31, (n,), dtype=torch.int32, device=gpu_util.DEVICE, generator=g)
     s0 = k.sum(dtype=torch.int64).item()
     x0 = 0
     for chunk in k.view(16, -1):
@@ -148,6 +150,7 @@ def test_sort_full_size_properties():
     assert int(np.bitwise_xor.reduce(hk)) == x0
 
 
+@pytest.mark.needs_device
 def test_lds_atomic_order_selftest():
     """The stable ranking of the sort kernels assumes that returning LDS atomics of one wavefront
     instruction are served in lane order; the library's self-test checks that on this device."""
@@ -156,11 +159,12 @@ def test_lds_atomic_order_selftest():
     from thrust_amd import capi
     L = capi.lib()
     bad = ctypes.c_longlong(-1)
-    rc = L.thrust_cdna4_selftest_lds_atomic_order(ctypes.byref(bad), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    rc = L.thrust_cdna4_selftest_lds_atomic_order(ctypes.byref(bad), gpu_util.stream_handle())
     assert rc == 0
     assert bad.value == 0
 
 
+@pytest.mark.needs_device
 def test_xcd_dispatch_selftest_and_both_tile_assignments():
     """Large sorts hand consecutive tiles to one XCD in groups (its L2 then merges the run ends that
     two tiles write into one cache line) on a device that passes the library's dispatch probe; MI355X
@@ -170,11 +174,11 @@ def test_xcd_dispatch_selftest_and_both_tile_assignments():
 
     from thrust_amd import capi
     L = capi.lib()
-    torch.cuda.synchronize()
+    gpu_util.synchronize()
     verdicts = []
     for _ in range(3):  # 1: the device qualifies; 0 / -1 / -2: why not (the probe times workgroups: it is conservative under load)
         grouped = ctypes.c_int(-9)
-        rc = L.thrust_cdna4_selftest_xcd_dispatch(ctypes.byref(grouped), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        rc = L.thrust_cdna4_selftest_xcd_dispatch(ctypes.byref(grouped), gpu_util.stream_handle())
         assert rc == 0
         verdicts.append(grouped.value)
     print("xcd dispatch probe:", verdicts)
@@ -252,32 +256,33 @@ def test_sort_pairs_large_tiles_stability(kd, vd):
         assert same_bits(host(dk), rk) and same_bits(host(dv), rv), descending
 
 
+@pytest.mark.needs_device
 def test_sort_beyond_2p30_items():
     """n >= 2^30 switches the tile descriptors to 64-bit words (digit counts no longer fit 30
     bits).  No oracle at this size: sortedness, multiset checksums, and for pairs stability and
     key/value association, all checked on the device."""
     n = (1 << 30) + 12345
-    g = torch.Generator(device="cuda").manual_seed(2030)
-    k = torch.randint(-2**31, 2**31, (n,), dtype=torch.int32, device="cuda", generator=g)
+    g = torch.Generator(device=gpu_util.DEVICE).manual_seed(2030)
+    k = torch.randint(-2**31, 2**31, (n,), dtype=torch.int32, device=gpu_util.DEVICE, generator=g)
     s0 = int(k.sum(dtype=torch.int64).item())
     thrust_amd.sort(k)
     assert bool((k[1:] >= k[:-1]).all())
     assert int(k.sum(dtype=torch.int64).item()) == s0
     del k
-    torch.cuda.empty_cache()
+    gpu_util.empty_cache()
     # pairs: few distinct keys, so every digit count of the top passes exceeds 2^30 / 256 by far
-    src = torch.randint(0, 1000, (n,), dtype=torch.int32, device="cuda", generator=g)
+    src = torch.randint(0, 1000, (n,), dtype=torch.int32, device=gpu_util.DEVICE, generator=g)
     k = src.clone()
-    v = torch.arange(n, dtype=torch.int32, device="cuda")
+    v = torch.arange(n, dtype=torch.int32, device=gpu_util.DEVICE)
     thrust_amd.sort_by_key(k, v)
     assert bool((k[1:] >= k[:-1]).all())
     assert bool(((k[1:] > k[:-1]) | (v[1:] > v[:-1])).all())  # equal keys keep their input order
     assert bool((src[v.long()] == k).all())
     del src, k, v
-    torch.cuda.empty_cache()
+    gpu_util.empty_cache()
     # one-byte keys at the largest size the entry point takes (2^32 - 2): run starts near 2^32
     n = (1 << 32) - 2
-    k = torch.randint(0, 4, (n,), dtype=torch.uint8, device="cuda", generator=g) * 85
+    k = torch.randint(0, 4, (n,), dtype=torch.uint8, device=gpu_util.DEVICE, generator=g) * 85
     step = 1 << 30
     counts = sum(torch.bincount(k[a:a + step].to(torch.int32), minlength=256) for a in range(0, n, step))
     thrust_amd.sort(k, descending=True)
@@ -344,7 +349,7 @@ def test_sort_one_byte_keys_by_counting(dtype):
         for name, k in cases.items():
             for descending in (False, True):
                 for shift in (0, 1, 7):
-                    buf = torch.zeros(n + 32, dtype=torch.int8 if dtype == np.int8 else torch.uint8, device="cuda")
+                    buf = torch.zeros(n + 32, dtype=torch.int8 if dtype == np.int8 else torch.uint8, device=gpu_util.DEVICE)
                     view = buf[shift:shift + n]
                     view.copy_(dev(k))
                     thrust_amd.sort(view, descending)

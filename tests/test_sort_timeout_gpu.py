@@ -17,6 +17,7 @@ import torch
 import oracle
 import thrust_amd
 from conftest import random_ints, same_bits
+import gpu_util
 from gpu_util import dev, host
 from thrust_amd import capi
 
@@ -53,11 +54,11 @@ def test_a_sort_whose_lookback_gives_up_reports_it_and_later_sorts_are_right():
         # and through the C ABI: the launch itself succeeds, the status call reports the time-out
         d = dev(k)
         v = dev(np.arange(n, dtype=np.uint32))
-        sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        sp = gpu_util.stream_handle()
         nb = ctypes.c_size_t(0)
         args = (capi.U32, ctypes.c_void_p(d.data_ptr()), 4, ctypes.c_void_p(v.data_ptr()), n, 0, sp)
         assert L.thrust_cdna4_sort_pairs(None, ctypes.byref(nb), *args) == 0
-        tmp = torch.empty(nb.value, dtype=torch.uint8, device="cuda")
+        tmp = torch.empty(nb.value, dtype=torch.uint8, device=gpu_util.DEVICE)
         assert L.thrust_cdna4_sort_pairs(ctypes.c_void_p(tmp.data_ptr()), ctypes.byref(nb), *args) == 0
         assert L.thrust_cdna4_sort_status(ctypes.c_void_p(tmp.data_ptr()), n, sp) == HIP_ERROR_LAUNCH_TIMEOUT
     finally:
@@ -77,10 +78,10 @@ def test_a_sort_whose_lookback_gives_up_reports_it_and_later_sorts_are_right():
 
 def test_small_and_one_byte_sorts_have_nothing_to_report():
     L = capi.lib()
-    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sp = gpu_util.stream_handle()
     # up to 4096 items nothing of the temporary storage is used, not even its status word
     assert L.thrust_cdna4_sort_status(None, 4096, sp) == 0
-    garbage = torch.full((4096,), 0xFF, dtype=torch.uint8, device="cuda")
+    garbage = torch.full((4096,), 0xFF, dtype=torch.uint8, device=gpu_util.DEVICE)
     assert L.thrust_cdna4_sort_status(ctypes.c_void_p(garbage.data_ptr()), 100, sp) == 0
     k = random_ints(1, 1 << 20, np.uint8)
     d = dev(k)

@@ -45,15 +45,9 @@ class Cdna4Error(RuntimeError):
 _lib = None
 
 
-def lib():
-    global _lib
-    if _lib is not None:
-        return _lib
-    if not os.path.exists(LIB_PATH):
-        raise ImportError(
-            f"{LIB_PATH} is missing: build it with `make -C thrust_amd/csrc` "
-            "(or __graft_entry__.build()); there is no CPU fallback")
-    L = ctypes.CDLL(LIB_PATH)
+def bind(path):
+    """Load a build of the C ABI from `path` and declare every entry point's argument types."""
+    L = ctypes.CDLL(path)
     vp, sz, i32, i64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int64
     psz = ctypes.POINTER(ctypes.c_size_t)
     dbl = ctypes.c_double
@@ -102,8 +96,19 @@ def lib():
     L.thrust_cdna4_set_test_sort_plain_tickets.argtypes = [i32]
     L.thrust_cdna4_profile_get.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p),
                                            ctypes.POINTER(ctypes.c_float)]
-    _lib = L
     return L
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `make -C thrust_amd/csrc` "
+            "(or __graft_entry__.build()); there is no CPU fallback")
+    _lib = bind(LIB_PATH)
+    return _lib
 
 
 def profile_records():
