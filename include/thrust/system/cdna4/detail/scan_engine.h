@@ -61,7 +61,7 @@ struct scan_desc {
       if (k == 0) st = s;
       else same = same && s == st;
     }
-    __builtin_memcpy(&a, w, sizeof(Acc));
+    __builtin_memcpy(static_cast<void*>(&a), w, sizeof(Acc));
     return same ? st : 0u;
   }
 };
@@ -75,7 +75,7 @@ __device__ inline Acc shfl_up_acc(const Acc& a, int d) {
 #pragma unroll
   for (int k = 0; k < NW; k++) w[k] = __shfl_up(w[k], (unsigned)d, 64);
   Acc r;
-  __builtin_memcpy(&r, w, sizeof(Acc));
+  __builtin_memcpy(static_cast<void*>(&r), w, sizeof(Acc));
   return r;
 }
 
@@ -88,7 +88,7 @@ __device__ inline Acc shfl_down_acc(const Acc& a, int d) {
 #pragma unroll
   for (int k = 0; k < NW; k++) w[k] = __shfl_down(w[k], (unsigned)d, 64);
   Acc r;
-  __builtin_memcpy(&r, w, sizeof(Acc));
+  __builtin_memcpy(static_cast<void*>(&r), w, sizeof(Acc));
   return r;
 }
 

@@ -101,11 +101,13 @@ int thrust_cdna4_sort_pairs(void* temp, size_t* temp_bytes, int key_dtype, void*
  * floating-point sums and products are a reassociation of the serial left fold: they differ from
  * it, and from one run to the next (which tile's look-back sees which neighbour's aggregate
  * first depends on timing, and with it the grouping), by rounding only.  Floating-point
- * maximum and minimum select an input value and are bit-exact; maximum (a < b ? b : a) is so
- * with NaNs as well — the serial fold keeps a NaN that starts it (element 0, or *init) and
- * skips NaNs met later, and so do scan, scan_by_key (per segment) and reduce_by_key (per run).
- * minimum (a < b ? a : b) with NaN inputs is NOT the serial fold, in which every NaN restarts
- * the fold: here the results around a NaN depend on the grouping.
+ * maximum and minimum select an input value and give the serial fold's bits, NaNs and signed
+ * zeros included, in scan, scan_by_key (per segment) and reduce_by_key (per run): maximum
+ * (a < b ? b : a) keeps a NaN that starts the fold (element 0, or *init) and skips NaNs met later,
+ * and keeps the first of +0 and -0; minimum (a < b ? a : b) restarts at every NaN (the NaN
+ * replaces the accumulator, the next element replaces the NaN) and keeps the last of +0 and -0.
+ * The price of minimum's restarts: its floating-point instantiations publish one more word per
+ * tile and always hand out tiles by ticket.
  */
 int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int op, int exclusive,
                       const void* in, void* out, int64_t n, const void* init, void* stream);
@@ -120,7 +122,8 @@ int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int op, int exc
  * first call on each device; no call allocates or frees memory.  That first call must be made
  * outside a stream capture: under capture on a device whose address is not known yet the call
  * returns hipErrorStreamCaptureUnsupported (900) and launches nothing.  Limit: at most 16384 tiles of 128 KiB, i.e. 2 GiB
- * of input (n <= 2^31 elements of 1 byte, 2^30 of 2 bytes, 2^29 of 4 bytes, 2^28 of 8 bytes);
+ * of input (n <= 2^31 elements of 1 byte, 2^30 of 2 bytes, 2^29 of 4 bytes, 2^28 of 8 bytes;
+ * 10922 tiles for minimum over 8-byte floating-point values, whose tiles publish three words);
  * a larger n returns hipErrorOutOfMemory (2) before anything else is looked
  * at, and launches nothing.  All calls on one GPU share the array: calls
  * that overlap in time on one GPU (different streams, or different host threads) race and must

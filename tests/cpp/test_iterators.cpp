@@ -5,6 +5,7 @@
 // histogram of examples/histogram.cu (sort, upper_bound of a counting range, adjacent_difference).
 // Compiled by hipcc.
 #include <algorithm>
+#include <cmath>
 #include <numeric>
 
 #include <thrust/adjacent_difference.h>

@@ -77,6 +77,7 @@ enum Op : int {
   kReadlane,
   kReadfirst,
   kBallot,
+  kShuffle,
   kWaveBarrier,
   kAtomicAdd32,
   kAtomicAdd64,
@@ -92,9 +93,12 @@ static bool is_cross_lane(int op) { return op >= kDpp && op <= kWaveBarrier; }
 
 struct Lane {
   void* sp = nullptr;
+  void* stack_top = nullptr;
   LaneView view;
   int op = kRun;
-  const void* site = nullptr;
+  const void* site = nullptr;  // return address of the call that parked the lane
+  long depth = 0;              // and how deep in its stack the lane was: the same call of the source, reached
+                               // through another caller of a function that was not inlined, is another operation
   int a[5] = {0, 0, 0, 0, 0};
   bool flag = false;
   void* ptr = nullptr;
@@ -163,14 +167,15 @@ LaneView& view() { return g_cur ? g_cur->view : g_host_view; }
 int lane() { return (int)(g_cur - g_lanes) % kWave; }
 uint64_t clock() { return g_clock += 100; }
 
-static void park(int op, const void* site) {
+static void park(int op, const void* site, const void* frame) {
   Lane* me = g_cur;
   me->op = op;
   me->site = site;
+  me->depth = static_cast<const char*>(me->stack_top) - static_cast<const char*>(frame);
   emu_switch(&me->sp, g_sched_sp);
 }
 
-#define EMU_SITE __builtin_extract_return_addr(__builtin_return_address(0))
+#define EMU_SITE __builtin_extract_return_addr(__builtin_return_address(0)), __builtin_frame_address(0)
 
 __attribute__((noinline)) int dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
   Lane* me = g_cur;
@@ -182,6 +187,12 @@ __attribute__((noinline)) int bpermute(int byte_address, int src) {
   Lane* me = g_cur;
   me->a[0] = byte_address, me->a[1] = src;
   park(kBpermute, EMU_SITE);
+  return (int)me->result;
+}
+__attribute__((noinline)) int shuffle(int v, int src_lane) {
+  Lane* me = g_cur;
+  me->a[0] = v, me->a[1] = src_lane;
+  park(kShuffle, EMU_SITE);
   return (int)me->result;
 }
 __attribute__((noinline)) int readlane(int v, int l) {
@@ -272,9 +283,9 @@ static int dpp_source(int l, int ctrl) {  // source lane of lane l, or -1 when t
   abort();
 }
 
-static void serve(Lane* w, int nl, int op, const void* site) {
+static void serve(Lane* w, int nl, int op, const void* site, long depth) {
   bool in[kWave];
-  for (int l = 0; l < kWave; l++) in[l] = l < nl && w[l].op == op && w[l].site == site;
+  for (int l = 0; l < kWave; l++) in[l] = l < nl && w[l].op == op && w[l].site == site && w[l].depth == depth;
   switch (op) {
     case kDpp:
       for (int l = 0; l < kWave; l++) {
@@ -300,6 +311,13 @@ static void serve(Lane* w, int nl, int op, const void* site) {
         // v_readlane reads the register of the lane whatever EXEC says; a lane that is not parked
         // here has no value to give, which the emulator reports as 0
         w[l].result = in[s] ? (uint32_t)w[s].a[0] : 0u;
+      }
+      break;
+    case kShuffle:
+      for (int l = 0; l < kWave; l++) {
+        if (!in[l]) continue;
+        const int s = w[l].a[1] & 63;
+        w[l].result = (uint32_t)(in[s] ? w[s].a[0] : w[l].a[0]);
       }
       break;
     case kReadfirst: {
@@ -397,6 +415,7 @@ static void run_workgroup(dim3 grid, dim3 block, unsigned bx, unsigned by, unsig
     *--top = reinterpret_cast<uint64_t>(&emu_lane_main);
     for (int i = 0; i < 6; i++) *--top = 0;
     l.sp = top;
+    l.stack_top = g_stacks + (size_t)(t + 1) * kStackBytes;
   }
   for (;;) {
     bool all_done = true;
@@ -422,15 +441,16 @@ static void run_workgroup(dim3 grid, dim3 block, unsigned bx, unsigned by, unsig
         if (best < 0) break;  // the wavefront waits at the workgroup barrier, or has returned
         const int op = w[best].op;
         const void* site = w[best].site;
+        const long depth = w[best].depth;
         if (op == kSleep) {
           for (int l = 0; l < nl; l++)
-            if (w[l].op == kSleep && w[l].site == site) w[l].slept = true;
+            if (w[l].op == kSleep && w[l].site == site && w[l].depth == depth) w[l].slept = true;
           break;  // the other wavefronts get their turn first
         }
         if (is_cross_lane(op))
           for (int l = 0; l < nl; l++)
-            if (is_cross_lane(w[l].op) && w[l].site != site) { g_divergent_cross_lane++; break; }
-        serve(w, nl, op, site);
+            if (is_cross_lane(w[l].op) && (w[l].site != site || w[l].depth != depth)) { g_divergent_cross_lane++; break; }
+        serve(w, nl, op, site, depth);
       }
       for (int l = 0; l < nl; l++) all_done &= w[l].op == kDone;
     }

@@ -22,7 +22,10 @@
 #include <string.h>
 
 #include <algorithm>
+#include <cmath>
+#include <tuple>
 #include <type_traits>
+#include <utility>
 
 #define __global__
 #define __device__
@@ -31,6 +34,8 @@
 #define __launch_bounds__(...)
 #define __forceinline__ inline __attribute__((always_inline))
 #define __align__(n) __attribute__((aligned(n)))
+// the occupancy attribute of a kernel means nothing on the host (attribute names are macro-expanded)
+#define amdgpu_waves_per_eu(...) unused
 
 // ---- the error codes and handle types the sources name ----
 typedef int hipError_t;
@@ -60,29 +65,42 @@ struct LaneView {  // what the running lane reads through threadIdx & co.
 };
 LaneView& view();
 
-// rendezvous operations of a wavefront; each blocks the calling lane until the wavefront's lanes
-// that execute the same operation have arrived, and returns the lane's result
-int dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl);
-int bpermute(int byte_address, int src);
-int readlane(int v, int lane);
-int readfirstlane(int v);
-uint64_t ballot(bool pred);
-void wave_barrier();
-void workgroup_barrier();
-void sleep();  // s_sleep: the wavefront steps aside until the others have had a turn
+// Rendezvous operations of a wavefront; each blocks the calling lane until the wavefront's lanes
+// that execute the same operation have arrived, and returns the lane's result.  The emulator tells
+// "the same operation" by the call's return address, so the compiler must keep ONE call per call in
+// the source (noduplicate: no tail duplication, no unrolling across a call) and must not move a
+// call into or out of a branch (convergent) — what a GPU compiler guarantees for these operations.
+#define EMU_COLLECTIVE __attribute__((convergent, noduplicate))
+EMU_COLLECTIVE int dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl);
+EMU_COLLECTIVE int bpermute(int byte_address, int src);
+EMU_COLLECTIVE int readlane(int v, int lane);
+EMU_COLLECTIVE int readfirstlane(int v);
+EMU_COLLECTIVE uint64_t ballot(bool pred);
+EMU_COLLECTIVE void wave_barrier();
+EMU_COLLECTIVE void workgroup_barrier();
+EMU_COLLECTIVE void sleep();  // s_sleep: the wavefront steps aside until the others have had a turn
 // atomics: all lanes of the wavefront that execute the instruction, served in lane order
-uint32_t atomic_add_u32(uint32_t* p, uint32_t v);
-uint64_t atomic_add_u64(uint64_t* p, uint64_t v);
-uint32_t atomic_or_u32(uint32_t* p, uint32_t v);
-uint64_t lockstep_load(const void* p, int bytes);
-void lockstep_store(void* p, uint64_t v, int bytes);
+EMU_COLLECTIVE uint32_t atomic_add_u32(uint32_t* p, uint32_t v);
+EMU_COLLECTIVE uint64_t atomic_add_u64(uint64_t* p, uint64_t v);
+EMU_COLLECTIVE uint32_t atomic_or_u32(uint32_t* p, uint32_t v);
+EMU_COLLECTIVE uint64_t lockstep_load(const void* p, int bytes);
+EMU_COLLECTIVE void lockstep_store(void* p, uint64_t v, int bytes);
+EMU_COLLECTIVE int shuffle(int v, int src_lane);  // value of src_lane, own value when that lane does not take part
 int lane();  // 0..63
 uint64_t clock();
 
 void launch(dim3 grid, dim3 block, void (*trampoline)(void*), void* closure);
-template <class F>
-inline void launch_closure(dim3 grid, dim3 block, const F& f) {
-  launch(grid, block, [](void* c) { (*static_cast<const F*>(c))(); }, const_cast<F*>(&f));
+// the launch arguments are evaluated once, here; every lane calls the kernel with copies of them
+template <class F, class... Args>
+inline void launch_with_args(dim3 grid, dim3 block, F call, Args&&... args) {
+  struct Closure {
+    F call;
+    std::tuple<typename std::decay<Args>::type...> args;
+  } c{call, std::tuple<typename std::decay<Args>::type...>(std::forward<Args>(args)...)};
+  launch(grid, block, [](void* p) {
+    Closure* cl = static_cast<Closure*>(p);
+    std::apply(cl->call, cl->args);
+  }, &c);
 }
 }  // namespace emu
 
@@ -93,13 +111,14 @@ inline void launch_closure(dim3 grid, dim3 block, const F& f) {
 
 // ---- launches: synchronous, one workgroup after the other ----
 #define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) \
-  ::emu::launch_closure(dim3(grid), dim3(block), [=]() { kernel(__VA_ARGS__); })
+  ::emu::launch_with_args(dim3(grid), dim3(block), [=](auto&... a) { kernel(a...); }, __VA_ARGS__)
 
 // ---- the host API the sources call ----
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
 inline hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus* s) { *s = hipStreamCaptureStatusNone; return hipSuccess; }
 inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
 inline hipError_t hipMemcpyAsync(void* dst, const void* src, size_t n, hipMemcpyKind, hipStream_t) { memcpy(dst, src, n); return hipSuccess; }
 #define HIP_SYMBOL(x) (&(x))
 template <class T> inline hipError_t hipGetSymbolAddress(void** p, T* sym) { *p = (void*)sym; return hipSuccess; }
@@ -107,10 +126,12 @@ template <class T> inline hipError_t hipMemcpyFromSymbol(void* dst, T* sym, size
 // device memory is host memory; events complete at once
 enum { hipDeviceAttributeMultiprocessorCount = 63, hipEventDisableTiming = 2, hipHostMallocDefault = 0, hipMemAttachGlobal = 1 };
 enum : int { hipErrorNotReady = 600 };
-inline hipError_t hipDeviceGetAttribute(int* v, int, int) { *v = 256; return hipSuccess; }
+// a small device: launches sized by the compute-unit count (self-checks, probes) stay cheap
+inline hipError_t hipDeviceGetAttribute(int* v, int, int) { *v = 8; return hipSuccess; }
 enum { hipHostMallocPortable = 1, hipStreamNonBlocking = 1 };
 inline const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "no error" : "error (emulated runtime)"; }
 inline hipError_t hipStreamCreateWithFlags(hipStream_t* s, unsigned) { *s = malloc(1); return hipSuccess; }
+inline hipError_t hipStreamCreate(hipStream_t* s) { *s = malloc(1); return hipSuccess; }
 inline hipError_t hipStreamDestroy(hipStream_t s) { free(s); return hipSuccess; }
 inline hipError_t hipStreamQuery(hipStream_t) { return hipSuccess; }
 struct emu_event {};
@@ -159,6 +180,33 @@ inline unsigned long long emu_fetch_add(unsigned long long* p, unsigned long lon
 inline uint32_t atomicAdd(uint32_t* p, uint32_t v) { return ::emu::atomic_add_u32(p, v); }
 inline unsigned long long atomicAdd(unsigned long long* p, unsigned long long v) { return ::emu::atomic_add_u64((uint64_t*)p, v); }
 inline uint32_t atomicOr(uint32_t* p, uint32_t v) { return ::emu::atomic_or_u32(p, v); }
+
+// ---- wavefront shuffles of the HIP headers (width is a power of two up to 64) ----
+template <class T>
+inline T emu_shuffle_any(T v, int src) {
+  static_assert(sizeof(T) % 4 == 0 && sizeof(T) <= 16, "whole dwords");
+  int w[sizeof(T) / 4];
+  memcpy(w, &v, sizeof(T));
+  for (unsigned i = 0; i < sizeof(T) / 4; i++) w[i] = ::emu::shuffle(w[i], src);
+  memcpy(&v, w, sizeof(T));
+  return v;
+}
+template <class T> inline T __shfl(T v, int src, int width = 64) {
+  const int l = ::emu::lane();
+  return emu_shuffle_any(v, (l & ~(width - 1)) | (src & (width - 1)));
+}
+template <class T> inline T __shfl_up(T v, unsigned delta, int width = 64) {
+  const int l = ::emu::lane(), s = l - (int)delta;
+  return emu_shuffle_any(v, s < (l & ~(width - 1)) ? l : s);
+}
+template <class T> inline T __shfl_down(T v, unsigned delta, int width = 64) {
+  const int l = ::emu::lane(), s = l + (int)delta;
+  return emu_shuffle_any(v, s >= (l & ~(width - 1)) + width ? l : s);
+}
+template <class T> inline T __shfl_xor(T v, int mask, int width = 64) {
+  const int l = ::emu::lane(), s = l ^ mask;
+  return emu_shuffle_any(v, s >= (l & ~(width - 1)) + width ? l : s);
+}
 
 // ---- gfx950 builtins ----
 #define __popcll(x) __builtin_popcountll(x)

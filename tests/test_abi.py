@@ -82,7 +82,15 @@ def test_scan_static_refuses_sizes_beyond_its_array_before_it_touches_a_device()
                         (capi.I64, 1 << 28), (capi.F64, 1 << 28)]:
         assert L.thrust_cdna4_scan_static(code, capi.PLUS, 0, None, None, limit + 1, None, None) == 2
         assert L.thrust_cdna4_scan_static(code, capi.PLUS, 0, None, None, limit, None, None) == 1  # NULL ranges
+    # minimum over 8-byte floating-point values publishes three words per tile (the fold restarts at
+    # NaNs, which a tile has to say): the array holds descriptors for 10922 tiles of 16384 elements
+    limit = 10922 * 16384
+    assert L.thrust_cdna4_scan_static(capi.F64, capi.MINIMUM, 0, None, None, limit + 1, None, None) == 2
+    assert L.thrust_cdna4_scan_static(capi.F64, capi.MINIMUM, 0, None, None, limit, None, None) == 1
+    assert L.thrust_cdna4_scan_static(capi.F32, capi.MINIMUM, 0, None, None, (1 << 29) + 1, None, None) == 2
+    assert L.thrust_cdna4_scan_static(capi.F32, capi.MINIMUM, 0, None, None, 1 << 29, None, None) == 1
     assert L.thrust_cdna4_scan_static(99, capi.PLUS, 0, None, None, 5, None, None) == 1
+    assert L.thrust_cdna4_scan_static(capi.I32, 99, 0, None, None, 5, None, None) == 1
     assert L.thrust_cdna4_scan_static(capi.I32, capi.PLUS, 0, None, None, -1, None, None) == 1
 
 

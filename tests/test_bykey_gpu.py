@@ -266,12 +266,14 @@ def test_by_key_mixed_run_lengths_match_oracle(kd, vd):
                          oracle.scan_by_key(k, v, exclusive=True, init=3)), n
 
 
+@pytest.mark.parametrize("op", ["maximum", "minimum"])
 @pytest.mark.parametrize("vd", [np.float32, np.float64])
-def test_float_maximum_by_key_with_nans_is_the_serial_fold(vd):
+def test_float_extrema_by_key_with_nans_are_the_serial_fold(vd, op):
     """thrust::maximum is a < b ? b : a: in the serial folds (thrust/system/detail/sequential/
     scan_by_key.h:46-142, reduce_by_key.h:43-95) a NaN at the head of a segment stays for the whole
     segment, a NaN inside one is skipped, and the exclusive form — whose folds start from `init` —
-    skips every NaN unless `init` is one.  Same bits from the kernels, over several tiles."""
+    skips every NaN unless `init` is one.  thrust::minimum is a < b ? a : b: its folds restart at
+    every NaN.  Same bits from the kernels, over several tiles, +0 / -0 ties and NaN payloads included."""
     rng = np.random.default_rng(21)
     for n in (1, 2, 9, 2049, 16385, 50021, 200003):
         for mean in (1, 3, 300):
@@ -281,27 +283,35 @@ def test_float_maximum_by_key_with_nans_is_the_serial_fold(vd):
             for where in ("none", "heads", "inside", "both", "all"):
                 v = rng.uniform(-5, 5, n).astype(vd)
                 v[rng.random(n) < 0.05] = vd(-np.inf)
+                v[rng.random(n) < 0.05] = vd(np.inf)
+                v[rng.random(n) < 0.04] = vd(0.0)
+                v[rng.random(n) < 0.04] = vd(-0.0)
                 if where in ("heads", "both"):
                     v[head & (rng.random(n) < 0.5)] = np.nan
                 if where in ("inside", "both"):
                     v[~head & (rng.random(n) < 0.3)] = np.nan
                 if where == "all":
                     v[:] = np.nan
+                nan = np.isnan(v)
+                u = v.view(np.uint32 if vd == np.float32 else np.uint64)
+                u[nan] ^= (rng.integers(0, 1 << 20, int(nan.sum())).astype(u.dtype)
+                           | (rng.integers(0, 2, int(nan.sum())).astype(u.dtype) << u.dtype.type(u.dtype.itemsize * 8 - 1)))
                 dk, dv = dev(k), dev(v)
-                assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op="maximum")),
-                                 oracle.scan_by_key(k, v, op="maximum")), (n, mean, where)
+                assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op=op)),
+                                 oracle.scan_by_key(k, v, op=op)), (n, mean, where)
                 for init in (vd(1.5), vd(np.nan)):
-                    assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=init, op="maximum")),
-                                     oracle.scan_by_key(k, v, op="maximum", exclusive=True, init=init)), (n, mean, where, init)
-                ko, vo = thrust_amd.reduce_by_key(dk, dv, op="maximum")
-                ek, ev = oracle.reduce_by_key(k, v, op="maximum")
+                    assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=init, op=op)),
+                                     oracle.scan_by_key(k, v, op=op, exclusive=True, init=init)), (n, mean, where, init)
+                ko, vo = thrust_amd.reduce_by_key(dk, dv, op=op)
+                ek, ev = oracle.reduce_by_key(k, v, op=op)
                 assert same_bits(host(ko), ek) and same_bits(host(vo), ev), (n, mean, where)
                 y = dev(v)
-                thrust_amd.inclusive_scan_by_key(dk, y, out=y, op="maximum")  # in place: tiles by ticket
-                assert same_bits(host(y), oracle.scan_by_key(k, v, op="maximum")), (n, mean, where, "in place")
+                thrust_amd.inclusive_scan_by_key(dk, y, out=y, op=op)  # in place: tiles by ticket
+                assert same_bits(host(y), oracle.scan_by_key(k, v, op=op)), (n, mean, where, "in place")
 
 
-def test_float_maximum_by_key_with_nans_on_the_recompute_path(no_patience, tile0_publishes_late):
+@pytest.mark.parametrize("op", ["maximum", "minimum"])
+def test_float_extrema_by_key_with_nans_on_the_recompute_path(no_patience, tile0_publishes_late, op):
     rng = np.random.default_rng(22)
     n = 16384 * 3 + 5
     for mean in (1, 40):
@@ -309,9 +319,35 @@ def test_float_maximum_by_key_with_nans_on_the_recompute_path(no_patience, tile0
         v = rng.uniform(-5, 5, n).astype(np.float32)
         v[rng.random(n) < 0.3] = np.nan
         dk, dv = dev(k), dev(v)
-        assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op="maximum")), oracle.scan_by_key(k, v, op="maximum")), mean
-        assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=np.float32(0.25), op="maximum")),
-                         oracle.scan_by_key(k, v, op="maximum", exclusive=True, init=np.float32(0.25))), mean
-        ko, vo = thrust_amd.reduce_by_key(dk, dv, op="maximum")
-        ek, ev = oracle.reduce_by_key(k, v, op="maximum")
+        assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op=op)), oracle.scan_by_key(k, v, op=op)), mean
+        assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=np.float32(0.25), op=op)),
+                         oracle.scan_by_key(k, v, op=op, exclusive=True, init=np.float32(0.25))), mean
+        ko, vo = thrust_amd.reduce_by_key(dk, dv, op=op)
+        ek, ev = oracle.reduce_by_key(k, v, op=op)
         assert same_bits(host(ko), ek) and same_bits(host(vo), ev), mean
+
+
+@pytest.mark.parametrize("op", ["maximum", "minimum"])
+@pytest.mark.parametrize("vd", [np.float32, np.float64])
+def test_float_extrema_by_key_keep_the_zero_the_serial_fold_keeps(vd, op):
+    """Values that are mostly +0 and -0: the SIGN of a result tells which operand the fold kept
+    (maximum the first of equals, minimum the last).  Long runs, so that the value of a run crosses
+    threads, wavefronts and tiles before it meets its last element."""
+    rng = np.random.default_rng(41)
+    for n in (9, 2049, 50021, 200003):
+        for mean in (3, 300, 40000):
+            k = runs(n + mean, n, mean)
+            v = np.where(rng.random(n) < 0.5, vd(0.0), vd(-0.0)).astype(vd)
+            losers = rng.random(n) < 0.3
+            v[losers] = (-1 if op == "maximum" else 1) * rng.uniform(1, 5, int(losers.sum())).astype(vd)
+            dk, dv = dev(k), dev(v)
+            assert same_bits(host(thrust_amd.inclusive_scan_by_key(dk, dv, op=op)), oracle.scan_by_key(k, v, op=op)), (n, mean)
+            for init in (vd(0.0), vd(-0.0), vd(-7.0), vd(7.0)):
+                assert same_bits(host(thrust_amd.exclusive_scan_by_key(dk, dv, init=init, op=op)),
+                                 oracle.scan_by_key(k, v, op=op, exclusive=True, init=init)), (n, mean, init)
+            ko, vo = thrust_amd.reduce_by_key(dk, dv, op=op)
+            ek, ev = oracle.reduce_by_key(k, v, op=op)
+            assert same_bits(host(ko), ek) and same_bits(host(vo), ev), (n, mean)
+            y = dev(v)
+            thrust_amd.exclusive_scan_by_key(dk, y, out=y, init=vd(-0.0), op=op)  # in place: tiles by ticket
+            assert same_bits(host(y), oracle.scan_by_key(k, v, op=op, exclusive=True, init=vd(-0.0))), (n, mean, "in place")

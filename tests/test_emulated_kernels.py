@@ -37,6 +37,20 @@ SLOW = [
 ]
 
 
+# C++ API tests (tests/cpp) that the default run leaves out: minutes of emulation each, or inputs of
+# 2^30 items and more that only a device gets through (the latter are left out in every mode)
+CPP_NEVER = ["BigIndexes"]
+CPP_SLOW = ["TestStableSortRepeatable", "TestCopyIfLarge", "TestVectorSearch", "TestFindMismatchLadder", "TestShuffle",
+            "TestStablePartitionLarge", "TestStableSortByKey<", "TestAsyncSort",
+            # of a typed test the default run keeps the int / int32_t instance
+            "<int8_t>", "<uint8_t>", "<int16_t>", "<uint16_t>", "<uint32_t>", "<int64_t>", "<uint64_t>", "<float>",
+            "<double>"]
+CPP_TESTS = ["test_sort", "test_scan", "test_by_key", "test_host_vector", "test_seq", "test_system_dir",
+             "test_dispatch", "test_complex", "test_memory", "test_merge_set", "test_algorithms",
+             "test_scan_generic", "test_merge_sort", "test_generic", "test_select", "test_partition",
+             "test_iterators", "test_async", "test_mr", "test_api_surface", "test_system"]
+
+
 @pytest.fixture(scope="module")
 def emulated_library():
     r = subprocess.run(["make", "-C", EMU_DIR, "-j8"], capture_output=True, text=True)
@@ -61,13 +75,11 @@ def run_session(files, resident="1", deselect=(), extra=()):
     return last[-1]
 
 
-def test_scans_by_key_and_histogram_one_workgroup_at_a_time(emulated_library):
-    print(run_session(["tests/test_scan_gpu.py", "tests/test_bykey_gpu.py", "tests/test_histogram_gpu.py",
-                       "tests/test_zz_no_alloc.py"], deselect=SLOW))
-
-
-def test_sorts_one_workgroup_at_a_time(emulated_library):
-    print(run_session(["tests/test_sort_gpu.py", "tests/test_random_gpu.py"], deselect=SLOW))
+def test_sorts_histogram_and_the_no_allocation_scan_one_workgroup_at_a_time(emulated_library):
+    files = ["tests/test_sort_gpu.py", "tests/test_random_gpu.py", "tests/test_histogram_gpu.py", "tests/test_zz_no_alloc.py"]
+    if ALL:  # the default run has scans and by-key in the session below only
+        files += ["tests/test_scan_gpu.py", "tests/test_bykey_gpu.py"]
+    print(run_session(files, deselect=SLOW))
 
 
 @pytest.mark.parametrize("resident", ["6:11", "16:5", "3:77"] if ALL else ["6:11"])
@@ -76,3 +88,24 @@ def test_look_back_with_several_workgroups_in_flight(emulated_library, resident)
     look-back is made to give up reports it (the status word, the error, the latch to plain tickets)."""
     print(run_session(["tests/test_scan_gpu.py", "tests/test_bykey_gpu.py", "tests/test_random_gpu.py",
                        "tests/test_sort_timeout_gpu.py"], resident=resident, deselect=SLOW))
+
+
+def test_cpp_api_tests_on_the_emulated_library(emulated_library):
+    """The header layer's own kernels (user operators, merge sort, select and partition, merge and
+    set operations, thrust::seq inside kernels) through the C++ API tests of tests/cpp, built for
+    the host by tests/emu/Makefile."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    env = dict(os.environ, THRUST_CDNA4_TEST_SKIP=",".join(CPP_NEVER + ([] if ALL else CPP_SLOW)))
+
+    def run(name):
+        r = subprocess.run([os.path.join(EMU_DIR, "build", "cpp", name)], env=env, capture_output=True, text=True,
+                           timeout=1800)
+        return name, r.returncode, r.stdout[-3000:] + r.stderr[-1000:]
+
+    with ThreadPoolExecutor(int(WORKERS)) as pool:
+        results = list(pool.map(run, CPP_TESTS))
+    failed = [(name, out) for name, rc, out in results if rc != 0 or "0 failed" not in out]
+    assert not failed, failed
+    ran = sum(int(out.strip().splitlines()[-1].split()[0]) for _, _, out in results)
+    assert ran > (380 if ALL else 200), ran

@@ -192,6 +192,9 @@ def test_scan_in_place_takes_the_ticket_path_and_out_of_place_does_not():
 def _with_nans(rng, n, where, dt):
     x = rng.uniform(-5, 5, n).astype(dt)
     x[rng.random(n) < 0.05] = dt(-np.inf)
+    x[rng.random(n) < 0.05] = dt(np.inf)
+    x[rng.random(n) < 0.04] = dt(0.0)   # ties between +0 and -0 show which operand a fold keeps
+    x[rng.random(n) < 0.04] = dt(-0.0)
     if where == "first":
         x[0] = np.nan
     elif where == "middle" and n > 2:
@@ -205,29 +208,38 @@ def _with_nans(rng, n, where, dt):
         x[0] = np.nan
     elif where == "all":
         x[:] = np.nan
+    # NaNs of both signs and with different payloads: the fold must hand on the very NaN it met
+    nan = np.isnan(x)
+    u = x.view(np.uint32 if dt == np.float32 else np.uint64)
+    width = u.dtype.itemsize * 8
+    u[nan] ^= (rng.integers(0, 1 << 20, int(nan.sum())).astype(u.dtype)
+               | (rng.integers(0, 2, int(nan.sum())).astype(u.dtype) << u.dtype.type(width - 1)))
     return x
 
 
+@pytest.mark.parametrize("op", ["maximum", "minimum"])
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
-def test_float_maximum_scans_with_nans_are_the_serial_fold(dt):
+def test_float_extrema_scans_with_nans_are_the_serial_fold(dt, op):
     """thrust::maximum is a < b ? b : a: the serial fold (thrust/system/detail/sequential/scan.h:54-72)
-    keeps a NaN that starts it and skips NaNs met later.  The kernel must give the same bits whatever
-    its grouping: NaN first, in the middle, scattered, everywhere; a NaN `init`; several tiles; in place."""
+    keeps a NaN that starts it and skips NaNs met later.  thrust::minimum is a < b ? a : b: the fold
+    restarts at every NaN (the NaN replaces the accumulator, the next element replaces the NaN).  The
+    kernel must give the same bits whatever its grouping: NaN first, in the middle, scattered,
+    everywhere; a NaN `init`; several tiles; in place."""
     rng = np.random.default_rng(11)
     for n in (1, 2, 5, 4097, 70001, 300007):
         for where in ("none", "first", "middle", "many", "many_and_first", "all"):
             x = _with_nans(rng, n, where, dt)
             d = dev(x)
-            assert same_bits(host(thrust_amd.inclusive_scan(d, op="maximum")), oracle.scan(x, op="maximum")), (n, where)
+            assert same_bits(host(thrust_amd.inclusive_scan(d, op=op)), oracle.scan(x, op=op)), (n, where)
             for init in (dt(0.5), dt(np.nan), dt(-np.inf)):
-                assert same_bits(host(thrust_amd.exclusive_scan(d, init=init, op="maximum")),
-                                 oracle.scan(x, op="maximum", exclusive=True, init=init)), (n, where, init)
+                assert same_bits(host(thrust_amd.exclusive_scan(d, init=init, op=op)),
+                                 oracle.scan(x, op=op, exclusive=True, init=init)), (n, where, init)
             y = dev(x)
-            thrust_amd.inclusive_scan(y, out=y, op="maximum")  # in place: tiles by ticket
-            assert same_bits(host(y), oracle.scan(x, op="maximum")), (n, where, "in place")
+            thrust_amd.inclusive_scan(y, out=y, op=op)  # in place: tiles by ticket
+            assert same_bits(host(y), oracle.scan(x, op=op)), (n, where, "in place")
             y = dev(x)
-            thrust_amd.exclusive_scan(y, out=y, init=dt(np.nan), op="maximum")
-            assert same_bits(host(y), oracle.scan(x, op="maximum", exclusive=True, init=dt(np.nan))), (n, where, "in place, NaN init")
+            thrust_amd.exclusive_scan(y, out=y, init=dt(np.nan), op=op)
+            assert same_bits(host(y), oracle.scan(x, op=op, exclusive=True, init=dt(np.nan))), (n, where, "in place, NaN init")
 
 
 def test_float_maximum_scan_with_nans_on_the_recompute_path(no_patience, tile0_publishes_late):
@@ -239,3 +251,40 @@ def test_float_maximum_scan_with_nans_on_the_recompute_path(no_patience, tile0_p
         assert same_bits(host(thrust_amd.inclusive_scan(d, op="maximum")), oracle.scan(x, op="maximum")), where
         assert same_bits(host(thrust_amd.exclusive_scan(d, init=np.float32(2.0), op="maximum")),
                          oracle.scan(x, op="maximum", exclusive=True, init=np.float32(2.0))), where
+
+
+def _zeros_of_both_signs(rng, n, dt, op):
+    """Mostly +0 and -0, the rest on the side that never wins: every result is a zero whose SIGN tells
+    which operand the fold kept (maximum keeps the first of equals, minimum the last)."""
+    x = np.where(rng.random(n) < 0.5, dt(0.0), dt(-0.0)).astype(dt)
+    losers = rng.random(n) < 0.3
+    x[losers] = (-1 if op == "maximum" else 1) * rng.uniform(1, 5, int(losers.sum())).astype(dt)
+    return x
+
+
+@pytest.mark.parametrize("op", ["maximum", "minimum"])
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_float_extrema_scans_keep_the_zero_the_serial_fold_keeps(dt, op):
+    rng = np.random.default_rng(31)
+    for n in (7, 4097, 70001, 300007):
+        x = _zeros_of_both_signs(rng, n, dt, op)
+        d = dev(x)
+        assert same_bits(host(thrust_amd.inclusive_scan(d, op=op)), oracle.scan(x, op=op)), n
+        for init in (dt(0.0), dt(-0.0)):
+            assert same_bits(host(thrust_amd.exclusive_scan(d, init=init, op=op)),
+                             oracle.scan(x, op=op, exclusive=True, init=init)), (n, init)
+        y = dev(x)
+        thrust_amd.exclusive_scan(y, out=y, init=dt(-0.0), op=op)  # in place: tiles by ticket
+        assert same_bits(host(y), oracle.scan(x, op=op, exclusive=True, init=dt(-0.0))), (n, "in place")
+
+
+@pytest.mark.parametrize("op", ["maximum", "minimum"])
+def test_float_extrema_scans_keep_that_zero_on_the_recompute_path(no_patience, tile0_publishes_late, op):
+    rng = np.random.default_rng(32)
+    n = 32768 * 4 + 77
+    for dt in (np.float32, np.float64):
+        x = _zeros_of_both_signs(rng, n, dt, op)
+        d = dev(x)
+        assert same_bits(host(thrust_amd.inclusive_scan(d, op=op)), oracle.scan(x, op=op)), dt
+        assert same_bits(host(thrust_amd.exclusive_scan(d, init=dt(-0.0), op=op)),
+                         oracle.scan(x, op=op, exclusive=True, init=dt(-0.0))), dt

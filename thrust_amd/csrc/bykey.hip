@@ -27,10 +27,28 @@ template <> struct key_bits<4> { using type = uint32_t; };
 template <> struct key_bits<8> { using type = uint64_t; };
 using KU = key_bits<TCD_KEY_BYTES>::type;
 
-template <class T>
+template <class T, bool RESTARTS = false>
 struct SegPair {
   uint32_t c;  // heads seen
   T v;         // value of the open segment
+};
+// minimum(a, b) = a < b ? a : b over floating-point values with NaNs: the serial fold RESTARTS at
+// every NaN (acc < NaN is false, so the NaN replaces the accumulator; NaN < x is false too, so the
+// next element replaces the NaN).  The raw operator does that by itself wherever values are folded
+// in input order; where PIECES are combined, a piece must also say whether it holds a NaN after its
+// last head — nothing to its left survives that NaN, just as nothing survives a head.  And the
+// empty piece needs a state of its own, because the operator's identity is none for a NaN
+// (minimum(NaN, +inf) is +inf) and accumulators are shown as they are (the value of a run that
+// ends with a NaN; exclusive scans).  Only the floating-point minimum instantiations carry this.
+template <class T>
+struct SegPair<T, true> {
+  uint32_t c;  // heads seen
+  uint32_t r;  // after the last head (or in all of a piece without one) — 0: no NaN, 1: a NaN; 2: the piece is empty
+  T v;         // value of the open segment
+};
+template <class T, class Op>
+struct seg_restarts {
+  static constexpr bool value = std::is_floating_point<T>::value && std::is_same<Op, OpMinimum>::value;
 };
 
 template <class T, class Op>
@@ -39,6 +57,37 @@ __device__ inline SegPair<T> seg_combine(const SegPair<T>& a, const SegPair<T>& 
   r.c = a.c + b.c;
   r.v = b.c ? b.v : Op::template apply<T>(a.v, b.v);
   return r;
+}
+template <class T, class Op>
+__device__ inline SegPair<T, true> seg_combine(const SegPair<T, true>& a, const SegPair<T, true>& b) {
+  if (b.r == 2u) return a;
+  if (a.r == 2u) return b;
+  SegPair<T, true> r;
+  r.c = a.c + b.c;
+  r.r = b.c ? b.r : (a.r | b.r);
+  r.v = (b.c || b.r) ? b.v : Op::template apply<T>(a.v, b.v);
+  return r;
+}
+// one more element at the end of a piece
+template <class T, class Op>
+__device__ inline void seg_append(SegPair<T>& a, bool is_head, T x) {
+  a.c += is_head ? 1u : 0u;
+  a.v = is_head ? x : Op::template apply<T>(a.v, x);
+}
+template <class T, class Op>
+__device__ inline void seg_append(SegPair<T, true>& a, bool is_head, T x) {
+  const bool fresh = is_head || a.r == 2u;
+  a.c += is_head ? 1u : 0u;
+  a.v = fresh ? x : Op::template apply<T>(a.v, x);
+  a.r = (fresh ? 0u : a.r) | (__builtin_isnan(x) ? 1u : 0u);
+}
+template <class P, class T>
+__device__ inline P seg_empty(T id) {
+  P p;
+  p.c = 0u;
+  p.v = id;
+  if constexpr (!std::is_same<P, SegPair<T>>::value) p.r = 2u;
+  return p;
 }
 
 template <class KU>
@@ -188,7 +237,8 @@ __device__ inline void wave_store_blocked_partial(E* dst, const E (&src)[VEC], t
 // elements once more from `off`; nothing per element is kept in between.
 template <class T, class Op, class G>
 struct SegTile {
-  using Pair = SegPair<T>;
+  static constexpr bool kRestarts = seg_restarts<T, Op>::value;
+  using Pair = SegPair<T, kRestarts>;
   static constexpr int VEC = G::VEC, NWAVES = G::NWAVES, BLOCK = G::BLOCK;
   static_assert(NWAVES <= kWave, "one wavefront scans the wavefronts' totals");
 
@@ -231,7 +281,7 @@ struct SegTile {
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const T id = Op::template identity<T>();
-    const Pair idp{0u, id};
+    const Pair idp = seg_empty<Pair>(id);
 
     tile = blockIdx.x;
     if constexpr (TICKET) {
@@ -286,10 +336,11 @@ struct SegTile {
           if ((folds_start_from_init || !is_head) && __builtin_isnan(val[j])) val[j] = id;
         }
         h |= (is_head ? 1u : 0u) << j;
-        agg.v = is_head ? val[j] : Op::template apply<T>(agg.v, val[j]);
+        if constexpr (kRestarts) seg_append<T, Op>(agg, is_head, val[j]);
+        else agg.v = is_head ? val[j] : Op::template apply<T>(agg.v, val[j]);
       }
       heads = h;
-      agg.c = __builtin_popcount(h);
+      if constexpr (!kRestarts) agg.c = __builtin_popcount(h);
       const Pair w = wave_inclusive_scan(agg, idp, comb);
       excl_w = wave_shift_up1(w, idp);
       if (lane == kWave - 1) sm.tot[wave] = w;
@@ -330,8 +381,7 @@ struct SegTile {
               if constexpr (kNanAware) {
                 if ((folds_start_from_init || !is_head) && __builtin_isnan(vv)) vv = Op::template identity<T>();
               }
-              a.c += is_head ? 1u : 0u;
-              a.v = is_head ? vv : Op::template apply<T>(a.v, vv);
+              seg_append<T, Op>(a, is_head, vv);
               before = kk;
             }
             return readlane(wave_inclusive_scan(a, idp, comb), kWave - 1);
@@ -372,15 +422,22 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void scan_by_key_ke
   bool parked = false;
   uint32_t first_head = 0;
   t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, exclusive != 0, [&] {
-    if (!t.full) return;
+    // (a restarting fold is not commutative: its tiles all take the walk from the tile's prefix below)
+    if (!t.full || ST::kRestarts) return;
     parked = true;
     T r[VEC];
     T open = t.excl_w.v;
+    // Floating-point maximum keeps the FIRST of +0 and -0: an exclusive result before the
+    // wavefront's first head is init (+) run so far (+) wavefront's fold, in that order, so `init`
+    // is left out of what is parked there and goes in front during the copy-out.
+    bool none_below = false;  // no head in the lanes below
+    if constexpr (ST::kNanAware) none_below = exclusive && !(__ballot(t.heads != 0u) & ((1ull << lane) - 1ull));
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
       const bool is_head = (t.heads >> j) & 1u;
       const T x = t.val[j];
-      if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
+      const bool before_first_head = ST::kNanAware && none_below && !(t.heads & ((2u << j) - 1u));
+      if (exclusive) r[j] = is_head ? init : before_first_head ? open : Op::template apply<T>(init, open);
       open = is_head ? x : Op::template apply<T>(open, x);
       if (!exclusive) r[j] = open;
     }
@@ -410,9 +467,15 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void scan_by_key_ke
         for (int e = 0; e < EPP; e++)
           if ((uint32_t)((q * kWave + lane) * EPP + e) < first_head) {
             // the run's value so far goes in front of what the wavefront folded; the exclusive
-            // form has `init` in front of both, inside x[e] (the operands commute unless one
-            // is a NaN, which — see kNanAware — can only be the first in fold order)
-            x[e] = exclusive ? Op::template apply<T>(x[e], carried) : Op::template apply<T>(carried, x[e]);
+            // form has `init` in front of both: already inside x[e] where the operands commute,
+            // applied here in fold order where they do not (floating-point maximum: a NaN, or
+            // +0 against -0)
+            if constexpr (ST::kNanAware) {
+              x[e] = Op::template apply<T>(carried, x[e]);
+              if (exclusive) x[e] = Op::template apply<T>(init, x[e]);
+            } else {
+              x[e] = exclusive ? Op::template apply<T>(x[e], carried) : Op::template apply<T>(carried, x[e]);
+            }
           }
         __builtin_memcpy(&piece, x, 16);
       }
@@ -423,13 +486,28 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void scan_by_key_ke
   // the last tile, and every tile of a call whose pointers are not aligned to their elements
   T r[VEC];
   T open = t.off.v;  // value of the open segment just before the element
+  if constexpr (ST::kRestarts) {
+    // the raw fold restarts at NaNs by itself; `init` of an exclusive scan is in front of the
+    // fold only until the segment's first NaN
+    bool restarted = t.off.r == 1u;
 #pragma unroll
-  for (int j = 0; j < VEC; j++) {
-    const bool is_head = (t.heads >> j) & 1u;
-    const T x = t.val[j];
-    if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
-    open = is_head ? x : Op::template apply<T>(open, x);
-    if (!exclusive) r[j] = open;
+    for (int j = 0; j < VEC; j++) {
+      const bool is_head = (t.heads >> j) & 1u;
+      const T x = t.val[j];
+      if (exclusive) r[j] = is_head ? init : restarted ? open : Op::template apply<T>(init, open);
+      open = is_head ? x : Op::template apply<T>(open, x);
+      restarted = (!is_head && restarted) || __builtin_isnan(x);
+      if (!exclusive) r[j] = open;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+      const bool is_head = (t.heads >> j) & 1u;
+      const T x = t.val[j];
+      if (exclusive) r[j] = is_head ? init : Op::template apply<T>(init, open);
+      open = is_head ? x : Op::template apply<T>(open, x);
+      if (!exclusive) r[j] = open;
+    }
   }
   if (vec_ok) {
     const int64_t w0 = t.base + (int64_t)wave * (kWave * VEC);
@@ -481,7 +559,7 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void reduce_by_key_
   uint32_t count = 0;
   t.template run<TICKET>(sm, keys, vals, n, float_keys, vec_ok, desc, ticket, xbuf, patience, publish_delay, false, [&] {
     count = (uint32_t)__builtin_amdgcn_readlane((int)(t.excl_w.c + __builtin_popcount(t.heads)), kWave - 1);
-    early = t.full && count <= kEarlyMax;
+    early = t.full && count <= kEarlyMax && !ST::kRestarts;  // (the early form counts on a commutative operator)
     if (!early) {
       if (t.full) {  // the keys alone always fit
         uint32_t slot = t.excl_w.c;
@@ -506,7 +584,7 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void reduce_by_key_
     }
   });
   if (early) {
-    const SegPair<T> before_wave = sm.tot[threadIdx.x / kWave];
+    const typename ST::Pair before_wave = sm.tot[threadIdx.x / kWave];
     const uint32_t first = before_wave.c;
     for (uint32_t i = lane; i < count; i += kWave) {
       keys_out[first + i] = early_k[sw(i)];
@@ -516,7 +594,7 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void reduce_by_key_
     }
     return;
   }
-  SegPair<T> run = t.off;  // (runs started so far, value of the open run) before the current element
+  typename ST::Pair run = t.off;  // (runs started so far, value of the open run) before the current element
   const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)run.c);  // runs before this wavefront
   const uint32_t heads = t.heads;
   const uint32_t mine = run.c - first;  // slot of this thread's first head
@@ -558,10 +636,10 @@ __global__ __launch_bounds__(SegGeom<T>::BLOCK) TCD_SEG_ATTR void reduce_by_key_
     if (first + i) vals_out[first + i - 1] = sv[sw(i)];  // value of the run that ended at this head
 }
 
-template <class T, class G>
+template <class T, class Op, class G>
 static size_t bykey_temp_bytes(int64_t n) {
   const int64_t ntiles = ceil_div(n, G::TILE);
-  return 256 + align_up((size_t)ntiles * TileDesc<SegPair<T>>::kBytesPerTile, 256);
+  return 256 + align_up((size_t)ntiles * TileDesc<SegPair<T, seg_restarts<T, Op>::value>>::kBytesPerTile, 256);
 }
 
 #define TCD_CAT2(a, b) a##b
@@ -582,7 +660,7 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
     using T = decltype(tv);
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
-      const size_t need = bykey_temp_bytes<T, SegGeom<T>>(n);
+      const size_t need = bykey_temp_bytes<T, Op, SegGeom<T>>(n);
       if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
       if (*temp_bytes < need) return;
       if (n == 0) { rc = hipSuccess; return; }
@@ -633,7 +711,7 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
     using T = decltype(tv);
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
-      const size_t need = bykey_temp_bytes<T, SegGeom<T>>(n);
+      const size_t need = bykey_temp_bytes<T, Op, SegGeom<T>>(n);
       if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
       if (*temp_bytes < need) return;
       if (n == 0) {  // no runs: only the count is written

@@ -21,6 +21,44 @@ struct alignas(16) Vec16 {
 // (used when the output overlaps the input).  Otherwise a tile is the workgroup of the same
 // index — no atomic and no barrier before the loads, 6 % faster at 2^28 and 25 % at 2^24 — and a
 // descriptor that stays missing is recomputed from the input after `patience` polls.
+// minimum(a, b) = a < b ? a : b over floating-point values with NaNs: the serial fold RESTARTS at
+// every NaN (acc < NaN is false, so the NaN replaces the accumulator; NaN < x is false too, so the
+// next element replaces the NaN).  What a piece of the input contributes to a fold is then a pair:
+// the raw fold of the piece, and whether the piece holds a NaN — in which case nothing to its left
+// survives it.  Pairs combine associatively, so they travel through the wavefront scans and the
+// tile descriptors in place of the plain value.  Only the floating-point minimum instantiations
+// carry them.
+template <class T, class Op>
+struct scan_restarts {
+  static constexpr bool value = std::is_floating_point<T>::value && std::is_same<Op, OpMinimum>::value;
+};
+template <class T>
+struct RestartPair {
+  uint32_t a[sizeof(T) / 4];  // the value's words (keeps an 8-byte value from padding the pair to 16 bytes)
+  uint32_t r;                 // 0: the piece holds no NaN, 1: it does, 2: the piece is empty
+  __device__ T value() const { T v; __builtin_memcpy(&v, a, sizeof(T)); return v; }
+  __device__ static RestartPair make(T v, uint32_t r) {
+    RestartPair p;
+    __builtin_memcpy(p.a, &v, sizeof(T));
+    p.r = r;
+    return p;
+  }
+  // The empty piece has a state of its own because the operator's identity is none for a NaN:
+  // minimum(NaN, +inf) is +inf, and an exclusive scan shows the accumulator itself.
+  template <class Op>
+  __device__ static RestartPair combine(const RestartPair& x, const RestartPair& y) {
+    if (y.r == 2u) return x;
+    if (x.r == 2u) return y;
+    return make(y.r ? y.value() : Op::template apply<T>(x.value(), y.value()), x.r | y.r);
+  }
+};
+// what a tile publishes and what travels across lanes: a dword container for 1- and 2-byte T
+template <class T, class Op>
+struct scan_payload {
+  using type = typename std::conditional<scan_restarts<T, Op>::value, RestartPair<T>,
+                                         typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type>::type;
+};
+
 template <class T, class Op, int BLOCK, int CHUNKS, bool TICKET>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void scan_kernel(const T* in, T* out, int64_t n, T init,
                                                      int exclusive, uint64_t* desc,
@@ -28,8 +66,10 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NWAVES = BLOCK / kWave;
   constexpr int64_t TILE = (int64_t)BLOCK * VEC * CHUNKS;
-  // cross-lane traffic, LDS and descriptors carry W (a dword container for 1- and 2-byte T)
-  using W = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
+  // cross-lane traffic, LDS and descriptors carry W
+  using W = typename scan_payload<T, Op>::type;
+  constexpr bool kRestarts = scan_restarts<T, Op>::value;
+  static_assert(!kRestarts || TICKET, "pieces of a restarting fold combine in input order only: no recomputation from strided reads");
 
   __shared__ W s_tot[CHUNKS * NWAVES];  // inclusive total of (chunk, wave), then its exclusive offset
   __shared__ uint32_t s_tile;
@@ -40,14 +80,22 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
   const T id = Op::template identity<T>();
   auto op = [](T a, T b) { return Op::template apply<T>(a, b); };
   auto toW = [](T a) {
-    if constexpr (std::is_same<W, T>::value) return a;
+    if constexpr (kRestarts) return W::make(a, __builtin_isnan(a) ? 1u : 0u);
+    else if constexpr (std::is_same<W, T>::value) return a;
     else return (W)(typename unsigned_of<T>::type)a;
   };
-  auto opW = [&](W a, W b) {
-    if constexpr (std::is_same<W, T>::value) return op(a, b);
+  auto fromW = [](const W& w) {
+    if constexpr (kRestarts) return w.value();
+    else return (T)w;
+  };
+  auto opW = [&](const W& a, const W& b) {
+    if constexpr (kRestarts) return W::template combine<Op>(a, b);
+    else if constexpr (std::is_same<W, T>::value) return op(a, b);
     else return (W)(typename unsigned_of<T>::type)op((T)a, (T)b);
   };
-  const W idW = toW(id);
+  W idW;
+  if constexpr (kRestarts) idW = W::make(id, 2u);
+  else idW = toW(id);
 
   int64_t tile = blockIdx.x;
   if constexpr (TICKET) {
@@ -99,13 +147,31 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
 
   // thread-local inclusive scan of each 16-byte group, then a wave scan of the group sums
   T excl[CHUNKS];
+  uint32_t nan_below = 0;  // kRestarts: bit c: a NaN in the wavefront's groups of chunk c below this thread's
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
+    if constexpr (kRestarts) {
+      // the elements stay as loaded: the results are formed by one more raw fold from the
+      // accumulator before the group, which restarts at NaNs by itself
+      T acc = x[c][0];
+      bool seen = __builtin_isnan(acc);
 #pragma unroll
-    for (int j = 1; j < VEC; j++) x[c][j] = op(x[c][j - 1], x[c][j]);
-    const W incl = wave_inclusive_scan(toW(x[c][VEC - 1]), idW, opW);
-    excl[c] = (T)wave_shift_up1(incl, idW);
-    if (lane == kWave - 1) s_tot[c * NWAVES + wave] = incl;
+      for (int j = 1; j < VEC; j++) {
+        seen = seen || __builtin_isnan(x[c][j]);
+        acc = op(acc, x[c][j]);
+      }
+      const W incl = wave_inclusive_scan(W::make(acc, seen ? 1u : 0u), idW, opW);
+      const W below = wave_shift_up1(incl, idW);  // empty in lane 0
+      excl[c] = below.value();
+      nan_below |= (below.r == 1u ? 1u : 0u) << c;
+      if (lane == kWave - 1) s_tot[c * NWAVES + wave] = incl;
+    } else {
+#pragma unroll
+      for (int j = 1; j < VEC; j++) x[c][j] = op(x[c][j - 1], x[c][j]);
+      const W incl = wave_inclusive_scan(toW(x[c][VEC - 1]), idW, opW);
+      excl[c] = fromW(wave_shift_up1(incl, idW));
+      if (lane == kWave - 1) s_tot[c * NWAVES + wave] = incl;
+    }
   }
   __syncthreads();
 
@@ -137,16 +203,26 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
         prefix = wave_lookback<W>(desc, tile, idW, opW);
       } else {
         // the aggregate of an earlier tile (always a whole one), straight from the input
+        // (a lane folds every 64th element: the operator must commute.  Floating-point maximum
+        // does not where +0 meets -0 — the fold keeps the one that comes first — so there a lane
+        // folds a contiguous piece and the pieces combine in lane order.)
         const auto aggregate_of = [&](int64_t t) -> W {
-          const T* p = in + t * TILE + lane;
+          constexpr int PIECE = (int)(TILE / kWave);
+          constexpr int64_t STRIDE = kNanAware ? 1 : kWave;
+          const T* p = in + t * TILE + (kNanAware ? (int64_t)lane * PIECE : (int64_t)lane);
           const auto element = [&](int k) {
-            const T e = p[(int64_t)k * kWave];
+            const T e = p[(int64_t)k * STRIDE];
             if constexpr (kNanAware) return __builtin_isnan(e) ? id : e;
             else return e;
           };
           T acc = element(0);
+          if constexpr (kNanAware) {
+#pragma unroll 2
+            for (int k = 1; k < PIECE; k++) acc = op(acc, element(k));
+          } else {
 #pragma unroll 8
-          for (int k = 1; k < (int)(TILE / kWave); k++) acc = op(acc, element(k));
+            for (int k = 1; k < PIECE; k++) acc = op(acc, element(k));
+          }
           return readlane(wave_inclusive_scan(toW(acc), idW, opW), kWave - 1);
         };
         prefix = wave_lookback_or_compute<W>(desc, tile, idW, opW, patience, aggregate_of);
@@ -167,14 +243,28 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void
   // results: element (c, j) = offset of its (chunk, wave) (+) lanes before it (+) its group prefix
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
-    const T off = op((T)s_tot[c * NWAVES + wave], excl[c]);
-    if (exclusive) {
+    if constexpr (kRestarts) {
+      // the accumulator before the group: what lies before the wavefront's groups counts unless
+      // those groups hold a NaN
+      const T before_wave = fromW(s_tot[c * NWAVES + wave]);
+      T acc = lane == 0 ? before_wave : ((nan_below >> c) & 1u) ? excl[c] : op(before_wave, excl[c]);
 #pragma unroll
-      for (int j = VEC - 1; j > 0; j--) x[c][j] = op(off, x[c][j - 1]);
-      x[c][0] = off;
+      for (int j = 0; j < VEC; j++) {
+        const T e = x[c][j];
+        if (exclusive) x[c][j] = acc;
+        acc = op(acc, e);
+        if (!exclusive) x[c][j] = acc;
+      }
     } else {
+      const T off = op(fromW(s_tot[c * NWAVES + wave]), excl[c]);
+      if (exclusive) {
 #pragma unroll
-      for (int j = 0; j < VEC; j++) x[c][j] = op(off, x[c][j]);
+        for (int j = VEC - 1; j > 0; j--) x[c][j] = op(off, x[c][j - 1]);
+        x[c][0] = off;
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) x[c][j] = op(off, x[c][j]);
+      }
     }
   }
   if constexpr (kNanAware) {
@@ -406,15 +496,16 @@ struct ScanConfig {
   static constexpr int BLOCK = 512;
   static constexpr int CHUNKS = 16;
   static constexpr int64_t TILE = (int64_t)BLOCK * (16 / sizeof(T)) * CHUNKS;
-  using P = typename std::conditional<(sizeof(T) < 4), uint32_t, T>::type;
 };
 
 template <class T, class Op>
 static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, const void* in,
                              void* out, int64_t n, const void* init, hipStream_t stream) {
   using C = ScanConfig<T>;
+  using Payload = typename scan_payload<T, Op>::type;
+  constexpr bool kRestarts = scan_restarts<T, Op>::value;
   const int64_t ntiles = ceil_div(n, C::TILE);
-  const size_t need = 256 + align_up((size_t)ntiles * TileDesc<typename C::P>::kBytesPerTile, 256);
+  const size_t need = 256 + align_up((size_t)ntiles * TileDesc<Payload>::kBytesPerTile, 256);
   if (temp == nullptr) {
     *temp_bytes = need;
     return hipSuccess;
@@ -423,7 +514,9 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   if (n == 0) return hipSuccess;
   // One tile consults no descriptor and reads its whole input before it writes any output: it
   // needs neither the cleared descriptors (a launch less: a third of a small call) nor tickets.
-  const bool single = ntiles == 1;
+  // (the restarting fold of floating-point minimum always takes tickets: its kernel exists in
+  // that form only)
+  const bool single = ntiles == 1 && !kRestarts;
   if (!single) {
     const hipError_t e = zero_async(temp, need, stream);
     if (e != hipSuccess) return e;
@@ -434,7 +527,7 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   uint64_t* desc = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + 256);
   // 128-bit accesses need no more than the elements' own alignment (see load16)
   const int vec_ok = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & (sizeof(T) - 1)) == 0;
-  const bool ticketed = !single && ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T));
+  const bool ticketed = kRestarts || (!single && ranges_overlap(in, (size_t)n * sizeof(T), out, (size_t)n * sizeof(T)));
   const int patience = ticketed ? 0 : lookback_patience(), delay = ticketed ? 0 : lookback_test_publish_delay();
   auto launch = [&](auto kernel) {
     TCD_LAUNCH("scan_kernel", kernel, dim3((unsigned)ntiles), dim3(C::BLOCK), stream, static_cast<const T*>(in),
@@ -443,6 +536,8 @@ static hipError_t scan_typed(void* temp, size_t* temp_bytes, int exclusive, cons
   if constexpr (sizeof(T) < 4) {
     if (ticketed) launch(scan_packed_kernel<T, Op, C::BLOCK, C::CHUNKS, true>);
     else launch(scan_packed_kernel<T, Op, C::BLOCK, C::CHUNKS, false>);
+  } else if constexpr (kRestarts) {
+    launch(scan_kernel<T, Op, C::BLOCK, C::CHUNKS, true>);
   } else {
     if (ticketed) launch(scan_kernel<T, Op, C::BLOCK, C::CHUNKS, true>);
     else launch(scan_kernel<T, Op, C::BLOCK, C::CHUNKS, false>);
@@ -516,10 +611,19 @@ extern "C" int thrust_cdna4_scan_static(int dtype, int op, int exclusive, const 
   using namespace tcd;
   if (n < 0) return hipErrorInvalidValue;
   // The size limit is checked first and has its own code, whatever the pointers are.
-  int64_t ntiles = -1;
-  dispatch_dtype(dtype, [&](auto t) { ntiles = ceil_div(n, ScanConfig<decltype(t)>::TILE); });
-  if (ntiles < 0) return hipErrorInvalidValue;  // unknown element type
-  if (ntiles > kStaticScanMaxTiles) return hipErrorOutOfMemory;
+  // (tiles the array has descriptors for: 16384, or 10922 for the three-word descriptors of a
+  // minimum scan over 8-byte floating-point values)
+  int64_t ntiles = -1, max_tiles = 0;
+  dispatch_dtype(dtype, [&](auto t) {
+    using T = decltype(t);
+    dispatch_op(op, [&](auto o) {
+      ntiles = ceil_div(n, ScanConfig<T>::TILE);
+      max_tiles = (int64_t)((kStaticScanScratchBytes - 256) / TileDesc<typename scan_payload<T, decltype(o)>::type>::kBytesPerTile);
+      if (max_tiles > kStaticScanMaxTiles) max_tiles = kStaticScanMaxTiles;
+    });
+  });
+  if (ntiles < 0) return hipErrorInvalidValue;  // unknown element type or operator
+  if (ntiles > max_tiles) return hipErrorOutOfMemory;
   if (n > 0 && (!in || !out)) return hipErrorInvalidValue;
   hipStream_t s = static_cast<hipStream_t>(stream);
   void* ptr = nullptr;
@@ -528,7 +632,6 @@ extern "C" int thrust_cdna4_scan_static(int dtype, int op, int exclusive, const 
   rc = hipErrorInvalidValue;
   dispatch_dtype(dtype, [&](auto t) {
     using T = decltype(t);
-    static_assert(TileDesc<typename ScanConfig<T>::P>::kBytesPerTile <= 16, "16 bytes of descriptor per tile");
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
       // scan_typed checks the size it needs against the bytes it is given and clears the

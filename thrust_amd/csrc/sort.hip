@@ -650,7 +650,8 @@ static hipError_t run_lds_order_check(hipStream_t s, int iters, unsigned long lo
   if (e != hipSuccess) return e;
   e = zero_async(sym, sizeof(unsigned long long), s);
   if (e != hipSuccess) return e;
-  TCD_LAUNCH("lds_atomic_order_kernel", lds_atomic_order_kernel, dim3(1024), dim3(512), s,
+  // four workgroups per compute unit: every LDS unit of the device is exercised
+  TCD_LAUNCH("lds_atomic_order_kernel", lds_atomic_order_kernel, dim3((unsigned)(4 * device_cu_count())), dim3(512), s,
              static_cast<unsigned long long*>(sym), iters);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
@@ -679,7 +680,7 @@ static hipError_t ensure_lds_order(hipStream_t s) {
   v = g_order_verdict[dev].load(std::memory_order_acquire);
   if (v == 0) {
     unsigned long long bad = 0;
-    e = run_lds_order_check(s, 24, &bad);  // 1.2e7 checked atomics
+    e = run_lds_order_check(s, 24, &bad);  // 1.2e7 checked atomics on 256 compute units
     if (e != hipSuccess) return e;
     v = bad == 0 ? 1 : 2;
     g_order_verdict[dev].store(v, std::memory_order_release);
