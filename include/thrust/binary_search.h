@@ -73,15 +73,32 @@ THRUST_CDNA4_SEARCH(binary_search, 2)
 #undef THRUST_CDNA4_SEARCH
 
 // scalar forms: an iterator for the bounds, a bool for binary_search
+// (the forms with a policy dispatch on the policy's own type by an unqualified call, thrust/detail/binary_search.inl:
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class)
 #define THRUST_CDNA4_SCALAR_BOUND(NAME, MODE)                                                                            \
-  template <class Policy, class Hay, class T, class Comp, detail::enable_if_policy<Policy> = 0>                          \
-  Hay NAME(const Policy& exec, Hay first, Hay last, const T& value, Comp comp) {                                         \
+  namespace system { namespace cdna4 {                                                                                  \
+  template <class D, class Hay, class T, class Comp>                                                                     \
+  Hay NAME(execution_policy<D>& exec, Hay first, Hay last, const T& value, Comp comp) {                                  \
+    return first + thrust::detail::scalar_search<MODE>(exec.derived(), first, last, value, comp);                        \
+  }                                                                                                                      \
+  template <class D, class Hay, class T>                                                                                 \
+  Hay NAME(execution_policy<D>& exec, Hay first, Hay last, const T& value) { return NAME(exec, first, last, value, thrust::less<>()); } \
+  }}                                                                                                                     \
+  template <class D, class Hay, class T, class Comp>                                                                     \
+  Hay NAME(const detail::execution_policy_base<D>& exec, Hay first, Hay last, const T& value, Comp comp) {               \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), first, last, value, comp);                              \
+  }                                                                                                                      \
+  template <class D, class Hay, class T>                                                                                 \
+  Hay NAME(const detail::execution_policy_base<D>& exec, Hay first, Hay last, const T& value) {                          \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), first, last, value);                                    \
+  }                                                                                                                      \
+  template <class Hay, class T, class Comp>                                                                              \
+  Hay NAME(const system::cpp::detail::par_t& exec, Hay first, Hay last, const T& value, Comp comp) {                     \
     return first + detail::scalar_search<MODE>(exec, first, last, value, comp);                                          \
   }                                                                                                                      \
-  template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>                                      \
-  Hay NAME(const Policy& exec, Hay first, Hay last, const T& value) {                                                    \
-    return first + detail::scalar_search<MODE>(exec, first, last, value, less<>());                                     \
-  }                                                                                                                      \
+  template <class Hay, class T>                                                                                          \
+  Hay NAME(const system::cpp::detail::par_t& exec, Hay first, Hay last, const T& value) { return NAME(exec, first, last, value, less<>()); } \
   template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(typename detail::implicit_policy<Hay, T>::type(), f, l, v); } \
   template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> Hay NAME(Hay f, Hay l, const T& v) { return NAME(host, f, l, v); } \
   template <class Hay, class T, class Comp, detail::enable_if_device<Hay, T> = 0,                                        \
@@ -93,14 +110,28 @@ THRUST_CDNA4_SEARCH(binary_search, 2)
 THRUST_CDNA4_SCALAR_BOUND(lower_bound, 0)
 THRUST_CDNA4_SCALAR_BOUND(upper_bound, 1)
 #undef THRUST_CDNA4_SCALAR_BOUND
-template <class Policy, class Hay, class T, class Comp, detail::enable_if_policy<Policy> = 0>
-bool binary_search(const Policy& exec, Hay first, Hay last, const T& value, Comp comp) {
+namespace system { namespace cdna4 {
+template <class D, class Hay, class T, class Comp>
+bool binary_search(execution_policy<D>& exec, Hay first, Hay last, const T& value, Comp comp) {
+  return thrust::detail::scalar_search<2>(exec.derived(), first, last, value, comp) != 0;
+}
+template <class D, class Hay, class T>
+bool binary_search(execution_policy<D>& exec, Hay first, Hay last, const T& value) { return binary_search(exec, first, last, value, thrust::less<>()); }
+}}  // namespace system::cdna4
+template <class D, class Hay, class T, class Comp>
+bool binary_search(const detail::execution_policy_base<D>& exec, Hay first, Hay last, const T& value, Comp comp) {
+  return binary_search(detail::derived_cast(detail::strip_const(exec)), first, last, value, comp);
+}
+template <class D, class Hay, class T>
+bool binary_search(const detail::execution_policy_base<D>& exec, Hay first, Hay last, const T& value) {
+  return binary_search(detail::derived_cast(detail::strip_const(exec)), first, last, value);
+}
+template <class Hay, class T, class Comp>
+bool binary_search(const system::cpp::detail::par_t& exec, Hay first, Hay last, const T& value, Comp comp) {
   return detail::scalar_search<2>(exec, first, last, value, comp) != 0;
 }
-template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>
-bool binary_search(const Policy& exec, Hay first, Hay last, const T& value) {
-  return detail::scalar_search<2>(exec, first, last, value, less<>()) != 0;
-}
+template <class Hay, class T>
+bool binary_search(const system::cpp::detail::par_t& exec, Hay first, Hay last, const T& value) { return binary_search(exec, first, last, value, less<>()); }
 template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(typename detail::implicit_policy<Hay, T>::type(), f, l, v); }
 template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> bool binary_search(Hay f, Hay l, const T& v) { return binary_search(host, f, l, v); }
 template <class Hay, class T, class Comp, detail::enable_if_device<Hay, T> = 0, typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>
@@ -109,15 +140,35 @@ template <class Hay, class T, class Comp, detail::enable_if_host<Hay, T> = 0, ty
 bool binary_search(Hay f, Hay l, const T& v, Comp c) { return binary_search(host, f, l, v, c); }
 
 // ---- equal_range (thrust/binary_search.h:727-1017): the pair (lower_bound, upper_bound) of one value
-template <class Policy, class Hay, class T, class Comp, detail::enable_if_policy<Policy> = 0>
-pair<Hay, Hay> equal_range(const Policy& exec, Hay first, Hay last, const T& value, Comp comp) {
+namespace detail {
+template <class Policy, class Hay, class T, class Comp>
+pair<Hay, Hay> composed_equal_range(const Policy& exec, Hay first, Hay last, const T& value, Comp comp) {
   const Hay lo = thrust::lower_bound(exec, first, last, value, comp);
   return pair<Hay, Hay>(lo, thrust::upper_bound(exec, lo, last, value, comp));
 }
-template <class Policy, class Hay, class T, detail::enable_if_policy<Policy> = 0>
-pair<Hay, Hay> equal_range(const Policy& exec, Hay first, Hay last, const T& value) {
-  return equal_range(exec, first, last, value, less<>());
+}  // namespace detail
+namespace system { namespace cdna4 {
+template <class D, class Hay, class T, class Comp>
+pair<Hay, Hay> equal_range(execution_policy<D>& exec, Hay first, Hay last, const T& value, Comp comp) {
+  return thrust::detail::composed_equal_range(exec.derived(), first, last, value, comp);
 }
+template <class D, class Hay, class T>
+pair<Hay, Hay> equal_range(execution_policy<D>& exec, Hay first, Hay last, const T& value) { return equal_range(exec, first, last, value, thrust::less<>()); }
+}}  // namespace system::cdna4
+template <class D, class Hay, class T, class Comp>
+pair<Hay, Hay> equal_range(const detail::execution_policy_base<D>& exec, Hay first, Hay last, const T& value, Comp comp) {
+  return equal_range(detail::derived_cast(detail::strip_const(exec)), first, last, value, comp);
+}
+template <class D, class Hay, class T>
+pair<Hay, Hay> equal_range(const detail::execution_policy_base<D>& exec, Hay first, Hay last, const T& value) {
+  return equal_range(detail::derived_cast(detail::strip_const(exec)), first, last, value);
+}
+template <class Hay, class T, class Comp>
+pair<Hay, Hay> equal_range(const system::cpp::detail::par_t& exec, Hay first, Hay last, const T& value, Comp comp) {
+  return detail::composed_equal_range(exec, first, last, value, comp);
+}
+template <class Hay, class T>
+pair<Hay, Hay> equal_range(const system::cpp::detail::par_t& exec, Hay first, Hay last, const T& value) { return equal_range(exec, first, last, value, less<>()); }
 template <class Hay, class T, detail::enable_if_device<Hay, T> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(typename detail::implicit_policy<Hay, T>::type(), f, l, v); }
 template <class Hay, class T, detail::enable_if_host<Hay, T> = 0> pair<Hay, Hay> equal_range(Hay f, Hay l, const T& v) { return equal_range(host, f, l, v); }
 template <class Hay, class T, class Comp, detail::enable_if_device<Hay, T, Comp> = 0, typename std::enable_if<!detail::is_policy<Hay>::value, int>::type = 0>

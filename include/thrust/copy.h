@@ -183,6 +183,14 @@ template <class D_, class In, class Size, class Out>
 Out copy_n(const detail::execution_policy_base<D_>& exec, In first, Size n, Out out) { return copy_n(detail::derived_cast(detail::strip_const(exec)), first, n, out); }
 template <class In, class Size, class Out>
 Out copy_n(const system::cpp::detail::par_t& exec, In first, Size n, Out out) { return detail::composed_copy_n(exec, first, n, out); }
-template <class In, class Size, class Out, typename std::enable_if<!detail::is_policy<In>::value, int>::type = 0>
+namespace detail {
+// iterators retagged with a user's policy type select that policy (testing/copy_n.cu:268-285)
+template <class... Its> struct has_user_policy {
+  static constexpr bool value = !std::is_same<typename implicit_policy<Its...>::type, system::cdna4::detail::par_t>::value;
+};
+}  // namespace detail
+template <class In, class Size, class Out, typename std::enable_if<!detail::is_policy<In>::value && !detail::has_user_policy<In, Out>::value, int>::type = 0>
 Out copy_n(In first, Size n, Out out) { return thrust::copy(first, detail::plus_n(first, n, 0), out); }
+template <class In, class Size, class Out, typename std::enable_if<!detail::is_policy<In>::value && detail::has_user_policy<In, Out>::value, int>::type = 0>
+Out copy_n(In first, Size n, Out out) { return copy_n(typename detail::implicit_policy<In, Out>::type(), first, n, out); }
 }  // namespace thrust

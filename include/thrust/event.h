@@ -128,6 +128,8 @@ class device_event {
   };
   stream_reference stream() const { return stream_reference{state().stream()}; }
   const std::shared_ptr<system::cdna4::detail::async_signal>& signal() const { return signal_; }
+  // gives the stream and its work away: the event is left without state
+  std::shared_ptr<system::cdna4::detail::async_signal> release_signal() { return std::move(signal_); }
  protected:
   system::cdna4::detail::async_signal& state() const {
     if (!signal_) throw event_error(event_errc::no_state);
@@ -214,10 +216,27 @@ execute_after par_t::after(Events&&... events) const {
 }
 }}}  // namespace system::cdna4::detail
 // an event that is ready when all of the given ones are
+// The given events are consumed, lvalues too (testing/event.cu:72-110: afterwards they have no
+// stream and are not ready), and the result continues the first one's stream, which waits for the
+// others (thrust/system/cuda/detail/future.inl:1349-: when_all acquires the streams of its arguments).
+namespace system { namespace cdna4 { namespace detail {
+inline void consume(std::vector<std::shared_ptr<async_signal>>&) {}
+template <class E, class... Es>
+void consume(std::vector<std::shared_ptr<async_signal>>& taken, E&& e, Es&&... es) {
+  if (e.valid_stream()) taken.push_back(e.release_signal());
+  consume(taken, std::forward<Es>(es)...);
+}
+}}}  // namespace system::cdna4::detail
 template <class... Events>
 device_event when_all(Events&&... events) {
-  system::cdna4::detail::execute_after p;
-  system::cdna4::detail::collect(p, std::forward<Events>(events)...);
-  return device_event(system::cdna4::detail::make_signal(p));
+  std::vector<std::shared_ptr<system::cdna4::detail::async_signal>> taken;
+  system::cdna4::detail::consume(taken, std::forward<Events>(events)...);
+  if (taken.empty()) return device_event(std::make_shared<system::cdna4::detail::async_signal>());
+  std::shared_ptr<system::cdna4::detail::async_signal> first = taken[0];
+  for (std::size_t i = 1; i < taken.size(); i++) {
+    first->depend_on(*taken[i]);
+    first->keep_alive(taken[i]);
+  }
+  return device_event(std::move(first));
 }
 }  // namespace thrust

@@ -71,7 +71,8 @@ pair<It, It> minmax_element(const system::cpp::detail::par_t&, It first, It last
   return thrust::make_pair(std::min_element(first, last, comp), std::max_element(first, last, comp));  // the FIRST maximum
 }
 #define THRUST_CDNA4_EXTREMA(NAME, RET)                                                                                     \
-  template <class Policy, class It, detail::enable_if_policy<Policy> = 0> RET NAME(const Policy& exec, It f, It l) { return NAME(exec, f, l, less<>()); } \
+  template <class D, class It> RET NAME(const detail::execution_policy_base<D>& exec, It f, It l) { return NAME(detail::derived_cast(detail::strip_const(exec)), f, l); } \
+  template <class It> RET NAME(const system::cpp::detail::par_t& exec, It f, It l) { return NAME(exec, f, l, less<>()); }     \
   template <class It, detail::enable_if_device<It> = 0> RET NAME(It f, It l) { return NAME(typename detail::implicit_policy<It>::type(), f, l); }                    \
   template <class It, detail::enable_if_host<It> = 0> RET NAME(It f, It l) { return NAME(host, f, l); }                        \
   template <class It, class C, detail::enable_if_device<It, C> = 0> RET NAME(It f, It l, C c) { return NAME(typename detail::implicit_policy<It, C>::type(), f, l, c); }  \

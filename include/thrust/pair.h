@@ -6,6 +6,7 @@
 #include <type_traits>
 #include <utility>
 #include <thrust/detail/hd.h>
+#include <thrust/detail/swap.h>
 
 namespace thrust {
 template <class T1, class T2>
@@ -31,11 +32,14 @@ struct pair {
     return *this;
   }
   template <class U1, class U2> operator std::pair<U1, U2>() const { return std::pair<U1, U2>(first, second); }
+  // member by member, each with the swap its type provides (thrust/pair.h: pair::swap)
   THRUST_CDNA4_HD void swap(pair& p) {
-    T1 a = first; first = p.first; p.first = a;
-    T2 b = second; second = p.second; p.second = b;
+    detail::adl_swap(first, p.first);
+    detail::adl_swap(second, p.second);
   }
 };
+template <class T1, class T2>
+THRUST_CDNA4_HD inline void swap(pair<T1, T2>& x, pair<T1, T2>& y) { x.swap(y); }
 
 template <class T1, class T2>
 THRUST_CDNA4_HD constexpr pair<typename std::decay<T1>::type, typename std::decay<T2>::type> make_pair(T1&& x, T2&& y) {

@@ -23,10 +23,19 @@ void sequence(const system::cpp::detail::par_t&, It first, It last, T init, T st
   std::size_t i = 0;
   for (; first != last; ++first, ++i) *first = detail::sequence_value(init, step, i, std::is_arithmetic<T>());
 }
-template <class Policy, class It, class T>
-void sequence(const Policy& exec, It first, It last, T init) { sequence(exec, first, last, init, T(1)); }
-template <class Policy, class It, class = typename std::iterator_traits<It>::iterator_category>
-void sequence(const Policy& exec, It first, It last) {
+// the shorter forms dispatch on the policy like the full one (testing/sequence.cu:8-24 overloads the shortest)
+template <class D, class It, class T>
+void sequence(const detail::execution_policy_base<D>& exec, It first, It last, T init) {
+  sequence(detail::derived_cast(detail::strip_const(exec)), first, last, init);
+}
+template <class D, class It, class = typename std::iterator_traits<It>::iterator_category>
+void sequence(const detail::execution_policy_base<D>& exec, It first, It last) {
+  sequence(detail::derived_cast(detail::strip_const(exec)), first, last);
+}
+template <class It, class T>
+void sequence(const system::cpp::detail::par_t& exec, It first, It last, T init) { sequence(exec, first, last, init, T(1)); }
+template <class It, class = typename std::iterator_traits<It>::iterator_category>
+void sequence(const system::cpp::detail::par_t& exec, It first, It last) {
   typedef typename detail::value_of<It>::type V;
   sequence(exec, first, last, V(0), V(1));
 }

@@ -110,14 +110,36 @@ std::int64_t set_operation(const system::cpp::detail::par_t&, K1 k1, K1 l1, K2 k
 }  // namespace detail
 
 // The four algorithms on keys: NAME(policy, first1, last1, first2, last2, result[, comp]) and the forms without a policy.
+// The forms with a policy dispatch on the policy's own type by an unqualified call (thrust/detail/set_operations.inl):
+// a user's overload for a policy type derived from thrust::device_execution_policy is preferred to
+// the device system's, which is found through the policy's base class.
 #define THRUST_CDNA4_SET_OPERATION(NAME, MODE)                                                                                        \
-  template <class Policy, class In1, class In2, class Out, class Comp, detail::enable_if_policy<Policy> = 0>                          \
-  Out NAME(const Policy& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp comp) {                                                    \
+  namespace system { namespace cdna4 {                                                                                               \
+  template <class D, class In1, class In2, class Out, class Comp>                                                                     \
+  Out NAME(execution_policy<D>& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp comp) {                                             \
+    return r + thrust::detail::set_operation<MODE, false>(exec.derived(), f1, l1, f2, l2, thrust::detail::no_value_iterator(),        \
+                                                          thrust::detail::no_value_iterator(), r, thrust::detail::no_value_iterator(), comp); \
+  }                                                                                                                                   \
+  template <class D, class In1, class In2, class Out>                                                                                 \
+  Out NAME(execution_policy<D>& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) {                                                        \
+    return NAME(exec, f1, l1, f2, l2, r, thrust::less<typename thrust::detail::value_of<In1>::type>());                               \
+  }                                                                                                                                   \
+  }}                                                                                                                                  \
+  template <class D, class In1, class In2, class Out, class Comp>                                                                     \
+  Out NAME(const detail::execution_policy_base<D>& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp comp) {                          \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), f1, l1, f2, l2, r, comp);                                            \
+  }                                                                                                                                   \
+  template <class D, class In1, class In2, class Out>                                                                                 \
+  Out NAME(const detail::execution_policy_base<D>& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) {                                     \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), f1, l1, f2, l2, r);                                                  \
+  }                                                                                                                                   \
+  template <class In1, class In2, class Out, class Comp>                                                                              \
+  Out NAME(const system::cpp::detail::par_t& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r, Comp comp) {                                \
     return r + detail::set_operation<MODE, false>(exec, f1, l1, f2, l2, detail::no_value_iterator(), detail::no_value_iterator(), r, \
                                                   detail::no_value_iterator(), comp);                                               \
   }                                                                                                                                   \
-  template <class Policy, class In1, class In2, class Out, detail::enable_if_policy<Policy> = 0>                                      \
-  Out NAME(const Policy& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) {                                                               \
+  template <class In1, class In2, class Out>                                                                                          \
+  Out NAME(const system::cpp::detail::par_t& exec, In1 f1, In1 l1, In2 f2, In2 l2, Out r) {                                           \
     return NAME(exec, f1, l1, f2, l2, r, less<typename detail::value_of<In1>::type>());                                               \
   }                                                                                                                                   \
   template <class In1, class In2, class Out, class Comp, detail::enable_if_device<In1, In2, Out, Comp> = 0>                                           \
@@ -128,22 +150,41 @@ std::int64_t set_operation(const system::cpp::detail::par_t&, K1 k1, K1 l1, K2 k
   Out NAME(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return NAME(typename detail::implicit_policy<In1, In2, Out>::type(), f1, l1, f2, l2, r); }                                         \
   template <class In1, class In2, class Out, detail::enable_if_host<In1, In2, Out> = 0>                                                         \
   Out NAME(In1 f1, In1 l1, In2 f2, In2 l2, Out r) { return NAME(host, f1, l1, f2, l2, r); }
-THRUST_CDNA4_SET_OPERATION(set_difference, detail::set_difference_mode)
-THRUST_CDNA4_SET_OPERATION(set_intersection, detail::set_intersection_mode)
-THRUST_CDNA4_SET_OPERATION(set_symmetric_difference, detail::set_symmetric_difference_mode)
-THRUST_CDNA4_SET_OPERATION(set_union, detail::set_union_mode)
+THRUST_CDNA4_SET_OPERATION(set_difference, thrust::detail::set_difference_mode)
+THRUST_CDNA4_SET_OPERATION(set_intersection, thrust::detail::set_intersection_mode)
+THRUST_CDNA4_SET_OPERATION(set_symmetric_difference, thrust::detail::set_symmetric_difference_mode)
+THRUST_CDNA4_SET_OPERATION(set_union, thrust::detail::set_union_mode)
 #undef THRUST_CDNA4_SET_OPERATION
 
 // The by-key forms with values for both ranges:
 // NAME(policy, kfirst1, klast1, kfirst2, klast2, vfirst1, vfirst2, kresult, vresult[, comp]).
 #define THRUST_CDNA4_SET_OPERATION_BY_KEY(NAME, MODE)                                                                                 \
-  template <class Policy, class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp, detail::enable_if_policy<Policy> = 0> \
-  pair<KOut, VOut> NAME(const Policy& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp comp) {              \
+  namespace system { namespace cdna4 {                                                                                               \
+  template <class D, class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp>                                      \
+  pair<KOut, VOut> NAME(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp comp) {       \
+    const std::int64_t c = thrust::detail::set_operation<MODE, true>(exec.derived(), kf1, kl1, kf2, kl2, v1, v2, kr, vr, comp);       \
+    return pair<KOut, VOut>(kr + c, vr + c);                                                                                          \
+  }                                                                                                                                   \
+  template <class D, class K1, class K2, class V1, class V2, class KOut, class VOut>                                                  \
+  pair<KOut, VOut> NAME(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) {                  \
+    return NAME(exec, kf1, kl1, kf2, kl2, v1, v2, kr, vr, thrust::less<typename thrust::detail::value_of<K1>::type>());               \
+  }                                                                                                                                   \
+  }}                                                                                                                                  \
+  template <class D, class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp>                                      \
+  pair<KOut, VOut> NAME(const detail::execution_policy_base<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp comp) { \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), kf1, kl1, kf2, kl2, v1, v2, kr, vr, comp);                           \
+  }                                                                                                                                   \
+  template <class D, class K1, class K2, class V1, class V2, class KOut, class VOut>                                                  \
+  pair<KOut, VOut> NAME(const detail::execution_policy_base<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), kf1, kl1, kf2, kl2, v1, v2, kr, vr);                                 \
+  }                                                                                                                                   \
+  template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp>                                               \
+  pair<KOut, VOut> NAME(const system::cpp::detail::par_t& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr, Comp comp) { \
     const std::int64_t c = detail::set_operation<MODE, true>(exec, kf1, kl1, kf2, kl2, v1, v2, kr, vr, comp);                         \
     return pair<KOut, VOut>(kr + c, vr + c);                                                                                          \
   }                                                                                                                                   \
-  template <class Policy, class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_policy<Policy> = 0>       \
-  pair<KOut, VOut> NAME(const Policy& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) {                         \
+  template <class K1, class K2, class V1, class V2, class KOut, class VOut>                                                           \
+  pair<KOut, VOut> NAME(const system::cpp::detail::par_t& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) {     \
     return NAME(exec, kf1, kl1, kf2, kl2, v1, v2, kr, vr, less<typename detail::value_of<K1>::type>());                               \
   }                                                                                                                                   \
   template <class K1, class K2, class V1, class V2, class KOut, class VOut, class Comp, detail::enable_if_device<K1, K2, V1, V2, KOut, VOut, Comp> = 0>             \
@@ -154,19 +195,38 @@ THRUST_CDNA4_SET_OPERATION(set_union, detail::set_union_mode)
   pair<KOut, VOut> NAME(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return NAME(typename detail::implicit_policy<K1, K2, V1, V2, KOut, VOut>::type(), kf1, kl1, kf2, kl2, v1, v2, kr, vr); } \
   template <class K1, class K2, class V1, class V2, class KOut, class VOut, detail::enable_if_host<K1, K2, V1, V2, KOut, VOut> = 0>                           \
   pair<KOut, VOut> NAME(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, V2 v2, KOut kr, VOut vr) { return NAME(host, kf1, kl1, kf2, kl2, v1, v2, kr, vr); }
-THRUST_CDNA4_SET_OPERATION_BY_KEY(set_difference_by_key, detail::set_difference_mode)
-THRUST_CDNA4_SET_OPERATION_BY_KEY(set_symmetric_difference_by_key, detail::set_symmetric_difference_mode)
-THRUST_CDNA4_SET_OPERATION_BY_KEY(set_union_by_key, detail::set_union_mode)
+THRUST_CDNA4_SET_OPERATION_BY_KEY(set_difference_by_key, thrust::detail::set_difference_mode)
+THRUST_CDNA4_SET_OPERATION_BY_KEY(set_symmetric_difference_by_key, thrust::detail::set_symmetric_difference_mode)
+THRUST_CDNA4_SET_OPERATION_BY_KEY(set_union_by_key, thrust::detail::set_union_mode)
 #undef THRUST_CDNA4_SET_OPERATION_BY_KEY
 
 // set_intersection_by_key takes values for the first range only (every result comes from it).
-template <class Policy, class K1, class K2, class V1, class KOut, class VOut, class Comp, detail::enable_if_policy<Policy> = 0>
-pair<KOut, VOut> set_intersection_by_key(const Policy& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr, Comp comp) {
+namespace system { namespace cdna4 {
+template <class D, class K1, class K2, class V1, class KOut, class VOut, class Comp>
+pair<KOut, VOut> set_intersection_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr, Comp comp) {
+  const std::int64_t c = thrust::detail::set_operation<thrust::detail::set_intersection_mode, true>(exec.derived(), kf1, kl1, kf2, kl2, v1, v1, kr, vr, comp);
+  return pair<KOut, VOut>(kr + c, vr + c);
+}
+template <class D, class K1, class K2, class V1, class KOut, class VOut>
+pair<KOut, VOut> set_intersection_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr) {
+  return set_intersection_by_key(exec, kf1, kl1, kf2, kl2, v1, kr, vr, thrust::less<typename thrust::detail::value_of<K1>::type>());
+}
+}}  // namespace system::cdna4
+template <class D, class K1, class K2, class V1, class KOut, class VOut, class Comp>
+pair<KOut, VOut> set_intersection_by_key(const detail::execution_policy_base<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr, Comp comp) {
+  return set_intersection_by_key(detail::derived_cast(detail::strip_const(exec)), kf1, kl1, kf2, kl2, v1, kr, vr, comp);
+}
+template <class D, class K1, class K2, class V1, class KOut, class VOut>
+pair<KOut, VOut> set_intersection_by_key(const detail::execution_policy_base<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr) {
+  return set_intersection_by_key(detail::derived_cast(detail::strip_const(exec)), kf1, kl1, kf2, kl2, v1, kr, vr);
+}
+template <class K1, class K2, class V1, class KOut, class VOut, class Comp>
+pair<KOut, VOut> set_intersection_by_key(const system::cpp::detail::par_t& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr, Comp comp) {
   const std::int64_t c = detail::set_operation<detail::set_intersection_mode, true>(exec, kf1, kl1, kf2, kl2, v1, v1, kr, vr, comp);
   return pair<KOut, VOut>(kr + c, vr + c);
 }
-template <class Policy, class K1, class K2, class V1, class KOut, class VOut, detail::enable_if_policy<Policy> = 0>
-pair<KOut, VOut> set_intersection_by_key(const Policy& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr) {
+template <class K1, class K2, class V1, class KOut, class VOut>
+pair<KOut, VOut> set_intersection_by_key(const system::cpp::detail::par_t& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 v1, KOut kr, VOut vr) {
   return set_intersection_by_key(exec, kf1, kl1, kf2, kl2, v1, kr, vr, less<typename detail::value_of<K1>::type>());
 }
 template <class K1, class K2, class V1, class KOut, class VOut, class Comp, detail::enable_if_device<K1, K2, V1, KOut, VOut, Comp> = 0>

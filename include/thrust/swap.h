@@ -3,10 +3,13 @@
 #include <algorithm>
 #include <utility>
 #include <thrust/detail/iterator_util.h>
+#include <thrust/detail/raw_reference_cast.h>
+#include <thrust/detail/swap.h>
 #include <thrust/execution_policy.h>
 #include <thrust/system/cdna4/detail/index_algorithms.h>
 
 namespace thrust {
+// thrust::swap(a, b) (thrust/swap.h:43-50): assignment through a temporary
 template <class A, class B> THRUST_CDNA4_HD inline void swap(A& a, B& b) {
   A t = a;
   a = b;
@@ -16,9 +19,8 @@ namespace detail {
 template <class A, class B> struct swap_body {
   A a; B b;
   THRUST_CDNA4_HD void operator()(std::int64_t i) {
-    typename std::iterator_traits<A>::value_type t = a[i];
-    a[i] = b[i];
-    b[i] = t;
+    // the elements' own swap where their type has one (testing/swap_ranges.cu:150-215)
+    adl_swap(thrust::raw_reference_cast(a[i]), thrust::raw_reference_cast(b[i]));
   }
 };
 }  // namespace detail

@@ -22,5 +22,12 @@ pair<It, It> minmax_element(const system::cdna4::execution_policy<D>& exec, It f
   const auto e = thrust::detail::extrema_of(exec.derived(), first, last, comp);
   return thrust::make_pair(first + e.lo_at, first + e.hi_at);
 }
+// without a comparison: operator< (thrust/extrema.h:79-81, :348-350, :606-608)
+template <class D, class It>
+It min_element(const system::cdna4::execution_policy<D>& exec, It first, It last) { return min_element(exec, first, last, thrust::less<>()); }
+template <class D, class It>
+It max_element(const system::cdna4::execution_policy<D>& exec, It first, It last) { return max_element(exec, first, last, thrust::less<>()); }
+template <class D, class It>
+pair<It, It> minmax_element(const system::cdna4::execution_policy<D>& exec, It first, It last) { return minmax_element(exec, first, last, thrust::less<>()); }
 }}  // namespace system::cdna4
 }  // namespace thrust

@@ -103,10 +103,35 @@ void generic_scan(const Policy& exec, In in, Out out, std::int64_t n, Acc init, 
 #endif
 }
 
+// An output written over the KEYS (testing/scan_by_key.inclusive.cu:325-334 does it): the engine
+// reads the key before an element from memory, some of them after other elements' results have
+// been stored.  Keys and output that are both given by raw pointers and share a byte are told apart
+// here, and the keys are then read from a copy; ranges behind other iterators cannot be compared.
+template <class KIn, class Out>
+inline std::size_t keys_to_set_aside(KIn, Out, std::int64_t) { return 0; }
+template <class K, class O>
+inline std::size_t keys_to_set_aside(K* keys, O* out, std::int64_t n) {
+  const char* k = reinterpret_cast<const char*>(keys);
+  const char* o = reinterpret_cast<const char*>(out);
+  const bool overlap = n > 0 && k < o + n * (std::int64_t)sizeof(O) && o < k + n * (std::int64_t)sizeof(K);
+  return overlap ? (std::size_t)n * sizeof(K) : 0;
+}
+template <class KIn>
+inline KIn keys_set_aside(KIn keys, void*, std::size_t, void*) { return keys; }
+template <class K>
+inline K* keys_set_aside(K* keys, void* copy, std::size_t bytes, void* stream) {
+  if (!bytes) return keys;
+  throw_on_error(thrust_cdna4_memcpy_dtod(copy, keys, bytes, stream), "by key: setting the keys aside");
+  return static_cast<K*>(copy);
+}
+
 template <bool EXCLUSIVE, class V, class Policy, class KIn, class VIn, class Out, class Pred, class Op>
 void generic_scan_by_key(const Policy& exec, KIn keys, VIn vals, Out out, std::int64_t n, V init, Pred pred, Op op) {
   THRUST_CDNA4_NEEDS_HIPCC(Op);
 #if defined(__HIPCC__)
+  const std::size_t aside = keys_to_set_aside(keys, out, n);
+  temporary_storage hold(aside, exec);
+  keys = keys_set_aside(keys, hold.data(), aside, stream_of(exec));
   generic::scan_engine(stream_of(exec), n, scan_by_key_body<KIn, VIn, Out, V, Pred, Op, EXCLUSIVE>{keys, vals, out, init, pred, op});
   synchronize_optional(exec, "scan_by_key: failed to synchronize");
 #else
@@ -121,6 +146,9 @@ std::int64_t generic_reduce_by_key(const Policy& exec, KIn keys, VIn vals, KOut 
   THRUST_CDNA4_NEEDS_HIPCC(Op);
 #if defined(__HIPCC__)
   if (n <= 0) return 0;
+  const std::size_t aside = keys_to_set_aside(keys, kout, n) ? keys_to_set_aside(keys, kout, n) : keys_to_set_aside(keys, vout, n);
+  temporary_storage hold(aside, exec);
+  keys = keys_set_aside(keys, hold.data(), aside, stream_of(exec));
   temporary_storage tmp(256, exec);
   long long* d_runs = static_cast<long long*>(tmp.data());
   if (n < (std::int64_t(1) << 32))

@@ -12,5 +12,12 @@ void sequence(const system::cdna4::execution_policy<D>& exec, It first, It last,
   // (thrust/system/detail/generic/sequence.inl:36-90)
   system::cdna4::detail::sequence_n(exec.derived(), thrust::detail::unwrap(first), (std::int64_t)(last - first), init, step);
 }
+template <class D, class It, class T>
+void sequence(const system::cdna4::execution_policy<D>& exec, It first, It last, T init) { sequence(exec, first, last, init, T(1)); }
+template <class D, class It, class = typename std::iterator_traits<It>::iterator_category>
+void sequence(const system::cdna4::execution_policy<D>& exec, It first, It last) {
+  typedef typename thrust::detail::value_of<It>::type V;
+  sequence(exec, first, last, V(0), V(1));
+}
 }}  // namespace system::cdna4
 }  // namespace thrust

@@ -42,5 +42,23 @@ pair<KIn, VIn> unique_by_key(const system::cdna4::execution_policy<D>& exec, KIn
                                                                      thrust::detail::unwrap(vfirst), n, eq);
   return thrust::make_pair(kfirst + c, vfirst + c);
 }
+// ---- default equality
+template <class D, class In, class Out, class = typename std::iterator_traits<In>::iterator_category,
+          class = typename std::iterator_traits<Out>::iterator_category>
+Out unique_copy(const system::cdna4::execution_policy<D>& exec, In first, In last, Out out) {
+  return unique_copy(exec, first, last, out, thrust::equal_to<typename thrust::detail::value_of<In>::type>());
+}
+template <class D, class In, class = typename std::iterator_traits<In>::iterator_category>
+In unique(const system::cdna4::execution_policy<D>& exec, In first, In last) {
+  return unique(exec, first, last, thrust::equal_to<typename thrust::detail::value_of<In>::type>());
+}
+template <class D, class KIn, class VIn, class = typename std::iterator_traits<VIn>::iterator_category>
+pair<KIn, VIn> unique_by_key(const system::cdna4::execution_policy<D>& exec, KIn kfirst, KIn klast, VIn vfirst) {
+  return unique_by_key(exec, kfirst, klast, vfirst, thrust::equal_to<typename thrust::detail::value_of<KIn>::type>());
+}
+template <class D, class KIn, class VIn, class KOut, class VOut, class = typename std::iterator_traits<VOut>::iterator_category>
+pair<KOut, VOut> unique_by_key_copy(const system::cdna4::execution_policy<D>& exec, KIn kfirst, KIn klast, VIn vfirst, KOut kout, VOut vout) {
+  return unique_by_key_copy(exec, kfirst, klast, vfirst, kout, vout, thrust::equal_to<typename thrust::detail::value_of<KIn>::type>());
+}
 }}  // namespace system::cdna4
 }  // namespace thrust

@@ -7,6 +7,7 @@
 #include <type_traits>
 #include <utility>
 #include <thrust/detail/hd.h>
+#include <thrust/detail/swap.h>
 
 namespace thrust {
 template <class... Ts> struct tuple;
@@ -202,8 +203,7 @@ THRUST_CDNA4_HD constexpr tuple<T0&, T1&, T2&, T3&, T4&, T5&, T6&, T7&, T8&, T9&
 namespace detail {
 template <std::size_t I, std::size_t N> struct tuple_swap {
   template <class A, class B> THRUST_CDNA4_HD static void run(A& a, B& b) {
-    using std::swap;
-    swap(get<I>(a), get<I>(b));
+    adl_swap(get<I>(a), get<I>(b));
     tuple_swap<I + 1, N>::run(a, b);
   }
 };

@@ -26,7 +26,16 @@ template <class D_, class In, class Size, class Out>
 Out uninitialized_copy_n(const detail::execution_policy_base<D_>& exec, In first, Size n, Out result) { return uninitialized_copy_n(detail::derived_cast(detail::strip_const(exec)), first, n, result); }
 template <class In, class Size, class Out>
 Out uninitialized_copy_n(const system::cpp::detail::par_t& exec, In first, Size n, Out result) { return detail::composed_uninitialized_copy_n(exec, first, n, result); }
-template <class In, class Out> Out uninitialized_copy(In f, In l, Out o) { return copy(f, l, o); }
-template <class In, class Size, class Out, class = typename std::iterator_traits<In>::iterator_category>
+// without a policy: iterators retagged with a user's policy type select that policy
+// (testing/uninitialized_copy.cu:37-100); any other pair of ranges is a copy between their systems
+template <class In, class Out, typename std::enable_if<!detail::has_user_policy<In, Out>::value, int>::type = 0>
+Out uninitialized_copy(In f, In l, Out o) { return copy(f, l, o); }
+template <class In, class Out, typename std::enable_if<detail::has_user_policy<In, Out>::value, int>::type = 0>
+Out uninitialized_copy(In f, In l, Out o) { return uninitialized_copy(typename detail::implicit_policy<In, Out>::type(), f, l, o); }
+template <class In, class Size, class Out, class = typename std::iterator_traits<In>::iterator_category,
+          typename std::enable_if<!detail::has_user_policy<In, Out>::value, int>::type = 0>
 Out uninitialized_copy_n(In f, Size n, Out o) { return copy(f, f + n, o); }
+template <class In, class Size, class Out, class = typename std::iterator_traits<In>::iterator_category,
+          typename std::enable_if<detail::has_user_policy<In, Out>::value, int>::type = 0>
+Out uninitialized_copy_n(In f, Size n, Out o) { return uninitialized_copy_n(typename detail::implicit_policy<In, Out>::type(), f, n, o); }
 }  // namespace thrust

@@ -63,18 +63,36 @@ template <class KIn, class VIn, class Eq>
 pair<KIn, VIn> unique_by_key(const system::cpp::detail::par_t& e, KIn kfirst, KIn klast, VIn vfirst, Eq eq) {
   return unique_by_key_copy(e, kfirst, klast, vfirst, kfirst, vfirst, eq);  // outputs trail the inputs
 }
-// ---- default equality, any policy
-template <class Policy, class In, class Out, class = typename std::iterator_traits<In>::iterator_category,
+// ---- default equality: the shorter forms dispatch on the policy like the full ones
+// (testing/unique.cu and testing/unique_by_key.cu overload the shortest for their own policy)
+template <class D, class In, class Out, class = typename std::iterator_traits<In>::iterator_category,
           class = typename std::iterator_traits<Out>::iterator_category>
-Out unique_copy(const Policy& exec, In first, In last, Out out) { return unique_copy(exec, first, last, out, equal_to<typename detail::value_of<In>::type>()); }
-template <class Policy, class In, class = typename std::iterator_traits<In>::iterator_category>
-In unique(const Policy& exec, In first, In last) { return unique(exec, first, last, equal_to<typename detail::value_of<In>::type>()); }
-template <class Policy, class KIn, class VIn, class = typename std::iterator_traits<VIn>::iterator_category>
-pair<KIn, VIn> unique_by_key(const Policy& exec, KIn kfirst, KIn klast, VIn vfirst) {
+Out unique_copy(const detail::execution_policy_base<D>& exec, In first, In last, Out out) {
+  return unique_copy(detail::derived_cast(detail::strip_const(exec)), first, last, out);
+}
+template <class D, class In, class = typename std::iterator_traits<In>::iterator_category>
+In unique(const detail::execution_policy_base<D>& exec, In first, In last) {
+  return unique(detail::derived_cast(detail::strip_const(exec)), first, last);
+}
+template <class D, class KIn, class VIn, class = typename std::iterator_traits<VIn>::iterator_category>
+pair<KIn, VIn> unique_by_key(const detail::execution_policy_base<D>& exec, KIn kfirst, KIn klast, VIn vfirst) {
+  return unique_by_key(detail::derived_cast(detail::strip_const(exec)), kfirst, klast, vfirst);
+}
+template <class D, class KIn, class VIn, class KOut, class VOut, class = typename std::iterator_traits<VOut>::iterator_category>
+pair<KOut, VOut> unique_by_key_copy(const detail::execution_policy_base<D>& exec, KIn kfirst, KIn klast, VIn vfirst, KOut kout, VOut vout) {
+  return unique_by_key_copy(detail::derived_cast(detail::strip_const(exec)), kfirst, klast, vfirst, kout, vout);
+}
+template <class In, class Out, class = typename std::iterator_traits<In>::iterator_category,
+          class = typename std::iterator_traits<Out>::iterator_category>
+Out unique_copy(const system::cpp::detail::par_t& exec, In first, In last, Out out) { return unique_copy(exec, first, last, out, equal_to<typename detail::value_of<In>::type>()); }
+template <class In, class = typename std::iterator_traits<In>::iterator_category>
+In unique(const system::cpp::detail::par_t& exec, In first, In last) { return unique(exec, first, last, equal_to<typename detail::value_of<In>::type>()); }
+template <class KIn, class VIn, class = typename std::iterator_traits<VIn>::iterator_category>
+pair<KIn, VIn> unique_by_key(const system::cpp::detail::par_t& exec, KIn kfirst, KIn klast, VIn vfirst) {
   return unique_by_key(exec, kfirst, klast, vfirst, equal_to<typename detail::value_of<KIn>::type>());
 }
-template <class Policy, class KIn, class VIn, class KOut, class VOut, class = typename std::iterator_traits<VOut>::iterator_category>
-pair<KOut, VOut> unique_by_key_copy(const Policy& exec, KIn kfirst, KIn klast, VIn vfirst, KOut kout, VOut vout) {
+template <class KIn, class VIn, class KOut, class VOut, class = typename std::iterator_traits<VOut>::iterator_category>
+pair<KOut, VOut> unique_by_key_copy(const system::cpp::detail::par_t& exec, KIn kfirst, KIn klast, VIn vfirst, KOut kout, VOut vout) {
   return unique_by_key_copy(exec, kfirst, klast, vfirst, kout, vout, equal_to<typename detail::value_of<KIn>::type>());
 }
 // ---- no policy

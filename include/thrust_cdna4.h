@@ -139,7 +139,9 @@ int thrust_cdna4_scan_static(int dtype, int op, int exclusive, const void* in, v
  * exclusive_scan_by_key_n and cub::DispatchScanByKey
  * (thrust/system/cuda/detail/scan_by_key.h:69-282).  The exclusive form restarts from
  * `*init` at every segment head (sequential/scan_by_key.h:95-140).  `values == out` is
- * allowed.  n must be < 2^32 (32-bit head counts; the reference switches to 64-bit offsets there,
+ * allowed, and so is an `out` that overlaps `keys` (testing/scan_by_key.inclusive.cu:325-334): the
+ * keys are then read from a copy in the temporary storage, which is n keys larger for it — make
+ * the size query with the pointers of the call.  n must be < 2^32 (32-bit head counts; the reference switches to 64-bit offsets there,
  * thrust/system/cuda/detail/dispatch.h:29-78 — the template layer's kernel templates take over).
  */
 int thrust_cdna4_scan_by_key(void* temp, size_t* temp_bytes, int key_dtype, int value_dtype,
@@ -152,7 +154,9 @@ int thrust_cdna4_scan_by_key(void* temp, size_t* temp_bytes, int key_dtype, int 
  * For each maximal run of equal consecutive keys writes the run's first key to keys_out
  * and the left-to-right reduction of its values to values_out; writes the number of runs
  * (int64) to the DEVICE location `num_runs_out`, which the caller reads back after
- * synchronising (reduce_by_key.h:1049-1052).  Outputs must not overlap inputs.  n must be < 2^32
+ * synchronising (reduce_by_key.h:1049-1052).  An output may overlap an input it has the element
+ * size of or begins at (the compaction only moves to the left); outputs over keys_in make the call
+ * read the keys from a copy in the temporary storage, as in scan_by_key.  n must be < 2^32
  * (32-bit run positions; beyond, the template layer's kernel templates take over).
  */
 int thrust_cdna4_reduce_by_key(void* temp, size_t* temp_bytes, int key_dtype, int value_dtype,

@@ -233,6 +233,31 @@ def test_by_key_aliased_outputs_take_the_ticket_path():
     assert same_bits(host(gk), rk) and same_bits(host(gv), rv)
 
 
+def test_outputs_written_over_the_keys():
+    """testing/scan_by_key.inclusive.cu:325-334 scans into the key range.  A tile reads the key before
+    its first element from memory, where the tile before it may have stored results already: the
+    library reads the keys from a copy then.  Every element a run of its own is the case in which
+    reduce_by_key's compaction writes exactly where the next tile looks."""
+    n = 16384 * 5 + 77
+    for mean in (1, 2, 40):
+        k = (runs(7 + mean, n, mean, np.int64) % 200).astype(np.int32)
+        v = (np.arange(n) % 10).astype(np.int32)
+        dk, dv = dev(k), dev(v)
+        thrust_amd.inclusive_scan_by_key(dk, dv, out=dk)
+        assert same_bits(host(dk), oracle.scan_by_key(k, v)), mean
+        assert same_bits(host(dv), v)
+        dk, dv = dev(k), dev(v)
+        thrust_amd.exclusive_scan_by_key(dk, dv, out=dk, init=3)
+        assert same_bits(host(dk), oracle.scan_by_key(k, v, exclusive=True, init=3)), mean
+        rk, rv = oracle.reduce_by_key(k, v)
+        dk, dv = dev(k), dev(v)
+        gk, gv = thrust_amd.reduce_by_key(dk, dv, keys_out=dk, values_out=dv)  # both in place
+        assert same_bits(host(gk), rk) and same_bits(host(gv), rv), mean
+        dk, dv, spare = dev(k), dev(v), dev(np.zeros(n, np.int32))
+        gk, gv = thrust_amd.reduce_by_key(dk, dv, keys_out=spare, values_out=dk)  # the values over the keys
+        assert same_bits(host(gk), rk) and same_bits(host(gv), rv), mean
+
+
 def piecewise_keys(seed, n, kd):
     """Stretches of very different run lengths side by side: none (one long run), 1 in 1000, 1 in 10,
     just below and just above every second element, every element.  A wavefront of a tile handles

