@@ -20,6 +20,11 @@ template <class T> struct bit_or;
 template <class T> struct bit_and;
 template <class T> struct bit_xor;
 
+// thrust::integral_constant, true_type, false_type (thrust/detail/type_traits.h:37-63): the standard ones
+using std::integral_constant;
+using std::true_type;
+using std::false_type;
+
 namespace detail {
 using std::integral_constant;
 using std::true_type;
@@ -62,6 +67,10 @@ template <class T> struct is_device_reference : std::false_type {};
 template <class T> struct is_device_reference<device_reference<T>> : std::true_type {};
 template <class T> struct is_reference_to_const : std::false_type {};
 template <class T> struct is_reference_to_const<const T&> : std::true_type {};
+// a reference through which a functor's result can be stored (thrust/detail/type_traits.h: user
+// code specialises it for proxy references of its own, testing/copy.cu:737-744)
+template <class T> struct is_non_const_reference
+    : std::integral_constant<bool, std::is_lvalue_reference<T>::value && !is_reference_to_const<T>::value> {};
 template <class T> struct add_reference { typedef typename std::add_lvalue_reference<T>::type type; };
 
 template <class A, class B> struct lazy_is_same : std::is_same<typename A::type, typename B::type> {};

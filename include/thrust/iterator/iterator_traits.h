@@ -4,12 +4,14 @@
 #include <iterator>
 #include <thrust/device_ptr.h>
 namespace thrust {
-template <class It> using iterator_traits = std::iterator_traits<It>;
-template <class It> struct iterator_value { typedef typename std::iterator_traits<It>::value_type type; };
-template <class It> struct iterator_pointer { typedef typename std::iterator_traits<It>::pointer type; };
-template <class It> struct iterator_difference { typedef typename std::iterator_traits<It>::difference_type type; };
-template <class It> struct iterator_reference { typedef typename std::iterator_traits<It>::reference type; };
-template <class It> struct iterator_traversal { typedef typename std::iterator_traits<It>::iterator_category type; };
+// A class template of its own, so that user code can specialise it for an iterator of theirs
+// (testing/scan.cu:649-656 does, for an output-only iterator); unspecialised it is the standard one.
+template <class It> struct iterator_traits : std::iterator_traits<It> {};
+template <class It> struct iterator_value { typedef typename iterator_traits<It>::value_type type; };
+template <class It> struct iterator_pointer { typedef typename iterator_traits<It>::pointer type; };
+template <class It> struct iterator_difference { typedef typename iterator_traits<It>::difference_type type; };
+template <class It> struct iterator_reference { typedef typename iterator_traits<It>::reference type; };
+template <class It> struct iterator_traversal { typedef typename iterator_traits<It>::iterator_category type; };
 template <class It> using iterator_value_t = typename iterator_value<It>::type;
 template <class It> using iterator_pointer_t = typename iterator_pointer<It>::type;
 template <class It> using iterator_difference_t = typename iterator_difference<It>::type;

@@ -117,7 +117,7 @@ REF_TESTING = "/root/reference/testing"
 # tests/emu/Makefile's ref_tests); THRUST_CDNA4_EMULATE_ALL=1 runs every file that compiles.
 REF_DEFAULT = ["sort", "sort_by_key", "stable_sort", "stable_sort_by_key", "sort_variable_bits", "sort_by_key_variable_bits",
                "stable_sort_large", "stable_sort_by_key_large_keys", "stable_sort_by_key_large_values",
-               "stable_sort_by_key_large_keys_and_values", "sort_permutation_iterator", "scan_by_key.inclusive",
+               "stable_sort_by_key_large_keys_and_values", "sort_permutation_iterator", "scan", "copy", "scan_by_key.inclusive",
                "scan_by_key.exclusive", "reduce_by_key", "transform_scan", "pair_scan", "pair_scan_by_key", "pair_sort",
                "pair_sort_by_key", "tuple_scan", "tuple_sort", "zip_iterator_scan", "zip_iterator_sort", "zip_iterator_sort_by_key",
                "zip_iterator_reduce_by_key", "transform_output_iterator_reduce_by_key"]
