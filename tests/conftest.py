@@ -42,11 +42,78 @@ def _enter_emulated_session():
     emu.emu_set_resident_workgroups(int(k), int(seed or 1))
     gpu_util.DEVICE = "cpu"
     gpu_util.dev = lambda a: torch.from_numpy(np.array(a, copy=True, order="C"))
+    if os.environ.get("THRUST_CDNA4_EMULATED_GUARD") == "1":
+        _guard_device_memory(gpu_util, api, torch)
     gpu_util.host = lambda t: t.numpy().copy()
     gpu_util.stream_handle = lambda: ctypes.c_void_p(0)
     gpu_util.synchronize = lambda: None
     gpu_util.empty_cache = lambda: None
     gpu_util.memory_allocated = lambda: 0
+
+
+def _guard_device_memory(gpu_util, api, torch):
+    """THRUST_CDNA4_EMULATED_GUARD=1: every "device" buffer of the session — inputs, outputs, the
+    temporary storage — ends exactly where an inaccessible page begins, and another one lies before
+    the page it starts in.  A kernel that reads or writes one byte past the end of a range it was
+    given ends the session with a segmentation fault in the test that made the call.  (The buffers
+    are then aligned to their element size only, like a view that starts inside an allocation.)"""
+    import ctypes
+    import mmap
+    import weakref
+
+    libc = ctypes.CDLL(None, use_errno=True)
+    libc.mmap.restype = ctypes.c_void_p
+    libc.mmap.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_long]
+    libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    libc.munmap.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    page = mmap.PAGESIZE
+
+    def guarded(shape, dtype):
+        dtype = np.dtype(dtype)
+        nbytes = int(np.prod(shape, dtype=np.int64)) * dtype.itemsize
+        body = max(page, -(-nbytes // page) * page)
+        total = body + 2 * page
+        base = libc.mmap(None, total, mmap.PROT_READ | mmap.PROT_WRITE, mmap.MAP_PRIVATE | mmap.MAP_ANONYMOUS, -1, 0)
+        assert base not in (None, ctypes.c_void_p(-1).value), ctypes.get_errno()
+        assert libc.mprotect(base, page, 0) == 0 and libc.mprotect(base + page + body, page, 0) == 0
+        raw = (ctypes.c_char * max(nbytes, 1)).from_address(base + page + body - max(nbytes, 1))
+        a = np.frombuffer(raw, dtype=dtype, count=int(np.prod(shape, dtype=np.int64))).reshape(shape)
+        weakref.finalize(raw, libc.munmap, base, total)  # the array keeps `raw` alive
+        return a
+
+    def dev(a):
+        a = np.asarray(a)
+        g = guarded(a.shape, a.dtype)
+        g[...] = a
+        return torch.from_numpy(g)
+
+    np_of = {torch.int8: np.int8, torch.uint8: np.uint8, torch.int16: np.int16, torch.int32: np.int32, torch.int64: np.int64,
+             torch.float32: np.float32, torch.float64: np.float64, torch.bool: np.bool_}
+    for name in ("uint16", "uint32", "uint64"):
+        if hasattr(torch, name):
+            np_of[getattr(torch, name)] = getattr(np, name)
+
+    class GuardedTorch:
+        """the allocations of thrust_amd.api, guarded; everything else is torch"""
+        def __getattr__(self, name):
+            return getattr(torch, name)
+
+        @staticmethod
+        def empty(size, dtype=torch.float32, device=None):
+            return torch.from_numpy(guarded((int(size),) if np.isscalar(size) else tuple(size), np_of[dtype]))
+
+        @staticmethod
+        def zeros(size, dtype=torch.float32, device=None):
+            t = GuardedTorch.empty(size, dtype)
+            t.zero_()
+            return t
+
+        @staticmethod
+        def empty_like(t):
+            return torch.from_numpy(guarded(tuple(t.shape), np_of[t.dtype]))
+
+    gpu_util.dev = dev
+    api.torch = GuardedTorch()
 
 
 def pytest_configure(config):
