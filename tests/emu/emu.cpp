@@ -68,6 +68,32 @@ emu_switch:
 .size emu_switch, .-emu_switch
 )");
 
+// ---- race detection (a build with -fsanitize=thread) ----
+// ThreadSanitizer sees every WAVEFRONT of the running workgroup as a thread of its own (a "fiber" of
+// its interface; the lanes of a wavefront share it, so accesses inside a wavefront are ordered as
+// the hardware orders them, by program order).  Switching between lanes tells it nothing
+// (no_sync); the only happens-before edges are the ones the kernel itself creates: a workgroup
+// barrier, the start and the end of a workgroup (a launch orders everything before it and after
+// it), and atomics, which the emulator performs as real atomic operations.  Two wavefronts that
+// touch the same LDS or global location without a barrier between them are then a reported race,
+// whatever order the emulator happened to run them in.
+// (This file itself is compiled WITHOUT the sanitizer, with -DEMU_TSAN: the scheduler's own
+// bookkeeping is no part of what is checked, and the atomics it performs for the lanes need no
+// report.  Only the calls into the sanitizer's fiber interface are made from here.)
+#if defined(EMU_TSAN)
+extern "C" {
+void* __tsan_get_current_fiber(void);
+void* __tsan_create_fiber(unsigned flags);
+void __tsan_destroy_fiber(void* fiber);
+void __tsan_switch_to_fiber(void* fiber, unsigned flags);
+void __tsan_acquire(void* addr);
+void __tsan_release(void* addr);
+}
+#define EMU_TSAN_ONLY(...) __VA_ARGS__
+#else
+#define EMU_TSAN_ONLY(...)
+#endif
+
 namespace emu {
 
 enum Op : int {
@@ -123,6 +149,7 @@ static uint64_t g_clock = 0;
 static int g_order = 0;          // 0 launch order, 1 reversed, 2 shuffled
 static uint64_t g_order_seed = 1;
 static int g_resident = 1;       // workgroups in flight
+static bool g_resident_set = false;
 static uint64_t g_resident_seed = 1;
 
 // the turn among the threads of a launch with several workgroups in flight
@@ -167,12 +194,25 @@ LaneView& view() { return g_cur ? g_cur->view : g_host_view; }
 int lane() { return (int)(g_cur - g_lanes) % kWave; }
 uint64_t clock() { return g_clock += 100; }
 
+#if defined(EMU_TSAN)
+constexpr unsigned kNoSync = 1u;  // __tsan_switch_to_fiber_no_sync
+static thread_local void* g_sched_fiber = nullptr;
+static thread_local void* g_wave_fiber[kMaxLanes / kWave];
+// addresses that stand for the orderings: a barrier; the start of a workgroup (released by the
+// scheduler, acquired by every lane); its end (released by every lane, acquired by the scheduler)
+static thread_local char g_barrier_token, g_start_token, g_end_token;
+static void* fiber_of(const Lane* l) { return g_wave_fiber[(l - g_lanes) / kWave]; }
+#endif
+
 static void park(int op, const void* site, const void* frame) {
   Lane* me = g_cur;
   me->op = op;
   me->site = site;
   me->depth = static_cast<const char*>(me->stack_top) - static_cast<const char*>(frame);
+  EMU_TSAN_ONLY(if (op == kWorkgroupBarrier) __tsan_release(&g_barrier_token);)
+  EMU_TSAN_ONLY(__tsan_switch_to_fiber(g_sched_fiber, kNoSync);)
   emu_switch(&me->sp, g_sched_sp);
+  EMU_TSAN_ONLY(if (op == kWorkgroupBarrier) __tsan_acquire(&g_barrier_token);)
 }
 
 #define EMU_SITE __builtin_extract_return_addr(__builtin_return_address(0)), __builtin_frame_address(0)
@@ -286,6 +326,7 @@ static int dpp_source(int l, int ctrl) {  // source lane of lane l, or -1 when t
 static void serve(Lane* w, int nl, int op, const void* site, long depth) {
   bool in[kWave];
   for (int l = 0; l < kWave; l++) in[l] = l < nl && w[l].op == op && w[l].site == site && w[l].depth == depth;
+  EMU_TSAN_ONLY(__tsan_switch_to_fiber(fiber_of(w), kNoSync);)  // the memory operations below are the wavefront's
   switch (op) {
     case kDpp:
       for (int l = 0; l < kWave; l++) {
@@ -341,17 +382,13 @@ static void serve(Lane* w, int nl, int op, const void* site, long depth) {
     case kAtomicAdd32:
       for (int l = 0; l < kWave; l++) {
         if (!in[l]) continue;
-        uint32_t* p = static_cast<uint32_t*>(w[l].ptr);
-        w[l].result = *p;
-        *p += (uint32_t)w[l].val;
+        w[l].result = __atomic_fetch_add(static_cast<uint32_t*>(w[l].ptr), (uint32_t)w[l].val, __ATOMIC_RELAXED);
       }
       break;
     case kAtomicAdd64:
       for (int l = 0; l < kWave; l++) {
         if (!in[l]) continue;
-        uint64_t* p = static_cast<uint64_t*>(w[l].ptr);
-        w[l].result = *p;
-        *p += w[l].val;
+        w[l].result = __atomic_fetch_add(static_cast<uint64_t*>(w[l].ptr), w[l].val, __ATOMIC_RELAXED);
       }
       break;
     case kLoad:
@@ -368,26 +405,29 @@ static void serve(Lane* w, int nl, int op, const void* site, long depth) {
     case kAtomicOr32:
       for (int l = 0; l < kWave; l++) {
         if (!in[l]) continue;
-        uint32_t* p = static_cast<uint32_t*>(w[l].ptr);
-        w[l].result = *p;
-        *p |= (uint32_t)w[l].val;
+        w[l].result = __atomic_fetch_or(static_cast<uint32_t*>(w[l].ptr), (uint32_t)w[l].val, __ATOMIC_RELAXED);
       }
       break;
   }
+  EMU_TSAN_ONLY(__tsan_switch_to_fiber(g_sched_fiber, kNoSync);)
   for (int l = 0; l < kWave; l++)
     if (in[l]) w[l].op = kRun;
 }
 
 extern "C" void emu_lane_main() {
+  EMU_TSAN_ONLY(__tsan_acquire(&g_start_token);)  // everything before the launch happened before this lane
   g_trampoline(g_closure);
   Lane* me = g_cur;
   me->op = kDone;
+  EMU_TSAN_ONLY(__tsan_release(&g_end_token);)
+  EMU_TSAN_ONLY(__tsan_switch_to_fiber(g_sched_fiber, kNoSync);)
   emu_switch(&me->sp, g_sched_sp);
   abort();  // a finished lane is never resumed
 }
 
 static void run_lane(Lane* l) {
   g_cur = l;
+  EMU_TSAN_ONLY(__tsan_switch_to_fiber(fiber_of(l), kNoSync);)
   emu_switch(&g_sched_sp, l->sp);
   g_cur = nullptr;
 }
@@ -401,6 +441,11 @@ static void run_workgroup(dim3 grid, dim3 block, unsigned bx, unsigned by, unsig
   }
   const int nthreads = (int)(block.x * block.y * block.z);
   const int nwaves = (nthreads + kWave - 1) / kWave;
+#if defined(EMU_TSAN)
+  g_sched_fiber = __tsan_get_current_fiber();
+  for (int wv = 0; wv < nwaves; wv++) g_wave_fiber[wv] = __tsan_create_fiber(0);
+  __tsan_release(&g_start_token);
+#endif
   for (int t = 0; t < nthreads; t++) {
     Lane& l = g_lanes[t];
     l = Lane();
@@ -463,6 +508,10 @@ static void run_workgroup(dim3 grid, dim3 block, unsigned bx, unsigned by, unsig
       for (int t = 0; t < nthreads; t++)
         if (g_lanes[t].op == kWorkgroupBarrier) g_lanes[t].op = kRun;
   }
+#if defined(EMU_TSAN)
+  __tsan_acquire(&g_end_token);  // what the workgroup did happened before whatever follows the launch
+  for (int wv = 0; wv < nwaves; wv++) __tsan_destroy_fiber(g_wave_fiber[wv]);
+#endif
 }
 
 void launch(dim3 grid, dim3 block, void (*trampoline)(void*), void* closure) {
@@ -488,6 +537,17 @@ void launch(dim3 grid, dim3 block, void (*trampoline)(void*), void* closure) {
     run_workgroup(grid, block, (unsigned)(b % grid.x), (unsigned)((b / grid.x) % grid.y), (unsigned)(b / ((uint64_t)grid.x * grid.y)));
     g_workgroups++;
   };
+  // programs that do not call emu_set_resident_workgroups (the C++ tests) take it from the environment
+  static const bool from_environment = [] {
+    const char* e = getenv("THRUST_CDNA4_EMULATED_RESIDENT");  // "k" or "k:seed"
+    if (e && !g_resident_set) {
+      g_resident = std::max(1, std::min(64, atoi(e)));
+      const char* colon = strchr(e, ':');
+      g_resident_seed = colon && atoll(colon + 1) ? (uint64_t)atoll(colon + 1) : 1;
+    }
+    return true;
+  }();
+  (void)from_environment;
   const int k = (int)std::min<uint64_t>((uint64_t)g_resident, total);
   if (k <= 1) {
     for (uint64_t i = 0; i < total; i++) run(i);
@@ -567,6 +627,7 @@ void emu_set_workgroup_order(int order, uint64_t seed) {
 // that chooses which of them runs next.
 void emu_set_resident_workgroups(int k, uint64_t seed) {
   emu::g_resident = k < 1 ? 1 : (k > 64 ? 64 : k);
+  emu::g_resident_set = true;
   emu::g_resident_seed = seed ? seed : 1;
 }
 uint64_t emu_turns_passed() { return emu::g_turns_passed; }

@@ -169,3 +169,41 @@ def test_reference_unit_tests_on_the_emulated_library(emulated_library):
     ran = sum(count for _, count, _, _ in results)
     assert ran >= (1200 if ALL else 110), ran
     print(f"{ran} tests of {len(names)} reference files")
+
+
+@pytest.mark.skipif(not ALL, reason="builds the library once more under ThreadSanitizer: THRUST_CDNA4_EMULATE_ALL=1")
+def test_no_data_race_between_wavefronts(emulated_library):
+    """The race-detecting build (tests/emu/Makefile, tsan): ThreadSanitizer sees every wavefront as a
+    thread, workgroup barriers (and the ends of a launch) as the only ordering between them, and the
+    workgroups in flight as threads of the process.  A missing barrier around an LDS exchange, or one
+    workgroup reading what another is still writing, is a reported data race.  The self-test shows that
+    such races ARE reported; then the scan, by-key and sort tests of tests/cpp must run clean."""
+    r = subprocess.run(["make", "-C", EMU_DIR, "-j8", "tsan"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    tsan = os.path.join(EMU_DIR, "build", "tsan")
+
+    def reports(args, resident="1"):
+        env = dict(os.environ, TSAN_OPTIONS="halt_on_error=0", THRUST_CDNA4_EMULATED_RESIDENT=resident)
+        p = subprocess.run([os.path.join(tsan, "selftest_race")] + args, env=env, capture_output=True, text=True, timeout=300)
+        return (p.stdout + p.stderr).count("WARNING: ThreadSanitizer: data race")
+
+    assert reports(["with_barrier"]) == 0
+    assert reports(["without_barrier"]) >= 1
+    assert reports(["global"]) >= 1
+    assert sum(reports(["across_workgroups"], f"2:{seed}") for seed in range(1, 9)) >= 1
+
+    from concurrent.futures import ThreadPoolExecutor
+
+    typed = "<int8_t>,<uint8_t>,<int16_t>,<uint16_t>,<uint32_t>,<uint64_t>,<float>,<short>"
+
+    def clean(case):
+        name, resident = case
+        env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1", THRUST_CDNA4_EMULATED_RESIDENT=resident, THRUST_CDNA4_TEST_SKIP=typed)
+        p = subprocess.run([os.path.join(tsan, name)], env=env, capture_output=True, text=True, timeout=3000)
+        out = p.stdout + p.stderr
+        return case, p.returncode == 0 and "ThreadSanitizer" not in out and ", 0 failed" in out, out[-4000:]
+
+    cases = [(name, resident) for resident in ("1", "4:9") for name in ("test_scan", "test_by_key", "test_sort")]
+    with ThreadPoolExecutor(int(WORKERS)) as pool:
+        bad = [(case, out) for case, ok, out in pool.map(clean, cases) if not ok]
+    assert not bad, bad
