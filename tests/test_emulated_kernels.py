@@ -194,7 +194,8 @@ def test_no_data_race_between_wavefronts(emulated_library):
 
     from concurrent.futures import ThreadPoolExecutor
 
-    typed = "<int8_t>,<uint8_t>,<int16_t>,<uint16_t>,<uint32_t>,<uint64_t>,<float>,<short>"
+    typed = ("BigIndexes,Repeatable,Large,VectorSearch,FindMismatch,Shuffle,"
+             "<int8_t>,<uint8_t>,<int16_t>,<uint16_t>,<uint32_t>,<uint64_t>,<float>,<short>")
 
     def clean(case):
         name, resident = case
@@ -203,7 +204,10 @@ def test_no_data_race_between_wavefronts(emulated_library):
         out = p.stdout + p.stderr
         return case, p.returncode == 0 and "ThreadSanitizer" not in out and ", 0 failed" in out, out[-4000:]
 
-    cases = [(name, resident) for resident in ("1", "4:9") for name in ("test_scan", "test_by_key", "test_sort")]
+    # the hot path's kernels, then the header layer's own (user operators, select, partition, merge sort, merge / set operations)
+    names = ["test_scan", "test_by_key", "test_sort", "test_scan_generic", "test_select", "test_partition", "test_merge_sort",
+             "test_merge_set", "test_generic", "test_algorithms", "test_seq"]
+    cases = [(name, resident) for resident in ("1", "4:9") for name in names]
     with ThreadPoolExecutor(int(WORKERS)) as pool:
         bad = [(case, out) for case, ok, out in pool.map(clean, cases) if not ok]
     assert not bad, bad
