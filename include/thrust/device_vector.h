@@ -44,7 +44,8 @@ class device_vector {
   explicit device_vector(const Alloc& alloc) : p_(nullptr), n_(0), cap_(0), alloc_(alloc) {}
   device_vector(size_type n, const T& v, const Alloc& alloc) : device_vector(alloc) { assign(n, v); }
   allocator_type get_allocator() const { return alloc_; }
-  explicit device_vector(size_type n) : device_vector() { resize(n); }
+  // (an allocator with a construct() of its own constructs the elements, thrust/detail/allocator_construct.h)
+  explicit device_vector(size_type n) : device_vector() { resize(n); construct_default(0, n_); }
   device_vector(size_type n, const T& v) : device_vector() { assign(n, v); }
   device_vector(const device_vector& o) : device_vector(o.alloc_) { assign_device(o.p_, o.n_); }
   device_vector(device_vector&& o) noexcept : p_(o.p_), n_(o.n_), cap_(o.cap_), alloc_(o.alloc_) { o.p_ = nullptr; o.n_ = o.cap_ = 0; }
@@ -55,11 +56,11 @@ class device_vector {
   device_vector(const device_vector& o, const Alloc& alloc) : device_vector(alloc) { assign_device(o.p_, o.n_); }
   device_vector(std::initializer_list<T> il, const Alloc& alloc) : device_vector(alloc) { assign_host(il.begin(), il.size()); }
   template <class It, class = typename std::iterator_traits<It>::iterator_category>
-  device_vector(It first, It last, const Alloc& alloc) : device_vector(alloc) { assign(first, last); }
-  device_vector(size_type n, const Alloc& alloc) : device_vector(alloc) { resize(n); }
+  device_vector(It first, It last, const Alloc& alloc) : device_vector(alloc) { assign(first, last); construct_copies(first); }
+  device_vector(size_type n, const Alloc& alloc) : device_vector(alloc) { resize(n); construct_default(0, n_); }
   device_vector(std::initializer_list<T> il) : device_vector() { assign_host(il.begin(), il.size()); }
   template <class It, class = typename std::iterator_traits<It>::iterator_category>
-  device_vector(It first, It last) : device_vector() { assign(first, last); }
+  device_vector(It first, It last) : device_vector() { assign(first, last); construct_copies(first); }
   ~device_vector() { release(); }
 
   device_vector& operator=(const device_vector& o) { if (this != &o) assign_device(o.p_, o.n_); return *this; }
@@ -171,6 +172,10 @@ class device_vector {
 
 
  private:
+  // the allocator's own construct(), where it has one: defined after the class, in allocator_construct.h
+  void construct_default(size_type at, size_type count);
+  template <class U> void construct_copies(device_ptr<U> from);
+  template <class It> void construct_copies(It) {}  // a range outside device memory: the bytes are the copy
   static void check(int rc, const char* what) { system::cdna4::detail::throw_on_error(rc, what); }
   static void sync() { check(thrust_cdna4_stream_synchronize(nullptr), "device_vector: synchronize"); }
   void release() { if (p_) alloc_.deallocate(typename Alloc::pointer(p_), cap_); p_ = nullptr; n_ = cap_ = 0; }
@@ -242,3 +247,11 @@ template <class T, class A> void swap(device_vector<T, A>& a, device_vector<T, A
 }  // namespace thrust
 
 #include <thrust/detail/vector_common.h>
+#include <thrust/detail/allocator_construct.h>
+namespace thrust {
+template <class T, class Alloc>
+void device_vector<T, Alloc>::construct_default(size_type at, size_type count) { detail::allocator_default_construct(alloc_, p_ + at, count); }
+template <class T, class Alloc>
+template <class U>
+void device_vector<T, Alloc>::construct_copies(device_ptr<U> from) { detail::allocator_copy_construct(alloc_, p_, static_cast<const U*>(from.get()), n_); }
+}  // namespace thrust

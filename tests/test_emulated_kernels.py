@@ -131,8 +131,6 @@ REF_FILES_LEFT_OUT = {
 }
 REF_TESTS_LEFT_OUT = {
     "WithBigIndexes": "2^30 to 2^33 elements: hours of emulation",
-    "TestAllocatorCustomDefaultConstruct": "device_vector does not call an allocator's own construct() (a gap of the vector, recorded)",
-    "TestAllocatorCustomCopyConstruct": "device_vector does not call an allocator's own construct() (a gap of the vector, recorded)",
 }
 
 
