@@ -209,3 +209,28 @@ def test_no_data_race_between_wavefronts(emulated_library):
     with ThreadPoolExecutor(int(WORKERS)) as pool:
         bad = [(case, out) for case, ok, out in pool.map(clean, cases) if not ok]
     assert not bad, bad
+
+
+@pytest.mark.skipif(not os.path.isdir("/root/reference/examples"), reason="needs the reference tree")
+def test_reference_examples_on_the_emulated_library(emulated_library):
+    """The reference's 51 example programs, compiled unchanged (tests/emu/Makefile, ref_examples): their
+    output must satisfy the golden outputs the reference keeps for them, as it must on the GPU
+    (tests/test_reference_examples.py, whose matcher and golden data this uses)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from test_reference_examples import EXAMPLES, GOLDEN, filecheck
+
+    r = subprocess.run(["make", "-C", EMU_DIR, "-j8", "ref_examples"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+
+    def run(name):
+        p = subprocess.run([os.path.join(EMU_DIR, "build", "examples", name)], capture_output=True, text=True, timeout=900)
+        if p.returncode != 0:
+            return name, "exit code %d\n%s" % (p.returncode, (p.stdout + p.stderr)[-1500:])
+        return name, filecheck(p.stdout, GOLDEN[name]["checks"])
+
+    with ThreadPoolExecutor(int(WORKERS)) as pool:
+        problems = [(name, why) for name, why in pool.map(run, EXAMPLES) if why is not None]
+    assert not problems, problems
+    assert len(EXAMPLES) == 51
