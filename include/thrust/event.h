@@ -144,6 +144,8 @@ class device_future : public device_event {
  public:
   typedef T value_type;
   device_future() : data_(nullptr), have_(false) {}
+  // a stream of its own and no content yet (thrust/system/cuda/detail/future.inl: unique_eager_future(new_stream))
+  explicit device_future(new_stream_t) : device_event(new_stream), data_(nullptr), have_(false) {}
   // the signal keeps the storage alive; data points into it
   device_future(std::shared_ptr<system::cdna4::detail::async_signal> s, T* data) : device_event(std::move(s)), data_(data), have_(false) {}
   device_future(device_future&&) = default;
@@ -152,7 +154,7 @@ class device_future : public device_event {
   // waits for the work, reads the value back (once) and returns it
   T get() {
     if (!have_) {
-      if (!data_) throw event_error(signal_ ? event_errc::no_content : event_errc::no_state);
+      if (!data_) throw event_error(event_errc::no_content);  // with or without a stream (testing/future.cu:77-88)
       wait();
       system::cdna4::detail::throw_on_error(thrust_cdna4_read_back(&value_, data_, sizeof(T), stream()), "future: read back");
       have_ = true;

@@ -58,6 +58,15 @@ struct dim3 {
   dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
 };
 
+// the small vector types of the HIP headers that test programs name
+struct float2 { float x, y; };
+struct float4 { float x, y, z, w; };
+struct double2 { double x, y; };
+struct int2 { int x, y; };
+struct uint2 { unsigned x, y; };
+inline float2 make_float2(float x, float y) { return float2{x, y}; }
+inline int2 make_int2(int x, int y) { return int2{x, y}; }
+
 namespace emu {
 struct Index3 { unsigned x, y, z; };
 struct LaneView {  // what the running lane reads through threadIdx & co.
