@@ -3,6 +3,7 @@
 // type, any device iterator to a device range otherwise.  A host range must stay alive and
 // untouched until the event is ready.
 #pragma once
+#include <algorithm>
 #include <thrust/copy.h>
 #include <thrust/event.h>
 
@@ -51,6 +52,40 @@ device_event copy(const Policy& exec, device_ptr<T> first, device_ptr<T> last, O
   if (n)
     system::cdna4::detail::throw_on_error(thrust_cdna4_memcpy_dtoh(&*out, first.get(), n * sizeof(T), signal->stream()), "async copy");
   return device_event(std::move(signal));
+}
+// host -> host: nothing to queue; the copy is done when the event is returned
+template <class Policy, class In, class Out, thrust::detail::enable_if_policy<Policy> = 0,
+          typename std::enable_if<!system::cdna4::detail::is_device_iterator<In>::value &&
+                                  !system::cdna4::detail::is_device_iterator<Out>::value, short>::type = 0>
+device_event copy(const Policy& exec, In first, In last, Out out) {
+  auto signal = system::cdna4::detail::make_signal(exec);
+  signal->wait();  // what the policy depends on
+  std::copy(first, last, out);
+  return device_event(std::move(signal));
+}
+// a device iterator that is no plain pointer (counting, transform, zip ...) -> host: the general
+// copy stages it; done when the event is returned
+template <class Policy, class In, class Out, thrust::detail::enable_if_policy<Policy> = 0,
+          typename std::enable_if<system::cdna4::detail::is_device_iterator<In>::value && !detail::is_device_ptr<In>::value &&
+                                  !system::cdna4::detail::is_device_iterator<Out>::value, char>::type = 0>
+device_event copy(const Policy& exec, In first, In last, Out out) {
+  auto signal = system::cdna4::detail::make_signal(exec);
+  signal->wait();  // what the policy depends on
+  thrust::copy(first, last, out);
+  return device_event(std::move(signal));
+}
+// a policy for the source and one for the destination (thrust/async/copy.h:96-130): the systems
+// are those of the iterators, which the overloads above tell apart
+namespace detail {
+// of the two policies the one that carries dependencies (thrust::device.after(...)) is the one to honour
+template <class From, class To>
+inline const To& policy_with_dependencies(const From&, const To& to, std::false_type) { return to; }
+template <class From, class To>
+inline const From& policy_with_dependencies(const From& from, const To&, std::true_type) { return from; }
+}  // namespace detail
+template <class From, class To, class In, class Out, thrust::detail::enable_if_policy<From> = 0, thrust::detail::enable_if_policy<To> = 0>
+device_event copy(const From& from, const To& to, In first, In last, Out out) {
+  return async::copy(detail::policy_with_dependencies(from, to, std::is_same<From, system::cdna4::detail::execute_after>()), first, last, out);
 }
 template <class In, class Out,
           typename std::enable_if<!thrust::detail::is_policy<In>::value, int>::type = 0>

@@ -186,27 +186,42 @@ typedef device_event device_unique_eager_event;
 template <class T> using device_unique_eager_future = device_future<T>;
 
 namespace system { namespace cdna4 { namespace detail {
-// thrust::device.after(events...): the next asynchronous algorithm starts after these
+// thrust::device.after(events...): the next asynchronous algorithm starts after these.  The events
+// are consumed — afterwards they have no stream (thrust/system/cuda/detail/future.inl: the policy
+// acquires the streams of its dependencies; testing/async_copy.cu:325-375) — and the algorithm
+// continues the first one's stream.  An event without a stream, or a policy used a second time,
+// is an event_error(no_state).
 struct execute_after : execution_policy<execute_after> {
-  std::vector<std::shared_ptr<async_signal>> deps;
+  struct state {
+    std::vector<std::shared_ptr<async_signal>> deps;
+    bool used = false;
+  };
+  std::shared_ptr<state> shared = std::make_shared<state>();  // copies of the policy are the same policy
 };
 inline void collect(execute_after&) {}
 template <class E, class... Es>
 void collect(execute_after& p, E&& e, Es&&... es) {
-  if (e.valid_stream()) p.deps.push_back(e.signal());
+  if (!e.valid_stream()) throw event_error(event_errc::no_state);
+  p.shared->deps.push_back(e.release_signal());
   collect(p, std::forward<Es>(es)...);
 }
-// a fresh signal whose stream waits for the dependencies and keeps them alive
+// the first dependency's signal, whose stream waits for the others and keeps them alive
 inline std::shared_ptr<async_signal> make_signal(const execute_after& p) {
-  auto s = std::make_shared<async_signal>();
-  for (const auto& d : p.deps) {
-    s->depend_on(*d);
-    s->keep_alive(d);
+  if (p.shared->used) throw event_error(event_errc::no_state);
+  p.shared->used = true;
+  if (p.shared->deps.empty()) return std::make_shared<async_signal>();
+  std::shared_ptr<async_signal> s = p.shared->deps[0];
+  for (std::size_t i = 1; i < p.shared->deps.size(); i++) {
+    s->depend_on(*p.shared->deps[i]);
+    s->keep_alive(p.shared->deps[i]);
   }
+  p.shared->deps.clear();
   return s;
 }
 inline std::shared_ptr<async_signal> make_signal(const par_t&) { return std::make_shared<async_signal>(); }
 inline std::shared_ptr<async_signal> make_signal(const par_nosync_t&) { return std::make_shared<async_signal>(); }
+// any other policy (the host system's, a user's): nothing to wait for
+template <class Policy> inline std::shared_ptr<async_signal> make_signal(const Policy&) { return std::make_shared<async_signal>(); }
 }}}  // namespace system::cdna4::detail
 
 namespace system { namespace cdna4 { namespace detail {

@@ -155,9 +155,13 @@ void TestAsyncDependencyChain() {
   const long long top = 2ll * (long long)(n - 1);
   ASSERT_EQUAL(f.get(), top * (long long)n);  // the running maximum of a descending range is its first element
   ASSERT_TRUE(f.ready());
+  // thrust::device.after(e) consumes e (testing/async_copy.cu:325-375): the chain ran on e0's stream
+  ASSERT_TRUE(!e0.valid_stream() && !e1.valid_stream() && !e2.valid_stream());
+  ASSERT_THROWS(thrust::device.after(e0), thrust::event_error);
   // an event moved from has no state; a default event neither
-  thrust::device_event moved = std::move(e0);
-  ASSERT_TRUE(!e0.valid_stream());
+  thrust::device_event fresh = thrust::when_all();
+  thrust::device_event moved = std::move(fresh);
+  ASSERT_TRUE(!fresh.valid_stream());
   ASSERT_TRUE(moved.valid_stream());
   thrust::device_event none;
   ASSERT_TRUE(!none.valid_stream() && !none.ready());
