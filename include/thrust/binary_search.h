@@ -47,13 +47,31 @@ std::ptrdiff_t scalar_search(const system::cpp::detail::par_t&, Hay first, Hay l
 // Without a comparator the elements and the values are compared as they are, by the transparent
 // less (thrust/system/detail/generic/binary_search.inl: `_1 < _2`), not converted to one type first.
 #define THRUST_CDNA4_SEARCH(NAME, MODE)                                                                                  \
-  template <class Policy, class Hay, class Needles, class Out, class Comp, detail::enable_if_policy<Policy> = 0>         \
-  Out NAME(const Policy& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out, Comp comp) {                 \
+  namespace system { namespace cdna4 {                                                                                  \
+  template <class D, class Hay, class Needles, class Out, class Comp>                                                    \
+  Out NAME(execution_policy<D>& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out, Comp comp) {          \
+    return thrust::detail::vector_search<MODE>(exec.derived(), first, last, vfirst, vlast, out, comp);                   \
+  }                                                                                                                      \
+  template <class D, class Hay, class Needles, class Out>                                                                \
+  Out NAME(execution_policy<D>& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out) {                     \
+    return NAME(exec, first, last, vfirst, vlast, out, thrust::less<>());                                                \
+  }                                                                                                                      \
+  }}                                                                                                                     \
+  template <class D, class Hay, class Needles, class Out, class Comp>                                                    \
+  Out NAME(const detail::execution_policy_base<D>& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out, Comp comp) { \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), first, last, vfirst, vlast, out, comp);                 \
+  }                                                                                                                      \
+  template <class D, class Hay, class Needles, class Out>                                                                \
+  Out NAME(const detail::execution_policy_base<D>& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out) {  \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), first, last, vfirst, vlast, out);                       \
+  }                                                                                                                      \
+  template <class Hay, class Needles, class Out, class Comp>                                                             \
+  Out NAME(const system::cpp::detail::par_t& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out, Comp comp) { \
     return detail::vector_search<MODE>(exec, first, last, vfirst, vlast, out, comp);                                     \
   }                                                                                                                      \
-  template <class Policy, class Hay, class Needles, class Out, detail::enable_if_policy<Policy> = 0>                     \
-  Out NAME(const Policy& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out) {                            \
-    return detail::vector_search<MODE>(exec, first, last, vfirst, vlast, out, less<>()); \
+  template <class Hay, class Needles, class Out>                                                                         \
+  Out NAME(const system::cpp::detail::par_t& exec, Hay first, Hay last, Needles vfirst, Needles vlast, Out out) {        \
+    return detail::vector_search<MODE>(exec, first, last, vfirst, vlast, out, less<>());                                 \
   }                                                                                                                      \
   template <class Hay, class Needles, class Out, detail::enable_if_device<Hay, Needles, Out> = 0,                                      \
             class = typename std::iterator_traits<Out>::iterator_category>                                               \

@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cstddef>
 #include <initializer_list>
+#include <memory>
 #include <vector>
 
 #include <thrust/device_allocator.h>
@@ -244,6 +245,19 @@ template <class T1, class A1, class T2, class A2>
 bool operator!=(const std::vector<T1, A1>& a, const device_vector<T2, A2>& b) { return !(a == b); }
 template <class T, class A> void swap(device_vector<T, A>& a, device_vector<T, A>& b) noexcept { a.swap(b); }
 
+}  // namespace thrust
+
+namespace thrust {
+namespace detail {
+// thrust::detail::vector_base<T, Alloc> (thrust/detail/vector_base.h) as generic code names it when it
+// derives a vector type from another vector's allocator (testing/binary_search_vector.cu:16-23): the
+// vector of the system the allocator's pointer belongs to.
+template <class T, class Alloc, class Pointer = typename std::allocator_traits<Alloc>::pointer>
+struct vector_base_of { typedef host_vector<T, Alloc> type; };
+template <class T, class Alloc, class U>
+struct vector_base_of<T, Alloc, device_ptr<U>> { typedef device_vector<T, Alloc> type; };
+template <class T, class Alloc> using vector_base = typename vector_base_of<T, Alloc>::type;
+}  // namespace detail
 }  // namespace thrust
 
 #include <thrust/detail/vector_common.h>
