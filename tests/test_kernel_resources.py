@@ -68,3 +68,17 @@ def test_hot_kernels_keep_four_wavefronts_per_simd():
             if u.get("VGPRs", 0) > 128:
                 over.append((name, u["VGPRs"]))
     assert not over, over[:10]
+
+
+def test_lds_fits_the_workgroups_per_compute_unit_the_kernels_are_sized_for():
+    # 160 KiB of LDS per compute unit: two 512-thread workgroups of the scan and by-key kernels, one
+    # workgroup of a onesweep pass (the tile's keys are staged whole)
+    over = []
+    for name, u in usage().items():
+        lds = u.get("LDS Size", 0)
+        if any(s in name for s in ["scan_by_key_kernel", "reduce_by_key_kernel", "scan_kernel", "scan_packed_kernel"]) and lds > 80 * 1024:
+            over.append((name, lds))
+        if lds > 160 * 1024:
+            over.append((name, lds))
+    assert not over, over[:10]
+    assert any(u.get("LDS Size", 0) > 60 * 1024 for u in usage().values())  # the report is being read
