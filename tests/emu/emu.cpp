@@ -43,6 +43,9 @@
 
 #include <hip/hip_runtime.h>
 
+#if !defined(__x86_64__) || !defined(__linux__)
+#error "the emulator's context switch is written for x86-64 Linux (System V calling convention)"
+#endif
 // ---- context switch: callee-saved registers on the fiber's own stack (SysV x86-64) ----
 extern "C" void emu_switch(void** save_sp, void* load_sp);
 asm(R"(

@@ -64,8 +64,17 @@ def run_session(files, resident="1", deselect=(), extra=(), guard=False):
     env = dict(os.environ, THRUST_CDNA4_EMULATED="1", THRUST_CDNA4_EMULATED_RESIDENT=resident,
                THRUST_CDNA4_EMULATED_GUARD="1" if guard else "0")
     env.pop("THRUST_CDNA4_LIB", None)
-    cmd = [sys.executable, "-X", "faulthandler", "-m", "pytest", "-m", "gpu", "-q", "-x", "-p", "no:cacheprovider", "-n", WORKERS,
-           "--timeout", "900", *files, *extra]
+    cmd = [sys.executable, "-X", "faulthandler", "-m", "pytest", "-m", "gpu", "-q", "-x", "-p", "no:cacheprovider", *files, *extra]
+    try:  # workers and a per-test time limit where the plugins are there
+        import xdist  # noqa: F401
+        cmd += ["-n", WORKERS]
+    except ImportError:
+        pass
+    try:
+        import pytest_timeout  # noqa: F401
+        cmd += ["--timeout", "900"]
+    except ImportError:
+        pass
     if not ALL:
         for d in deselect:
             cmd += ["--deselect", d]
