@@ -18,7 +18,15 @@
 #error "compile with -DTCD_KEY_BYTES=1|2|4|8"
 #endif
 
+#define TCD_CAT2(a, b) a##b
+#define TCD_CAT(a, b) TCD_CAT2(a, b)
+
 namespace tcd {
+// One namespace per key width.  This file is compiled four times into one library, and the key
+// type is a file-level alias, not a template argument: SegGeom<T>, SegTile<...> and the host
+// helpers below differ between the four objects under one name.  Inside a namespace of their
+// own no linker can fold a copy from one key width into another's.
+inline namespace TCD_CAT(keys_of_bytes_, TCD_KEY_BYTES) {
 
 template <int B> struct key_bits;
 template <> struct key_bits<1> { using type = uint8_t; };
@@ -642,9 +650,7 @@ static size_t bykey_temp_bytes(int64_t n) {
   return 256 + align_up((size_t)ntiles * TileDesc<SegPair<T, seg_restarts<T, Op>::value>>::kBytesPerTile, 256);
 }
 
-#define TCD_CAT2(a, b) a##b
-#define TCD_CAT(a, b) TCD_CAT2(a, b)
-
+}  // namespace keys_of_bytes_<width>
 }  // namespace tcd
 
 // Internal entry points, one pair per key width; the public C ABI in bykey_dispatch.hip
