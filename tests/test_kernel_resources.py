@@ -82,3 +82,21 @@ def test_lds_fits_the_workgroups_per_compute_unit_the_kernels_are_sized_for():
             over.append((name, lds))
     assert not over, over[:10]
     assert any(u.get("LDS Size", 0) > 60 * 1024 for u in usage().values())  # the report is being read
+
+
+def test_the_by_key_objects_of_the_four_key_widths_share_no_symbol():
+    """bykey.hip is compiled once per key width into one library, and the key type is a file-level
+    alias: a template of one name in two of the objects can differ in its body, and a linker keeps
+    one copy of a weak symbol.  A kernel's host stub folded like that makes every key width launch
+    one width's kernel.  Each build has a namespace of its own; nothing weak may be common to two
+    objects."""
+    usage()  # builds the objects where they are missing
+    weak = {}
+    for k in (1, 2, 4, 8):
+        out = subprocess.run(["nm", os.path.join(BUILD, "bykey_k%d.o" % k)], stdout=subprocess.PIPE, text=True, check=True).stdout
+        weak[k] = {line.split()[-1] for line in out.splitlines() if len(line.split()) == 3 and line.split()[1] in "WVu"}
+        assert len(weak[k]) >= 100, (k, len(weak[k]))  # the kernels' host stubs
+    for a in (1, 2, 4, 8):
+        for b in (1, 2, 4, 8):
+            if a < b:
+                assert not (weak[a] & weak[b]), (a, b, sorted(weak[a] & weak[b])[:5])
