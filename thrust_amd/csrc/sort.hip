@@ -98,15 +98,30 @@ struct RadixHistGeom {
   static constexpr int COPIES = 16384 / (P * kRadix) > 32 ? 32 : 16384 / (P * kRadix);
 };
 
+// The kernel also clears the tile descriptors of the passes that follow (`clear`, `clear_bytes`:
+// a multiple of 16).  Nothing reads them before the first pass starts, the stores need no answer
+// and go out under the key loads, and the clearing launch in front of this kernel is left with the
+// few KiB that must be zero before the first count arrives (status, histogram, tickets).
 template <class U, bool FLOAT>
 __global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const U* __restrict__ keys, int64_t n,
-                                                                  U xor_mask, uint32_t* ghist, int vec_ok) {
+                                                                  U xor_mask, uint32_t* ghist, int vec_ok,
+                                                                  void* clear, size_t clear_bytes) {
   constexpr int P = RadixHistGeom<U>::P;
   constexpr int COPIES = RadixHistGeom<U>::COPIES;
   constexpr int VEC = 16 / sizeof(U);
   constexpr int UNROLL = 8;  // 128-bit loads in flight per thread
   __shared__ uint32_t h[P * kRadix * COPIES];
   const int tid = threadIdx.x;
+  {
+    const size_t first = (size_t)blockIdx.x * kHistThreads + tid, step = (size_t)gridDim.x * kHistThreads;
+    if ((reinterpret_cast<uintptr_t>(clear) & 15u) == 0) {
+      tcd_v4u* c16 = static_cast<tcd_v4u*>(clear);
+      for (size_t i = first; i < clear_bytes / 16; i += step) c16[i] = tcd_v4u{0u, 0u, 0u, 0u};
+    } else {  // temporary storage that is not aligned as asked for: words
+      uint32_t* c4 = static_cast<uint32_t*>(clear);
+      for (size_t i = first; i < clear_bytes / 4; i += step) c4[i] = 0u;
+    }
+  }
   for (int i = tid; i < P * kRadix * COPIES; i += kHistThreads) h[i] = 0;
   __syncthreads();
 
@@ -825,7 +840,8 @@ constexpr int64_t small_sort_limit(int value_bytes) { return int64_t(1) << (21 +
 struct SortPlan {
   size_t status, keys_alt, vals_alt, hist, tickets, xcd, desc, total;
   int xcd_slots;  // groups an XCD may take in one pass
-  size_t zero_begin, zero_bytes;
+  size_t zero_begin, zero_bytes;  // cleared by a launch of its own before anything else
+  size_t desc_bytes;              // cleared by the histogram kernel
   int64_t ntiles;
 };
 
@@ -880,8 +896,10 @@ static SortPlan make_plan(int64_t n) {
   // per pass: a counter per XCD (a cache line each) and the numbers of the groups each XCD took
   p.xcd_slots = (int)ceil_div(p.ntiles, (int64_t)kXcds * kXcdGroup);
   p.xcd = off; off += kCounting ? 0 : align_up((size_t)P * xcd_words_per_pass(p.xcd_slots) * 4, 256);
-  p.desc = off; off += kCounting ? 0 : align_up((size_t)P * p.ntiles * kRadix * sizeof(D), 256);
   p.zero_bytes = off - p.zero_begin;
+  // the descriptors start at zero too: the histogram kernel clears them
+  p.desc = off; off += kCounting ? 0 : align_up((size_t)P * p.ntiles * kRadix * sizeof(D), 256);
+  p.desc_bytes = off - p.desc;
   p.keys_alt = off; off += kCounting ? 0 : align_up((size_t)n * sizeof(U), 256);
   p.vals_alt = off; off += align_up((size_t)n * VB, 256);
   p.total = off;
@@ -927,7 +945,7 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   const int cus = device_cu_count();
   if (hblocks > cus) hblocks = cus;  // one workgroup per CU, eight loads in flight per thread: 1 % of a 2^28 sort over two with two
   TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(kHistThreads), stream,
-             kbuf[0], n, xor_mask, ghist, vec_ok);
+             kbuf[0], n, xor_mask, ghist, vec_ok, static_cast<void*>(t + plan.desc), plan.desc_bytes);
   // passes over places where all keys agree are skipped on the device; with an even number of
   // places the passes that run are an even number too and the result ends in the caller's buffer
   constexpr int kSkipping = (P % 2 == 0) ? 1 : 0;
