@@ -2,8 +2,9 @@
 //
 //   1. radix_hist_kernel   one read of the keys; LDS-privatised 256-bin histograms of ALL
 //                          digit places (replicated per lane), merged into global memory
-//                          with atomics.
-//   2. radix_bins_kernel   exclusive scan of each digit place's 256 bins.
+//                          with atomics.  It also clears the passes' tile descriptors.
+//   2. radix_bins          exclusive scan of each digit place's 256 bins and the choice of the
+//                          passes that run, by the histogram kernel's last workgroup.
 //   3. onesweep_kernel     one launch per 8-bit digit.  A workgroup takes a tile by ticket,
 //                          ranks its keys stably (returning LDS atomics on per-wave digit
 //                          counters), publishes its 256 digit counts, finds the counts
@@ -84,7 +85,60 @@ __device__ __host__ inline U decode_key(U e, U xor_mask) {
 }
 
 // ---------------------------------------------------------------------------------------
-// 1. Histogram of every digit place
+// 2. Exclusive scan of the 256 bins of each digit place, and which passes run
+// ---------------------------------------------------------------------------------------
+// Run by ONE workgroup of at least 256 threads — the histogram kernel's workgroup that finishes
+// last (below) — for all P places; it then decides which passes run.  A place where every
+// key has the same digit is the identity permutation for a stable sort, so its pass is skipped
+// (64-bit keys that hold small numbers, keys with constant fields, all-equal keys).  The number of
+// passes that run is kept even, so that the result ends in the caller's buffer without a copy: if
+// an odd number of places need their pass, one of the skippable ones runs as well.  The decision
+// travels in the pass's ticket counter, which every workgroup of the pass reads anyway: the
+// counter starts at kPassSkipped for a pass that does not run and at kPassReadsAlt for one whose
+// input is the alternate buffer; the tile number is in the low bits.  With skipping off every
+// pass runs (places = 1: the caller copies the result back).
+// The counts are read with agent-scope loads: the other workgroups added them with agent-scope
+// atomics, possibly from another XCD, and this workgroup's L2 must not answer from an older line.
+constexpr uint32_t kPassSkipped = 0x80000000u, kPassReadsAlt = 0x40000000u, kTicketMask = 0x3FFFFFFFu;
+__device__ inline void radix_bins(uint32_t* ghist, int places, uint32_t n, uint32_t* tickets, int skipping) {
+  __shared__ uint32_t s_w[4];
+  __shared__ uint32_t s_same[8];  // places is at most 8
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const bool mine = tid < kRadix;  // thread d has digit d; the others only keep the barriers' count
+  if (tid < 8) s_same[tid] = 0;
+  for (int p = 0; p < places; p++) {
+    __syncthreads();
+    uint32_t* h = ghist + (size_t)p * kRadix;
+    const uint32_t c = mine ? ld_agent(&h[tid]) : 0u;
+    if (mine && c == n) s_same[p] = 1;  // all keys in one bin
+    uint32_t incl = wave_inclusive_scan(c, 0u, [](uint32_t a, uint32_t b) { return a + b; });
+    if (mine && lane == 63) s_w[wave] = incl;
+    __syncthreads();
+    uint32_t base = 0;
+    for (int w = 0; w < wave && w < 4; w++) base += s_w[w];
+    if (mine) h[tid] = base + incl - c;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int needed = 0;
+    for (int p = 0; p < places; p++) needed += s_same[p] ? 0 : 1;
+    bool one_more = skipping && (needed & 1);  // keep the number of passes even
+    uint32_t reads_alt = 0;
+    for (int p = 0; p < places; p++) {
+      bool runs = !skipping || !s_same[p];
+      if (!runs && one_more) {
+        runs = true;
+        one_more = false;
+      }
+      tickets[p] = runs ? reads_alt : kPassSkipped;
+      if (runs) reads_alt ^= kPassReadsAlt;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// 1. Histogram of every digit place (and, in its last workgroup, step 2)
 // ---------------------------------------------------------------------------------------
 // Counters are replicated per lane: the counter of (place, digit, copy) lives at word
 // (place*256 + digit)*COPIES + copy with copy = lane % COPIES, so the lanes of a wave spread
@@ -105,7 +159,8 @@ struct RadixHistGeom {
 template <class U, bool FLOAT>
 __global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const U* __restrict__ keys, int64_t n,
                                                                   U xor_mask, uint32_t* ghist, int vec_ok,
-                                                                  void* clear, size_t clear_bytes) {
+                                                                  void* clear, size_t clear_bytes,
+                                                                  uint32_t* tickets, uint32_t* done, int skipping) {
   constexpr int P = RadixHistGeom<U>::P;
   constexpr int COPIES = RadixHistGeom<U>::COPIES;
   constexpr int VEC = 16 / sizeof(U);
@@ -167,55 +222,17 @@ __global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const U* __res
     for (int r = 0; r < COPIES; r++) c += h[b * COPIES + ((r + b) & (COPIES - 1))];  // rotated: spread over banks
     if (c) atomicAdd(&ghist[b], c);
   }
-}
-
-// ---------------------------------------------------------------------------------------
-// 2. Exclusive scan of the 256 bins of each digit place (one workgroup per place)
-// ---------------------------------------------------------------------------------------
-// One workgroup handles all P places, and then decides which passes run.  A place where every
-// key has the same digit is the identity permutation for a stable sort, so its pass is skipped
-// (64-bit keys that hold small numbers, keys with constant fields, all-equal keys).  The number of
-// passes that run is kept even, so that the result ends in the caller's buffer without a copy: if
-// an odd number of places need their pass, one of the skippable ones runs as well.  The decision
-// travels in the pass's ticket counter, which every workgroup of the pass reads anyway: the
-// counter starts at kPassSkipped for a pass that does not run and at kPassReadsAlt for one whose
-// input is the alternate buffer; the tile number is in the low bits.  With skipping off every
-// pass runs (places = 1: the caller copies the result back).
-constexpr uint32_t kPassSkipped = 0x80000000u, kPassReadsAlt = 0x40000000u, kTicketMask = 0x3FFFFFFFu;
-__global__ __launch_bounds__(256) void radix_bins_kernel(uint32_t* ghist, int places, uint32_t n, uint32_t* tickets, int skipping) {
-  __shared__ uint32_t s_w[4];
-  __shared__ uint32_t s_same[8];  // places is at most 8
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  if (tid < 8) s_same[tid] = 0;
-  for (int p = 0; p < places; p++) {
-    __syncthreads();
-    uint32_t* h = ghist + (size_t)p * kRadix;
-    const uint32_t c = h[tid];
-    if (c == n) s_same[p] = 1;  // all keys in one bin
-    uint32_t incl = wave_inclusive_scan(c, 0u, [](uint32_t a, uint32_t b) { return a + b; });
-    if (lane == 63) s_w[wave] = incl;
-    __syncthreads();
-    uint32_t base = 0;
-    for (int w = 0; w < wave; w++) base += s_w[w];
-    h[tid] = base + incl - c;
-  }
+  // The workgroup that finishes last scans the bins: every thread's counts are out (fence) before
+  // its workgroup is counted as done, and the one that counts the last sees them all (fence).
+  // `done` starts at zero like the histogram.
+  __shared__ uint32_t s_last;
+  __threadfence();
   __syncthreads();
-  if (tid == 0) {
-    int needed = 0;
-    for (int p = 0; p < places; p++) needed += s_same[p] ? 0 : 1;
-    bool one_more = skipping && (needed & 1);  // keep the number of passes even
-    uint32_t reads_alt = 0;
-    for (int p = 0; p < places; p++) {
-      bool runs = !skipping || !s_same[p];
-      if (!runs && one_more) {
-        runs = true;
-        one_more = false;
-      }
-      tickets[p] = runs ? reads_alt : kPassSkipped;
-      if (runs) reads_alt ^= kPassReadsAlt;
-    }
-  }
+  if (tid == 0) s_last = atomicAdd(done, 1u) == gridDim.x - 1u ? 1u : 0u;
+  __syncthreads();
+  if (s_last == 0u) return;
+  __threadfence();
+  radix_bins(ghist, P, (uint32_t)n, tickets, skipping);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -317,7 +334,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(WPE))) vo
     for (int w = 0; w < NWAVES; w++) reinterpret_cast<uint32_t*>(sm.wave_cnt[w])[tid] = 0;
   }
   __syncthreads();
-  const uint32_t ticket_word = sm.tile;  // tile number, and what radix_bins_kernel decided about this pass
+  const uint32_t ticket_word = sm.tile;  // tile number, and what radix_bins decided about this pass
   if (ticket_word & kPassSkipped) return;  // every key has the same digit here
   const bool from_alt = (ticket_word & kPassReadsAlt) != 0;
   const U* __restrict__ kin = from_alt ? kalt : kmain;
@@ -878,6 +895,7 @@ __global__ __launch_bounds__(kFillThreads) void counting_fill_kernel(uint8_t* ou
   }
 }
 
+constexpr int kHistDoneWord = 8;  // in the 64 words of the ticket block
 constexpr size_t kSortStatusOffset = 0;  // of the status word in a sort call's temporary storage
 static std::atomic<uint32_t> g_test_spin_limit{kLookbackSpinLimit};  // test knob
 static constexpr size_t xcd_words_per_pass(int slots) { return (size_t)kXcds * kXcdCounterStride + (size_t)kXcds * (size_t)slots; }
@@ -892,7 +910,7 @@ static SortPlan make_plan(int64_t n) {
   p.zero_begin = off;
   p.status = off; off += 256;
   p.hist = off; off += align_up((size_t)P * kRadix * 4, 256);
-  p.tickets = off; off += 256;
+  p.tickets = off; off += 256;  // a counter per pass (at most 8), and the histogram kernel's count of finished workgroups
   // per pass: a counter per XCD (a cache line each) and the numbers of the groups each XCD took
   p.xcd_slots = (int)ceil_div(p.ntiles, (int64_t)kXcds * kXcdGroup);
   p.xcd = off; off += kCounting ? 0 : align_up((size_t)P * xcd_words_per_pass(p.xcd_slots) * 4, 256);
@@ -940,16 +958,16 @@ static hipError_t sort_with(void* temp, size_t* temp_bytes, void* keys, void* va
   hipError_t e = zero_async(t + plan.zero_begin, plan.zero_bytes, stream);
   if (e != hipSuccess) return e;
 
+  // passes over places where all keys agree are skipped on the device; with an even number of
+  // places the passes that run are an even number too and the result ends in the caller's buffer
+  constexpr int kSkipping = (P % 2 == 0) ? 1 : 0;
   const int vec_ok = (reinterpret_cast<uintptr_t>(keys) & (sizeof(U) - 1)) == 0;  // see load16
   int64_t hblocks = ceil_div(n, kHistThreads * 64);
   const int cus = device_cu_count();
   if (hblocks > cus) hblocks = cus;  // one workgroup per CU, eight loads in flight per thread: 1 % of a 2^28 sort over two with two
   TCD_LAUNCH("radix_hist_kernel", (radix_hist_kernel<U, FLOAT>), dim3((unsigned)hblocks), dim3(kHistThreads), stream,
-             kbuf[0], n, xor_mask, ghist, vec_ok, static_cast<void*>(t + plan.desc), plan.desc_bytes);
-  // passes over places where all keys agree are skipped on the device; with an even number of
-  // places the passes that run are an even number too and the result ends in the caller's buffer
-  constexpr int kSkipping = (P % 2 == 0) ? 1 : 0;
-  TCD_LAUNCH("radix_bins_kernel", radix_bins_kernel, dim3(1), dim3(256), stream, ghist, P, (uint32_t)n, tickets, kSkipping);
+             kbuf[0], n, xor_mask, ghist, vec_ok, static_cast<void*>(t + plan.desc), plan.desc_bytes,
+             tickets, tickets + kHistDoneWord, kSkipping);
   if constexpr (sizeof(U) == 1 && VB == 0) {
     int64_t fblocks = ceil_div(n, (int64_t)kFillThreads * 16 * 4);
     if (fblocks > (int64_t)cus * 8) fblocks = (int64_t)cus * 8;
