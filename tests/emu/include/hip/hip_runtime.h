@@ -242,6 +242,10 @@ inline unsigned emu_mbcnt_hi(unsigned mask, unsigned base) {
 #define __builtin_amdgcn_wave_barrier() ::emu::wave_barrier()
 #define __builtin_amdgcn_s_barrier() ::emu::workgroup_barrier()
 #define __builtin_amdgcn_fence(...) ((void)0)
+// workgroups in flight are OS threads: the device-wide fences are real ones
+#define __threadfence() __atomic_thread_fence(__ATOMIC_SEQ_CST)
+#define __threadfence_block() __atomic_thread_fence(__ATOMIC_SEQ_CST)
+#define __threadfence_system() __atomic_thread_fence(__ATOMIC_SEQ_CST)
 #define __builtin_amdgcn_s_sleep(n) ::emu::sleep()
 #define __builtin_amdgcn_s_setprio(n) ((void)0)
 #define __builtin_amdgcn_sched_barrier(n) ((void)0)
