@@ -11,7 +11,8 @@
  * its own device primitives (thrust/system/cuda/detail/sort.h:330-365,
  * scan.h:80-117, reduce_by_key.h:1012-1031): call once with `temp == NULL` and the entry
  * point only writes the number of bytes it needs to `*temp_bytes`; call again with a
- * device buffer of at least that many bytes (256-byte aligned) to run.  Data pointers need the
+ * device buffer of at least that many bytes (256-byte aligned; an address that is not even a
+ * multiple of 8 is refused with an invalid-value error) to run.  Data pointers need the
  * alignment of their element type and no more: a range that starts a few elements into an
  * allocation runs at the same speed as one that starts at it.
  *

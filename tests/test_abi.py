@@ -56,7 +56,7 @@ def test_size_queries_need_no_device():
     assert rc == 0
 
 
-@pytest.mark.parametrize("bad", ["dtype", "negative_n", "op", "value_bytes", "bins", "range"])
+@pytest.mark.parametrize("bad", ["dtype", "negative_n", "op", "value_bytes", "bins", "range", "temp_alignment"])
 def test_bad_arguments_return_an_error_code(bad):
     L = capi.lib()
     n = 100
@@ -68,6 +68,22 @@ def test_bad_arguments_return_an_error_code(bad):
         rc, _ = _size(L.thrust_cdna4_scan, capi.I32, 17, 0, None, None, n, None, None)
     elif bad == "value_bytes":
         rc, _ = _size(L.thrust_cdna4_sort_pairs, capi.U32, None, 3, None, n, 0, None)
+    elif bad == "temp_alignment":
+        # the descriptors in the temporary storage are 64-bit atoms: an address that would fault there
+        # is refused on the host.  Empty inputs, so that the accepted calls touch no device either.
+        import ctypes
+        nb = ctypes.c_size_t(1 << 20)
+
+        def calls(temp):
+            t = ctypes.c_void_p(temp)
+            return [L.thrust_cdna4_sort_keys(t, ctypes.byref(nb), capi.U32, None, 0, 0, None),
+                    L.thrust_cdna4_sort_pairs(t, ctypes.byref(nb), capi.U32, None, 4, None, 0, 0, None),
+                    L.thrust_cdna4_scan(t, ctypes.byref(nb), capi.I32, capi.PLUS, 0, None, None, 0, None, None),
+                    L.thrust_cdna4_scan_by_key(t, ctypes.byref(nb), capi.I32, capi.I32, capi.PLUS, 0, None, None, None, 0, None, None)]
+        assert calls(0x1000) == [0, 0, 0, 0]
+        assert calls(0x1004) == [1, 1, 1, 1]
+        rc = L.thrust_cdna4_reduce_by_key(ctypes.c_void_p(0x1004), ctypes.byref(nb), capi.I32, capi.I32, capi.PLUS,
+                                          None, None, None, None, ctypes.c_void_p(0x2000), 0, None)
     elif bad == "bins":
         rc, _ = _size(L.thrust_cdna4_histogram_even, capi.U8, None, n, None, 0, 0.0, 1.0, None)
     else:

@@ -20,7 +20,7 @@ static inline int is_float_dtype(int dt) { return dt == THRUST_CDNA4_F32 || dt =
 extern "C" int thrust_cdna4_scan_by_key(void* temp, size_t* temp_bytes, int key_dtype, int value_dtype,
                                         int op, int exclusive, const void* keys, const void* values,
                                         void* out, int64_t n, const void* init, void* stream) {
-  if (!temp_bytes || n < 0 || n > kByKeyMaxN || (n > 0 && temp && (!keys || !values || !out)))
+  if (!temp_bytes || n < 0 || n > kByKeyMaxN || tcd::temp_misaligned(temp) || (n > 0 && temp && (!keys || !values || !out)))
     return hipErrorInvalidValue;
   const int fk = is_float_dtype(key_dtype);
   switch (tcd::dtype_size(key_dtype)) {
@@ -36,7 +36,7 @@ extern "C" int thrust_cdna4_reduce_by_key(void* temp, size_t* temp_bytes, int ke
                                           int op, const void* keys_in, const void* values_in,
                                           void* keys_out, void* values_out, int64_t* num_runs_out,
                                           int64_t n, void* stream) {
-  if (!temp_bytes || n < 0 || n > kByKeyMaxN ||
+  if (!temp_bytes || n < 0 || n > kByKeyMaxN || tcd::temp_misaligned(temp) ||
       (temp && (!num_runs_out || (n > 0 && (!keys_in || !values_in || !keys_out || !values_out)))))
     return hipErrorInvalidValue;
   const int fk = is_float_dtype(key_dtype);

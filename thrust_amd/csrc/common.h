@@ -425,6 +425,10 @@ void profile_end(hipStream_t stream);
 // recorded into a HIP graph.
 __global__ void zero_words_kernel(uint32_t* p, size_t nwords);
 
+// The descriptors in a call's temporary storage are 64-bit atoms: an address that is not a multiple
+// of 8 would fault on the device, so such a call is refused on the host (the interface asks for 256).
+inline bool temp_misaligned(const void* temp) { return (reinterpret_cast<uintptr_t>(temp) & 7u) != 0; }
+
 hipError_t zero_async(void* p, size_t bytes, hipStream_t stream);
 // dst[0, bytes) = src[0, bytes) on the device, enqueued on `stream` (non-overlapping ranges)
 hipError_t copy_async(void* dst, const void* src, size_t bytes, hipStream_t stream);

@@ -551,7 +551,7 @@ extern "C" int thrust_cdna4_scan(void* temp, size_t* temp_bytes, int dtype, int 
                                  const void* in, void* out, int64_t n, const void* init,
                                  void* stream) {
   using namespace tcd;
-  if (!temp_bytes || n < 0 || (n > 0 && temp && (!in || !out))) return hipErrorInvalidValue;
+  if (!temp_bytes || n < 0 || temp_misaligned(temp) || (n > 0 && temp && (!in || !out))) return hipErrorInvalidValue;
   hipError_t rc = hipErrorInvalidValue;
   hipStream_t s = static_cast<hipStream_t>(stream);
   bool ok = dispatch_dtype(dtype, [&](auto t) {

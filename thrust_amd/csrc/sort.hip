@@ -1043,7 +1043,7 @@ static hipError_t sort_dispatch(void* temp, size_t* temp_bytes, int key_dtype, v
 
 extern "C" int thrust_cdna4_sort_keys(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
                                       int64_t n, int descending, void* stream) {
-  if (!temp_bytes || n < 0 || n >= tcd::kSortMaxN || (n > 0 && temp && !keys))
+  if (!temp_bytes || n < 0 || n >= tcd::kSortMaxN || tcd::temp_misaligned(temp) || (n > 0 && temp && !keys))
     return hipErrorInvalidValue;
   return (int)tcd::sort_dispatch<0>(temp, temp_bytes, key_dtype, keys, nullptr, n, descending,
                                     static_cast<hipStream_t>(stream));
@@ -1052,7 +1052,7 @@ extern "C" int thrust_cdna4_sort_keys(void* temp, size_t* temp_bytes, int key_dt
 extern "C" int thrust_cdna4_sort_pairs(void* temp, size_t* temp_bytes, int key_dtype, void* keys,
                                        int value_bytes, void* values, int64_t n, int descending,
                                        void* stream) {
-  if (!temp_bytes || n < 0 || n >= tcd::kSortMaxN || (n > 0 && temp && (!keys || !values)))
+  if (!temp_bytes || n < 0 || n >= tcd::kSortMaxN || tcd::temp_misaligned(temp) || (n > 0 && temp && (!keys || !values)))
     return hipErrorInvalidValue;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (value_bytes) {
