@@ -98,7 +98,8 @@ def test_one_workgroup_at_a_time_and_no_byte_outside_the_ranges(emulated_library
 def test_look_back_with_several_workgroups_in_flight(emulated_library, resident):
     """Tiles meet predecessors that have published a partial result or nothing yet; a sort whose
     look-back is made to give up reports it (the status word, the error, the latch to plain tickets)."""
-    files = ["tests/test_scan_gpu.py", "tests/test_bykey_gpu.py", "tests/test_random_gpu.py", "tests/test_sort_timeout_gpu.py"]
+    files = ["tests/test_scan_gpu.py", "tests/test_bykey_gpu.py", "tests/test_random_gpu.py", "tests/test_sort_timeout_gpu.py",
+             "tests/test_dirty_temp_gpu.py"]  # (dirty descriptors only matter to a tile that runs before its predecessor is done)
     if ALL:  # (buffers aligned as an allocator aligns them; the default run has the sorts in the guarded session only)
         files += ["tests/test_sort_gpu.py", "tests/test_histogram_gpu.py", "tests/test_zz_no_alloc.py"]
     print(run_session(files, resident=resident, deselect=SLOW))
